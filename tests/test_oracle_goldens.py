@@ -1,0 +1,469 @@
+"""Pins the CPU oracle against the reference's own golden vectors, known-answer
+tests and closed forms.  Each test names the reference test it restates
+(paths relative to the reference root)."""
+import numpy as np
+import pytest
+
+import oracle as fo
+from tests.refdata import k_quant_fixture, q8_0_sample_input
+
+RNG = np.random.default_rng(20240607)
+
+
+def hexbytes(s):
+    return np.frombuffer(bytes.fromhex(s), np.uint8)
+
+
+# ---------------------------------------------------------------- f16
+
+def test_f16_to_f32_matches_ieee_for_every_bit_pattern():
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([fo.f16_to_f32(int(b)) for b in bits], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_f32_to_f16_rounds_to_nearest_even():
+    # every f16 value's neighbourhood: exact, both half-way points, and one ulp either side
+    cases = []
+    for b in list(range(0, 0x7C00, 37)) + [0, 1, 2, 0x3FF, 0x400, 0x401, 0x7BFF]:
+        lo = np.float32(np.uint16(b).view(np.float16))
+        hi = np.float32(np.uint16(b + 1).view(np.float16)) if b + 1 < 0x7C00 else np.float32(65536.0)
+        mid = np.float32((np.float64(lo) + np.float64(hi)) / 2)
+        for v in (lo, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9))):
+            cases += [v, -v]
+    cases += list(RNG.standard_normal(4000).astype(np.float32) * np.float32(0.05))
+    cases += [np.float32(65504.0), np.float32(65519.9), np.float32(65520.0), np.float32(1e9),
+              np.float32(2.0 ** -25), np.float32(2.0 ** -24), np.float32(1e-10)]
+    with np.errstate(over="ignore"):
+        for v in cases:
+            want = int(np.float32(v).astype(np.float16).view(np.uint16))
+            assert fo.f32_to_f16(v) == want, (float(v), hex(want))
+
+
+# ---------------------------------------------------------------- Q8_0 encoder
+# crates/frink-quant/src/encode.rs:165-265
+
+def test_q8_0_matches_llama_cpp_quantize_row_q8_0_ref(vectors):
+    got = fo.encode_row(fo.Q8_0, q8_0_sample_input(64))
+    assert got.tobytes() == bytes.fromhex(vectors["q8_0_encode_golden"])
+
+
+def test_q8_0_scale_is_applied_as_a_reciprocal_multiply(vectors):
+    x = np.array(vectors["q8_0_tie_block_f16_bits"], np.uint16).view(np.float16).astype(np.float32)
+    got = fo.encode_row(fo.Q8_0, x)
+    gold = bytes.fromhex(vectors["q8_0_tie_block_golden"])
+    assert got.tobytes() == gold
+    # the divide spelling differs on this block, so the golden asserts something
+    d = np.float32(np.abs(x).max()) / np.float32(127.0)
+    divided = np.array([int(np.sign(v) * np.floor(abs(v) + np.float32(0.5))) for v in (x / d)], np.int8)
+    assert divided.tobytes() != gold[2:]
+
+
+def test_q8_0_all_zero_block_is_34_zero_bytes():
+    assert fo.encode_row(fo.Q8_0, np.zeros(32, np.float32)).tobytes() == bytes(34)
+
+
+@pytest.mark.parametrize("kind,ragged", [(fo.Q8_0, 33), (fo.Q8_0, 1), (fo.Q4_K, 257), (fo.Q4_K, 32),
+                                         (fo.Q6_K, 257), (fo.Q6_K, 16)])
+def test_a_ragged_row_is_refused_and_an_empty_one_accepted(kind, ragged):
+    assert fo.encode_row(kind, np.full(ragged, 0.5, np.float32)) is None
+    assert fo.encode_row(kind, np.zeros(0, np.float32)).size == 0
+
+
+def test_q8_0_round_trip_is_within_a_quantization_step():
+    x = q8_0_sample_input(8 * 32)
+    back = fo.dequant(fo.Q8_0, fo.encode_row(fo.Q8_0, x))
+    for b in range(8):
+        c = x[b * 32:(b + 1) * 32]
+        bound = np.abs(c).max() / 127.0 * (0.5 + 127.0 * 2.0 ** -11)
+        assert np.abs(c - back[b * 32:(b + 1) * 32]).max() <= bound
+
+
+# ---------------------------------------------------------------- K-quant encoders
+# crates/frink-quant/src/encode/q4_k.rs:152-362, encode/q6_k.rs:221-504
+
+@pytest.fixture(scope="module")
+def kfix(vectors):
+    return k_quant_fixture(vectors["real_weight_blocks_f16_bits"])
+
+
+def test_q4_k_matches_llama_cpp_quantize_row_q4_k_ref(vectors, kfix):
+    got = fo.encode_row(fo.Q4_K, kfix).reshape(12, 144)
+    gold = hexbytes(vectors["q4_k_encode_golden"]).reshape(12, 144)
+    for b in range(12):
+        assert got[b].tobytes() == gold[b].tobytes(), "super-block %d disagrees with llama.cpp" % b
+
+
+def test_q6_k_matches_llama_cpp_quantize_row_q6_k_ref(vectors, kfix):
+    got = fo.encode_row(fo.Q6_K, kfix).reshape(12, 210)
+    gold = hexbytes(vectors["q6_k_encode_golden"]).reshape(12, 210)
+    for b in range(12):
+        assert got[b].tobytes() == gold[b].tobytes(), "super-block %d disagrees with llama.cpp" % b
+
+
+def test_q6_k_all_zero_super_block_is_210_zero_bytes():
+    assert fo.encode_row(fo.Q6_K, np.zeros(256, np.float32)).tobytes() == bytes(210)
+
+
+def test_q6_k_group_scales_are_stored_signed(kfix):
+    blocks = fo.encode_row(fo.Q6_K, kfix).reshape(12, 210)
+    assert (blocks[:, 192:208].view(np.int8) < 0).any()
+
+
+def test_q4_k_every_element_lands_on_its_nearest_level(kfix):
+    data = fo.encode_row(fo.Q4_K, kfix)
+    back = fo.dequant(fo.Q4_K, data)
+    blocks = data.reshape(12, 144)
+    for b in range(12):
+        d = np.float32(blocks[b, 0:2].view(np.float16)[0])
+        dmin = np.float32(blocks[b, 2:4].view(np.float16)[0])
+        s = blocks[b, 4:16]
+        for j in range(8):
+            if j < 4:
+                sc, m = s[j] & 63, s[j + 4] & 63
+            else:
+                sc = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4)
+                m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+            dj, dm = d * np.float32(sc), dmin * np.float32(m)
+            levels = dj * np.arange(16, dtype=np.float32) - dm
+            sl = slice(b * 256 + 32 * j, b * 256 + 32 * j + 32)
+            chosen = np.abs(kfix[sl] - back[sl])
+            best = np.abs(kfix[sl][:, None] - levels[None, :]).min(axis=1)
+            assert (best >= chosen).all(), (b, j)
+
+
+def test_q6_k_every_element_lands_on_its_nearest_level(kfix):
+    data = fo.encode_row(fo.Q6_K, kfix)
+    back = fo.dequant(fo.Q6_K, data)
+    blocks = data.reshape(12, 210)
+    for b in range(12):
+        d = np.float32(blocks[b, 208:210].view(np.float16)[0])
+        for g in range(16):
+            dg = d * np.float32(blocks[b, 192 + g].view(np.int8))
+            levels = dg * np.arange(-32, 32, dtype=np.float32)
+            sl = slice(b * 256 + 16 * g, b * 256 + 16 * g + 16)
+            chosen = np.abs(kfix[sl] - back[sl])
+            best = np.abs(kfix[sl][:, None] - levels[None, :]).min(axis=1)
+            assert (best >= chosen).all(), (b, g)
+
+
+# crates/frink-quant/src/encode/fit.rs:601-646
+def test_nearest_int_rounds_ties_to_even():
+    for f, want in [(0.5, 0), (1.5, 2), (2.5, 2), (-0.5, 0), (-1.5, -2), (3.7, 4), (-3.7, -4), (3.2, 3)]:
+        assert fo.nearest_int(f) == want
+
+
+def test_make_qx_quants_zero_group_and_sign_convention():
+    s, l = fo.make_qx_quants(np.zeros(16, np.float32))
+    assert s == 0.0 and (l == 0).all()
+    x = np.array([1.0, -0.5, 0.25, 0.0, 0.125, -0.75, 0.5, -0.25, 0.0625, -0.0625, 0.3, -0.3, 0.9, -0.9,
+                  0.7, -0.1], np.float32)
+    s, l = fo.make_qx_quants(x)
+    assert s < 0 and l[0] == 0 and l[13] > 32
+    x2 = np.full(16, 0.001, np.float32)
+    x2[0], x2[7] = 1.0, -0.4
+    assert fo.make_qx_quants(x2, 32, 1)[0] != fo.make_qx_quants(x2, 32, 2)[0]
+
+
+# ---------------------------------------------------------------- dequant
+# crates/frink-quant/src/lib.rs:6297-6341, 6423-6529, 7108-7246 (goldens printed to 6 digits: 1e-3)
+
+@pytest.mark.parametrize("kind,blk,gold", [
+    (fo.Q4_K, "q4_k_test_block", "q4_k_golden"),
+    (fo.Q6_K, "q6_k_test_block", "q6_k_golden"),
+    (fo.Q6_K, "q6_k_signed_scales_test_block", "q6_k_signed_scales_golden"),
+    (fo.Q6_K, "q6_k_signed_test_block", "q6_k_signed_golden"),
+])
+def test_dequant_matches_independent_python_reference(vectors, kind, blk, gold):
+    got = fo.dequant(kind, hexbytes(vectors[blk]))
+    want = np.array(vectors[gold], np.float32)
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() < 1e-3
+
+
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K])
+def test_block_walk_and_index_formula_decoders_agree_bit_for_bit(kind):
+    bb, be = fo.BLOCK[kind]
+    for _ in range(64):
+        blk = RNG.integers(0, 256, bb, dtype=np.uint8)
+        # keep the f16 super-scales finite
+        for off in ((0, 2) if kind == fo.Q4_K else (208,)):
+            blk[off:off + 2] = np.frombuffer(np.float16(RNG.uniform(-0.01, 0.01)).tobytes(), np.uint8)
+        walk = fo.dequant(kind, blk)
+        elem = np.array([fo.element(kind, blk, i) for i in range(be)], np.float32)
+        assert np.array_equal(walk.view(np.uint32), elem.view(np.uint32))
+
+
+def test_q8_0_dequant_is_q_times_f16_scale():
+    blk = RNG.integers(0, 256, 34 * 5, dtype=np.uint8).reshape(5, 34)
+    blk[:, 0:2] = np.frombuffer(np.float16([0.01, -0.5, 1.0, 6e-6, 0.0]).tobytes(), np.uint8).reshape(5, 2)
+    got = fo.dequant(fo.Q8_0, blk.ravel()).reshape(5, 32)
+    want = blk[:, 2:].view(np.int8).astype(np.float32) * blk[:, 0:2].copy().view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_misaligned_buffers_are_refused():
+    for kind in (fo.Q8_0, fo.Q4_K, fo.Q6_K):
+        with pytest.raises(ValueError):
+            fo.dequant(kind, np.zeros(5, np.uint8))
+
+
+# fused dot == dequant-then-dot (crates/frink-quant/src/lib.rs:6544-6577, 7170-7246)
+@pytest.mark.parametrize("kind,blk,freq,fn", [
+    (fo.Q4_K, "q4_k_test_block", 0.017, np.sin),
+    (fo.Q6_K, "q6_k_test_block", 0.021, np.cos),
+    (fo.Q6_K, "q6_k_signed_test_block", 0.023, np.sin),
+    (fo.Q6_K, "q6_k_signed_scales_test_block", 0.023, np.sin),
+])
+def test_fused_dot_matches_dequant_then_dot(vectors, kind, blk, freq, fn):
+    b = hexbytes(vectors[blk])
+    x = fn(np.arange(256, dtype=np.float32) * np.float32(freq)).astype(np.float32)
+    expected = float(np.dot(fo.dequant(kind, b).astype(np.float64), x.astype(np.float64)))
+    assert abs(fo.dot_f32(kind, b, x) - expected) < 1e-2
+
+
+def test_q6_k_scalar_dot_matches_python_golden_with_negative_scales(vectors):
+    x = np.sin(np.arange(256, dtype=np.float32) * np.float32(0.023)).astype(np.float32)
+    expected = float(np.dot(np.array(vectors["q6_k_signed_scales_golden"], np.float64), x.astype(np.float64)))
+    got = fo.dot_f32(fo.Q6_K, hexbytes(vectors["q6_k_signed_scales_test_block"]), x)
+    assert abs(got - expected) < 1e-2
+
+
+def _python_order_dot_q4_k(row, x):
+    """dot_q4_k_f32_scalar's summation order in numpy float32, one op at a time."""
+    acc = np.float32(0)
+    w = fo.dequant(fo.Q4_K, row)
+    for wi, xi in zip(w, x):
+        acc = np.float32(acc + np.float32(wi * xi))
+    return acc
+
+
+def test_q4_k_f32_dot_is_the_sequential_sum_of_dequantized_products(vectors):
+    row = np.tile(hexbytes(vectors["q4_k_test_block"]), 3)
+    x = RNG.standard_normal(768).astype(np.float32)
+    got = np.float32(fo.dot_f32(fo.Q4_K, row, x))
+    assert got.view(np.uint32) == _python_order_dot_q4_k(row, x).view(np.uint32)
+
+
+# ---------------------------------------------------------------- activation quantizers
+# crates/frink-quant/src/act_quant.rs:215-300 (libggml's own outputs)
+
+def _block(head, n):
+    x = np.zeros(n, np.float32)
+    x[:len(head)] = head
+    return x
+
+
+def test_q8_k_rounds_ties_to_even():
+    q, d, bs = fo.quantize_q8_k(_block([127.0, 2.5, -3.5, 0.5, -0.5, 126.5], 256))
+    assert d[0] == 1.0
+    assert list(q[:6]) == [127, 2, -4, 0, 0, 126]
+    assert bs[0] == 127 + 2 - 4 + 126
+
+
+def test_q8_k_takes_its_scale_from_the_inverse():
+    amax = np.uint32(0x3FE46A64).view(np.float32)
+    x = np.uint32(0x3DD7D365).view(np.float32)
+    q, d, _ = fo.quantize_q8_k(_block([-amax, x], 256))
+    assert d.view(np.uint32)[0] == 0x3C6636D1
+    assert list(q[:2]) == [-127, 8]
+
+
+def test_q8_k_scale_is_never_negative_and_quants_are_odd_symmetric():
+    qn, dn, _ = fo.quantize_q8_k(_block([-127.0, 2.5], 256))
+    qp, dp, _ = fo.quantize_q8_k(_block([127.0, -2.5], 256))
+    assert (dn[0], dp[0]) == (1.0, 1.0)
+    assert (qn[1], qp[1]) == (2, -2)
+    assert np.array_equal(qn, -qp)
+
+
+def test_q8_k_all_zero_block_is_all_zero():
+    q, d, bs = fo.quantize_q8_k(np.zeros(256, np.float32))
+    assert d[0] == 0.0 and not q.any() and not bs.any()
+
+
+def test_q8_k_bsums_are_the_16_wide_sums_and_blocks_are_independent():
+    x = RNG.standard_normal(1024).astype(np.float32)
+    q, d, bs = fo.quantize_q8_k(x)
+    assert np.array_equal(bs, q.reshape(-1, 16).astype(np.int32).sum(axis=1).astype(np.int16))
+    q1, d1, bs1 = fo.quantize_q8_k(x[256:512])
+    assert np.array_equal(q1, q[256:512]) and d1[0] == d[1] and np.array_equal(bs1, bs[16:32])
+    # closed form, computed independently in numpy float32
+    for b in range(4):
+        c = x[b * 256:(b + 1) * 256]
+        iscale = np.float32(127.0) / np.abs(c).max()
+        assert d[b] == np.float32(1.0) / iscale
+        assert np.array_equal(q[b * 256:(b + 1) * 256], np.rint(iscale * c).astype(np.int8))
+
+
+def test_q8_0_act_forms():
+    head = [127.0, 2.5, -3.5, 0.5, 1.5]
+    q, d = fo.quantize_q8_0(_block(head, 32), fo.FORM_NEON)
+    assert d[0] == 1.0 and list(q[:5]) == [127, 2, -4, 0, 2]
+    assert list(fo.quantize_q8_0(_block(head, 32), fo.FORM_AVX)[0][:5]) == [127, 2, -4, 0, 2]
+    assert list(fo.quantize_q8_0(_block(head, 32), fo.FORM_SCALAR)[0][:5]) == [127, 3, -4, 1, 2]
+    q, d = fo.quantize_q8_0(_block([1.0, 0.5], 32), fo.FORM_NEON)
+    assert d[0] == np.float32(np.uint16(0x2008).view(np.float16)) and d[0] != np.float32(1.0) / np.float32(127.0)
+    assert list(q[:2]) == [127, 64]
+    x = _block([np.uint32(0x4013E709).view(np.float32), np.uint32(0x3CDF99C0).view(np.float32)], 32)
+    q, d = fo.quantize_q8_0(x, fo.FORM_NEON)
+    assert d[0] == np.float32(np.uint16(0x24A9).view(np.float16)) and list(q[:2]) == [127, 2]
+    assert fo.quantize_q8_0(x, fo.FORM_AVX)[0][1] == 1
+    for form in (fo.FORM_NEON, fo.FORM_AVX, fo.FORM_SCALAR):
+        q, d = fo.quantize_q8_0(np.zeros(32, np.float32), form)
+        assert d[0] == 0.0 and not q.any()
+
+
+# ---------------------------------------------------------------- integer dots
+# No reference-held vector exists for these; pinned by the exact identity
+#   int_dot(w, q8) == sum_i dequant(w)_i * (q8_i * d_act)      (in exact arithmetic)
+# against the vector-pinned dequantizers, and by int-dot ~= f32-dot
+# (crates/frink-quant/src/lib.rs:5624-5656, 5756-5808: rel < 0.05).
+
+def _weights(kind, rows, cols, sigma=0.02):
+    w = (RNG.standard_normal((rows, cols)) * sigma).astype(np.float32)
+    return fo.encode_matrix(kind, w)
+
+
+@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q6_K])
+def test_int_dot_equals_dequant_dot_in_exact_arithmetic(kind):
+    rows, cols = 6, 1024
+    bb, be = fo.BLOCK[kind]
+    data = _weights(kind, rows, cols)
+    row_bytes = cols // be * bb
+    x = RNG.standard_normal(cols).astype(np.float32)
+    acts = fo.quantize_q8_0(x) if kind == fo.Q8_0 else fo.quantize_q8_k(x)
+    q, d = acts[0], acts[1]
+    xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), be)
+    for r in range(rows):
+        row = data[r * row_bytes:(r + 1) * row_bytes]
+        # exact-arithmetic value of the dequantized row: Q4_K's d*sc and dmin*m are rounded in the
+        # dequantizer but not in the int dot, so rebuild the unrounded weights for Q4_K
+        if kind == fo.Q4_K:
+            wq = _q4_k_exact(row)
+        else:
+            wq = fo.dequant(kind, row).astype(np.float64)
+            if kind == fo.Q6_K:
+                wq = _q6_k_exact(row)
+        want = float(np.dot(wq, xa))
+        got = fo.dot_int(kind, row, acts)
+        scale = float(np.abs(wq * xa).sum())
+        assert abs(got - want) <= 2e-6 * scale + 1e-12, (kind, r, got, want)
+        f32 = fo.dot_f32(kind, row, x)
+        assert abs(got - f32) <= 0.05 * max(abs(f32), 0.5)
+
+
+def _q4_k_exact(row):
+    out = []
+    for blk in row.reshape(-1, 144):
+        d = float(blk[0:2].view(np.float16)[0])
+        dmin = float(blk[2:4].view(np.float16)[0])
+        s = blk[4:16].astype(int)
+        for j in range(8):
+            if j < 4:
+                sc, m = s[j] & 63, s[j + 4] & 63
+            else:
+                sc = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4)
+                m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+            qs = blk[16 + (j // 2) * 32:16 + (j // 2) * 32 + 32].astype(int)
+            nib = (qs >> 4) if j & 1 else (qs & 15)
+            out.append(d * sc * nib - dmin * m)
+    return np.concatenate(out)
+
+
+def _q6_k_exact(row):
+    out = np.empty(row.size // 210 * 256)
+    for b, blk in enumerate(row.reshape(-1, 210)):
+        d = float(blk[208:210].view(np.float16)[0])
+        sc = blk[192:208].view(np.int8).astype(int)
+        for i in range(256):
+            half, r = divmod(i, 128)
+            quarter, l = divmod(r, 32)
+            qlb = int(blk[half * 64 + (quarter & 1) * 32 + l])
+            lo = (qlb >> 4) if quarter & 2 else (qlb & 15)
+            hi = (int(blk[128 + half * 32 + l]) >> (2 * quarter)) & 3
+            out[b * 256 + i] = d * sc[i // 16] * ((lo | (hi << 4)) - 32)
+    return out
+
+
+def test_exact_rebuilds_agree_with_the_dequantizers():
+    # the float64 rebuilds above are themselves checked against the pinned dequantizers
+    for kind, fn in ((fo.Q4_K, _q4_k_exact), (fo.Q6_K, _q6_k_exact)):
+        data = _weights(kind, 2, 512)
+        assert np.abs(fn(data) - fo.dequant(kind, data)).max() < 1e-6
+
+
+# ---------------------------------------------------------------- dispatch level
+# crates/frink-core/src/weight_matrix.rs:4747-5350: apply_batch == N x apply; out is [batch][rows]
+
+@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q6_K])
+@pytest.mark.parametrize("mode", [fo.F32_DOT, fo.INT_DOT])
+def test_gemm_is_batch_times_gemv_and_output_is_batch_major(kind, mode):
+    rows, cols, batch = 24, 512, 5
+    data = _weights(kind, rows, cols)
+    x = RNG.standard_normal((batch, cols)).astype(np.float32)
+    y = fo.gemm(kind, data, rows, cols, x, mode, threads=3)
+    assert y.shape == (batch, rows)
+    for b in range(batch):
+        yb = fo.gemv(kind, data, rows, cols, x[b], mode, threads=1)
+        assert np.array_equal(y[b].view(np.uint32), yb.view(np.uint32))
+    part = fo.gemm(kind, data, rows, cols, x, mode, row0=8, nrows=8)
+    assert np.array_equal(part, y[:, 8:16])
+    # against a plain float64 matmul of the dequantized matrix
+    w = fo.dequant(kind, data).reshape(rows, cols).astype(np.float64)
+    ref = x.astype(np.float64) @ w.T
+    tol = 1e-5 if mode == fo.F32_DOT else 0.05
+    assert np.abs(y - ref).max() <= tol * np.abs(ref).max()
+
+
+# ---------------------------------------------------------------- MoE
+# crates/frink-moe/src/lib.rs:1345-1404
+
+def test_route_top_k_softmax_kats():
+    ids, w = fo.route_top_k_softmax([0.1, 5.0, 0.2, 3.0, -1.0], 2, True)
+    assert list(ids) == [1, 3] and abs(w.sum() - 1) < 1e-5 and w[0] > w[1]
+    logits = np.arange(1, 9, dtype=np.float32)
+    for k in range(1, 9):
+        assert abs(fo.route_top_k_softmax(logits, k, True)[1].sum() - 1) < 1e-5
+    ids, w = fo.route_top_k_softmax(logits, 3, False)
+    assert list(ids) == [7, 6, 5]
+    assert np.abs(w - np.array([0.6323223, 0.2326232, 0.0855683], np.float32)).max() < 1e-4
+    assert abs(w.sum() - 0.9505138) < 1e-4
+    ids2, w2 = fo.route_top_k_softmax(logits, 3, True)
+    assert list(ids2) == list(ids) and np.abs(w / w.sum() - w2).max() < 1e-4
+
+
+def test_silu_and_swiglu_are_the_textbook_forms():
+    g = RNG.standard_normal(100).astype(np.float32) * 3
+    u = RNG.standard_normal(100).astype(np.float32)
+    want = g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u
+    assert (np.abs(fo.swiglu(g, u) - want) <= 4e-7 * np.maximum(np.abs(want), 1)).all()
+    assert fo.silu(0.0) == 0.0
+
+
+def test_moe_batch_equals_per_token_experts_combined():
+    E, k, hidden, ffn, batch = 6, 2, 256, 512, 9
+    gate = _weights(fo.Q4_K, E * ffn, hidden)
+    up = _weights(fo.Q4_K, E * ffn, hidden)
+    down = _weights(fo.Q4_K, E * hidden, ffn)
+    x = RNG.standard_normal((batch, hidden)).astype(np.float32)
+    logits = RNG.standard_normal((batch, E)).astype(np.float32)
+    routed = [fo.route_top_k_softmax(l, k, True) for l in logits]
+    ids = np.stack([r[0] for r in routed])
+    w = np.stack([r[1] for r in routed])
+    got = fo.moe_ffn_batch(fo.Q4_K, gate, up, down, E, hidden, ffn, x, ids, w)
+    gu = ffn * (hidden // 256) * 144
+    dn = hidden * (ffn // 256) * 144
+    for b in range(batch):
+        acc = np.zeros(hidden, np.float32)
+        # accumulation order in the batch path is expert id ascending
+        for e in sorted(ids[b]):
+            we = w[b][list(ids[b]).index(e)]
+            g = fo.gemv(fo.Q4_K, gate[e * gu:(e + 1) * gu], ffn, hidden, x[b])
+            u = fo.gemv(fo.Q4_K, up[e * gu:(e + 1) * gu], ffn, hidden, x[b])
+            o = fo.gemv(fo.Q4_K, down[e * dn:(e + 1) * dn], hidden, ffn, fo.swiglu(g, u))
+            acc = acc + we * o
+        assert np.array_equal(got[b].view(np.uint32), acc.view(np.uint32))
