@@ -1,0 +1,247 @@
+"""frink_amd -- MI355X (gfx950) quantized-matmul backend for Frink: Python binding of the C ABI.
+
+The product is ``lib/libfrink_hip.so`` (HIP kernels + C ABI, ``include/frink_hip.h``).  This
+module only loads it with ctypes and passes device pointers of torch tensors through; torch is
+used for device memory and streams, nothing else.  There is no CPU fallback: if the library is
+missing or no gfx950 device answers, calls raise.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libfrink_hip.so")
+
+# quant kinds (ggml type ids) and their QuantKind::name()
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+KIND_NAME = {Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K"}
+BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}  # (block_bytes, block_elems)
+ACT_F32, ACT_INT8 = 0, 1
+
+OK, ERR_NO_DEVICE, ERR_UNSUPPORTED, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_OOM = 0, -1, -2, -3, -4, -5, -6
+
+EXPORTS = [
+    "frk_hip_probe", "frk_hip_dense_enabled", "frk_hip_last_error", "frk_hip_matvec_kernel",
+    "frk_hip_gemm_supported", "frk_hip_has_launch", "frk_hip_block_bytes", "frk_hip_block_elems",
+    "frk_hip_worth_a_gemm", "frk_hip_weights_register", "frk_hip_weights_from_device",
+    "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
+    "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
+    "frk_hip_gemm_dev",
+    "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
+    "frk_hip_copy_dev", "frk_hip_read_dev",
+]
+
+
+class BackendError(RuntimeError):
+    """A failed call; carries the C ABI's status code and message
+    (the reference's BackendError, crates/frink-core/src/weight_matrix/gpu_backend.rs:90)."""
+
+    def __init__(self, code, message):
+        super().__init__("%s (status %d)" % (message, code))
+        self.code = code
+        self.message = message
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("device_count", C.c_int32), ("compute_units", C.c_int32), ("name", C.c_char * 128),
+                ("gcn_arch", C.c_char * 64), ("total_vram_bytes", C.c_uint64), ("free_vram_bytes", C.c_uint64)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded C ABI library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `python -m frink_amd.build`" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        vp, sz, i = C.c_void_p, C.c_size_t, C.c_int
+        sig = {
+            "frk_hip_probe": (i, [C.POINTER(DeviceInfo)]),
+            "frk_hip_dense_enabled": (i, []),
+            "frk_hip_last_error": (C.c_char_p, []),
+            "frk_hip_matvec_kernel": (C.c_char_p, [i]),
+            "frk_hip_gemm_supported": (i, [i]),
+            "frk_hip_has_launch": (i, [i]),
+            "frk_hip_block_bytes": (i, [i]),
+            "frk_hip_block_elems": (i, [i]),
+            "frk_hip_worth_a_gemm": (i, [sz]),
+            "frk_hip_weights_register": (i, [i, vp, sz, sz, sz, C.POINTER(vp)]),
+            "frk_hip_weights_from_device": (i, [i, vp, sz, sz, sz, vp, C.POINTER(vp)]),
+            "frk_hip_weights_release": (i, [vp]),
+            "frk_hip_weights_rows": (sz, [vp]),
+            "frk_hip_weights_cols": (sz, [vp]),
+            "frk_hip_weights_kind": (i, [vp]),
+            "frk_hip_launch_matvec": (i, [i, vp, sz, vp, sz, sz, sz, vp]),
+            "frk_hip_launch_mul_mm": (i, [i, vp, sz, vp, sz, sz, sz, sz, sz, vp]),
+            "frk_hip_gemv_dev": (i, [vp, vp, vp, i, vp]),
+            "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
+            "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
+            "frk_hip_quantize_q8_k_dev": (i, [vp, sz, vp, vp, vp, vp]),
+            "frk_hip_quantize_q8_0_dev": (i, [vp, sz, vp, vp, vp]),
+            "frk_hip_dequant_dev": (i, [vp, vp, vp]),
+            "frk_hip_copy_dev": (i, [vp, vp, sz, vp]),
+            "frk_hip_read_dev": (i, [vp, sz, vp, vp]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().frk_hip_last_error().decode()
+
+
+def check(status):
+    if status != OK:
+        raise BackendError(status, last_error())
+
+
+def probe():
+    """Device facts, or raises BackendError(ERR_NO_DEVICE) on a host without a gfx950 GPU."""
+    info = DeviceInfo()
+    check(lib().frk_hip_probe(C.byref(info)))
+    return {"device_count": info.device_count, "compute_units": info.compute_units,
+            "name": info.name.decode(), "gcn_arch": info.gcn_arch.decode(),
+            "total_vram_bytes": info.total_vram_bytes, "free_vram_bytes": info.free_vram_bytes}
+
+
+def matvec_kernel(kind):
+    r = lib().frk_hip_matvec_kernel(kind)
+    return r.decode() if r else None
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _np_ptr(a):
+    return C.c_void_p(a.ctypes.data)
+
+
+class Weights:
+    """One quantized weight matrix resident in HBM (the reference's
+    WeightMatrix::Quantized{data, rows, cols, kind}, crates/frink-core/src/weight_matrix.rs:780-787)."""
+
+    def __init__(self, handle, kind, rows, cols, keepalive=None):
+        self.handle, self.kind, self.rows, self.cols = handle, kind, rows, cols
+        self._keepalive = keepalive
+
+    @classmethod
+    def from_host(cls, kind, data, rows, cols):
+        data = np.ascontiguousarray(np.frombuffer(data, np.uint8) if isinstance(data, (bytes, bytearray)) else data,
+                                    dtype=np.uint8)
+        h = C.c_void_p()
+        check(lib().frk_hip_weights_register(kind, _np_ptr(data), data.size, rows, cols, C.byref(h)))
+        return cls(h, kind, rows, cols, keepalive=data)
+
+    @classmethod
+    def from_device(cls, kind, data_dev, rows, cols):
+        """data_dev: a uint8 torch tensor on the GPU holding GGUF block bytes."""
+        h = C.c_void_p()
+        check(lib().frk_hip_weights_from_device(kind, C.c_void_p(data_dev.data_ptr()), data_dev.numel(), rows, cols,
+                                                _stream(), C.byref(h)))
+        return cls(h, kind, rows, cols)
+
+    def release(self):
+        if self.handle:
+            check(lib().frk_hip_weights_release(self.handle))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            if self.handle and _lib is not None:
+                _lib.frk_hip_weights_release(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+    # ---- device-resident operations (torch tensors on cuda:0) ----
+    def gemv(self, x, out=None, act_mode=ACT_F32):
+        import torch
+        assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.numel() == self.cols
+        y = out if out is not None else torch.empty(self.rows, dtype=torch.float32, device=x.device)
+        check(lib().frk_hip_gemv_dev(self.handle, C.c_void_p(x.data_ptr()), C.c_void_p(y.data_ptr()), act_mode,
+                                     _stream()))
+        return y
+
+    def gemv_q8k(self, acts, out=None):
+        """acts = (q, d, bsums) from quantize_q8_k: one activation shared by several projections."""
+        import torch
+        q, d, bs = acts
+        y = out if out is not None else torch.empty(self.rows, dtype=torch.float32, device=q.device)
+        check(lib().frk_hip_gemv_q8k_dev(self.handle, C.c_void_p(q.data_ptr()), C.c_void_p(d.data_ptr()),
+                                         C.c_void_p(bs.data_ptr()), C.c_void_p(y.data_ptr()), _stream()))
+        return y
+
+    def gemm(self, x, out=None):
+        import torch
+        assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.shape[-1] == self.cols
+        batch = x.numel() // self.cols
+        y = out if out is not None else torch.empty((batch, self.rows), dtype=torch.float32, device=x.device)
+        check(lib().frk_hip_gemm_dev(self.handle, C.c_void_p(x.data_ptr()), batch, C.c_void_p(y.data_ptr()),
+                                     _stream()))
+        return y
+
+    def dequant(self):
+        import torch
+        out = torch.empty((self.rows, self.cols), dtype=torch.float32, device="cuda")
+        check(lib().frk_hip_dequant_dev(self.handle, C.c_void_p(out.data_ptr()), _stream()))
+        return out
+
+
+def quantize_q8_k(x):
+    """quantize_activations_q8_k on the device: returns (q int8[n], d f32[n/256], bsums int16[n/16])."""
+    import torch
+    x = x.contiguous()
+    n = x.numel()
+    q = torch.empty(n, dtype=torch.int8, device=x.device)
+    d = torch.empty(n // 256, dtype=torch.float32, device=x.device)
+    bs = torch.empty(n // 16, dtype=torch.int16, device=x.device)
+    check(lib().frk_hip_quantize_q8_k_dev(C.c_void_p(x.data_ptr()), n, C.c_void_p(q.data_ptr()),
+                                          C.c_void_p(d.data_ptr()), C.c_void_p(bs.data_ptr()), _stream()))
+    return q, d, bs
+
+
+def quantize_q8_0(x):
+    """quantize_activations_q8 (Avx form) on the device: returns (q int8[n], d f32[n/32])."""
+    import torch
+    x = x.contiguous()
+    n = x.numel()
+    q = torch.empty(n, dtype=torch.int8, device=x.device)
+    d = torch.empty(n // 32, dtype=torch.float32, device=x.device)
+    check(lib().frk_hip_quantize_q8_0_dev(C.c_void_p(x.data_ptr()), n, C.c_void_p(q.data_ptr()),
+                                          C.c_void_p(d.data_ptr()), _stream()))
+    return q, d
+
+
+# ---- host-buffer entry points: numpy in, numpy out ----
+
+def launch_matvec(kind, weights, x, rows, row_bytes):
+    """BackendDispatch::launch_matvec: None when the backend has no kernel for `kind`
+    (the reference's `None`), raises BackendError when the launch fails (`Some(Err)`)."""
+    if not lib().frk_hip_has_launch(kind):
+        return None
+    weights = np.ascontiguousarray(weights, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(rows, np.float32)
+    check(lib().frk_hip_launch_matvec(kind, _np_ptr(weights), weights.size, _np_ptr(x), x.size, rows, row_bytes,
+                                      _np_ptr(out)))
+    return out
+
+
+def launch_mul_mm(kind, weights, x_batch, n_rows, n_cols, batch, row_bytes):
+    """frink_cuda::mul_mm_launch::launch_mul_mm: out[token*n_rows + row]."""
+    weights = np.ascontiguousarray(weights, np.uint8)
+    x_batch = np.ascontiguousarray(x_batch, np.float32)
+    out = np.empty((batch, n_rows), np.float32)
+    check(lib().frk_hip_launch_mul_mm(kind, _np_ptr(weights), weights.size, _np_ptr(x_batch), x_batch.size, n_rows,
+                                      n_cols, batch, row_bytes, _np_ptr(out)))
+    return out

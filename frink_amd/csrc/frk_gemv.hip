@@ -1,0 +1,335 @@
+// Decode GEMV over GGUF block formats: y[r] = sum_k W[r][k] * x[k], one activation vector.
+//
+// Bandwidth-bound: every weight byte is read once from HBM with 16-byte loads, the quantized
+// activation lives in LDS, the integer products run on v_dot4_i32_i8 and a block's scale is
+// applied once per 64 weights.  A wavefront (or an LPR-lane part of one, for short rows) owns a
+// row; lanes walk the row in "units" of 64 weights.
+#include "frk_internal.hpp"
+
+namespace frk {
+
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    _Float16 v;
+    uint16_t h = (uint16_t)bits16;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
+    return v + __int_as_float(o);
+}
+
+// Sum over the LPR lanes that share a row; every lane of the part ends with the total.
+template <int LPR>
+__device__ __forceinline__ float part_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror
+    v = dpp_add<0x140>(v);  // row_mirror: all 16 lanes of a row hold the row's sum
+    if (LPR >= 32) v += __shfl_xor(v, 16);
+    if (LPR >= 64) v += __shfl_xor(v, 32);
+    return v;
+}
+
+// ------------------------------------------------------------------ Q4_K x Q8_K
+// dot_q4_k_q8 (crates/frink-quant/src/lib.rs:822-869).  Unit = (block b, pair p): the 32 bytes
+// qs[32p..32p+32] hold sub-block 2p in their low nibbles and 2p+1 in their high nibbles.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows,
+                                                        int nb, const int8_t *__restrict__ aq,
+                                                        const float *__restrict__ ad,
+                                                        const int16_t *__restrict__ absums, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    int8_t *sq = reinterpret_cast<int8_t *>(smem);      // nb*256 activation quants
+    int *sbs = reinterpret_cast<int *>(sq + nb * 256);  // nb*8 sums over 32
+    float *sd = reinterpret_cast<float *>(sbs + nb * 8);
+    for (int i = threadIdx.x; i < nb * 16; i += 256) smem[i] = reinterpret_cast<const uint4 *>(aq)[i];
+    for (int i = threadIdx.x; i < nb * 8; i += 256) sbs[i] = (int)absums[2 * i] + (int)absums[2 * i + 1];
+    for (int i = threadIdx.x; i < nb; i += 256) sd[i] = ad[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const int units = nb * 4;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * row_stride;
+            for (int u = l; u < units; u += LPR) {
+                const int b = u >> 2, p = u & 3;
+                const uint4 *blk = reinterpret_cast<const uint4 *>(row + (size_t)b * Q4_K_BYTES);
+                const uint4 h = blk[0];
+                const uint4 qa = blk[1 + 2 * p], qb = blk[2 + 2 * p];
+                const uint4 *a = reinterpret_cast<const uint4 *>(sq + b * 256 + p * 64);
+                const uint4 a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];
+                // 6-bit scales and mins of sub-blocks 2p and 2p+1 (q4_k_scale_min, lib.rs:321-330)
+                uint32_t scw, mw;
+                if (p < 2) {
+                    scw = h.y & 0x3f3f3f3fu;
+                    mw = h.z & 0x3f3f3f3fu;
+                } else {
+                    scw = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
+                    mw = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
+                }
+                const int sh = (p & 1) * 16;
+                const int sc1 = (scw >> sh) & 0xff, sc2 = (scw >> (sh + 8)) & 0xff;
+                const int m1 = (mw >> sh) & 0xff, m2 = (mw >> (sh + 8)) & 0xff;
+                int is1 = 0, is2 = 0;
+                is1 = dot4(qa.x & 0x0f0f0f0fu, a0.x, is1);
+                is1 = dot4(qa.y & 0x0f0f0f0fu, a0.y, is1);
+                is1 = dot4(qa.z & 0x0f0f0f0fu, a0.z, is1);
+                is1 = dot4(qa.w & 0x0f0f0f0fu, a0.w, is1);
+                is1 = dot4(qb.x & 0x0f0f0f0fu, a1.x, is1);
+                is1 = dot4(qb.y & 0x0f0f0f0fu, a1.y, is1);
+                is1 = dot4(qb.z & 0x0f0f0f0fu, a1.z, is1);
+                is1 = dot4(qb.w & 0x0f0f0f0fu, a1.w, is1);
+                is2 = dot4((qa.x >> 4) & 0x0f0f0f0fu, a2.x, is2);
+                is2 = dot4((qa.y >> 4) & 0x0f0f0f0fu, a2.y, is2);
+                is2 = dot4((qa.z >> 4) & 0x0f0f0f0fu, a2.z, is2);
+                is2 = dot4((qa.w >> 4) & 0x0f0f0f0fu, a2.w, is2);
+                is2 = dot4((qb.x >> 4) & 0x0f0f0f0fu, a3.x, is2);
+                is2 = dot4((qb.y >> 4) & 0x0f0f0f0fu, a3.y, is2);
+                is2 = dot4((qb.z >> 4) & 0x0f0f0f0fu, a3.z, is2);
+                is2 = dot4((qb.w >> 4) & 0x0f0f0f0fu, a3.w, is2);
+                const int s1 = sc1 * is1 + sc2 * is2;
+                const int s2 = m1 * sbs[b * 8 + 2 * p] + m2 * sbs[b * 8 + 2 * p + 1];
+                const float da = sd[b];
+                const float d = h2f(h.x & 0xffffu), dmin = h2f(h.x >> 16);
+                acc += (d * da) * (float)s1 - (dmin * da) * (float)s2;
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
+// ------------------------------------------------------------------ Q6_K x Q8_K
+// dot_q6_k_q8 (crates/frink-quant/src/lib.rs:1069-1110) over the planar resident layout.
+// Unit = (block b, half h, 16-lane column t): ql[64h+16t..], ql[64h+32+16t..], qh[32h+16t..]
+// hold four 16-weight groups with scales sc[8h+t+{0,2,4,6}].  The -32 offset is folded as
+// -32 * (sum of the 16 activation quants), which Q8_K's bsums already hold.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q6_k_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
+                                                        const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                                        const int16_t *__restrict__ absums, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    int8_t *sq = reinterpret_cast<int8_t *>(smem);
+    int *sbs = reinterpret_cast<int *>(sq + nb * 256);  // nb*16 sums over 16
+    float *sd = reinterpret_cast<float *>(sbs + nb * 16);
+    for (int i = threadIdx.x; i < nb * 16; i += 256) smem[i] = reinterpret_cast<const uint4 *>(aq)[i];
+    for (int i = threadIdx.x; i < nb * 16; i += 256) sbs[i] = (int)absums[i];
+    for (int i = threadIdx.x; i < nb; i += 256) sd[i] = ad[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const int units = nb * 4;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * lay.row_stride;
+            for (int u = l; u < units; u += LPR) {
+                const int b = u >> 2, h = (u >> 1) & 1, t = u & 1;
+                const uint4 qla = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + t * 16);
+                const uint4 qlb = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + 32 + t * 16);
+                const uint4 qh = *reinterpret_cast<const uint4 *>(row + lay.off_a + (size_t)b * 64 + h * 32 + t * 16);
+                const uint2 scv = *reinterpret_cast<const uint2 *>(row + lay.off_b + (size_t)b * 16 + h * 8);
+                const uint32_t dbits = *reinterpret_cast<const uint16_t *>(row + lay.off_c + (size_t)b * 2);
+                const int8_t *abase = sq + b * 256 + h * 128 + t * 16;
+                const uint4 a0 = *reinterpret_cast<const uint4 *>(abase);
+                const uint4 a1 = *reinterpret_cast<const uint4 *>(abase + 32);
+                const uint4 a2 = *reinterpret_cast<const uint4 *>(abase + 64);
+                const uint4 a3 = *reinterpret_cast<const uint4 *>(abase + 96);
+                const int g = b * 16 + h * 8 + t;
+                int d1 = 0, d2 = 0, d3 = 0, d4 = 0;
+#define FRK_Q6_STEP(c)                                                                                \
+    d1 = dot4((qla.c & 0x0f0f0f0fu) | ((qh.c << 4) & 0x30303030u), a0.c, d1);                         \
+    d2 = dot4((qlb.c & 0x0f0f0f0fu) | ((qh.c << 2) & 0x30303030u), a1.c, d2);                         \
+    d3 = dot4(((qla.c >> 4) & 0x0f0f0f0fu) | (qh.c & 0x30303030u), a2.c, d3);                         \
+    d4 = dot4(((qlb.c >> 4) & 0x0f0f0f0fu) | ((qh.c >> 2) & 0x30303030u), a3.c, d4);
+                FRK_Q6_STEP(x)
+                FRK_Q6_STEP(y)
+                FRK_Q6_STEP(z)
+                FRK_Q6_STEP(w)
+#undef FRK_Q6_STEP
+                const uint32_t slo = t ? (scv.x >> 8) : scv.x, shi = t ? (scv.y >> 8) : scv.y;
+                const int s1 = (int)(int8_t)(slo & 0xff), s2 = (int)(int8_t)((slo >> 16) & 0xff);
+                const int s3 = (int)(int8_t)(shi & 0xff), s4 = (int)(int8_t)((shi >> 16) & 0xff);
+                const int isum = s1 * (d1 - 32 * sbs[g]) + s2 * (d2 - 32 * sbs[g + 2]) + s3 * (d3 - 32 * sbs[g + 4]) +
+                                 s4 * (d4 - 32 * sbs[g + 6]);
+                acc += (h2f(dbits) * sd[b]) * (float)isum;
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
+// ------------------------------------------------------------------ Q8_0 x f32
+// dot_q8_0_f32 (crates/frink-quant/src/lib.rs:663-686) over the planar resident layout.
+// Unit = 16 quants (half a block); the f32 activation is staged in LDS.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q8_0_f32_kernel(const uint8_t *__restrict__ W, Layout lay, int rows,
+                                                            int nb, const float *__restrict__ x,
+                                                            float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    float *sx = reinterpret_cast<float *>(smem);
+    for (int i = threadIdx.x; i < nb * 8; i += 256) smem[i] = reinterpret_cast<const uint4 *>(x)[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const int units = nb * 2;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * lay.row_stride;
+            for (int u = l; u < units; u += LPR) {
+                const uint4 qv = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+                const float scale = h2f(*reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2));
+                const float4 *xv = reinterpret_cast<const float4 *>(sx + u * 16);
+                float s = 0.0f;
+#define FRK_Q8_STEP(c, k)                                                  \
+    {                                                                      \
+        const float4 xx = xv[k];                                           \
+        s = fmaf((float)(int8_t)(qv.c & 0xff), xx.x, s);                   \
+        s = fmaf((float)(int8_t)((qv.c >> 8) & 0xff), xx.y, s);            \
+        s = fmaf((float)(int8_t)((qv.c >> 16) & 0xff), xx.z, s);           \
+        s = fmaf((float)(int8_t)(qv.c >> 24), xx.w, s);                    \
+    }
+                FRK_Q8_STEP(x, 0)
+                FRK_Q8_STEP(y, 1)
+                FRK_Q8_STEP(z, 2)
+                FRK_Q8_STEP(w, 3)
+#undef FRK_Q8_STEP
+                acc = fmaf(s, scale, acc);
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
+// ------------------------------------------------------------------ Q8_0 x Q8_0
+// dot_q8_0_q8 (crates/frink-quant/src/lib.rs:711-733).  Unit = 16 quants.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q8_0_q8_kernel(const uint8_t *__restrict__ W, Layout lay, int rows,
+                                                           int nb, const int8_t *__restrict__ aq,
+                                                           const float *__restrict__ ad, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    float *sd = reinterpret_cast<float *>(smem + nb * 2);
+    for (int i = threadIdx.x; i < nb * 2; i += 256) smem[i] = reinterpret_cast<const uint4 *>(aq)[i];
+    for (int i = threadIdx.x; i < nb; i += 256) sd[i] = ad[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const int units = nb * 2;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * lay.row_stride;
+            for (int u = l; u < units; u += LPR) {
+                const uint4 qv = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+                const float dw = h2f(*reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2));
+                const uint4 a = smem[u];
+                int isum = dot4(qv.x, a.x, 0);
+                isum = dot4(qv.y, a.y, isum);
+                isum = dot4(qv.z, a.z, isum);
+                isum = dot4(qv.w, a.w, isum);
+                acc += (dw * sd[u >> 1]) * (float)isum;
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
+// ------------------------------------------------------------------ launchers
+
+static int lanes_per_row(int units) { return units > 32 ? 64 : units > 16 ? 32 : 16; }
+
+static unsigned gemv_grid(size_t rows, int lpr) {
+    // enough 4-wave workgroups that each wave owns two rows; never more than 16 per CU's worth
+    const size_t rows_per_wg = 4 * (size_t)(64 / lpr) * 2;
+    size_t g = (rows + rows_per_wg - 1) / rows_per_wg;
+    if (g > 4096) g = 4096;
+    if (g < 1) g = 1;
+    return (unsigned)g;
+}
+
+#define FRK_LAUNCH_CHECK(what)                                                                          \
+    do {                                                                                                \
+        hipError_t e_ = hipGetLastError();                                                              \
+        if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
+    } while (0)
+
+#define FRK_DISPATCH_LPR(lpr, KERNEL, grid, shmem, s, ...)                                             \
+    do {                                                                                                \
+        if ((shmem) > 64 * 1024)                                                                        \
+            return set_error(FRK_ERR_SHAPE, "activation of this width needs %zu bytes of LDS (limit 65536)", \
+                             (size_t)(shmem));                                                          \
+        if (lpr == 64) hipLaunchKernelGGL(KERNEL<64>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__);    \
+        else if (lpr == 32) hipLaunchKernelGGL(KERNEL<32>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__); \
+        else hipLaunchKernelGGL(KERNEL<16>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__);              \
+    } while (0)
+
+int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    const int lpr = lanes_per_row(nb * 4);
+    const size_t shmem = (size_t)nb * (256 + 8 * 4 + 4);
+    FRK_DISPATCH_LPR(lpr, gemv_q4_k_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout.row_stride,
+                     (int)w->rows, nb, a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("gemv_q4_k");
+    return FRK_OK;
+}
+
+int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    const int lpr = lanes_per_row(nb * 4);
+    const size_t shmem = (size_t)nb * (256 + 16 * 4 + 4);
+    FRK_DISPATCH_LPR(lpr, gemv_q6_k_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows, nb,
+                     a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("gemv_q6_k");
+    return FRK_OK;
+}
+
+int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS);
+    const int lpr = lanes_per_row(nb * 2);
+    const size_t shmem = (size_t)nb * 32 * 4;
+    FRK_DISPATCH_LPR(lpr, gemv_q8_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+                     nb, x, y);
+    FRK_LAUNCH_CHECK("gemv_q8_0_f32");
+    return FRK_OK;
+}
+
+int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS);
+    const int lpr = lanes_per_row(nb * 2);
+    const size_t shmem = (size_t)nb * (32 + 4);
+    FRK_DISPATCH_LPR(lpr, gemv_q8_0_q8_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+                     nb, q, d, y);
+    FRK_LAUNCH_CHECK("gemv_q8_0_q8");
+    return FRK_OK;
+}
+
+}  // namespace frk

@@ -1,0 +1,121 @@
+// Shared internals of libfrink_hip: error plumbing, the weights handle, kernel launchers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/frink_hip.h"
+
+namespace frk {
+
+// ---- errors ----
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+#define FRK_HIP_TRY(expr)                                                                     \
+    do {                                                                                      \
+        hipError_t e_ = (expr);                                                               \
+        if (e_ != hipSuccess)                                                                 \
+            return frk::set_error(e_ == hipErrorOutOfMemory ? FRK_ERR_OOM : FRK_ERR_HIP,      \
+                                  "%s failed: %s", #expr, hipGetErrorString(e_));             \
+    } while (0)
+
+// ---- block geometry ----
+constexpr int QK_K = 256;
+constexpr int Q8_0_BYTES = 34, Q8_0_ELEMS = 32;
+constexpr int Q4_K_BYTES = 144;
+constexpr int Q6_K_BYTES = 210;
+
+inline int block_bytes(int kind) {
+    return kind == FRK_KIND_Q8_0 ? Q8_0_BYTES : kind == FRK_KIND_Q4_K ? Q4_K_BYTES
+         : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : 0;
+}
+inline int block_elems(int kind) {
+    return kind == FRK_KIND_Q8_0 ? Q8_0_ELEMS : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K) ? QK_K : 0;
+}
+
+// ---- resident layouts ----
+// Q4_K stays verbatim: a 144-byte block is nine 16-byte words (header + 8 words of nibbles)
+// and every row starts 16-byte aligned.
+// Q6_K (210-byte blocks, 2-byte aligned) and Q8_0 (34-byte blocks) are permuted per row into
+// planes so every load is a 16-byte word:
+//   Q6_K row of nb blocks: ql[nb][128] | qh[nb][64] | sc[nb][16] | d[nb] f16, padded to 16
+//   Q8_0 row of nb blocks: qs[nb][32] | d[nb] f16, padded to 16
+// Same bytes, same count per block; only their order changes.
+struct Layout {
+    size_t row_stride = 0;  // bytes between resident rows
+    size_t off_a = 0;       // Q6_K: qh plane offset in a row; Q8_0: d plane offset
+    size_t off_b = 0;       // Q6_K: sc plane offset
+    size_t off_c = 0;       // Q6_K: d plane offset
+};
+
+inline size_t round_up(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+inline Layout layout_for(int kind, size_t cols) {
+    Layout l;
+    size_t nb = cols / (size_t)block_elems(kind);
+    if (kind == FRK_KIND_Q4_K) {
+        l.row_stride = nb * Q4_K_BYTES;
+    } else if (kind == FRK_KIND_Q6_K) {
+        l.off_a = nb * 128;
+        l.off_b = l.off_a + nb * 64;
+        l.off_c = l.off_b + nb * 16;
+        l.row_stride = round_up(l.off_c + nb * 2, 16);
+    } else if (kind == FRK_KIND_Q8_0) {
+        l.off_a = nb * 32;
+        l.row_stride = round_up(l.off_a + nb * 2, 16);
+    }
+    return l;
+}
+
+}  // namespace frk
+
+// The handle behind frk_weights.
+struct frk_weights {
+    int kind = 0;
+    size_t rows = 0, cols = 0;
+    size_t src_row_bytes = 0;  // GGUF bytes per row
+    frk::Layout layout;
+    uint8_t *dev = nullptr;    // resident copy (library-owned)
+    size_t dev_bytes = 0;
+    int device = 0;
+    // residency-cache identity (host pointer, length, sampled bytes)
+    const void *host_key = nullptr;
+    size_t host_len = 0;
+    uint8_t fingerprint[192] = {0};
+    int refcount = 1;
+    bool cached = false;
+};
+
+namespace frk {
+
+// ---- per-device scratch the library owns (quantized activations etc.) ----
+// Returns a buffer of at least `bytes` on the current device, growing it if needed.
+// Grown with the stream idle (hipStreamSynchronize) so no kernel still reads the old one.
+int workspace(size_t bytes, hipStream_t stream, void **out);
+hipStream_t own_stream();  // the stream host-buffer entry points run on
+
+// ---- launchers (each validates nothing: callers have checked shapes) ----
+int launch_quantize_q8_k(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s);
+int launch_quantize_q8_0(const float *x, size_t n, int8_t *q, float *d, hipStream_t s);
+int launch_dequant(const frk_weights *w, float *out, hipStream_t s);
+int launch_repack(int kind, const uint8_t *src, uint8_t *dst, size_t rows, size_t cols, const Layout &l,
+                  hipStream_t s);
+int launch_copy(const void *src, void *dst, size_t bytes, hipStream_t s);
+int launch_read(const void *src, size_t bytes, void *sink, hipStream_t s);
+
+struct Q8KActs {  // Q8_K activations in HBM, struct-of-arrays per activation row
+    const int8_t *q;      // [batch][cols]
+    const float *d;       // [batch][cols/256]
+    const int16_t *bsums; // [batch][cols/16]
+};
+int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
+
+}  // namespace frk

@@ -1,0 +1,481 @@
+// Host runtime of libfrink_hip: error strings, device probe, the env switch, the resident
+// weight cache, the per-device workspace and the extern "C" entry points.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <utility>
+
+#include "frk_internal.hpp"
+
+namespace frk {
+
+static thread_local char g_err[512] = {0};
+
+int set_error(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+void clear_error() { g_err[0] = 0; }
+
+// ---- device state ----
+struct DeviceState {
+    std::mutex mu;
+    bool probed = false;
+    int device_count = 0;
+    hipStream_t stream = nullptr;  // for host-buffer entry points
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    // host staging for the host-buffer entry points
+    void *x_dev = nullptr, *y_dev = nullptr;
+    size_t x_bytes = 0, y_bytes = 0;
+    std::map<std::pair<const void *, size_t>, frk_weights *> cache;
+};
+static DeviceState g_dev;
+
+static int ensure_device_locked() {
+    if (!g_dev.probed) {
+        int n = 0;
+        hipError_t e = hipGetDeviceCount(&n);
+        g_dev.probed = true;
+        g_dev.device_count = (e == hipSuccess) ? n : 0;
+        if (e != hipSuccess) (void)hipGetLastError();
+    }
+    if (g_dev.device_count <= 0) return set_error(FRK_ERR_NO_DEVICE, "no HIP device is visible");
+    if (!g_dev.stream) {
+        // default priority on purpose
+        hipError_t e = hipStreamCreateWithFlags(&g_dev.stream, hipStreamNonBlocking);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipStreamCreateWithFlags: %s", hipGetErrorString(e));
+    }
+    return FRK_OK;
+}
+
+hipStream_t own_stream() { return g_dev.stream; }
+
+int workspace(size_t bytes, hipStream_t stream, void **out) {
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    if (bytes > g_dev.ws_bytes) {
+        if (g_dev.ws) {
+            FRK_HIP_TRY(hipDeviceSynchronize());
+            FRK_HIP_TRY(hipFree(g_dev.ws));
+            g_dev.ws = nullptr;
+            g_dev.ws_bytes = 0;
+        }
+        size_t want = std::max<size_t>(round_up(bytes, 1 << 20), 4u << 20);
+        FRK_HIP_TRY(hipMalloc(&g_dev.ws, want));
+        g_dev.ws_bytes = want;
+    }
+    (void)stream;
+    *out = g_dev.ws;
+    return FRK_OK;
+}
+
+static void fingerprint_of(const uint8_t *bytes, size_t len, uint8_t out[192]) {
+    // first, middle and last 64 bytes (crates/frink-quant/src/fingerprint.rs:17-40)
+    auto take = [&](size_t at, uint8_t *dst) {
+        memset(dst, 0, 64);
+        at = std::min(at, len);
+        size_t n = std::min<size_t>(len - at, 64);
+        memcpy(dst, bytes + at, n);
+    };
+    take(0, out);
+    take(len / 2, out + 64);
+    take(len >= 64 ? len - 64 : 0, out + 128);
+}
+
+static int check_matrix_shape(int kind, size_t len, size_t rows, size_t cols) {
+    int be = block_elems(kind), bb = block_bytes(kind);
+    if (!be) return set_error(FRK_ERR_UNSUPPORTED, "no kernel for quant kind %d", kind);
+    if (rows == 0 || cols == 0) return set_error(FRK_ERR_SHAPE, "empty shape: rows=%zu cols=%zu", rows, cols);
+    if (cols % (size_t)be) return set_error(FRK_ERR_SHAPE, "cols %zu is not a multiple of the %d-element block", cols, be);
+    size_t want = rows * (cols / (size_t)be) * (size_t)bb;
+    if (len != want) return set_error(FRK_ERR_SHAPE, "weights are %zu bytes, shape %zux%zu needs %zu", len, rows, cols, want);
+    if (rows > 0x7fffffffu || cols > 0x7fffffffu) return set_error(FRK_ERR_SHAPE, "shape too large");
+    return FRK_OK;
+}
+
+// Creates the resident copy from GGUF bytes already on the device.
+static int make_resident(int kind, const uint8_t *src_dev, size_t rows, size_t cols, hipStream_t s,
+                         frk_weights **out) {
+    auto *w = new frk_weights();
+    w->kind = kind;
+    w->rows = rows;
+    w->cols = cols;
+    w->src_row_bytes = cols / (size_t)block_elems(kind) * (size_t)block_bytes(kind);
+    w->layout = layout_for(kind, cols);
+    // 256 bytes of slack: kernels may issue (masked-out or clamped) 16-byte loads near the end
+    w->dev_bytes = w->layout.row_stride * rows + 256;
+    (void)hipGetDevice(&w->device);
+    hipError_t e = hipMalloc((void **)&w->dev, w->dev_bytes);
+    if (e != hipSuccess) {
+        delete w;
+        return set_error(FRK_ERR_OOM, "hipMalloc(%zu) for resident weights: %s", w->dev_bytes, hipGetErrorString(e));
+    }
+    int rc = launch_repack(kind, src_dev, w->dev, rows, cols, w->layout, s);
+    if (rc == FRK_OK) {
+        e = hipMemsetAsync(w->dev + w->layout.row_stride * rows, 0, 256, s);
+        if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
+    }
+    if (rc != FRK_OK) {
+        (void)hipFree(w->dev);
+        delete w;
+        return rc;
+    }
+    *out = w;
+    return FRK_OK;
+}
+
+}  // namespace frk
+
+using namespace frk;
+
+extern "C" {
+
+const char *frk_hip_last_error(void) { return g_err; }
+
+int frk_hip_probe(frk_device_info *out) {
+    clear_error();
+    if (!out) return set_error(FRK_ERR_ARG, "frk_hip_probe: out is null");
+    memset(out, 0, sizeof *out);
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    int rc = ensure_device_locked();
+    if (rc) return rc;
+    out->device_count = g_dev.device_count;
+    hipDeviceProp_t p;
+    FRK_HIP_TRY(hipGetDeviceProperties(&p, 0));
+    snprintf(out->name, sizeof out->name, "%s", p.name);
+    snprintf(out->gcn_arch, sizeof out->gcn_arch, "%s", p.gcnArchName);
+    out->compute_units = p.multiProcessorCount;
+    size_t fr = 0, tot = 0;
+    FRK_HIP_TRY(hipMemGetInfo(&fr, &tot));
+    out->free_vram_bytes = fr;
+    out->total_vram_bytes = tot;
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return set_error(FRK_ERR_NO_DEVICE, "device 0 is %s; this library holds gfx950 code only", p.gcnArchName);
+    return FRK_OK;
+}
+
+int frk_hip_dense_enabled(void) {
+    static std::once_flag once;
+    static int enabled = 0;
+    std::call_once(once, [] {
+        const char *v = getenv("FRINK_HIP");
+        std::string s = v ? v : "";
+        std::transform(s.begin(), s.end(), s.begin(), [](unsigned char c) { return (char)tolower(c); });
+        if (s == "0" || s == "false" || s == "off" || s == "cpu") {
+            enabled = 0;  // forced off: no device is opened
+            return;
+        }
+        frk_device_info info;
+        int rc = frk_hip_probe(&info);
+        enabled = (rc == FRK_OK);
+        clear_error();
+    });
+    return enabled;
+}
+
+const char *frk_hip_matvec_kernel(int kind) {
+    switch (kind) {
+    case FRK_KIND_Q8_0: return "Q8_0";
+    case FRK_KIND_Q4_K: return "Q4_K";
+    case FRK_KIND_Q6_K: return "Q6_K";
+    }
+    return nullptr;
+}
+int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
+int frk_hip_gemm_supported(int kind) { return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K; }
+int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
+int frk_hip_block_elems(int kind) { return block_elems(kind); }
+int frk_hip_worth_a_gemm(size_t batch) { return batch >= 2; }
+
+int frk_hip_weights_register(int kind, const void *host_bytes, size_t len, size_t rows, size_t cols,
+                             frk_weights **out) {
+    clear_error();
+    if (!host_bytes || !out) return set_error(FRK_ERR_ARG, "frk_hip_weights_register: null argument");
+    int rc = check_matrix_shape(kind, len, rows, cols);
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    rc = ensure_device_locked();
+    if (rc) return rc;
+    uint8_t fp[192];
+    fingerprint_of((const uint8_t *)host_bytes, len, fp);
+    auto key = std::make_pair(host_bytes, len);
+    auto it = g_dev.cache.find(key);
+    if (it != g_dev.cache.end()) {
+        frk_weights *c = it->second;
+        if (c->kind == kind && c->rows == rows && c->cols == cols && memcmp(c->fingerprint, fp, 192) == 0) {
+            c->refcount++;
+            *out = c;
+            return FRK_OK;
+        }
+        // same address and length, different bytes: the buffer that entry came from is gone
+        g_dev.cache.erase(it);
+        c->cached = false;
+        if (--c->refcount == 0) {
+            (void)hipFree(c->dev);
+            delete c;
+        }
+    }
+    uint8_t *staging = nullptr;
+    FRK_HIP_TRY(hipMalloc((void **)&staging, len));
+    hipError_t e = hipMemcpyAsync(staging, host_bytes, len, hipMemcpyHostToDevice, g_dev.stream);
+    frk_weights *w = nullptr;
+    if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(weights): %s", hipGetErrorString(e));
+    if (!rc) rc = make_resident(kind, staging, rows, cols, g_dev.stream, &w);
+    hipError_t e2 = hipStreamSynchronize(g_dev.stream);
+    (void)hipFree(staging);
+    if (!rc && e2 != hipSuccess) {
+        rc = set_error(FRK_ERR_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e2));
+        (void)hipFree(w->dev);
+        delete w;
+    }
+    if (rc) return rc;
+    w->host_key = host_bytes;
+    w->host_len = len;
+    memcpy(w->fingerprint, fp, 192);
+    w->cached = true;
+    w->refcount = 2;  // one for the cache, one for the caller
+    g_dev.cache[key] = w;
+    *out = w;
+    return FRK_OK;
+}
+
+int frk_hip_weights_from_device(int kind, const void *dev_bytes, size_t len, size_t rows, size_t cols,
+                                void *stream, frk_weights **out) {
+    clear_error();
+    if (!dev_bytes || !out) return set_error(FRK_ERR_ARG, "frk_hip_weights_from_device: null argument");
+    int rc = check_matrix_shape(kind, len, rows, cols);
+    if (rc) return rc;
+    {
+        std::lock_guard<std::mutex> lk(g_dev.mu);
+        rc = ensure_device_locked();
+        if (rc) return rc;
+    }
+    return make_resident(kind, (const uint8_t *)dev_bytes, rows, cols, (hipStream_t)stream, out);
+}
+
+int frk_hip_weights_release(frk_weights *w) {
+    clear_error();
+    if (!w) return FRK_OK;
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    if (--w->refcount > 0) {
+        // the cache keeps its own reference until the process ends or the bytes change
+        return FRK_OK;
+    }
+    if (w->cached) g_dev.cache.erase(std::make_pair(w->host_key, w->host_len));
+    hipError_t e = hipFree(w->dev);
+    delete w;
+    if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFree: %s", hipGetErrorString(e));
+    return FRK_OK;
+}
+
+size_t frk_hip_weights_rows(const frk_weights *w) { return w ? w->rows : 0; }
+size_t frk_hip_weights_cols(const frk_weights *w) { return w ? w->cols : 0; }
+int frk_hip_weights_kind(const frk_weights *w) { return w ? w->kind : 0; }
+
+// ---- device-pointer entry points ----
+
+int frk_hip_quantize_q8_k_dev(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums, void *stream) {
+    clear_error();
+    if (!x || !q || !d || !bsums) return set_error(FRK_ERR_ARG, "frk_hip_quantize_q8_k_dev: null argument");
+    if (n % QK_K) return set_error(FRK_ERR_SHAPE, "length %zu is not a multiple of 256", n);
+    if (n == 0) return FRK_OK;
+    return launch_quantize_q8_k(x, n, q, d, bsums, (hipStream_t)stream);
+}
+
+int frk_hip_quantize_q8_0_dev(const float *x, size_t n, int8_t *q, float *d, void *stream) {
+    clear_error();
+    if (!x || !q || !d) return set_error(FRK_ERR_ARG, "frk_hip_quantize_q8_0_dev: null argument");
+    if (n % Q8_0_ELEMS) return set_error(FRK_ERR_SHAPE, "length %zu is not a multiple of 32", n);
+    if (n == 0) return FRK_OK;
+    return launch_quantize_q8_0(x, n, q, d, (hipStream_t)stream);
+}
+
+int frk_hip_dequant_dev(const frk_weights *w, float *out, void *stream) {
+    clear_error();
+    if (!w || !out) return set_error(FRK_ERR_ARG, "frk_hip_dequant_dev: null argument");
+    return launch_dequant(w, out, (hipStream_t)stream);
+}
+
+int frk_hip_copy_dev(const void *src, void *dst, size_t bytes, void *stream) {
+    clear_error();
+    if (!src || !dst) return set_error(FRK_ERR_ARG, "frk_hip_copy_dev: null argument");
+    if (bytes % 16) return set_error(FRK_ERR_SHAPE, "bytes %zu is not a multiple of 16", bytes);
+    return launch_copy(src, dst, bytes, (hipStream_t)stream);
+}
+
+int frk_hip_read_dev(const void *src, size_t bytes, void *sink, void *stream) {
+    clear_error();
+    if (!src || !sink) return set_error(FRK_ERR_ARG, "frk_hip_read_dev: null argument");
+    if (bytes % 16) return set_error(FRK_ERR_SHAPE, "bytes %zu is not a multiple of 16", bytes);
+    return launch_read(src, bytes, sink, (hipStream_t)stream);
+}
+
+// Quantizes `batch` activation rows of w->cols values to Q8_K in the workspace.
+static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch, hipStream_t s, Q8KActs *a) {
+    size_t n = batch * w->cols;
+    size_t q_bytes = round_up(n, 256), d_bytes = round_up(n / QK_K * 4, 256), b_bytes = round_up(n / 16 * 2, 256);
+    void *ws = nullptr;
+    int rc = workspace(q_bytes + d_bytes + b_bytes, s, &ws);
+    if (rc) return rc;
+    int8_t *q = (int8_t *)ws;
+    float *d = (float *)((char *)ws + q_bytes);
+    int16_t *b = (int16_t *)((char *)ws + q_bytes + d_bytes);
+    rc = launch_quantize_q8_k(x, n, q, d, b, s);
+    if (rc) return rc;
+    a->q = q;
+    a->d = d;
+    a->bsums = b;
+    return FRK_OK;
+}
+
+int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mode, void *stream) {
+    clear_error();
+    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_dev: null argument");
+    hipStream_t s = (hipStream_t)stream;
+    switch (w->kind) {
+    case FRK_KIND_Q4_K:
+    case FRK_KIND_Q6_K: {
+        Q8KActs a;
+        int rc = quantize_acts_q8_k(w, x, 1, s, &a);
+        if (rc) return rc;
+        return w->kind == FRK_KIND_Q4_K ? launch_gemv_q4_k(w, a, y, s) : launch_gemv_q6_k(w, a, y, s);
+    }
+    case FRK_KIND_Q8_0: {
+        if (act_mode == FRK_ACT_F32) return launch_gemv_q8_0_f32(w, x, y, s);
+        size_t n = w->cols;
+        void *ws = nullptr;
+        int rc = workspace(round_up(n, 256) + n / 32 * 4, s, &ws);
+        if (rc) return rc;
+        int8_t *q = (int8_t *)ws;
+        float *d = (float *)((char *)ws + round_up(n, 256));
+        rc = launch_quantize_q8_0(x, n, q, d, s);
+        if (rc) return rc;
+        return launch_gemv_q8_0_q8(w, q, d, y, s);
+    }
+    }
+    return set_error(FRK_ERR_UNSUPPORTED, "no matvec kernel for quant kind %d", w->kind);
+}
+
+int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, const int16_t *bsums, float *y,
+                         void *stream) {
+    clear_error();
+    if (!w || !q || !d || !bsums || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_q8k_dev: null argument");
+    Q8KActs a{q, d, bsums};
+    if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
+    if (w->kind == FRK_KIND_Q6_K) return launch_gemv_q6_k(w, a, y, (hipStream_t)stream);
+    return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K and Q6_K weights only (kind %d)", w->kind);
+}
+
+int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *y, void *stream) {
+    clear_error();
+    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
+    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+    // first slice: one matvec per activation row (the reference's own path below its GEMM threshold,
+    // crates/frink-core/src/weight_matrix.rs:2636-2652)
+    for (size_t b = 0; b < batch; b++) {
+        int rc = frk_hip_gemv_dev(w, x + b * w->cols, y + b * w->rows, FRK_ACT_F32, stream);
+        if (rc) return rc;
+    }
+    return FRK_OK;
+}
+
+// ---- host-buffer entry points ----
+
+static int stage_buffers(size_t x_bytes, size_t y_bytes) {
+    if (x_bytes > g_dev.x_bytes) {
+        if (g_dev.x_dev) (void)hipFree(g_dev.x_dev);
+        g_dev.x_dev = nullptr;
+        g_dev.x_bytes = 0;
+        FRK_HIP_TRY(hipMalloc(&g_dev.x_dev, round_up(x_bytes, 1 << 16)));
+        g_dev.x_bytes = round_up(x_bytes, 1 << 16);
+    }
+    if (y_bytes > g_dev.y_bytes) {
+        if (g_dev.y_dev) (void)hipFree(g_dev.y_dev);
+        g_dev.y_dev = nullptr;
+        g_dev.y_bytes = 0;
+        FRK_HIP_TRY(hipMalloc(&g_dev.y_dev, round_up(y_bytes, 1 << 16)));
+        g_dev.y_bytes = round_up(y_bytes, 1 << 16);
+    }
+    return FRK_OK;
+}
+
+// One mutex serialises the host-buffer entry points: they share the staging buffers and the
+// library's stream, and the reference calls them from many worker threads at once
+// (crates/frink-core/src/weight_matrix/gpu_backend.rs:722-725).
+static std::mutex g_launch_mu;
+
+static int host_launch(int kind, const uint8_t *weights, size_t weights_len, const float *x, size_t rows,
+                       size_t cols, size_t batch, float *out) {
+    frk_weights *w = nullptr;
+    int rc = frk_hip_weights_register(kind, weights, weights_len, rows, cols, &w);
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lk(g_launch_mu);
+    size_t xb = batch * cols * sizeof(float), yb = batch * rows * sizeof(float);
+    rc = stage_buffers(xb, yb);
+    hipStream_t s = g_dev.stream;
+    if (!rc) {
+        hipError_t e = hipMemcpyAsync(g_dev.x_dev, x, xb, hipMemcpyHostToDevice, s);
+        if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(x): %s", hipGetErrorString(e));
+    }
+    if (!rc)
+        rc = batch == 1 ? frk_hip_gemv_dev(w, (const float *)g_dev.x_dev, (float *)g_dev.y_dev, FRK_ACT_F32, s)
+                        : frk_hip_gemm_dev(w, (const float *)g_dev.x_dev, batch, (float *)g_dev.y_dev, s);
+    if (!rc) {
+        hipError_t e = hipMemcpyAsync(out, g_dev.y_dev, yb, hipMemcpyDeviceToHost, s);
+        if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(y): %s", hipGetErrorString(e));
+    }
+    hipError_t e = hipStreamSynchronize(s);
+    if (!rc && e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e));
+    char keep[sizeof g_err];
+    memcpy(keep, g_err, sizeof keep);
+    frk_hip_weights_release(w);
+    memcpy(g_err, keep, sizeof keep);
+    return rc;
+}
+
+int frk_hip_launch_matvec(int kind, const uint8_t *weights, size_t weights_len, const float *x, size_t x_len,
+                          size_t rows, size_t row_bytes, float *out) {
+    clear_error();
+    if (!frk_hip_has_launch(kind)) return set_error(FRK_ERR_UNSUPPORTED, "no matvec kernel for quant kind %d", kind);
+    if (!weights || !x || !out) return set_error(FRK_ERR_ARG, "frk_hip_launch_matvec: null argument");
+    size_t bb = (size_t)block_bytes(kind), be = (size_t)block_elems(kind);
+    if (rows == 0) return set_error(FRK_ERR_SHAPE, "empty shape: rows=0");
+    if (row_bytes == 0 || row_bytes % bb)
+        return set_error(FRK_ERR_SHAPE, "row_bytes %zu is not a whole number of %zu-byte %s blocks", row_bytes, bb,
+                         frk_hip_matvec_kernel(kind));
+    size_t nb = row_bytes / bb;
+    if (weights_len != rows * row_bytes)
+        return set_error(FRK_ERR_SHAPE, "weights are %zu bytes, %zu rows of %zu bytes need %zu", weights_len, rows,
+                         row_bytes, rows * row_bytes);
+    if (x_len != nb * be)
+        return set_error(FRK_ERR_SHAPE, "activation has %zu values, %zu blocks of %zu need %zu", x_len, nb, be, nb * be);
+    return host_launch(kind, weights, weights_len, x, rows, nb * be, 1, out);
+}
+
+int frk_hip_launch_mul_mm(int kind, const uint8_t *weights, size_t weights_len, const float *x_batch, size_t x_len,
+                          size_t n_rows, size_t n_cols, size_t batch, size_t row_bytes, float *out) {
+    clear_error();
+    if (!frk_hip_has_launch(kind)) return set_error(FRK_ERR_UNSUPPORTED, "no GEMM kernel for quant kind %d", kind);
+    if (!weights || !x_batch || !out) return set_error(FRK_ERR_ARG, "frk_hip_launch_mul_mm: null argument");
+    size_t bb = (size_t)block_bytes(kind), be = (size_t)block_elems(kind);
+    if (n_rows == 0 || n_cols == 0 || batch == 0)
+        return set_error(FRK_ERR_SHAPE, "empty shape: rows=%zu cols=%zu batch=%zu", n_rows, n_cols, batch);
+    if (n_cols % be)
+        return set_error(FRK_ERR_SHAPE, "cols %zu is not a multiple of the %zu-element %s block", n_cols, be,
+                         frk_hip_matvec_kernel(kind));
+    size_t expect = n_cols / be * bb;
+    if (row_bytes != expect) return set_error(FRK_ERR_SHAPE, "row_bytes %zu, expected %zu", row_bytes, expect);
+    if (weights_len < n_rows * row_bytes)
+        return set_error(FRK_ERR_SHAPE, "weights too small: got %zu bytes, want %zu", weights_len, n_rows * row_bytes);
+    if (x_len < batch * n_cols)
+        return set_error(FRK_ERR_SHAPE, "activations too small: got %zu values, want %zu", x_len, batch * n_cols);
+    return host_launch(kind, weights, n_rows * row_bytes, x_batch, n_rows, n_cols, batch, out);
+}
+
+}  // extern "C"

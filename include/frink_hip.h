@@ -1,0 +1,170 @@
+/*
+ * frink_hip.h -- C ABI of the MI355X (gfx950) quantized-matmul backend for Frink.
+ *
+ * What a `frink-hip` backend crate binds: plain pointers and sizes, an int
+ * status, a thread-local error string.  No function here panics, aborts or
+ * throws across the boundary; shapes are validated before any kernel is
+ * launched (the reference's seam contract: a failed launch is an error value
+ * the caller logs before falling back, crates/frink-core/src/weight_matrix/
+ * gpu_backend.rs:185-194, 676-703).
+ *
+ * Layouts are the reference's: quantized weights are verbatim GGUF block
+ * bytes, row-major, one row = cols/block_elems consecutive blocks, no padding
+ * (crates/frink-core/src/weight_matrix.rs:978-1052); activations are
+ * [batch][cols] f32; outputs are [batch][rows] f32 (weight_matrix.rs:2310-2316,
+ * crates/frink-cuda/src/mul_mm_launch.rs:34-35).
+ *
+ * Two families of entry points:
+ *   frk_hip_launch_*   host buffers in, host buffers out: the drop-in for the
+ *                      reference's per-backend launch functions.  Weights are
+ *                      kept resident on the device between calls.
+ *   frk_hip_*_dev      operands already in HBM, asynchronous on a caller's
+ *                      stream: what a resident decode/prefill stack and the
+ *                      benchmark use.
+ */
+#ifndef FRINK_HIP_H
+#define FRINK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes.  0 is success; negative values are errors and
+ * frk_hip_last_error() holds the message. */
+enum {
+    FRK_OK = 0,
+    FRK_ERR_NO_DEVICE = -1,   /* no usable gfx950 device, or the backend is switched off */
+    FRK_ERR_UNSUPPORTED = -2, /* no kernel for this quant kind: the reference's `None` */
+    FRK_ERR_SHAPE = -3,       /* shape/length violation caught before launch */
+    FRK_ERR_ARG = -4,         /* null pointer or otherwise unusable argument */
+    FRK_ERR_HIP = -5,         /* a HIP runtime call failed: the reference's `Some(Err)` */
+    FRK_ERR_OOM = -6
+};
+
+/* Quant kinds, numbered by ggml type id (crates/frink-gguf/src/lib.rs:236-242).
+ * Names are QuantKind::name() (crates/frink-core/src/weight_matrix.rs:264-290). */
+enum { FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q6_K = 14 };
+
+/* Q8_0 GEMV arithmetic.  F32 multiplies dequantized weights by the f32
+ * activation (dot_q8_0_f32, crates/frink-quant/src/lib.rs:663-686); INT8
+ * quantizes the activation to Q8_0 blocks first (dot_q8_0_q8, lib.rs:711-733,
+ * activation form Avx of crates/frink-quant/src/act_quant.rs:157-189).  The
+ * K-quants always take the integer path against Q8_K activations
+ * (dot_q4_k_q8 lib.rs:822-869, dot_q6_k_q8 lib.rs:1069-1110). */
+enum { FRK_ACT_F32 = 0, FRK_ACT_INT8 = 1 };
+
+typedef struct frk_weights frk_weights; /* opaque: one weight matrix resident in HBM */
+
+/* replaces frink_cuda::gpu::probe / CudaInfo (crates/frink-cuda/src/gpu.rs:79-145) */
+typedef struct {
+    int32_t device_count;
+    int32_t compute_units;
+    char name[128];      /* first device's marketing name */
+    char gcn_arch[64];   /* e.g. "gfx950:sramecc+:xnack-" */
+    uint64_t total_vram_bytes;
+    uint64_t free_vram_bytes;
+} frk_device_info;
+
+/* Never aborts on a GPU-less host: returns FRK_ERR_NO_DEVICE there. */
+int frk_hip_probe(frk_device_info *out);
+
+/* BackendDispatch::dense_enabled (gpu_backend.rs:153-195): env FRINK_HIP with the
+ * reference's grammar (0|false|off|cpu = off without opening a device,
+ * 1|true|on|hip|rocm = on, anything else = probe; gpu_backend.rs:545-552).
+ * Decided once per process. */
+int frk_hip_dense_enabled(void);
+
+/* Message of the last error on the calling thread ("" if none). */
+const char *frk_hip_last_error(void);
+
+/* BackendCaps::matvec_kernel / gemm_supported / BackendDispatch::has_launch
+ * (gpu_backend.rs:110-150, 153-195).  matvec_kernel returns the kind's name
+ * ("Q8_0", "Q4_K", "Q6_K") or NULL when there is no decode kernel. */
+const char *frk_hip_matvec_kernel(int kind);
+int frk_hip_gemm_supported(int kind);
+int frk_hip_has_launch(int kind);
+/* block geometry (crates/frink-gguf/src/lib.rs:308-314); 0 for an unknown kind */
+int frk_hip_block_bytes(int kind);
+int frk_hip_block_elems(int kind);
+/* worth_a_gemm (crates/frink-cuda/src/mul_mm.rs:634-638): batch sizes the GEMM entry
+ * point should take rather than `batch` matvecs.  Here every batch >= 2 qualifies. */
+int frk_hip_worth_a_gemm(size_t batch);
+
+/* ---- resident weights (crates/frink-cuda/src/resident.rs:1-120) ----
+ * register: uploads `len` bytes of GGUF blocks (borrowed for the duration of the
+ * call) and returns a handle.  A later register of the same (pointer, len) whose
+ * 192 sampled bytes (first, middle, last 64) still match returns the cached
+ * handle; a mismatch re-uploads.  Q6_K and Q8_0 are byte-permuted once into
+ * 16-byte-aligned planes on the device; dequantization is bit-identical. */
+int frk_hip_weights_register(int kind, const void *host_bytes, size_t len, size_t rows,
+                             size_t cols, frk_weights **out);
+/* Same, from `len` bytes of GGUF blocks already in device memory (copied/permuted
+ * into the library's own allocation; the source may be freed afterwards). */
+int frk_hip_weights_from_device(int kind, const void *dev_bytes, size_t len, size_t rows,
+                                size_t cols, void *stream, frk_weights **out);
+int frk_hip_weights_release(frk_weights *w);
+size_t frk_hip_weights_rows(const frk_weights *w);
+size_t frk_hip_weights_cols(const frk_weights *w);
+int frk_hip_weights_kind(const frk_weights *w);
+
+/* ---- host-buffer entry points: the reference's launch functions ---- */
+
+/* BackendDispatch::launch_matvec (gpu_backend.rs:188-194) /
+ * frink_cuda::gpu::launch_q4_k_matvec and siblings (crates/frink-cuda/src/gpu.rs:319-446):
+ * out[rows] = W x.  Checks weights_len == rows*row_bytes, row_bytes a whole number of
+ * blocks, x_len == blocks*block_elems, rows > 0. */
+int frk_hip_launch_matvec(int kind, const uint8_t *weights, size_t weights_len, const float *x,
+                          size_t x_len, size_t rows, size_t row_bytes, float *out);
+
+/* frink_cuda::mul_mm_launch::launch_mul_mm (crates/frink-cuda/src/mul_mm_launch.rs:40-68) with
+ * validate_shape's checks (crates/frink-cuda/src/mul_mm.rs:581-625):
+ * out[token*n_rows + row] = sum_k W[row][k] * x_batch[token*n_cols + k]. */
+int frk_hip_launch_mul_mm(int kind, const uint8_t *weights, size_t weights_len,
+                          const float *x_batch, size_t x_len, size_t n_rows, size_t n_cols,
+                          size_t batch, size_t row_bytes, float *out);
+
+/* ---- device-pointer entry points (asynchronous on `stream`, a hipStream_t or NULL) ---- */
+
+/* y[rows] = W x for one activation vector in HBM.  K-quants: x is quantized to Q8_K
+ * on the device first (bit-exact with quantize_activations_q8_k,
+ * crates/frink-quant/src/act_quant.rs:69-104). */
+int frk_hip_gemv_dev(const frk_weights *w, const float *x_dev, float *y_dev, int act_mode,
+                     void *stream);
+
+/* The same from activations the caller has already quantized to Q8_K (q[cols] i8, d[cols/256] f32,
+ * bsums[cols/16] i16 in HBM), so projections that read one activation -- q/k/v, gate/up -- quantize
+ * it once: the reference's shared MatvecInput (crates/frink-cuda/src/matvec_launch.rs:500-534) and
+ * BatchActs::Q8K (crates/frink-core/src/weight_matrix.rs:757-768).  K-quants only. */
+int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float *d_dev,
+                         const int16_t *bsums_dev, float *y_dev, void *stream);
+
+/* y[batch][rows] = x[batch][cols] W^T (WeightMatrix::apply_batch_with_acts,
+ * crates/frink-core/src/weight_matrix.rs:2481).  Any batch >= 1. */
+int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
+                     void *stream);
+
+/* Test hooks for the bit-exact gates. */
+/* quantize_activations_q8_k over n = 256*k values: q[n] i8, d[n/256] f32, bsums[n/16] i16 */
+int frk_hip_quantize_q8_k_dev(const float *x_dev, size_t n, int8_t *q_dev, float *d_dev,
+                              int16_t *bsums_dev, void *stream);
+/* quantize_activations_q8 (Avx form) over n = 32*k values: q[n] i8, d[n/32] f32 */
+int frk_hip_quantize_q8_0_dev(const float *x_dev, size_t n, int8_t *q_dev, float *d_dev,
+                              void *stream);
+/* dequant_q8_0 / dequant_q4_k / dequant_q6_k (crates/frink-quant/src/lib.rs:271-286, 334-364,
+ * 519-552) from the resident (possibly permuted) copy: out[rows*cols] f32. */
+int frk_hip_dequant_dev(const frk_weights *w, float *out_dev, void *stream);
+
+/* Plain device copy of `bytes` (multiple of 16), used to calibrate HBM counters and as the
+ * practical bandwidth ceiling a streaming kernel of the same size can reach. */
+int frk_hip_copy_dev(const void *src_dev, void *dst_dev, size_t bytes, void *stream);
+/* Read-only stream over `bytes` (multiple of 16): every 16-byte word is loaded and folded
+ * into 4 bytes per workgroup written to sink_dev (>= 64 KiB). */
+int frk_hip_read_dev(const void *src_dev, size_t bytes, void *sink_dev, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

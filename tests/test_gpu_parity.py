@@ -1,0 +1,251 @@
+"""Parity of the HIP path against the CPU oracle, through the C ABI, on a real MI355X.
+
+Gates (crates and lines are the reference's):
+  * bit-exact: dequantized weights (dequant_q8_0 / dequant_q4_k / dequant_q6_k,
+    crates/frink-quant/src/lib.rs:271-286, 334-364, 519-552) and activation quantization
+    (quantize_activations_q8_k / quantize_activations_q8, crates/frink-quant/src/act_quant.rs:69-189);
+  * fp32 outputs: max |err| <= 1e-3 * ||y||_inf per output row of the batch.
+"""
+import numpy as np
+import pytest
+
+import oracle as fo
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3  # of ||y||_inf, per activation row
+
+
+@pytest.fixture(scope="module")
+def fa():
+    import torch
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    import frink_amd
+    info = frink_amd.probe()
+    assert info["gcn_arch"].startswith("gfx950"), info
+    print("device:", info, flush=True)
+    return frink_amd
+
+
+def to_dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def make_weights(kind, rows, cols, seed, sigma=0.02):
+    from frink_amd import synth
+    return fo.encode_matrix(kind, synth.weights(seed, rows, cols, sigma))
+
+
+def assert_rows_close(got, want, what):
+    got = np.asarray(got, np.float32).reshape(want.shape)
+    for b in range(want.shape[0]):
+        ninf = np.abs(want[b]).max()
+        err = np.abs(got[b] - want[b]).max()
+        assert err <= TOL * ninf, "%s: row %d max|err| %.3g > %.3g (||y||inf %.3g)" % (what, b, err, TOL * ninf, ninf)
+
+
+# ------------------------------------------------------------------ dequant (bit-exact)
+
+@pytest.mark.parametrize("kind,rows,cols", [
+    (fo.Q4_K, 33, 4096), (fo.Q4_K, 5, 256), (fo.Q4_K, 7, 768),
+    (fo.Q6_K, 9, 14336), (fo.Q6_K, 5, 256), (fo.Q6_K, 3, 768),
+    (fo.Q8_0, 17, 4096), (fo.Q8_0, 4, 32), (fo.Q8_0, 3, 96),
+])
+def test_dequant_is_bit_exact(fa, kind, rows, cols):
+    data = make_weights(kind, rows, cols, seed=100 + kind)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    got = w.dequant().cpu().numpy()
+    want = fo.dequant(kind, data).reshape(rows, cols)
+    assert np.array_equal(bits(got), bits(want))
+    w.release()
+
+
+def test_dequant_of_arbitrary_block_bytes_is_bit_exact(fa):
+    # any byte pattern is a structurally valid block; only the f16 super-scales are kept finite
+    rng = np.random.default_rng(7)
+    for kind, offs in ((fo.Q4_K, (0, 2)), (fo.Q6_K, (208,)), (fo.Q8_0, (0,))):
+        bb, be = fo.BLOCK[kind]
+        rows, nb = 6, 4
+        data = rng.integers(0, 256, rows * nb * bb, dtype=np.uint8).reshape(rows * nb, bb)
+        for off in offs:
+            data[:, off:off + 2] = rng.uniform(-0.05, 0.05, rows * nb).astype(np.float16).view(np.uint8).reshape(-1, 2)
+        data = data.ravel()
+        w = fa.Weights.from_host(kind, data, rows, nb * be)
+        got = w.dequant().cpu().numpy()
+        assert np.array_equal(bits(got), bits(fo.dequant(kind, data).reshape(rows, nb * be))), kind
+        w.release()
+
+
+def test_dequant_of_the_reference_golden_blocks(fa, vectors):
+    for kind, blk, gold in ((fo.Q4_K, "q4_k_test_block", "q4_k_golden"), (fo.Q6_K, "q6_k_test_block", "q6_k_golden"),
+                            (fo.Q6_K, "q6_k_signed_scales_test_block", "q6_k_signed_scales_golden"),
+                            (fo.Q6_K, "q6_k_signed_test_block", "q6_k_signed_golden")):
+        data = np.frombuffer(bytes.fromhex(vectors[blk]), np.uint8)
+        w = fa.Weights.from_host(kind, data, 1, 256)
+        got = w.dequant().cpu().numpy().ravel()
+        assert np.abs(got - np.array(vectors[gold], np.float32)).max() < 1e-3
+        w.release()
+
+
+def test_weights_from_device_bytes_match_from_host(fa):
+    data = make_weights(fo.Q6_K, 8, 512, seed=5)
+    a = fa.Weights.from_host(fo.Q6_K, data, 8, 512)
+    b = fa.Weights.from_device(fo.Q6_K, to_dev(data), 8, 512)
+    assert np.array_equal(bits(a.dequant().cpu().numpy()), bits(b.dequant().cpu().numpy()))
+
+
+# ------------------------------------------------------------------ activation quantizers (bit-exact)
+
+def _q8k_cases():
+    from frink_amd import synth
+    head = lambda h: np.concatenate([np.array(h, np.float32), np.zeros(256 - len(h), np.float32)])
+    amax = np.uint32(0x3FE46A64).view(np.float32)
+    xx = np.uint32(0x3DD7D365).view(np.float32)
+    return {
+        "ties": head([127.0, 2.5, -3.5, 0.5, -0.5, 126.5]),
+        "inverse_scale": head([-amax, xx]),
+        "zero": np.zeros(256, np.float32),
+        "normal": synth.activations(11, 8, 4096).ravel(),
+        "outliers": synth.activations(12, 16, 4096, outlier_frac=0.01).ravel(),
+        "tiny": synth.normal(13, 1024, 1e-30),
+        "huge": synth.normal(14, 1024, 1e30),
+        "wide": synth.activations(15, 2, 14336).ravel(),
+    }
+
+
+def test_quantize_q8_k_is_bit_exact(fa):
+    for name, x in _q8k_cases().items():
+        q, d, bs = fa.quantize_q8_k(to_dev(x))
+        wq, wd, wbs = fo.quantize_q8_k(x)
+        assert np.array_equal(q.cpu().numpy(), wq), name
+        assert np.array_equal(bits(d.cpu().numpy()), bits(wd)), name
+        assert np.array_equal(bs.cpu().numpy(), wbs), name
+
+
+def test_quantize_q8_k_kats(fa):
+    c = _q8k_cases()
+    q, d, bs = fa.quantize_q8_k(to_dev(c["ties"]))
+    assert d.cpu().numpy()[0] == 1.0 and list(q.cpu().numpy()[:6]) == [127, 2, -4, 0, 0, 126]
+    assert bs.cpu().numpy()[0] == 251
+    q, d, _ = fa.quantize_q8_k(to_dev(c["inverse_scale"]))
+    assert bits(d.cpu().numpy())[0] == 0x3C6636D1 and list(q.cpu().numpy()[:2]) == [-127, 8]
+
+
+def test_quantize_q8_0_is_bit_exact(fa):
+    from frink_amd import synth
+    head = lambda h: np.concatenate([np.array(h, np.float32), np.zeros(32 - len(h), np.float32)])
+    cases = [head([127.0, 2.5, -3.5, 0.5, 1.5]), head([1.0, 0.5]), np.zeros(32, np.float32),
+             head([np.uint32(0x4013E709).view(np.float32), np.uint32(0x3CDF99C0).view(np.float32)]),
+             synth.activations(21, 4, 4096).ravel(), synth.normal(22, 320, 1e-6)]
+    for x in cases:
+        q, d = fa.quantize_q8_0(to_dev(x))
+        wq, wd = fo.quantize_q8_0(x, fo.FORM_AVX)
+        assert np.array_equal(q.cpu().numpy(), wq)
+        assert np.array_equal(bits(d.cpu().numpy()), bits(wd))
+
+
+# ------------------------------------------------------------------ GEMV
+
+GEMV_SHAPES = [
+    (fo.Q4_K, 64, 4096), (fo.Q4_K, 37, 4096), (fo.Q4_K, 19, 2048), (fo.Q4_K, 21, 768), (fo.Q4_K, 9, 256),
+    (fo.Q4_K, 6, 14336),
+    (fo.Q6_K, 48, 14336), (fo.Q6_K, 13, 4096), (fo.Q6_K, 11, 768), (fo.Q6_K, 9, 256), (fo.Q6_K, 5, 2048),
+    (fo.Q8_0, 64, 4096), (fo.Q8_0, 7, 32), (fo.Q8_0, 9, 544), (fo.Q8_0, 5, 2048),
+]
+
+
+@pytest.mark.parametrize("kind,rows,cols", GEMV_SHAPES)
+def test_gemv_matches_the_oracle(fa, kind, rows, cols):
+    from frink_amd import synth
+    print("gemv", kind, rows, cols, flush=True)
+    data = make_weights(kind, rows, cols, seed=rows * 7 + cols)
+    x = synth.activations(rows + cols, 1, cols)[0]
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    # K-quants: integer dots against Q8_K activations.  Q8_0: the f32 dot (no activation
+    # quantization), and the integer tier as a second mode.
+    mode = fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT
+    want = fo.gemv(kind, data, rows, cols, x, mode)
+    got = w.gemv(to_dev(x), act_mode=fa.ACT_F32).cpu().numpy()
+    assert_rows_close(got[None], want[None], "gemv kind %d %dx%d" % (kind, rows, cols))
+    if kind == fo.Q8_0:
+        want_i = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT)
+        got_i = w.gemv(to_dev(x), act_mode=fa.ACT_INT8).cpu().numpy()
+        assert_rows_close(got_i[None], want_i[None], "gemv q8_0 int tier")
+    w.release()
+
+
+def test_gemv_outliers_and_zero_activation(fa):
+    from frink_amd import synth
+    data = make_weights(fo.Q4_K, 32, 4096, seed=3)
+    w = fa.Weights.from_host(fo.Q4_K, data, 32, 4096)
+    x = synth.activations(4, 1, 4096, outlier_frac=0.01)[0]
+    assert_rows_close(w.gemv(to_dev(x)).cpu().numpy()[None], fo.gemv(fo.Q4_K, data, 32, 4096, x)[None], "outliers")
+    z = np.zeros(4096, np.float32)
+    assert not w.gemv(to_dev(z)).cpu().numpy().any()
+
+
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K, fo.Q8_0])
+def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
+    from frink_amd import synth
+    rows, cols = 24, 1024
+    bb, be = fo.BLOCK[kind]
+    data = make_weights(kind, rows, cols, seed=9)
+    x = synth.activations(10, 1, cols)[0]
+    got = fa.launch_matvec(kind, data, x, rows, cols // be * bb)
+    want = fo.gemv(kind, data, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT)
+    assert_rows_close(got[None], want[None], "launch_matvec")
+    # the resident copy is keyed by (pointer, length) and checked against sampled bytes: overwrite the
+    # buffer in place and the next call must see the new weights
+    data2 = make_weights(kind, rows, cols, seed=99)
+    data[:] = data2
+    got2 = fa.launch_matvec(kind, data, x, rows, cols // be * bb)
+    want2 = fo.gemv(kind, data2, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT)
+    assert_rows_close(got2[None], want2[None], "launch_matvec after the host bytes changed")
+
+
+def test_gemm_entry_point_is_batch_major(fa):
+    from frink_amd import synth
+    rows, cols, batch = 40, 1024, 3
+    data = make_weights(fo.Q4_K, rows, cols, seed=17)
+    x = synth.activations(18, batch, cols)
+    got = fa.launch_mul_mm(fo.Q4_K, data, x, rows, cols, batch, cols // 256 * 144)
+    want = fo.gemm(fo.Q4_K, data, rows, cols, x)
+    assert got.shape == (batch, rows)
+    assert_rows_close(got, want, "launch_mul_mm")
+
+
+# ------------------------------------------------------------------ full-size configurations
+
+FULL = [
+    ("Q8_0 4096x4096", fo.Q8_0, 4096, 4096, 31),
+    ("Q4_K 14336x4096 (gate/up)", fo.Q4_K, 14336, 4096, 32),
+    ("Q6_K 4096x14336 (down)", fo.Q6_K, 4096, 14336, 33),
+]
+
+
+@pytest.mark.parametrize("name,kind,rows,cols,seed", FULL)
+def test_full_size_gemv(fa, name, kind, rows, cols, seed):
+    """The configured shapes: the whole output against the oracle (a few seconds of CPU), plus
+    two size-independent properties: linearity in the output rows (a permutation of W's rows
+    permutes y) is implied by per-row ownership, so check homogeneity instead -- scaling x by a
+    power of two scales Q8_K's d exactly and leaves q unchanged, so y scales exactly."""
+    from frink_amd import synth
+    print("full", name, flush=True)
+    data = make_weights(kind, rows, cols, seed)
+    x = synth.activations(seed + 100, 1, cols)[0]
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    mode = fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT
+    want = fo.gemv(kind, data, rows, cols, x, mode)
+    y = w.gemv(to_dev(x)).cpu().numpy()
+    assert_rows_close(y[None], want[None], name)
+    y4 = w.gemv(to_dev(x * np.float32(4.0))).cpu().numpy()
+    assert np.array_equal(bits(y4), bits(y * np.float32(4.0)))
+    # and the dequantized matrix, every value
+    got = w.dequant().cpu().numpy()
+    assert np.array_equal(bits(got), bits(fo.dequant(kind, data).reshape(rows, cols)))
+    w.release()
