@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+A "step" is one decode GEMV of the headline workload: Q4_K weights, rows=14336, cols=4096
+(Llama-3-8B FFN gate/up), one f32 activation vector quantized to Q8_K on the device, f32 output.
+Operands are resident in HBM before the timed region.  Every step reads a different one of
+COPIES weight copies (COPIES x 33 MB > the 256 MB Infinity Cache), so the weights come from HBM
+and not from cache.  The metric is the reference's: quantized weight bytes / seconds per step
+(crates/frink-cuda/examples/matvec_bench.rs:56-61), in GB/s.
+
+Prints ONE JSON line (see the fields at the bottom).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+COPIES = 16
+
+
+def random_blocks(kind, rows, cols, seed):
+    """Structurally valid GGUF blocks with weight-like magnitudes, straight from a seeded
+    generator (timing does not depend on the values; the parity tests use encoded N(0, 0.02))."""
+    from frink_amd import BLOCK
+    bb, be = BLOCK[kind]
+    nb = rows * (cols // be)
+    rng = np.random.default_rng(seed)
+    data = rng.integers(0, 256, (nb, bb), dtype=np.uint8)
+
+    def f16(lo, hi):
+        return rng.uniform(lo, hi, nb).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    if kind == 12:      # Q4_K: d, dmin
+        data[:, 0:2] = f16(1e-4, 3e-4)
+        data[:, 2:4] = f16(1e-3, 3e-3)
+    elif kind == 14:    # Q6_K: d
+        data[:, 208:210] = f16(2e-5, 6e-5)
+    else:               # Q8_0: d
+        data[:, 0:2] = f16(3e-4, 6e-4)
+    return data.reshape(-1)
+
+
+def time_graph(torch, fn_steps, n_steps, copies):
+    """Captures `copies` consecutive steps in one HIP graph and replays it; returns seconds for
+    exactly n_steps steps (a second, shorter graph runs the remainder)."""
+    stream = torch.cuda.Stream()
+    graphs = []
+    with torch.cuda.stream(stream):
+        for i in range(copies):
+            fn_steps(i)  # warm: sizes the library workspace before capture
+        torch.cuda.synchronize()
+        full, rem = divmod(n_steps, copies)
+        for count in ([copies] if full else []) + ([rem] if rem else []):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for i in range(count):
+                    fn_steps(i)
+            graphs.append((g, count))
+        g_full = graphs[0][0] if full else None
+        g_rem = graphs[-1][0] if rem else None
+        # one untimed replay of each
+        for g, _ in graphs:
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(full):
+            g_full.replay()
+        if g_rem is not None:
+            g_rem.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e-3
+
+
+def cpu_baseline(kind, data, rows, cols, x, y_gpu, budget_s=8.0):
+    """Times the CPU oracle (a C restatement of Frink's integer-dot CPU path, row-parallel over
+    OpenMP threads) on the same weights and activation, and checks the GPU result against it."""
+    import oracle as fo
+    threads = min(16, os.cpu_count() or 1)
+    want = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads)
+    reps, spent = 0, 0.0
+    best = float("inf")
+    while spent < budget_s and reps < 200:
+        t = time.perf_counter()
+        fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads)
+        dt = time.perf_counter() - t
+        best = min(best, dt)
+        spent += dt
+        reps += 1
+    err = float(np.abs(y_gpu - want).max() / np.abs(want).max())
+    return {"value": round(data.size / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "the whole workload (Q8_K activation quantization + %dx%d Q4_K integer dots), best of %d "
+                      "repetitions, scalar C restatement of dot_q4_k_q8 with OpenMP row partition" % (rows, cols, reps),
+            "gpu_vs_cpu_max_err_over_ninf": err}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import frink_amd as fa
+
+    info = fa.probe()
+    dev = torch.device("cuda:0")
+    rows, cols, kind = 14336, 4096, fa.Q4_K
+    from frink_amd import synth
+    data = random_blocks(kind, rows, cols, seed=1234)
+    x = synth.activations(4321, 1, cols)[0]
+    data_dev = torch.from_numpy(data).to(dev)
+    ws = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(COPIES)]
+    xd = torch.from_numpy(x).to(dev)
+    y = torch.empty(rows, dtype=torch.float32, device=dev)
+    torch.cuda.synchronize()
+
+    # ---- headline: whole step (Q8_K quantization + GEMV) ----
+    def step(i):
+        ws[i % COPIES].gemv(xd, out=y)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    wall, ev = time_graph(torch, step, args.steps, COPIES)
+    sec_per_step = ev / args.steps
+    wbytes = data.size
+    value = wbytes / sec_per_step / 1e9
+
+    # ---- roofline of the dominant kernel: GEMV alone, activation already quantized ----
+    acts = fa.quantize_q8_k(xd)
+
+    def gemv_only(i):
+        ws[i % COPIES].gemv_q8k(acts, out=y)
+
+    n_k = max(COPIES * 8, min(args.steps, 4000))
+    _, ev_k = time_graph(torch, gemv_only, n_k, COPIES)
+    k_sec = ev_k / n_k
+    alg_bytes = wbytes + cols + cols // 256 * 4 + cols // 16 * 2 + rows * 4  # W + Q8_K activation + y
+    achieved = alg_bytes / k_sec / 1e9
+    y_gpu = y.cpu().numpy()
+
+    out = {
+        "metric": "Q4_K GEMV HBM GB/s", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": "Q4_K decode GEMV, rows=14336 cols=4096 batch=1 (Llama-3-8B FFN gate/up): Q8_K "
+                               "activation quantization + GEMV per step, %d weight copies rotated (cache-cold)" % COPIES,
+                   "weight_bytes": int(wbytes), "device": info["name"], "arch": info["gcn_arch"],
+                   "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "gemv_q4_k_kernel", "algorithmic_bytes": int(alg_bytes),
+                     "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        # practical ceilings at the same size: a read-only stream and a copy
+        src = [torch.empty(wbytes, dtype=torch.uint8, device=dev).random_() for _ in range(COPIES)]
+        dst = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+        sink = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+        L, C = fa.lib(), __import__("ctypes")
+
+        def read_only(i):
+            fa.check(L.frk_hip_read_dev(C.c_void_p(src[i % COPIES].data_ptr()), wbytes, C.c_void_p(sink.data_ptr()),
+                                        fa._stream()))
+
+        def copy(i):
+            fa.check(L.frk_hip_copy_dev(C.c_void_p(src[i % COPIES].data_ptr()), C.c_void_p(dst.data_ptr()), wbytes,
+                                        fa._stream()))
+        _, t = time_graph(torch, read_only, 800, COPIES)
+        extra["read_only_stream_33MB_GBs"] = round(wbytes / (t / 800) / 1e9, 1)
+        _, t = time_graph(torch, copy, 800, COPIES)
+        extra["copy_33MB_read_plus_write_GBs"] = round(2 * wbytes / (t / 800) / 1e9, 1)
+        del src, dst
+        for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
+                                 ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096)):
+            d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
+            n_copies = COPIES if k2 != fa.Q8_0 else 32
+            w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]
+            x2 = torch.from_numpy(synth.activations(5, 1, c2)[0]).to(dev)
+            y2 = torch.empty(r2, dtype=torch.float32, device=dev)
+
+            def step2(i):
+                w2[i % n_copies].gemv(x2, out=y2)
+            _, t = time_graph(torch, step2, 1600, n_copies)
+            extra[name] = {"GBs": round(d2.numel() / (t / 1600) / 1e9, 1), "us_per_step": round(t / 1600 * 1e6, 3),
+                           "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
+            for w in w2:
+                w.release()
+        out["extra"] = extra
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(kind, data, rows, cols, x, y_gpu)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

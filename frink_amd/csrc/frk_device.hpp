@@ -1,0 +1,102 @@
+// Device-side helpers shared by the kernels: f16 conversion, dot4, DPP reductions and the Q8_K
+// block quantizer.
+#pragma once
+
+#include "frk_internal.hpp"
+
+namespace frk {
+
+__device__ __forceinline__ float h2f(uint32_t bits16) {
+    _Float16 v;
+    uint16_t h = (uint16_t)bits16;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;  // exact, subnormals included
+}
+
+__device__ __forceinline__ uint16_t f2h_bits(float f) {
+    _Float16 v = (_Float16)f;  // round to nearest even
+    uint16_t h;
+    __builtin_memcpy(&h, &v, 2);
+    return h;
+}
+
+__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// v (op) lane-permuted v, the permutation given by a DPP control word
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+
+// Workgroup barrier that publishes LDS writes but does NOT wait for outstanding global loads.
+// __syncthreads() is a full fence: it drains vmcnt too, which would stall every wavefront until
+// all the weight loads it prefetched have landed.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
+constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <- lane 7-i of its group of 8
+constexpr int DPP_ROW_MIRROR = 0x140;   // lane i <- lane 15-i of its row of 16
+
+// Sum over the LPR lanes (16, 32 or 64) that share a row; every lane ends with the total.
+template <int LPR>
+__device__ __forceinline__ float part_sum(float v) {
+    v += dpp_f<DPP_QUAD_XOR1>(v);
+    v += dpp_f<DPP_QUAD_XOR2>(v);
+    v += dpp_f<DPP_HALF_MIRROR>(v);
+    v += dpp_f<DPP_ROW_MIRROR>(v);
+    if (LPR >= 32) v += __shfl_xor(v, 16);
+    if (LPR >= 64) v += __shfl_xor(v, 32);
+    return v;
+}
+
+// Max over all 64 lanes.  max is exact, so any fold order gives the reference's amax.
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
+    v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
+    v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f<DPP_ROW_MIRROR>(v));
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+
+// quantize_activations_q8_k (crates/frink-quant/src/act_quant.rs:69-104) for one 256-value block
+// held four consecutive values per lane by one wavefront.  Returns the lane's four quants packed
+// little-endian; d_out is the block scale (same in every lane); bsum16 is the sum of the 16-wide
+// group this lane belongs to (same in the four lanes of a quad).
+__device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, int &bsum16) {
+    // f32::max ignores a NaN operand, as fmaxf does
+    const float amax = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+    d_out = 0.0f;
+    if (amax != 0.0f) {  // uniform across the wavefront
+        const float iscale = __fdiv_rn(127.0f, amax);
+        auto quant = [&](float e) {
+            float r = rintf(iscale * e);  // round half to even
+            r = fminf(fmaxf(r, -127.0f), 127.0f);
+            return (r != r) ? 0 : (int)r;  // a NaN becomes 0, as Rust's `as i8` makes it
+        };
+        q0 = quant(v.x);
+        q1 = quant(v.y);
+        q2 = quant(v.z);
+        q3 = quant(v.w);
+        d_out = __fdiv_rn(1.0f, iscale);
+    }
+    int s = q0 + q1 + q2 + q3;
+    s += dpp_i<DPP_QUAD_XOR1>(s);
+    s += dpp_i<DPP_QUAD_XOR2>(s);
+    bsum16 = s;
+    return (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) | ((uint32_t)(q2 & 0xff) << 16) |
+           ((uint32_t)(q3 & 0xff) << 24);
+}
+
+}  // namespace frk

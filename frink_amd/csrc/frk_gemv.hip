@@ -4,38 +4,9 @@
 // activation lives in LDS, the integer products run on v_dot4_i32_i8 and a block's scale is
 // applied once per 64 weights.  A wavefront (or an LPR-lane part of one, for short rows) owns a
 // row; lanes walk the row in "units" of 64 weights.
-#include "frk_internal.hpp"
+#include "frk_device.hpp"
 
 namespace frk {
-
-__device__ __forceinline__ float h2f(uint32_t bits16) {
-    _Float16 v;
-    uint16_t h = (uint16_t)bits16;
-    __builtin_memcpy(&v, &h, 2);
-    return (float)v;
-}
-
-__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
-}
-
-template <int CTRL>
-__device__ __forceinline__ float dpp_add(float v) {
-    int o = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true);
-    return v + __int_as_float(o);
-}
-
-// Sum over the LPR lanes that share a row; every lane of the part ends with the total.
-template <int LPR>
-__device__ __forceinline__ float part_sum(float v) {
-    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141>(v);  // row_half_mirror
-    v = dpp_add<0x140>(v);  // row_mirror: all 16 lanes of a row hold the row's sum
-    if (LPR >= 32) v += __shfl_xor(v, 16);
-    if (LPR >= 64) v += __shfl_xor(v, 32);
-    return v;
-}
 
 // ------------------------------------------------------------------ Q4_K x Q8_K
 // dot_q4_k_q8 (crates/frink-quant/src/lib.rs:822-869).  Unit = (block b, pair p): the 32 bytes

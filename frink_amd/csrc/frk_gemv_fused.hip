@@ -1,0 +1,331 @@
+// Decode GEMV for Q4_K weights, one launch per matrix.
+//
+// FUSED mode: the workgroup quantizes the f32 activation to Q8_K itself (bit-exact with
+// quantize_activations_q8_k) while its weight loads are already in flight, so a decode step is a
+// single kernel.  PREQ modes take an activation quantized earlier (shared by gate/up or q/k/v).
+//
+// Shape of the kernel: every wavefront issues the 16-byte loads of all the rows it handles in a
+// round before doing anything else; the activation's own loads go out first (a wavefront's loads
+// return in order); the workgroup barrier in front of the arithmetic waits for LDS only, never
+// for the weight loads.  A lane multiplies the same columns in every row, so its slice of the
+// quantized activation is read once into registers.
+#include "frk_device.hpp"
+
+namespace frk {
+
+enum { MODE_FUSED = 0, MODE_PREQ_LDS = 1, MODE_PREQ_DIRECT = 2 };
+
+// Loads of the activation, issued before the weight loads, and their later deposit in LDS.
+// LDS layout: sq[nb*256] i8 | sbs[nb*16] i16 | sd[nb] f32.  XB = ceil(nb / wavefronts).
+template <int MODE, int XB>
+struct ActStage {
+    float4 xv[MODE == MODE_FUSED ? XB : 1];
+    uint4 qv[MODE == MODE_PREQ_LDS ? XB : 1];
+    uint32_t bv;  // two bsums
+    float dv;
+
+    __device__ __forceinline__ void load(int nb, const float *__restrict__ x, const int8_t *__restrict__ aq,
+                                         const float *__restrict__ ad, const int16_t *__restrict__ absums) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+        if (MODE == MODE_PREQ_LDS) {
+            // nb*16 words of quants over blockDim threads: XB >= nb*16 / blockDim
+#pragma unroll
+            for (int i = 0; i < XB; i++) {
+                const int idx = min((int)threadIdx.x + i * (int)blockDim.x, nb * 16 - 1);
+                qv[i] = reinterpret_cast<const uint4 *>(aq)[idx];
+            }
+            bv = reinterpret_cast<const uint32_t *>(absums)[min((int)threadIdx.x, nb * 8 - 1)];
+            dv = ad[min((int)threadIdx.x, nb - 1)];
+        } else if (MODE == MODE_FUSED) {
+#pragma unroll
+            for (int i = 0; i < XB; i++) {
+                const int b = min(wave + i * nwaves, nb - 1);
+                xv[i] = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K)[lane];
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(int nb, int8_t *sq, int16_t *sbs, float *sd) {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+        if (MODE == MODE_PREQ_LDS) {
+#pragma unroll
+            for (int i = 0; i < XB; i++) {
+                const int idx = (int)threadIdx.x + i * (int)blockDim.x;
+                if (idx < nb * 16) reinterpret_cast<uint4 *>(sq)[idx] = qv[i];
+            }
+            if ((int)threadIdx.x < nb * 8) reinterpret_cast<uint32_t *>(sbs)[threadIdx.x] = bv;
+            if ((int)threadIdx.x < nb) sd[threadIdx.x] = dv;
+        } else if (MODE == MODE_FUSED) {
+#pragma unroll
+            for (int i = 0; i < XB; i++) {
+                const int b = wave + i * nwaves;
+                float d;
+                int bs;
+                const uint32_t packed = quantize_q8_k_lane(xv[i], d, bs);
+                if (b < nb) {  // uniform across the wavefront
+                    reinterpret_cast<uint32_t *>(sq + b * QK_K)[lane] = packed;
+                    if ((lane & 3) == 0) sbs[b * 16 + (lane >> 2)] = (int16_t)bs;
+                    if (lane == 0) sd[b] = d;
+                }
+            }
+        }
+    }
+};
+
+// A lane owns "half blocks": unit u = 2*b + q covers pairs p = q and p = q + 2 of block b, that is
+// qs[32q..32q+32] and qs[64+32q..64+32q+32] (sub-blocks 2q, 2q+1, 2q+4, 2q+5; 128 weights) plus the
+// block's 16-byte header, all of which the two pairs need between them: p < 2 reads its 6-bit
+// scales from the plain layout, p >= 2 from the split one (q4_k_scale_min,
+// crates/frink-quant/src/lib.rs:321-330).
+struct Q4Unit {
+    uint4 a[8];  // 128 activation quants: pair q -> a[0..3], pair q+2 -> a[4..7]
+    int bs[4];   // activation sums over sub-blocks 2q, 2q+1, 2q+4, 2q+5
+    float da;    // Q8_K block scale (0 for a lane past the end of the row)
+    int sh;      // 16*q: where this unit's two scale bytes sit in the decoded words
+};
+
+// dot_q4_k_q8 (crates/frink-quant/src/lib.rs:822-869) for one unit of one row.
+__device__ __forceinline__ float q4_k_unit_dot(const uint4 h, const uint4 w0, const uint4 w1, const uint4 w2,
+                                               const uint4 w3, const Q4Unit &U) {
+    const uint32_t hy = h.y >> U.sh, hz = h.z >> U.sh, hw = h.w >> U.sh;  // bytes 0,1 are ours now
+    const uint32_t sc_lo = hy & 0x3f3fu, m_lo = hz & 0x3f3fu;
+    const uint32_t sc_hi = (hw & 0x0f0fu) | (((hy >> 6) & 0x0303u) << 4);
+    const uint32_t m_hi = ((hw >> 4) & 0x0f0fu) | (((hz >> 6) & 0x0303u) << 4);
+    int i0 = 0, i1 = 0, i2 = 0, i3 = 0;
+#define FRK_LO(ACC, WW, AV)                      \
+    ACC = dot4(WW.x & 0x0f0f0f0fu, AV.x, ACC);   \
+    ACC = dot4(WW.y & 0x0f0f0f0fu, AV.y, ACC);   \
+    ACC = dot4(WW.z & 0x0f0f0f0fu, AV.z, ACC);   \
+    ACC = dot4(WW.w & 0x0f0f0f0fu, AV.w, ACC);
+#define FRK_HI(ACC, WW, AV)                             \
+    ACC = dot4((WW.x >> 4) & 0x0f0f0f0fu, AV.x, ACC);   \
+    ACC = dot4((WW.y >> 4) & 0x0f0f0f0fu, AV.y, ACC);   \
+    ACC = dot4((WW.z >> 4) & 0x0f0f0f0fu, AV.z, ACC);   \
+    ACC = dot4((WW.w >> 4) & 0x0f0f0f0fu, AV.w, ACC);
+    FRK_LO(i0, w0, U.a[0])
+    FRK_LO(i0, w1, U.a[1])
+    FRK_HI(i1, w0, U.a[2])
+    FRK_HI(i1, w1, U.a[3])
+    FRK_LO(i2, w2, U.a[4])
+    FRK_LO(i2, w3, U.a[5])
+    FRK_HI(i3, w2, U.a[6])
+    FRK_HI(i3, w3, U.a[7])
+#undef FRK_LO
+#undef FRK_HI
+    // every factor fits 24 bits: scales and mins < 64, |isum| <= 32*15*127, |bsum| <= 32*127
+    int s1 = __mul24((int)(sc_lo & 0xff), i0);
+    s1 += __mul24((int)(sc_lo >> 8), i1);
+    s1 += __mul24((int)(sc_hi & 0xff), i2);
+    s1 += __mul24((int)(sc_hi >> 8), i3);
+    int s2 = __mul24((int)(m_lo & 0xff), U.bs[0]);
+    s2 += __mul24((int)(m_lo >> 8), U.bs[1]);
+    s2 += __mul24((int)(m_hi & 0xff), U.bs[2]);
+    s2 += __mul24((int)(m_hi >> 8), U.bs[3]);
+    const float d = h2f(h.x & 0xffffu), dmin = h2f(h.x >> 16);
+    return (d * U.da) * (float)s1 - (dmin * U.da) * (float)s2;
+}
+
+// LPR lanes share a row (a wavefront works on 64/LPR rows at once), a lane owns units
+// l, l+LPR, ... (J of them) and keeps RPW rounds of rows in flight.
+template <int LPR, int J, int RPW, int XB, int MODE, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
+    const uint8_t *__restrict__ W, size_t row_stride, int rows, int rows_per_wg, int nb,
+    const float *__restrict__ x, const int8_t *__restrict__ aq, const float *__restrict__ ad,
+    const int16_t *__restrict__ absums, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    int8_t *sq = reinterpret_cast<int8_t *>(smem);
+    int16_t *sbs = reinterpret_cast<int16_t *>(sq + nb * QK_K);
+    float *sd = reinterpret_cast<float *>(sbs + nb * 16);
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int part = lane / LPR, l = lane % LPR;
+    const int units = nb * 2;
+    const int row_begin = blockIdx.x * rows_per_wg;
+    const int row_end = min(rows, row_begin + rows_per_wg);
+    const int slot = wave * PARTS + part, slots = nwaves * PARTS;
+
+    int ub[J], uq[J];
+    bool uok[J];
+    size_t uoff[J];  // byte offset of the unit's block in a row
+#pragma unroll
+    for (int j = 0; j < J; j++) {
+        const int u = l + j * LPR;
+        uok[j] = u < units;
+        const int uc = uok[j] ? u : units - 1;
+        ub[j] = uc >> 1;
+        uq[j] = uc & 1;
+        uoff[j] = (size_t)ub[j] * Q4_K_BYTES;
+    }
+
+    // ---- the activation's loads go out first ----
+    ActStage<MODE, XB> act;
+    Q4Unit U[J];
+    act.load(nb, x, aq, ad, absums);
+    if (MODE == MODE_PREQ_DIRECT) {
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            const uint4 *ap = reinterpret_cast<const uint4 *>(aq + ub[j] * QK_K + uq[j] * 64);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                U[j].a[i] = ap[i];
+                U[j].a[4 + i] = ap[8 + i];
+            }
+            const uint2 b0 = *reinterpret_cast<const uint2 *>(absums + ub[j] * 16 + uq[j] * 4);
+            const uint2 b1 = *reinterpret_cast<const uint2 *>(absums + ub[j] * 16 + 8 + uq[j] * 4);
+            U[j].bs[0] = (int)(int16_t)(b0.x & 0xffff) + (int)(int16_t)(b0.x >> 16);
+            U[j].bs[1] = (int)(int16_t)(b0.y & 0xffff) + (int)(int16_t)(b0.y >> 16);
+            U[j].bs[2] = (int)(int16_t)(b1.x & 0xffff) + (int)(int16_t)(b1.x >> 16);
+            U[j].bs[3] = (int)(int16_t)(b1.y & 0xffff) + (int)(int16_t)(b1.y >> 16);
+            U[j].da = uok[j] ? ad[ub[j]] : 0.0f;
+            U[j].sh = uq[j] * 16;
+        }
+    }
+
+    // ---- then all the weight loads of the first round ----
+    uint4 wh[RPW][J], w0[RPW][J], w1[RPW][J], w2[RPW][J], w3[RPW][J];
+    auto issue = [&](int rbase) {
+#pragma unroll
+        for (int k = 0; k < RPW; k++) {
+            const int r = min(rbase + slot + k * slots, rows - 1);
+            const uint8_t *row = W + (size_t)r * row_stride;
+#pragma unroll
+            for (int j = 0; j < J; j++) {
+                const uint4 *blk = reinterpret_cast<const uint4 *>(row + uoff[j]);
+                const int q2 = 2 * uq[j];
+                wh[k][j] = blk[0];
+                w0[k][j] = blk[1 + q2];
+                w1[k][j] = blk[2 + q2];
+                w2[k][j] = blk[5 + q2];
+                w3[k][j] = blk[6 + q2];
+            }
+        }
+    };
+    issue(row_begin);
+
+    if (MODE != MODE_PREQ_DIRECT) {
+        act.store(nb, sq, sbs, sd);
+        lds_barrier();
+#pragma unroll
+        for (int j = 0; j < J; j++) {
+            const uint4 *ap = reinterpret_cast<const uint4 *>(sq + ub[j] * QK_K + uq[j] * 64);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                U[j].a[i] = ap[i];
+                U[j].a[4 + i] = ap[8 + i];
+            }
+            const int16_t *bp = sbs + ub[j] * 16 + uq[j] * 4;
+            U[j].bs[0] = (int)bp[0] + (int)bp[1];
+            U[j].bs[1] = (int)bp[2] + (int)bp[3];
+            U[j].bs[2] = (int)bp[8] + (int)bp[9];
+            U[j].bs[3] = (int)bp[10] + (int)bp[11];
+            U[j].da = uok[j] ? sd[ub[j]] : 0.0f;  // a lane past the end of the row contributes nothing
+            U[j].sh = uq[j] * 16;
+        }
+    }
+
+    for (int rbase = row_begin; rbase < row_end; rbase += slots * RPW) {
+        if (rbase != row_begin) issue(rbase);
+#pragma unroll
+        for (int k = 0; k < RPW; k++) {
+            const int r = rbase + slot + k * slots;
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < J; j++) acc += q4_k_unit_dot(wh[k][j], w0[k][j], w1[k][j], w2[k][j], w3[k][j], U[j]);
+            acc = part_sum<LPR>(acc);
+            if (l == 0 && r < row_end) y[r] = acc;
+        }
+    }
+}
+
+// ------------------------------------------------------------------ launchers
+
+#define FRK_LAUNCH_CHECK(what)                                                                          \
+    do {                                                                                                \
+        hipError_t e_ = hipGetLastError();                                                              \
+        if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
+    } while (0)
+
+static int g_cus = 0;
+static int compute_units() {
+    if (!g_cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            g_cus = n;
+        else
+            g_cus = 256;
+    }
+    return g_cus;
+}
+
+struct FusedGeom {
+    int lpr, j, rpw, threads, grid, rows_per_wg;
+};
+
+// units = half blocks per row.  J units per lane: 1 up to 64 units (cols <= 8192), then 2, then 4.
+// Measured on the 14336x4096 gate/up shape: FUSED runs best with two 512-thread workgroups per
+// compute unit, each quantizing the activation once and walking its rows in rounds of one row per
+// wavefront part; PREQ runs best with 256-thread workgroups that each take a single round.
+static FusedGeom fused_geom(size_t rows, int units, bool fused) {
+    FusedGeom g;
+    g.lpr = units > 32 ? 64 : units > 16 ? 32 : 16;
+    const int per_lane = (units + g.lpr - 1) / g.lpr;
+    g.j = per_lane <= 1 ? 1 : per_lane <= 2 ? 2 : 4;
+    g.rpw = 1;
+    const int parts = 64 / g.lpr;
+    g.threads = fused ? 512 : 256;
+    const size_t slots = (size_t)(g.threads / 64) * parts;
+    size_t grid = (rows + slots - 1) / slots;  // a single round of rows per workgroup ...
+    if (fused) {
+        const size_t two_per_cu = (size_t)compute_units() * 2;
+        if (grid > two_per_cu) grid = two_per_cu;  // ... or several, so x is quantized 512 times at most
+    }
+    g.grid = (int)grid;
+    g.rows_per_wg = (int)((rows + grid - 1) / grid);
+    return g;
+}
+
+template <int MODE>
+static int launch_q4_k_fused(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    FusedGeom g = fused_geom(w->rows, nb * 2, MODE == MODE_FUSED);
+    const size_t shmem = MODE == MODE_PREQ_DIRECT ? 0 : (size_t)nb * (256 + 32 + 4);
+    const int nwaves = g.threads / 64;
+    const int xb = (nb + nwaves - 1) / nwaves;
+#define FRK_GO2(LPR, J, RPW, XB, MAXT)                                                                            \
+    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT>), dim3(g.grid), dim3(g.threads), shmem, \
+                       s, w->dev, w->layout.row_stride, (int)w->rows, g.rows_per_wg, nb, x, a.q, a.d, a.bsums, y)
+#define FRK_GO(LPR, J, RPW, MAXT)                                               \
+    do {                                                                        \
+        if (MODE == MODE_PREQ_DIRECT || xb <= 1) FRK_GO2(LPR, J, RPW, 1, MAXT); \
+        else if (xb <= 2) FRK_GO2(LPR, J, RPW, 2, MAXT);                        \
+        else if (xb <= 4) FRK_GO2(LPR, J, RPW, 4, MAXT);                        \
+        else FRK_GO2(LPR, J, RPW, 8, MAXT);                                     \
+    } while (0)
+    if (g.lpr == 16) FRK_GO(16, 1, 1, 512);
+    else if (g.lpr == 32) FRK_GO(32, 1, 1, 512);
+    else if (g.j == 1) FRK_GO(64, 1, 1, 512);
+    else if (g.j == 2) FRK_GO(64, 2, 1, 512);
+    else FRK_GO(64, 4, 1, 512);
+#undef FRK_GO
+#undef FRK_GO2
+    FRK_LAUNCH_CHECK("gemv_q4_k_fused");
+    return FRK_OK;
+}
+
+bool fused_gemv_fits(const frk_weights *w) {
+    // up to 4 half blocks per lane and 8 activation blocks per wavefront: rows of at most 64
+    // blocks; wider rows take the generic kernels
+    return w->cols <= 16384;
+}
+
+int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    return launch_q4_k_fused<MODE_FUSED>(w, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
+}
+int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, a, y, s);
+    return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, a, y, s);
+}
+
+}  // namespace frk

@@ -115,6 +115,10 @@ struct Q8KActs {  // Q8_K activations in HBM, struct-of-arrays per activation ro
 };
 int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+// one-launch kernels (activation quantized inside the GEMV); cols <= 16384
+bool fused_gemv_fits(const frk_weights *w);
+int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
 

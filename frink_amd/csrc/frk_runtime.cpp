@@ -340,6 +340,8 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
     hipStream_t s = (hipStream_t)stream;
     switch (w->kind) {
     case FRK_KIND_Q4_K:
+        if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
+        [[fallthrough]];
     case FRK_KIND_Q6_K: {
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, &a);
@@ -367,7 +369,9 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     clear_error();
     if (!w || !q || !d || !bsums || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_q8k_dev: null argument");
     Q8KActs a{q, d, bsums};
-    if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
+    if (w->kind == FRK_KIND_Q4_K)
+        return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
+                                  : launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
     if (w->kind == FRK_KIND_Q6_K) return launch_gemv_q6_k(w, a, y, (hipStream_t)stream);
     return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K and Q6_K weights only (kind %d)", w->kind);
 }
