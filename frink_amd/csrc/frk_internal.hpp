@@ -119,6 +119,9 @@ int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 bool fused_gemv_fits(const frk_weights *w);
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+// batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
+int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
 

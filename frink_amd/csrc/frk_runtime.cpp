@@ -380,7 +380,13 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     clear_error();
     if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
     if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
-    // first slice: one matvec per activation row (the reference's own path below its GEMM threshold,
+    if (w->kind == FRK_KIND_Q4_K && batch >= 16) {
+        void *ws = nullptr;
+        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        if (rc) return rc;
+        return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
+    }
+    // otherwise one matvec per activation row (the reference's own path below its GEMM threshold,
     // crates/frink-core/src/weight_matrix.rs:2636-2652)
     for (size_t b = 0; b < batch; b++) {
         int rc = frk_hip_gemv_dev(w, x + b * w->cols, y + b * w->rows, FRK_ACT_F32, stream);

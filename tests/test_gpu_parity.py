@@ -249,3 +249,41 @@ def test_full_size_gemv(fa, name, kind, rows, cols, seed):
     got = w.dequant().cpu().numpy()
     assert np.array_equal(bits(got), bits(fo.dequant(kind, data).reshape(rows, cols)))
     w.release()
+
+
+# ------------------------------------------------------------------ batched GEMM (int8 MFMA)
+
+@pytest.mark.parametrize("rows,cols,batch", [(256, 1024, 128), (96, 512, 40), (64, 256, 16), (200, 768, 130),
+                                             (128, 2048, 512)])
+def test_gemm_mfma_matches_the_oracle(fa, rows, cols, batch):
+    from frink_amd import synth
+    print("gemm", rows, cols, batch, flush=True)
+    data = make_weights(fo.Q4_K, rows, cols, seed=rows + cols + batch)
+    x = synth.activations(rows * 3 + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    want = fo.gemm(fo.Q4_K, data, rows, cols, x)
+    assert got.shape == (batch, rows)
+    assert_rows_close(got, want, "gemm %dx%d batch %d" % (rows, cols, batch))
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 4096), (14336, 4096)])
+def test_full_size_prefill_gemm(fa, rows, cols):
+    """M=512 with 1% outliers at +-20: every output row of the batch against the oracle on a
+    slice of weight rows (the oracle takes seconds per 512 rows), plus exact homogeneity."""
+    from frink_amd import synth
+    print("full gemm", rows, cols, flush=True)
+    batch = 512
+    data = make_weights(fo.Q4_K, rows, cols, seed=rows)
+    x = synth.activations(77, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    y = w.gemm(to_dev(x)).cpu().numpy()
+    for row0 in (0, rows // 2 - 64, rows - 256):
+        want = fo.gemm(fo.Q4_K, data, rows, cols, x, row0=row0, nrows=256)
+        ninf = np.abs(want).max(axis=1)
+        err = np.abs(y[:, row0:row0 + 256] - want).max(axis=1)
+        assert (err <= TOL * ninf).all(), (row0, float((err / ninf).max()))
+    y2 = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
+    assert np.array_equal(bits(y2), bits(y * np.float32(0.5)))
+    w.release()
