@@ -27,7 +27,8 @@ EXPORTS = [
     "frk_hip_worth_a_gemm", "frk_hip_weights_register", "frk_hip_weights_from_device",
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
-    "frk_hip_gemm_dev",
+    "frk_hip_gemm_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
+    "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_copy_dev", "frk_hip_read_dev",
 ]
@@ -80,6 +81,9 @@ def lib():
             "frk_hip_gemv_dev": (i, [vp, vp, vp, i, vp]),
             "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
+            "frk_hip_route_top_k_softmax_dev": (i, [vp, sz, sz, sz, i, vp, vp, vp]),
+            "frk_hip_moe_ffn_dev": (i, [vp, vp, vp, sz, vp, sz, vp, vp, sz, vp, vp]),
+            "frk_hip_moe_intermediates_dev": (i, [sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
             "frk_hip_quantize_q8_k_dev": (i, [vp, sz, vp, vp, vp, vp]),
             "frk_hip_quantize_q8_0_dev": (i, [vp, sz, vp, vp, vp]),
             "frk_hip_dequant_dev": (i, [vp, vp, vp]),
@@ -220,6 +224,46 @@ def quantize_q8_0(x):
     check(lib().frk_hip_quantize_q8_0_dev(C.c_void_p(x.data_ptr()), n, C.c_void_p(q.data_ptr()),
                                           C.c_void_p(d.data_ptr()), _stream()))
     return q, d
+
+
+def route_top_k_softmax(logits, k, norm):
+    """frink_moe::route_top_k_softmax per row of logits[batch][n_experts]: (ids int32[batch][k], weights f32[batch][k])."""
+    import torch
+    logits = logits.contiguous()
+    batch, n_experts = logits.shape
+    ids = torch.empty((batch, k), dtype=torch.int32, device=logits.device)
+    w = torch.empty((batch, k), dtype=torch.float32, device=logits.device)
+    check(lib().frk_hip_route_top_k_softmax_dev(C.c_void_p(logits.data_ptr()), batch, n_experts, k, int(bool(norm)),
+                                                C.c_void_p(ids.data_ptr()), C.c_void_p(w.data_ptr()), _stream()))
+    return ids, w
+
+
+def moe_ffn(gate, up, down, n_experts, x, ids, weights, out=None):
+    """Decoder::moe_ffn_batch over experts stacked row-wise in three Weights: x[batch][hidden],
+    ids/weights[batch][k] -> out[batch][hidden]."""
+    import torch
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous()
+    assert ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
+    batch, k = ids.shape
+    y = out if out is not None else torch.empty((batch, down.rows // n_experts), dtype=torch.float32, device=x.device)
+    check(lib().frk_hip_moe_ffn_dev(gate.handle, up.handle, down.handle, n_experts, C.c_void_p(x.data_ptr()), batch,
+                                    C.c_void_p(ids.data_ptr()), C.c_void_p(weights.data_ptr()), k,
+                                    C.c_void_p(y.data_ptr()), _stream()))
+    return y
+
+
+def moe_intermediates(batch, k, n_experts, hidden, ffn):
+    """Test hook: (gate_out, up_out, act_q, act_d, pos_of) of the last moe_ffn call of this shape."""
+    import torch
+    pairs = batch * k
+    g = torch.empty((pairs, ffn), dtype=torch.float32, device="cuda")
+    u = torch.empty((pairs, ffn), dtype=torch.float32, device="cuda")
+    q = torch.empty((pairs, ffn), dtype=torch.int8, device="cuda")
+    d = torch.empty((pairs, ffn // 256), dtype=torch.float32, device="cuda")
+    pos = torch.empty((batch, k), dtype=torch.int32, device="cuda")
+    check(lib().frk_hip_moe_intermediates_dev(batch, k, n_experts, hidden, ffn, *(C.c_void_p(t.data_ptr())
+                                              for t in (g, u, q, d, pos)), _stream()))
+    return g, u, q, d, pos
 
 
 # ---- host-buffer entry points: numpy in, numpy out ----

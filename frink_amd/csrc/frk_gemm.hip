@@ -58,6 +58,12 @@ struct GemmArgs {
     const int8_t *bs_lo;
     float *y;             // [M][rows]
     int row_tiles, tok_tiles;
+    // grouped (per-expert) form: tile t covers output rows first..first+count of expert e, whose
+    // weights are rows [e*rows, (e+1)*rows) of W; activation row of output row p is gather[p]
+    // (p itself when gather is null).  Tiles past *n_tiles exit at once.
+    const int4 *tiles;    // {expert, first, count, 0}
+    const int *n_tiles;
+    const int *gather;
 };
 
 // One block's worth of global loads in flight: a lane's weights and a thread's share of the
@@ -74,7 +80,7 @@ struct GemmPrefetch {
 // tokens; they share an activation tile of 32*MT*WT tokens staged through LDS.  Nothing but
 // activations goes through LDS.  With WT = 2 there are two wavefronts per SIMD, so one's epilogue
 // arithmetic runs under the other's MFMAs.
-template <int MT, int WT>
+template <int MT, int WT, bool GROUPED>
 __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
     constexpr int TM = 32 * MT * WT;  // tokens per workgroup
     static_assert(TM * 4 <= 256, "activation staging assumes one pass of 256 threads");
@@ -87,24 +93,42 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lg = lane >> 5;
 
-    // workgroups that share weight rows (different token tiles) sit on one XCD (block id mod 8)
     const int bid = blockIdx.x;
-    const int per_group = 8 * g.tok_tiles;
-    const int grp = bid / per_group, in_grp = bid % per_group;
-    const int row_tile = grp * 8 + (in_grp & 7), tok_tile = in_grp >> 3;
-    if (row_tile >= g.row_tiles) return;  // uniform per workgroup
+    int row_tile, tok0, n_tok, w_first_row;
+    if (GROUPED) {
+        row_tile = bid % g.row_tiles;
+        const int t = bid / g.row_tiles;
+        if (t >= *g.n_tiles) return;  // uniform per workgroup
+        const int4 ti = g.tiles[t];
+        tok0 = ti.y;
+        n_tok = ti.y + ti.z;  // one past the last output row of this tile
+        w_first_row = ti.x * g.rows;
+    } else {
+        // workgroups that share weight rows (different token tiles) sit on one XCD (block id mod 8)
+        const int per_group = 8 * g.tok_tiles;
+        const int grp = bid / per_group, in_grp = bid % per_group;
+        row_tile = grp * 8 + (in_grp & 7);
+        if (row_tile >= g.row_tiles) return;  // uniform per workgroup
+        tok0 = (in_grp >> 3) * TM;
+        n_tok = g.M;
+        w_first_row = 0;
+    }
     const int wtok = wave >> 2;  // token group of this wavefront
     const int row = row_tile * 128 + (wave & 3) * 32 + li;
-    const int tok0 = tok_tile * TM;
     const int K = g.nb * QK_K;
+    // activation row that feeds output row tok0 + t (clamped into the tile)
+    auto act_row = [&](int t) {
+        const int p = min(tok0 + min(t, TM - 1), n_tok - 1);
+        return (GROUPED && g.gather) ? g.gather[p] : p;
+    };
 
     // weight side: this lane's row, bytes 16*lg.. of every 32-byte nibble pair
-    const uint8_t *wrow = g.W + (size_t)min(row, g.rows - 1) * g.row_stride;
+    const uint8_t *wrow = g.W + (size_t)(w_first_row + min(row, g.rows - 1)) * g.row_stride;
     // activation side: thread t moves the 64 bytes (t & 3) of token t >> 2, 16 digit bytes of
     // token t >> 1 and the block scale of token t
-    const int8_t *s_src = g.aq + (size_t)min(tok0 + min(tid >> 2, TM - 1), g.M - 1) * K + (tid & 3) * 64;
-    const int8_t *d_src = ((tid & 1) ? g.bs_lo : g.bs_hi) + (size_t)min(tok0 + min(tid >> 1, TM - 1), g.M - 1) * g.nb * 16;
-    const float *a_src = g.ad + (size_t)min(tok0 + min(tid, TM - 1), g.M - 1) * g.nb;
+    const int8_t *s_src = g.aq + (size_t)act_row(tid >> 2) * K + (tid & 3) * 64;
+    const int8_t *d_src = ((tid & 1) ? g.bs_lo : g.bs_hi) + (size_t)act_row(tid >> 1) * g.nb * 16;
+    const float *a_src = g.ad + (size_t)act_row(tid) * g.nb;
 
     auto issue_loads = [&](GemmPrefetch &pf, int kb) {
         const uint8_t *blk = wrow + (size_t)kb * Q4_K_BYTES;
@@ -241,17 +265,11 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
     lds_barrier();
 
     for (int kb = 0; kb < g.nb; kb++) {
-#ifndef GM_SKIP_COMPUTE
         compute_block(kb);
-#endif
         if (kb + 1 < g.nb) {
             store_stage(pf, (kb + 1) & 1);  // the other stage: nobody reads it during this iteration
-#ifndef GM_SKIP_UNPACK
             unpack(pf);
-#endif
-#ifndef GM_SKIP_LOADS
             if (kb + 2 < g.nb) issue_loads(pf, kb + 2);
-#endif
         }
         lds_barrier();
     }
@@ -262,7 +280,7 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (wtok * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < n_tok) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
         }
 }
 
@@ -285,10 +303,8 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     float *d = (float *)((char *)ws + round_up(n, 256));
     int8_t *bh = (int8_t *)((char *)d + round_up(n / QK_K * 4, 256));
     int8_t *bl = bh + round_up(n / 16, 256);
-    const size_t nblk = n / QK_K;
-    hipLaunchKernelGGL(quantize_q8_k_gemm_kernel, dim3((unsigned)((nblk + 3) / 4)), dim3(256), 0, s, x, nblk, q, d, bh,
-                       bl);
-    FRK_LAUNCH_CHECK("quantize_q8_k_gemm");
+    int rc = launch_quantize_q8_k_gemm(x, n, q, d, bh, bl, s);
+    if (rc) return rc;
 
     GemmArgs g;
     g.W = w->dev;
@@ -301,6 +317,9 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.bs_hi = bh;
     g.bs_lo = bl;
     g.y = y;
+    g.tiles = nullptr;
+    g.n_tiles = nullptr;
+    g.gather = nullptr;
     g.row_tiles = (int)((w->rows + 127) / 128);
     const int wt = M > 32 ? 2 : 1;  // token groups per workgroup, one 32-token tile per wavefront
     const int tm = 32 * wt;
@@ -308,9 +327,48 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     const int groups = (g.row_tiles + 7) / 8;
     const unsigned grid = (unsigned)(groups * 8 * g.tok_tiles);
     const size_t shmem = 2 * ((size_t)tm * GM_LDW + (size_t)tm * 36);
-    if (wt == 2) hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 2>), dim3(grid), dim3(512), shmem, s, g);
-    else hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 1>), dim3(grid), dim3(256), shmem, s, g);
+    if (wt == 2) hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 2, false>), dim3(grid), dim3(512), shmem, s, g);
+    else hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 1, false>), dim3(grid), dim3(256), shmem, s, g);
     FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
+    return FRK_OK;
+}
+
+
+int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, int8_t *bs_hi, int8_t *bs_lo,
+                              hipStream_t s) {
+    const size_t nblk = n / QK_K;
+    if (nblk == 0) return FRK_OK;
+    hipLaunchKernelGGL(quantize_q8_k_gemm_kernel, dim3((unsigned)((nblk + 3) / 4)), dim3(256), 0, s, x, nblk, q, d,
+                       bs_hi, bs_lo);
+    FRK_LAUNCH_CHECK("quantize_q8_k_gemm");
+    return FRK_OK;
+}
+
+// Grouped GEMM over the experts stacked in `w` (expert e = rows [e*rows_e, (e+1)*rows_e)):
+// y[p][rows_e] for every output row p listed in the tiles (32 rows per tile at most).
+int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
+                             const int8_t *bs_hi, const int8_t *bs_lo, const int4 *tiles, const int *n_tiles,
+                             int max_tiles, const int *gather, float *y, hipStream_t s) {
+    GemmArgs g;
+    g.W = w->dev;
+    g.row_stride = w->layout.row_stride;
+    g.rows = (int)rows_e;
+    g.nb = (int)(w->cols / QK_K);
+    g.M = 0;
+    g.aq = aq;
+    g.ad = ad;
+    g.bs_hi = bs_hi;
+    g.bs_lo = bs_lo;
+    g.y = y;
+    g.tiles = tiles;
+    g.n_tiles = n_tiles;
+    g.gather = gather;
+    g.row_tiles = (int)((rows_e + 127) / 128);
+    g.tok_tiles = max_tiles;
+    const unsigned grid = (unsigned)(g.row_tiles * max_tiles);
+    const size_t shmem = 2 * ((size_t)32 * GM_LDW + (size_t)32 * 36);
+    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 1, true>), dim3(grid), dim3(256), shmem, s, g);
+    FRK_LAUNCH_CHECK("gemm_q4_k_grouped");
     return FRK_OK;
 }
 

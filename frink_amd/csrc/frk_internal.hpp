@@ -122,6 +122,22 @@ int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+// Q8_K quantization in the GEMM's form: bsums split into digits bs = 64*hi + lo, hi in [-32, 31], lo in [0, 63]
+int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, int8_t *bs_hi, int8_t *bs_lo,
+                              hipStream_t s);
+// grouped (per-expert) GEMM: tiles {expert, first, count, 0} of at most 32 output rows each
+int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
+                             const int8_t *bs_hi, const int8_t *bs_lo, const int4 *tiles, const int *n_tiles,
+                             int max_tiles, const int *gather, float *y, hipStream_t s);
+// MoE expert FFN over stacked Q4_K experts; ws must hold moe_workspace_bytes(...)
+size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);
+int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
+                   const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
+                   void *ws, hipStream_t s);
+int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hidden, int ffn, float *gate_out,
+                           float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of, hipStream_t s);
+int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, int k, int norm, int32_t *ids,
+                               float *weights, hipStream_t s);
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
 

@@ -395,6 +395,58 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     return FRK_OK;
 }
 
+int frk_hip_route_top_k_softmax_dev(const float *logits, size_t batch, size_t n_experts, size_t k, int norm,
+                                    int32_t *ids, float *weights, void *stream) {
+    clear_error();
+    if (!logits || !ids || !weights) return set_error(FRK_ERR_ARG, "frk_hip_route_top_k_softmax_dev: null argument");
+    if (batch == 0 || n_experts == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=%zu experts=%zu", batch, n_experts);
+    if (k == 0 || k > n_experts)
+        return set_error(FRK_ERR_SHAPE, "top-k %zu must be between 1 and the %zu experts", k, n_experts);
+    return launch_route_top_k_softmax(logits, (int)batch, (int)n_experts, (int)k, norm, ids, weights,
+                                      (hipStream_t)stream);
+}
+
+int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t n_experts,
+                        const float *x, size_t batch, const int32_t *ids, const float *weights, size_t k, float *out,
+                        void *stream) {
+    clear_error();
+    if (!gate || !up || !down || !x || !ids || !weights || !out)
+        return set_error(FRK_ERR_ARG, "frk_hip_moe_ffn_dev: null argument");
+    if (batch == 0 || n_experts == 0 || k == 0)
+        return set_error(FRK_ERR_SHAPE, "empty shape: batch=%zu experts=%zu k=%zu", batch, n_experts, k);
+    if (n_experts > 1024 || k > 64 || k > n_experts)
+        return set_error(FRK_ERR_SHAPE, "experts=%zu (max 1024), k=%zu (max 64, at most the expert count)", n_experts, k);
+    if (gate->kind != FRK_KIND_Q4_K || up->kind != FRK_KIND_Q4_K || down->kind != FRK_KIND_Q4_K)
+        return set_error(FRK_ERR_UNSUPPORTED, "the grouped expert GEMM takes Q4_K experts (got kinds %d/%d/%d)", gate->kind,
+                         up->kind, down->kind);
+    if (gate->rows % n_experts || down->rows % n_experts)
+        return set_error(FRK_ERR_SHAPE, "stacked rows %zu/%zu do not divide into %zu experts", gate->rows, down->rows,
+                         n_experts);
+    const size_t ffn = gate->rows / n_experts, hidden = down->rows / n_experts;
+    if (up->rows != gate->rows || up->cols != gate->cols || gate->cols != hidden || down->cols != ffn)
+        return set_error(FRK_ERR_SHAPE,
+                         "expert shapes disagree: gate %zux%zu up %zux%zu down %zux%zu over %zu experts (hidden %zu, ffn %zu)",
+                         gate->rows, gate->cols, up->rows, up->cols, down->rows, down->cols, n_experts, hidden, ffn);
+    if (batch * k > (size_t)1 << 30) return set_error(FRK_ERR_SHAPE, "batch*k = %zu pairs is too many", batch * k);
+    void *ws = nullptr;
+    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);
+    if (rc) return rc;
+    return launch_moe_ffn(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, ws, (hipStream_t)stream);
+}
+
+int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size_t hidden, size_t ffn,
+                                  float *gate_out, float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of,
+                                  void *stream) {
+    clear_error();
+    if (batch == 0 || k == 0 || n_experts == 0 || hidden == 0 || ffn == 0)
+        return set_error(FRK_ERR_SHAPE, "frk_hip_moe_intermediates_dev: empty shape");
+    void *ws = nullptr;
+    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);
+    if (rc) return rc;
+    return moe_copy_intermediates(ws, batch, (int)k, (int)n_experts, (int)hidden, (int)ffn, gate_out, up_out, act_q,
+                                  act_d, pos_of, (hipStream_t)stream);
+}
+
 // ---- host-buffer entry points ----
 
 static int stage_buffers(size_t x_bytes, size_t y_bytes) {

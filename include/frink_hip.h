@@ -146,7 +146,33 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float 
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
                      void *stream);
 
+/* frink_moe::route_top_k_softmax (crates/frink-moe/src/lib.rs:567-589) for a batch of tokens:
+ * logits[batch][n_experts] -> ids[batch][k] (probability descending), weights[batch][k]
+ * (probs[ids], divided by their sum when norm != 0).  Equal probabilities, which the reference's
+ * unstable sort leaves undefined, resolve to the lower expert id. */
+int frk_hip_route_top_k_softmax_dev(const float *logits_dev, size_t batch, size_t n_experts, size_t k,
+                                    int norm, int32_t *ids_dev, float *weights_dev, void *stream);
+
+/* Decoder::moe_ffn_batch (crates/frink-models/src/decoder/ffn_batch.rs:343-434) with SwiGLU experts
+ * (frink_moe::run_expert, crates/frink-moe/src/lib.rs:1068-1165): out[batch][hidden] =
+ * sum over each token's k routed experts, in ascending expert id, of
+ * weights * down_e(silu(gate_e x) * up_e x).  gate/up/down hold the experts stacked row-wise
+ * (expert e = rows [e*ffn, (e+1)*ffn) of gate and up, [e*hidden, (e+1)*hidden) of down), Q4_K.
+ * ids[batch][k] / weights[batch][k] are a RoutingDecision per token (lib.rs:112-115); an id outside
+ * [0, n_experts) contributes nothing. */
+int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down,
+                        size_t n_experts, const float *x_dev, size_t batch, const int32_t *ids_dev,
+                        const float *weights_dev, size_t k, float *out_dev, void *stream);
+
 /* Test hooks for the bit-exact gates. */
+/* What the last frk_hip_moe_ffn_dev call of this shape on this stream left behind, copied out
+ * (null = skip): the gate and up projections [batch*k][ffn], silu(gate)*up quantized to Q8_K
+ * (act_q [batch*k][ffn] i8, act_d [batch*k][ffn/256] f32), rows in grouped order, and
+ * pos_of[tok*k + slot] = the row of a (token, slot) pair (the reference's bucket order,
+ * crates/frink-models/src/decoder/ffn_batch.rs:362-386). */
+int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size_t hidden, size_t ffn,
+                                  float *gate_out_dev, float *up_out_dev, int8_t *act_q_dev,
+                                  float *act_d_dev, int32_t *pos_of_dev, void *stream);
 /* quantize_activations_q8_k over n = 256*k values: q[n] i8, d[n/256] f32, bsums[n/16] i16 */
 int frk_hip_quantize_q8_k_dev(const float *x_dev, size_t n, int8_t *q_dev, float *d_dev,
                               int16_t *bsums_dev, void *stream);
