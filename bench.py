@@ -23,6 +23,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA
 COPIES = 16
 
 
@@ -207,6 +208,42 @@ def main():
                            "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
             for w in w2:
                 w.release()
+        # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step
+        # (activation quantization is inside the step)
+        xb = torch.from_numpy(synth.activations(6, 512, cols, outlier_frac=0.01)).to(dev)
+        for name, r2 in (("Q4_K GEMM M=512 4096x4096", 4096), ("Q4_K GEMM M=512 14336x4096", 14336)):
+            d2 = torch.from_numpy(random_blocks(kind, r2, cols, seed=78)).to(dev)
+            w2 = [fa.Weights.from_device(kind, d2, r2, cols) for _ in range(4)]
+            yb = torch.empty((512, r2), dtype=torch.float32, device=dev)
+
+            def step3(i):
+                w2[i % 4].gemm(xb, out=yb)
+            _, t = time_graph(torch, step3, 200, 4)
+            tops = 2.0 * 512 * r2 * cols / (t / 200) / 1e12
+            extra[name] = {"TOPS": round(tops, 1), "us_per_step": round(t / 200 * 1e6, 2),
+                           "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            for w in w2:
+                w.release()
+        # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
+        E, K, H, F, T = 128, 8, 2048, 768, 512
+        experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)
+                   for j, (r, c) in enumerate(((E * F, H), (E * F, H), (E * H, F)))]
+        xm = torch.from_numpy(synth.activations(7, T, H)).to(dev)
+        logits = torch.from_numpy(synth.normal(8, T * E).reshape(T, E)).to(dev)
+        ids, wts = fa.route_top_k_softmax(logits, K, True)
+        ym = torch.empty((T, H), dtype=torch.float32, device=dev)
+
+        def step4(i):
+            fa.moe_ffn(experts[0], experts[1], experts[2], E, xm, ids, wts, out=ym)
+        _, t = time_graph(torch, step4, 100, 2)
+        moe_bytes = 3 * E * F * H // 256 * 144 + 2 * T * H * 4 + 2 * T * K * 4
+        extra["MoE layer 128x top-8, 2048/768, 512 tokens"] = {
+            "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
+            "algorithmic_GBs": round(moe_bytes / (t / 100) / 1e9, 1),
+            "frac_of_hbm_peak": round(moe_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4),
+            "TOPS": round(2.0 * T * K * 3 * F * H / (t / 100) / 1e12, 1)}
+        for w in experts:
+            w.release()
         out["extra"] = extra
 
     if not args.no_cpu:

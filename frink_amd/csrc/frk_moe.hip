@@ -7,41 +7,84 @@
 
 namespace frk {
 
-// route_top_k_softmax (crates/frink-moe/src/lib.rs:567-589): one thread per token, the same
-// sequential f32 sums as the reference; among equal probabilities the lowest index wins (the
-// reference's unstable sort leaves that case undefined).
-__global__ void route_top_k_softmax_kernel(const float *__restrict__ logits, int batch, int n_experts, int k,
-                                           int norm, int32_t *__restrict__ ids, float *__restrict__ weights) {
-    const int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b >= batch) return;
+// route_top_k_softmax (crates/frink-moe/src/lib.rs:567-589): one wavefront per token.  The
+// exponentials are computed in parallel, the softmax denominator is then summed by one lane in
+// index order (the reference's sequential f32 sum); among equal probabilities the lowest index
+// wins (the reference's unstable sort leaves that case undefined).  n_experts <= 1024, k <= 64.
+__global__ __launch_bounds__(64) void route_top_k_softmax_kernel(const float *__restrict__ logits, int batch,
+                                                                 int n_experts, int k, int norm,
+                                                                 int32_t *__restrict__ ids,
+                                                                 float *__restrict__ weights) {
+    __shared__ float prob[1024];
+    __shared__ float s_sum;
+    const int b = blockIdx.x, lane = threadIdx.x;
     const float *l = logits + (size_t)b * n_experts;
     float mx = -INFINITY;
-    for (int i = 0; i < n_experts; i++) mx = fmaxf(mx, l[i]);
-    float sum = 0.0f;
-    for (int i = 0; i < n_experts; i++) sum += expf(l[i] - mx);
-    float last = INFINITY;
-    int last_i = -1;
-    float top_sum = 0.0f;
+    for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, l[i]);
+    mx = wave_max(mx);
+    for (int i = lane; i < n_experts; i += 64) prob[i] = expf(l[i] - mx);
+    __syncthreads();
+    if (lane == 0) {
+        float sum = 0.0f;
+        for (int i = 0; i < n_experts; i++) sum += prob[i];
+        s_sum = sum;
+    }
+    __syncthreads();
+    const float sum = s_sum;
+    for (int i = lane; i < n_experts; i += 64) prob[i] = __fdiv_rn(prob[i], sum);
+    __syncthreads();
+    float top_sum = 0.0f, mine = 0.0f;  // lane s keeps the s-th weight
     for (int s = 0; s < k; s++) {
-        // next in (probability descending, index ascending) order after (last, last_i)
+        // wave argmax: larger probability, then smaller index
         float best = -1.0f;
-        int best_i = -1;
-        for (int i = 0; i < n_experts; i++) {
-            const float p = expf(l[i] - mx) / sum;
-            const bool after = p < last || (p == last && i > last_i);
-            if (after && p > best) {
+        int best_i = 0x7fffffff;
+        for (int i = lane; i < n_experts; i += 64) {
+            const float p = prob[i];
+            if (p > best) {
                 best = p;
                 best_i = i;
             }
         }
-        ids[(size_t)b * k + s] = best_i;
-        weights[(size_t)b * k + s] = best;
-        top_sum += best;
-        last = best;
-        last_i = best_i;
+#pragma unroll
+        for (int m = 1; m < 64; m <<= 1) {
+            const float ob = __shfl_xor(best, m);
+            const int oi = __shfl_xor(best_i, m);
+            if (ob > best || (ob == best && oi < best_i)) {
+                best = ob;
+                best_i = oi;
+            }
+        }
+        if (lane == 0) {
+            ids[(size_t)b * k + s] = best_i;
+            prob[best_i] = -2.0f;  // taken
+        }
+        if (lane == s) mine = best;
+        top_sum += best;  // same order in every lane: the reference's sum over the k weights
+        __syncthreads();
     }
-    if (norm)
-        for (int s = 0; s < k; s++) weights[(size_t)b * k + s] /= top_sum;
+    if (lane < k) weights[(size_t)b * k + lane] = norm ? __fdiv_rn(mine, top_sum) : mine;
+}
+
+// Exclusive scan over the workgroup's 1024 threads (16 wavefronts); `total` gets the sum.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *wave_tot, int &total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) {
+        const int o = __shfl_up(inc, m);
+        if (lane >= m) inc += o;
+    }
+    if (lane == 63) wave_tot[wave] = inc;
+    __syncthreads();
+    int base = 0, tot = 0;
+    for (int w = 0; w < 16; w++) {
+        const int t = wave_tot[w];
+        if (w < wave) base += t;
+        tot += t;
+    }
+    __syncthreads();
+    total = tot;
+    return base + inc - v;
 }
 
 // Buckets the batch*k (token, slot) pairs by expert, tokens ascending inside a bucket.
@@ -49,45 +92,74 @@ __global__ void route_top_k_softmax_kernel(const float *__restrict__ logits, int
 //   gather[pairs]    token of each grouped position
 //   pos_of[pairs]    grouped position of pair (tok*k + slot); -1 for an id outside [0, E)
 //   tiles / n_tiles  the buckets cut into runs of at most 32 positions for the grouped GEMM
-// One workgroup; E <= 1024.
+// One workgroup of 1024 threads; E <= 1024.  Pairs are taken 1024 at a time in pair order (which
+// is token-major); a pair's place in its bucket is the count of earlier pairs of that expert:
+// those of earlier rounds (run), of earlier wavefronts of this round (a prefix over the
+// per-wavefront counts) and of lower lanes of its own wavefront.
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restrict__ ids, int pairs, int k,
                                                          int n_experts, int *__restrict__ group_off,
                                                          int *__restrict__ gather, int *__restrict__ pos_of,
                                                          int4 *__restrict__ tiles, int *__restrict__ n_tiles) {
     __shared__ int cnt[1024];
-    __shared__ int off[1025];
-    const int tid = threadIdx.x;
-    for (int e = tid; e < n_experts; e += blockDim.x) cnt[e] = 0;
+    __shared__ int off[1024];
+    __shared__ int run[1024];
+    __shared__ unsigned short wcnt[16][1024];
+    __shared__ int wave_tot[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    cnt[tid] = 0;
+    run[tid] = 0;
     __syncthreads();
-    for (int p = tid; p < pairs; p += blockDim.x) {
+    for (int p = tid; p < pairs; p += 1024) {
         const int e = ids[p];
         if (e >= 0 && e < n_experts) atomicAdd(&cnt[e], 1);
         else pos_of[p] = -1;
     }
     __syncthreads();
-    if (tid == 0) {
-        int acc = 0, nt = 0;
-        for (int e = 0; e < n_experts; e++) {
-            off[e] = acc;
-            for (int t0 = 0; t0 < cnt[e]; t0 += 32) tiles[nt++] = make_int4(e, acc + t0, min(32, cnt[e] - t0), 0);
-            acc += cnt[e];
+    {
+        const int c = tid < n_experts ? cnt[tid] : 0;
+        const int nt = (c + 31) >> 5;
+        int total, total_tiles;
+        const int o = block_exclusive_scan(c, wave_tot, total);
+        const int t = block_exclusive_scan(nt, wave_tot, total_tiles);
+        off[tid] = o;
+        if (tid < n_experts) {
+            group_off[tid] = o;
+            for (int i = 0; i < nt; i++) tiles[t + i] = make_int4(tid, o + 32 * i, min(32, c - 32 * i), 0);
         }
-        off[n_experts] = acc;
-        *n_tiles = nt;
+        if (tid == 0) {
+            group_off[n_experts] = total;
+            *n_tiles = total_tiles;
+        }
     }
-    __syncthreads();
-    for (int e = tid; e <= n_experts; e += blockDim.x) group_off[e] = off[e];
-    // pair order is token-major, so walking it in order fills each bucket with ascending tokens
-    for (int e = tid; e < n_experts; e += blockDim.x) {
-        if (cnt[e] == 0) continue;
-        int pos = off[e];
-        for (int p = 0; p < pairs; p++) {
-            if (ids[p] == e) {
-                gather[pos] = p / k;
-                pos_of[p] = pos;
-                pos++;
-            }
+    for (int p0 = 0; p0 < pairs; p0 += 1024) {
+        for (int w = 0; w < 16; w++) wcnt[w][tid] = 0;
+        __syncthreads();
+        const int p = p0 + tid;
+        int e = p < pairs ? ids[p] : -1;
+        if (e >= n_experts) e = -1;
+        int rank = 0, same = 0;
+        for (int j = 0; j < 64; j++) {
+            const int ej = __shfl(e, j);
+            same += (ej == e);
+            rank += (ej == e && j < lane);
         }
+        if (e >= 0 && rank == 0) wcnt[wave][e] = (unsigned short)same;
+        __syncthreads();
+        int before = 0;
+        if (e >= 0)
+            for (int w = 0; w < wave; w++) before += wcnt[w][e];
+        if (e >= 0) {
+            const int pos = off[e] + run[e] + before + rank;
+            gather[pos] = p / k;
+            pos_of[p] = pos;
+        }
+        __syncthreads();
+        {
+            int tot = 0;
+            for (int w = 0; w < 16; w++) tot += wcnt[w][tid];
+            run[tid] += tot;
+        }
+        __syncthreads();
     }
 }
 
@@ -169,7 +241,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
 
 int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, int k, int norm, int32_t *ids,
                                float *weights, hipStream_t s) {
-    hipLaunchKernelGGL(route_top_k_softmax_kernel, dim3((batch + 63) / 64), dim3(64), 0, s, logits, batch, n_experts, k,
+    hipLaunchKernelGGL(route_top_k_softmax_kernel, dim3(batch), dim3(64), 0, s, logits, batch, n_experts, k,
                        norm, ids, weights);
     FRK_LAUNCH_CHECK("route_top_k_softmax");
     return FRK_OK;

@@ -402,6 +402,8 @@ int frk_hip_route_top_k_softmax_dev(const float *logits, size_t batch, size_t n_
     if (batch == 0 || n_experts == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=%zu experts=%zu", batch, n_experts);
     if (k == 0 || k > n_experts)
         return set_error(FRK_ERR_SHAPE, "top-k %zu must be between 1 and the %zu experts", k, n_experts);
+    if (n_experts > 1024 || k > 64)
+        return set_error(FRK_ERR_SHAPE, "experts=%zu (max 1024), k=%zu (max 64)", n_experts, k);
     return launch_route_top_k_softmax(logits, (int)batch, (int)n_experts, (int)k, norm, ids, weights,
                                       (hipStream_t)stream);
 }
