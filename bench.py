@@ -25,6 +25,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA
 COPIES = 16
+# HBM bytes per launch of the roofline kernel at 14336x4096, from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE 16163.5, WRITE_SIZE 56.0 per dispatch), each scaled by what the same counter
+# reads for copy_kernel over 32,256 KiB (FETCH_SIZE 16138.0 -> x1.9988, WRITE_SIZE 32256.0 -> x1.0).
+GEMV_TRAFFIC_BYTES = int((16163.5 * 32256.0 / 16138.0 + 56.0) * 1024)
 
 
 def random_blocks(kind, rows, cols, seed):
@@ -168,8 +172,8 @@ def main():
                    "weight_bytes": int(wbytes), "device": info["name"], "arch": info["gcn_arch"],
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_q4_k_kernel", "algorithmic_bytes": int(alg_bytes),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
+                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512>", "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
     }
 

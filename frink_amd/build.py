@@ -54,5 +54,18 @@ def build_lib(verbose=False):
     return SO
 
 
+HOST_CHECK_SRC = os.path.join(os.path.dirname(HERE), "tests", "host_mirror_check.cpp")
+HOST_CHECK_BIN = os.path.join(LIBDIR, "host_mirror_check")
+
+
+def build_host_check():
+    """The C++ host mirror's test driver (g++, host only), linked against the shared library."""
+    os.makedirs(LIBDIR, exist_ok=True)
+    subprocess.check_call(["g++", "-std=c++17", "-O1", "-Wall", HOST_CHECK_SRC, "-o", HOST_CHECK_BIN,
+                           "-L" + LIBDIR, "-lfrink_hip", "-Wl,-rpath," + LIBDIR, "-Wl,-rpath,/opt/rocm/lib"])
+    return HOST_CHECK_BIN
+
+
 if __name__ == "__main__":
     print(build_lib(verbose="-v" in sys.argv))
+    print(build_host_check())

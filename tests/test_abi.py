@@ -117,3 +117,21 @@ def test_forced_off_never_opens_a_device():
             "print(fa.lib().frk_hip_dense_enabled())" % ROOT)
     out = subprocess.check_output([sys.executable, "-c", code], text=True)
     assert out.strip() == "0"
+
+
+def _host_check_binary():
+    from frink_amd import build as fb
+    if not os.path.exists(fb.HOST_CHECK_BIN):
+        fb.build_host_check()
+    return fb.HOST_CHECK_BIN
+
+
+def test_cpp_host_mirror_without_a_device():
+    """frink_amd/host/frink_hip.hpp (the C++ form of BackendCaps / BackendDispatch) driven by
+    tests/host_mirror_check.cpp: capability tables agree over all 23 kinds, None vs Some(Err),
+    shape errors before launch, FRINK_HIP=off."""
+    import subprocess
+    env = dict(os.environ, FRINK_HIP="off")
+    r = subprocess.run([_host_check_binary()], env=env, text=True, capture_output=True, timeout=120)
+    assert r.returncode == 0 and "FAIL" not in r.stdout, r.stdout + r.stderr
+    assert "FRINK_HIP=off disables the backend" in r.stdout

@@ -407,3 +407,19 @@ def test_moe_ffn_full_size_layer(fa):
     CPU would take minutes); the expert arithmetic does not care where the bytes came from."""
     got, want = _moe_case(fa, 128, 8, 2048, 768, 512, seed=5, random_blocks=True)
     assert np.isfinite(got).all()
+
+
+# ------------------------------------------------------------------ the C++ host mirror
+
+def test_cpp_host_mirror_launches(fa):
+    """tests/host_mirror_check.cpp --gpu: probe, launch_matvec and launch_mul_mm through
+    frink_amd/host/frink_hip.hpp against closed forms."""
+    import os
+    import subprocess
+    from frink_amd import build as fb
+    if not os.path.exists(fb.HOST_CHECK_BIN):
+        fb.build_host_check()
+    env = {k: v for k, v in os.environ.items() if k != "FRINK_HIP"}
+    r = subprocess.run([fb.HOST_CHECK_BIN, "--gpu"], env=env, text=True, capture_output=True, timeout=120)
+    print(r.stdout, flush=True)
+    assert r.returncode == 0 and "FAIL" not in r.stdout, r.stdout + r.stderr
