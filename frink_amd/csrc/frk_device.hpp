@@ -41,6 +41,21 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// global_load_lds: every lane names its own global source; the wavefront's 64 pieces of BYTES
+// (4 or 16) bytes land in LDS at lds_chunk + BYTES * lane, without passing through registers.
+// Completion is counted by vmcnt like any other global load.  lds_chunk must be wavefront-uniform.
+// (The builtin exists in the device pass only, hence the guard.)
+__device__ __forceinline__ void load_to_lds16(const void *src, void *lds_chunk) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void *)lds_chunk, 16, 0, 0);
+#endif
+}
+__device__ __forceinline__ void load_to_lds4(const void *src, void *lds_chunk) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_global_load_lds(src, (__attribute__((address_space(3))) void *)lds_chunk, 4, 0, 0);
+#endif
+}
+
 constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
 constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
 constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <- lane 7-i of its group of 8

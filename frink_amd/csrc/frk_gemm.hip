@@ -1,13 +1,14 @@
-// Prefill / batched GEMM over Q4_K weights on the int8 matrix cores:
+// Prefill / batched GEMM over Q4_K weights on the matrix cores:
 //   y[tok][row] = sum_k W[row][k] * x[tok][k],  x quantized per token to Q8_K first.
 //
 // Arithmetic is dot_q4_k_q8's (crates/frink-quant/src/lib.rs:822-869), regrouped so that a whole
-// 256-weight block accumulates in int32 inside the MFMA:
-//   sum_j sc_j * isum_j      with sc_j = 8*sh_j + sl_j (sh, sl < 8): a weight row's block becomes two
-//                            int8 operand planes  H = sh_j * q  and  L = sl_j * q  (each < 106), so
-//                            sum = 8 * (acts . H) + (acts . L), exact, no per-sub-block rescale;
-//   sum_j m_j * bsum_j       the activation's 16-wide sums are split as bsum = 64*hi + lo (both int8)
-//                            and multiplied by the 6-bit mins on the K=16 MFMA: 64*(hi . m) + (lo . m).
+// 256-weight block accumulates inside the MFMA:
+//   S1 = sum_j sc_j * isum_j   with sc_j = 8*sh_j + sl_j (sh, sl < 8): a weight row's block becomes two
+//                              int8 operand planes  H = sh_j * q  and  L = sl_j * q  (each < 106), so
+//                              S1 = 8 * (acts . H) + (acts . L), exact, no per-sub-block rescale;
+//   S2 = sum_j m_j * bsum_j    the activation's 16-wide sums (|bsum| <= 2032) and the 6-bit mins are both
+//                              exact in f16, their products and the 16-term sum exact in f32, so one
+//                              v_mfma_f32_32x32x16_f16 gives S2 already as a float.
 // Per block and output the epilogue is then  acc += da * (d * S1 - dmin * S2)  in f32.
 // (Scaling each sub-block's product after a K=32 MFMA instead -- one v_mad_i32_i24 per result and
 // sub-block -- was measured slower here: it is bound by the vector ALU and needs more registers.)
@@ -15,24 +16,31 @@
 // MFMA operand roles: A = activations (tile row = token), B = weights (tile column = weight row), so
 // a lane's 16 results share one weight row (its d, dmin are per-lane values) and span 16 tokens.
 // Operand layout of v_mfma_i32_32x32x32_i8 (checked on the device): lane l holds, for row/column
-// l % 32, the 16 k-values 16*(l/32) .. +15; result register r of lane l is
-// D[8*(r/4) + 4*(l/32) + r%4][l % 32].
+// l % 32, the 16 k-values 16*(l/32) .. +15 (8*(l/32) .. +7 for the K=16 f16 form); result register
+// r of lane l is D[8*(r/4) + 4*(l/32) + r%4][l % 32].
+//
+// Data movement: everything a block needs -- the workgroup's 128 weight rows (raw 144-byte blocks)
+// and its activation tile -- goes from global memory straight into LDS with global_load_lds_dwordx4
+// (the 64 lanes' 16-byte pieces land in 1 KB of consecutive LDS; each lane chooses which piece it
+// fetches, so the LDS image is whatever order the consumer wants), several blocks ahead, in rings of
+// stages.  No prefetch lives in registers, and the only waits on memory are "the stage issued P
+// iterations ago has landed".
 #include "frk_device.hpp"
 
 namespace frk {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 
-constexpr int GM_LDW = 272;  // LDS bytes per token and block: 256 quants + 16 of padding (bank spread)
-
-// Activation side: Q8_K quantization plus the base-64 digits of the 16-wide sums.
+// Activation side: Q8_K quantization plus the 16-wide sums as f16 (exact: |bsum| <= 16*127).
 // One wavefront per 256-value block.
 __global__ __launch_bounds__(256) void quantize_q8_k_gemm_kernel(const float *__restrict__ x, size_t n_blocks,
                                                                  int8_t *__restrict__ q, float *__restrict__ d,
-                                                                 int8_t *__restrict__ bs_hi,
-                                                                 int8_t *__restrict__ bs_lo) {
+                                                                 _Float16 *__restrict__ bsf) {
     const int lane = threadIdx.x & 63;
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= n_blocks) return;
@@ -41,10 +49,7 @@ __global__ __launch_bounds__(256) void quantize_q8_k_gemm_kernel(const float *__
     int bs;
     const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
     reinterpret_cast<uint32_t *>(q + b * QK_K)[lane] = packed;
-    if ((lane & 3) == 0) {
-        bs_hi[b * 16 + (lane >> 2)] = (int8_t)(bs >> 6);  // floor(bs / 64) in [-32, 31]
-        bs_lo[b * 16 + (lane >> 2)] = (int8_t)(bs & 63);
-    }
+    if ((lane & 3) == 0) bsf[b * 16 + (lane >> 2)] = (_Float16)bs;
     if (lane == 0) d[b] = dd;
 }
 
@@ -54,8 +59,7 @@ struct GemmArgs {
     int rows, nb, M;
     const int8_t *aq;     // [M][nb*256]
     const float *ad;      // [M][nb]
-    const int8_t *bs_hi;  // [M][nb*16]
-    const int8_t *bs_lo;
+    const _Float16 *bsf;  // [M][nb*16]
     float *y;             // [M][rows]
     int row_tiles, tok_tiles;
     // grouped (per-expert) form: tile t covers output rows first..first+count of expert e, whose
@@ -66,32 +70,222 @@ struct GemmArgs {
     const int *gather;
 };
 
-// One block's worth of global loads in flight: a lane's weights and a thread's share of the
-// activation tile, requested one block-iteration before they are needed.
-struct GemmPrefetch {
-    uint4 wh, wq0, wq1, wq2, wq3;  // header, the lane's 16-byte half of each 32-byte nibble pair
-    uint4 sa0, sa1, sa2, sa3, sdig;
-    float sda;
+// One block of a lane's weight row as MFMA B operands: the two pre-scaled planes of the 8 sub-blocks,
+// the mins as f16 and the block's two f32 scales.  (Named members, not arrays: they must stay in
+// registers.)
+struct BPlanes {
+    v4i H0, H1, H2, H3, H4, H5, H6, H7;
+    v4i L0, L1, L2, L3, L4, L5, L6, L7;
+    v8h m;
+    float d, ndmin;
+};
+struct RawBlock {  // header + the lane's 16-byte half of each 32-byte nibble pair, as read from LDS
+    v4i wh, q0, q1, q2, q3;
+};
+struct TileOperands {  // one 32-token tile of a block: 8 k-slices of quants and the bsums
+    v4i a0, a1, a2, a3, a4, a5, a6, a7;
+    v8h bs;
+};
+struct TileScales {  // the tile's 16 block scales this lane's results need
+    v4f da0, da1, da2, da3;
+};
+struct TileAcc {
+    v16i s1;  // sum_j sc_j * isum_j
+    v16f s2;  // sum_j m_j * bsum_j
 };
 
-// A wavefront owns 32 weight rows and keeps their current block in registers, already unpacked
-// into MFMA B operands (a lane holds k = 16g..16g+15 of row l%32 for each of the 8 sub-blocks).
-// The workgroup has 4*WT wavefronts: four row groups (128 rows) times WT token groups of 32*MT
-// tokens; they share an activation tile of 32*MT*WT tokens staged through LDS.  Nothing but
-// activations goes through LDS.  With WT = 2 there are two wavefronts per SIMD, so one's epilogue
-// arithmetic runs under the other's MFMAs.
-template <int MT, int WT, bool GROUPED>
-__global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
-    constexpr int TM = 32 * MT * WT;  // tokens per workgroup
-    static_assert(TM * 4 <= 256, "activation staging assumes one pass of 256 threads");
-    constexpr int OFF_DIG = TM * GM_LDW;
-    constexpr int OFF_DA = OFF_DIG + TM * 32;
-    constexpr int STAGE = OFF_DA + TM * 4;
+// LDS reads are issued from inline assembly so that the compiler's wait-count insertion does not see
+// them: it cannot tell that an LDS read does not alias a stage a global_load_lds is still filling
+// and would wait for vmcnt(0), i.e. for the whole prefetch, in front of every read.  The price is
+// that the waits are placed by hand.  LDS operations of a wavefront complete in order, so
+// "at most N outstanding" means everything but the N youngest reads has arrived; each wait names the
+// registers it releases so that their uses cannot be scheduled above it.
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+#else
+    return 0;
+#endif
+}
+
+#define FRK_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
+
+__device__ __forceinline__ void read_raw(RawBlock &R, uint32_t header, uint32_t quants) {
+    FRK_DS_READ(R.wh, header, 0);
+    FRK_DS_READ(R.q0, quants, 16);
+    FRK_DS_READ(R.q1, quants, 48);
+    FRK_DS_READ(R.q2, quants, 80);
+    FRK_DS_READ(R.q3, quants, 112);
+}
+__device__ __forceinline__ void read_ops(TileOperands &T, uint32_t quants, uint32_t bsums) {
+    FRK_DS_READ(T.a0, quants, 0);
+    FRK_DS_READ(T.a1, quants, 1024);
+    FRK_DS_READ(T.a2, quants, 2048);
+    FRK_DS_READ(T.a3, quants, 3072);
+    FRK_DS_READ(T.a4, quants, 4096);
+    FRK_DS_READ(T.a5, quants, 5120);
+    FRK_DS_READ(T.a6, quants, 6144);
+    FRK_DS_READ(T.a7, quants, 7168);
+    FRK_DS_READ(T.bs, bsums, 0);
+}
+// result register r belongs to token 8*(r/4) + 4*(lane/32) + r%4 of the tile
+__device__ __forceinline__ void read_scales(TileScales &S, uint32_t scales) {
+    FRK_DS_READ(S.da0, scales, 0);
+    FRK_DS_READ(S.da1, scales, 32);
+    FRK_DS_READ(S.da2, scales, 64);
+    FRK_DS_READ(S.da3, scales, 96);
+}
+template <int N>
+__device__ __forceinline__ void wait_ops(TileOperands &T) {
+    asm volatile("s_waitcnt lgkmcnt(%9)"
+                 : "+v"(T.a0), "+v"(T.a1), "+v"(T.a2), "+v"(T.a3), "+v"(T.a4), "+v"(T.a5), "+v"(T.a6), "+v"(T.a7),
+                   "+v"(T.bs)
+                 : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_scales(TileScales &S) {
+    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(S.da0), "+v"(S.da1), "+v"(S.da2), "+v"(S.da3) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_raw(RawBlock &R) {
+    asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(R.wh), "+v"(R.q0), "+v"(R.q1), "+v"(R.q2), "+v"(R.q3) : "n"(N));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// raw block -> operand planes.  lg = lane / 32 selects which half of every sub-block this lane holds.
+__device__ __forceinline__ void unpack_block(const RawBlock &R, int lg, BPlanes &B) {
+    const uint32_t hx = (uint32_t)R.wh.x, hy = (uint32_t)R.wh.y, hz = (uint32_t)R.wh.z, hw = (uint32_t)R.wh.w;
+    const uint32_t sc_lo = hy & 0x3f3f3f3fu, m_lo = hz & 0x3f3f3f3fu;
+    const uint32_t sc_hi = (hw & 0x0f0f0f0fu) | (((hy >> 6) & 0x03030303u) << 4);
+    const uint32_t m_hi = ((hw >> 4) & 0x0f0f0f0fu) | (((hz >> 6) & 0x03030303u) << 4);
+    // one nibble pair: 16 bytes -> the lane's H and L operands of sub-blocks 2p and 2p+1
+    auto pair = [&](const v4i q, const uint32_t scw, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
+        const uint32_t s0 = scw & 0xff, s1 = (scw >> 8) & 0xff;
+        const us2 h0 = {(unsigned short)(s0 >> 3), (unsigned short)(s0 >> 3)};
+        const us2 l0 = {(unsigned short)(s0 & 7), (unsigned short)(s0 & 7)};
+        const us2 h1 = {(unsigned short)(s1 >> 3), (unsigned short)(s1 >> 3)};
+        const us2 l1 = {(unsigned short)(s1 & 7), (unsigned short)(s1 & 7)};
+        auto one = [&](const int wi, int &o0, int &o1, int &o2, int &o3) {
+            const uint32_t w = (uint32_t)wi;
+            const uint32_t nl = w & 0x0f0f0f0fu, nh = (w >> 4) & 0x0f0f0f0fu;
+            us2 a, b;
+            __builtin_memcpy(&a, &nl, 4);
+            __builtin_memcpy(&b, &nh, 4);
+            const us2 r0 = a * h0, r1 = a * l0, r2 = b * h1, r3 = b * l1;  // bytes stay below 106
+            __builtin_memcpy(&o0, &r0, 4);
+            __builtin_memcpy(&o1, &r1, 4);
+            __builtin_memcpy(&o2, &r2, 4);
+            __builtin_memcpy(&o3, &r3, 4);
+        };
+        int a0, a1, a2, a3, b0, b1, b2, b3, c0, c1, c2, c3, d0, d1, d2, d3;
+        one(q.x, a0, a1, a2, a3);
+        one(q.y, b0, b1, b2, b3);
+        one(q.z, c0, c1, c2, c3);
+        one(q.w, d0, d1, d2, d3);
+        H0 = v4i{a0, b0, c0, d0};  // sub-block 2p: low nibbles
+        L0 = v4i{a1, b1, c1, d1};
+        H1 = v4i{a2, b2, c2, d2};  // sub-block 2p+1: high nibbles
+        L1 = v4i{a3, b3, c3, d3};
+    };
+    pair(R.q0, sc_lo, B.H0, B.L0, B.H1, B.L1);
+    pair(R.q1, sc_lo >> 16, B.H2, B.L2, B.H3, B.L3);
+    pair(R.q2, sc_hi, B.H4, B.L4, B.H5, B.L5);
+    pair(R.q3, sc_hi >> 16, B.H6, B.L6, B.H7, B.L7);
+    // mins of the four sub-blocks whose 16-wide groups are 8*lg .. 8*lg+7, each twice
+    const uint32_t mw = lg ? m_hi : m_lo;
+    const _Float16 m0 = (_Float16)(int)(mw & 0xff), m1 = (_Float16)(int)((mw >> 8) & 0xff);
+    const _Float16 m2 = (_Float16)(int)((mw >> 16) & 0xff), m3 = (_Float16)(int)(mw >> 24);
+    B.m = v8h{m0, m0, m1, m1, m2, m2, m3, m3};
+    B.d = h2f(hx & 0xffffu);
+    B.ndmin = -h2f(hx >> 16);
+}
+
+// S1 = 8 * (acts . H) + (acts . L) in ONE accumulator: the H chain first, its result shifted left by
+// three, then the L chain on top of it.  (Two accumulators would cost 16 more registers per lane.)
+__device__ __forceinline__ void tile_mfmas(const TileOperands &T, const BPlanes &B, TileAcc &X) {
+    const v16i zi = {0};
+    const v16f zf = {0.0f};
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);  // runs while the shift waits
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+}
+
+__device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales &S, const BPlanes &B, v16f &acc) {
+    const v4f dav[4] = {S.da0, S.da1, S.da2, S.da3};
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int r = c * 4 + e;
+            const float v = fmaf(B.ndmin, X.s2[r], B.d * (float)X.s1[r]);
+            acc[r] = fmaf(dav[c][e], v, acc[r]);
+        }
+}
+
+// A workgroup = RG*WT wavefronts = RG row groups of 32 weight rows x WT token groups of MT 32-token
+// tiles.  A wavefront keeps the current block of its 32 rows in registers as MFMA B operands and
+// runs its MT tiles against them, so a block of a row is unpacked once per MT tiles.  A SIMD holds
+// two wavefronts: while one issues a tile's MFMAs the other does its vector work (unpack,
+// epilogue), which is how the matrix cores and the vector ALU overlap here.
+//
+// What bounds the tile shape: every block moves (32*RG*144 + 32*NT*292) bytes from L2 into LDS for
+// 2*32*RG*32*NT*256 operations, and the L2-to-LDS path sustained roughly 9 TB/s over the chip when
+// measured with the arithmetic switched off, so more rows and tokens per workgroup is better -- until
+// the registers run out: 256 rows x 64 tokens (8 wavefronts, two tiles each) is the largest shape
+// that compiles without spills at two wavefronts per SIMD (256 registers per lane), and a spill is
+// fatal here because scratch reloads wait on the same counter as the prefetch.
+//
+// LDS rings.  Activations, 2 stages:
+//     quants [NT][8 k-slices][1 KB] | bsums f16 [NT][1 KB] | scales f32 [NT*32],  NT = MT*WT tiles
+// weights, WS stages of [RG][32 rows][144 B] raw blocks; block kb+1 is unpacked at the end of
+// iteration kb, so with WS = 2 a stage is refilled two blocks ahead, with WS = 4 three.
+template <int RG, int WT, int MT, int WS>
+struct GemmLds {
+    static constexpr int NT = WT * MT;
+    static constexpr int OFF_BS = NT * 8192;
+    static constexpr int OFF_DA = NT * 9216;
+    static constexpr int A_STAGE = OFF_DA + ((NT + 1) / 2) * 256;
+    static constexpr int W_GROUP = 32 * Q4_K_BYTES;  // 4608
+    static constexpr int W_STAGE = RG * W_GROUP;
+    static constexpr size_t BYTES = (size_t)2 * A_STAGE + (size_t)WS * W_STAGE;
+};
+
+template <int RG, int WT, int MT, int WS, bool GROUPED>
+__global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
+    using L = GemmLds<RG, WT, MT, WS>;
+    constexpr int NW = RG * WT, NT = L::NT, TM = 32 * NT, ROWS = 32 * RG;
+    constexpr int N_DA = (NT + 1) / 2;
+    static_assert(NW == 4 || NW == 8, "the k-slice to wavefront map assumes 4 or 8 wavefronts");
+    static_assert(WS == 2 || WS == 4, "weight ring of 2 or 4 stages");
+    static_assert(WT == 1 || WT == 2, "one or two token groups");
+    constexpr int WD = WS == 4 ? 3 : 2;  // weights are requested WD blocks ahead
+    // global_load_lds instructions per wavefront for one block of weights
+    constexpr int C_W = WT == 1 ? 5 : 3;
     extern __shared__ uint4 smem_gemm[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
+    uint8_t *lds_w = lds + 2 * L::A_STAGE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lg = lane >> 5;
+    const int rgrp = wave % RG, tgrp = wave / RG;
 
     const int bid = blockIdx.x;
     int row_tile, tok0, n_tok, w_first_row;
@@ -113,163 +307,118 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
         n_tok = g.M;
         w_first_row = 0;
     }
-    const int wtok = wave >> 2;  // token group of this wavefront
-    const int row = row_tile * 128 + (wave & 3) * 32 + li;
+    const int row0 = row_tile * ROWS + rgrp * 32;  // this wavefront's first weight row
+    const int row = row0 + li;
     const int K = g.nb * QK_K;
+    const int nb = g.nb;
     // activation row that feeds output row tok0 + t (clamped into the tile)
     auto act_row = [&](int t) {
-        const int p = min(tok0 + min(t, TM - 1), n_tok - 1);
+        const int p = min(tok0 + t, n_tok - 1);
         return (GROUPED && g.gather) ? g.gather[p] : p;
     };
 
-    // weight side: this lane's row, bytes 16*lg.. of every 32-byte nibble pair
-    const uint8_t *wrow = g.W + (size_t)(w_first_row + min(row, g.rows - 1)) * g.row_stride;
-    // activation side: thread t moves the 64 bytes (t & 3) of token t >> 2, 16 digit bytes of
-    // token t >> 1 and the block scale of token t
-    const int8_t *s_src = g.aq + (size_t)act_row(tid >> 2) * K + (tid & 3) * 64;
-    const int8_t *d_src = ((tid & 1) ? g.bs_lo : g.bs_hi) + (size_t)act_row(tid >> 1) * g.nb * 16;
-    const float *a_src = g.ad + (size_t)act_row(tid) * g.nb;
+    // ---- what this lane fetches ----
+    // quants chunk (tile t, slice ks): lane j brings the k-half j/32 (16 bytes) of token j%32's 32-byte
+    // slice to byte 16*j of the chunk, which is what lane j of the consumer reads.  Same for the bsums.
+    const int8_t *a_src[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) a_src[t] = g.aq + (size_t)act_row(t * 32 + li) * K + lg * 16;
+    // with fewer chunks than wavefronts some fetch a chunk twice, into the same place
+    const int bs_tile = wave % NT, da_chunk = wave % N_DA;
+    const _Float16 *b_src = g.bsf + (size_t)act_row(bs_tile * 32 + li) * nb * 16 + lg * 8;
+    const float *d_src = g.ad + (size_t)act_row(da_chunk * 64 + lane) * nb;
+    // weights: a row group's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of chunk c, so that
+    // LDS holds the rows back to back (144 bytes each) and consecutive lanes read consecutive memory.
+    // With WT = 2 the two wavefronts of a row group split the five chunks (3 + 2, one fetched twice).
+    const int wc0 = (WT == 1) ? 0 : (tgrp == 0 ? 0 : 3);
+    const uint8_t *w_src[C_W];
+    int w_chunk[C_W];
+#pragma unroll
+    for (int i = 0; i < C_W; i++) {
+        const int c = min(wc0 + i, 4) - ((WT == 2 && tgrp == 1 && i == 2) ? 1 : 0);  // tgrp 1: chunks 3, 4, 3
+        w_chunk[i] = c;
+        const int p = min(c * 64 + lane, 287);
+        const int r = min(row0 + p / 9, g.rows - 1);
+        w_src[i] = g.W + (size_t)(w_first_row + r) * g.row_stride + (p % 9) * 16;
+    }
 
-    auto issue_loads = [&](GemmPrefetch &pf, int kb) {
-        const uint8_t *blk = wrow + (size_t)kb * Q4_K_BYTES;
-        pf.wh = *reinterpret_cast<const uint4 *>(blk);
-        pf.wq0 = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * lg);
-        pf.wq1 = *reinterpret_cast<const uint4 *>(blk + 48 + 16 * lg);
-        pf.wq2 = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * lg);
-        pf.wq3 = *reinterpret_cast<const uint4 *>(blk + 112 + 16 * lg);
-        const uint4 *src = reinterpret_cast<const uint4 *>(s_src + (size_t)kb * QK_K);
-        pf.sa0 = src[0];
-        pf.sa1 = src[1];
-        pf.sa2 = src[2];
-        pf.sa3 = src[3];
-        pf.sdig = *reinterpret_cast<const uint4 *>(d_src + (size_t)kb * 16);
-        pf.sda = a_src[kb];
+    auto issue_acts = [&](int kb) {
+        uint8_t *st = lds + (kb & 1) * L::A_STAGE;
+#pragma unroll
+        for (int t = 0; t < NT; t++)
+#pragma unroll
+            for (int i = 0; i < 8 / NW; i++) {
+                const int ks = ((wave + t) % NW) + NW * i;
+                load_to_lds16(a_src[t] + (size_t)kb * QK_K + ks * 32, st + (t * 8 + ks) * 1024);
+            }
+        load_to_lds16(b_src + (size_t)kb * 16, st + L::OFF_BS + bs_tile * 1024);
+        load_to_lds4(d_src + kb, st + L::OFF_DA + da_chunk * 256);
     };
-    auto store_stage = [&](const GemmPrefetch &pf, int stage) {
-        uint8_t *st = lds + stage * STAGE;
-        if (tid < TM * 4) {
-            uint4 *dst = reinterpret_cast<uint4 *>(st + (tid >> 2) * GM_LDW + (tid & 3) * 64);
-            dst[0] = pf.sa0;
-            dst[1] = pf.sa1;
-            dst[2] = pf.sa2;
-            dst[3] = pf.sa3;
+    auto issue_weights = [&](int kb) {  // C_W loads
+        uint8_t *st = lds_w + (kb % WS) * L::W_STAGE + rgrp * L::W_GROUP;
+#pragma unroll
+        for (int i = 0; i < C_W; i++) {
+            // chunk 4 is half a chunk: 32 pieces
+            if (w_chunk[i] < 4 || lane < 32) load_to_lds16(w_src[i] + (size_t)kb * Q4_K_BYTES, st + w_chunk[i] * 1024);
         }
-        if (tid < TM * 2) *reinterpret_cast<uint4 *>(st + OFF_DIG + (tid >> 1) * 32 + (tid & 1) * 16) = pf.sdig;
-        if (tid < TM) *reinterpret_cast<float *>(st + OFF_DA + tid * 4) = pf.sda;
     };
 
-    // the current block of this lane's row as MFMA operands
-    v4i bH[8], bL[8];
-    long mB;
-    float wd, wdmin;
-    auto unpack = [&](const GemmPrefetch &pf) {
-        const uint4 wh = pf.wh;
-        const uint32_t sc_lo = wh.y & 0x3f3f3f3fu, m_lo = wh.z & 0x3f3f3f3fu;
-        const uint32_t sc_hi = (wh.w & 0x0f0f0f0fu) | (((wh.y >> 6) & 0x03030303u) << 4);
-        const uint32_t m_hi = ((wh.w >> 4) & 0x0f0f0f0fu) | (((wh.z >> 6) & 0x03030303u) << 4);
-        // one nibble pair: 16 bytes -> the lane's H and L operands of sub-blocks 2p and 2p+1
-        auto pair = [&](const uint4 q, const uint32_t scw, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
-            const uint32_t s0 = scw & 0xff, s1 = (scw >> 8) & 0xff;
-            const us2 h0 = {(unsigned short)(s0 >> 3), (unsigned short)(s0 >> 3)};
-            const us2 l0 = {(unsigned short)(s0 & 7), (unsigned short)(s0 & 7)};
-            const us2 h1 = {(unsigned short)(s1 >> 3), (unsigned short)(s1 >> 3)};
-            const us2 l1 = {(unsigned short)(s1 & 7), (unsigned short)(s1 & 7)};
-            auto one = [&](const uint32_t w, int &o0, int &o1, int &o2, int &o3) {
-                const uint32_t nl = w & 0x0f0f0f0fu, nh = (w >> 4) & 0x0f0f0f0fu;
-                us2 a, b;
-                __builtin_memcpy(&a, &nl, 4);
-                __builtin_memcpy(&b, &nh, 4);
-                const us2 r0 = a * h0, r1 = a * l0, r2 = b * h1, r3 = b * l1;  // bytes stay below 106
-                __builtin_memcpy(&o0, &r0, 4);
-                __builtin_memcpy(&o1, &r1, 4);
-                __builtin_memcpy(&o2, &r2, 4);
-                __builtin_memcpy(&o3, &r3, 4);
-            };
-            int a0, a1, a2, a3, b0, b1, b2, b3, c0, c1, c2, c3, d0, d1, d2, d3;
-            one(q.x, a0, a1, a2, a3);
-            one(q.y, b0, b1, b2, b3);
-            one(q.z, c0, c1, c2, c3);
-            one(q.w, d0, d1, d2, d3);
-            H0 = v4i{a0, b0, c0, d0};  // sub-block 2p: low nibbles
-            L0 = v4i{a1, b1, c1, d1};
-            H1 = v4i{a2, b2, c2, d2};  // sub-block 2p+1: high nibbles
-            L1 = v4i{a3, b3, c3, d3};
-        };
-        pair(pf.wq0, sc_lo, bH[0], bL[0], bH[1], bL[1]);
-        pair(pf.wq1, sc_lo >> 16, bH[2], bL[2], bH[3], bL[3]);
-        pair(pf.wq2, sc_hi, bH[4], bL[4], bH[5], bL[5]);
-        pair(pf.wq3, sc_hi >> 16, bH[6], bL[6], bH[7], bL[7]);
-        // mins of the four sub-blocks whose 16-wide groups are 8*lg .. 8*lg+7, each twice
-        const uint32_t mw = lg ? m_hi : m_lo;
-        const uint32_t mlo = __builtin_amdgcn_perm(0, mw, 0x01010000u), mhi = __builtin_amdgcn_perm(0, mw, 0x03030202u);
-        mB = (long)(((unsigned long)mhi << 32) | mlo);
-        wd = h2f(wh.x & 0xffffu);
-        wdmin = h2f(wh.x >> 16);
-    };
+    const uint32_t lds_a = lds_address(lds);
+    const uint32_t lds_wv = lds_address(lds_w) + rgrp * L::W_GROUP + li * Q4_K_BYTES;
 
-    float accF[MT][16];
+    v16f accF[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) accF[mt][r] = 0.0f;
+    for (int mt = 0; mt < MT; mt++) accF[mt] = v16f{0.0f};
 
-    auto compute_block = [&](int kb) {
-        const uint8_t *st = lds + (kb & 1) * STAGE;
+    BPlanes B;
+    RawBlock R;
+
+    // prologue: weights of blocks 0..WD-1, activations of block 0; the last weights may stay in flight
+    issue_weights(0);
+    issue_acts(0);
+#pragma unroll
+    for (int i = 1; i < WD; i++)
+        if (i < nb) issue_weights(i);
+    if (WS == 4 && nb > 2) wait_vm<C_W>();
+    else wait_vm<0>();
+    lds_barrier();
+    read_raw(R, lds_wv, lds_wv + 16 * lg);
+    wait_raw<0>(R);
+    unpack_block(R, lg, B);
+
+    for (int kb = 0; kb < nb; kb++) {
+        // the stages refilled here were last read in iteration kb-1, which every wavefront has left
+        if (kb + 1 < nb) issue_acts(kb + 1);
+        if (kb + WD < nb) issue_weights(kb + WD);
+
+        const uint32_t st = lds_a + (kb & 1) * L::A_STAGE;
+        const uint32_t qa = st + lane * 16, ba = st + L::OFF_BS + lane * 16, sa = st + L::OFF_DA + lg * 16;
+        const uint32_t wa = lds_wv + ((kb + 1) % WS) * L::W_STAGE;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
-            const int t0 = (wtok * MT + mt) * 32;  // first token of this tile within the stage
-            const uint8_t *arow = st + (t0 + li) * GM_LDW + 16 * lg;
-            const v16i z = {0};
-            // all of the tile's LDS reads go out before the first MFMA needs one
-            v4i a[8];
-#pragma unroll
-            for (int ks = 0; ks < 8; ks++) a[ks] = *reinterpret_cast<const v4i *>(arow + ks * 32);
-            const uint8_t *drow = st + OFF_DIG + (t0 + li) * 32 + 8 * lg;
-            const long dgh = *reinterpret_cast<const long *>(drow);
-            const long dgl = *reinterpret_cast<const long *>(drow + 16);
-            v16i accH, accL;
-#pragma unroll
-            for (int ks = 0; ks < 8; ks++) {
-                if (ks == 0) {
-                    accH = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], bH[ks], z, 0, 0, 0);
-                    accL = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], bL[ks], z, 0, 0, 0);
-                } else {
-                    accH = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], bH[ks], accH, 0, 0, 0);
-                    accL = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ks], bL[ks], accL, 0, 0, 0);
-                }
-            }
-            const v16i Dh = __builtin_amdgcn_mfma_i32_32x32x16_i8(dgh, mB, z, 0, 0, 0);
-            const v16i Dl = __builtin_amdgcn_mfma_i32_32x32x16_i8(dgl, mB, z, 0, 0, 0);
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const float4 da4 = *reinterpret_cast<const float4 *>(st + OFF_DA + (t0 + 4 * lg + 8 * c) * 4);
-                const float dav[4] = {da4.x, da4.y, da4.z, da4.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int r = c * 4 + e;
-                    const int s1 = (accH[r] << 3) + accL[r];
-                    const int s2 = (Dh[r] << 6) + Dl[r];
-                    const float v = wd * (float)s1 - wdmin * (float)s2;
-                    accF[mt][r] = fmaf(dav[e], v, accF[mt][r]);
-                }
-            }
+            const int t = tgrp * MT + mt;
+            TileOperands T;
+            TileScales S;
+            TileAcc X;
+            read_ops(T, qa + t * 8192, ba + t * 1024);
+            wait_ops<0>(T);
+            tile_mfmas(T, B, X);
+            // the scales, and with the last tile the next block's raw weights (landed since iteration
+            // kb-1), are fetched while the MFMAs run; their registers are the ones the operands leave
+            read_scales(S, sa + t * 128);
+            if (mt == MT - 1) read_raw(R, wa, wa + 16 * lg);
+            if (mt == MT - 1) wait_scales<5>(S);
+            else wait_scales<0>(S);
+            tile_epilogue(X, S, B, accF[mt]);
+            __builtin_amdgcn_sched_barrier(0);  // keep a tile's registers from living into the next tile
         }
-    };
-
-    // prologue: block 0 staged and unpacked, block 1 in flight
-    GemmPrefetch pf;
-    issue_loads(pf, 0);
-    store_stage(pf, 0);
-    unpack(pf);
-    if (g.nb > 1) issue_loads(pf, 1);
-    lds_barrier();
-
-    for (int kb = 0; kb < g.nb; kb++) {
-        compute_block(kb);
-        if (kb + 1 < g.nb) {
-            store_stage(pf, (kb + 1) & 1);  // the other stage: nobody reads it during this iteration
-            unpack(pf);
-            if (kb + 2 < g.nb) issue_loads(pf, kb + 2);
+        if (kb + 1 < nb) {
+            wait_raw<0>(R);
+            unpack_block(R, lg, B);
+            // activations of block kb+1 and weights of block kb+2 must have landed; with four weight
+            // stages the weights requested above (younger than both) may stay in flight
+            if (WS == 4 && kb + WD < nb) wait_vm<C_W>();
+            else wait_vm<0>();
         }
         lds_barrier();
     }
@@ -279,7 +428,7 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int tok = tok0 + (wtok * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
+            const int tok = tok0 + (tgrp * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
             if (row < g.rows && tok < n_tok) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
         }
 }
@@ -292,18 +441,33 @@ __global__ __launch_bounds__(256 * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
+template <int RG, int WT, int MT, int WS, bool GROUPED>
+static int launch_variant(const GemmArgs &g, unsigned grid, hipStream_t s) {
+    constexpr size_t shmem = GemmLds<RG, WT, MT, WS>::BYTES;
+    static_assert(shmem <= 160 * 1024, "LDS of a CU");
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (shmem > 65536 && !sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_mfma_kernel<RG, WT, MT, WS, GROUPED>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", shmem, hipGetErrorString(e));
+        sized = true;
+    }
+    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS, GROUPED>), dim3(grid), dim3(64 * RG * WT), shmem, s, g);
+    FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
+    return FRK_OK;
+}
+
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) {
     const size_t n = M * cols;
-    return round_up(n, 256) + round_up(n / QK_K * 4, 256) + 2 * round_up(n / 16, 256);
+    return round_up(n, 256) + round_up(n / QK_K * 4, 256) + round_up(n / 16 * 2, 256);
 }
 
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     const size_t n = M * w->cols;
     int8_t *q = (int8_t *)ws;
     float *d = (float *)((char *)ws + round_up(n, 256));
-    int8_t *bh = (int8_t *)((char *)d + round_up(n / QK_K * 4, 256));
-    int8_t *bl = bh + round_up(n / 16, 256);
-    int rc = launch_quantize_q8_k_gemm(x, n, q, d, bh, bl, s);
+    _Float16 *bsf = (_Float16 *)((char *)d + round_up(n / QK_K * 4, 256));
+    int rc = launch_quantize_q8_k_gemm(x, n, q, d, bsf, s);
     if (rc) return rc;
 
     GemmArgs g;
@@ -314,32 +478,29 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.M = (int)M;
     g.aq = q;
     g.ad = d;
-    g.bs_hi = bh;
-    g.bs_lo = bl;
+    g.bsf = bsf;
     g.y = y;
     g.tiles = nullptr;
     g.n_tiles = nullptr;
     g.gather = nullptr;
-    g.row_tiles = (int)((w->rows + 127) / 128);
-    const int wt = M > 32 ? 2 : 1;  // token groups per workgroup, one 32-token tile per wavefront
-    const int tm = 32 * wt;
-    g.tok_tiles = (int)((M + tm - 1) / tm);
-    const int groups = (g.row_tiles + 7) / 8;
-    const unsigned grid = (unsigned)(groups * 8 * g.tok_tiles);
-    const size_t shmem = 2 * ((size_t)tm * GM_LDW + (size_t)tm * 36);
-    if (wt == 2) hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 2, false>), dim3(grid), dim3(512), shmem, s, g);
-    else hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 1, false>), dim3(grid), dim3(256), shmem, s, g);
-    FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
-    return FRK_OK;
+    // shape of a workgroup's tile: 256 rows x 64 tokens when that still gives every CU a workgroup,
+    // else 128 rows x 64 or 32 tokens
+    auto grid_for = [&](int rows_wg, int tm) {
+        g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
+        g.tok_tiles = (int)((M + tm - 1) / tm);
+        return (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
+    };
+    const size_t wgs_big = ((w->rows + 255) / 256) * ((M + 63) / 64);
+    if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2, false>(g, grid_for(256, 64), s);
+    if (M > 32) return launch_variant<4, 2, 1, 4, false>(g, grid_for(128, 64), s);
+    return launch_variant<4, 1, 1, 2, false>(g, grid_for(128, 32), s);
 }
 
-
-int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, int8_t *bs_hi, int8_t *bs_lo,
-                              hipStream_t s) {
+int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Float16 *bsf, hipStream_t s) {
     const size_t nblk = n / QK_K;
     if (nblk == 0) return FRK_OK;
     hipLaunchKernelGGL(quantize_q8_k_gemm_kernel, dim3((unsigned)((nblk + 3) / 4)), dim3(256), 0, s, x, nblk, q, d,
-                       bs_hi, bs_lo);
+                       bsf);
     FRK_LAUNCH_CHECK("quantize_q8_k_gemm");
     return FRK_OK;
 }
@@ -347,8 +508,8 @@ int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, int
 // Grouped GEMM over the experts stacked in `w` (expert e = rows [e*rows_e, (e+1)*rows_e)):
 // y[p][rows_e] for every output row p listed in the tiles (32 rows per tile at most).
 int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
-                             const int8_t *bs_hi, const int8_t *bs_lo, const int4 *tiles, const int *n_tiles,
-                             int max_tiles, const int *gather, float *y, hipStream_t s) {
+                             const _Float16 *bsf, const int4 *tiles, const int *n_tiles, int max_tiles,
+                             const int *gather, float *y, hipStream_t s) {
     GemmArgs g;
     g.W = w->dev;
     g.row_stride = w->layout.row_stride;
@@ -357,19 +518,14 @@ int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *
     g.M = 0;
     g.aq = aq;
     g.ad = ad;
-    g.bs_hi = bs_hi;
-    g.bs_lo = bs_lo;
+    g.bsf = bsf;
     g.y = y;
     g.tiles = tiles;
     g.n_tiles = n_tiles;
     g.gather = gather;
     g.row_tiles = (int)((rows_e + 127) / 128);
     g.tok_tiles = max_tiles;
-    const unsigned grid = (unsigned)(g.row_tiles * max_tiles);
-    const size_t shmem = 2 * ((size_t)32 * GM_LDW + (size_t)32 * 36);
-    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<1, 1, true>), dim3(grid), dim3(256), shmem, s, g);
-    FRK_LAUNCH_CHECK("gemm_q4_k_grouped");
-    return FRK_OK;
+    return launch_variant<4, 1, 1, 2, true>(g, (unsigned)(g.row_tiles * max_tiles), s);
 }
 
 }  // namespace frk

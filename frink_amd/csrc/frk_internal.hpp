@@ -122,12 +122,12 @@ int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
-// Q8_K quantization in the GEMM's form: bsums split into digits bs = 64*hi + lo, hi in [-32, 31], lo in [0, 63]
-int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, int8_t *bs_hi, int8_t *bs_lo,
+// Q8_K quantization in the GEMM's form: the 16-wide sums as f16 (exact)
+int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Float16 *bsf,
                               hipStream_t s);
 // grouped (per-expert) GEMM: tiles {expert, first, count, 0} of at most 32 output rows each
 int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
-                             const int8_t *bs_hi, const int8_t *bs_lo, const int4 *tiles, const int *n_tiles,
+                             const _Float16 *bsf, const int4 *tiles, const int *n_tiles,
                              int max_tiles, const int *gather, float *y, hipStream_t s);
 // MoE expert FFN over stacked Q4_K experts; ws must hold moe_workspace_bytes(...)
 size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);

@@ -169,8 +169,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__restrict__ gate,
                                                               const float *__restrict__ up, size_t n_blocks,
                                                               int8_t *__restrict__ q, float *__restrict__ d,
-                                                              int8_t *__restrict__ bs_hi,
-                                                              int8_t *__restrict__ bs_lo) {
+                                                              _Float16 *__restrict__ bsf) {
     const int lane = threadIdx.x & 63;
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= n_blocks) return;
@@ -185,8 +184,7 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__res
     const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
     reinterpret_cast<uint32_t *>(q + b * QK_K)[lane] = packed;
     if ((lane & 3) == 0) {
-        bs_hi[b * 16 + (lane >> 2)] = (int8_t)(bs >> 6);
-        bs_lo[b * 16 + (lane >> 2)] = (int8_t)(bs & 63);
+        bsf[b * 16 + (lane >> 2)] = (_Float16)bs;
     }
     if (lane == 0) d[b] = dd;
 }
@@ -248,10 +246,12 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
 }
 
 struct MoeScratch {
-    int8_t *xq, *xh, *xl;  // Q8_K of the token rows and the digit planes
+    int8_t *xq;  // Q8_K of the token rows; bsums as f16
+    _Float16 *xb;
     float *xd;
     float *gate_out, *up_out, *down_out;
-    int8_t *aq, *ah, *al;  // Q8_K of silu(gate)*up
+    int8_t *aq;  // Q8_K of silu(gate)*up
+    _Float16 *ab;
     float *ad;
     int *group_off, *gather, *pos_of, *n_tiles;
     int4 *tiles;
@@ -268,15 +268,13 @@ static MoeScratch moe_carve(void *base, size_t batch, int k, int n_experts, int 
     };
     MoeScratch m;
     m.xq = (int8_t *)take(batch * hidden);
-    m.xh = (int8_t *)take(batch * hidden / 16);
-    m.xl = (int8_t *)take(batch * hidden / 16);
+    m.xb = (_Float16 *)take(batch * hidden / 16 * 2);
     m.xd = (float *)take(batch * hidden / QK_K * 4);
     m.gate_out = (float *)take(pairs * ffn * 4);
     m.up_out = (float *)take(pairs * ffn * 4);
     m.down_out = (float *)take(pairs * hidden * 4);
     m.aq = (int8_t *)take(pairs * ffn);
-    m.ah = (int8_t *)take(pairs * ffn / 16);
-    m.al = (int8_t *)take(pairs * ffn / 16);
+    m.ab = (_Float16 *)take(pairs * ffn / 16 * 2);
     m.ad = (float *)take(pairs * ffn / QK_K * 4);
     m.group_off = (int *)take((n_experts + 1) * 4);
     m.gather = (int *)take(pairs * 4);
@@ -323,20 +321,20 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, k, n_experts, m.group_off, m.gather,
                        m.pos_of, m.tiles, m.n_tiles);
     FRK_LAUNCH_CHECK("moe_group");
-    int rc = launch_quantize_q8_k_gemm(x, batch * hidden, m.xq, m.xd, m.xh, m.xl, s);
+    int rc = launch_quantize_q8_k_gemm(x, batch * hidden, m.xq, m.xd, m.xb, s);
     if (rc) return rc;
     // gate and up read the same quantized token rows through the gather list
-    rc = launch_gemm_q4_k_grouped(gate, (size_t)ffn, m.xq, m.xd, m.xh, m.xl, m.tiles, m.n_tiles, max_tiles, m.gather,
+    rc = launch_gemm_q4_k_grouped(gate, (size_t)ffn, m.xq, m.xd, m.xb, m.tiles, m.n_tiles, max_tiles, m.gather,
                                   m.gate_out, s);
     if (rc) return rc;
-    rc = launch_gemm_q4_k_grouped(up, (size_t)ffn, m.xq, m.xd, m.xh, m.xl, m.tiles, m.n_tiles, max_tiles, m.gather,
+    rc = launch_gemm_q4_k_grouped(up, (size_t)ffn, m.xq, m.xd, m.xb, m.tiles, m.n_tiles, max_tiles, m.gather,
                                   m.up_out, s);
     if (rc) return rc;
     const size_t ablk = pairs * ffn / QK_K;
     hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)((ablk + 3) / 4)), dim3(256), 0, s, m.gate_out, m.up_out,
-                       ablk, m.aq, m.ad, m.ah, m.al);
+                       ablk, m.aq, m.ad, m.ab);
     FRK_LAUNCH_CHECK("swiglu_quantize");
-    rc = launch_gemm_q4_k_grouped(down, (size_t)hidden, m.aq, m.ad, m.ah, m.al, m.tiles, m.n_tiles, max_tiles, nullptr,
+    rc = launch_gemm_q4_k_grouped(down, (size_t)hidden, m.aq, m.ad, m.ab, m.tiles, m.n_tiles, max_tiles, nullptr,
                                   m.down_out, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights, m.pos_of, k,
