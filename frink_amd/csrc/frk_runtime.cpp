@@ -386,6 +386,21 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
+    // thin batches of the K-quants: the weights are read once per 8 activation rows
+    const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q6_K) && batch >= 2 ? thin_gemm_max_batch(w) : 0;
+    if (thin >= 2) {
+        Q8KActs a;
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
+        if (rc) return rc;
+        const size_t nb = w->cols / QK_K;
+        for (size_t b0 = 0; b0 < batch; b0 += (size_t)thin) {
+            const int n = (int)std::min<size_t>((size_t)thin, batch - b0);
+            Q8KActs c = {a.q + b0 * w->cols, a.d + b0 * nb, a.bsums + b0 * nb * 16};
+            rc = launch_thin_gemm(w, n, c, y + b0 * w->rows, (hipStream_t)stream);
+            if (rc) return rc;
+        }
+        return FRK_OK;
+    }
     // otherwise one matvec per activation row (the reference's own path below its GEMM threshold,
     // crates/frink-core/src/weight_matrix.rs:2636-2652)
     for (size_t b = 0; b < batch; b++) {

@@ -423,3 +423,50 @@ def test_cpp_host_mirror_launches(fa):
     r = subprocess.run([fb.HOST_CHECK_BIN, "--gpu"], env=env, text=True, capture_output=True, timeout=120)
     print(r.stdout, flush=True)
     assert r.returncode == 0 and "FAIL" not in r.stdout, r.stdout + r.stderr
+
+
+# ------------------------------------------------------------------ thin batched GEMM (batched decode)
+
+@pytest.mark.parametrize("kind,rows,cols,batch", [
+    (fo.Q4_K, 70, 1024, 2), (fo.Q4_K, 33, 512, 3), (fo.Q4_K, 128, 4096, 8), (fo.Q4_K, 64, 256, 5),
+    (fo.Q4_K, 40, 2048, 11), (fo.Q4_K, 16, 768, 15),
+    (fo.Q6_K, 70, 1024, 2), (fo.Q6_K, 33, 512, 3), (fo.Q6_K, 48, 14336, 8), (fo.Q6_K, 64, 256, 7),
+    (fo.Q6_K, 40, 2048, 11), (fo.Q6_K, 24, 768, 40),
+])
+def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
+    from frink_amd import synth
+    print("thin gemm", kind, rows, cols, batch, flush=True)
+    data = make_weights(kind, rows, cols, seed=kind * 1000 + rows + batch)
+    x = synth.activations(rows + cols + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    xd = to_dev(x)
+    got = w.gemm(xd).cpu().numpy()
+    assert got.shape == (batch, rows)
+    assert_rows_close(got, fo.gemm(kind, data, rows, cols, x), "thin gemm kind %d batch %d" % (kind, batch))
+    # same integer sums, same scale expression, but a different lane-to-unit map than the decode
+    # GEMV: equal to it within float summation order
+    for b in (0, batch - 1):
+        one = w.gemv(xd[b].contiguous()).cpu().numpy()
+        assert np.abs(one - got[b]).max() <= 1e-5 * np.abs(one).max()
+    w.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols,seed", [(fo.Q4_K, 14336, 4096, 21), (fo.Q6_K, 4096, 14336, 22)])
+def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
+    """Batched decode, M=8, at the FFN shapes: slices of weight rows against the oracle for every
+    activation row, and each batch row against the decode GEMV of that row."""
+    from frink_amd import synth
+    print("full thin gemm", kind, rows, cols, flush=True)
+    data = make_weights(kind, rows, cols, seed=seed)
+    x = synth.activations(seed + 1, 8, cols)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    xd = to_dev(x)
+    y = w.gemm(xd).cpu().numpy()
+    for row0 in (0, rows // 2 - 100, rows - 200):
+        want = fo.gemm(kind, data, rows, cols, x, row0=row0, nrows=200)
+        ninf = np.abs(want).max(axis=1)
+        err = np.abs(y[:, row0:row0 + 200] - want).max(axis=1)
+        assert (err <= TOL * ninf).all(), (row0, float((err / ninf).max()))
+    one = w.gemv(xd[5].contiguous()).cpu().numpy()
+    assert np.abs(one - y[5]).max() <= 1e-5 * np.abs(one).max()
+    w.release()
