@@ -1,0 +1,253 @@
+// Decode GEMV for Q6_K and Q8_0 with every load of a row in flight at once.
+//
+// One wavefront owns one weight row; lane l owns units l, l+64, ... (a unit is 64 weights of Q6_K or
+// 16 of Q8_0, the same units as the looping kernels in frk_gemv.hip).  All of a lane's loads -- its
+// share of the activation first, because a wavefront's loads return in issue order and the
+// activation comes from L2, then its weights from HBM -- are issued before any arithmetic, so a CU
+// holds tens of kilobytes in flight instead of one loop iteration's worth.  No LDS, no barrier: the
+// quantized activation (a few kilobytes) is read by every lane straight from L2.
+// Rows longer than 64*U units fall back to the looping kernels.
+#include "frk_device.hpp"
+
+namespace frk {
+
+// ------------------------------------------------------------------ Q6_K x Q8_K
+// dot_q6_k_q8 (crates/frink-quant/src/lib.rs:1069-1110) over the planar resident layout.
+// Unit = (block b, half h, 16-lane column t): ql[64h+16t..], ql[64h+32+16t..], qh[32h+16t..]
+// hold four 16-weight groups with scales sc[8h+t+{0,2,4,6}].  The -32 offset is folded as
+// -32 * (sum of the 16 activation quants), which Q8_K's bsums already hold.
+// FUSED: the workgroup (16 wavefronts, XB blocks of the activation each) quantizes the f32 activation
+// to Q8_K into LDS itself, bit-exact with quantize_activations_q8_k, while its weight loads are in
+// flight, and its 16 rows share that one copy (a row of this kind is shorter than the activation it
+// multiplies, so per-lane reads of the activation from L2 would double the traffic); otherwise the
+// quantized activation is read from global memory.
+template <int U, int XB, bool FUSED>
+__global__ __launch_bounds__(FUSED ? 1024 : 256) void gemv_q6_k_direct_kernel(
+    const uint8_t *__restrict__ W, Layout lay, int rows, int nb, const float *__restrict__ x,
+    const int8_t *__restrict__ aq, const float *__restrict__ ad, const int16_t *__restrict__ absums,
+    float *__restrict__ y) {
+    constexpr int WAVES = FUSED ? 16 : 4;
+    extern __shared__ uint4 smem_direct[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = min((int)blockIdx.x * WAVES + wave, rows - 1);  // a wavefront past the end repeats the last row
+    const bool store = (int)blockIdx.x * WAVES + wave < rows;
+    const uint8_t *row = W + (size_t)r * lay.row_stride;
+    const int units = nb * 4;
+
+    // the activation's loads go out before the weights': a wavefront's loads return in issue order
+    float4 xv[FUSED ? XB : 1];
+    if (FUSED) {
+#pragma unroll
+        for (int i = 0; i < XB; i++) {
+            const int b = min(wave + i * WAVES, nb - 1);
+            xv[i] = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K)[lane];
+        }
+    }
+    uint4 a0[U], a1[U], a2[U], a3[U], bs[U];
+    float da[U];
+    if (!FUSED) {
+#pragma unroll
+        for (int j = 0; j < U; j++) {
+            const int u = min(lane + 64 * j, units - 1);  // a lane past the end repeats the last unit, unused
+            const int b = u >> 2, h = (u >> 1) & 1, t = u & 1;
+            const int8_t *abase = aq + b * 256 + h * 128 + t * 16;
+            a0[j] = *reinterpret_cast<const uint4 *>(abase);
+            a1[j] = *reinterpret_cast<const uint4 *>(abase + 32);
+            a2[j] = *reinterpret_cast<const uint4 *>(abase + 64);
+            a3[j] = *reinterpret_cast<const uint4 *>(abase + 96);
+            bs[j] = *reinterpret_cast<const uint4 *>(absums + b * 16 + h * 8);  // the half's eight 16-wide sums
+            da[j] = ad[b];
+        }
+    }
+    uint4 qla[U], qlb[U], qh[U];
+    uint2 scv[U];
+    uint32_t dbits[U];
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int u = min(lane + 64 * j, units - 1);
+        const int b = u >> 2, h = (u >> 1) & 1, t = u & 1;
+        qla[j] = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + t * 16);
+        qlb[j] = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + 32 + t * 16);
+        qh[j] = *reinterpret_cast<const uint4 *>(row + lay.off_a + (size_t)b * 64 + h * 32 + t * 16);
+        scv[j] = *reinterpret_cast<const uint2 *>(row + lay.off_b + (size_t)b * 16 + h * 8);
+        dbits[j] = *reinterpret_cast<const uint16_t *>(row + lay.off_c + (size_t)b * 2);
+    }
+    if (FUSED) {
+        int8_t *sq = reinterpret_cast<int8_t *>(smem_direct);
+        int16_t *sbs = reinterpret_cast<int16_t *>(sq + (size_t)nb * 256);
+        float *sd = reinterpret_cast<float *>(sbs + (size_t)nb * 16);
+#pragma unroll
+        for (int i = 0; i < XB; i++) {
+            const int b = wave + i * WAVES;
+            float d;
+            int s16;
+            const uint32_t packed = quantize_q8_k_lane(xv[i], d, s16);
+            if (b < nb) {  // uniform across the wavefront
+                reinterpret_cast<uint32_t *>(sq + b * QK_K)[lane] = packed;
+                if ((lane & 3) == 0) sbs[b * 16 + (lane >> 2)] = (int16_t)s16;
+                if (lane == 0) sd[b] = d;
+            }
+        }
+        lds_barrier();  // publishes LDS, does not wait for the weight loads
+    }
+
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int t = lane & 1;  // (lane + 64*j) & 1
+        if (FUSED) {  // this unit's slice of the activation, from the workgroup's copy
+            const int8_t *sq = reinterpret_cast<const int8_t *>(smem_direct);
+            const int16_t *sbs = reinterpret_cast<const int16_t *>(sq + (size_t)nb * 256);
+            const float *sd = reinterpret_cast<const float *>(sbs + (size_t)nb * 16);
+            const int u = min(lane + 64 * j, units - 1);
+            const int b = u >> 2, h = (u >> 1) & 1;
+            const int8_t *abase = sq + b * 256 + h * 128 + t * 16;
+            a0[j] = *reinterpret_cast<const uint4 *>(abase);
+            a1[j] = *reinterpret_cast<const uint4 *>(abase + 32);
+            a2[j] = *reinterpret_cast<const uint4 *>(abase + 64);
+            a3[j] = *reinterpret_cast<const uint4 *>(abase + 96);
+            bs[j] = *reinterpret_cast<const uint4 *>(sbs + b * 16 + h * 8);
+            da[j] = sd[b];
+        }
+        int d1 = 0, d2 = 0, d3 = 0, d4 = 0;
+#define FRK_Q6_STEP(c)                                                                                   \
+    d1 = dot4((qla[j].c & 0x0f0f0f0fu) | ((qh[j].c << 4) & 0x30303030u), a0[j].c, d1);                    \
+    d2 = dot4((qlb[j].c & 0x0f0f0f0fu) | ((qh[j].c << 2) & 0x30303030u), a1[j].c, d2);                    \
+    d3 = dot4(((qla[j].c >> 4) & 0x0f0f0f0fu) | (qh[j].c & 0x30303030u), a2[j].c, d3);                    \
+    d4 = dot4(((qlb[j].c >> 4) & 0x0f0f0f0fu) | ((qh[j].c >> 2) & 0x30303030u), a3[j].c, d4);
+        FRK_Q6_STEP(x)
+        FRK_Q6_STEP(y)
+        FRK_Q6_STEP(z)
+        FRK_Q6_STEP(w)
+#undef FRK_Q6_STEP
+        const uint32_t slo = t ? (scv[j].x >> 8) : scv[j].x, shi = t ? (scv[j].y >> 8) : scv[j].y;
+        const int s1 = (int)(int8_t)(slo & 0xff), s2 = (int)(int8_t)((slo >> 16) & 0xff);
+        const int s3 = (int)(int8_t)(shi & 0xff), s4 = (int)(int8_t)((shi >> 16) & 0xff);
+        // sums of groups t, t+2, t+4, t+6 of the half: 16-bit fields t, t+2 (x, y) and t+4, t+6 (z, w)
+        const int sh = 16 * t;
+        const int b1 = (int)(int16_t)(bs[j].x >> sh), b2 = (int)(int16_t)(bs[j].y >> sh);
+        const int b3 = (int)(int16_t)(bs[j].z >> sh), b4 = (int)(int16_t)(bs[j].w >> sh);
+        const int isum = s1 * (d1 - 32 * b1) + s2 * (d2 - 32 * b2) + s3 * (d3 - 32 * b3) + s4 * (d4 - 32 * b4);
+        const float term = (h2f(dbits[j]) * da[j]) * (float)isum;
+        acc += (lane + 64 * j < units) ? term : 0.0f;
+    }
+    acc = part_sum<64>(acc);
+    if (lane == 0 && store) y[r] = acc;
+}
+
+// ------------------------------------------------------------------ Q8_0 x f32
+// dot_q8_0_f32 (crates/frink-quant/src/lib.rs:663-686) over the planar resident layout.
+// Unit = 16 quants (half a block).
+template <int U>
+__global__ __launch_bounds__(256) void gemv_q8_0_f32_direct_kernel(const uint8_t *__restrict__ W, Layout lay,
+                                                                   int rows, int nb, const float *__restrict__ x,
+                                                                   float *__restrict__ y) {
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;  // uniform per wavefront
+    const uint8_t *row = W + (size_t)r * lay.row_stride;
+    const int units = nb * 2;
+
+    float4 x0[U], x1[U], x2[U], x3[U];
+    uint4 qv[U];
+    uint32_t dbits[U];
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int u = min(lane + 64 * j, units - 1);
+        const float4 *xv = reinterpret_cast<const float4 *>(x + u * 16);
+        x0[j] = xv[0];
+        x1[j] = xv[1];
+        x2[j] = xv[2];
+        x3[j] = xv[3];
+    }
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        const int u = min(lane + 64 * j, units - 1);
+        qv[j] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+        dbits[j] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2);
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+        float s = 0.0f;
+#define FRK_Q8_STEP(c, xx)                                         \
+    s = fmaf((float)(int8_t)(qv[j].c & 0xff), xx.x, s);            \
+    s = fmaf((float)(int8_t)((qv[j].c >> 8) & 0xff), xx.y, s);     \
+    s = fmaf((float)(int8_t)((qv[j].c >> 16) & 0xff), xx.z, s);    \
+    s = fmaf((float)(int8_t)(qv[j].c >> 24), xx.w, s);
+        FRK_Q8_STEP(x, x0[j])
+        FRK_Q8_STEP(y, x1[j])
+        FRK_Q8_STEP(z, x2[j])
+        FRK_Q8_STEP(w, x3[j])
+#undef FRK_Q8_STEP
+        const float term = s * h2f(dbits[j]);
+        acc += (lane + 64 * j < units) ? term : 0.0f;
+    }
+    acc = part_sum<64>(acc);
+    if (lane == 0) y[r] = acc;
+}
+
+// ------------------------------------------------------------------ launchers
+
+#define FRK_LAUNCH_CHECK(what)                                                                          \
+    do {                                                                                                \
+        hipError_t e_ = hipGetLastError();                                                              \
+        if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
+    } while (0)
+
+// rows of at most 64*4 units, and long enough that a wavefront per row is not mostly idle lanes
+bool direct_gemv_fits(const frk_weights *w) {
+    const size_t units = w->kind == FRK_KIND_Q6_K ? w->cols / QK_K * 4 : w->cols / Q8_0_ELEMS * 2;
+    return (w->kind == FRK_KIND_Q6_K || w->kind == FRK_KIND_Q8_0) && units > 32 && units <= 256;
+}
+
+int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    const int u = (nb * 4 + 63) / 64;
+    const dim3 grid((unsigned)((w->rows + 3) / 4)), block(256);
+#define FRK_GO(UU)                                                                                              \
+    hipLaunchKernelGGL((gemv_q6_k_direct_kernel<UU, 1, false>), grid, block, 0, s, w->dev, w->layout, (int)w->rows, \
+                       nb, (const float *)nullptr, a.q, a.d, a.bsums, y)
+    if (u == 1) FRK_GO(1);
+    else if (u == 2) FRK_GO(2);
+    else if (u == 3) FRK_GO(3);
+    else FRK_GO(4);
+#undef FRK_GO
+    FRK_LAUNCH_CHECK("gemv_q6_k_direct");
+    return FRK_OK;
+}
+
+// One launch: Q8_K quantization of x inside the kernel.  nb <= 64 (direct_gemv_fits).
+int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    const int u = (nb * 4 + 63) / 64;
+    const dim3 grid((unsigned)((w->rows + 15) / 16)), block(1024);
+    const size_t shmem = (size_t)nb * (256 + 32 + 4);
+#define FRK_GO(UU, XX)                                                                                              \
+    hipLaunchKernelGGL((gemv_q6_k_direct_kernel<UU, XX, true>), grid, block, shmem, s, w->dev, w->layout, (int)w->rows, \
+                       nb, x, (const int8_t *)nullptr, (const float *)nullptr, (const int16_t *)nullptr, y)
+    if (u == 1) FRK_GO(1, 1);       // nb <= 16
+    else if (u == 2) FRK_GO(2, 2);  // nb <= 32
+    else if (u == 3) FRK_GO(3, 3);  // nb <= 48
+    else FRK_GO(4, 4);              // nb <= 64
+#undef FRK_GO
+    FRK_LAUNCH_CHECK("gemv_q6_k_fused");
+    return FRK_OK;
+}
+
+int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS);
+    const int u = (nb * 2 + 63) / 64;
+    const dim3 grid((unsigned)((w->rows + 3) / 4)), block(256);
+#define FRK_GO(UU) \
+    hipLaunchKernelGGL(gemv_q8_0_f32_direct_kernel<UU>, grid, block, 0, s, w->dev, w->layout, (int)w->rows, nb, x, y)
+    if (u == 1) FRK_GO(1);
+    else if (u == 2) FRK_GO(2);
+    else if (u == 3) FRK_GO(3);
+    else FRK_GO(4);
+#undef FRK_GO
+    FRK_LAUNCH_CHECK("gemv_q8_0_f32_direct");
+    return FRK_OK;
+}
+
+}  // namespace frk

@@ -138,6 +138,11 @@ int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hid
                            float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of, hipStream_t s);
 int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, int k, int norm, int32_t *ids,
                                float *weights, hipStream_t s);
+// prefetch-all GEMVs (one wavefront per row, no LDS) for rows of 33..256 units
+bool direct_gemv_fits(const frk_weights *w);
+int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // thin batched GEMM of the K-quants: 1 <= batch <= thin_gemm_max_batch(w) rows per launch (0: does not fit)
 int thin_gemm_max_batch(const frk_weights *w);
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s);

@@ -343,13 +343,16 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
         if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
         [[fallthrough]];
     case FRK_KIND_Q6_K: {
+        if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, &a);
         if (rc) return rc;
-        return w->kind == FRK_KIND_Q4_K ? launch_gemv_q4_k(w, a, y, s) : launch_gemv_q6_k(w, a, y, s);
+        if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, s);
+        return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, s) : launch_gemv_q6_k(w, a, y, s);
     }
     case FRK_KIND_Q8_0: {
-        if (act_mode == FRK_ACT_F32) return launch_gemv_q8_0_f32(w, x, y, s);
+        if (act_mode == FRK_ACT_F32)
+            return direct_gemv_fits(w) ? launch_gemv_q8_0_f32_direct(w, x, y, s) : launch_gemv_q8_0_f32(w, x, y, s);
         size_t n = w->cols;
         void *ws = nullptr;
         int rc = workspace(round_up(n, 256) + n / 32 * 4, s, &ws);
@@ -372,7 +375,9 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     if (w->kind == FRK_KIND_Q4_K)
         return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
                                   : launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
-    if (w->kind == FRK_KIND_Q6_K) return launch_gemv_q6_k(w, a, y, (hipStream_t)stream);
+    if (w->kind == FRK_KIND_Q6_K)
+        return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, (hipStream_t)stream)
+                                   : launch_gemv_q6_k(w, a, y, (hipStream_t)stream);
     return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K and Q6_K weights only (kind %d)", w->kind);
 }
 
