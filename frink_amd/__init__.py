@@ -26,7 +26,8 @@ EXPORTS = [
     "frk_hip_gemm_supported", "frk_hip_has_launch", "frk_hip_block_bytes", "frk_hip_block_elems",
     "frk_hip_worth_a_gemm", "frk_hip_weights_register", "frk_hip_weights_from_device",
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
-    "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
+    "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
+    "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
     "frk_hip_gemm_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
@@ -78,6 +79,10 @@ def lib():
             "frk_hip_weights_kind": (i, [vp]),
             "frk_hip_launch_matvec": (i, [i, vp, sz, vp, sz, sz, sz, vp]),
             "frk_hip_launch_mul_mm": (i, [i, vp, sz, vp, sz, sz, sz, sz, sz, vp]),
+            "frk_hip_launch_matvec_multi": (i, [vp, sz, vp, sz, vp]),
+            "frk_hip_launch_dense_ffn_swiglu": (i, [vp, vp, vp, vp, sz, vp]),
+            "frk_hip_gemv_multi_dev": (i, [vp, sz, vp, vp, vp]),
+            "frk_hip_ffn_swiglu_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemv_dev": (i, [vp, vp, vp, i, vp]),
             "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
@@ -264,6 +269,59 @@ def moe_intermediates(batch, k, n_experts, hidden, ffn):
     check(lib().frk_hip_moe_intermediates_dev(batch, k, n_experts, hidden, ffn, *(C.c_void_p(t.data_ptr())
                                               for t in (g, u, q, d, pos)), _stream()))
     return g, u, q, d, pos
+
+
+def gemv_multi(ws, x, outs=None):
+    """WeightMatrix::apply_gpu_multi on the device: matrices of equal column count share one
+    activation (and one Q8_K quantization of it)."""
+    import torch
+    n = len(ws)
+    ys = outs if outs is not None else [torch.empty(w.rows, dtype=torch.float32, device=x.device) for w in ws]
+    hs = (C.c_void_p * n)(*[w.handle for w in ws])
+    ps = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+    check(lib().frk_hip_gemv_multi_dev(hs, n, C.c_void_p(x.data_ptr()), ps, _stream()))
+    return ys
+
+
+def ffn_swiglu(gate, up, down, x, out=None):
+    """down(silu(gate x) * up x), all on the device."""
+    import torch
+    y = out if out is not None else torch.empty(down.rows, dtype=torch.float32, device=x.device)
+    check(lib().frk_hip_ffn_swiglu_dev(gate.handle, up.handle, down.handle, C.c_void_p(x.data_ptr()),
+                                       C.c_void_p(y.data_ptr()), _stream()))
+    return y
+
+
+class MatvecLaunch(C.Structure):
+    _fields_ = [("kind", C.c_int), ("weights", C.c_void_p), ("weights_len", C.c_size_t), ("rows", C.c_size_t),
+                ("row_bytes", C.c_size_t)]
+
+    @classmethod
+    def of(cls, kind, weights, rows, row_bytes):
+        weights = np.ascontiguousarray(weights, np.uint8)
+        m = cls(kind, weights.ctypes.data, weights.size, rows, row_bytes)
+        m._keep = weights
+        return m
+
+
+def launch_matvec_multi(x, launches):
+    """frink_cuda::matvec_launch::launch_matvec_multi over host buffers."""
+    x = np.ascontiguousarray(x, np.float32)
+    n = len(launches)
+    arr = (MatvecLaunch * n)(*launches)
+    outs = [np.empty(l.rows, np.float32) for l in launches]
+    ps = (C.c_void_p * n)(*[o.ctypes.data for o in outs])
+    check(lib().frk_hip_launch_matvec_multi(_np_ptr(x), x.size, arr, n, ps))
+    return outs
+
+
+def launch_dense_ffn_swiglu(gate, up, down, x):
+    """frink_cuda::matvec_launch::launch_dense_ffn_swiglu over host buffers."""
+    x = np.ascontiguousarray(x, np.float32)
+    out = np.empty(down.rows, np.float32)
+    check(lib().frk_hip_launch_dense_ffn_swiglu(C.byref(gate), C.byref(up), C.byref(down), _np_ptr(x), x.size,
+                                                _np_ptr(out)))
+    return out
 
 
 # ---- host-buffer entry points: numpy in, numpy out ----

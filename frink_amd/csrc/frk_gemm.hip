@@ -506,7 +506,7 @@ int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Fl
 }
 
 // Grouped GEMM over the experts stacked in `w` (expert e = rows [e*rows_e, (e+1)*rows_e)):
-// y[p][rows_e] for every output row p listed in the tiles (32 rows per tile at most).
+// y[p][rows_e] for every output row p listed in the tiles (MOE_TILE rows per tile at most).
 int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
                              const _Float16 *bsf, const int4 *tiles, const int *n_tiles, int max_tiles,
                              const int *gather, float *y, hipStream_t s) {
@@ -525,7 +525,7 @@ int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *
     g.gather = gather;
     g.row_tiles = (int)((rows_e + 127) / 128);
     g.tok_tiles = max_tiles;
-    return launch_variant<4, 1, 1, 2, true>(g, (unsigned)(g.row_tiles * max_tiles), s);
+        return launch_variant<4, 1, MOE_TILE / 32, 2, true>(g, (unsigned)(g.row_tiles * max_tiles), s);
 }
 
 }  // namespace frk

@@ -125,7 +125,8 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
 // Q8_K quantization in the GEMM's form: the 16-wide sums as f16 (exact)
 int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Float16 *bsf,
                               hipStream_t s);
-// grouped (per-expert) GEMM: tiles {expert, first, count, 0} of at most 32 output rows each
+// grouped (per-expert) GEMM: tiles {expert, first, count, 0} of at most MOE_TILE output rows each
+constexpr int MOE_TILE = 32;  // 64 was measured slower: fewer, longer workgroups
 int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
                              const _Float16 *bsf, const int4 *tiles, const int *n_tiles,
                              int max_tiles, const int *gather, float *y, hipStream_t s);
@@ -136,6 +137,7 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
                    void *ws, hipStream_t s);
 int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hidden, int ffn, float *gate_out,
                            float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of, hipStream_t s);
+int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s);
 int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, int k, int norm, int32_t *ids,
                                float *weights, hipStream_t s);
 // prefetch-all GEMVs (one wavefront per row, no LDS) for rows of 33..256 units

@@ -91,7 +91,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *wave_tot, int &t
 //   group_off[E+1]   bucket boundaries in the grouped order
 //   gather[pairs]    token of each grouped position
 //   pos_of[pairs]    grouped position of pair (tok*k + slot); -1 for an id outside [0, E)
-//   tiles / n_tiles  the buckets cut into runs of at most 32 positions for the grouped GEMM
+//   tiles / n_tiles  the buckets cut into runs of at most MOE_TILE positions for the grouped GEMM
 // One workgroup of 1024 threads; E <= 1024.  Pairs are taken 1024 at a time in pair order (which
 // is token-major); a pair's place in its bucket is the count of earlier pairs of that expert:
 // those of earlier rounds (run), of earlier wavefronts of this round (a prefix over the
@@ -117,14 +117,14 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
     __syncthreads();
     {
         const int c = tid < n_experts ? cnt[tid] : 0;
-        const int nt = (c + 31) >> 5;
+        const int nt = (c + MOE_TILE - 1) / MOE_TILE;
         int total, total_tiles;
         const int o = block_exclusive_scan(c, wave_tot, total);
         const int t = block_exclusive_scan(nt, wave_tot, total_tiles);
         off[tid] = o;
         if (tid < n_experts) {
             group_off[tid] = o;
-            for (int i = 0; i < nt; i++) tiles[t + i] = make_int4(tid, o + 32 * i, min(32, c - 32 * i), 0);
+            for (int i = 0; i < nt; i++) tiles[t + i] = make_int4(tid, o + MOE_TILE * i, min(MOE_TILE, c - MOE_TILE * i), 0);
         }
         if (tid == 0) {
             group_off[n_experts] = total;
@@ -189,6 +189,18 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__res
     if (lane == 0) d[b] = dd;
 }
 
+// silu(gate) * up, elementwise (frink_core::matmul::swiglu, crates/frink-core/src/matmul.rs:634-650;
+// glu_mul_device in crates/frink-cuda/src/matvec_launch.rs:551-570)
+__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up,
+                                                     size_t n, float *__restrict__ act) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float g = gate[i];
+    act[i] = __fdiv_rn(g, 1.0f + (float)exp(-(double)g)) * up[i];
+}
+
+int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s);
+
 // out[tok] = sum over the token's slots, ascending expert id, of w * down[pos]: the order of the
 // reference's expert loop (ffn_batch.rs:388-423), each term a separate multiply and add.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ down, const int32_t *__restrict__ ids,
@@ -237,6 +249,12 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
+int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s) {
+    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gate, up, n, act);
+    FRK_LAUNCH_CHECK("swiglu");
+    return FRK_OK;
+}
+
 int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, int k, int norm, int32_t *ids,
                                float *weights, hipStream_t s) {
     hipLaunchKernelGGL(route_top_k_softmax_kernel, dim3(batch), dim3(64), 0, s, logits, batch, n_experts, k,
@@ -280,7 +298,7 @@ static MoeScratch moe_carve(void *base, size_t batch, int k, int n_experts, int 
     m.gather = (int *)take(pairs * 4);
     m.pos_of = (int *)take(pairs * 4);
     m.n_tiles = (int *)take(256);
-    m.tiles = (int4 *)take((pairs / 32 + n_experts + 1) * 16);
+    m.tiles = (int4 *)take((pairs / MOE_TILE + n_experts + 1) * 16);
     if (end) *end = (size_t)(p - (char *)base);
     return m;
 }
@@ -316,7 +334,7 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     const int hidden = (int)gate->cols, ffn = (int)down->cols;
     const size_t pairs = batch * (size_t)k;
     const MoeScratch m = moe_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
-    const int max_tiles = (int)(pairs / 32 + n_experts);
+    const int max_tiles = (int)(pairs / MOE_TILE + n_experts);
 
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, k, n_experts, m.group_off, m.gather,
                        m.pos_of, m.tiles, m.n_tiles);

@@ -7,6 +7,7 @@
 #include <mutex>
 #include <string>
 #include <utility>
+#include <vector>
 
 #include "frk_internal.hpp"
 
@@ -415,6 +416,60 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     return FRK_OK;
 }
 
+int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *x, float *const *ys, void *stream) {
+    clear_error();
+    if (n == 0) return FRK_OK;
+    if (!ws || !x || !ys) return set_error(FRK_ERR_ARG, "frk_hip_gemv_multi_dev: null argument");
+    hipStream_t s = (hipStream_t)stream;
+    bool any_k = false;
+    for (size_t i = 0; i < n; i++) {
+        if (!ws[i] || !ys[i]) return set_error(FRK_ERR_ARG, "frk_hip_gemv_multi_dev: null matrix or output %zu", i);
+        if (ws[i]->cols != ws[0]->cols)
+            return set_error(FRK_ERR_SHAPE, "matrix %zu has %zu columns, matrix 0 has %zu: they share one activation", i,
+                             ws[i]->cols, ws[0]->cols);
+        any_k = any_k || ws[i]->kind == FRK_KIND_Q4_K || ws[i]->kind == FRK_KIND_Q6_K;
+    }
+    // one Q8_K quantization for every K-quant matrix of the group
+    Q8KActs a = {nullptr, nullptr, nullptr};
+    if (any_k) {
+        int rc = quantize_acts_q8_k(ws[0], x, 1, s, &a);
+        if (rc) return rc;
+    }
+    for (size_t i = 0; i < n; i++) {
+        int rc;
+        if (ws[i]->kind == FRK_KIND_Q8_0) rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
+        else rc = frk_hip_gemv_q8k_dev(ws[i], a.q, a.d, a.bsums, ys[i], stream);
+        if (rc) return rc;
+    }
+    return FRK_OK;
+}
+
+int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down, const float *x,
+                           float *y, void *stream) {
+    clear_error();
+    if (!gate || !up || !down || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_ffn_swiglu_dev: null argument");
+    if (gate->rows != up->rows || gate->cols != up->cols || down->cols != gate->rows)
+        return set_error(FRK_ERR_SHAPE, "FFN shapes disagree: gate %zux%zu up %zux%zu down %zux%zu", gate->rows, gate->cols,
+                         up->rows, up->cols, down->rows, down->cols);
+    hipStream_t s = (hipStream_t)stream;
+    const size_t ffn = gate->rows;
+    // scratch for gate(x), up(x) and silu(gate)*up behind the quantized activation
+    const size_t q_cols = std::max(gate->cols, down->cols);  // either projection may quantize its input here
+    const size_t q_area = round_up(q_cols, 256) + round_up(q_cols / 32 * 4, 256) + round_up(q_cols / 8, 256);
+    void *ws = nullptr;
+    int rc = workspace(q_area + 3 * round_up(ffn * 4, 256), s, &ws);
+    if (rc) return rc;
+    float *g_out = (float *)((char *)ws + q_area), *u_out = g_out + round_up(ffn * 4, 256) / 4,
+          *act = u_out + round_up(ffn * 4, 256) / 4;
+    const frk_weights *pair[2] = {gate, up};
+    float *outs[2] = {g_out, u_out};
+    rc = frk_hip_gemv_multi_dev(pair, 2, x, outs, stream);
+    if (rc) return rc;
+    rc = launch_swiglu(g_out, u_out, ffn, act, s);
+    if (rc) return rc;
+    return frk_hip_gemv_dev(down, act, y, FRK_ACT_F32, stream);
+}
+
 int frk_hip_route_top_k_softmax_dev(const float *logits, size_t batch, size_t n_experts, size_t k, int norm,
                                     int32_t *ids, float *weights, void *stream) {
     clear_error();
@@ -560,6 +615,110 @@ int frk_hip_launch_mul_mm(int kind, const uint8_t *weights, size_t weights_len, 
     if (x_len < batch * n_cols)
         return set_error(FRK_ERR_SHAPE, "activations too small: got %zu values, want %zu", x_len, batch * n_cols);
     return host_launch(kind, weights, n_rows * row_bytes, x_batch, n_rows, n_cols, batch, out);
+}
+
+
+static int check_launch(const frk_matvec_launch *l, size_t *cols) {
+    if (!l || !l->weights) return set_error(FRK_ERR_ARG, "null launch or weights");
+    if (!frk_hip_has_launch(l->kind)) return set_error(FRK_ERR_UNSUPPORTED, "no matvec kernel for quant kind %d", l->kind);
+    size_t bb = (size_t)block_bytes(l->kind), be = (size_t)block_elems(l->kind);
+    if (l->rows == 0) return set_error(FRK_ERR_SHAPE, "empty shape: rows=0");
+    if (l->row_bytes == 0 || l->row_bytes % bb)
+        return set_error(FRK_ERR_SHAPE, "row_bytes %zu is not a whole number of %zu-byte blocks", l->row_bytes, bb);
+    if (l->weights_len != l->rows * l->row_bytes)
+        return set_error(FRK_ERR_SHAPE, "weights are %zu bytes, %zu rows of %zu bytes need %zu", l->weights_len, l->rows,
+                         l->row_bytes, l->rows * l->row_bytes);
+    *cols = l->row_bytes / bb * be;
+    return FRK_OK;
+}
+
+// Uploads x once, runs `dev_fn` on the library's stream, downloads n outputs; weights stay resident.
+int frk_hip_launch_matvec_multi(const float *x, size_t x_len, const frk_matvec_launch *launches, size_t n,
+                                float *const *outs) {
+    clear_error();
+    if (n == 0) return FRK_OK;
+    if (!x || !launches || !outs) return set_error(FRK_ERR_ARG, "frk_hip_launch_matvec_multi: null argument");
+    std::vector<frk_weights *> ws(n, nullptr);
+    size_t total_rows = 0;
+    int rc = FRK_OK;
+    for (size_t i = 0; i < n && !rc; i++) {
+        size_t cols = 0;
+        rc = check_launch(&launches[i], &cols);
+        if (!rc && cols != x_len)
+            rc = set_error(FRK_ERR_SHAPE, "activation has %zu values, matrix %zu needs %zu", x_len, i, cols);
+        if (!rc && !outs[i]) rc = set_error(FRK_ERR_ARG, "output %zu is null", i);
+        if (!rc)
+            rc = frk_hip_weights_register(launches[i].kind, launches[i].weights, launches[i].weights_len, launches[i].rows,
+                                          cols, &ws[i]);
+        total_rows += launches[i].rows;
+    }
+    if (!rc) {
+        std::lock_guard<std::mutex> lk(g_launch_mu);
+        rc = stage_buffers(x_len * sizeof(float), total_rows * sizeof(float));
+        hipStream_t s = g_dev.stream;
+        if (!rc) {
+            hipError_t e = hipMemcpyAsync(g_dev.x_dev, x, x_len * sizeof(float), hipMemcpyHostToDevice, s);
+            if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(x): %s", hipGetErrorString(e));
+        }
+        std::vector<float *> ys(n);
+        size_t off = 0;
+        for (size_t i = 0; i < n; i++) {
+            ys[i] = (float *)g_dev.y_dev + off;
+            off += launches[i].rows;
+        }
+        if (!rc) rc = frk_hip_gemv_multi_dev(ws.data(), n, (const float *)g_dev.x_dev, ys.data(), s);
+        for (size_t i = 0; i < n && !rc; i++) {
+            hipError_t e = hipMemcpyAsync(outs[i], ys[i], launches[i].rows * sizeof(float), hipMemcpyDeviceToHost, s);
+            if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(y): %s", hipGetErrorString(e));
+        }
+        hipError_t e = hipStreamSynchronize(s);
+        if (!rc && e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e));
+    }
+    char keep[sizeof g_err];
+    memcpy(keep, g_err, sizeof keep);
+    for (frk_weights *w : ws)
+        if (w) frk_hip_weights_release(w);
+    memcpy(g_err, keep, sizeof keep);
+    return rc;
+}
+
+int frk_hip_launch_dense_ffn_swiglu(const frk_matvec_launch *gate, const frk_matvec_launch *up,
+                                    const frk_matvec_launch *down, const float *x, size_t x_len, float *out) {
+    clear_error();
+    if (!x || !out) return set_error(FRK_ERR_ARG, "frk_hip_launch_dense_ffn_swiglu: null argument");
+    const frk_matvec_launch *ls[3] = {gate, up, down};
+    frk_weights *ws[3] = {nullptr, nullptr, nullptr};
+    size_t cols[3] = {0, 0, 0};
+    int rc = FRK_OK;
+    for (int i = 0; i < 3 && !rc; i++) rc = check_launch(ls[i], &cols[i]);
+    if (!rc && (cols[0] != x_len || cols[1] != x_len))
+        rc = set_error(FRK_ERR_SHAPE, "activation has %zu values, gate/up need %zu/%zu", x_len, cols[0], cols[1]);
+    if (!rc && (gate->rows != up->rows || cols[2] != gate->rows))
+        rc = set_error(FRK_ERR_SHAPE, "gate rows %zu, up rows %zu, down columns %zu must agree", gate->rows, up->rows, cols[2]);
+    for (int i = 0; i < 3 && !rc; i++)
+        rc = frk_hip_weights_register(ls[i]->kind, ls[i]->weights, ls[i]->weights_len, ls[i]->rows, cols[i], &ws[i]);
+    if (!rc) {
+        std::lock_guard<std::mutex> lk(g_launch_mu);
+        rc = stage_buffers(x_len * sizeof(float), down->rows * sizeof(float));
+        hipStream_t s = g_dev.stream;
+        if (!rc) {
+            hipError_t e = hipMemcpyAsync(g_dev.x_dev, x, x_len * sizeof(float), hipMemcpyHostToDevice, s);
+            if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(x): %s", hipGetErrorString(e));
+        }
+        if (!rc) rc = frk_hip_ffn_swiglu_dev(ws[0], ws[1], ws[2], (const float *)g_dev.x_dev, (float *)g_dev.y_dev, s);
+        if (!rc) {
+            hipError_t e = hipMemcpyAsync(out, g_dev.y_dev, down->rows * sizeof(float), hipMemcpyDeviceToHost, s);
+            if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(y): %s", hipGetErrorString(e));
+        }
+        hipError_t e = hipStreamSynchronize(s);
+        if (!rc && e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e));
+    }
+    char keep[sizeof g_err];
+    memcpy(keep, g_err, sizeof keep);
+    for (frk_weights *w : ws)
+        if (w) frk_hip_weights_release(w);
+    memcpy(g_err, keep, sizeof keep);
+    return rc;
 }
 
 }  // extern "C"

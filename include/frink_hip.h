@@ -126,6 +126,29 @@ int frk_hip_launch_mul_mm(int kind, const uint8_t *weights, size_t weights_len,
                           const float *x_batch, size_t x_len, size_t n_rows, size_t n_cols,
                           size_t batch, size_t row_bytes, float *out);
 
+/* One matvec of a group that shares an activation:
+ * frink_cuda::matvec_launch::MatvecLaunch (crates/frink-cuda/src/matvec_launch.rs:485-493). */
+typedef struct {
+    int kind;
+    const uint8_t *weights;
+    size_t weights_len;
+    size_t rows;
+    size_t row_bytes;
+} frk_matvec_launch;
+
+/* frink_cuda::matvec_launch::launch_matvec_multi (matvec_launch.rs:500-534): uploads x once, runs
+ * the n matvecs (q/k/v, or gate and up) on resident weights -- the K-quant matrices share ONE Q8_K
+ * quantization of x -- and downloads outs[i][launches[i].rows]. */
+int frk_hip_launch_matvec_multi(const float *x, size_t x_len, const frk_matvec_launch *launches,
+                                size_t n, float *const *outs);
+
+/* frink_cuda::matvec_launch::launch_dense_ffn_swiglu (matvec_launch.rs:551-570):
+ * out = down(silu(gate x) * up x) with one upload of x and one download of out.  gate and up have
+ * the same rows and columns; down's columns equal their rows. */
+int frk_hip_launch_dense_ffn_swiglu(const frk_matvec_launch *gate, const frk_matvec_launch *up,
+                                    const frk_matvec_launch *down, const float *x, size_t x_len,
+                                    float *out);
+
 /* ---- device-pointer entry points (asynchronous on `stream`, a hipStream_t or NULL) ---- */
 
 /* y[rows] = W x for one activation vector in HBM.  K-quants: x is quantized to Q8_K
@@ -140,6 +163,15 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x_dev, float *y_dev, int
  * BatchActs::Q8K (crates/frink-core/src/weight_matrix.rs:757-768).  K-quants only. */
 int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float *d_dev,
                          const int16_t *bsums_dev, float *y_dev, void *stream);
+
+/* The device forms of the two calls above: ys[i][ws[i]->rows] = ws[i] x for matrices of equal
+ * column count (WeightMatrix::apply_gpu_multi, crates/frink-core/src/weight_matrix.rs:3504-3667), and
+ * y[down->rows] = down(silu(gate x) * up x) (WeightMatrix::apply_gpu_dense_ffn_swiglu,
+ * weight_matrix.rs:3676-3787; silu as crates/frink-core/src/matmul.rs:634-650). */
+int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *x_dev,
+                           float *const *ys_dev, void *stream);
+int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down,
+                           const float *x_dev, float *y_dev, void *stream);
 
 /* y[batch][rows] = x[batch][cols] W^T (WeightMatrix::apply_batch_with_acts,
  * crates/frink-core/src/weight_matrix.rs:2481).  Any batch >= 1. */

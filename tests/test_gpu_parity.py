@@ -470,3 +470,69 @@ def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
     one = w.gemv(xd[5].contiguous()).cpu().numpy()
     assert np.abs(one - y[5]).max() <= 1e-5 * np.abs(one).max()
     w.release()
+
+
+# ------------------------------------------------------------------ shared activation, fused FFN
+
+def _ffn_oracle(gate, up, down, ffn, hidden, x):
+    g = fo.gemv(fo.Q4_K, gate, ffn, hidden, x)
+    u = fo.gemv(fo.Q4_K, up, ffn, hidden, x)
+    return g, u, fo.swiglu(g, u)
+
+
+def test_gemv_multi_shares_one_quantized_activation(fa):
+    from frink_amd import synth
+    hidden = 1024
+    shapes = [(fo.Q4_K, 96), (fo.Q6_K, 40), (fo.Q8_0, 72), (fo.Q4_K, 33)]
+    datas = [make_weights(k, r, hidden, seed=300 + i) for i, (k, r) in enumerate(shapes)]
+    ws = [fa.Weights.from_host(k, d, r, hidden) for (k, r), d in zip(shapes, datas)]
+    x = synth.activations(301, 1, hidden, outlier_frac=0.01)[0]
+    ys = fa.gemv_multi(ws, to_dev(x))
+    for (k, r), d, y in zip(shapes, datas, ys):
+        want = fo.gemv(k, d, r, hidden, x, fo.F32_DOT if k == fo.Q8_0 else fo.INT_DOT)
+        assert_rows_close(y.cpu().numpy()[None], want[None], "gemv_multi kind %d" % k)
+    # the host-buffer form (launch_matvec_multi)
+    launches = [fa.MatvecLaunch.of(k, d, r, hidden // fo.BLOCK[k][1] * fo.BLOCK[k][0]) for (k, r), d in zip(shapes, datas)]
+    outs = fa.launch_matvec_multi(x, launches)
+    for o, y in zip(outs, ys):
+        assert np.array_equal(bits(o), bits(y.cpu().numpy()))
+    with pytest.raises(fa.BackendError) as e:
+        fa.launch_matvec_multi(x[:512], launches)
+    assert e.value.code == fa.ERR_SHAPE
+    for w in ws:
+        w.release()
+
+
+@pytest.mark.parametrize("hidden,ffn", [(512, 768), (4096, 14336)])
+def test_dense_ffn_swiglu(fa, hidden, ffn):
+    """gate/up Q4_K, down Q6_K (the Llama-3-8B FFN at full size): each stage from the device's own
+    previous stage, as for the MoE layer -- the down projection quantizes its input, a step function."""
+    from frink_amd import synth
+    print("ffn", hidden, ffn, flush=True)
+    gate = make_weights(fo.Q4_K, ffn, hidden, seed=401)
+    up = make_weights(fo.Q4_K, ffn, hidden, seed=402)
+    down = make_weights(fo.Q6_K, hidden, ffn, seed=403)
+    x = synth.activations(404, 1, hidden)[0]
+    wg, wu, wd = (fa.Weights.from_host(k, d, r, c) for k, d, r, c in
+                  ((fo.Q4_K, gate, ffn, hidden), (fo.Q4_K, up, ffn, hidden), (fo.Q6_K, down, hidden, ffn)))
+    xd = to_dev(x)
+    y = fa.ffn_swiglu(wg, wu, wd, xd).cpu().numpy()
+    g_dev, u_dev = (t.cpu().numpy() for t in fa.gemv_multi([wg, wu], xd))
+    g, u, _ = _ffn_oracle(gate, up, down, ffn, hidden, x)
+    assert_rows_close(g_dev[None], g[None], "gate")
+    assert_rows_close(u_dev[None], u[None], "up")
+    act = fo.swiglu(g_dev, u_dev)                      # the device's gate/up through the oracle's SwiGLU
+    want = fo.gemv(fo.Q6_K, down, hidden, ffn, act)
+    assert_rows_close(y[None], want[None], "down(silu(gate)*up)")
+    # end to end against the oracle's own chain
+    e2e = fo.gemv(fo.Q6_K, down, hidden, ffn, fo.swiglu(g, u))
+    rel = np.abs(y - e2e).max() / np.abs(e2e).max()
+    print("ffn end to end: %.3g of ||y||inf" % rel, flush=True)
+    assert rel <= 10 * TOL
+    if hidden == 512:  # the host-buffer form (launch_dense_ffn_swiglu)
+        out = fa.launch_dense_ffn_swiglu(fa.MatvecLaunch.of(fo.Q4_K, gate, ffn, hidden // 256 * 144),
+                                         fa.MatvecLaunch.of(fo.Q4_K, up, ffn, hidden // 256 * 144),
+                                         fa.MatvecLaunch.of(fo.Q6_K, down, hidden, ffn // 256 * 210), x)
+        assert np.array_equal(bits(out), bits(y))
+    for w in (wg, wu, wd):
+        w.release()
