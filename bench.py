@@ -248,6 +248,35 @@ def main():
             "TOPS": round(2.0 * T * K * 3 * F * H / (t / 100) / 1e12, 1)}
         for w in experts:
             w.release()
+        # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call
+        # (gate and up share one quantized activation, SwiGLU, down)
+        g8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
+        u8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
+        d6 = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=79)).to(dev)
+        dn = [fa.Weights.from_device(fa.Q6_K, d6, cols, rows) for _ in range(8)]
+        x8 = torch.from_numpy(synth.activations(9, 8, cols)).to(dev)
+        h8 = torch.from_numpy(synth.activations(10, 8, rows)).to(dev)
+        y8 = torch.empty((8, rows), dtype=torch.float32, device=dev)
+        z8 = torch.empty((8, cols), dtype=torch.float32, device=dev)
+        for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096", g8, x8, y8),
+                                      ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8)):
+            def step5(i, mats=mats, xin=xin, yout=yout):
+                mats[i % 8].gemm(xin, out=yout)
+            _, t = time_graph(torch, step5, 400, 8)
+            wb = mats[0].rows * (mats[0].cols // 256) * (144 if mats[0].kind == kind else 210)
+            extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
+                           "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+        yf = torch.empty(cols, dtype=torch.float32, device=dev)
+
+        def step6(i):
+            fa.ffn_swiglu(g8[i % 8], u8[i % 8], dn[i % 8], xd, out=yf)
+        _, t = time_graph(torch, step6, 400, 8)
+        fb = 2 * wbytes + d6.numel()
+        extra["decode FFN 4096->14336->4096 (gate, up Q4_K; down Q6_K)"] = {
+            "us_per_step": round(t / 400 * 1e6, 2), "GBs": round(fb / (t / 400) / 1e9, 1),
+            "frac_of_hbm_peak": round(fb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+        for w in g8 + u8 + dn:
+            w.release()
         out["extra"] = extra
 
     if not args.no_cpu:
