@@ -114,4 +114,45 @@ __device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, i
            ((uint32_t)(q3 & 0xff) << 24);
 }
 
+// One record of the tiled Q8_K form (32 rows x one 256-wide block) by a workgroup of 256 threads:
+// wavefront w quantizes rows 8w..8w+7 (`load(r)` returns this lane's four values of row r, zeros for
+// a row that does not exist), the record is put together in LDS and leaves as three contiguous
+// copies -- quantizing straight into the tiled form would write it in 4-byte pieces.
+struct Q8KRecordLds {
+    uint32_t q[2048];
+    _Float16 bs[512];
+    float d[32];
+};
+template <class Load>
+__device__ __forceinline__ void quantize_q8k_record(const Q8KTiled &a, size_t rec, Q8KRecordLds &L, Load load) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float4 v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = load(wave * 8 + i);
+    // the lane's four values are k = 4*lane..: 32-wide slice lane/8, 16-byte half (lane/4)%2 of it
+    const int ks = lane >> 3, half = (lane >> 2) & 1, g = lane >> 2;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int r = wave * 8 + i;
+        float dd;
+        int bs;
+        const uint32_t packed = quantize_q8_k_lane(v[i], dd, bs);
+        L.q[ks * 256 + (half * 32 + r) * 4 + (lane & 3)] = packed;
+        if ((lane & 3) == 0) L.bs[((g >> 3) * 32 + r) * 8 + (g & 7)] = (_Float16)bs;
+        if (lane == 0) L.d[r] = dd;
+    }
+    __syncthreads();
+    uint4 *dq = reinterpret_cast<uint4 *>(a.q + rec * 8192);
+    const uint4 *sq = reinterpret_cast<const uint4 *>(L.q);
+    dq[tid] = sq[tid];
+    dq[tid + 256] = sq[tid + 256];
+    if (tid < 64) reinterpret_cast<uint4 *>(a.bs + rec * 512)[tid] = reinterpret_cast<const uint4 *>(L.bs)[tid];
+    if (tid < 32) a.d[rec * 32 + tid] = L.d[tid];
+}
+// where quant k of (row, block kb) lives in the tiled form
+__device__ __forceinline__ size_t q8k_tiled_index(int nb, int row, int kb, int k) {
+    const size_t rec = (size_t)(row >> 5) * nb + kb;
+    return rec * 8192 + (k >> 5) * 1024 + (((k >> 4) & 1) * 32 + (row & 31)) * 16 + (k & 15);
+}
+
 }  // namespace frk

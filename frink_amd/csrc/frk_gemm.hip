@@ -27,8 +27,11 @@
 // iterations ago has landed".
 #include "frk_device.hpp"
 
+#include <type_traits>
+
 namespace frk {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -36,38 +39,49 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 
-// Activation side: Q8_K quantization plus the 16-wide sums as f16 (exact: |bsum| <= 16*127).
-// One wavefront per 256-value block.
-__global__ __launch_bounds__(256) void quantize_q8_k_gemm_kernel(const float *__restrict__ x, size_t n_blocks,
-                                                                 int8_t *__restrict__ q, float *__restrict__ d,
-                                                                 _Float16 *__restrict__ bsf) {
-    const int lane = threadIdx.x & 63;
-    const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (b >= n_blocks) return;
-    const float4 v = reinterpret_cast<const float4 *>(x + b * QK_K)[lane];
-    float dd;
-    int bs;
-    const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
-    reinterpret_cast<uint32_t *>(q + b * QK_K)[lane] = packed;
-    if ((lane & 3) == 0) bsf[b * 16 + (lane >> 2)] = (_Float16)bs;
-    if (lane == 0) d[b] = dd;
+// Activation side: Q8_K quantization (quantize_activations_q8_k, crates/frink-quant/src/act_quant.rs:69-104)
+// into the tiled form, one workgroup per record (32 rows x one block).
+// Without `gather`, out row r = x[r] (rows from `rows` to the end of the last tile become zeros); with
+// it, out row r = x[gather[r]] (zeros where the entry is negative) for the records that the first
+// *n_tiles tiles {expert, first row, rows in use, 0} of MOE_TILE rows have rows in.
+__global__ __launch_bounds__(256) void quantize_q8_k_tiled_kernel(const float *__restrict__ x, int rows, int nb,
+                                                                  const int *__restrict__ gather,
+                                                                  const int4 *__restrict__ tiles,
+                                                                  const int *__restrict__ n_tiles, Q8KTiled out) {
+    __shared__ Q8KRecordLds L;
+    const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
+    if (gather) {
+        const int t = t32 * 32 / MOE_TILE;
+        if (t >= *n_tiles || tiles[t].z <= t32 * 32 - t * MOE_TILE) return;
+    }
+    quantize_q8k_record(out, (size_t)t32 * nb + kb, L, [&](int r) {
+        const int row = t32 * 32 + r;
+        const int src = gather ? gather[row] : (row < rows ? row : -1);
+        if (src < 0) return make_float4(0.f, 0.f, 0.f, 0.f);
+        return reinterpret_cast<const float4 *>(x + ((size_t)src * nb + kb) * QK_K)[lane];
+    });
 }
 
 struct GemmArgs {
     const uint8_t *W;
     size_t row_stride;
     int rows, nb, M;
-    const int8_t *aq;     // [M][nb*256]
-    const float *ad;      // [M][nb]
-    const _Float16 *bsf;  // [M][nb*16]
-    float *y;             // [M][rows]
+    Q8KTiled a;  // ceil(M / 32) tiles
+    float *y;    // [M][rows]
     int row_tiles, tok_tiles;
-    // grouped (per-expert) form: tile t covers output rows first..first+count of expert e, whose
-    // weights are rows [e*rows, (e+1)*rows) of W; activation row of output row p is gather[p]
-    // (p itself when gather is null).  Tiles past *n_tiles exit at once.
-    const int4 *tiles;    // {expert, first, count, 0}
+};
+
+// The grouped form: work items (tile, matrix, row group of 256 rows) streamed by persistent workgroups.
+struct StreamArgs {
+    const uint8_t *W[2];
+    float *y[2];  // [32 * tiles][rows]
+    int n_mat;
+    size_t row_stride;
+    int rows, nb;  // of one expert
+    Q8KTiled a;
+    const int4 *tiles;  // {expert, 32 * t, rows in use, 0}
     const int *n_tiles;
-    const int *gather;
+    int row_tiles;  // ceil(rows / 256)
 };
 
 // One block of a lane's weight row as MFMA B operands: the two pre-scaled planes of the 8 sub-blocks,
@@ -268,7 +282,7 @@ struct GemmLds {
     static constexpr size_t BYTES = (size_t)2 * A_STAGE + (size_t)WS * W_STAGE;
 };
 
-template <int RG, int WT, int MT, int WS, bool GROUPED>
+template <int RG, int WT, int MT, int WS>
 __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
     using L = GemmLds<RG, WT, MT, WS>;
     constexpr int NW = RG * WT, NT = L::NT, TM = 32 * NT, ROWS = 32 * RG;
@@ -287,46 +301,28 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     const int li = lane & 31, lg = lane >> 5;
     const int rgrp = wave % RG, tgrp = wave / RG;
 
+    // workgroups that share weight rows (different token tiles) sit on one XCD (block id mod 8)
     const int bid = blockIdx.x;
-    int row_tile, tok0, n_tok, w_first_row;
-    if (GROUPED) {
-        row_tile = bid % g.row_tiles;
-        const int t = bid / g.row_tiles;
-        if (t >= *g.n_tiles) return;  // uniform per workgroup
-        const int4 ti = g.tiles[t];
-        tok0 = ti.y;
-        n_tok = ti.y + ti.z;  // one past the last output row of this tile
-        w_first_row = ti.x * g.rows;
-    } else {
-        // workgroups that share weight rows (different token tiles) sit on one XCD (block id mod 8)
-        const int per_group = 8 * g.tok_tiles;
-        const int grp = bid / per_group, in_grp = bid % per_group;
-        row_tile = grp * 8 + (in_grp & 7);
-        if (row_tile >= g.row_tiles) return;  // uniform per workgroup
-        tok0 = (in_grp >> 3) * TM;
-        n_tok = g.M;
-        w_first_row = 0;
-    }
+    const int per_group = 8 * g.tok_tiles;
+    const int grp = bid / per_group, in_grp = bid % per_group;
+    const int row_tile = grp * 8 + (in_grp & 7);
+    if (row_tile >= g.row_tiles) return;  // uniform per workgroup
+    const int tok0 = (in_grp >> 3) * TM;
     const int row0 = row_tile * ROWS + rgrp * 32;  // this wavefront's first weight row
     const int row = row0 + li;
-    const int K = g.nb * QK_K;
     const int nb = g.nb;
-    // activation row that feeds output row tok0 + t (clamped into the tile)
-    auto act_row = [&](int t) {
-        const int p = min(tok0 + t, n_tok - 1);
-        return (GROUPED && g.gather) ? g.gather[p] : p;
-    };
+    const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
 
     // ---- what this lane fetches ----
-    // quants chunk (tile t, slice ks): lane j brings the k-half j/32 (16 bytes) of token j%32's 32-byte
-    // slice to byte 16*j of the chunk, which is what lane j of the consumer reads.  Same for the bsums.
+    // activations: the tiled form is the LDS image, so chunk (tile t, slice ks) is 1 KB of consecutive
+    // memory and lane j brings its bytes 16*j..; same for the sums.  Tiles past the last one repeat it.
     const int8_t *a_src[NT];
 #pragma unroll
-    for (int t = 0; t < NT; t++) a_src[t] = g.aq + (size_t)act_row(t * 32 + li) * K + lg * 16;
+    for (int t = 0; t < NT; t++) a_src[t] = g.a.q + (size_t)min(tile0 + t, last_tile) * nb * 8192 + lane * 16;
     // with fewer chunks than wavefronts some fetch a chunk twice, into the same place
     const int bs_tile = wave % NT, da_chunk = wave % N_DA;
-    const _Float16 *b_src = g.bsf + (size_t)act_row(bs_tile * 32 + li) * nb * 16 + lg * 8;
-    const float *d_src = g.ad + (size_t)act_row(da_chunk * 64 + lane) * nb;
+    const _Float16 *b_src = g.a.bs + (size_t)min(tile0 + bs_tile, last_tile) * nb * 512 + lane * 8;
+    const float *d_src = g.a.d + (size_t)min(tile0 + 2 * da_chunk + lg, last_tile) * nb * 32 + li;
     // weights: a row group's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of chunk c, so that
     // LDS holds the rows back to back (144 bytes each) and consecutive lanes read consecutive memory.
     // With WT = 2 the two wavefronts of a row group split the five chunks (3 + 2, one fetched twice).
@@ -339,7 +335,7 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
         w_chunk[i] = c;
         const int p = min(c * 64 + lane, 287);
         const int r = min(row0 + p / 9, g.rows - 1);
-        w_src[i] = g.W + (size_t)(w_first_row + r) * g.row_stride + (p % 9) * 16;
+        w_src[i] = g.W + (size_t)r * g.row_stride + (p % 9) * 16;
     }
 
     auto issue_acts = [&](int kb) {
@@ -349,10 +345,10 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
 #pragma unroll
             for (int i = 0; i < 8 / NW; i++) {
                 const int ks = ((wave + t) % NW) + NW * i;
-                load_to_lds16(a_src[t] + (size_t)kb * QK_K + ks * 32, st + (t * 8 + ks) * 1024);
+                load_to_lds16(a_src[t] + (size_t)kb * 8192 + ks * 1024, st + (t * 8 + ks) * 1024);
             }
-        load_to_lds16(b_src + (size_t)kb * 16, st + L::OFF_BS + bs_tile * 1024);
-        load_to_lds4(d_src + kb, st + L::OFF_DA + da_chunk * 256);
+        load_to_lds16(b_src + (size_t)kb * 512, st + L::OFF_BS + bs_tile * 1024);
+        load_to_lds4(d_src + kb * 32, st + L::OFF_DA + da_chunk * 256);
     };
     auto issue_weights = [&](int kb) {  // C_W loads
         uint8_t *st = lds_w + (kb % WS) * L::W_STAGE + rgrp * L::W_GROUP;
@@ -429,8 +425,320 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tgrp * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < n_tok) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < g.M) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
         }
+}
+
+// The 16 + 1 MFMAs of a tile, each waiting only for the operand it needs: the tile's nine LDS reads
+// (a0..a7, bs, in that order) must be the wavefront's youngest LDS operations.
+// (Each wait also names the running sum as modified, which pins it between its two MFMAs: without
+// that the MFMAs are free to sink below all the waits, and the chain starts only when the last
+// operand is there.)
+#define FRK_WAIT_LGKM(n, reg, acc) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(reg), "+v"(acc))
+__device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const BPlanes &B, TileAcc &X) {
+    const v16i zi = {0};
+    const v16f zf = {0.0f};
+    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    FRK_WAIT_LGKM(7, T.a1, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(6, T.a2, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(5, T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(4, T.a4, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(3, T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(2, T.a6, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(1, T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(0, T.bs, acc);
+    X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+}
+
+// The grouped (per-expert) GEMM for tiles of at most 32 activation rows: with so few rows per
+// expert the work is a stream over the experts' weights, bound by HBM, and what matters is that the
+// stream never stops.  Persistent workgroups (one per CU, 8 wavefronts, 256 weight rows) walk a list
+// of work items (tile, matrix, row group); one step = one 256-wide block of one item.  A step's data
+// travels into LDS two steps ahead, across item boundaries: the weights (a wavefront fetches and
+// reads only its own 32 rows, so that ring needs no barrier and a stage is refilled as soon as it
+// has been unpacked: two stages are two steps of distance) and the tile's activation record (shared,
+// four stages, one barrier per step).  A tile is up to 64 activation rows, two 32-row halves that
+// share the unpacked weights; the second half is neither fetched nor multiplied when not in use.
+// The two wavefronts of a SIMD (w and w+4) run half a step apart: the leading one unpacks step s
+// and then runs its MFMAs and epilogue; the lagging one runs the MFMAs and epilogue of step s-1
+// first and unpacks step s after them.  One's vector-ALU phase then faces the other's matrix phase
+// instead of both waiting for LDS, multiplying and scaling in lockstep behind the barrier.
+// Items of a tile sit on one XCD (block id mod 8), whose L2 then serves the tile's activations.
+struct StreamLds {
+    static constexpr int RG = 8;
+    static constexpr int W_WAVE = 32 * Q4_K_BYTES;  // a wavefront's 32 rows of one block
+    static constexpr int W_STAGE = RG * W_WAVE;     // 36864
+    static constexpr int W_STAGES = 2;
+    static constexpr int A_BS = 8192, A_DA = 9216;  // record of 32 rows: quants | sums | scales
+    static constexpr int A_HALF = 9472;
+    static constexpr int A_STAGE = 2 * A_HALF;       // a tile is two records
+    static constexpr int A_STAGES = 4;
+    static constexpr int OFF_A = W_STAGES * W_STAGE;
+    // {expert, rows in use} of each of the workgroup's items, filled once: looked up from LDS, an
+    // item change costs no global load (whose completion would count in vmcnt, in the middle of the
+    // prefetch bookkeeping)
+    static constexpr int OFF_ITEMS = OFF_A + A_STAGES * A_STAGE;
+    static constexpr int MAX_ITEMS = 128;
+    static constexpr size_t BYTES = (size_t)OFF_ITEMS + MAX_ITEMS * 8;
+};
+
+__global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(StreamArgs g) {
+    using L = StreamLds;
+    extern __shared__ uint4 smem_gemm[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lg = lane >> 5;
+    const int nb = g.nb;
+    const bool lagging = wave >= L::RG / 2;
+
+    // this workgroup's items: the list of its XCD holds the tiles t = xcd (mod 8), every (matrix, row
+    // group) of a tile in a row; the XCD's workgroups take list entries slot, slot + per_xcd, ...
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+    const int n_tiles = *g.n_tiles;
+    const int per_tile = g.n_mat * g.row_tiles;
+    const int list_len = (n_tiles > xcd ? (n_tiles - xcd + 7) / 8 : 0) * per_tile;
+    const int my_items = list_len > slot ? (list_len - slot + per_xcd - 1) / per_xcd : 0;
+    const int total_steps = my_items * nb;
+    if (total_steps == 0) return;
+    // (the quotients are wavefront-uniform but come out of the vector ALU; back in scalar registers
+    // they keep the address arithmetic that follows scalar)
+    auto item_of = [&](int ord, int &t, int &m, int &rg) {
+        const int j = slot + ord * per_xcd;
+        const int jt = __builtin_amdgcn_readfirstlane(j / per_tile);
+        const int w = j - jt * per_tile;
+        t = xcd + 8 * jt;
+        m = __builtin_amdgcn_readfirstlane(w / g.row_tiles);
+        rg = w - m * g.row_tiles;
+    };
+    {
+        int2 *table = reinterpret_cast<int2 *>(lds + L::OFF_ITEMS);
+        for (int i = tid; i < my_items; i += 64 * L::RG) {
+            const int4 ti = g.tiles[xcd + 8 * ((slot + i * per_xcd) / per_tile)];
+            table[i] = make_int2(ti.x, ti.z);
+        }
+        __syncthreads();
+    }
+    const uint32_t lds_items = lds_address(lds + L::OFF_ITEMS);
+    auto item_info = [&](int ord, int &expert, int &count) {
+        v2i v;
+        asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_items + ord * 8));
+        expert = __builtin_amdgcn_readfirstlane(v.x);
+        count = __builtin_amdgcn_readfirstlane(v.y);
+    };
+
+    // ---- the fetch side: a cursor (item, block) two steps ahead of the arithmetic ----
+    // weights of a step: this wavefront's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of
+    // chunk c (4.5 chunks, 5 loads); activations: quant slice `wave`, plus the sums (wavefront 0) or
+    // the scales (wavefront 1).  Addresses are a uniform base that moves with the cursor plus a lane
+    // offset that is fixed per item.  Registers are short here, so of the five weight offsets only
+    // the first is kept: piece p + 64 = 7 rows + 1 piece further on, one more row where the piece
+    // index wraps past 8.  (Everything else the fetch needs is recomputed from the lane number.)
+    uint32_t w_off0 = 0;
+    // activations: quant slice `wave` of each half in use, plus one of the four small pieces: sums
+    // (wavefronts 0, 2) and scales (1, 3) of the first (0, 1) and second half (2, 3)
+    const bool x_sums = (wave & 1) == 0;
+    auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
+    };
+    const uint8_t *f_w, *f_x;
+    const int8_t *f_q;
+    int f_ord = 0, f_kb = 0, f_step = 0;
+    bool f_two = false;  // the cursor's tile has rows in its second half
+    int issued = 0;      // loads of the fetch most recently issued by this wavefront
+    auto point_at = [&](int ord) {  // uniform
+        int t, m, rg, expert, count;
+        item_of(ord, t, m, rg);
+        item_info(ord, expert, count);
+        f_w = (m ? g.W[1] : g.W[0]) + (size_t)expert * g.rows * g.row_stride;
+        const int l = opaque_lane();
+        w_off0 = (uint32_t)(rg * (32 * L::RG) + wave * 32 + l / 9) * (uint32_t)g.row_stride + (uint32_t)(l % 9) * 16;
+        f_two = count > 32;
+        const size_t rec = (size_t)(2 * t + (wave >> 1 & 1)) * nb;  // the small piece's half
+        f_q = g.a.q + (size_t)2 * t * nb * 8192;
+        f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.a.bs + rec * 512)
+                     : reinterpret_cast<const uint8_t *>(g.a.d + rec * 32);
+    };
+    auto fetch_acts = [&]() {  // of the cursor's step
+        uint8_t *st = lds + L::OFF_A + (f_step & 3) * L::A_STAGE;
+        const int l = opaque_lane();
+        const uint32_t q_off = (uint32_t)(wave * 1024 + l * 16);
+        const uint32_t x_off = x_sums ? (uint32_t)l * 16 : (uint32_t)(l & 31) * 4;
+        load_to_lds16(f_q + q_off, st + wave * 1024);
+        issued = 1;
+        if (f_two) {
+            load_to_lds16(f_q + (size_t)nb * 8192 + q_off, st + L::A_HALF + wave * 1024);
+            issued = 2;
+        }
+        if (wave < 2 || (wave < 4 && f_two)) {
+            uint8_t *half = st + (wave >> 1) * L::A_HALF;
+            if (x_sums) load_to_lds16(f_x + x_off, half + L::A_BS);
+            else load_to_lds4(f_x + x_off, half + L::A_DA);  // both lane halves fetch the same 32 scales
+            issued++;
+        }
+    };
+    auto fetch_weights = [&]() {  // of the cursor's step; moves the cursor on
+        uint8_t *st = lds + (f_step & 1) * L::W_STAGE + wave * L::W_WAVE;
+        const int l = opaque_lane();
+        const uint32_t r0 = (uint32_t)l % 9, stride = (uint32_t)g.row_stride;
+        // rows past the matrix (a last, partial row group) fetch its last piece instead
+        const uint32_t last = (uint32_t)(g.rows - 1) * stride + 128;
+#pragma unroll
+        for (int c = 0; c < 5; c++) {
+            const uint32_t off = w_off0 + c * (7 * stride + 16) + (r0 + c >= 9 ? stride - Q4_K_BYTES : 0u);
+            if (c < 4 || l < 32) load_to_lds16(f_w + min(off, last), st + c * 1024);
+        }
+        issued += 5;
+        f_step++;
+        f_w += Q4_K_BYTES;
+        f_q += 8192;
+        f_x += x_sums ? 1024 : 128;
+        if (++f_kb == nb) {
+            f_kb = 0;
+            if (++f_ord < my_items) point_at(f_ord);
+        }
+    };
+    auto wait_all_but_newest_step = [&]() {  // newest: the `issued` loads of the last fetch
+        if (issued == 6) wait_vm<6>();
+        else if (issued == 7) wait_vm<7>();
+        else wait_vm<8>();
+    };
+
+    point_at(0);
+    fetch_acts();
+    fetch_weights();
+    if (total_steps > 1) {
+        fetch_acts();
+        fetch_weights();
+        wait_all_but_newest_step();
+    } else {
+        wait_vm<0>();
+    }
+    lds_barrier();
+
+    // ---- the arithmetic: the whole loop once per role (one copy serving both roles needs more
+    // registers than there are) ----
+    const uint32_t lds0 = lds_address(lds);
+    auto run = [&](auto role) {
+    constexpr bool LAGGING = decltype(role)::value;
+    BPlanes B;
+    v16f accF0 = v16f{0.0f}, accF1 = v16f{0.0f};  // the tile's two halves
+    int c_ord = 0, c_kb = 0, c_count = 0;
+    int pending = -1, pending_count = 0;  // item whose results wait to be stored
+    auto unpack_step = [&](int s) {
+        const int l = opaque_lane(), li = l & 31, lg = l >> 5;
+        const uint32_t wa = lds0 + (s & 1) * L::W_STAGE + (wave * 32 + li) * Q4_K_BYTES;
+        RawBlock R;
+        read_raw(R, wa, wa + 16 * lg);
+        wait_raw<0>(R);
+        unpack_block(R, lg, B);
+        __builtin_amdgcn_sched_barrier(0);  // keep the phases' registers apart
+    };
+    auto multiply_half = [&](uint32_t st, v16f &accF) {
+        const int lane = opaque_lane(), lg = lane >> 5;
+        TileOperands T;
+        TileScales S;
+        TileAcc X;
+        read_ops(T, st + lane * 16, st + L::A_BS + lane * 16);
+        tile_mfmas_as_they_land(T, B, X);
+        read_scales(S, st + L::A_DA + lg * 16);
+        wait_scales<0>(S);
+        tile_epilogue(X, S, B, accF);
+        // the epilogue must not sink below the next half's operand reads (its inputs would stay
+        // live through that half's MFMAs): an empty volatile statement that "modifies" the sums
+        // keeps its place among the volatile LDS reads
+        asm volatile("" : "+v"(accF));
+    };
+    auto multiply_step = [&](int s) {
+        const uint32_t st = lds0 + L::OFF_A + (s & 3) * L::A_STAGE;
+        if (c_kb == 0) {
+            int expert;
+            item_info(c_ord, expert, c_count);
+        }
+        multiply_half(st, accF0);
+        if (c_count > 32) multiply_half(st + L::A_HALF, accF1);
+        if (++c_kb == nb) {
+            pending = c_ord++;
+            pending_count = c_count;
+            c_kb = 0;
+        }
+    };
+    // a finished item's results are stored at the top of the next step, before that step's fetch: a
+    // store counts in vmcnt like a load, and "all but the newest n" must keep meaning "all but the
+    // fetch just issued"
+    auto store_item = [&](int ord) {  // a lane holds one weight row and 16 rows of the tile
+        int t, m, rg;
+        item_of(ord, t, m, rg);
+        const int count = pending_count;
+        const int l = opaque_lane(), li = l & 31, lg = l >> 5;
+        const int row = rg * (32 * L::RG) + wave * 32 + li;
+        int rows = g.rows;
+        asm volatile("" : "+s"(rows));  // opaque: keeps the 16 row offsets from being hoisted out of the loop and held
+        float *y = (m ? g.y[1] : g.y[0]) + (size_t)t * MOE_TILE * rows;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int tok = (r >> 2) * 8 + lg * 4 + (r & 3);
+            if (row < rows && tok < count) y[(uint32_t)(tok * rows + row)] = accF0[r];
+        }
+        accF0 = v16f{0.0f};
+        if (count > 32) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int tok = 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
+                if (row < rows && tok < count) y[(uint32_t)(tok * rows + row)] = accF1[r];
+            }
+            accF1 = v16f{0.0f};
+        }
+    };
+
+    for (int s = 0; s <= total_steps; s++) {
+        if (pending >= 0) {
+            store_item(pending);
+            pending = -1;
+        }
+        const bool more = s + 2 < total_steps;
+        if (more) fetch_acts();  // the stage was last read (by the lagging wavefronts) in step s-1
+        if (!LAGGING) {
+            if (s < total_steps) {
+                unpack_step(s);
+                if (more) fetch_weights();  // into the stage just unpacked
+                multiply_step(s);
+            }
+        } else {
+            if (s > 0) multiply_step(s - 1);
+            if (s < total_steps) {
+                unpack_step(s);
+                if (more) fetch_weights();
+            }
+        }
+        // step s+1 must have landed; the step requested above (younger) may stay in flight
+        if (more) wait_all_but_newest_step();
+        else wait_vm<0>();
+        lds_barrier();
+    }
+    if (pending >= 0) store_item(pending);
+    };
+    if (lagging) run(std::true_type{});
+    else run(std::false_type{});
 }
 
 // ------------------------------------------------------------------ launchers
@@ -441,48 +749,67 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
-template <int RG, int WT, int MT, int WS, bool GROUPED>
+template <int RG, int WT, int MT, int WS>
 static int launch_variant(const GemmArgs &g, unsigned grid, hipStream_t s) {
     constexpr size_t shmem = GemmLds<RG, WT, MT, WS>::BYTES;
     static_assert(shmem <= 160 * 1024, "LDS of a CU");
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (shmem > 65536 && !sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_mfma_kernel<RG, WT, MT, WS, GROUPED>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_mfma_kernel<RG, WT, MT, WS>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS, GROUPED>), dim3(grid), dim3(64 * RG * WT), shmem, s, g);
+    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS>), dim3(grid), dim3(64 * RG * WT), shmem, s, g);
     FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
     return FRK_OK;
 }
 
-size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) {
-    const size_t n = M * cols;
-    return round_up(n, 256) + round_up(n / QK_K * 4, 256) + round_up(n / 16 * 2, 256);
+// ---- the tiled activations ----
+static size_t tiled_records(size_t rows, size_t cols) { return (rows + 31) / 32 * (cols / QK_K); }
+size_t q8k_tiled_bytes(size_t rows, size_t cols) {
+    // the scales end with slack: a wavefront fetches 64 of them where 32 are used
+    return tiled_records(rows, cols) * (8192 + 1024 + 128) + 256;
+}
+Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols) {
+    const size_t rec = tiled_records(rows, cols);
+    Q8KTiled a;
+    a.q = (int8_t *)base;
+    a.bs = (_Float16 *)((char *)base + rec * 8192);
+    a.d = (float *)((char *)base + rec * (8192 + 1024));
+    return a;
+}
+int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTiled out, hipStream_t s) {
+    const size_t nb = cols / QK_K, n_rec = (rows + 31) / 32 * nb;
+    if (n_rec == 0) return FRK_OK;
+    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(256), 0, s, x, (int)rows, (int)nb,
+                       nullptr, nullptr, nullptr, out);
+    FRK_LAUNCH_CHECK("quantize_q8_k_tiled");
+    return FRK_OK;
+}
+int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, const int4 *tiles, const int *n_tiles,
+                                size_t max_rows, Q8KTiled out, hipStream_t s) {
+    const size_t nb = cols / QK_K, n_rec = max_rows / 32 * nb;
+    if (n_rec == 0) return FRK_OK;
+    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(256), 0, s, x, 0, (int)nb, gather,
+                       tiles, n_tiles, out);
+    FRK_LAUNCH_CHECK("quantize_q8_k_gather");
+    return FRK_OK;
 }
 
-int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
-    const size_t n = M * w->cols;
-    int8_t *q = (int8_t *)ws;
-    float *d = (float *)((char *)ws + round_up(n, 256));
-    _Float16 *bsf = (_Float16 *)((char *)d + round_up(n / QK_K * 4, 256));
-    int rc = launch_quantize_q8_k_gemm(x, n, q, d, bsf, s);
-    if (rc) return rc;
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
 
+int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     GemmArgs g;
+    g.a = q8k_tiled_carve(ws, M, w->cols);
+    int rc = launch_quantize_q8_k_tiled(x, M, w->cols, g.a, s);
+    if (rc) return rc;
     g.W = w->dev;
     g.row_stride = w->layout.row_stride;
     g.rows = (int)w->rows;
     g.nb = (int)(w->cols / QK_K);
     g.M = (int)M;
-    g.aq = q;
-    g.ad = d;
-    g.bsf = bsf;
     g.y = y;
-    g.tiles = nullptr;
-    g.n_tiles = nullptr;
-    g.gather = nullptr;
     // shape of a workgroup's tile: 256 rows x 64 tokens when that still gives every CU a workgroup,
     // else 128 rows x 64 or 32 tokens
     auto grid_for = [&](int rows_wg, int tm) {
@@ -491,41 +818,47 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
         return (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
     };
     const size_t wgs_big = ((w->rows + 255) / 256) * ((M + 63) / 64);
-    if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2, false>(g, grid_for(256, 64), s);
-    if (M > 32) return launch_variant<4, 2, 1, 4, false>(g, grid_for(128, 64), s);
-    return launch_variant<4, 1, 1, 2, false>(g, grid_for(128, 32), s);
+    if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2>(g, grid_for(256, 64), s);
+    if (M > 32) return launch_variant<4, 2, 1, 4>(g, grid_for(128, 64), s);
+    return launch_variant<4, 1, 1, 2>(g, grid_for(128, 32), s);
 }
 
-int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Float16 *bsf, hipStream_t s) {
-    const size_t nblk = n / QK_K;
-    if (nblk == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_k_gemm_kernel, dim3((unsigned)((nblk + 3) / 4)), dim3(256), 0, s, x, nblk, q, d,
-                       bsf);
-    FRK_LAUNCH_CHECK("quantize_q8_k_gemm");
-    return FRK_OK;
-}
-
-// Grouped GEMM over the experts stacked in `w` (expert e = rows [e*rows_e, (e+1)*rows_e)):
-// y[p][rows_e] for every output row p listed in the tiles (MOE_TILE rows per tile at most).
-int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
-                             const _Float16 *bsf, const int4 *tiles, const int *n_tiles, int max_tiles,
-                             const int *gather, float *y, hipStream_t s) {
-    GemmArgs g;
-    g.W = w->dev;
-    g.row_stride = w->layout.row_stride;
+int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
+                            const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,
+                            hipStream_t s) {
+    StreamArgs g;
+    g.W[0] = w0->dev;
+    g.W[1] = w1 ? w1->dev : w0->dev;
+    g.y[0] = y0;
+    g.y[1] = y1;
+    g.n_mat = w1 ? 2 : 1;
+    g.row_stride = w0->layout.row_stride;
     g.rows = (int)rows_e;
-    g.nb = (int)(w->cols / QK_K);
-    g.M = 0;
-    g.aq = aq;
-    g.ad = ad;
-    g.bsf = bsf;
-    g.y = y;
+    g.nb = (int)(w0->cols / QK_K);
+    g.a = a;
     g.tiles = tiles;
     g.n_tiles = n_tiles;
-    g.gather = gather;
-    g.row_tiles = (int)((rows_e + 127) / 128);
-    g.tok_tiles = max_tiles;
-        return launch_variant<4, 1, MOE_TILE / 32, 2, true>(g, (unsigned)(g.row_tiles * max_tiles), s);
+    g.row_tiles = (int)((rows_e + 255) / 256);
+    static int grid = 0;
+    if (grid == 0) {
+        int dev = 0, cus = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_stream_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)StreamLds::BYTES);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "gemm_q4_k_stream setup: %s", hipGetErrorString(e));
+        grid = cus < 8 ? 8 : cus / 8 * 8;  // one workgroup per CU, a multiple of the 8 XCDs
+    }
+    // more workgroups than CUs when a workgroup's share of the largest possible list would not fit
+    // its item table
+    const size_t most_items = ((size_t)max_tiles + 7) / 8 * g.n_mat * g.row_tiles;
+    const unsigned rounds = (unsigned)((most_items + (size_t)(grid / 8) * StreamLds::MAX_ITEMS - 1) /
+                                       ((size_t)(grid / 8) * StreamLds::MAX_ITEMS));
+    hipLaunchKernelGGL(gemm_q4_k_stream_kernel, dim3((unsigned)grid * (rounds ? rounds : 1)), dim3(64 * StreamLds::RG),
+                       StreamLds::BYTES, s, g);
+    FRK_LAUNCH_CHECK("gemm_q4_k_stream");
+    return FRK_OK;
 }
 
 }  // namespace frk

@@ -119,17 +119,37 @@ int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 bool fused_gemv_fits(const frk_weights *w);
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+// Q8_K activations in the form the matrix-core GEMMs stream: rows in tiles of 32 and, per
+// (tile, 256-wide block kb), one record that is exactly what a workgroup copies into LDS:
+//   q  [tile][kb][8 slices of 32 k][2 halves of 16 k][32 rows][16 bytes]
+//   bs [tile][kb][2 halves of 8 groups][32 rows][8]     the 16-wide sums as f16 (exact: |sum| <= 2032)
+//   d  [tile][kb][32 rows]
+// Rows past the last one of a partly used tile hold zeros.
+struct Q8KTiled {
+    int8_t *q;
+    _Float16 *bs;
+    float *d;
+};
+size_t q8k_tiled_bytes(size_t rows, size_t cols);
+Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols);
+// out row r = x[r] quantized, r < rows; the rest of the last tile becomes zeros
+int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTiled out, hipStream_t s);
+// out row r = x[gather[r]] quantized (zeros where gather[r] < 0), for the 32-row records that the
+// first *n_tiles tiles (MOE_TILE rows each, tiles[t].z of them in use) have rows in; max_rows bounds them
+int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, const int4 *tiles, const int *n_tiles,
+                                size_t max_rows, Q8KTiled out, hipStream_t s);
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
-// Q8_K quantization in the GEMM's form: the 16-wide sums as f16 (exact)
-int launch_quantize_q8_k_gemm(const float *x, size_t n, int8_t *q, float *d, _Float16 *bsf,
-                              hipStream_t s);
-// grouped (per-expert) GEMM: tiles {expert, first, count, 0} of at most MOE_TILE output rows each
-constexpr int MOE_TILE = 32;  // 64 was measured slower: fewer, longer workgroups
-int launch_gemm_q4_k_grouped(const frk_weights *w, size_t rows_e, const int8_t *aq, const float *ad,
-                             const _Float16 *bsf, const int4 *tiles, const int *n_tiles,
-                             int max_tiles, const int *gather, float *y, hipStream_t s);
+// grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
+// tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the
+// stacked matrices; *n_tiles <= max_tiles.  w1/y1 (nullable) is a second stacked matrix over the
+// same activations.  (64 rows: an expert's weights are then fetched and unpacked once for up to 64
+// of its rows; the second half of a tile costs nothing when it is not in use.)
+constexpr int MOE_TILE = 64;
+int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
+                            const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,
+                            hipStream_t s);
 // MoE expert FFN over stacked Q4_K experts; ws must hold moe_workspace_bytes(...)
 size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);
 int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,

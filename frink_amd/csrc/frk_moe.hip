@@ -87,106 +87,151 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *wave_tot, int &t
     return base + inc - v;
 }
 
-// Buckets the batch*k (token, slot) pairs by expert, tokens ascending inside a bucket.
-//   group_off[E+1]   bucket boundaries in the grouped order
-//   gather[pairs]    token of each grouped position
-//   pos_of[pairs]    grouped position of pair (tok*k + slot); -1 for an id outside [0, E)
-//   tiles / n_tiles  the buckets cut into runs of at most MOE_TILE positions for the grouped GEMM
-// One workgroup of 1024 threads; E <= 1024.  Pairs are taken 1024 at a time in pair order (which
-// is token-major); a pair's place in its bucket is the count of earlier pairs of that expert:
-// those of earlier rounds (run), of earlier wavefronts of this round (a prefix over the
-// per-wavefront counts) and of lower lanes of its own wavefront.
+// Buckets the batch*k (token, slot) pairs by expert, pairs ascending inside a bucket (which is tokens
+// ascending: pairs are token-major).  A bucket is cut into tiles of MOE_TILE rows; tile t is rows
+// [MOE_TILE*t, MOE_TILE*(t+1)) of the grouped order and belongs to one expert, so the order has gaps.
+// Tiles with more than 32 rows in use come first: they cost the grouped GEMM twice the arithmetic of
+// the others, and its workgroups, which deal the tile list out among themselves round-robin, then
+// get an even share of both kinds.
+//   group_off[E+1]   bucket boundaries in the order without the gaps
+//   gather[rows]     token of each row of the grouped order, -1 in a gap
+//   pos_of[pairs]    row of pair (tok*k + slot); -1 for an id outside [0, E)
+//   cpos_of[pairs]   the pair's place in the order without the gaps
+//   tiles / n_tiles  {expert, first row, rows in use, 0} per tile
+// One workgroup of 1024 threads; E <= 1024.  No atomic decides an order: a round takes `round`
+// pairs, marks pair j of expert e as bit j of row e of a bit matrix in LDS (an OR, so the result
+// does not depend on who comes first; the matrix is stored word-major so that the per-expert
+// pass below is free of bank conflicts), and a pair's rank in its bucket is the number of set bits
+// before its own in that row plus the bucket's count from earlier rounds.
+constexpr int GROUP_BIT_WORDS = 16384;  // 64 KB of bits: round = 524288 / E pairs (a multiple of 32)
+struct GroupLds {
+    uint32_t bits[GROUP_BIT_WORDS];
+    unsigned short before[GROUP_BIT_WORDS];  // set bits of the row in the words before this one
+    int cnt[1024], off_cmp[1024], run[1024];
+    int tile_big[1024], n_big[1024], tile_small[1024], seg_sum[1024];  // first heavy tile, their number, the light tile
+    int wave_tot[16];
+};
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restrict__ ids, int pairs, int k,
                                                          int n_experts, int *__restrict__ group_off,
                                                          int *__restrict__ gather, int *__restrict__ pos_of,
-                                                         int4 *__restrict__ tiles, int *__restrict__ n_tiles) {
-    __shared__ int cnt[1024];
-    __shared__ int off[1024];
-    __shared__ int run[1024];
-    __shared__ unsigned short wcnt[16][1024];
-    __shared__ int wave_tot[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    cnt[tid] = 0;
-    run[tid] = 0;
+                                                         int *__restrict__ cpos_of, int4 *__restrict__ tiles,
+                                                         int *__restrict__ n_tiles) {
+    extern __shared__ uint4 smem_group[];
+    GroupLds &L = *reinterpret_cast<GroupLds *>(smem_group);
+    const int tid = threadIdx.x;
+    L.cnt[tid] = 0;
+    L.run[tid] = 0;
     __syncthreads();
     for (int p = tid; p < pairs; p += 1024) {
         const int e = ids[p];
-        if (e >= 0 && e < n_experts) atomicAdd(&cnt[e], 1);
-        else pos_of[p] = -1;
+        if (e >= 0 && e < n_experts) atomicAdd(&L.cnt[e], 1);
+        else pos_of[p] = cpos_of[p] = -1;
     }
     __syncthreads();
     {
-        const int c = tid < n_experts ? cnt[tid] : 0;
+        const int c = tid < n_experts ? L.cnt[tid] : 0;
         const int nt = (c + MOE_TILE - 1) / MOE_TILE;
-        int total, total_tiles;
-        const int o = block_exclusive_scan(c, wave_tot, total);
-        const int t = block_exclusive_scan(nt, wave_tot, total_tiles);
-        off[tid] = o;
+        const int last = c - MOE_TILE * (nt - 1);  // rows in use of the last tile (nt > 0)
+        const int big = nt == 0 ? 0 : nt - 1 + (last > 32);
+        const int small = nt - big;  // 0 or 1
+        int total, total_big, total_small;
+        const int o = block_exclusive_scan(c, L.wave_tot, total);
+        const int tb = block_exclusive_scan(big, L.wave_tot, total_big);
+        const int ts = total_big + block_exclusive_scan(small, L.wave_tot, total_small);
+        L.off_cmp[tid] = o;
+        L.tile_big[tid] = tb;
+        L.n_big[tid] = big;
+        L.tile_small[tid] = ts;
         if (tid < n_experts) {
             group_off[tid] = o;
-            for (int i = 0; i < nt; i++) tiles[t + i] = make_int4(tid, o + MOE_TILE * i, min(MOE_TILE, c - MOE_TILE * i), 0);
+            for (int i = 0; i < nt; i++) {
+                const int t = i < big ? tb + i : ts;
+                const int used = min(MOE_TILE, c - MOE_TILE * i);
+                tiles[t] = make_int4(tid, MOE_TILE * t, used, 0);
+                for (int r = used; r < MOE_TILE; r++) gather[MOE_TILE * t + r] = -1;
+            }
         }
         if (tid == 0) {
             group_off[n_experts] = total;
-            *n_tiles = total_tiles;
+            *n_tiles = total_big + total_small;
         }
     }
-    for (int p0 = 0; p0 < pairs; p0 += 1024) {
-        for (int w = 0; w < 16; w++) wcnt[w][tid] = 0;
+    // words per row; `before` is 16 bits wide, so a round stays below 65536 pairs
+    const int rw = max(1, min(min(GROUP_BIT_WORDS / n_experts, 2047), (pairs + 31) / 32));
+    const int round = rw * 32;
+    for (int p0 = 0; p0 < pairs; p0 += round) {
+        for (int i = tid; i < rw * n_experts; i += 1024) L.bits[i] = 0;
         __syncthreads();
-        const int p = p0 + tid;
-        int e = p < pairs ? ids[p] : -1;
-        if (e >= n_experts) e = -1;
-        int rank = 0, same = 0;
-        for (int j = 0; j < 64; j++) {
-            const int ej = __shfl(e, j);
-            same += (ej == e);
-            rank += (ej == e && j < lane);
-        }
-        if (e >= 0 && rank == 0) wcnt[wave][e] = (unsigned short)same;
-        __syncthreads();
-        int before = 0;
-        if (e >= 0)
-            for (int w = 0; w < wave; w++) before += wcnt[w][e];
-        if (e >= 0) {
-            const int pos = off[e] + run[e] + before + rank;
-            gather[pos] = p / k;
-            pos_of[p] = pos;
+        for (int j = tid; j < round && p0 + j < pairs; j += 1024) {
+            const int e = ids[p0 + j];
+            if (e >= 0 && e < n_experts) atomicOr(&L.bits[(j >> 5) * n_experts + e], 1u << (j & 31));
         }
         __syncthreads();
         {
-            int tot = 0;
-            for (int w = 0; w < 16; w++) tot += wcnt[w][tid];
-            run[tid] += tot;
+            // prefix of the set bits along every row: the row's words are cut into `segs` runs, one
+            // thread each
+            const int segs = max(1, 1024 / n_experts), ws = (rw + segs - 1) / segs;
+            const int e = tid % n_experts, seg = tid / n_experts;
+            const int w0 = min(rw, seg * ws), w1 = min(rw, w0 + ws);
+            int sum = 0;
+            if (seg < segs)
+                for (int w = w0; w < w1; w++) sum += __popc(L.bits[w * n_experts + e]);
+            L.seg_sum[tid] = sum;
+            __syncthreads();
+            if (seg < segs) {
+                int run = 0;
+                for (int s2 = 0; s2 < seg; s2++) run += L.seg_sum[s2 * n_experts + e];
+                for (int w = w0; w < w1; w++) {
+                    L.before[w * n_experts + e] = (unsigned short)run;
+                    run += __popc(L.bits[w * n_experts + e]);
+                }
+                if (seg == segs - 1) L.cnt[e] = run;  // this round's pairs of the expert
+            }
         }
+        __syncthreads();
+        for (int j = tid; j < round && p0 + j < pairs; j += 1024) {
+            const int p = p0 + j;
+            const int e = ids[p];
+            if (e >= 0 && e < n_experts) {
+                const int w = (j >> 5) * n_experts + e;
+                const int rank = L.run[e] + L.before[w] + __popc(L.bits[w] & ((1u << (j & 31)) - 1u));
+                const int j = rank / MOE_TILE;
+                const int pos = MOE_TILE * (j < L.n_big[e] ? L.tile_big[e] + j : L.tile_small[e]) + rank % MOE_TILE;
+                gather[pos] = p / k;
+                pos_of[p] = pos;
+                cpos_of[p] = L.off_cmp[e] + rank;
+            }
+        }
+        __syncthreads();
+        if (tid < n_experts) L.run[tid] += L.cnt[tid];
         __syncthreads();
     }
 }
 
 // GluAct::Swiglu (crates/frink-core/src/matmul.rs:634-650): act = gate / (1 + exp(-gate)) * up, quantized
-// straight to Q8_K (with the GEMM's digit split) -- the down projection quantizes its own input
-// in the reference too (ffn_batch.rs:405-415).  One wavefront per 256 values.
+// straight to Q8_K in the tiled form -- the down projection quantizes its own input in the
+// reference too (ffn_batch.rs:405-415).  One workgroup per record (32 rows of the grouped order x
+// one block); rows in a gap become zeros, records without rows in use are skipped.
 __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__restrict__ gate,
-                                                              const float *__restrict__ up, size_t n_blocks,
-                                                              int8_t *__restrict__ q, float *__restrict__ d,
-                                                              _Float16 *__restrict__ bsf) {
-    const int lane = threadIdx.x & 63;
-    const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (b >= n_blocks) return;
-    const float4 gv = reinterpret_cast<const float4 *>(gate + b * QK_K)[lane];
-    const float4 uv = reinterpret_cast<const float4 *>(up + b * QK_K)[lane];
+                                                              const float *__restrict__ up, int nb,
+                                                              const int *__restrict__ gather,
+                                                              const int4 *__restrict__ tiles,
+                                                              const int *__restrict__ n_tiles, Q8KTiled out) {
+    __shared__ Q8KRecordLds L;
+    const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
+    const int t = t32 * 32 / MOE_TILE;
+    if (t >= *n_tiles || tiles[t].z <= t32 * 32 - t * MOE_TILE) return;
     // exp in double, rounded once to f32: the correctly rounded value, which is what a host libm's
-    // expf returns in all but a vanishing share of cases, so the quantizer below sees the same input
+    // expf returns in all but a vanishing share of cases, so the quantizer sees the same input
     auto silu = [](float x) { return __fdiv_rn(x, 1.0f + (float)exp(-(double)x)); };
-    const float4 v = make_float4(silu(gv.x) * uv.x, silu(gv.y) * uv.y, silu(gv.z) * uv.z, silu(gv.w) * uv.w);
-    float dd;
-    int bs;
-    const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
-    reinterpret_cast<uint32_t *>(q + b * QK_K)[lane] = packed;
-    if ((lane & 3) == 0) {
-        bsf[b * 16 + (lane >> 2)] = (_Float16)bs;
-    }
-    if (lane == 0) d[b] = dd;
+    quantize_q8k_record(out, (size_t)t32 * nb + kb, L, [&](int r) {
+        const int row = t32 * 32 + r;
+        if (gather[row] < 0) return make_float4(0.f, 0.f, 0.f, 0.f);
+        const size_t src = ((size_t)row * nb + kb) * QK_K;
+        const float4 gv = reinterpret_cast<const float4 *>(gate + src)[lane];
+        const float4 uv = reinterpret_cast<const float4 *>(up + src)[lane];
+        return make_float4(silu(gv.x) * uv.x, silu(gv.y) * uv.y, silu(gv.z) * uv.z, silu(gv.w) * uv.w);
+    });
 }
 
 // silu(gate) * up, elementwise (frink_core::matmul::swiglu, crates/frink-core/src/matmul.rs:634-650;
@@ -209,23 +254,16 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
                                                           float *__restrict__ out) {
     __shared__ int s_pos[64];
     __shared__ float s_w[64];
-    const int tok = blockIdx.x;
-    if (threadIdx.x == 0) {
-        int order[64];
-        for (int s = 0; s < k; s++) order[s] = s;
-        for (int a = 1; a < k; a++) {  // insertion sort by expert id
-            const int v = order[a];
-            int j = a - 1;
-            while (j >= 0 && ids[(size_t)tok * k + order[j]] > ids[(size_t)tok * k + v]) {
-                order[j + 1] = order[j];
-                j--;
-            }
-            order[j + 1] = v;
-        }
-        for (int s = 0; s < k; s++) {
-            s_pos[s] = pos_of[(size_t)tok * k + order[s]];
-            s_w[s] = weights[(size_t)tok * k + order[s]];
-        }
+    __shared__ int s_id[64];
+    const int tok = blockIdx.x, tid = threadIdx.x;
+    if (tid < k) s_id[tid] = ids[(size_t)tok * k + tid];
+    __syncthreads();
+    if (tid < k) {  // place in the ascending order of expert ids, equal ids in slot order
+        const int mine = s_id[tid];
+        int rank = 0;
+        for (int j = 0; j < k; j++) rank += (s_id[j] < mine) || (s_id[j] == mine && j < tid);
+        s_pos[rank] = pos_of[(size_t)tok * k + tid];
+        s_w[rank] = weights[(size_t)tok * k + tid];
     }
     __syncthreads();
     for (int h = threadIdx.x * 4; h < hidden; h += blockDim.x * 4) {
@@ -264,20 +302,21 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
 }
 
 struct MoeScratch {
-    int8_t *xq;  // Q8_K of the token rows; bsums as f16
-    _Float16 *xb;
-    float *xd;
-    float *gate_out, *up_out, *down_out;
-    int8_t *aq;  // Q8_K of silu(gate)*up
-    _Float16 *ab;
-    float *ad;
-    int *group_off, *gather, *pos_of, *n_tiles;
+    Q8KTiled xa;                          // the token rows in the grouped order, Q8_K
+    float *gate_out, *up_out, *down_out;  // rows in the grouped order (with its gaps)
+    Q8KTiled act;                         // Q8_K of silu(gate)*up
+    int *group_off, *gather, *pos_of, *cpos_of, *n_tiles;
     int4 *tiles;
 };
 
+// rows of the grouped order at most: every bucket may end in a partly used tile
+static size_t moe_max_rows(size_t pairs, int n_experts) {
+    return (pairs / MOE_TILE + (size_t)n_experts) * MOE_TILE;
+}
+
 // Carves the workspace; with base == nullptr the returned pointers are offsets and `end` the size.
 static MoeScratch moe_carve(void *base, size_t batch, int k, int n_experts, int hidden, int ffn, size_t *end) {
-    const size_t pairs = batch * (size_t)k;
+    const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts);
     char *p = (char *)base;
     auto take = [&](size_t bytes) {
         char *r = p;
@@ -285,20 +324,17 @@ static MoeScratch moe_carve(void *base, size_t batch, int k, int n_experts, int 
         return r;
     };
     MoeScratch m;
-    m.xq = (int8_t *)take(batch * hidden);
-    m.xb = (_Float16 *)take(batch * hidden / 16 * 2);
-    m.xd = (float *)take(batch * hidden / QK_K * 4);
-    m.gate_out = (float *)take(pairs * ffn * 4);
-    m.up_out = (float *)take(pairs * ffn * 4);
-    m.down_out = (float *)take(pairs * hidden * 4);
-    m.aq = (int8_t *)take(pairs * ffn);
-    m.ab = (_Float16 *)take(pairs * ffn / 16 * 2);
-    m.ad = (float *)take(pairs * ffn / QK_K * 4);
+    m.xa = q8k_tiled_carve(take(q8k_tiled_bytes(rows, hidden)), rows, hidden);
+    m.gate_out = (float *)take(rows * ffn * 4);
+    m.up_out = (float *)take(rows * ffn * 4);
+    m.down_out = (float *)take(rows * hidden * 4);
+    m.act = q8k_tiled_carve(take(q8k_tiled_bytes(rows, ffn)), rows, ffn);
     m.group_off = (int *)take((n_experts + 1) * 4);
-    m.gather = (int *)take(pairs * 4);
+    m.gather = (int *)take(rows * 4);
     m.pos_of = (int *)take(pairs * 4);
+    m.cpos_of = (int *)take(pairs * 4);
     m.n_tiles = (int *)take(256);
-    m.tiles = (int4 *)take((pairs / MOE_TILE + n_experts + 1) * 16);
+    m.tiles = (int4 *)take((rows / MOE_TILE + 1) * 16);
     if (end) *end = (size_t)(p - (char *)base);
     return m;
 }
@@ -309,51 +345,65 @@ size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int f
     return end;
 }
 
-// Test hook: copies out what the last launch_moe_ffn of this shape left in `ws` (null = skip).
-// Rows are in grouped order; pos_of[tok*k + slot] is the row of a (token, slot) pair.
+// Test hook: one workgroup per (token, slot) pair copies the pair's rows of the intermediates to
+// the pair's place in the grouped order without gaps (null outputs are skipped).
+__global__ __launch_bounds__(256) void moe_export_kernel(MoeScratch m, int ffn, float *__restrict__ gate_out,
+                                                         float *__restrict__ up_out, int8_t *__restrict__ act_q,
+                                                         float *__restrict__ act_d, int32_t *__restrict__ pos) {
+    const int pair = blockIdx.x, tid = threadIdx.x;
+    const int src = m.pos_of[pair], dst = m.cpos_of[pair];
+    if (pos && tid == 0) pos[pair] = dst;
+    if (src < 0) return;
+    const int nb = ffn / QK_K;
+    for (int i = tid; i < ffn; i += 256) {
+        if (gate_out) gate_out[(size_t)dst * ffn + i] = m.gate_out[(size_t)src * ffn + i];
+        if (up_out) up_out[(size_t)dst * ffn + i] = m.up_out[(size_t)src * ffn + i];
+        if (act_q) act_q[(size_t)dst * ffn + i] = m.act.q[q8k_tiled_index(nb, src, i / QK_K, i % QK_K)];
+    }
+    if (act_d)
+        for (int i = tid; i < nb; i += 256)
+            act_d[(size_t)dst * nb + i] = m.act.d[((size_t)(src >> 5) * nb + i) * 32 + (src & 31)];
+}
+
+// Copies out what the last launch_moe_ffn of this shape left in `ws`: row i of every output is the
+// i-th (token, slot) pair in the order experts ascending, tokens ascending; pos[tok*k + slot] = i.
 int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hidden, int ffn, float *gate_out,
                            float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of, hipStream_t s) {
     const MoeScratch m = moe_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
     const size_t pairs = batch * (size_t)k;
-    auto copy = [&](void *dst, const void *src, size_t bytes) -> int {
-        if (!dst) return FRK_OK;
-        hipError_t e = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
-        return e == hipSuccess ? FRK_OK : set_error(FRK_ERR_HIP, "hipMemcpyAsync: %s", hipGetErrorString(e));
-    };
-    int rc = copy(gate_out, m.gate_out, pairs * ffn * 4);
-    if (!rc) rc = copy(up_out, m.up_out, pairs * ffn * 4);
-    if (!rc) rc = copy(act_q, m.aq, pairs * ffn);
-    if (!rc) rc = copy(act_d, m.ad, pairs * ffn / QK_K * 4);
-    if (!rc) rc = copy(pos_of, m.pos_of, pairs * 4);
-    return rc;
+    hipLaunchKernelGGL(moe_export_kernel, dim3((unsigned)pairs), dim3(256), 0, s, m, ffn, gate_out, up_out, act_q, act_d,
+                       pos_of);
+    FRK_LAUNCH_CHECK("moe_export");
+    return FRK_OK;
 }
 
 int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
                    const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
                    void *ws, hipStream_t s) {
     const int hidden = (int)gate->cols, ffn = (int)down->cols;
-    const size_t pairs = batch * (size_t)k;
+    const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts);
     const MoeScratch m = moe_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
-    const int max_tiles = (int)(pairs / MOE_TILE + n_experts);
+    const int max_tiles = (int)(rows / MOE_TILE);
 
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), 0, s, ids, (int)pairs, k, n_experts, m.group_off, m.gather,
-                       m.pos_of, m.tiles, m.n_tiles);
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_group_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GroupLds));
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(moe_group): %s", hipGetErrorString(e));
+        sized = true;
+    }
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ids, (int)pairs, k, n_experts,
+                       m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles);
     FRK_LAUNCH_CHECK("moe_group");
-    int rc = launch_quantize_q8_k_gemm(x, batch * hidden, m.xq, m.xd, m.xb, s);
+    // the token rows, gathered into the grouped order and quantized; gate and up share them
+    int rc = launch_quantize_q8_k_gather(x, (size_t)hidden, m.gather, m.tiles, m.n_tiles, rows, m.xa, s);
     if (rc) return rc;
-    // gate and up read the same quantized token rows through the gather list
-    rc = launch_gemm_q4_k_grouped(gate, (size_t)ffn, m.xq, m.xd, m.xb, m.tiles, m.n_tiles, max_tiles, m.gather,
-                                  m.gate_out, s);
+    rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, m.tiles, m.n_tiles, max_tiles, m.gate_out, m.up_out, s);
     if (rc) return rc;
-    rc = launch_gemm_q4_k_grouped(up, (size_t)ffn, m.xq, m.xd, m.xb, m.tiles, m.n_tiles, max_tiles, m.gather,
-                                  m.up_out, s);
-    if (rc) return rc;
-    const size_t ablk = pairs * ffn / QK_K;
-    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)((ablk + 3) / 4)), dim3(256), 0, s, m.gate_out, m.up_out,
-                       ablk, m.aq, m.ad, m.ab);
+    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(256), 0, s, m.gate_out,
+                       m.up_out, ffn / QK_K, m.gather, m.tiles, m.n_tiles, m.act);
     FRK_LAUNCH_CHECK("swiglu_quantize");
-    rc = launch_gemm_q4_k_grouped(down, (size_t)hidden, m.aq, m.ad, m.ab, m.tiles, m.n_tiles, max_tiles, nullptr,
-                                  m.down_out, s);
+    rc = launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights, m.pos_of, k,
                        hidden, out);
