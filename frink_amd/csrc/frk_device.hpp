@@ -116,8 +116,11 @@ __device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, i
 
 // One record of the tiled Q8_K form (32 rows x one 256-wide block) by a workgroup of 256 threads:
 // wavefront w quantizes rows 8w..8w+7 (`load(r)` returns this lane's four values of row r, zeros for
-// a row that does not exist), the record is put together in LDS and leaves as three contiguous
-// copies -- quantizing straight into the tiled form would write it in 4-byte pieces.
+// a row that does not exist; all eight loads are in flight before the first row is quantized), the
+// record is put together in LDS and leaves as three contiguous copies -- quantizing straight into
+// the tiled form would write it in 4-byte pieces.  (Small workgroups: these kernels are bound by the
+// latency of their two dependent loads, and what hides it is how many workgroups a CU holds at once.)
+constexpr int Q8K_RECORD_THREADS = 256;
 struct Q8KRecordLds {
     uint32_t q[2048];
     _Float16 bs[512];

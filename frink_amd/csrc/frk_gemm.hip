@@ -42,18 +42,13 @@ typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 // Activation side: Q8_K quantization (quantize_activations_q8_k, crates/frink-quant/src/act_quant.rs:69-104)
 // into the tiled form, one workgroup per record (32 rows x one block).
 // Without `gather`, out row r = x[r] (rows from `rows` to the end of the last tile become zeros); with
-// it, out row r = x[gather[r]] (zeros where the entry is negative) for the records that the first
-// *n_tiles tiles {expert, first row, rows in use, 0} of MOE_TILE rows have rows in.
-__global__ __launch_bounds__(256) void quantize_q8_k_tiled_kernel(const float *__restrict__ x, int rows, int nb,
-                                                                  const int *__restrict__ gather,
-                                                                  const int4 *__restrict__ tiles,
-                                                                  const int *__restrict__ n_tiles, Q8KTiled out) {
+// it, out row r = x[gather[r]] (zeros where the entry is negative) for the records whose first entry
+// is not negative.
+__global__ __launch_bounds__(Q8K_RECORD_THREADS) void quantize_q8_k_tiled_kernel(const float *__restrict__ x, int rows, int nb,
+                                                                  const int *__restrict__ gather, Q8KTiled out) {
     __shared__ Q8KRecordLds L;
     const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
-    if (gather) {
-        const int t = t32 * 32 / MOE_TILE;
-        if (t >= *n_tiles || tiles[t].z <= t32 * 32 - t * MOE_TILE) return;
-    }
+    if (gather && gather[t32 * 32] < 0) return;
     quantize_q8k_record(out, (size_t)t32 * nb + kb, L, [&](int r) {
         const int row = t32 * 32 + r;
         const int src = gather ? gather[row] : (row < rows ? row : -1);
@@ -782,17 +777,17 @@ Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols) {
 int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTiled out, hipStream_t s) {
     const size_t nb = cols / QK_K, n_rec = (rows + 31) / 32 * nb;
     if (n_rec == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(256), 0, s, x, (int)rows, (int)nb,
-                       nullptr, nullptr, nullptr, out);
+    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(Q8K_RECORD_THREADS), 0, s, x, (int)rows, (int)nb,
+                       nullptr, out);
     FRK_LAUNCH_CHECK("quantize_q8_k_tiled");
     return FRK_OK;
 }
-int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, const int4 *tiles, const int *n_tiles,
-                                size_t max_rows, Q8KTiled out, hipStream_t s) {
+int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, size_t max_rows, Q8KTiled out,
+                                hipStream_t s) {
     const size_t nb = cols / QK_K, n_rec = max_rows / 32 * nb;
     if (n_rec == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(256), 0, s, x, 0, (int)nb, gather,
-                       tiles, n_tiles, out);
+    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(Q8K_RECORD_THREADS), 0, s, x, 0, (int)nb, gather,
+                       out);
     FRK_LAUNCH_CHECK("quantize_q8_k_gather");
     return FRK_OK;
 }

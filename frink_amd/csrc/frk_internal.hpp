@@ -134,10 +134,10 @@ size_t q8k_tiled_bytes(size_t rows, size_t cols);
 Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols);
 // out row r = x[r] quantized, r < rows; the rest of the last tile becomes zeros
 int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTiled out, hipStream_t s);
-// out row r = x[gather[r]] quantized (zeros where gather[r] < 0), for the 32-row records that the
-// first *n_tiles tiles (MOE_TILE rows each, tiles[t].z of them in use) have rows in; max_rows bounds them
-int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, const int4 *tiles, const int *n_tiles,
-                                size_t max_rows, Q8KTiled out, hipStream_t s);
+// out row r = x[gather[r]] quantized (zeros where gather[r] < 0), for the 32-row records of the first
+// max_rows rows whose first entry is not negative
+int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, size_t max_rows, Q8KTiled out,
+                                hipStream_t s);
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);

@@ -94,7 +94,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *wave_tot, int &t
 // the others, and its workgroups, which deal the tile list out among themselves round-robin, then
 // get an even share of both kinds.
 //   group_off[E+1]   bucket boundaries in the order without the gaps
-//   gather[rows]     token of each row of the grouped order, -1 in a gap
+//   gather[max_rows] token of each row of the grouped order, -1 in a gap and past the last tile
 //   pos_of[pairs]    row of pair (tok*k + slot); -1 for an id outside [0, E)
 //   cpos_of[pairs]   the pair's place in the order without the gaps
 //   tiles / n_tiles  {expert, first row, rows in use, 0} per tile
@@ -115,12 +115,13 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
                                                          int n_experts, int *__restrict__ group_off,
                                                          int *__restrict__ gather, int *__restrict__ pos_of,
                                                          int *__restrict__ cpos_of, int4 *__restrict__ tiles,
-                                                         int *__restrict__ n_tiles) {
+                                                         int *__restrict__ n_tiles, int max_rows) {
     extern __shared__ uint4 smem_group[];
     GroupLds &L = *reinterpret_cast<GroupLds *>(smem_group);
     const int tid = threadIdx.x;
     L.cnt[tid] = 0;
     L.run[tid] = 0;
+    for (int r = tid; r < max_rows; r += 1024) gather[r] = -1;
     __syncthreads();
     for (int p = tid; p < pairs; p += 1024) {
         const int e = ids[p];
@@ -148,7 +149,6 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
                 const int t = i < big ? tb + i : ts;
                 const int used = min(MOE_TILE, c - MOE_TILE * i);
                 tiles[t] = make_int4(tid, MOE_TILE * t, used, 0);
-                for (int r = used; r < MOE_TILE; r++) gather[MOE_TILE * t + r] = -1;
             }
         }
         if (tid == 0) {
@@ -211,16 +211,14 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
 // GluAct::Swiglu (crates/frink-core/src/matmul.rs:634-650): act = gate / (1 + exp(-gate)) * up, quantized
 // straight to Q8_K in the tiled form -- the down projection quantizes its own input in the
 // reference too (ffn_batch.rs:405-415).  One workgroup per record (32 rows of the grouped order x
-// one block); rows in a gap become zeros, records without rows in use are skipped.
-__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__restrict__ gate,
+// one block); rows in a gap become zeros, records without rows in use are skipped (a record's rows
+// in use come first, so its first row tells).
+__global__ __launch_bounds__(Q8K_RECORD_THREADS) void swiglu_quantize_kernel(const float *__restrict__ gate,
                                                               const float *__restrict__ up, int nb,
-                                                              const int *__restrict__ gather,
-                                                              const int4 *__restrict__ tiles,
-                                                              const int *__restrict__ n_tiles, Q8KTiled out) {
+                                                              const int *__restrict__ gather, Q8KTiled out) {
     __shared__ Q8KRecordLds L;
     const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
-    const int t = t32 * 32 / MOE_TILE;
-    if (t >= *n_tiles || tiles[t].z <= t32 * 32 - t * MOE_TILE) return;
+    if (gather[t32 * 32] < 0) return;  // rows in use come first in a tile
     // exp in double, rounded once to f32: the correctly rounded value, which is what a host libm's
     // expf returns in all but a vanishing share of cases, so the quantizer sees the same input
     auto silu = [](float x) { return __fdiv_rn(x, 1.0f + (float)exp(-(double)x)); };
@@ -393,15 +391,15 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
         sized = true;
     }
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ids, (int)pairs, k, n_experts,
-                       m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles);
+                       m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles, (int)rows);
     FRK_LAUNCH_CHECK("moe_group");
     // the token rows, gathered into the grouped order and quantized; gate and up share them
-    int rc = launch_quantize_q8_k_gather(x, (size_t)hidden, m.gather, m.tiles, m.n_tiles, rows, m.xa, s);
+    int rc = launch_quantize_q8_k_gather(x, (size_t)hidden, m.gather, rows, m.xa, s);
     if (rc) return rc;
     rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, m.tiles, m.n_tiles, max_tiles, m.gate_out, m.up_out, s);
     if (rc) return rc;
-    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(256), 0, s, m.gate_out,
-                       m.up_out, ffn / QK_K, m.gather, m.tiles, m.n_tiles, m.act);
+    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(Q8K_RECORD_THREADS), 0, s, m.gate_out,
+                       m.up_out, ffn / QK_K, m.gather, m.act);
     FRK_LAUNCH_CHECK("swiglu_quantize");
     rc = launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
     if (rc) return rc;
