@@ -56,6 +56,15 @@ __device__ __forceinline__ void load_to_lds4(const void *src, void *lds_chunk) {
 #endif
 }
 
+// the 32-bit LDS address of a pointer into shared memory, for LDS instructions written as inline assembly
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+#else
+    return 0;
+#endif
+}
+
 constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
 constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
 constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <- lane 7-i of its group of 8

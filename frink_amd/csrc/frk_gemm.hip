@@ -109,14 +109,6 @@ struct TileAcc {
 // that the waits are placed by hand.  LDS operations of a wavefront complete in order, so
 // "at most N outstanding" means everything but the N youngest reads has arrived; each wait names the
 // registers it releases so that their uses cannot be scheduled above it.
-__device__ __forceinline__ uint32_t lds_address(const void *p) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
-#else
-    return 0;
-#endif
-}
-
 #define FRK_DS_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:" #off : "=v"(dst) : "v"(addr))
 
 __device__ __forceinline__ void read_raw(RawBlock &R, uint32_t header, uint32_t quants) {

@@ -386,13 +386,13 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     clear_error();
     if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
     if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
-    if (w->kind == FRK_KIND_Q4_K && batch >= 16) {
+    if (w->kind == FRK_KIND_Q4_K && batch > 16) {
         void *ws = nullptr;
         int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
-    // thin batches of the K-quants: the weights are read once per 8 activation rows
+    // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q6_K) && batch >= 2 ? thin_gemm_max_batch(w) : 0;
     if (thin >= 2) {
         Q8KActs a;

@@ -27,7 +27,9 @@ __device__ __forceinline__ int granule_slot(int g, int units) {
 }
 
 // Stages NB Q8_K activation rows in LDS: quants | sums over GROUP*16 quants (as int) | block scales.
-// Rows past `batch` repeat the last one (their results are not stored).
+// Rows past `batch` repeat the last one (their results are not stored).  All of a thread's loads
+// are issued before the first LDS write: a load, its wait and its write in turn, once per row,
+// made the staging cost as much as the arithmetic.
 template <int NB, int SUMS_PER_BLOCK>
 __device__ __forceinline__ void stage_acts(uint4 *smem, int nb, int batch, const int8_t *aq, const float *ad,
                                            const int16_t *absums, int8_t *&sq, int *&sbs, float *&sd) {
@@ -35,29 +37,60 @@ __device__ __forceinline__ void stage_acts(uint4 *smem, int nb, int batch, const
     sbs = reinterpret_cast<int *>(sq + (size_t)NB * nb * 256);
     sd = reinterpret_cast<float *>(sbs + (size_t)NB * nb * SUMS_PER_BLOCK);
     constexpr int FOLD = 16 / SUMS_PER_BLOCK;  // bsums folded per stored sum
+    constexpr int CHUNK = 4;
+    const int tid = threadIdx.x;
+    const int row_g = nb * 16, row_s = nb * SUMS_PER_BLOCK;
+    for (int base = 0; base < NB * row_g; base += CHUNK * THIN_THREADS) {
+        uint4 v[CHUNK];
 #pragma unroll
-    for (int b = 0; b < NB; b++) {
-        const int src = min(b, batch - 1);
-        const uint4 *q4 = reinterpret_cast<const uint4 *>(aq + (size_t)src * nb * 256);
-        for (int i = threadIdx.x; i < nb * 16; i += THIN_THREADS)
-            smem[(size_t)b * nb * 16 + granule_slot<SUMS_PER_BLOCK == 16>(i, nb * 4)] = q4[i];
-        const int16_t *bs = absums + (size_t)src * nb * 16;
-        for (int i = threadIdx.x; i < nb * SUMS_PER_BLOCK; i += THIN_THREADS) {
-            int v = 0;
-#pragma unroll
-            for (int f = 0; f < FOLD; f++) v += (int)bs[FOLD * i + f];
-            sbs[(size_t)b * nb * SUMS_PER_BLOCK + i] = v;
+        for (int j = 0; j < CHUNK; j++) {  // (past the end: a valid address, the value is not written)
+            const int idx = min(base + j * THIN_THREADS + tid, NB * row_g - 1);
+            const int b = idx / row_g, i = idx - b * row_g;
+            v[j] = reinterpret_cast<const uint4 *>(aq + (size_t)min(b, batch - 1) * nb * 256)[i];
         }
-        for (int i = threadIdx.x; i < nb; i += THIN_THREADS) sd[(size_t)b * nb + i] = ad[(size_t)src * nb + i];
+#pragma unroll
+        for (int j = 0; j < CHUNK; j++) {
+            const int idx = base + j * THIN_THREADS + tid;
+            if (idx < NB * row_g) {
+                const int b = idx / row_g, i = idx - b * row_g;
+                smem[(size_t)b * row_g + granule_slot<SUMS_PER_BLOCK == 16>(i, nb * 4)] = v[j];
+            }
+        }
+    }
+    for (int base = 0; base < NB * row_s; base += CHUNK * THIN_THREADS) {
+        int v[CHUNK];
+#pragma unroll
+        for (int j = 0; j < CHUNK; j++) {
+            const int idx = base + j * THIN_THREADS + tid;
+            v[j] = 0;
+            {
+                const int idc = min(idx, NB * row_s - 1);
+                const int b = idc / row_s, i = idc - b * row_s;
+                const int16_t *bs = absums + (size_t)min(b, batch - 1) * nb * 16;
+#pragma unroll
+                for (int f = 0; f < FOLD; f++) v[j] += (int)bs[FOLD * i + f];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CHUNK; j++) {
+            const int idx = base + j * THIN_THREADS + tid;
+            if (idx < NB * row_s) sbs[idx] = v[j];
+        }
+    }
+    for (int idx = tid; idx < NB * nb; idx += THIN_THREADS) {
+        const int b = idx / nb, i = idx - b * nb;
+        sd[idx] = ad[(size_t)min(b, batch - 1) * nb + i];
     }
     __syncthreads();
 }
 
-// Both kernels: LPR lanes share R consecutive weight rows (a wavefront works on 64/LPR such row
-// groups at once) and walk them in units of 64 weights; a lane multiplies its unit of all R rows
-// against the same slice of each activation row, so that slice is read from LDS once per R rows.
+// Both kernels: LPR lanes share a weight row (a wavefront works on 64/LPR rows at once) and walk it
+// in units of 64 weights; a lane unpacks its unit once and multiplies it against the same slice of
+// each activation row.  A wavefront's (row, unit) steps form one sequence, and the weights of step
+// i+1 are requested before step i is computed: with one workgroup per CU there is nothing else to
+// hide the load latency behind.
 
-template <int LPR, int NB, int R>
+template <int LPR, int NB>
 __global__ __launch_bounds__(THIN_THREADS) void thin_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride,
                                                                  int rows, int nb, int batch,
                                                                  const int8_t *__restrict__ aq,
@@ -68,86 +101,107 @@ __global__ __launch_bounds__(THIN_THREADS) void thin_q4_k_kernel(const uint8_t *
     int8_t *sq;
     int *sbs;
     float *sd;
-    stage_acts<NB, 8>(smem, nb, batch, aq, ad, absums, sq, sbs, sd);
-
     constexpr int PARTS = 64 / LPR;
     const int lane = threadIdx.x & 63;
     const int part = lane / LPR, l = lane % LPR;
-    const int units = nb * 4;
-    const long n_waves = (long)gridDim.x * (THIN_THREADS / 64);
-    for (long g0 = ((long)blockIdx.x * (THIN_THREADS / 64) + (threadIdx.x >> 6)) * PARTS; g0 * R < rows;
-         g0 += n_waves * PARTS) {
-        const long r0 = (g0 + part) * R;  // this lane's first row of the group
-        float acc[R][NB];
+    const int units = nb * 4, upl = (units + LPR - 1) / LPR;  // steps per row
+    const int wave_id = blockIdx.x * (THIN_THREADS / 64) + (threadIdx.x >> 6), n_waves = gridDim.x * (THIN_THREADS / 64);
+    const int n_groups = (rows + PARTS - 1) / PARTS;
+    const int my_groups = wave_id < n_groups ? (n_groups - wave_id + n_waves - 1) / n_waves : 0;
+
+    struct Unit {
+        uint4 h, qa, qb;
+    };
+    // the unit of step (group gi, pass ui); past the end of a row or of the matrix it repeats a
+    // valid one, whose product is not used
+    auto load_unit = [&](int gi, int ui, Unit &U) {
+        const int row = min((wave_id + gi * n_waves) * PARTS + part, rows - 1);
+        const int u = min(l + ui * LPR, units - 1);
+        const uint4 *blk = reinterpret_cast<const uint4 *>(W + (size_t)row * row_stride + (size_t)(u >> 2) * Q4_K_BYTES);
+        U.h = blk[0];
+        U.qa = blk[1 + 2 * (u & 3)];
+        U.qb = blk[2 + 2 * (u & 3)];
+    };
+    Unit cur;
+    if (my_groups > 0) load_unit(0, 0, cur);  // in flight while the activations are staged
+    stage_acts<NB, 8>(smem, nb, batch, aq, ad, absums, sq, sbs, sd);
+
+    float acc[NB];
 #pragma unroll
-        for (int k = 0; k < R; k++)
-#pragma unroll
-            for (int b = 0; b < NB; b++) acc[k][b] = 0.0f;
-        if (r0 < rows) {
-            for (int u = l; u < units; u += LPR) {
-                const int blk_i = u >> 2, p = u & 3;
-                uint4 h[R], qa[R], qb[R];
-#pragma unroll
-                for (int k = 0; k < R; k++) {  // rows past the end repeat the last one; their results are dropped
-                    const uint4 *blk = reinterpret_cast<const uint4 *>(
-                        W + (size_t)min(r0 + k, (long)rows - 1) * row_stride + (size_t)blk_i * Q4_K_BYTES);
-                    h[k] = blk[0];
-                    qa[k] = blk[1 + 2 * p];
-                    qb[k] = blk[2 + 2 * p];
-                }
-                const int sh = (p & 1) * 16;
-#pragma unroll
-                for (int b = 0; b < NB; b++) {
-                    const uint4 *a = smem + (size_t)b * nb * 16 + u;  // pieces k at [k][unit]
-                    const uint4 a0 = a[0], a1 = a[units], a2 = a[2 * units], a3 = a[3 * units];
-                    const int *bs = sbs + ((size_t)b * nb + blk_i) * 8 + 2 * p;
-                    const int bs0 = bs[0], bs1 = bs[1];
-                    const float da = sd[(size_t)b * nb + blk_i];
-#pragma unroll
-                    for (int k = 0; k < R; k++) {
-                        // 6-bit scales and mins of sub-blocks 2p and 2p+1 (q4_k_scale_min, lib.rs:321-330)
-                        uint32_t scw, mw;
-                        if (p < 2) {
-                            scw = h[k].y & 0x3f3f3f3fu;
-                            mw = h[k].z & 0x3f3f3f3fu;
-                        } else {
-                            scw = (h[k].w & 0x0f0f0f0fu) | (((h[k].y >> 6) & 0x03030303u) << 4);
-                            mw = ((h[k].w >> 4) & 0x0f0f0f0fu) | (((h[k].z >> 6) & 0x03030303u) << 4);
-                        }
-                        const int sc1 = (scw >> sh) & 0xff, sc2 = (scw >> (sh + 8)) & 0xff;
-                        const int m1 = (mw >> sh) & 0xff, m2 = (mw >> (sh + 8)) & 0xff;
-                        int is1 = 0, is2 = 0;
-                        is1 = dot4(qa[k].x & 0x0f0f0f0fu, a0.x, is1);
-                        is1 = dot4(qa[k].y & 0x0f0f0f0fu, a0.y, is1);
-                        is1 = dot4(qa[k].z & 0x0f0f0f0fu, a0.z, is1);
-                        is1 = dot4(qa[k].w & 0x0f0f0f0fu, a0.w, is1);
-                        is1 = dot4(qb[k].x & 0x0f0f0f0fu, a1.x, is1);
-                        is1 = dot4(qb[k].y & 0x0f0f0f0fu, a1.y, is1);
-                        is1 = dot4(qb[k].z & 0x0f0f0f0fu, a1.z, is1);
-                        is1 = dot4(qb[k].w & 0x0f0f0f0fu, a1.w, is1);
-                        is2 = dot4((qa[k].x >> 4) & 0x0f0f0f0fu, a2.x, is2);
-                        is2 = dot4((qa[k].y >> 4) & 0x0f0f0f0fu, a2.y, is2);
-                        is2 = dot4((qa[k].z >> 4) & 0x0f0f0f0fu, a2.z, is2);
-                        is2 = dot4((qa[k].w >> 4) & 0x0f0f0f0fu, a2.w, is2);
-                        is2 = dot4((qb[k].x >> 4) & 0x0f0f0f0fu, a3.x, is2);
-                        is2 = dot4((qb[k].y >> 4) & 0x0f0f0f0fu, a3.y, is2);
-                        is2 = dot4((qb[k].z >> 4) & 0x0f0f0f0fu, a3.z, is2);
-                        is2 = dot4((qb[k].w >> 4) & 0x0f0f0f0fu, a3.w, is2);
-                        const int s1 = __mul24(sc1, is1) + __mul24(sc2, is2);
-                        const int s2 = __mul24(m1, bs0) + __mul24(m2, bs1);
-                        const float d = h2f(h[k].x & 0xffffu), dmin = h2f(h[k].x >> 16);
-                        acc[k][b] += (d * da) * (float)s1 - (dmin * da) * (float)s2;
-                    }
-                }
-            }
+    for (int b = 0; b < NB; b++) acc[b] = 0.0f;
+    int gi = 0, ui = 0;
+    for (int it = 0; it < my_groups * upl; it++) {
+        int gn = gi, un = ui + 1;
+        if (un == upl) {
+            un = 0;
+            gn++;
         }
-#pragma unroll
-        for (int k = 0; k < R; k++)
+        Unit nxt = cur;
+        if (gn < my_groups) load_unit(gn, un, nxt);
+
+        const int u = l + ui * LPR;
+        const int row = (wave_id + gi * n_waves) * PARTS + part;
+        if (u < units && row < rows) {
+            const int blk_i = u >> 2, p = u & 3;
+            // 6-bit scales and mins of sub-blocks 2p and 2p+1 (q4_k_scale_min, lib.rs:321-330)
+            uint32_t scw, mw;
+            if (p < 2) {
+                scw = cur.h.y & 0x3f3f3f3fu;
+                mw = cur.h.z & 0x3f3f3f3fu;
+            } else {
+                scw = (cur.h.w & 0x0f0f0f0fu) | (((cur.h.y >> 6) & 0x03030303u) << 4);
+                mw = ((cur.h.w >> 4) & 0x0f0f0f0fu) | (((cur.h.z >> 6) & 0x03030303u) << 4);
+            }
+            const int sh = (p & 1) * 16;
+            const int sc1 = (scw >> sh) & 0xff, sc2 = (scw >> (sh + 8)) & 0xff;
+            const int m1 = (mw >> sh) & 0xff, m2 = (mw >> (sh + 8)) & 0xff;
+            const float d = h2f(cur.h.x & 0xffffu), dmin = h2f(cur.h.x >> 16);
+            const uint32_t la[4] = {cur.qa.x & 0x0f0f0f0fu, cur.qa.y & 0x0f0f0f0fu, cur.qa.z & 0x0f0f0f0fu, cur.qa.w & 0x0f0f0f0fu};
+            const uint32_t lb[4] = {cur.qb.x & 0x0f0f0f0fu, cur.qb.y & 0x0f0f0f0fu, cur.qb.z & 0x0f0f0f0fu, cur.qb.w & 0x0f0f0f0fu};
+            const uint32_t ha[4] = {(cur.qa.x >> 4) & 0x0f0f0f0fu, (cur.qa.y >> 4) & 0x0f0f0f0fu, (cur.qa.z >> 4) & 0x0f0f0f0fu,
+                                    (cur.qa.w >> 4) & 0x0f0f0f0fu};
+            const uint32_t hb[4] = {(cur.qb.x >> 4) & 0x0f0f0f0fu, (cur.qb.y >> 4) & 0x0f0f0f0fu, (cur.qb.z >> 4) & 0x0f0f0f0fu,
+                                    (cur.qb.w >> 4) & 0x0f0f0f0fu};
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                const float v = part_sum<LPR>(acc[k][b]);
-                if (l == 0 && r0 + k < rows && b < batch) y[(size_t)b * rows + r0 + k] = v;
+                const uint4 *a = smem + (size_t)b * nb * 16 + u;  // pieces k at [k][unit]
+                const uint4 a0 = a[0], a1 = a[units], a2 = a[2 * units], a3 = a[3 * units];
+                const int *bs = sbs + ((size_t)b * nb + blk_i) * 8 + 2 * p;
+                const int bs0 = bs[0], bs1 = bs[1];
+                const float da = sd[(size_t)b * nb + blk_i];
+                int is1 = 0, is2 = 0;
+                is1 = dot4(la[0], a0.x, is1);
+                is1 = dot4(la[1], a0.y, is1);
+                is1 = dot4(la[2], a0.z, is1);
+                is1 = dot4(la[3], a0.w, is1);
+                is1 = dot4(lb[0], a1.x, is1);
+                is1 = dot4(lb[1], a1.y, is1);
+                is1 = dot4(lb[2], a1.z, is1);
+                is1 = dot4(lb[3], a1.w, is1);
+                is2 = dot4(ha[0], a2.x, is2);
+                is2 = dot4(ha[1], a2.y, is2);
+                is2 = dot4(ha[2], a2.z, is2);
+                is2 = dot4(ha[3], a2.w, is2);
+                is2 = dot4(hb[0], a3.x, is2);
+                is2 = dot4(hb[1], a3.y, is2);
+                is2 = dot4(hb[2], a3.z, is2);
+                is2 = dot4(hb[3], a3.w, is2);
+                const int s1 = __mul24(sc1, is1) + __mul24(sc2, is2);
+                const int s2 = __mul24(m1, bs0) + __mul24(m2, bs1);
+                acc[b] += (d * da) * (float)s1 - (dmin * da) * (float)s2;
             }
+        }
+        if (ui == upl - 1) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const float v = part_sum<LPR>(acc[b]);
+                if (l == 0 && row < rows && b < batch) y[(size_t)b * rows + row] = v;
+                acc[b] = 0.0f;
+            }
+        }
+        cur = nxt;
+        gi = gn;
+        ui = un;
     }
 }
 
@@ -251,6 +305,242 @@ __global__ __launch_bounds__(THIN_THREADS) void thin_q6_k_kernel(const uint8_t *
     }
 }
 
+// ------------------------------------------------------------------ thin GEMM on the matrix cores (Q4_K)
+//
+// Up to 16 activation rows against 16 weight rows per wavefront with v_mfma_i32_16x16x32_i8: one
+// MFMA is the integer dot of one 32-weight sub-block for all 16 x 16 (activation, weight row) pairs,
+// so the eight sub-block dots of a block cost eight short MFMAs instead of 16 dot4 per activation,
+// and the 6-bit scale multiplies each MFMA's four results (one v_mul_i32_i24 each: the weight row,
+// hence the scale, is the lane's own).  Integers are exactly dot_q4_k_q8's
+// (crates/frink-quant/src/lib.rs:822-869); the min term sum_j m_j * bsum_j is one f16 MFMA (both
+// factors and all sums exact); per block the float step is the batched GEMM's
+// acc += da * (d * S1 - dmin * S2).
+// Operand layout (checked on the device): lane l holds row/column l % 16 and the eight k
+// 8*(l/16) .. +7 (four for the K=16 f16 form); result register r is D[4*(l/16) + r][l % 16].  A =
+// activations, B = weights: a lane's four results are four activation rows of its own weight row.
+//
+// Data movement.  An MFMA lane wants 8 bytes of ITS row, so loading operands straight from memory
+// touches 16 rows per instruction, and the address unit then costs more than the data (measured:
+// 20 us, with or without the weights streaming).  Instead:
+//   * the quantized activations (acts x cols bytes, plus sums as f16 and scales) are staged in LDS
+//     once per workgroup with contiguous loads;
+//   * each wavefront streams the raw blocks of its 16 rows (16 x 144 bytes, contiguous per row) with
+//     ordinary 16-byte loads, TM_AHEAD blocks ahead in registers, and turns a block into the per-row
+//     view through a 2.25 KB LDS area of its own: a wavefront reads only what it wrote, in order,
+//     so after the staging there is no barrier in the loop.  (global_load_lds would save the
+//     registers, but it moved a KB per 60 to 100 clocks and CU here, a quarter of what the
+//     ordinary loads do.)
+// A workgroup is 8 wavefronts = RG groups of 16 rows x KS splits of the blocks (block kb goes to split
+// kb % KS); the splits add up through LDS in order at the end.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
+
+constexpr int TM_WAVES = 8;
+constexpr int TM_AHEAD = 4;                    // blocks of a wavefront in flight
+constexpr int TM_WBLOCK = 16 * Q4_K_BYTES;     // 2304: one block of 16 rows
+// LDS rows of the activations are padded so that the 16 rows a read touches fall in different banks
+__host__ __device__ constexpr int tm_q_stride(int cols) { return cols + 16; }
+__host__ __device__ constexpr int tm_bs_stride(int cols) { return cols / 8 + 8; }  // f16 sums, bytes
+__host__ __device__ inline size_t tm_lds_bytes(int acts, int cols) {
+    return (size_t)acts * (tm_q_stride(cols) + tm_bs_stride(cols)) + (size_t)(cols / QK_K) * 64 +
+           (size_t)TM_WAVES * TM_WBLOCK;
+}
+
+// (at most 4 wavefronts per SIMD: without the bound the compiler aims for 7, with 72 registers,
+// and keeps the ring in scratch memory)
+template <int RG, int ACTS>
+__global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2, 4))) void thin_mfma_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride,
+                                                                        int rows, int nb, int batch,
+                                                                        const int8_t *__restrict__ aq,
+                                                                        const float *__restrict__ ad,
+                                                                        const int16_t *__restrict__ absums,
+                                                                        float *__restrict__ y) {
+    constexpr int KS = TM_WAVES / RG;
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    const int cols = nb * QK_K;
+    const int q_stride = tm_q_stride(cols), bs_stride = tm_bs_stride(cols);
+    uint8_t *lds_q = lds;                                     // [ACTS][q_stride]
+    uint8_t *lds_bs = lds_q + (size_t)ACTS * q_stride;        // [ACTS][bs_stride] f16
+    float *lds_d = reinterpret_cast<float *>(lds_bs + (size_t)ACTS * bs_stride);  // [nb][16]
+    uint8_t *lds_w = reinterpret_cast<uint8_t *>(lds_d + (size_t)nb * 16);        // [wave][2304]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int rgrp = wave % RG, ksp = wave / RG;
+    const int row0 = (blockIdx.x * RG + rgrp) * 16;
+    const int my_blocks = nb > ksp ? (nb - ksp + KS - 1) / KS : 0;
+
+    // ---- this wavefront's weight stream: piece p = 64*c + lane of chunk c is row p/9, piece p%9 ----
+    const uint8_t *w_src[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        const int p = min(64 * c + lane, 143);
+        w_src[c] = W + (size_t)min(row0 + p / 9, rows - 1) * row_stride + (p % 9) * 16 + (size_t)ksp * Q4_K_BYTES;
+    }
+    struct Raw {
+        uint4 a, b, c;
+    };
+    auto fetch_block = [&](int i) {  // (past the last block: the last one again, never used)
+        const size_t off = (size_t)KS * max(min(i, my_blocks - 1), 0) * Q4_K_BYTES;
+        Raw R;
+        R.a = *reinterpret_cast<const uint4 *>(w_src[0] + off);
+        R.b = *reinterpret_cast<const uint4 *>(w_src[1] + off);
+        R.c = *reinterpret_cast<const uint4 *>(w_src[2] + off);  // lanes 16.. repeat piece 143
+        return R;
+    };
+    static_assert(TM_AHEAD == 4, "the ring is four named buffers");
+    // (named values handed around by value: an array, or structs passed by reference, end up in memory)
+    Raw R0, R1, R2, R3;
+
+    // ---- the activations, once per workgroup ----
+    // A wavefront's loads complete in order.  The staging loads (four per thread and array in a
+    // round; one round is the whole of it at the usual sizes) therefore go out first and the
+    // weight ring right behind them: the staging is over after one trip to the L2, and the first
+    // blocks are multiplied while the rest of the matrix is still streaming in.
+    {
+        constexpr int T = 64 * TM_WAVES;
+        const int row_g = cols / 16;   // 16-byte granules of quants per row
+        const int row_s4 = cols / 64;  // sums per row, four at a time
+        auto load_q = [&](int base, int u) {  // (past the end: a valid address, the value is not written)
+            const int idx = min(base + u * T + tid, ACTS * row_g - 1);
+            const int a = idx / row_g, i = idx - a * row_g;
+            return reinterpret_cast<const uint4 *>(aq + (size_t)min(a, batch - 1) * cols)[i];
+        };
+        auto store_q = [&](int base, int u, uint4 v) {
+            const int idx = base + u * T + tid;
+            if (idx < ACTS * row_g) {
+                const int a = idx / row_g, i = idx - a * row_g;
+                *reinterpret_cast<uint4 *>(lds_q + (size_t)a * q_stride + i * 16) = v;
+            }
+        };
+        auto load_s = [&](int base, int u) {
+            const int idx = min(base + u * T + tid, ACTS * row_s4 - 1);
+            const int a = idx / row_s4, i = idx - a * row_s4;
+            return reinterpret_cast<const uint2 *>(absums + (size_t)min(a, batch - 1) * row_s4 * 4)[i];
+        };
+        auto store_s = [&](int base, int u, uint2 v) {
+            const int idx = base + u * T + tid;
+            if (idx < ACTS * row_s4) {
+                const int a = idx / row_s4, i = idx - a * row_s4;
+                const v4h_t h = {(_Float16)(int)(int16_t)(v.x & 0xffff), (_Float16)(int)(int16_t)(v.x >> 16),
+                                 (_Float16)(int)(int16_t)(v.y & 0xffff), (_Float16)(int)(int16_t)(v.y >> 16)};
+                *reinterpret_cast<v4h_t *>(lds_bs + (size_t)a * bs_stride + i * 8) = h;
+            }
+        };
+        auto load_d = [&](int idx) {
+            idx = min(idx, nb * 16 - 1);
+            return ad[(size_t)min(idx & 15, batch - 1) * nb + (idx >> 4)];
+        };
+        const uint4 q0 = load_q(0, 0), q1 = load_q(0, 1), q2 = load_q(0, 2), q3 = load_q(0, 3);
+        const uint2 s0 = load_s(0, 0), s1 = load_s(0, 1), s2 = load_s(0, 2), s3 = load_s(0, 3);
+        const float d0 = load_d(tid);
+        R0 = fetch_block(0);
+        R1 = fetch_block(1);
+        R2 = fetch_block(2);
+        R3 = fetch_block(3);
+        store_q(0, 0, q0);
+        store_q(0, 1, q1);
+        store_q(0, 2, q2);
+        store_q(0, 3, q3);
+        store_s(0, 0, s0);
+        store_s(0, 1, s1);
+        store_s(0, 2, s2);
+        store_s(0, 3, s3);
+        if (tid < nb * 16) lds_d[tid] = d0;
+        // what one round does not cover (long rows): behind the ring, at the ring's pace
+        for (int base = 4 * T; base < ACTS * row_g; base += 4 * T)
+#pragma unroll
+            for (int u = 0; u < 4; u++) store_q(base, u, load_q(base, u));
+        for (int base = 4 * T; base < ACTS * row_s4; base += 4 * T)
+#pragma unroll
+            for (int u = 0; u < 4; u++) store_s(base, u, load_s(base, u));
+        for (int idx = T + tid; idx < nb * 16; idx += T) lds_d[idx] = load_d(idx);
+    }
+    __syncthreads();
+
+    // ---- the loop: no barrier; a wavefront writes its block to its own area and reads it back by row ----
+    const int act = min(j, ACTS - 1);  // rows past the staged ones repeat the last; their results are not stored
+    const uint8_t *a_q = lds_q + (size_t)act * q_stride + 8 * g;
+    const uint8_t *a_bs = lds_bs + (size_t)act * bs_stride + 8 * g;
+    const float *a_d = lds_d + 4 * g;
+    uint8_t *area = lds_w + (size_t)wave * TM_WBLOCK;
+    const uint8_t *a_w = area + j * Q4_K_BYTES;
+    auto as_long = [](uint2 v) { return (long)(((unsigned long)v.y << 32) | v.x); };
+    v4f_t acc = {0.f, 0.f, 0.f, 0.f};
+    auto multiply_block = [&](int i, Raw R) {  // returns the block that takes this one's place in the ring
+        const int kb = ksp + KS * i;
+        reinterpret_cast<uint4 *>(area)[lane] = R.a;
+        reinterpret_cast<uint4 *>(area)[64 + lane] = R.b;
+        if (lane < 16) reinterpret_cast<uint4 *>(area)[128 + lane] = R.c;
+        R = fetch_block(i + TM_AHEAD);  // the registers are free again
+        const uint4 h = *reinterpret_cast<const uint4 *>(a_w);
+        // 6-bit scales and mins (q4_k_scale_min, lib.rs:321-330): bytes of sc_lo/m_lo are sub-blocks
+        // 0..3, of sc_hi/m_hi sub-blocks 4..7
+        const uint32_t sc_lo = h.y & 0x3f3f3f3fu, m_lo = h.z & 0x3f3f3f3fu;
+        const uint32_t sc_hi = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
+        const uint32_t m_hi = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
+        v4i_t s1 = {0, 0, 0, 0};
+        const v4i_t zero = {0, 0, 0, 0};
+        const uint8_t *aq_k = a_q + (size_t)kb * QK_K;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {  // sub-blocks 2c (low nibbles) and 2c+1 (high)
+            const uint2 q = *reinterpret_cast<const uint2 *>(a_w + 16 + 32 * c + 8 * g);
+            const uint2 alo = *reinterpret_cast<const uint2 *>(aq_k + 64 * c);
+            const uint2 ahi = *reinterpret_cast<const uint2 *>(aq_k + 64 * c + 32);
+            const uint32_t scw = (c < 2 ? sc_lo : sc_hi) >> (16 * (c & 1));
+            const int sc0 = scw & 0xff, sc1 = (scw >> 8) & 0xff;
+            const uint2 lo = make_uint2(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu);
+            const uint2 hi = make_uint2((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu);
+            const v4i_t t0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(alo), as_long(lo), zero, 0, 0, 0);
+            const v4i_t t1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(ahi), as_long(hi), zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; r++) s1[r] += __mul24(sc0, t0[r]) + __mul24(sc1, t1[r]);
+        }
+        // mins of the 16-wide groups 4g..4g+3, i.e. of sub-blocks 2g and 2g+1, against the sums
+        const uint32_t mw = (g < 2 ? m_lo : m_hi) >> (16 * (g & 1));
+        const _Float16 m0 = (_Float16)(int)(mw & 0xff), m1 = (_Float16)(int)((mw >> 8) & 0xff);
+        const v4h_t mh = {m0, m0, m1, m1};
+        const v4h_t bh = *reinterpret_cast<const v4h_t *>(a_bs + (size_t)kb * 32);
+        const v4f_t da = *reinterpret_cast<const v4f_t *>(a_d + (size_t)kb * 16);
+        const v4f_t zf = {0.f, 0.f, 0.f, 0.f};
+        const v4f_t s2 = __builtin_amdgcn_mfma_f32_16x16x16f16(bh, mh, zf, 0, 0, 0);
+        const float d = h2f(h.x & 0xffffu), ndmin = -h2f(h.x >> 16);
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] = fmaf(da[r], fmaf(ndmin, s2[r], d * (float)s1[r]), acc[r]);
+        return R;
+    };
+    // the ring's buffers take turns by position, so no buffer is ever copied into another (a copy
+    // would wait for the loads in flight)
+    for (int i = 0; i < my_blocks; i += TM_AHEAD) {
+        R0 = multiply_block(i, R0);
+        if (i + 1 < my_blocks) R1 = multiply_block(i + 1, R1);
+        if (i + 2 < my_blocks) R2 = multiply_block(i + 2, R2);
+        if (i + 3 < my_blocks) R3 = multiply_block(i + 3, R3);
+    }
+
+    if (KS > 1) {  // add the splits up in order, through the (now idle) activation area
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(lds);
+        if (ksp > 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) red[(((ksp - 1) * RG + rgrp) * 4 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (ksp > 0) return;
+#pragma unroll
+        for (int k = 0; k < KS - 1; k++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += red[((k * RG + rgrp) * 4 + r) * 64 + lane];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int b = 4 * g + r;
+        if (b < batch && row0 + j < rows) y[(size_t)b * rows + row0 + j] = acc[r];
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -280,11 +570,11 @@ static int launch_thin_one(const frk_weights *w, int batch, Q8KActs a, float *y,
     if (q4) {
         static bool sized = false;
         if (shmem > 65536 && !sized) {
-            FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_q4_k_kernel<LPR, NB, R4>),
+            FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_q4_k_kernel<LPR, NB>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)THIN_LDS_LIMIT));
             sized = true;
         }
-        hipLaunchKernelGGL((thin_q4_k_kernel<LPR, NB, R4>), dim3(grid), dim3(THIN_THREADS), shmem, s, w->dev,
+        hipLaunchKernelGGL((thin_q4_k_kernel<LPR, NB>), dim3(grid), dim3(THIN_THREADS), shmem, s, w->dev,
                            w->layout.row_stride, (int)w->rows, nb, batch, a.q, a.d, a.bsums, y);
     } else {
         static bool sized = false;
@@ -308,8 +598,50 @@ static int launch_thin_nb(const frk_weights *w, int batch, Q8KActs a, float *y, 
     return launch_thin_one<16, NB>(w, batch, a, y, s);
 }
 
-// Largest number of activation rows one launch can take for this matrix (LDS), at most 8.
+constexpr size_t TM_LDS_LIMIT = 160 * 1024;
+
+template <int RG, int ACTS>
+static int launch_thin_mfma(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t shmem = tm_lds_bytes(ACTS, (int)w->cols);
+    static bool sized = false;
+    if (!sized) {
+        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_mfma_q4_k_kernel<RG, ACTS>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)TM_LDS_LIMIT));
+        sized = true;
+    }
+    const size_t groups = (w->rows + 15) / 16;
+    hipLaunchKernelGGL((thin_mfma_q4_k_kernel<RG, ACTS>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
+                       shmem, s, w->dev, w->layout.row_stride, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d,
+                       a.bsums, y);
+    FRK_LAUNCH_CHECK("thin mfma gemm");
+    return FRK_OK;
+}
+// rows of activations the matrix-core kernel can stage for this matrix (16, 8, 4 or 0)
+static int thin_mfma_acts(const frk_weights *w) {
+    for (int acts = 16; acts >= 4; acts /= 2)
+        if (tm_lds_bytes(acts, (int)w->cols) <= TM_LDS_LIMIT) return acts;
+    return 0;
+}
+template <int ACTS>
+static int launch_thin_mfma_rg(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    // row groups per workgroup: as many as still give (nearly) every CU a workgroup -- one per CU was
+    // measured faster than two, the activations being staged half as often; the rest of the 8
+    // wavefronts split the blocks, four or more each
+    const size_t groups = (w->rows + 15) / 16, nb = w->cols / QK_K;
+    int rg = 8;
+    while (rg > 1 && ((groups + rg - 1) / rg < 224 && (size_t)(TM_WAVES / rg) * 4 <= nb)) rg /= 2;
+    switch (rg) {
+        case 8: return launch_thin_mfma<8, ACTS>(w, batch, a, y, s);
+        case 4: return launch_thin_mfma<4, ACTS>(w, batch, a, y, s);
+        case 2: return launch_thin_mfma<2, ACTS>(w, batch, a, y, s);
+        default: return launch_thin_mfma<1, ACTS>(w, batch, a, y, s);
+    }
+}
+
+// Largest number of activation rows one launch can take for this matrix: up to 16 on the
+// matrix-core path (Q4_K), else what fits LDS, at most 8.
 int thin_gemm_max_batch(const frk_weights *w) {
+    if (w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0) return thin_mfma_acts(w);
     const size_t per_row = (w->cols / QK_K) * (256 + (w->kind == FRK_KIND_Q4_K ? 8 : 16) * 4 + 4);
     for (int nbatch = 8; nbatch >= 2; nbatch /= 2)
         if (per_row * nbatch <= THIN_LDS_LIMIT) return nbatch;
@@ -318,9 +650,16 @@ int thin_gemm_max_batch(const frk_weights *w) {
 
 // y[batch][rows] for 1 <= batch <= thin_gemm_max_batch(w) quantized activation rows (K-quants).
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    if (w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0 && batch > 2) {  // (two rows: the dot4 kernel is still ahead)
+        // the fewest staged rows that hold the batch
+        if (batch <= 4) return launch_thin_mfma_rg<4>(w, batch, a, y, s);
+        if (batch <= 8) return launch_thin_mfma_rg<8>(w, batch, a, y, s);
+        return launch_thin_mfma_rg<16>(w, batch, a, y, s);
+    }
     if (batch > 4) return launch_thin_nb<8>(w, batch, a, y, s);
     if (batch > 2) return launch_thin_nb<4>(w, batch, a, y, s);
     return launch_thin_nb<2>(w, batch, a, y, s);
 }
 
 }  // namespace frk
+
