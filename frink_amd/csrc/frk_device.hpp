@@ -123,29 +123,29 @@ __device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, i
            ((uint32_t)(q3 & 0xff) << 24);
 }
 
-// One record of the tiled Q8_K form (32 rows x one 256-wide block) by a workgroup of 256 threads:
-// wavefront w quantizes rows 8w..8w+7 (`load(r)` returns this lane's four values of row r, zeros for
-// a row that does not exist; all eight loads are in flight before the first row is quantized), the
-// record is put together in LDS and leaves as three contiguous copies -- quantizing straight into
-// the tiled form would write it in 4-byte pieces.  (Small workgroups: these kernels are bound by the
-// latency of their two dependent loads, and what hides it is how many workgroups a CU holds at once.)
-constexpr int Q8K_RECORD_THREADS = 256;
+// One record of the tiled Q8_K form (32 rows x one 256-wide block) by a workgroup of WAVES wavefronts
+// (4 or 16): wavefront w quantizes rows 32/WAVES * w .. (`load(r)` returns this lane's four values of
+// row r, zeros for a row that does not exist; all of a wavefront's loads are in flight before its
+// first row is quantized), the record is put together in LDS and leaves as three contiguous copies
+// -- quantizing straight into the tiled form would write it in 4-byte pieces.  These kernels are
+// bound by latency: few records want many wavefronts each, many records small workgroups.
 struct Q8KRecordLds {
     uint32_t q[2048];
     _Float16 bs[512];
     float d[32];
 };
-template <class Load>
+template <int WAVES, class Load>
 __device__ __forceinline__ void quantize_q8k_record(const Q8KTiled &a, size_t rec, Q8KRecordLds &L, Load load) {
+    constexpr int RPW = 32 / WAVES;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    float4 v[8];
+    float4 v[RPW];
 #pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = load(wave * 8 + i);
+    for (int i = 0; i < RPW; i++) v[i] = load(wave * RPW + i);
     // the lane's four values are k = 4*lane..: 32-wide slice lane/8, 16-byte half (lane/4)%2 of it
     const int ks = lane >> 3, half = (lane >> 2) & 1, g = lane >> 2;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int r = wave * 8 + i;
+    for (int i = 0; i < RPW; i++) {
+        const int r = wave * RPW + i;
         float dd;
         int bs;
         const uint32_t packed = quantize_q8_k_lane(v[i], dd, bs);
@@ -156,8 +156,7 @@ __device__ __forceinline__ void quantize_q8k_record(const Q8KTiled &a, size_t re
     __syncthreads();
     uint4 *dq = reinterpret_cast<uint4 *>(a.q + rec * 8192);
     const uint4 *sq = reinterpret_cast<const uint4 *>(L.q);
-    dq[tid] = sq[tid];
-    dq[tid + 256] = sq[tid + 256];
+    for (int i = tid; i < 512; i += 64 * WAVES) dq[i] = sq[i];
     if (tid < 64) reinterpret_cast<uint4 *>(a.bs + rec * 512)[tid] = reinterpret_cast<const uint4 *>(L.bs)[tid];
     if (tid < 32) a.d[rec * 32 + tid] = L.d[tid];
 }

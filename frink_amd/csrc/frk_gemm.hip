@@ -44,12 +44,13 @@ typedef unsigned short us2 __attribute__((ext_vector_type(2)));
 // Without `gather`, out row r = x[r] (rows from `rows` to the end of the last tile become zeros); with
 // it, out row r = x[gather[r]] (zeros where the entry is negative) for the records whose first entry
 // is not negative.
-__global__ __launch_bounds__(Q8K_RECORD_THREADS) void quantize_q8_k_tiled_kernel(const float *__restrict__ x, int rows, int nb,
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void quantize_q8_k_tiled_kernel(const float *__restrict__ x, int rows, int nb,
                                                                   const int *__restrict__ gather, Q8KTiled out) {
     __shared__ Q8KRecordLds L;
     const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
     if (gather && gather[t32 * 32] < 0) return;
-    quantize_q8k_record(out, (size_t)t32 * nb + kb, L, [&](int r) {
+    quantize_q8k_record<WAVES>(out, (size_t)t32 * nb + kb, L, [&](int r) {
         const int row = t32 * 32 + r;
         const int src = gather ? gather[row] : (row < rows ? row : -1);
         if (src < 0) return make_float4(0.f, 0.f, 0.f, 0.f);
@@ -766,22 +767,26 @@ Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols) {
     a.d = (float *)((char *)base + rec * (8192 + 1024));
     return a;
 }
+template <int WAVES>
+static int launch_quantize_records(const float *x, size_t rows, size_t nb, const int *gather, size_t n_rec, Q8KTiled out,
+                                   hipStream_t s) {
+    hipLaunchKernelGGL((quantize_q8_k_tiled_kernel<WAVES>), dim3((unsigned)n_rec), dim3(64 * WAVES), 0, s, x, (int)rows,
+                       (int)nb, gather, out);
+    FRK_LAUNCH_CHECK("quantize_q8_k_tiled");
+    return FRK_OK;
+}
 int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTiled out, hipStream_t s) {
     const size_t nb = cols / QK_K, n_rec = (rows + 31) / 32 * nb;
     if (n_rec == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(Q8K_RECORD_THREADS), 0, s, x, (int)rows, (int)nb,
-                       nullptr, out);
-    FRK_LAUNCH_CHECK("quantize_q8_k_tiled");
-    return FRK_OK;
+    return n_rec <= 1024 ? launch_quantize_records<16>(x, rows, nb, nullptr, n_rec, out, s)
+                         : launch_quantize_records<4>(x, rows, nb, nullptr, n_rec, out, s);
 }
 int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, size_t max_rows, Q8KTiled out,
                                 hipStream_t s) {
     const size_t nb = cols / QK_K, n_rec = max_rows / 32 * nb;
     if (n_rec == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_k_tiled_kernel, dim3((unsigned)n_rec), dim3(Q8K_RECORD_THREADS), 0, s, x, 0, (int)nb, gather,
-                       out);
-    FRK_LAUNCH_CHECK("quantize_q8_k_gather");
-    return FRK_OK;
+    return n_rec <= 1024 ? launch_quantize_records<16>(x, 0, nb, gather, n_rec, out, s)
+                         : launch_quantize_records<4>(x, 0, nb, gather, n_rec, out, s);
 }
 
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }

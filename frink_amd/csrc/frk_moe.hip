@@ -213,7 +213,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
 // reference too (ffn_batch.rs:405-415).  One workgroup per record (32 rows of the grouped order x
 // one block); rows in a gap become zeros, records without rows in use are skipped (a record's rows
 // in use come first, so its first row tells).
-__global__ __launch_bounds__(Q8K_RECORD_THREADS) void swiglu_quantize_kernel(const float *__restrict__ gate,
+__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__restrict__ gate,
                                                               const float *__restrict__ up, int nb,
                                                               const int *__restrict__ gather, Q8KTiled out) {
     __shared__ Q8KRecordLds L;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(Q8K_RECORD_THREADS) void swiglu_quantize_kernel(con
     // exp in double, rounded once to f32: the correctly rounded value, which is what a host libm's
     // expf returns in all but a vanishing share of cases, so the quantizer sees the same input
     auto silu = [](float x) { return __fdiv_rn(x, 1.0f + (float)exp(-(double)x)); };
-    quantize_q8k_record(out, (size_t)t32 * nb + kb, L, [&](int r) {
+    quantize_q8k_record<4>(out, (size_t)t32 * nb + kb, L, [&](int r) {
         const int row = t32 * 32 + r;
         if (gather[row] < 0) return make_float4(0.f, 0.f, 0.f, 0.f);
         const size_t src = ((size_t)row * nb + kb) * QK_K;
@@ -398,7 +398,7 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     if (rc) return rc;
     rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, m.tiles, m.n_tiles, max_tiles, m.gate_out, m.up_out, s);
     if (rc) return rc;
-    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(Q8K_RECORD_THREADS), 0, s, m.gate_out,
+    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(256), 0, s, m.gate_out,
                        m.up_out, ffn / QK_K, m.gather, m.act);
     FRK_LAUNCH_CHECK("swiglu_quantize");
     rc = launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
