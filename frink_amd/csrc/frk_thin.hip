@@ -541,6 +541,197 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     }
 }
 
+// ------------------------------------------------------------------ thin GEMM on the matrix cores (Q6_K)
+//
+// Same plan as the Q4_K kernel above, for up to 8 activation rows.  Q6_K scales sixteen weights at
+// a time, and a K=32 MFMA would add up two such groups.  So the 16 rows of the MFMA's activation
+// operand hold the (at most 8) activation rows twice: rows 0..7 with only the first sixteen k of
+// every 32 (the rest zero), rows 8..15 with only the second sixteen.  One MFMA then returns, for
+// each (activation, weight row), the two 16-wide dots side by side -- in the lanes of k-groups 0..1
+// and 2..3, which multiply them by their own group's int8 scale; the two halves of a result meet
+// once, at the end.  The 6-bit codes go in as signed bytes q - 32 (one add and one xor per four
+// codes), so there is no "-32 * sum of the activations" term to carry: the integers are
+// dot_q6_k_q8's (crates/frink-quant/src/lib.rs:1069-1110), split in two partial sums per block.
+// Weights are the resident planar form (ql | qh | sc | d per row); in LDS a row of a block is
+// [ql 128 | qh 64 | sc 16 | d 2], 240 bytes apart so that the 16 rows of a read fall in
+// different banks.
+constexpr int T6_ROW = 240;
+constexpr int T6_WBLOCK = 16 * T6_ROW;  // 3840
+__host__ __device__ inline size_t t6_lds_bytes(int acts, int cols) {
+    return (size_t)acts * tm_q_stride(cols) + (size_t)(cols / QK_K) * 32 + (size_t)TM_WAVES * T6_WBLOCK;
+}
+
+template <int RG, int ACTS>
+__global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2, 4))) void thin_mfma_q6_k_kernel(
+    const uint8_t *__restrict__ W, Layout lay, int rows, int nb, int batch, const int8_t *__restrict__ aq,
+    const float *__restrict__ ad, float *__restrict__ y) {
+    constexpr int KS = TM_WAVES / RG;
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    const int cols = nb * QK_K;
+    const int q_stride = tm_q_stride(cols);
+    uint8_t *lds_q = lds;                                                         // [ACTS][q_stride]
+    float *lds_d = reinterpret_cast<float *>(lds_q + (size_t)ACTS * q_stride);    // [nb][8]
+    uint8_t *lds_w = reinterpret_cast<uint8_t *>(lds_d + (size_t)nb * 8);         // [wave][3840]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int rgrp = wave % RG, ksp = wave / RG;
+    const int row0 = (blockIdx.x * RG + rgrp) * 16;
+    const int my_blocks = nb > ksp ? (nb - ksp + KS - 1) / KS : 0;
+
+    // ---- this wavefront's weight stream: the four planes of its 16 rows, 16-byte pieces ----
+    // ql: piece p = 64*c + lane (c = 0, 1) is row p/8, piece p%8; qh: piece lane is row lane/4, piece
+    // lane%4; sc: lanes 0..15, one piece per row; d: lanes 0..15, two bytes per row
+    auto row_ptr = [&](int r) { return W + (size_t)min(row0 + r, rows - 1) * lay.row_stride; };
+    const uint8_t *src_ql0 = row_ptr(lane >> 3) + (lane & 7) * 16 + (size_t)ksp * 128;
+    const uint8_t *src_ql1 = row_ptr(8 + (lane >> 3)) + (lane & 7) * 16 + (size_t)ksp * 128;
+    const uint8_t *src_qh = row_ptr(lane >> 2) + lay.off_a + (lane & 3) * 16 + (size_t)ksp * 64;
+    const uint8_t *src_sc = row_ptr(lane & 15) + lay.off_b + (size_t)ksp * 16;
+    const uint8_t *src_d = row_ptr(lane & 15) + lay.off_c + (size_t)ksp * 2;
+    struct Raw {
+        uint4 ql0, ql1, qh, sc;
+        uint32_t d;
+    };
+    auto fetch_block = [&](int i) {  // (past the last block: the last one again, never used)
+        const size_t k = (size_t)KS * max(min(i, my_blocks - 1), 0);
+        Raw R;
+        R.ql0 = *reinterpret_cast<const uint4 *>(src_ql0 + k * 128);
+        R.ql1 = *reinterpret_cast<const uint4 *>(src_ql1 + k * 128);
+        R.qh = *reinterpret_cast<const uint4 *>(src_qh + k * 64);
+        R.sc = *reinterpret_cast<const uint4 *>(src_sc + k * 16);  // lanes 16.. repeat rows 0..15
+        R.d = *reinterpret_cast<const uint16_t *>(src_d + k * 2);
+        return R;
+    };
+    static_assert(TM_AHEAD == 4, "the ring is four named buffers");
+    Raw R0, R1, R2, R3;
+
+    // ---- the activations, once per workgroup: staging loads first, the weight ring behind them ----
+    {
+        constexpr int T = 64 * TM_WAVES;
+        const int row_g = cols / 16;  // 16-byte granules of quants per row
+        auto load_q = [&](int base, int u) {  // (past the end: a valid address, the value is not written)
+            const int idx = min(base + u * T + tid, ACTS * row_g - 1);
+            const int a = idx / row_g, i = idx - a * row_g;
+            return reinterpret_cast<const uint4 *>(aq + (size_t)min(a, batch - 1) * cols)[i];
+        };
+        auto store_q = [&](int base, int u, uint4 v) {
+            const int idx = base + u * T + tid;
+            if (idx < ACTS * row_g) {
+                const int a = idx / row_g, i = idx - a * row_g;
+                *reinterpret_cast<uint4 *>(lds_q + (size_t)a * q_stride + i * 16) = v;
+            }
+        };
+        auto load_d = [&](int idx) {
+            idx = min(idx, nb * 8 - 1);
+            return ad[(size_t)min(idx & 7, batch - 1) * nb + (idx >> 3)];
+        };
+        const uint4 q0 = load_q(0, 0), q1 = load_q(0, 1), q2 = load_q(0, 2), q3 = load_q(0, 3);
+        const float d0 = load_d(tid);
+        R0 = fetch_block(0);
+        R1 = fetch_block(1);
+        R2 = fetch_block(2);
+        R3 = fetch_block(3);
+        store_q(0, 0, q0);
+        store_q(0, 1, q1);
+        store_q(0, 2, q2);
+        store_q(0, 3, q3);
+        if (tid < nb * 8) lds_d[tid] = d0;
+        // what one round does not cover (long rows): behind the ring, at the ring's pace
+        for (int base = 4 * T; base < ACTS * row_g; base += 4 * T)
+#pragma unroll
+            for (int u = 0; u < 4; u++) store_q(base, u, load_q(base, u));
+        for (int idx = T + tid; idx < nb * 8; idx += T) lds_d[idx] = load_d(idx);
+    }
+    __syncthreads();
+
+    // ---- the loop ----
+    // activation operand row j: activation j % 8, and only the k-groups of its half are real
+    const bool real = (j < 8) == (g < 2);
+    const uint8_t *a_q = lds_q + (size_t)min(j & 7, ACTS - 1) * q_stride + 8 * g;
+    const float *a_d = lds_d + 4 * (g & 1);
+    uint8_t *area = lds_w + (size_t)wave * T6_WBLOCK;
+    const uint8_t *a_w = area + j * T6_ROW;
+    auto as_long = [](uint2 v) { return (long)(((unsigned long)v.y << 32) | v.x); };
+    v4f_t acc = {0.f, 0.f, 0.f, 0.f};
+    auto multiply_block = [&](int i, Raw R) {  // returns the block that takes this one's place in the ring
+        const int kb = ksp + KS * i;
+        *reinterpret_cast<uint4 *>(area + (lane >> 3) * T6_ROW + (lane & 7) * 16) = R.ql0;
+        *reinterpret_cast<uint4 *>(area + (8 + (lane >> 3)) * T6_ROW + (lane & 7) * 16) = R.ql1;
+        *reinterpret_cast<uint4 *>(area + (lane >> 2) * T6_ROW + 128 + (lane & 3) * 16) = R.qh;
+        if (lane < 16) {
+            *reinterpret_cast<uint4 *>(area + lane * T6_ROW + 192) = R.sc;
+            *reinterpret_cast<uint32_t *>(area + lane * T6_ROW + 208) = R.d;
+        }
+        R = fetch_block(i + TM_AHEAD);  // the registers are free again
+        const uint4 scv = *reinterpret_cast<const uint4 *>(a_w + 192);
+        const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+        const float d = h2f(*reinterpret_cast<const uint32_t *>(a_w + 208) & 0xffffu);
+        const v4i_t zero = {0, 0, 0, 0};
+        v4i_t isum = {0, 0, 0, 0};
+        const uint8_t *aq_k = a_q + (size_t)kb * QK_K;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint2 qla = *reinterpret_cast<const uint2 *>(a_w + h * 64 + 8 * g);
+            const uint2 qlb = *reinterpret_cast<const uint2 *>(a_w + h * 64 + 32 + 8 * g);
+            const uint2 qh = *reinterpret_cast<const uint2 *>(a_w + 128 + h * 32 + 8 * g);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {  // weights h*128 + 32*v + l, l = 8g .. 8g+7
+                const uint2 ql = (v & 1) ? qlb : qla;
+                auto code = [&](uint32_t lo, uint32_t hi) {  // four 6-bit codes, as signed bytes q - 32
+                    const uint32_t nib = (v >= 2 ? lo >> 4 : lo) & 0x0f0f0f0fu;
+                    const uint32_t top = ((hi >> (2 * v)) & 0x03030303u) << 4;
+                    return ((nib | top) + 0x60606060u) ^ 0x80808080u;
+                };
+                const uint2 wq = make_uint2(code(ql.x, qh.x), code(ql.y, qh.y));
+                uint2 a = *reinterpret_cast<const uint2 *>(aq_k + h * 128 + 32 * v);
+                if (!real) a = make_uint2(0u, 0u);
+                const v4i_t t = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(a), as_long(wq), zero, 0, 0, 0);
+                // the scale of this lane's 16-wide group: sc[h*8 + 2*v + g/2]
+                const int si = h * 8 + 2 * v + (g >> 1);
+                const int sc = (int)(int8_t)((scw[si >> 2] >> (8 * (si & 3))) & 0xff);
+#pragma unroll
+                for (int r = 0; r < 4; r++) isum[r] += __mul24(sc, t[r]);
+            }
+        }
+        const v4f_t da = *reinterpret_cast<const v4f_t *>(a_d + (size_t)kb * 8);
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] += (d * da[r]) * (float)isum[r];
+        return R;
+    };
+    for (int i = 0; i < my_blocks; i += TM_AHEAD) {
+        R0 = multiply_block(i, R0);
+        if (i + 1 < my_blocks) R1 = multiply_block(i + 1, R1);
+        if (i + 2 < my_blocks) R2 = multiply_block(i + 2, R2);
+        if (i + 3 < my_blocks) R3 = multiply_block(i + 3, R3);
+    }
+    // the two 16-wide halves of every result sit 32 lanes apart
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] += __shfl_xor(acc[r], 32);
+
+    if (KS > 1) {  // add the splits up in order, through the (now idle) activation area
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(lds);
+        if (ksp > 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) red[(((ksp - 1) * RG + rgrp) * 4 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (ksp > 0) return;
+#pragma unroll
+        for (int k = 0; k < KS - 1; k++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += red[((k * RG + rgrp) * 4 + r) * 64 + lane];
+    }
+    if (g < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int b = 4 * g + r;
+            if (b < batch && row0 + j < rows) y[(size_t)b * rows + row0 + j] = acc[r];
+        }
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -638,6 +829,40 @@ static int launch_thin_mfma_rg(const frk_weights *w, int batch, Q8KActs a, float
     }
 }
 
+template <int RG, int ACTS>
+static int launch_thin_mfma6(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t shmem = t6_lds_bytes(ACTS, (int)w->cols);
+    static bool sized = false;
+    if (!sized) {
+        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_mfma_q6_k_kernel<RG, ACTS>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)TM_LDS_LIMIT));
+        sized = true;
+    }
+    const size_t groups = (w->rows + 15) / 16;
+    hipLaunchKernelGGL((thin_mfma_q6_k_kernel<RG, ACTS>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
+                       shmem, s, w->dev, w->layout, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d, y);
+    FRK_LAUNCH_CHECK("thin mfma gemm");
+    return FRK_OK;
+}
+// rows of activations the Q6_K matrix-core kernel can stage for this matrix (8, 4 or 0)
+static int thin_mfma6_acts(const frk_weights *w) {
+    for (int acts = 8; acts >= 4; acts /= 2)
+        if (t6_lds_bytes(acts, (int)w->cols) <= TM_LDS_LIMIT) return acts;
+    return 0;
+}
+template <int ACTS>
+static int launch_thin_mfma6_rg(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t groups = (w->rows + 15) / 16, nb = w->cols / QK_K;
+    int rg = 8;
+    while (rg > 1 && ((groups + rg - 1) / rg < 224 && (size_t)(TM_WAVES / rg) * 4 <= nb)) rg /= 2;
+    switch (rg) {
+        case 8: return launch_thin_mfma6<8, ACTS>(w, batch, a, y, s);
+        case 4: return launch_thin_mfma6<4, ACTS>(w, batch, a, y, s);
+        case 2: return launch_thin_mfma6<2, ACTS>(w, batch, a, y, s);
+        default: return launch_thin_mfma6<1, ACTS>(w, batch, a, y, s);
+    }
+}
+
 // Largest number of activation rows one launch can take for this matrix: up to 16 on the
 // matrix-core path (Q4_K), else what fits LDS, at most 8.
 int thin_gemm_max_batch(const frk_weights *w) {
@@ -656,6 +881,8 @@ int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipSt
         if (batch <= 8) return launch_thin_mfma_rg<8>(w, batch, a, y, s);
         return launch_thin_mfma_rg<16>(w, batch, a, y, s);
     }
+    if (w->kind == FRK_KIND_Q6_K && batch > 2 && thin_mfma6_acts(w) >= (batch > 4 ? 8 : 4))
+        return batch > 4 ? launch_thin_mfma6_rg<8>(w, batch, a, y, s) : launch_thin_mfma6_rg<4>(w, batch, a, y, s);
     if (batch > 4) return launch_thin_nb<8>(w, batch, a, y, s);
     if (batch > 2) return launch_thin_nb<4>(w, batch, a, y, s);
     return launch_thin_nb<2>(w, batch, a, y, s);
