@@ -127,9 +127,12 @@ __device__ __forceinline__ float q4_k_unit_dot(const uint4 h, const uint4 w0, co
 
 // LPR lanes share a row (a wavefront works on 64/LPR rows at once), a lane owns units
 // l, l+LPR, ... (J of them) and keeps RPW rounds of rows in flight.
-template <int LPR, int J, int RPW, int XB, int MODE, int MAXT>
+// GLU: two matrices of one shape (gate = W, up = W2) in one launch; row r of both is computed by the
+// same lanes and y[r] = silu(W[r] . x) * (W2[r] . x) (frink_core::matmul::swiglu,
+// crates/frink-core/src/matmul.rs:634-650), each dot the very sum the plain kernel forms.
+template <int LPR, int J, int RPW, int XB, int MODE, int MAXT, bool GLU = false>
 __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
-    const uint8_t *__restrict__ W, size_t row_stride, int rows, int rows_per_wg, int nb,
+    const uint8_t *__restrict__ W, const uint8_t *__restrict__ W2, size_t row_stride, int rows, int rows_per_wg, int nb,
     const float *__restrict__ x, const int8_t *__restrict__ aq, const float *__restrict__ ad,
     const int16_t *__restrict__ absums, float *__restrict__ y) {
     extern __shared__ uint4 smem[];
@@ -184,6 +187,8 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
 
     // ---- then all the weight loads of the first round ----
     uint4 wh[RPW][J], w0[RPW][J], w1[RPW][J], w2[RPW][J], w3[RPW][J];
+    constexpr int RPW2 = GLU ? RPW : 1, J2 = GLU ? J : 1;
+    uint4 vh[RPW2][J2], v0[RPW2][J2], v1[RPW2][J2], v2[RPW2][J2], v3[RPW2][J2];  // the second matrix's rows
     auto issue = [&](int rbase) {
 #pragma unroll
         for (int k = 0; k < RPW; k++) {
@@ -198,6 +203,19 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
                 w1[k][j] = blk[2 + q2];
                 w2[k][j] = blk[5 + q2];
                 w3[k][j] = blk[6 + q2];
+            }
+            if (GLU) {
+                const uint8_t *row2 = W2 + (size_t)r * row_stride;
+#pragma unroll
+                for (int j = 0; j < J2; j++) {
+                    const uint4 *blk = reinterpret_cast<const uint4 *>(row2 + uoff[j]);
+                    const int q2 = 2 * uq[j];
+                    vh[k][j] = blk[0];
+                    v0[k][j] = blk[1 + q2];
+                    v1[k][j] = blk[2 + q2];
+                    v2[k][j] = blk[5 + q2];
+                    v3[k][j] = blk[6 + q2];
+                }
             }
         }
     };
@@ -233,6 +251,15 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
 #pragma unroll
             for (int j = 0; j < J; j++) acc += q4_k_unit_dot(wh[k][j], w0[k][j], w1[k][j], w2[k][j], w3[k][j], U[j]);
             acc = part_sum<LPR>(acc);
+            if (GLU) {
+                float up = 0.0f;
+#pragma unroll
+                for (int j = 0; j < J2; j++) up += q4_k_unit_dot(vh[k][j], v0[k][j], v1[k][j], v2[k][j], v3[k][j], U[j]);
+                up = part_sum<LPR>(up);
+                // exp in double, rounded once: what a host libm's expf returns in all but a vanishing
+                // share of cases, so a quantizer downstream sees the same input as the reference's
+                acc = __fdiv_rn(acc, 1.0f + (float)exp(-(double)acc)) * up;
+            }
             if (l == 0 && r < row_end) y[r] = acc;
         }
     }
@@ -286,16 +313,18 @@ static FusedGeom fused_geom(size_t rows, int units, bool fused) {
     return g;
 }
 
-template <int MODE>
-static int launch_q4_k_fused(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+template <int MODE, bool GLU = false>
+static int launch_q4_k_fused(const frk_weights *w, const frk_weights *w2, const float *x, Q8KActs a, float *y,
+                             hipStream_t s) {
     const int nb = (int)(w->cols / QK_K);
     FusedGeom g = fused_geom(w->rows, nb * 2, MODE == MODE_FUSED);
     const size_t shmem = MODE == MODE_PREQ_DIRECT ? 0 : (size_t)nb * (256 + 32 + 4);
     const int nwaves = g.threads / 64;
     const int xb = (nb + nwaves - 1) / nwaves;
 #define FRK_GO2(LPR, J, RPW, XB, MAXT)                                                                            \
-    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT>), dim3(g.grid), dim3(g.threads), shmem, \
-                       s, w->dev, w->layout.row_stride, (int)w->rows, g.rows_per_wg, nb, x, a.q, a.d, a.bsums, y)
+    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT, GLU>), dim3(g.grid), dim3(g.threads),   \
+                       shmem, s, w->dev, GLU ? w2->dev : nullptr, w->layout.row_stride, (int)w->rows, g.rows_per_wg, \
+                       nb, x, a.q, a.d, a.bsums, y)
 #define FRK_GO(LPR, J, RPW, MAXT)                                               \
     do {                                                                        \
         if (MODE == MODE_PREQ_DIRECT || xb <= 1) FRK_GO2(LPR, J, RPW, 1, MAXT); \
@@ -321,11 +350,15 @@ bool fused_gemv_fits(const frk_weights *w) {
 }
 
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
-    return launch_q4_k_fused<MODE_FUSED>(w, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
+    return launch_q4_k_fused<MODE_FUSED>(w, nullptr, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
 }
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
-    if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, a, y, s);
-    return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, a, y, s);
+    if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, nullptr, a, y, s);
+    return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, nullptr, a, y, s);
+}
+// act[r] = silu(gate[r] . x) * (up[r] . x): both matrices Q4_K of one shape, fused_gemv_fits
+int launch_gemv_q4_k_glu(const frk_weights *gate, const frk_weights *up, const float *x, float *act, hipStream_t s) {
+    return launch_q4_k_fused<MODE_FUSED, true>(gate, up, x, Q8KActs{nullptr, nullptr, nullptr}, act, s);
 }
 
 }  // namespace frk

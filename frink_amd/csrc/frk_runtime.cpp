@@ -429,7 +429,23 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
                              ws[i]->cols, ws[0]->cols);
         any_k = any_k || ws[i]->kind == FRK_KIND_Q4_K || ws[i]->kind == FRK_KIND_Q6_K;
     }
-    // one Q8_K quantization for every K-quant matrix of the group
+    // Where every matrix has a one-launch GEMV that quantizes the activation inside the kernel (in
+    // the shadow of its first weight loads), sharing a quantization launch is slower than not having
+    // one: measured 8.5 us per fused launch against 4.7 + 8.2 per matrix with the shared pass.
+    bool all_fused = true;
+    for (size_t i = 0; i < n; i++) {
+        const frk_weights *w = ws[i];
+        all_fused = all_fused && ((w->kind == FRK_KIND_Q4_K && fused_gemv_fits(w)) ||
+                                  (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) || w->kind == FRK_KIND_Q8_0);
+    }
+    if (all_fused) {
+        for (size_t i = 0; i < n; i++) {
+            int rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
+            if (rc) return rc;
+        }
+        return FRK_OK;
+    }
+    // otherwise one Q8_K quantization for every K-quant matrix of the group
     Q8KActs a = {nullptr, nullptr, nullptr};
     if (any_k) {
         int rc = quantize_acts_q8_k(ws[0], x, 1, s, &a);
@@ -461,12 +477,19 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
     if (rc) return rc;
     float *g_out = (float *)((char *)ws + q_area), *u_out = g_out + round_up(ffn * 4, 256) / 4,
           *act = u_out + round_up(ffn * 4, 256) / 4;
-    const frk_weights *pair[2] = {gate, up};
-    float *outs[2] = {g_out, u_out};
-    rc = frk_hip_gemv_multi_dev(pair, 2, x, outs, stream);
-    if (rc) return rc;
-    rc = launch_swiglu(g_out, u_out, ffn, act, s);
-    if (rc) return rc;
+    if (gate->kind == FRK_KIND_Q4_K && up->kind == FRK_KIND_Q4_K && fused_gemv_fits(gate) &&
+        gate->layout.row_stride == up->layout.row_stride) {
+        // gate, up and SwiGLU in one launch: row r of both matrices is computed by the same lanes
+        rc = launch_gemv_q4_k_glu(gate, up, x, act, s);
+        if (rc) return rc;
+    } else {
+        const frk_weights *pair[2] = {gate, up};
+        float *outs[2] = {g_out, u_out};
+        rc = frk_hip_gemv_multi_dev(pair, 2, x, outs, stream);
+        if (rc) return rc;
+        rc = launch_swiglu(g_out, u_out, ffn, act, s);
+        if (rc) return rc;
+    }
     return frk_hip_gemv_dev(down, act, y, FRK_ACT_F32, stream);
 }
 
