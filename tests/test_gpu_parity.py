@@ -430,9 +430,9 @@ def test_cpp_host_mirror_launches(fa):
 @pytest.mark.parametrize("kind,rows,cols,batch", [
     (fo.Q4_K, 70, 1024, 2), (fo.Q4_K, 33, 512, 3), (fo.Q4_K, 128, 4096, 8), (fo.Q4_K, 64, 256, 5),
     (fo.Q4_K, 40, 2048, 11), (fo.Q4_K, 16, 768, 15), (fo.Q4_K, 100, 1024, 16), (fo.Q4_K, 17, 256, 16),
-    (fo.Q4_K, 1000, 4096, 9), (fo.Q4_K, 31, 8192, 13),
+    (fo.Q4_K, 1000, 4096, 9), (fo.Q4_K, 31, 8192, 13), (fo.Q4_K, 20, 16384, 6), (fo.Q4_K, 18, 32768, 5),
     (fo.Q6_K, 70, 1024, 2), (fo.Q6_K, 33, 512, 3), (fo.Q6_K, 48, 14336, 8), (fo.Q6_K, 64, 256, 7),
-    (fo.Q6_K, 40, 2048, 11), (fo.Q6_K, 24, 768, 40),
+    (fo.Q6_K, 40, 2048, 11), (fo.Q6_K, 24, 768, 40), (fo.Q6_K, 19, 28672, 4), (fo.Q6_K, 50, 4096, 5),
 ])
 def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
     from frink_amd import synth
