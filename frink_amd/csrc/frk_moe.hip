@@ -123,8 +123,17 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
     L.run[tid] = 0;
     for (int r = tid; r < max_rows; r += 1024) gather[r] = -1;
     __syncthreads();
+    // the first 4096 ids stay in registers for all three passes (each pass from memory costs a
+    // round trip this one-workgroup kernel has nothing to hide behind)
+    int held[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) held[i] = tid + 1024 * i < pairs ? ids[tid + 1024 * i] : -1;
+    auto id_of = [&](int p) {  // p = tid (mod 1024)
+        const int i = p >> 10;
+        return i == 0 ? held[0] : i == 1 ? held[1] : i == 2 ? held[2] : i == 3 ? held[3] : ids[p];
+    };
     for (int p = tid; p < pairs; p += 1024) {
-        const int e = ids[p];
+        const int e = id_of(p);
         if (e >= 0 && e < n_experts) atomicAdd(&L.cnt[e], 1);
         else pos_of[p] = cpos_of[p] = -1;
     }
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
         for (int i = tid; i < rw * n_experts; i += 1024) L.bits[i] = 0;
         __syncthreads();
         for (int j = tid; j < round && p0 + j < pairs; j += 1024) {
-            const int e = ids[p0 + j];
+            const int e = (p0 & 1023) == 0 ? id_of(p0 + j) : ids[p0 + j];
             if (e >= 0 && e < n_experts) atomicOr(&L.bits[(j >> 5) * n_experts + e], 1u << (j & 31));
         }
         __syncthreads();
@@ -191,7 +200,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
         __syncthreads();
         for (int j = tid; j < round && p0 + j < pairs; j += 1024) {
             const int p = p0 + j;
-            const int e = ids[p];
+            const int e = (p0 & 1023) == 0 ? id_of(p) : ids[p];
             if (e >= 0 && e < n_experts) {
                 const int w = (j >> 5) * n_experts + e;
                 const int rank = L.run[e] + L.before[w] + __popc(L.bits[w] & ((1u << (j & 31)) - 1u));
