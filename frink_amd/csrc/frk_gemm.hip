@@ -138,13 +138,6 @@ __device__ __forceinline__ void read_scales(TileScales &S, uint32_t scales) {
     FRK_DS_READ(S.da3, scales, 96);
 }
 template <int N>
-__device__ __forceinline__ void wait_ops(TileOperands &T) {
-    asm volatile("s_waitcnt lgkmcnt(%9)"
-                 : "+v"(T.a0), "+v"(T.a1), "+v"(T.a2), "+v"(T.a3), "+v"(T.a4), "+v"(T.a5), "+v"(T.a6), "+v"(T.a7),
-                   "+v"(T.bs)
-                 : "n"(N));
-}
-template <int N>
 __device__ __forceinline__ void wait_scales(TileScales &S) {
     asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(S.da0), "+v"(S.da1), "+v"(S.da2), "+v"(S.da3) : "n"(N));
 }
@@ -205,31 +198,6 @@ __device__ __forceinline__ void unpack_block(const RawBlock &R, int lg, BPlanes 
     B.ndmin = -h2f(hx >> 16);
 }
 
-// S1 = 8 * (acts . H) + (acts . L) in ONE accumulator: the H chain first, its result shifted left by
-// three, then the L chain on top of it.  (Two accumulators would cost 16 more registers per lane.)
-__device__ __forceinline__ void tile_mfmas(const TileOperands &T, const BPlanes &B, TileAcc &X) {
-    const v16i zi = {0};
-    const v16f zf = {0.0f};
-    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
-    X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);  // runs while the shift waits
-    acc = acc << 3;
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
-    X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
-}
-
 __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales &S, const BPlanes &B, v16f &acc) {
     const v4f dav[4] = {S.da0, S.da1, S.da2, S.da3};
 #pragma unroll
@@ -242,6 +210,121 @@ __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales
         }
 }
 
+// The 16 + 1 MFMAs of a tile, each waiting only for the operand it needs: the tile's nine LDS reads
+// (a0..a7, bs, in that order) must be the wavefront's youngest LDS operations.
+// (Each wait also names the running sum as modified, which pins it between its two MFMAs: without
+// that the MFMAs are free to sink below all the waits, and the chain starts only when the last
+// operand is there.)
+#define FRK_WAIT_LGKM(n, reg, acc) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(reg), "+v"(acc))
+__device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const BPlanes &B, TileAcc &X) {
+    const v16i zi = {0};
+    const v16f zf = {0.0f};
+    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    FRK_WAIT_LGKM(7, T.a1, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(6, T.a2, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(5, T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(4, T.a4, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(3, T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(2, T.a6, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(1, T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(0, T.bs, acc);
+    X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+}
+
+// The dense kernel's form of a tile, one accumulator less: the mins' MFMA adds onto the converted
+// integer sums instead of into registers of its own.  With d' = d / (-dmin):
+//     d * S1 - dmin * S2 = (-dmin) * (d' * S1 + S2),
+// so the f16 MFMA takes d' * S1 as its C operand and the epilogue multiplies by -dmin (and the token's
+// scale).  A row whose dmin is zero keeps d and a factor of one, and zero mins.  (Not the same
+// rounding as the two-term form: both are within a few ulp of the exact sum.)
+__device__ __forceinline__ void fold_mins(BPlanes &B) {
+    const bool z = B.ndmin == 0.0f;
+    B.d = z ? B.d : B.d * __builtin_amdgcn_rcpf(B.ndmin);
+    B.ndmin = z ? 1.0f : B.ndmin;
+    if (z) B.m = v8h{0, 0, 0, 0, 0, 0, 0, 0};
+}
+// between(i, acc) is called after MFMA i has been issued, i = 0..15: what it issues (the prefetch)
+// shares the gaps of the chain, every MFMA of which waits for the one before it.
+struct NothingBetween {
+    __device__ __forceinline__ void operator()(int, v16i &) const {}
+};
+template <class Between = NothingBetween>
+__device__ __forceinline__ v16f tile_mfmas_folded(TileOperands &T, const BPlanes &B, Between between = Between()) {
+    const v16i zi = {0};
+    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    between(0, acc);
+    FRK_WAIT_LGKM(7, T.a1, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    between(1, acc);
+    FRK_WAIT_LGKM(6, T.a2, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    between(2, acc);
+    FRK_WAIT_LGKM(5, T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    between(3, acc);
+    FRK_WAIT_LGKM(4, T.a4, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    between(4, acc);
+    FRK_WAIT_LGKM(3, T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    between(5, acc);
+    FRK_WAIT_LGKM(2, T.a6, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    between(6, acc);
+    FRK_WAIT_LGKM(1, T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    between(7, acc);
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    between(8, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    between(9, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    between(10, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    between(11, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    between(12, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    between(13, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    between(14, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+    FRK_WAIT_LGKM(0, T.bs, acc);
+    v16f c;
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[r] = B.d * (float)acc[r];
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, c, 0, 0, 0);
+}
+__device__ __forceinline__ void tile_epilogue_folded(const v16f &c, const TileScales &S, const BPlanes &B, v16f &acc) {
+    const v4f dav[4] = {S.da0, S.da1, S.da2, S.da3};
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int r = q * 4 + e;
+            acc[r] = fmaf(dav[q][e] * B.ndmin, c[r], acc[r]);
+        }
+}
+
 // A workgroup = RG*WT wavefronts = RG row groups of 32 weight rows x WT token groups of MT 32-token
 // tiles.  A wavefront keeps the current block of its 32 rows in registers as MFMA B operands and
 // runs its MT tiles against them, so a block of a row is unpacked once per MT tiles.  A SIMD holds
@@ -249,11 +332,14 @@ __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales
 // epilogue), which is how the matrix cores and the vector ALU overlap here.
 //
 // What bounds the tile shape: every block moves (32*RG*144 + 32*NT*292) bytes from L2 into LDS for
-// 2*32*RG*32*NT*256 operations, and the L2-to-LDS path sustained roughly 9 TB/s over the chip when
-// measured with the arithmetic switched off, so more rows and tokens per workgroup is better -- until
-// the registers run out: 256 rows x 64 tokens (8 wavefronts, two tiles each) is the largest shape
-// that compiles without spills at two wavefronts per SIMD (256 registers per lane), and a spill is
-// fatal here because scratch reloads wait on the same counter as the prefetch.
+// 2*32*RG*32*NT*256 operations, and a CU's address unit takes roughly 40 cycles per kilobyte of such
+// loads (whether they write LDS directly or go through registers), so more rows and tokens per
+// workgroup is better -- until the registers run out: 256 rows x 128 tokens (8 wavefronts, four
+// tiles each) fits two wavefronts per SIMD (256 registers per lane) without spills, and a spill is
+// fatal here because scratch reloads wait on the same counter as the prefetch.  What keeps the
+// registers down: the prefetch writes LDS directly, its addresses are recomputed from the lane
+// number at every use (made opaque, or the compiler keeps them all), the mins' term shares the
+// integer sums' accumulator (tile_mfmas_folded) and every tile's epilogue is pinned to its tile.
 //
 // LDS rings.  Activations, 2 stages:
 //     quants [NT][8 k-slices][1 KB] | bsums f16 [NT][1 KB] | scales f32 [NT*32],  NT = MT*WT tiles
@@ -302,49 +388,70 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
 
     // ---- what this lane fetches ----
+    // Only 32-bit offsets of the first piece are kept in registers; everything else is uniform or is
+    // recomputed from them where it is used.
     // activations: the tiled form is the LDS image, so chunk (tile t, slice ks) is 1 KB of consecutive
     // memory and lane j brings its bytes 16*j..; same for the sums.  Tiles past the last one repeat it.
-    const int8_t *a_src[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) a_src[t] = g.a.q + (size_t)min(tile0 + t, last_tile) * nb * 8192 + lane * 16;
+    // (offsets from the quants: the three arrays of the tiled form are carved from one allocation,
+    // quants first)
+    const uint8_t *Qb = reinterpret_cast<const uint8_t *>(g.a.q);
+    const uint32_t bs_base = (uint32_t)(reinterpret_cast<const uint8_t *>(g.a.bs) - Qb);
+    const uint32_t d_base = (uint32_t)(reinterpret_cast<const uint8_t *>(g.a.d) - Qb);
+    auto tile_rec = [&](int t) { return (uint32_t)min(tile0 + t, last_tile) * (uint32_t)nb; };  // uniform
     // with fewer chunks than wavefronts some fetch a chunk twice, into the same place
     const int bs_tile = wave % NT, da_chunk = wave % N_DA;
-    const _Float16 *b_src = g.a.bs + (size_t)min(tile0 + bs_tile, last_tile) * nb * 512 + lane * 8;
-    const float *d_src = g.a.d + (size_t)min(tile0 + 2 * da_chunk + lg, last_tile) * nb * 32 + li;
     // weights: a row group's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of chunk c, so that
-    // LDS holds the rows back to back (144 bytes each) and consecutive lanes read consecutive memory.
+    // LDS holds the rows back to back (144 bytes each) and consecutive lanes read consecutive memory:
+    // chunk c is 7c rows further down and c pieces to the right of chunk 0, modulo the nine of a row.
+    // Offsets past the matrix are pulled back to its last 16 bytes (such rows are never stored).
     // With WT = 2 the two wavefronts of a row group split the five chunks (3 + 2, one fetched twice).
+    const uint8_t *Wb = g.W;
+    const uint32_t stride = (uint32_t)g.row_stride;
+    const uint32_t w_last = (uint32_t)g.rows * stride - 16;
     const int wc0 = (WT == 1) ? 0 : (tgrp == 0 ? 0 : 3);
-    const uint8_t *w_src[C_W];
-    int w_chunk[C_W];
-#pragma unroll
-    for (int i = 0; i < C_W; i++) {
-        const int c = min(wc0 + i, 4) - ((WT == 2 && tgrp == 1 && i == 2) ? 1 : 0);  // tgrp 1: chunks 3, 4, 3
-        w_chunk[i] = c;
-        const int p = min(c * 64 + lane, 287);
-        const int r = min(row0 + p / 9, g.rows - 1);
-        w_src[i] = g.W + (size_t)r * g.row_stride + (p % 9) * 16;
-    }
-
-    auto issue_acts = [&](int kb) {
-        uint8_t *st = lds + (kb & 1) * L::A_STAGE;
-#pragma unroll
-        for (int t = 0; t < NT; t++)
-#pragma unroll
-            for (int i = 0; i < 8 / NW; i++) {
-                const int ks = ((wave + t) % NW) + NW * i;
-                load_to_lds16(a_src[t] + (size_t)kb * 8192 + ks * 1024, st + (t * 8 + ks) * 1024);
-            }
-        load_to_lds16(b_src + (size_t)kb * 512, st + L::OFF_BS + bs_tile * 1024);
-        load_to_lds4(d_src + kb * 32, st + L::OFF_DA + da_chunk * 256);
+    auto chunk_of = [&](int i) { return min(wc0 + i, 4) - ((WT == 2 && tgrp == 1 && i == 2) ? 1 : 0); };  // tgrp 1: 3, 4, 3
+    auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return l;
     };
-    auto issue_weights = [&](int kb) {  // C_W loads
-        uint8_t *st = lds_w + (kb % WS) * L::W_STAGE + rgrp * L::W_GROUP;
-#pragma unroll
-        for (int i = 0; i < C_W; i++) {
-            // chunk 4 is half a chunk: 32 pieces
-            if (w_chunk[i] < 4 || lane < 32) load_to_lds16(w_src[i] + (size_t)kb * Q4_K_BYTES, st + w_chunk[i] * 1024);
+
+    // the prefetch of one block, as N_A + 2 + C_W separate loads so that they can be issued one by one
+    constexpr int N_A = NT * (8 / NW), N_DMA = N_A + 2 + C_W;
+    auto act_part = [&](int j, int kb) {  // j = 0 .. N_A + 1
+        asm volatile("" : "+s"(kb));  // (seen as the loop counter, every address becomes a pointer of its own)
+        uint8_t *st = lds + (kb & 1) * L::A_STAGE;
+        const uint32_t l = (uint32_t)opaque_lane();
+        if (j < N_A) {
+            const int t = j / (8 / NW), i = j % (8 / NW);
+            const int ks = ((wave + t) % NW) + NW * i;
+            load_to_lds16(Qb + ((tile_rec(t) + kb) * 8192 + ks * 1024 + l * 16), st + (t * 8 + ks) * 1024);
+        } else if (j == N_A) {
+            load_to_lds16(Qb + (bs_base + (tile_rec(bs_tile) + kb) * 1024 + l * 16), st + L::OFF_BS + bs_tile * 1024);
+        } else {
+            load_to_lds4(Qb + (d_base + (tile_rec(2 * da_chunk + (l >> 5)) + kb) * 128 + (l & 31) * 4),
+                         st + L::OFF_DA + da_chunk * 256);
         }
+    };
+    auto weight_part = [&](int i, int kb) {  // i = 0 .. C_W - 1
+        asm volatile("" : "+s"(kb));
+        uint8_t *st = lds_w + (kb % WS) * L::W_STAGE + rgrp * L::W_GROUP;
+        const uint32_t l = (uint32_t)opaque_lane();
+        const uint32_t pc0 = l % 9;
+        const uint32_t off0 = ((uint32_t)(row_tile * ROWS + rgrp * 32) + l / 9) * stride + pc0 * 16 + (uint32_t)kb * Q4_K_BYTES;
+        const int c = chunk_of(i);
+        const uint32_t v = pc0 + c, wrap = v >= 9 ? 1u : 0u;  // c <= 4: at most one wrap
+        const uint32_t off = off0 + (uint32_t)(7 * c) * stride + wrap * (stride - 144) + c * 16;
+        // chunk 4 is half a chunk: 32 pieces
+        if (c < 4 || l < 32) load_to_lds16(Wb + min(off, w_last), st + c * 1024);
+    };
+    auto issue_acts = [&](int kb) {
+#pragma unroll
+        for (int j = 0; j < N_A + 2; j++) act_part(j, kb);
+    };
+    auto issue_weights = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < C_W; i++) weight_part(i, kb);
     };
 
     const uint32_t lds_a = lds_address(lds);
@@ -356,6 +463,8 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
 
     BPlanes B;
     RawBlock R;
+    v16i accI0 = {0};  // (an argument the prefetch does not use)
+    const int pf_tile = __builtin_amdgcn_readfirstlane(wave >= NW / 2 ? MT / 2 : 0);
 
     // prologue: weights of blocks 0..WD-1, activations of block 0; the last weights may stay in flight
     issue_weights(0);
@@ -369,36 +478,67 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     read_raw(R, lds_wv, lds_wv + 16 * lg);
     wait_raw<0>(R);
     unpack_block(R, lg, B);
+    fold_mins(B);
 
     for (int kb = 0; kb < nb; kb++) {
-        // the stages refilled here were last read in iteration kb-1, which every wavefront has left
-        if (kb + 1 < nb) issue_acts(kb + 1);
-        if (kb + WD < nb) issue_weights(kb + WD);
-
+        // The first tile's operands are requested before anything else: they travel from LDS while
+        // the prefetch below is issued.  In the same way every later tile's operands are requested
+        // before the epilogue of the tile before it.
         const uint32_t st = lds_a + (kb & 1) * L::A_STAGE;
         const uint32_t qa = st + lane * 16, ba = st + L::OFF_BS + lane * 16, sa = st + L::OFF_DA + lg * 16;
         const uint32_t wa = lds_wv + ((kb + 1) % WS) * L::W_STAGE;
+        TileOperands T;
+        read_ops(T, qa + (tgrp * MT) * 8192, ba + (tgrp * MT) * 1024);
+        // The prefetch (the stages refilled were last read in iteration kb-1, which every wavefront
+        // has left).  A wavefront is stalled while its loads wait for the CU's one address unit, and
+        // a block's loads keep that unit busy for about as long as half the block's MFMAs take: so the
+        // two wavefronts of a SIMD (w and w + NW/2) issue theirs at different times, from inside the
+        // chain of MFMAs of their first and of their middle tile, one load per gap; while one is
+        // stalled the other has the matrix core.  With one tile per wavefront there is no such choice.
+        auto prefetch_part = [&](int j, v16i &) {
+            if (j < N_A + 2) {
+                if (kb + 1 < nb) act_part(j, kb + 1);
+            } else if (j < N_DMA) {
+                if (kb + WD < nb) weight_part(j - (N_A + 2), kb + WD);
+            }
+        };
+        if (MT == 1) {
+#pragma unroll
+            for (int j = 0; j < N_DMA; j++) prefetch_part(j, accI0);
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             const int t = tgrp * MT + mt;
-            TileOperands T;
             TileScales S;
-            TileAcc X;
-            read_ops(T, qa + t * 8192, ba + t * 1024);
-            wait_ops<0>(T);
-            tile_mfmas(T, B, X);
-            // the scales, and with the last tile the next block's raw weights (landed since iteration
-            // kb-1), are fetched while the MFMAs run; their registers are the ones the operands leave
+            v16f c;
+            if (MT > 1 && (mt == 0 || mt == MT / 2)) {
+                // (one chain for both cases, the choice made per load: two copies of the chain behind
+                // a branch would meet in register copies of the operands, which the compiler, blind
+                // to the hand-placed waits, is free to put in front of them)
+                c = tile_mfmas_folded(T, B, [&](int j, v16i &a) {
+                    if (mt == pf_tile) prefetch_part(j, a);
+                });
+            } else {
+                c = tile_mfmas_folded(T, B);
+            }
             read_scales(S, sa + t * 128);
-            if (mt == MT - 1) read_raw(R, wa, wa + 16 * lg);
-            if (mt == MT - 1) wait_scales<5>(S);
-            else wait_scales<0>(S);
-            tile_epilogue(X, S, B, accF[mt]);
-            __builtin_amdgcn_sched_barrier(0);  // keep a tile's registers from living into the next tile
+            if (mt + 1 < MT) {
+                read_ops(T, qa + (t + 1) * 8192, ba + (t + 1) * 1024);
+                wait_scales<9>(S);
+            } else {
+                wait_scales<0>(S);
+            }
+            tile_epilogue_folded(c, S, B, accF[mt]);
+            // (the sums are next used in the following iteration, which lets the compiler sink the
+            // epilogues of all tiles to the end of this one, every tile's MFMA result alive until then)
+            asm volatile("" : "+v"(accF[mt]));
         }
         if (kb + 1 < nb) {
+            // the next block's raw weights landed during iteration kb-1
+            read_raw(R, wa, wa + 16 * lg);
             wait_raw<0>(R);
             unpack_block(R, lg, B);
+            fold_mins(B);
             // activations of block kb+1 and weights of block kb+2 must have landed; with four weight
             // stages the weights requested above (younger than both) may stay in flight
             if (WS == 4 && kb + WD < nb) wait_vm<C_W>();
@@ -415,44 +555,6 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
             const int tok = tok0 + (tgrp * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
             if (row < g.rows && tok < g.M) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
         }
-}
-
-// The 16 + 1 MFMAs of a tile, each waiting only for the operand it needs: the tile's nine LDS reads
-// (a0..a7, bs, in that order) must be the wavefront's youngest LDS operations.
-// (Each wait also names the running sum as modified, which pins it between its two MFMAs: without
-// that the MFMAs are free to sink below all the waits, and the chain starts only when the last
-// operand is there.)
-#define FRK_WAIT_LGKM(n, reg, acc) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(reg), "+v"(acc))
-__device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const BPlanes &B, TileAcc &X) {
-    const v16i zi = {0};
-    const v16f zf = {0.0f};
-    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
-    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
-    FRK_WAIT_LGKM(7, T.a1, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(6, T.a2, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(5, T.a3, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(4, T.a4, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(3, T.a5, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(2, T.a6, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(1, T.a7, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(0, T.bs, acc);
-    X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);
-    acc = acc << 3;
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
-    X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
 }
 
 // The grouped (per-expert) GEMM for tiles of at most 32 activation rows: with so few rows per
@@ -810,6 +912,7 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
         return (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
     };
     const size_t wgs_big = ((w->rows + 255) / 256) * ((M + 63) / 64);
+    if (M > 64 && ((w->rows + 255) / 256) * ((M + 127) / 128) >= 200) return launch_variant<8, 1, 4, 2>(g, grid_for(256, 128), s);
     if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2>(g, grid_for(256, 64), s);
     if (M > 32) return launch_variant<4, 2, 1, 4>(g, grid_for(128, 64), s);
     return launch_variant<4, 1, 1, 2>(g, grid_for(128, 32), s);

@@ -1,0 +1,47 @@
+"""The GEMM kernels read LDS from inline assembly and wait by hand; this compiles them to assembly
+and checks that nothing touches a register before the wait that releases it (isa_wait_lint)."""
+import os
+import subprocess
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+import isa_wait_lint  # noqa: E402
+
+
+def _assembly(tmp_path, name):
+    from frink_amd import build as fb
+    out = str(tmp_path / (name + ".s"))
+    cmd = [fb.hipcc()] + fb.HIPCC_FLAGS + ["-x", "hip", "--cuda-device-only", "-S", os.path.join(fb.CSRC, name), "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return open(out).read()
+
+
+def test_no_use_of_lds_reads_before_their_waits(tmp_path):
+    asm = _assembly(tmp_path, "frk_gemm.hip")
+    names = isa_wait_lint.kernels(asm)
+    assert sum("gemm_q4_k" in k for k in names) >= 5, names  # the dense variants and the streaming kernel
+    for k in names:
+        assert isa_wait_lint.violations(asm, k) == [], k
+    asm = _assembly(tmp_path, "frk_gemv_direct.hip")
+    names = isa_wait_lint.kernels(asm)
+    assert names
+    for k in names:
+        assert isa_wait_lint.violations(asm, k) == [], k
+
+
+def test_lint_sees_an_early_copy():
+    asm = "\n".join([
+        "k:",
+        "\tds_read_b128 v[4:7], v1 offset:0",
+        "\tds_read_b128 v[8:11], v1 offset:16",
+        "\tv_mov_b64_e32 v[20:21], v[4:5]",
+        "\ts_waitcnt lgkmcnt(1)",
+        "\tv_add_u32_e32 v30, v4, v5",
+        "\tv_add_u32_e32 v31, v8, v5",
+        "\ts_waitcnt lgkmcnt(0)",
+        "\tv_add_u32_e32 v31, v8, v5",
+        "\ts_endpgm",
+    ])
+    got = isa_wait_lint.violations(asm, "k")
+    assert len(got) == 2 and "line 4" in got[0] and "line 7" in got[1], got
