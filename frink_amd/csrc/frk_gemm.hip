@@ -894,6 +894,10 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
 
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
+    // the kernel addresses the weights and the tiled activations with 32-bit byte offsets
+    if ((uint64_t)w->rows * w->layout.row_stride >= (1ull << 32) || (uint64_t)q8k_tiled_bytes(M, w->cols) >= (1ull << 32))
+        return set_error(FRK_ERR_SHAPE, "gemm_q4_k: %zu x %zu weights with %zu activation rows exceed 4 GiB per operand", w->rows,
+                         w->cols, M);
     GemmArgs g;
     g.a = q8k_tiled_carve(ws, M, w->cols);
     int rc = launch_quantize_q8_k_tiled(x, M, w->cols, g.a, s);
@@ -904,8 +908,8 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.nb = (int)(w->cols / QK_K);
     g.M = (int)M;
     g.y = y;
-    // shape of a workgroup's tile: 256 rows x 64 tokens when that still gives every CU a workgroup,
-    // else 128 rows x 64 or 32 tokens
+    // shape of a workgroup's tile: 256 rows x 128 or 64 tokens when that still gives (about) every CU a
+    // workgroup, else 128 rows x 64 or 32 tokens
     auto grid_for = [&](int rows_wg, int tm) {
         g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
         g.tok_tiles = (int)((M + tm - 1) / tm);

@@ -268,6 +268,24 @@ def test_gemm_mfma_matches_the_oracle(fa, rows, cols, batch):
     w.release()
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(13000, 512, 500), (14336, 512, 320), (13001, 768, 1000)])
+def test_gemm_large_tiles_with_ragged_edges(fa, rows, cols, batch):
+    """Shapes that take the 256-row workgroup tiles (x128 tokens: 13000x500 and 13001x1000; x64:
+    14336x320) with a last row tile and a last token tile that are partly empty: the first, a middle
+    and the last 256 weight rows against the oracle, and zeros nowhere they do not belong."""
+    from frink_amd import synth
+    print("gemm large tiles", rows, cols, batch, flush=True)
+    data = make_weights(fo.Q4_K, rows, cols, seed=rows + batch)
+    x = synth.activations(rows + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    y = w.gemm(to_dev(x)).cpu().numpy()
+    assert y.shape == (batch, rows)
+    for row0 in (0, (rows // 2) // 32 * 32 + 7, rows - 256):
+        want = fo.gemm(fo.Q4_K, data, rows, cols, x, row0=row0, nrows=256)
+        assert_rows_close(y[:, row0:row0 + 256], want, "gemm %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
+    w.release()
+
+
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (14336, 4096)])
 def test_full_size_prefill_gemm(fa, rows, cols):
     """M=512 with 1% outliers at +-20: every output row of the batch against the oracle on a
