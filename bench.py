@@ -173,7 +173,7 @@ def main():
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512>", "algorithmic_bytes": int(alg_bytes),
+                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false>", "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
     }
 
