@@ -173,7 +173,7 @@ def main():
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false>", "algorithmic_bytes": int(alg_bytes),
+                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false, false>", "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
     }
 
@@ -277,6 +277,23 @@ def main():
             "frac_of_hbm_peak": round(fb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
         for w in g8 + u8 + dn:
             w.release()
+        # q/k/v of a Llama-3-8B layer (4096, 1024 and 1024 rows of 4096): one launch for the three;
+        # 40 sets of weights in turn (566 MB > the 256 MB Infinity Cache)
+        qkv_rows = (4096, 1024, 1024)
+        qkv_dev = [torch.from_numpy(random_blocks(kind, r, cols, seed=90 + j)).to(dev) for j, r in enumerate(qkv_rows)]
+        qkv_sets = [[fa.Weights.from_device(kind, d.clone(), r, cols) for d, r in zip(qkv_dev, qkv_rows)] for _ in range(40)]
+        qkv_out = [torch.empty(r, dtype=torch.float32, device=dev) for r in qkv_rows]
+
+        def step7(i):
+            fa.gemv_multi(qkv_sets[i % 40], xd, outs=qkv_out)
+        _, t = time_graph(torch, step7, 800, 40)
+        qb = sum(qkv_rows) * (cols // 256) * 144
+        extra["Q4_K q/k/v multi-GEMV (4096+1024+1024)x4096, one launch"] = {
+            "us_per_step": round(t / 800 * 1e6, 2), "GBs": round(qb / (t / 800) / 1e9, 1),
+            "frac_of_hbm_peak": round(qb / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+        for ws_ in qkv_sets:
+            for w in ws_:
+                w.release()
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -130,11 +130,20 @@ __device__ __forceinline__ float q4_k_unit_dot(const uint4 h, const uint4 w0, co
 // GLU: two matrices of one shape (gate = W, up = W2) in one launch; row r of both is computed by the
 // same lanes and y[r] = silu(W[r] . x) * (W2[r] . x) (frink_core::matmul::swiglu,
 // crates/frink-core/src/matmul.rs:634-650), each dot the very sum the plain kernel forms.
-template <int LPR, int J, int RPW, int XB, int MODE, int MAXT, bool GLU = false>
+// MULTI: up to four matrices of one row length that multiply the same activation (q/k/v, or any
+// group launch_matvec_multi gets, crates/frink-cuda/src/matvec_launch.rs:485-534) in one launch: the
+// kernel walks the matrices' rows as one list, `rows` long; row v of the list belongs to the last
+// matrix m with first[m] <= v.
+struct MultiArgs {
+    const uint8_t *W[4];
+    float *y[4];
+    int first[4];  // unused entries hold the total
+};
+template <int LPR, int J, int RPW, int XB, int MODE, int MAXT, bool GLU = false, bool MULTI = false>
 __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ W2, size_t row_stride, int rows, int rows_per_wg, int nb,
     const float *__restrict__ x, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-    const int16_t *__restrict__ absums, float *__restrict__ y) {
+    const int16_t *__restrict__ absums, float *__restrict__ y, MultiArgs ma) {
     extern __shared__ uint4 smem[];
     int8_t *sq = reinterpret_cast<int8_t *>(smem);
     int16_t *sbs = reinterpret_cast<int16_t *>(sq + nb * QK_K);
@@ -194,6 +203,14 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
         for (int k = 0; k < RPW; k++) {
             const int r = min(rbase + slot + k * slots, rows - 1);
             const uint8_t *row = W + (size_t)r * row_stride;
+            if (MULTI) {
+                const uint8_t *base = ma.W[0];
+                int first = 0;
+                if (r >= ma.first[1]) base = ma.W[1], first = ma.first[1];
+                if (r >= ma.first[2]) base = ma.W[2], first = ma.first[2];
+                if (r >= ma.first[3]) base = ma.W[3], first = ma.first[3];
+                row = base + (size_t)(r - first) * row_stride;
+            }
 #pragma unroll
             for (int j = 0; j < J; j++) {
                 const uint4 *blk = reinterpret_cast<const uint4 *>(row + uoff[j]);
@@ -260,7 +277,16 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
                 // share of cases, so a quantizer downstream sees the same input as the reference's
                 acc = __fdiv_rn(acc, 1.0f + (float)exp(-(double)acc)) * up;
             }
-            if (l == 0 && r < row_end) y[r] = acc;
+            if (MULTI) {
+                float *out = ma.y[0];
+                int first = 0;
+                if (r >= ma.first[1]) out = ma.y[1], first = ma.first[1];
+                if (r >= ma.first[2]) out = ma.y[2], first = ma.first[2];
+                if (r >= ma.first[3]) out = ma.y[3], first = ma.first[3];
+                if (l == 0 && r < row_end) out[r - first] = acc;
+            } else if (l == 0 && r < row_end) {
+                y[r] = acc;
+            }
         }
     }
 }
@@ -313,18 +339,20 @@ static FusedGeom fused_geom(size_t rows, int units, bool fused) {
     return g;
 }
 
-template <int MODE, bool GLU = false>
+template <int MODE, bool GLU = false, bool MULTI = false>
 static int launch_q4_k_fused(const frk_weights *w, const frk_weights *w2, const float *x, Q8KActs a, float *y,
-                             hipStream_t s) {
+                             hipStream_t s, size_t rows_total = 0, const MultiArgs *multi = nullptr) {
     const int nb = (int)(w->cols / QK_K);
-    FusedGeom g = fused_geom(w->rows, nb * 2, MODE == MODE_FUSED);
+    const size_t rows = MULTI ? rows_total : w->rows;
+    const MultiArgs ma = MULTI ? *multi : MultiArgs{};
+    FusedGeom g = fused_geom(rows, nb * 2, MODE == MODE_FUSED);
     const size_t shmem = MODE == MODE_PREQ_DIRECT ? 0 : (size_t)nb * (256 + 32 + 4);
     const int nwaves = g.threads / 64;
     const int xb = (nb + nwaves - 1) / nwaves;
 #define FRK_GO2(LPR, J, RPW, XB, MAXT)                                                                            \
-    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT, GLU>), dim3(g.grid), dim3(g.threads),   \
-                       shmem, s, w->dev, GLU ? w2->dev : nullptr, w->layout.row_stride, (int)w->rows, g.rows_per_wg, \
-                       nb, x, a.q, a.d, a.bsums, y)
+    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT, GLU, MULTI>), dim3(g.grid),          \
+                       dim3(g.threads), shmem, s, w->dev, GLU ? w2->dev : nullptr, w->layout.row_stride, (int)rows, \
+                       g.rows_per_wg, nb, x, a.q, a.d, a.bsums, y, ma)
 #define FRK_GO(LPR, J, RPW, MAXT)                                               \
     do {                                                                        \
         if (MODE == MODE_PREQ_DIRECT || xb <= 1) FRK_GO2(LPR, J, RPW, 1, MAXT); \
@@ -355,6 +383,20 @@ int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipSt
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
     if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, nullptr, a, y, s);
     return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, nullptr, a, y, s);
+}
+// ys[i] = ws[i] . x for 2..4 Q4_K matrices of one row length (fused_gemv_fits), one launch
+int launch_gemv_q4_k_group(const frk_weights *const *ws, size_t n, const float *x, float *const *ys, hipStream_t s) {
+    MultiArgs ma;
+    size_t total = 0;
+    for (size_t i = 0; i < 4; i++) {
+        const size_t j = i < n ? i : n - 1;
+        ma.W[i] = ws[j]->dev;
+        ma.y[i] = ys[j];
+        ma.first[i] = (int)total;
+        if (i < n) total += ws[i]->rows;
+    }
+    for (size_t i = n; i < 4; i++) ma.first[i] = (int)total;
+    return launch_q4_k_fused<MODE_FUSED, false, true>(ws[0], nullptr, x, Q8KActs{nullptr, nullptr, nullptr}, ys[0], s, total, &ma);
 }
 // act[r] = silu(gate[r] . x) * (up[r] . x): both matrices Q4_K of one shape, fused_gemv_fits
 int launch_gemv_q4_k_glu(const frk_weights *gate, const frk_weights *up, const float *x, float *act, hipStream_t s) {

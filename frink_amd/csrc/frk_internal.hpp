@@ -120,6 +120,7 @@ bool fused_gemv_fits(const frk_weights *w);
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 // gate and up in one launch: act[r] = silu(gate[r] . x) * (up[r] . x) (both Q4_K, one shape, fused_gemv_fits)
+int launch_gemv_q4_k_group(const frk_weights *const *ws, size_t n, const float *x, float *const *ys, hipStream_t s);
 int launch_gemv_q4_k_glu(const frk_weights *gate, const frk_weights *up, const float *x, float *act, hipStream_t s);
 // Q8_K activations in the form the matrix-core GEMMs stream: rows in tiles of 32 and, per
 // (tile, 256-wide block kb), one record that is exactly what a workgroup copies into LDS:

@@ -439,9 +439,20 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
                                   (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) || w->kind == FRK_KIND_Q8_0);
     }
     if (all_fused) {
-        for (size_t i = 0; i < n; i++) {
-            int rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
+        // Q4_K neighbours go out in one launch, four at most: the kernel walks their rows as one list
+        size_t i = 0;
+        while (i < n) {
+            size_t m = 1;
+            size_t rows = ws[i]->rows;
+            if (ws[i]->kind == FRK_KIND_Q4_K)
+                while (i + m < n && m < 4 && ws[i + m]->kind == FRK_KIND_Q4_K && rows + ws[i + m]->rows < (1u << 30)) {
+                    rows += ws[i + m]->rows;
+                    m++;
+                }
+            int rc = m > 1 ? launch_gemv_q4_k_group(ws + i, m, x, ys + i, s)
+                           : frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
             if (rc) return rc;
+            i += m;
         }
         return FRK_OK;
     }

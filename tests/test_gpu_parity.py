@@ -522,6 +522,28 @@ def test_gemv_multi_shares_one_quantized_activation(fa):
         w.release()
 
 
+@pytest.mark.parametrize("hidden,rows", [(4096, (4096, 1024, 1024)), (1024, (33, 7)), (2048, (100, 5, 64, 31, 9)),
+                                         (16384, (40, 24))])
+def test_gemv_multi_groups_q4_k_matrices_in_one_launch(fa, hidden, rows):
+    """q/k/v and other groups of Q4_K matrices (up to four per launch, a fifth starts the next): every
+    output equals, bit for bit, the lone GEMV of its matrix, and agrees with the oracle."""
+    from frink_amd import synth
+    print("gemv group", hidden, rows, flush=True)
+    datas = [make_weights(fo.Q4_K, r, hidden, seed=700 + i) for i, r in enumerate(rows)]
+    ws = [fa.Weights.from_host(fo.Q4_K, d, r, hidden) for r, d in zip(rows, datas)]
+    x = synth.activations(701, 1, hidden, outlier_frac=0.01)[0]
+    xd = to_dev(x)
+    ys = fa.gemv_multi(ws, xd)
+    for w, r, d, y in zip(ws, rows, datas, ys):
+        got = y.cpu().numpy()
+        assert got.shape == (r,)
+        assert np.array_equal(bits(got), bits(w.gemv(xd).cpu().numpy()))
+        if r <= 1024:
+            assert_rows_close(got[None], fo.gemv(fo.Q4_K, d, r, hidden, x)[None], "grouped gemv %d rows" % r)
+    for w in ws:
+        w.release()
+
+
 @pytest.mark.parametrize("hidden,ffn", [(512, 768), (4096, 14336)])
 def test_dense_ffn_swiglu(fa, hidden, ffn):
     """gate/up Q4_K, down Q6_K (the Llama-3-8B FFN at full size): each stage from the device's own
