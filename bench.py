@@ -173,7 +173,7 @@ def main():
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false, false>", "algorithmic_bytes": int(alg_bytes),
+                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false, false, false>", "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
     }
 
@@ -246,6 +246,21 @@ def main():
             "algorithmic_GBs": round(moe_bytes / (t / 100) / 1e9, 1),
             "frac_of_hbm_peak": round(moe_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4),
             "TOPS": round(2.0 * T * K * 3 * F * H / (t / 100) / 1e12, 1)}
+        # the same layer for ONE token (decode): 16 routings in turn that between them visit all 128
+        # experts once, so that no expert's weights are still cached when its turn comes again
+        perm = np.random.default_rng(11).permutation(E).astype(np.int32).reshape(16, 1, K)
+        ids1 = [torch.from_numpy(np.ascontiguousarray(p)).to(dev) for p in perm]
+        w1 = torch.full((1, K), 1.0 / K, dtype=torch.float32, device=dev)
+        x1 = xm[:1].contiguous()
+        y1 = torch.empty((1, H), dtype=torch.float32, device=dev)
+
+        def step4b(i):
+            fa.moe_ffn(experts[0], experts[1], experts[2], E, x1, ids1[i % 16], w1, out=y1)
+        _, t = time_graph(torch, step4b, 800, 16)
+        tok_bytes = K * 3 * F * H // 256 * 144
+        extra["MoE layer 128x top-8, 2048/768, 1 token (decode)"] = {
+            "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok_bytes / (t / 800) / 1e9, 1),
+            "frac_of_hbm_peak": round(tok_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
         for w in experts:
             w.release()
         # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call

@@ -257,6 +257,10 @@ def moe_ffn(gate, up, down, n_experts, x, ids, weights, out=None):
     return y
 
 
+# batches of at most this many tokens run per (token, slot) pair on the decode kernels (frk_internal.hpp)
+MOE_PER_TOKEN_MAX_BATCH = 16
+
+
 def moe_intermediates(batch, k, n_experts, hidden, ffn):
     """Test hook: (gate_out, up_out, act_q, act_d, pos_of) of the last moe_ffn call of this shape."""
     import torch

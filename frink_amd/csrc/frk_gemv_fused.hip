@@ -138,17 +138,47 @@ struct MultiArgs {
     const uint8_t *W[4];
     float *y[4];
     int first[4];  // unused entries hold the total
+    // INDEXED (below)
+    const int32_t *ids;
+    int n_experts;
+    int x_stride;
 };
-template <int LPR, int J, int RPW, int XB, int MODE, int MAXT, bool GLU = false, bool MULTI = false>
+// INDEXED: the expert projections of the per-token MoE path (run_expert / gate_up_projections,
+// crates/frink-moe/src/lib.rs:1068-1165): W (and W2) are stacks of n_experts matrices of `rows` rows
+// each; workgroup (_, job, sub) multiplies activation row `job` with expert ids[job*gridDim.z + sub]
+// and writes output row job*gridDim.z + sub.  Gate/up: job = token, sub = the token's slot, all slots
+// share the token's activation.  Down: job = (token, slot), gridDim.z = 1, every job its own.
+// (the plain kernel takes an empty struct in their place: a hundred bytes more of kernel arguments
+// cost the 14336x4096 GEMV 0.06 us)
+template <bool ANY>
+struct MultiArgsFor {
+    using type = MultiArgs;
+};
+template <>
+struct MultiArgsFor<false> {
+    struct type {};
+};
+template <int LPR, int J, int RPW, int XB, int MODE, int MAXT, bool GLU = false, bool MULTI = false, bool INDEXED = false>
 __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ W2, size_t row_stride, int rows, int rows_per_wg, int nb,
     const float *__restrict__ x, const int8_t *__restrict__ aq, const float *__restrict__ ad,
-    const int16_t *__restrict__ absums, float *__restrict__ y, MultiArgs ma) {
+    const int16_t *__restrict__ absums, float *__restrict__ y, typename MultiArgsFor<MULTI || INDEXED>::type ma_in) {
+    // (only the variants that have one look into it)
+    MultiArgs ma = {};
+    if constexpr (MULTI || INDEXED) ma = ma_in;
     extern __shared__ uint4 smem[];
     int8_t *sq = reinterpret_cast<int8_t *>(smem);
     int16_t *sbs = reinterpret_cast<int16_t *>(sq + nb * QK_K);
     float *sd = reinterpret_cast<float *>(sbs + nb * 16);
 
+    if (INDEXED) {
+        const int out_row = blockIdx.y * gridDim.z + blockIdx.z;
+        const int e = min(max(ma.ids[out_row], 0), ma.n_experts - 1);
+        W += (size_t)e * rows * row_stride;
+        if (GLU) W2 += (size_t)e * rows * row_stride;
+        x += (size_t)blockIdx.y * ma.x_stride;
+        y += (size_t)out_row * rows;
+    }
     constexpr int PARTS = 64 / LPR;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const int part = lane / LPR, l = lane % LPR;
@@ -339,20 +369,22 @@ static FusedGeom fused_geom(size_t rows, int units, bool fused) {
     return g;
 }
 
-template <int MODE, bool GLU = false, bool MULTI = false>
+template <int MODE, bool GLU = false, bool MULTI = false, bool INDEXED = false>
 static int launch_q4_k_fused(const frk_weights *w, const frk_weights *w2, const float *x, Q8KActs a, float *y,
-                             hipStream_t s, size_t rows_total = 0, const MultiArgs *multi = nullptr) {
+                             hipStream_t s, size_t rows_total = 0, const MultiArgs *multi = nullptr, unsigned jobs = 1,
+                             unsigned per_job = 1) {
     const int nb = (int)(w->cols / QK_K);
-    const size_t rows = MULTI ? rows_total : w->rows;
-    const MultiArgs ma = MULTI ? *multi : MultiArgs{};
+    const size_t rows = (MULTI || INDEXED) ? rows_total : w->rows;
+    typename MultiArgsFor<MULTI || INDEXED>::type ma;
+    if constexpr (MULTI || INDEXED) ma = *multi;
     FusedGeom g = fused_geom(rows, nb * 2, MODE == MODE_FUSED);
     const size_t shmem = MODE == MODE_PREQ_DIRECT ? 0 : (size_t)nb * (256 + 32 + 4);
     const int nwaves = g.threads / 64;
     const int xb = (nb + nwaves - 1) / nwaves;
 #define FRK_GO2(LPR, J, RPW, XB, MAXT)                                                                            \
-    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT, GLU, MULTI>), dim3(g.grid),          \
-                       dim3(g.threads), shmem, s, w->dev, GLU ? w2->dev : nullptr, w->layout.row_stride, (int)rows, \
-                       g.rows_per_wg, nb, x, a.q, a.d, a.bsums, y, ma)
+    hipLaunchKernelGGL((gemv_q4_k_fused_kernel<LPR, J, RPW, XB, MODE, MAXT, GLU, MULTI, INDEXED>),                \
+                       dim3(g.grid, jobs, per_job), dim3(g.threads), shmem, s, w->dev, GLU ? w2->dev : nullptr,      \
+                       w->layout.row_stride, (int)rows, g.rows_per_wg, nb, x, a.q, a.d, a.bsums, y, ma)
 #define FRK_GO(LPR, J, RPW, MAXT)                                               \
     do {                                                                        \
         if (MODE == MODE_PREQ_DIRECT || xb <= 1) FRK_GO2(LPR, J, RPW, 1, MAXT); \
@@ -374,7 +406,7 @@ static int launch_q4_k_fused(const frk_weights *w, const frk_weights *w2, const 
 bool fused_gemv_fits(const frk_weights *w) {
     // up to 4 half blocks per lane and 8 activation blocks per wavefront: rows of at most 64
     // blocks; wider rows take the generic kernels
-    return w->cols <= 16384;
+    return w->cols <= FUSED_GEMV_MAX_COLS;
 }
 
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
@@ -397,6 +429,19 @@ int launch_gemv_q4_k_group(const frk_weights *const *ws, size_t n, const float *
     }
     for (size_t i = n; i < 4; i++) ma.first[i] = (int)total;
     return launch_q4_k_fused<MODE_FUSED, false, true>(ws[0], nullptr, x, Q8KActs{nullptr, nullptr, nullptr}, ys[0], s, total, &ma);
+}
+// One launch for `jobs` activation rows against `per_job` experts each, out of a stack of n_experts
+// Q4_K matrices of rows_e rows (fused_gemv_fits): y[(job*per_job + sub)][rows_e]; with w2, silu(w.x)*(w2.x).
+int launch_gemv_q4_k_experts(const frk_weights *w, const frk_weights *w2, int n_experts, size_t rows_e, const float *x,
+                             size_t x_stride, const int32_t *ids, size_t jobs, size_t per_job, float *y, hipStream_t s) {
+    if (jobs > 65535 || per_job > 65535) return set_error(FRK_ERR_SHAPE, "%zu x %zu expert launches exceed the grid", jobs, per_job);
+    MultiArgs ma = {};
+    ma.ids = ids;
+    ma.n_experts = n_experts;
+    ma.x_stride = (int)x_stride;
+    const Q8KActs none = {nullptr, nullptr, nullptr};
+    if (w2) return launch_q4_k_fused<MODE_FUSED, true, false, true>(w, w2, x, none, y, s, rows_e, &ma, (unsigned)jobs, (unsigned)per_job);
+    return launch_q4_k_fused<MODE_FUSED, false, false, true>(w, nullptr, x, none, y, s, rows_e, &ma, (unsigned)jobs, (unsigned)per_job);
 }
 // act[r] = silu(gate[r] . x) * (up[r] . x): both matrices Q4_K of one shape, fused_gemv_fits
 int launch_gemv_q4_k_glu(const frk_weights *gate, const frk_weights *up, const float *x, float *act, hipStream_t s) {

@@ -269,7 +269,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
         const int mine = s_id[tid];
         int rank = 0;
         for (int j = 0; j < k; j++) rank += (s_id[j] < mine) || (s_id[j] == mine && j < tid);
-        s_pos[rank] = pos_of[(size_t)tok * k + tid];
+        s_pos[rank] = pos_of ? pos_of[(size_t)tok * k + tid] : tok * k + tid;  // (no map: rows in pair order)
         s_w[rank] = weights[(size_t)tok * k + tid];
     }
     __syncthreads();
@@ -384,6 +384,30 @@ int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hid
     return FRK_OK;
 }
 
+// The per-token path (cpu_moe_topk_parallel_slots / run_expert, crates/frink-models/src/decoder/
+// moe_host.rs:102-203, crates/frink-moe/src/lib.rs:1068-1165): with a token or a few, every (token,
+// slot) pair reads its expert's three matrices alone, so the layer is three launches of decode
+// kernels -- gate, up and silu(g)*u of all pairs; down of all pairs, each quantizing its own
+// intermediate; the weighted sum in ascending expert id -- instead of the six of the grouped path.
+bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn) {
+    return batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS && ffn <= FUSED_GEMV_MAX_COLS;
+}
+static int launch_moe_ffn_per_token(const frk_weights *gate, const frk_weights *up, const frk_weights *down,
+                                    int n_experts, const float *x, size_t batch, const int32_t *ids,
+                                    const float *weights, int k, float *out, const MoeScratch &m, hipStream_t s) {
+    const int hidden = (int)gate->cols, ffn = (int)down->cols;
+    float *act = m.gate_out;  // [batch*k][ffn]
+    int rc = launch_gemv_q4_k_experts(gate, up, n_experts, (size_t)ffn, x, (size_t)hidden, ids, batch, (size_t)k, act, s);
+    if (rc) return rc;
+    rc = launch_gemv_q4_k_experts(down, nullptr, n_experts, (size_t)hidden, act, (size_t)ffn, ids, batch * (size_t)k, 1,
+                                  m.down_out, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights,
+                       (const int *)nullptr, k, hidden, out);
+    FRK_LAUNCH_CHECK("moe_combine");
+    return FRK_OK;
+}
+
 int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
                    const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
                    void *ws, hipStream_t s) {
@@ -391,6 +415,8 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts);
     const MoeScratch m = moe_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
     const int max_tiles = (int)(rows / MOE_TILE);
+    if (moe_takes_per_token_path(batch, (size_t)hidden, (size_t)ffn))
+        return launch_moe_ffn_per_token(gate, up, down, n_experts, x, batch, ids, weights, k, out, m, s);
 
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {

@@ -551,6 +551,8 @@ int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size
     clear_error();
     if (batch == 0 || k == 0 || n_experts == 0 || hidden == 0 || ffn == 0)
         return set_error(FRK_ERR_SHAPE, "frk_hip_moe_intermediates_dev: empty shape");
+    if (moe_takes_per_token_path(batch, hidden, ffn))
+        return set_error(FRK_ERR_UNSUPPORTED, "a batch of %zu runs per token and keeps no grouped intermediates", batch);
     void *ws = nullptr;
     int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);
     if (rc) return rc;

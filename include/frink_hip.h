@@ -201,7 +201,8 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
  * (null = skip): the gate and up projections [batch*k][ffn], silu(gate)*up quantized to Q8_K
  * (act_q [batch*k][ffn] i8, act_d [batch*k][ffn/256] f32), rows in grouped order, and
  * pos_of[tok*k + slot] = the row of a (token, slot) pair (the reference's bucket order,
- * crates/frink-models/src/decoder/ffn_batch.rs:362-386). */
+ * crates/frink-models/src/decoder/ffn_batch.rs:362-386).  FRK_ERR_UNSUPPORTED for the small batches
+ * (at most 16 tokens) that run per (token, slot) pair on the decode kernels: they have no grouped order. */
 int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size_t hidden, size_t ffn,
                                   float *gate_out_dev, float *up_out_dev, int8_t *act_q_dev,
                                   float *act_d_dev, int32_t *pos_of_dev, void *stream);

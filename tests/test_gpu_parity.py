@@ -371,6 +371,10 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     wu = fa.Weights.from_host(fo.Q4_K, up, n_experts * ffn, hidden)
     wd = fa.Weights.from_host(fo.Q4_K, down, n_experts * hidden, ffn)
     got = fa.moe_ffn(wg, wu, wd, n_experts, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    if batch <= fa.MOE_PER_TOKEN_MAX_BATCH:
+        for h in (wg, wu, wd):
+            h.release()
+        return _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, batch, x, ids, w)
     g_out, u_out, act_q, act_d, pos = (t.cpu().numpy() for t in fa.moe_intermediates(batch, k, n_experts, hidden, ffn))
     for h in (wg, wu, wd):
         h.release()
@@ -404,11 +408,52 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     return got, want
 
 
+def _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, batch, x, ids, w):
+    """A token or a few run per (token, slot) pair on the decode kernels.  Each pair is then the dense
+    SwiGLU FFN of its expert's three matrices -- the very kernels, so the layer must equal, bit for
+    bit, the library's own frk_hip_ffn_swiglu_dev on the expert's slices summed in ascending expert id
+    (that FFN is gated against the oracle in test_dense_ffn_swiglu and the GEMV tests) -- and end to
+    end it must agree with moe_ffn_batch like the grouped path."""
+    with pytest.raises(fa.BackendError) as e:
+        fa.moe_intermediates(batch, k, n_experts, hidden, ffn)
+    assert e.value.code == fa.ERR_UNSUPPORTED
+    gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
+    composed = np.zeros((batch, hidden), np.float32)
+    cache = {}
+    for t in range(batch):
+        xd = to_dev(x[t])
+        for s in sorted(range(k), key=lambda s: (int(ids[t, s]), s)):
+            ex = int(ids[t, s])
+            if ex not in cache:
+                cache[ex] = (fa.Weights.from_host(fo.Q4_K, gb[ex], ffn, hidden), fa.Weights.from_host(fo.Q4_K, ub[ex], ffn, hidden),
+                             fa.Weights.from_host(fo.Q4_K, db[ex], hidden, ffn))
+            ge, ue, de = cache[ex]
+            y = fa.ffn_swiglu(ge, ue, de, xd).cpu().numpy()
+            composed[t] = composed[t] + np.float32(w[t, s]) * y
+    for hs in cache.values():
+        for h in hs:
+            h.release()
+    assert np.array_equal(bits(got), bits(composed)), np.abs(got - composed).max()
+    want = fo.moe_ffn_batch(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
+    print("moe per token end-to-end: worst %.3g" % rel.max(), flush=True)
+    assert (rel <= TOL).mean() >= 0.5 and rel.max() <= 10 * TOL, rel.max()
+    return got, want
+
+
+@pytest.mark.parametrize("n_experts,k,hidden,ffn,batch", [
+    (16, 4, 512, 768, 1), (8, 8, 256, 256, 2), (64, 6, 1024, 512, 4), (4, 1, 2048, 256, 3), (128, 8, 2048, 768, 1),
+    (32, 4, 512, 512, 16),
+])
+def test_moe_ffn_of_a_few_tokens_runs_per_token(fa, n_experts, k, hidden, ffn, batch):
+    _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 10 + batch, random_blocks=n_experts >= 64)
+
+
 @pytest.mark.parametrize("n_experts,k,hidden,ffn,batch", [
     (8, 2, 512, 256, 40),     # a few experts hold more than one 32-row tile
     (16, 4, 256, 512, 70),
     (4, 4, 256, 256, 33),     # every token visits every expert: 33 rows -> tiles of 32 + 1
-    (32, 2, 256, 256, 1),     # one token, most experts idle
+    (32, 2, 256, 256, 17),    # just above the batches that run per token: most experts idle
 ])
 def test_moe_ffn_matches_the_oracle(fa, n_experts, k, hidden, ffn, batch):
     _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 100 + batch)
