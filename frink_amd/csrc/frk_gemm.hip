@@ -150,52 +150,68 @@ __device__ __forceinline__ void wait_vm() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// raw block -> operand planes.  lg = lane / 32 selects which half of every sub-block this lane holds.
-__device__ __forceinline__ void unpack_block(const RawBlock &R, int lg, BPlanes &B) {
-    const uint32_t hx = (uint32_t)R.wh.x, hy = (uint32_t)R.wh.y, hz = (uint32_t)R.wh.z, hw = (uint32_t)R.wh.w;
-    const uint32_t sc_lo = hy & 0x3f3f3f3fu, m_lo = hz & 0x3f3f3f3fu;
-    const uint32_t sc_hi = (hw & 0x0f0f0f0fu) | (((hy >> 6) & 0x03030303u) << 4);
-    const uint32_t m_hi = ((hw >> 4) & 0x0f0f0f0fu) | (((hz >> 6) & 0x03030303u) << 4);
-    // one nibble pair: 16 bytes -> the lane's H and L operands of sub-blocks 2p and 2p+1
-    auto pair = [&](const v4i q, const uint32_t scw, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
-        const uint32_t s0 = scw & 0xff, s1 = (scw >> 8) & 0xff;
-        const us2 h0 = {(unsigned short)(s0 >> 3), (unsigned short)(s0 >> 3)};
-        const us2 l0 = {(unsigned short)(s0 & 7), (unsigned short)(s0 & 7)};
-        const us2 h1 = {(unsigned short)(s1 >> 3), (unsigned short)(s1 >> 3)};
-        const us2 l1 = {(unsigned short)(s1 & 7), (unsigned short)(s1 & 7)};
-        auto one = [&](const int wi, int &o0, int &o1, int &o2, int &o3) {
-            const uint32_t w = (uint32_t)wi;
-            const uint32_t nl = w & 0x0f0f0f0fu, nh = (w >> 4) & 0x0f0f0f0fu;
-            us2 a, b;
-            __builtin_memcpy(&a, &nl, 4);
-            __builtin_memcpy(&b, &nh, 4);
-            const us2 r0 = a * h0, r1 = a * l0, r2 = b * h1, r3 = b * l1;  // bytes stay below 106
-            __builtin_memcpy(&o0, &r0, 4);
-            __builtin_memcpy(&o1, &r1, 4);
-            __builtin_memcpy(&o2, &r2, 4);
-            __builtin_memcpy(&o3, &r3, 4);
-        };
-        int a0, a1, a2, a3, b0, b1, b2, b3, c0, c1, c2, c3, d0, d1, d2, d3;
-        one(q.x, a0, a1, a2, a3);
-        one(q.y, b0, b1, b2, b3);
-        one(q.z, c0, c1, c2, c3);
-        one(q.w, d0, d1, d2, d3);
-        H0 = v4i{a0, b0, c0, d0};  // sub-block 2p: low nibbles
-        L0 = v4i{a1, b1, c1, d1};
-        H1 = v4i{a2, b2, c2, d2};  // sub-block 2p+1: high nibbles
-        L1 = v4i{a3, b3, c3, d3};
+// raw block -> operand planes, in pieces (so that a caller can spread them between other work):
+// the 6-bit scales and mins, one nibble pair at a time, the rest.  lg = lane / 32 selects which half
+// of every sub-block this lane holds.
+struct BlockScales {
+    uint32_t sc_lo, sc_hi, m_lo, m_hi;  // a byte per sub-block: 0..3 and 4..7
+};
+__device__ __forceinline__ BlockScales block_scales(const RawBlock &R) {
+    const uint32_t hy = (uint32_t)R.wh.y, hz = (uint32_t)R.wh.z, hw = (uint32_t)R.wh.w;
+    BlockScales s;
+    s.sc_lo = hy & 0x3f3f3f3fu;
+    s.m_lo = hz & 0x3f3f3f3fu;
+    s.sc_hi = (hw & 0x0f0f0f0fu) | (((hy >> 6) & 0x03030303u) << 4);
+    s.m_hi = ((hw >> 4) & 0x0f0f0f0fu) | (((hz >> 6) & 0x03030303u) << 4);
+    return s;
+}
+// one nibble pair: 16 bytes -> the lane's H and L operands of sub-blocks 2p (low nibbles) and 2p+1
+// (high nibbles); scw holds their two scales in its low bytes
+__device__ __forceinline__ void unpack_pair(const v4i q, const uint32_t scw, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
+    const uint32_t s0 = scw & 0xff, s1 = (scw >> 8) & 0xff;
+    const us2 h0 = {(unsigned short)(s0 >> 3), (unsigned short)(s0 >> 3)};
+    const us2 l0 = {(unsigned short)(s0 & 7), (unsigned short)(s0 & 7)};
+    const us2 h1 = {(unsigned short)(s1 >> 3), (unsigned short)(s1 >> 3)};
+    const us2 l1 = {(unsigned short)(s1 & 7), (unsigned short)(s1 & 7)};
+    auto one = [&](const int wi, int &o0, int &o1, int &o2, int &o3) {
+        const uint32_t w = (uint32_t)wi;
+        const uint32_t nl = w & 0x0f0f0f0fu, nh = (w >> 4) & 0x0f0f0f0fu;
+        us2 a, b;
+        __builtin_memcpy(&a, &nl, 4);
+        __builtin_memcpy(&b, &nh, 4);
+        const us2 r0 = a * h0, r1 = a * l0, r2 = b * h1, r3 = b * l1;  // bytes stay below 106
+        __builtin_memcpy(&o0, &r0, 4);
+        __builtin_memcpy(&o1, &r1, 4);
+        __builtin_memcpy(&o2, &r2, 4);
+        __builtin_memcpy(&o3, &r3, 4);
     };
-    pair(R.q0, sc_lo, B.H0, B.L0, B.H1, B.L1);
-    pair(R.q1, sc_lo >> 16, B.H2, B.L2, B.H3, B.L3);
-    pair(R.q2, sc_hi, B.H4, B.L4, B.H5, B.L5);
-    pair(R.q3, sc_hi >> 16, B.H6, B.L6, B.H7, B.L7);
+    int a0, a1, a2, a3, b0, b1, b2, b3, c0, c1, c2, c3, d0, d1, d2, d3;
+    one(q.x, a0, a1, a2, a3);
+    one(q.y, b0, b1, b2, b3);
+    one(q.z, c0, c1, c2, c3);
+    one(q.w, d0, d1, d2, d3);
+    H0 = v4i{a0, b0, c0, d0};
+    L0 = v4i{a1, b1, c1, d1};
+    H1 = v4i{a2, b2, c2, d2};
+    L1 = v4i{a3, b3, c3, d3};
+}
+__device__ __forceinline__ void unpack_rest(const RawBlock &R, const BlockScales &s, int lg, BPlanes &B) {
     // mins of the four sub-blocks whose 16-wide groups are 8*lg .. 8*lg+7, each twice
-    const uint32_t mw = lg ? m_hi : m_lo;
+    const uint32_t hx = (uint32_t)R.wh.x;
+    const uint32_t mw = lg ? s.m_hi : s.m_lo;
     const _Float16 m0 = (_Float16)(int)(mw & 0xff), m1 = (_Float16)(int)((mw >> 8) & 0xff);
     const _Float16 m2 = (_Float16)(int)((mw >> 16) & 0xff), m3 = (_Float16)(int)(mw >> 24);
     B.m = v8h{m0, m0, m1, m1, m2, m2, m3, m3};
     B.d = h2f(hx & 0xffffu);
     B.ndmin = -h2f(hx >> 16);
+}
+__device__ __forceinline__ void unpack_block(const RawBlock &R, int lg, BPlanes &B) {
+    const BlockScales s = block_scales(R);
+    unpack_pair(R.q0, s.sc_lo, B.H0, B.L0, B.H1, B.L1);
+    unpack_pair(R.q1, s.sc_lo >> 16, B.H2, B.L2, B.H3, B.L3);
+    unpack_pair(R.q2, s.sc_hi, B.H4, B.L4, B.H5, B.L5);
+    unpack_pair(R.q3, s.sc_hi >> 16, B.H6, B.L6, B.H7, B.L7);
+    unpack_rest(R, s, lg, B);
 }
 
 __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales &S, const BPlanes &B, v16f &acc) {
@@ -216,35 +232,57 @@ __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales
 // that the MFMAs are free to sink below all the waits, and the chain starts only when the last
 // operand is there.)
 #define FRK_WAIT_LGKM(n, reg, acc) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(reg), "+v"(acc))
-__device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const BPlanes &B, TileAcc &X) {
+// between(i, acc) is called after MFMA i of the integer chain has been issued, i = 0..14: what it does
+// shares the gaps of the chain, every MFMA of which waits for the one before it.
+struct NothingBetween {
+    __device__ __forceinline__ void operator()(int, v16i &) const {}
+};
+template <class Between = NothingBetween>
+__device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const BPlanes &B, TileAcc &X,
+                                                        Between between = Between()) {
     const v16i zi = {0};
     const v16f zf = {0.0f};
     asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
     v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    between(0, acc);
     FRK_WAIT_LGKM(7, T.a1, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    between(1, acc);
     FRK_WAIT_LGKM(6, T.a2, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    between(2, acc);
     FRK_WAIT_LGKM(5, T.a3, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    between(3, acc);
     FRK_WAIT_LGKM(4, T.a4, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    between(4, acc);
     FRK_WAIT_LGKM(3, T.a5, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    between(5, acc);
     FRK_WAIT_LGKM(2, T.a6, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    between(6, acc);
     FRK_WAIT_LGKM(1, T.a7, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    between(7, acc);
     FRK_WAIT_LGKM(0, T.bs, acc);
     X.s2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, zf, 0, 0, 0);
     acc = acc << 3;
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    between(8, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    between(9, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    between(10, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    between(11, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    between(12, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    between(13, acc);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    between(14, acc);
     X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
 }
 
@@ -260,11 +298,6 @@ __device__ __forceinline__ void fold_mins(BPlanes &B) {
     B.ndmin = z ? 1.0f : B.ndmin;
     if (z) B.m = v8h{0, 0, 0, 0, 0, 0, 0, 0};
 }
-// between(i, acc) is called after MFMA i has been issued, i = 0..15: what it issues (the prefetch)
-// shares the gaps of the chain, every MFMA of which waits for the one before it.
-struct NothingBetween {
-    __device__ __forceinline__ void operator()(int, v16i &) const {}
-};
 template <class Between = NothingBetween>
 __device__ __forceinline__ v16f tile_mfmas_folded(TileOperands &T, const BPlanes &B, Between between = Between()) {
     const v16i zi = {0};
@@ -557,19 +590,18 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
         }
 }
 
-// The grouped (per-expert) GEMM for tiles of at most 32 activation rows: with so few rows per
-// expert the work is a stream over the experts' weights, bound by HBM, and what matters is that the
-// stream never stops.  Persistent workgroups (one per CU, 8 wavefronts, 256 weight rows) walk a list
-// of work items (tile, matrix, row group); one step = one 256-wide block of one item.  A step's data
-// travels into LDS two steps ahead, across item boundaries: the weights (a wavefront fetches and
-// reads only its own 32 rows, so that ring needs no barrier and a stage is refilled as soon as it
-// has been unpacked: two stages are two steps of distance) and the tile's activation record (shared,
-// four stages, one barrier per step).  A tile is up to 64 activation rows, two 32-row halves that
-// share the unpacked weights; the second half is neither fetched nor multiplied when not in use.
-// The two wavefronts of a SIMD (w and w+4) run half a step apart: the leading one unpacks step s
-// and then runs its MFMAs and epilogue; the lagging one runs the MFMAs and epilogue of step s-1
-// first and unpacks step s after them.  One's vector-ALU phase then faces the other's matrix phase
-// instead of both waiting for LDS, multiplying and scaling in lockstep behind the barrier.
+// The grouped (per-expert) GEMM: with a few dozen activation rows per expert the work is a stream
+// over the experts' weights.  Persistent workgroups (one per CU, 8 wavefronts, 256 weight rows) walk
+// a list of work items (tile, matrix, row group); one step = one 256-wide block of one item.  A
+// step's data travels into LDS three steps ahead, across item boundaries: the weights (a wavefront
+// fetches and reads only its own 32 rows, so that ring needs no barrier: two stages, each refilled as
+// soon as its block has left it for the registers) and the tile's activation record (shared, four
+// stages, one barrier per step).  A tile is up to 64 activation rows, two 32-row halves that share
+// the unpacked weights; the second half is neither fetched nor multiplied when not in use.
+// The unpacked weights are double-buffered in registers: step s+1 is unpacked from inside the chain
+// of MFMAs of step s.  The two wavefronts of a SIMD (w and w+4) issue their loads at different
+// times, one before its MFMAs and one after: a wavefront is stalled while its loads wait for the
+// CU's address unit, and this way the other one has the matrix core meanwhile.
 // Items of a tile sit on one XCD (block id mod 8), whose L2 then serves the tile's activations.
 struct StreamLds {
     static constexpr int RG = 8;
@@ -597,7 +629,6 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lg = lane >> 5;
     const int nb = g.nb;
-    const bool lagging = wave >= L::RG / 2;
 
     // this workgroup's items: the list of its XCD holds the tiles t = xcd (mod 8), every (matrix, row
     // group) of a tile in a row; the XCD's workgroups take list entries slot, slot + per_xcd, ...
@@ -634,7 +665,7 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         count = __builtin_amdgcn_readfirstlane(v.y);
     };
 
-    // ---- the fetch side: a cursor (item, block) two steps ahead of the arithmetic ----
+    // ---- the fetch side: a cursor (item, block) three steps ahead of the arithmetic ----
     // weights of a step: this wavefront's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of
     // chunk c (4.5 chunks, 5 loads); activations: quant slice `wave`, plus the sums (wavefront 0) or
     // the scales (wavefront 1).  Addresses are a uniform base that moves with the cursor plus a lane
@@ -654,6 +685,7 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
     const int8_t *f_q;
     int f_ord = 0, f_kb = 0, f_step = 0;
     bool f_two = false;  // the cursor's tile has rows in its second half
+    int issued = 0;      // loads of the fetch most recently issued by this wavefront
     auto point_at = [&](int ord) {  // uniform
         int t, m, rg, expert, count;
         item_of(ord, t, m, rg);
@@ -673,13 +705,16 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         const uint32_t q_off = (uint32_t)(wave * 1024 + l * 16);
         const uint32_t x_off = x_sums ? (uint32_t)l * 16 : (uint32_t)(l & 31) * 4;
         load_to_lds16(f_q + q_off, st + wave * 1024);
+        issued = 1;
         if (f_two) {
             load_to_lds16(f_q + (size_t)nb * 8192 + q_off, st + L::A_HALF + wave * 1024);
+            issued = 2;
         }
         if (wave < 2 || (wave < 4 && f_two)) {
             uint8_t *half = st + (wave >> 1) * L::A_HALF;
             if (x_sums) load_to_lds16(f_x + x_off, half + L::A_BS);
             else load_to_lds4(f_x + x_off, half + L::A_DA);  // both lane halves fetch the same 32 scales
+            issued++;
         }
     };
     auto fetch_weights = [&]() {  // of the cursor's step; moves the cursor on
@@ -693,6 +728,7 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
             const uint32_t off = w_off0 + c * (7 * stride + 16) + (r0 + c >= 9 ? stride - Q4_K_BYTES : 0u);
             if (c < 4 || l < 32) load_to_lds16(f_w + min(off, last), st + c * 1024);
         }
+        issued += 5;
         f_step++;
         f_w += Q4_K_BYTES;
         f_q += 8192;
@@ -702,6 +738,7 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
             if (++f_ord < my_items) point_at(f_ord);
         }
     };
+    // prologue: the data of steps 0 and 1
     point_at(0);
     fetch_acts();
     fetch_weights();
@@ -712,31 +749,32 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
     wait_vm<0>();
     lds_barrier();
 
-    // ---- the arithmetic: the whole loop once per role (one copy serving both roles needs more
-    // registers than there are) ----
+    // ---- the arithmetic.  The unpacked weights are double-buffered in registers: while step s is
+    // multiplied out of one set, step s+1 is unpacked into the other, the unpacking's vector
+    // instructions filling the gaps between the MFMAs, each of which waits for the one before it.
+    // (Every wavefront overlaps its own two kinds of work, so the wavefronts of a SIMD need not
+    // be kept in different phases.)  The loop body exists twice, one copy per set. ----
     const uint32_t lds0 = lds_address(lds);
-    auto run = [&](auto role) {
-    constexpr bool LAGGING = decltype(role)::value;
-    BPlanes B;
+    BPlanes B0, B1;
     v16f accF0 = v16f{0.0f}, accF1 = v16f{0.0f};  // the tile's two halves
+    const bool fetch_late = wave >= L::RG / 2;
     int c_ord = 0, c_kb = 0, c_count = 0;
     int pending = -1, pending_count = 0;  // item whose results wait to be stored
-    auto unpack_step = [&](int s) {
+    auto raw_of_step = [&](int s) {  // this lane's part of its row's block, read and arrived
         const int l = opaque_lane(), li = l & 31, lg = l >> 5;
         const uint32_t wa = lds0 + (s & 1) * L::W_STAGE + (wave * 32 + li) * Q4_K_BYTES;
         RawBlock R;
         read_raw(R, wa, wa + 16 * lg);
         wait_raw<0>(R);
-        unpack_block(R, lg, B);
-        __builtin_amdgcn_sched_barrier(0);  // keep the phases' registers apart
+        return R;
     };
-    auto multiply_half = [&](uint32_t st, v16f &accF) {
+    auto multiply_half = [&](uint32_t st, v16f &accF, const BPlanes &B, auto between) {
         const int lane = opaque_lane(), lg = lane >> 5;
         TileOperands T;
         TileScales S;
         TileAcc X;
         read_ops(T, st + lane * 16, st + L::A_BS + lane * 16);
-        tile_mfmas_as_they_land(T, B, X);
+        tile_mfmas_as_they_land(T, B, X, between);
         read_scales(S, st + L::A_DA + lg * 16);
         wait_scales<0>(S);
         tile_epilogue(X, S, B, accF);
@@ -745,14 +783,23 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         // keeps its place among the volatile LDS reads
         asm volatile("" : "+v"(accF));
     };
-    auto multiply_step = [&](int s) {
+    // (the next step's block R is unpacked into Bnext from inside the first half's chain of MFMAs)
+    auto multiply_step = [&](int s, const BPlanes &B, const RawBlock &R, BPlanes &Bnext) {
         const uint32_t st = lds0 + L::OFF_A + (s & 3) * L::A_STAGE;
         if (c_kb == 0) {
             int expert;
             item_info(c_ord, expert, c_count);
         }
-        multiply_half(st, accF0);
-        if (c_count > 32) multiply_half(st + L::A_HALF, accF1);
+        const BlockScales sc = block_scales(R);
+        const int lg_next = opaque_lane() >> 5;
+        multiply_half(st, accF0, B, [&](int i, v16i &) {
+            if (i == 0) unpack_pair(R.q0, sc.sc_lo, Bnext.H0, Bnext.L0, Bnext.H1, Bnext.L1);
+            if (i == 2) unpack_pair(R.q1, sc.sc_lo >> 16, Bnext.H2, Bnext.L2, Bnext.H3, Bnext.L3);
+            if (i == 4) unpack_pair(R.q2, sc.sc_hi, Bnext.H4, Bnext.L4, Bnext.H5, Bnext.L5);
+            if (i == 6) unpack_pair(R.q3, sc.sc_hi >> 16, Bnext.H6, Bnext.L6, Bnext.H7, Bnext.L7);
+            if (i == 8) unpack_rest(R, sc, lg_next, Bnext);
+        });
+        if (c_count > 32) multiply_half(st + L::A_HALF, accF1, B, NothingBetween());
         if (++c_kb == nb) {
             pending = c_ord++;
             pending_count = c_count;
@@ -786,36 +833,49 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         }
     };
 
-    for (int s = 0; s <= total_steps; s++) {
+    {  // step 0's weights into the first set; its stage is refilled at once
+        const RawBlock R = raw_of_step(0);
+        unpack_block(R, lg, B0);
+        if (total_steps > 2) {
+            fetch_acts();
+            fetch_weights();
+        }
+    }
+    auto step = [&](int s, const BPlanes &Bcur, BPlanes &Bnext) {
         if (pending >= 0) {
             store_item(pending);
             pending = -1;
         }
-        const bool more = s + 2 < total_steps;
-        if (more) fetch_acts();  // the stage was last read (by the lagging wavefronts) in step s-1
-        if (!LAGGING) {
-            if (s < total_steps) {
-                unpack_step(s);
-                if (more) fetch_weights();  // into the stage just unpacked
-                multiply_step(s);
-            }
-        } else {
-            if (s > 0) multiply_step(s - 1);
-            if (s < total_steps) {
-                unpack_step(s);
-                if (more) fetch_weights();
-            }
+        // step s+1's raw weights leave LDS, which frees their stage for step s+3 (past the last step:
+        // whatever the stage holds, unpacked into a set nobody will use)
+        const RawBlock R = raw_of_step(s + 1);
+        // A wavefront is stalled while its loads wait for the CU's one address unit (600 clocks for
+        // the first four wavefronts that ask, 1700 for the other four): so half of the wavefronts,
+        // one of every SIMD's two, fetch before they multiply and half after, and the unit serves
+        // the one half while the other half has the matrix cores.
+        const bool more = s + 3 < total_steps;
+        if (more && !fetch_late) {
+            fetch_acts();  // (into the stage last read in step s-1)
+            fetch_weights();
         }
-        // Everything requested has landed before the step ends, the data of step s+2 included: it had
-        // the whole step.  (Letting that newest request stay in flight, "all but the newest n", was
-        // measured 7 % slower: memory latency is not what a step waits for.)
-        wait_vm<0>();
+        multiply_step(s, Bcur, R, Bnext);
+        if (more && fetch_late) {
+            fetch_acts();
+            fetch_weights();
+        }
+        // steps s+1 and s+2 must have landed; the request just made (step s+3, the `issued` youngest
+        // loads; a finished item's stores are older) may stay in flight
+        if (!more) wait_vm<0>();
+        else if (issued == 6) wait_vm<6>();
+        else if (issued == 7) wait_vm<7>();
+        else wait_vm<8>();
         lds_barrier();
+    };
+    for (int s = 0; s < total_steps; s += 2) {
+        step(s, B0, B1);
+        if (s + 1 < total_steps) step(s + 1, B1, B0);
     }
     if (pending >= 0) store_item(pending);
-    };
-    if (lagging) run(std::true_type{});
-    else run(std::false_type{});
 }
 
 // ------------------------------------------------------------------ launchers
