@@ -25,6 +25,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA
 COPIES = 16
+# steps captured per HIP graph in the two timed loops of the headline (a multiple of COPIES): a graph
+# replay starts with a few microseconds of nothing, which 400 steps dilute and 16 would not
+GRAPH_STEPS = 400
 # HBM bytes per launch of the roofline kernel at 14336x4096, from two rocprofv3 --pmc runs of this
 # script (FETCH_SIZE 16163.5, WRITE_SIZE 56.0 per dispatch), each scaled by what the same counter
 # reads for copy_kernel over 32,256 KiB (FETCH_SIZE 16138.0 -> x1.9988, WRITE_SIZE 32256.0 -> x1.0).
@@ -53,8 +56,9 @@ def random_blocks(kind, rows, cols, seed):
 
 
 def time_graph(torch, fn_steps, n_steps, copies):
-    """Captures `copies` consecutive steps in one HIP graph and replays it; returns seconds for
-    exactly n_steps steps (a second, shorter graph runs the remainder)."""
+    """Captures `copies` consecutive steps in one HIP graph (fn_steps(i) chooses its operands by i
+    modulo whatever it rotates over) and replays it; returns seconds for exactly n_steps steps (a
+    second, shorter graph runs the remainder)."""
     stream = torch.cuda.Stream()
     graphs = []
     with torch.cuda.stream(stream):
@@ -144,7 +148,7 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    wall, ev = time_graph(torch, step, args.steps, COPIES)
+    wall, ev = time_graph(torch, step, args.steps, GRAPH_STEPS)
     sec_per_step = ev / args.steps
     wbytes = data.size
     value = wbytes / sec_per_step / 1e9
@@ -156,7 +160,7 @@ def main():
         ws[i % COPIES].gemv_q8k(acts, out=y)
 
     n_k = max(COPIES * 8, min(args.steps, 4000))
-    _, ev_k = time_graph(torch, gemv_only, n_k, COPIES)
+    _, ev_k = time_graph(torch, gemv_only, n_k, GRAPH_STEPS)
     k_sec = ev_k / n_k
     alg_bytes = wbytes + cols + cols // 256 * 4 + cols // 16 * 2 + rows * 4  # W + Q8_K activation + y
     achieved = alg_bytes / k_sec / 1e9
@@ -192,9 +196,9 @@ def main():
         def copy(i):
             fa.check(L.frk_hip_copy_dev(C.c_void_p(src[i % COPIES].data_ptr()), C.c_void_p(dst.data_ptr()), wbytes,
                                         fa._stream()))
-        _, t = time_graph(torch, read_only, 800, COPIES)
+        _, t = time_graph(torch, read_only, 800, GRAPH_STEPS)
         extra["read_only_stream_33MB_GBs"] = round(wbytes / (t / 800) / 1e9, 1)
-        _, t = time_graph(torch, copy, 800, COPIES)
+        _, t = time_graph(torch, copy, 800, GRAPH_STEPS)
         extra["copy_33MB_read_plus_write_GBs"] = round(2 * wbytes / (t / 800) / 1e9, 1)
         del src, dst
         for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
@@ -207,7 +211,7 @@ def main():
 
             def step2(i):
                 w2[i % n_copies].gemv(x2, out=y2)
-            _, t = time_graph(torch, step2, 1600, n_copies)
+            _, t = time_graph(torch, step2, 1600, 25 * n_copies)
             extra[name] = {"GBs": round(d2.numel() / (t / 1600) / 1e9, 1), "us_per_step": round(t / 1600 * 1e6, 3),
                            "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
             for w in w2:
@@ -222,7 +226,7 @@ def main():
 
             def step3(i):
                 w2[i % 4].gemm(xb, out=yb)
-            _, t = time_graph(torch, step3, 200, 4)
+            _, t = time_graph(torch, step3, 200, 100)
             tops = 2.0 * 512 * r2 * cols / (t / 200) / 1e12
             extra[name] = {"TOPS": round(tops, 1), "us_per_step": round(t / 200 * 1e6, 2),
                            "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
@@ -239,7 +243,7 @@ def main():
 
         def step4(i):
             fa.moe_ffn(experts[0], experts[1], experts[2], E, xm, ids, wts, out=ym)
-        _, t = time_graph(torch, step4, 100, 2)
+        _, t = time_graph(torch, step4, 100, 50)
         moe_bytes = 3 * E * F * H // 256 * 144 + 2 * T * H * 4 + 2 * T * K * 4
         extra["MoE layer 128x top-8, 2048/768, 512 tokens"] = {
             "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
@@ -256,7 +260,7 @@ def main():
 
         def step4b(i):
             fa.moe_ffn(experts[0], experts[1], experts[2], E, x1, ids1[i % 16], w1, out=y1)
-        _, t = time_graph(torch, step4b, 800, 16)
+        _, t = time_graph(torch, step4b, 800, 400)
         tok_bytes = K * 3 * F * H // 256 * 144
         extra["MoE layer 128x top-8, 2048/768, 1 token (decode)"] = {
             "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok_bytes / (t / 800) / 1e9, 1),
@@ -277,7 +281,7 @@ def main():
                                       ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8)):
             def step5(i, mats=mats, xin=xin, yout=yout):
                 mats[i % 8].gemm(xin, out=yout)
-            _, t = time_graph(torch, step5, 400, 8)
+            _, t = time_graph(torch, step5, 400, 200)
             wb = mats[0].rows * (mats[0].cols // 256) * (144 if mats[0].kind == kind else 210)
             extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
                            "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -285,7 +289,7 @@ def main():
 
         def step6(i):
             fa.ffn_swiglu(g8[i % 8], u8[i % 8], dn[i % 8], xd, out=yf)
-        _, t = time_graph(torch, step6, 400, 8)
+        _, t = time_graph(torch, step6, 400, 200)
         fb = 2 * wbytes + d6.numel()
         extra["decode FFN 4096->14336->4096 (gate, up Q4_K; down Q6_K)"] = {
             "us_per_step": round(t / 400 * 1e6, 2), "GBs": round(fb / (t / 400) / 1e9, 1),
@@ -301,7 +305,7 @@ def main():
 
         def step7(i):
             fa.gemv_multi(qkv_sets[i % 40], xd, outs=qkv_out)
-        _, t = time_graph(torch, step7, 800, 40)
+        _, t = time_graph(torch, step7, 800, 400)
         qb = sum(qkv_rows) * (cols // 256) * 144
         extra["Q4_K q/k/v multi-GEMV (4096+1024+1024)x4096, one launch"] = {
             "us_per_step": round(t / 800 * 1e6, 2), "GBs": round(qb / (t / 800) / 1e9, 1),
