@@ -627,7 +627,7 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 31, lg = lane >> 5;
+    const int lg = lane >> 5;
     const int nb = g.nb;
 
     // this workgroup's items: the list of its XCD holds the tiles t = xcd (mod 8), every (matrix, row
