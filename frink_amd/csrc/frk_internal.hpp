@@ -179,6 +179,8 @@ int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipSt
 int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // thin batched GEMM of the K-quants: 1 <= batch <= thin_gemm_max_batch(w) rows per launch (0: does not fit)
 int thin_gemm_max_batch(const frk_weights *w);
+int thin_gemm_wide_rows(const frk_weights *w);
+int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s);
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);

@@ -399,6 +399,8 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
         if (rc) return rc;
         const size_t nb = w->cols / QK_K;
+        if (batch > (size_t)thin && batch <= (size_t)thin_gemm_wide_rows(w))
+            return launch_thin_gemm_wide(w, (int)batch, a, y, (hipStream_t)stream);
         for (size_t b0 = 0; b0 < batch; b0 += (size_t)thin) {
             const int n = (int)std::min<size_t>((size_t)thin, batch - b0);
             Q8KActs c = {a.q + b0 * w->cols, a.d + b0 * nb, a.bsums + b0 * nb * 16};

@@ -569,6 +569,12 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     extern __shared__ uint4 smem[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
     const int cols = nb * QK_K;
+    // a batch wider than ACTS is a grid of groups of ACTS activation rows: blockIdx.y picks the group
+    // (every group streams the matrix again; the groups after the first find it in the caches)
+    aq += (size_t)blockIdx.y * ACTS * cols;
+    ad += (size_t)blockIdx.y * ACTS * nb;
+    y += (size_t)blockIdx.y * ACTS * rows;
+    batch = min(ACTS, batch - (int)blockIdx.y * ACTS);
     const int q_stride = tm_q_stride(cols);
     uint8_t *lds_q = lds;                                                         // [ACTS][q_stride]
     float *lds_d = reinterpret_cast<float *>(lds_q + (size_t)ACTS * q_stride);    // [nb][8]
@@ -839,8 +845,8 @@ static int launch_thin_mfma6(const frk_weights *w, int batch, Q8KActs a, float *
         sized = true;
     }
     const size_t groups = (w->rows + 15) / 16;
-    hipLaunchKernelGGL((thin_mfma_q6_k_kernel<RG, ACTS>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
-                       shmem, s, w->dev, w->layout, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d, y);
+    hipLaunchKernelGGL((thin_mfma_q6_k_kernel<RG, ACTS>), dim3((unsigned)((groups + RG - 1) / RG), (unsigned)((batch + ACTS - 1) / ACTS)),
+                       dim3(64 * TM_WAVES), shmem, s, w->dev, w->layout, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d, y);
     FRK_LAUNCH_CHECK("thin mfma gemm");
     return FRK_OK;
 }
@@ -871,6 +877,15 @@ int thin_gemm_max_batch(const frk_weights *w) {
     for (int nbatch = 8; nbatch >= 2; nbatch /= 2)
         if (per_row * nbatch <= THIN_LDS_LIMIT) return nbatch;
     return 0;
+}
+
+// A batch of any width in one launch, where the kind has a kernel that takes one (Q6_K on the matrix
+// cores: a grid of 8-row groups); 0 rows = no such kernel for this matrix.
+int thin_gemm_wide_rows(const frk_weights *w) {
+    return (w->kind == FRK_KIND_Q6_K && thin_mfma6_acts(w) >= 8) ? 65535 * 8 : 0;
+}
+int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    return launch_thin_mfma6_rg<8>(w, batch, a, y, s);
 }
 
 // y[batch][rows] for 1 <= batch <= thin_gemm_max_batch(w) quantized activation rows (K-quants).

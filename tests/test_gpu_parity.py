@@ -515,6 +515,24 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
     w.release()
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(100, 1024, 40), (33, 2048, 37), (50, 4096, 9), (4096, 14336, 64)])
+def test_wide_q6_k_batch_is_one_launch_of_row_groups(fa, rows, cols, batch):
+    """A Q6_K batch wider than the 8 rows one workgroup stages runs as a grid of 8-row groups (the
+    last one ragged): every activation row against the oracle, on a slice of weight rows at full size."""
+    from frink_amd import synth
+    print("wide q6_k", rows, cols, batch, flush=True)
+    data = make_weights(fo.Q6_K, rows, cols, seed=rows + batch)
+    x = synth.activations(rows * 7 + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q6_K, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert got.shape == (batch, rows)
+    for row0 in sorted({0, max(rows - 64, 0)}):
+        n = min(64, rows - row0)
+        want = fo.gemm(fo.Q6_K, data, rows, cols, x, row0=row0, nrows=n)
+        assert_rows_close(got[:, row0:row0 + n], want, "wide q6_k %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
+    w.release()
+
+
 @pytest.mark.parametrize("kind,rows,cols,seed", [(fo.Q4_K, 14336, 4096, 21), (fo.Q6_K, 4096, 14336, 22)])
 def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
     """Batched decode, M=8, at the FFN shapes: slices of weight rows against the oracle for every
