@@ -148,6 +148,9 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+// the same for Q6_K (frk_gemm_q6.hip)
+size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols);
+int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
 // tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the
 // stacked matrices; *n_tiles <= max_tiles.  w1/y1 (nullable) is a second stacked matrix over the

@@ -392,6 +392,14 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
+    // Q6_K: from about a hundred rows on the matrix-core GEMM (whose time hardly depends on the batch
+    // up to 512 rows: 230 us at 4096x14336) is ahead of the thin kernel's 8-row groups (15 us each)
+    if (w->kind == FRK_KIND_Q6_K && batch >= 112) {
+        void *ws = nullptr;
+        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        if (rc) return rc;
+        return launch_gemm_q6_k(w, x, batch, y, ws, (hipStream_t)stream);
+    }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q6_K) && batch >= 2 ? thin_gemm_max_batch(w) : 0;
     if (thin >= 2) {

@@ -533,6 +533,29 @@ def test_wide_q6_k_batch_is_one_launch_of_row_groups(fa, rows, cols, batch):
     w.release()
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(300, 768, 130), (64, 256, 112), (13000, 512, 500), (257, 1024, 200),
+                                             (4096, 14336, 512)])
+def test_gemm_q6_k_on_the_matrix_cores(fa, rows, cols, batch):
+    """Q6_K batches of 112 rows and more take the int8 MFMA kernel (four pre-scaled planes per
+    16-weight group): both workgroup shapes (256 weight rows at 13000x512, 128 elsewhere), ragged last
+    row and token tiles, every activation row against the oracle on the first, a middle and the last
+    weight rows, and exact homogeneity."""
+    from frink_amd import synth
+    print("gemm q6_k", rows, cols, batch, flush=True)
+    data = make_weights(fo.Q6_K, rows, cols, seed=rows + batch)
+    x = synth.activations(rows * 5 + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q6_K, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert got.shape == (batch, rows)
+    n = min(64, rows)
+    for row0 in sorted({0, (rows // 2) // 32 * 32 + 5 if rows > 128 else 0, rows - n}):
+        want = fo.gemm(fo.Q6_K, data, rows, cols, x, row0=row0, nrows=n)
+        assert_rows_close(got[:, row0:row0 + n], want, "gemm q6_k %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
+    half = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
+    assert np.array_equal(bits(half), bits(got * np.float32(0.5)))
+    w.release()
+
+
 @pytest.mark.parametrize("kind,rows,cols,seed", [(fo.Q4_K, 14336, 4096, 21), (fo.Q6_K, 4096, 14336, 22)])
 def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
     """Batched decode, M=8, at the FFN shapes: slices of weight rows against the oracle for every
