@@ -232,6 +232,20 @@ def main():
                            "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
             for w in w2:
                 w.release()
+        # the FFN down projection of a Q4_K_M model at M=512: Q6_K on the matrix cores
+        d6g = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=78)).to(dev)
+        w6 = [fa.Weights.from_device(fa.Q6_K, d6g, cols, rows) for _ in range(4)]
+        xb6 = torch.from_numpy(synth.activations(6, 512, rows)).to(dev)
+        yb6 = torch.empty((512, cols), dtype=torch.float32, device=dev)
+
+        def step3b(i):
+            w6[i % 4].gemm(xb6, out=yb6)
+        _, t = time_graph(torch, step3b, 100, 50)
+        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+        extra["Q6_K GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        for w in w6:
+            w.release()
         # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
         E, K, H, F, T = 128, 8, 2048, 768, 512
         experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)
