@@ -8,10 +8,10 @@
 // s is a lane value.  With  s = 16*sh + sl  (sh = s >> 4 in -8..7, sl = s & 15)  and the raw code
 // q6 = 8*qu + ql  (qu, ql in 0..7), so that  q6 - 32 = 8*(qu - 4) + ql:
 //     s * (q6 - 32) = 128 * sh*(qu-4) + 16 * sh*ql + 8 * sl*(qu-4) + sl*ql
-//                   = 8 * (2 * (8*HH + HL) + LH) + LL
-// and the four planes HH = sh*(qu-4) in -28..32, HL = sh*ql in -56..49, LH = sl*(qu-4) in -60..45,
-// LL = sl*ql in 0..105 are int8.  One accumulator runs four chains of MFMAs with shifts by 3, 1 and 3
-// between them.  Half a block (four 32-weight sub-blocks) is unpacked at a time: 16 operand planes,
+//                   = 8 * (8*HH + HL + LH) + LL
+// and the four planes HH = 2*sh*(qu-4) in -56..64, HL = 2*sh*ql in -112..98, LH = sl*(qu-4) in
+// -60..45, LL = sl*ql in 0..105 are int8.  One accumulator runs four chains of MFMAs with a shift by
+// 3 after the first and before the last.  Half a block (four 32-weight sub-blocks) is unpacked at a time: 16 operand planes,
 // 64 registers; the block's two halves add up as integers before the one float step per block.
 //
 // The planes are built four bytes at a time: a packed 16-bit multiply serves two bytes at once as
@@ -82,27 +82,27 @@ __device__ __forceinline__ uint32_t q6_pk_mul(uint32_t bytes, uint32_t factor) {
 }
 
 // What a lane needs of its group's scale s = 16*sh + sl to build the planes' bytes, four at a time.
-// With K = 0x80 in every byte and x, y, z the packed products |sh|*ql, sl*qu, |sh|*qu (all < 128):
+// With K = 0x80 in every byte, m = 2*|sh| and x, y, z the packed products m*ql, sl*qu, m*qu (all < 128):
 //     LL = sl*ql                                                   (as multiplied)
 //     LH = sl*(qu-4)      = ((y + (K - 4sl)) ^ K                   (biased by 128, bias removed)
-//     HL = sh*ql          = x                       or, sh < 0:  (K - x) ^ K
-//     HH = sh*(qu-4)      = (z + (K - 4|sh|)) ^ K   or, sh < 0:  ((K + 4|sh|) - z) ^ K
+//     HL = 2*sh*ql        = x                       or, sh < 0:  (K - x) ^ K
+//     HH = 2*sh*(qu-4)    = (z + (K - 4m)) ^ K      or, sh < 0:  ((K + 4m) - z) ^ K
 // and "c - v" is written "(v ^ ~0) + (c + 1)", so that both signs are one xor, one add, one xor with
 // lane constants.  No byte ever borrows from or carries into its neighbour: every biased value
-// stays within 0x60..0xE9.
+// stays within 0x10..0xF0.
 struct Q6Scale {
-    uint32_t sl, m;           // sl and |sh|
+    uint32_t sl, m;           // sl and 2*|sh|
     uint32_t flip;            // ~0 where sh < 0
     uint32_t lh_add;          // K - 4*sl
     uint32_t hl_add, hl_xor;  // 0, 0  or  K + 1, K
-    uint32_t hh_add;          // K - 4*|sh|  or  K + 4*|sh| + 1
+    uint32_t hh_add;          // K - 4*m  or  K + 4*m + 1
 };
 __device__ __forceinline__ Q6Scale q6_scale(int s) {
     const uint32_t K = 0x80808080u;
     const int sh = s >> 4;
     Q6Scale c;
     c.sl = (uint32_t)(s & 15);
-    c.m = (uint32_t)(sh < 0 ? -sh : sh);
+    c.m = 2u * (uint32_t)(sh < 0 ? -sh : sh);
     const bool neg = sh < 0;
     c.flip = neg ? 0xffffffffu : 0u;
     c.lh_add = K - (4u * c.sl) * 0x01010101u;
@@ -193,7 +193,6 @@ __device__ __forceinline__ q6_v16i q6_tile_half(const Q6Ops &T, const Q6Planes &
     between(6);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, P.HL3, acc, 0, 0, 0);
     between(7);
-    acc = acc << 1;
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, P.LH0, acc, 0, 0, 0);
     between(8);
     acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, P.LH1, acc, 0, 0, 0);
@@ -408,6 +407,9 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
+#ifndef Q6_NARROW_BELOW
+#define Q6_NARROW_BELOW 200
+#endif
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
 
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
@@ -430,7 +432,7 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.y = y;
     g.tok_tiles = (int)((M + 63) / 64);
     // 256 weight rows per workgroup when that gives every CU one, else 128
-    const bool narrow = ((w->rows + 255) / 256) * (size_t)g.tok_tiles < 200;
+    const bool narrow = ((w->rows + 255) / 256) * (size_t)g.tok_tiles < Q6_NARROW_BELOW;
     const int rows_wg = narrow ? 128 : 256;
     g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
     const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
