@@ -44,6 +44,7 @@ struct Q6GemmArgs {
     Q8KTiled a;
     float *y;
     int row_tiles, tok_tiles;
+    int k_split;  // 1, or 2: blockIdx.y takes half of the blocks and the results are added into a zeroed y
 };
 
 struct Q6Lds {
@@ -111,54 +112,45 @@ __device__ __forceinline__ Q6Scale q6_scale(int s) {
     c.hh_add = neg ? K + (4u * c.m) * 0x01010101u + 1u : K - (4u * c.m) * 0x01010101u;
     return c;
 }
-// four codes of one group -> their bytes of the four planes
-__device__ __forceinline__ void q6_word(uint32_t w, const Q6Scale &c, int &hh, int &hl, int &lh, int &ll) {
+// four codes of one group, given as their low three bits ql and their high three bits qu (a byte
+// each) -> their bytes of the four planes
+__device__ __forceinline__ void q6_word(uint32_t ql, uint32_t qu, const Q6Scale &c, int &hh, int &hl, int &lh, int &ll) {
     const uint32_t K = 0x80808080u;
-    const uint32_t ql = w & 0x07070707u, qu = (w >> 3) & 0x07070707u;
     ll = (int)q6_pk_mul(ql, c.sl);
     hl = (int)(((q6_pk_mul(ql, c.m) ^ c.flip) + c.hl_add) ^ c.hl_xor);
     lh = (int)((q6_pk_mul(qu, c.sl) + c.lh_add) ^ K);
     hh = (int)(((q6_pk_mul(qu, c.m) ^ c.flip) + c.hh_add) ^ K);
 }
 
-// sub-block j of the half: its 16 codes for this lane (four words) and the group's scale -> planes
-__device__ __forceinline__ void q6_sub_block(const q6_v4i w, int s, q6_v4i &HH, q6_v4i &HL, q6_v4i &LH, q6_v4i &LL) {
-    const Q6Scale c = q6_scale(s);
+// dequant_q6_k's code assembly (crates/frink-quant/src/lib.rs:519-552) for a lane's 16 columns of
+// the half: sub-blocks 0..3 are the weights 128h + 32j + 16lg + (0..15), the code of a weight is
+// a nibble of ql (low nibbles: sub-blocks 0 and 1, high: 2 and 3) under two bits of qh (bits 2j..).
+// The code is never put together: its low three bits are the nibble's, its high three the nibble's
+// top bit under the two bits of qh.  One sub-block per call, so that a caller can spread the four
+// between other work.
+template <int J>
+__device__ __forceinline__ void q6_unpack_sub(const Q6Raw &R, int lg, q6_v4i &HH, q6_v4i &HL, q6_v4i &LH, q6_v4i &LL) {
+    const q6_v4i nib = (J & 1) ? R.qb : R.qa;
+    // the group's scale: byte 2j + lg of the half's eight
+    const uint32_t word = (uint32_t)(J < 2 ? R.sc.x : R.sc.y) >> (8 * lg + 16 * (J & 1));
+    const Q6Scale c = q6_scale((int)(int8_t)(word & 0xff));
+    auto one = [&](int nw, int hw, int &hh, int &hl, int &lh, int &ll) {
+        const uint32_t n = (uint32_t)nw >> (J < 2 ? 0 : 4), h = (uint32_t)hw;
+        const uint32_t ql = n & 0x07070707u;
+        // bit 0 of qu: the nibble's bit 3; bits 1..2: qh's bits 2J, 2J+1
+        const uint32_t top = (n >> 3) & 0x01010101u;
+        const uint32_t two = (J == 0 ? (h << 1) : (h >> (2 * J - 1))) & 0x06060606u;
+        q6_word(ql, top | two, c, hh, hl, lh, ll);
+    };
     int h0, h1, h2, h3, a0, a1, a2, a3, b0, b1, b2, b3, l0, l1, l2, l3;
-    q6_word((uint32_t)w.x, c, h0, a0, b0, l0);
-    q6_word((uint32_t)w.y, c, h1, a1, b1, l1);
-    q6_word((uint32_t)w.z, c, h2, a2, b2, l2);
-    q6_word((uint32_t)w.w, c, h3, a3, b3, l3);
+    one(nib.x, R.qh.x, h0, a0, b0, l0);
+    one(nib.y, R.qh.y, h1, a1, b1, l1);
+    one(nib.z, R.qh.z, h2, a2, b2, l2);
+    one(nib.w, R.qh.w, h3, a3, b3, l3);
     HH = q6_v4i{h0, h1, h2, h3};
     HL = q6_v4i{a0, a1, a2, a3};
     LH = q6_v4i{b0, b1, b2, b3};
     LL = q6_v4i{l0, l1, l2, l3};
-}
-
-// dequant_q6_k's code assembly (crates/frink-quant/src/lib.rs:519-552) for a lane's 16 columns of
-// the half: sub-blocks 0..3 are the weights 128h + 32j + 16lg + (0..15).  One sub-block per call, so
-// that a caller can spread the four between other work.
-template <int J>
-__device__ __forceinline__ void q6_unpack_sub(const Q6Raw &R, int lg, q6_v4i &HH, q6_v4i &HL, q6_v4i &LH, q6_v4i &LL) {
-    const uint32_t N = 0x0f0f0f0fu;
-    auto and4 = [](q6_v4i v, uint32_t mask) {
-        return q6_v4i{(int)((uint32_t)v.x & mask), (int)((uint32_t)v.y & mask), (int)((uint32_t)v.z & mask),
-                      (int)((uint32_t)v.w & mask)};
-    };
-    auto shr4 = [](q6_v4i v, int n) {
-        return q6_v4i{(int)((uint32_t)v.x >> n), (int)((uint32_t)v.y >> n), (int)((uint32_t)v.z >> n), (int)((uint32_t)v.w >> n)};
-    };
-    auto shl4 = [](q6_v4i v, int n) {
-        return q6_v4i{(int)((uint32_t)v.x << n), (int)((uint32_t)v.y << n), (int)((uint32_t)v.z << n), (int)((uint32_t)v.w << n)};
-    };
-    q6_v4i w;
-    if (J == 0) w = and4(R.qa, N) | shl4(and4(R.qh, 0x03030303u), 4);
-    if (J == 1) w = and4(R.qb, N) | and4(shl4(R.qh, 2), 0x30303030u);
-    if (J == 2) w = and4(shr4(R.qa, 4), N) | and4(R.qh, 0x30303030u);
-    if (J == 3) w = and4(shr4(R.qb, 4), N) | and4(shr4(R.qh, 2), 0x30303030u);
-    // the group's scale: byte 2j + lg of the half's eight
-    const uint32_t word = (uint32_t)(J < 2 ? R.sc.x : R.sc.y) >> (8 * lg + 16 * (J & 1));
-    q6_sub_block(w, (int)(int8_t)(word & 0xff), HH, HL, LH, LL);
 }
 __device__ __forceinline__ void q6_unpack_half(const Q6Raw &R, int lg, Q6Planes &P) {
     q6_unpack_sub<0>(R, lg, P.HH0, P.HL0, P.LH0, P.LL0);
@@ -238,7 +230,10 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
     if (row_tile >= g.row_tiles) return;  // uniform per workgroup
     const int tok0 = (in_grp >> 3) * (32 * L::MT);
     const int row0 = row_tile * (32 * RGS) + rgrp * 32;  // this wavefront's first weight row
-    const int nb = g.nb;
+    const int nb = g.nb;  // blocks of a row (strides); this workgroup multiplies blocks kb_begin .. kb_end - 1
+    const int per_part = (nb + g.k_split - 1) / g.k_split;
+    const int kb_begin = blockIdx.y * per_part, kb_end = min(nb, kb_begin + per_part);
+    if (kb_begin >= kb_end) return;  // uniform per workgroup
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
     auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
         int l = lane;
@@ -319,16 +314,16 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) accF[mt] = q6_v16f{0.0f};
 
-    // prologue: weights of blocks 0 and 1, activations of block 0; block 0's first half unpacked
-    issue_weights(0);
-    issue_acts(0);
-    if (nb > 1) issue_weights(1);
-    uint32_t d_bits = load_d(0);
+    // prologue: weights of the first two blocks, activations of the first; its first half unpacked
+    issue_weights(kb_begin);
+    issue_acts(kb_begin);
+    if (kb_begin + 1 < kb_end) issue_weights(kb_begin + 1);
+    uint32_t d_bits = load_d(kb_begin);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
     Q6Planes P0, P1;
     {
-        const Q6Raw R = read_raw(0, 0);
+        const Q6Raw R = read_raw(kb_begin, 0);
         q6_unpack_half(R, lg, P0);
     }
 
@@ -339,7 +334,7 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
         // the half after this one: this block's second, or the next block's first
         const Q6Raw R = H == 0 ? read_raw(kb, 1) : read_raw(kb + 1, 0);
         // with the block's second half in registers its stage is free for block kb+2
-        if (H == 0 && kb + 2 < nb) issue_weights(kb + 2);
+        if (H == 0 && kb + 2 < kb_end) issue_weights(kb + 2);
         const int k = opaque_lane() >> 5;
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
@@ -363,10 +358,10 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
         }
     };
 
-    for (int kb = 0; kb < nb; kb++) {
+    for (int kb = kb_begin; kb < kb_end; kb++) {
         const float dw = h2f(d_bits & 0xffffu);  // (before anything new is requested: its load is long done)
         // the activation stage refilled here was last read in iteration kb-1, which every wavefront has left
-        if (kb + 1 < nb) issue_acts(kb + 1);
+        if (kb + 1 < kb_end) issue_acts(kb + 1);
         d_bits = load_d(kb + 1);
         half_step(kb, std::integral_constant<int, 0>(), P0, P1);
         half_step(kb, std::integral_constant<int, 1>(), P1, P0);
@@ -397,8 +392,18 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tile_first + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < g.M) {
+                float *out = g.y + (size_t)tok * g.rows + row;
+                // two parts: both add into the zeroed output (two addends: the order does not matter)
+                if (g.k_split > 1) unsafeAtomicAdd(out, accF[mt][r]);
+                else *out = accF[mt][r];
+            }
         }
+}
+
+__global__ __launch_bounds__(256) void q6_zero_kernel(float4 *p, size_t n4) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -431,11 +436,16 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.M = (int)M;
     g.y = y;
     g.tok_tiles = (int)((M + 63) / 64);
-    // 256 weight rows per workgroup when that gives every CU one, else 128
-    const bool narrow = ((w->rows + 255) / 256) * (size_t)g.tok_tiles < Q6_NARROW_BELOW;
+    // 256 weight rows per workgroup (a block is unpacked once for two tiles) when that gives about
+    // every CU one; for a short and wide matrix the same with the blocks split between two workgroups
+    // that add into a zeroed output; 128 rows for what is left
+    const size_t wgs256 = ((w->rows + 255) / 256) * (size_t)g.tok_tiles;
+    const bool split = wgs256 < Q6_NARROW_BELOW && 2 * wgs256 >= 128 && g.nb >= 8 && (M * w->rows) % 4 == 0;
+    const bool narrow = wgs256 < Q6_NARROW_BELOW && !split;
     const int rows_wg = narrow ? 128 : 256;
+    g.k_split = split ? 2 : 1;
     g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
-    const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
+    const dim3 grid((unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles), (unsigned)g.k_split);
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6_k_mfma_kernel<1>),
@@ -446,8 +456,12 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", Q6Lds::BYTES, hipGetErrorString(e));
         sized = true;
     }
-    if (narrow) hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<2>, dim3(grid), dim3(512), Q6Lds::BYTES, s, g);
-    else hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, dim3(grid), dim3(512), Q6Lds::BYTES, s, g);
+    if (split) {
+        const size_t n4 = M * w->rows / 4;
+        hipLaunchKernelGGL(q6_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, reinterpret_cast<float4 *>(y), n4);
+    }
+    if (narrow) hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<2>, grid, dim3(512), Q6Lds::BYTES, s, g);
+    else hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, grid, dim3(512), Q6Lds::BYTES, s, g);
     FRK_LAUNCH_CHECK("gemm_q6_k_mfma");
     return FRK_OK;
 }
