@@ -515,6 +515,27 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
     w.release()
 
 
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K, fo.Q8_0])
+def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
+    """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
+    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 17 rows (Q4_K) or 112 (Q6_K); Q8_0:
+    per-row GEMVs): every size on either side of a threshold, on a ragged matrix, against the oracle."""
+    from frink_amd import synth
+    rows, cols = 72, 512
+    data = make_weights(kind, rows, cols, seed=900 + kind)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 64, 65, 111, 112, 113, 129):
+        if kind == fo.Q8_0 and batch > 9:
+            continue
+        print("gemm boundary", kind, batch, flush=True)
+        x = synth.activations(901 + batch, batch, cols, outlier_frac=0.01)
+        got = w.gemm(to_dev(x)).cpu().numpy()
+        want = fo.gemm(kind, data, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT)
+        assert got.shape == (batch, rows)
+        assert_rows_close(got, want, "gemm kind %d batch %d" % (kind, batch))
+    w.release()
+
+
 @pytest.mark.parametrize("rows,cols,batch", [(100, 1024, 40), (33, 2048, 37), (50, 4096, 9), (4096, 14336, 64)])
 def test_wide_q6_k_batch_is_one_launch_of_row_groups(fa, rows, cols, batch):
     """A Q6_K batch wider than the 8 rows one workgroup stages runs as a grid of 8-row groups (the
