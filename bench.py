@@ -246,6 +246,18 @@ def main():
                                                "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
         for w in w6:
             w.release()
+        # the shape the reference quotes its int8 Q8_0 GEMM on (crates/frink-cuda/src/mmq/kernel.rs:30-36)
+        d8g = torch.from_numpy(random_blocks(fa.Q8_0, cols, rows, seed=79)).to(dev)
+        w8 = [fa.Weights.from_device(fa.Q8_0, d8g, cols, rows) for _ in range(4)]
+
+        def step3c(i):
+            w8[i % 4].gemm(xb6, out=yb6)
+        _, t = time_graph(torch, step3c, 100, 50)
+        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+        extra["Q8_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        for w in w8:
+            w.release()
         # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
         E, K, H, F, T = 128, 8, 2048, 768, 512
         experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)

@@ -151,6 +151,9 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
 // the same for Q6_K (frk_gemm_q6.hip)
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+// and for Q8_0 (frk_gemm_q8.hip), over activations quantized 32 at a time
+size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols);
+int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
 // tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the
 // stacked matrices; *n_tiles <= max_tiles.  w1/y1 (nullable) is a second stacked matrix over the

@@ -189,7 +189,7 @@ const char *frk_hip_matvec_kernel(int kind) {
     return nullptr;
 }
 int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
-int frk_hip_gemm_supported(int kind) { return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K; }
+int frk_hip_gemm_supported(int kind) { return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0; }
 int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
 int frk_hip_block_elems(int kind) { return block_elems(kind); }
 int frk_hip_worth_a_gemm(size_t batch) { return batch >= 2; }
@@ -399,6 +399,14 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q6_k(w, x, batch, y, ws, (hipStream_t)stream);
+    }
+    // Q8_0: a batch is the integer path, as in the reference (Q8_0 activation blocks and dot_q8_0_q8,
+    // crates/frink-core/src/weight_matrix.rs:2701-2829); a single row keeps the f32 dot of its decode path
+    if (w->kind == FRK_KIND_Q8_0 && batch >= 2) {
+        void *ws = nullptr;
+        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        if (rc) return rc;
+        return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q6_K) && batch >= 2 ? thin_gemm_max_batch(w) : 0;

@@ -519,18 +519,17 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
 def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
     """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
     the matrix cores; wider: 8-row groups, or the MFMA GEMM from 17 rows (Q4_K) or 112 (Q6_K); Q8_0:
-    per-row GEMVs): every size on either side of a threshold, on a ragged matrix, against the oracle."""
+    the MFMA GEMM from two rows, its token tile growing at 33 and 65): every size on either side of a threshold, on a ragged matrix, against the oracle."""
     from frink_amd import synth
     rows, cols = 72, 512
     data = make_weights(kind, rows, cols, seed=900 + kind)
     w = fa.Weights.from_host(kind, data, rows, cols)
     for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 64, 65, 111, 112, 113, 129):
-        if kind == fo.Q8_0 and batch > 9:
-            continue
         print("gemm boundary", kind, batch, flush=True)
         x = synth.activations(901 + batch, batch, cols, outlier_frac=0.01)
         got = w.gemm(to_dev(x)).cpu().numpy()
-        want = fo.gemm(kind, data, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT)
+        # one Q8_0 row is the f32 dot of the decode path, a Q8_0 batch the integer path
+        want = fo.gemm(kind, data, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 and batch == 1 else fo.INT_DOT)
         assert got.shape == (batch, rows)
         assert_rows_close(got, want, "gemm kind %d batch %d" % (kind, batch))
     w.release()
@@ -574,6 +573,55 @@ def test_gemm_q6_k_on_the_matrix_cores(fa, rows, cols, batch):
         assert_rows_close(got[:, row0:row0 + n], want, "gemm q6_k %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
     half = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
     assert np.array_equal(bits(half), bits(got * np.float32(0.5)))
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(72, 512, 5), (100, 96, 33), (33, 288, 70), (64, 4096, 129),
+                                             (1000, 1056, 300), (4096, 4096, 512), (4096, 14336, 512)])
+def test_gemm_q8_0_on_the_matrix_cores(fa, rows, cols, batch):
+    """A Q8_0 batch is quantized to Q8_0 activation blocks and multiplied on the int8 MFMA, one
+    instruction per 32-wide block, the block's scales dw*da formed by an f16 MFMA: the three workgroup
+    shapes, ragged row and token tiles, rows that are not a multiple of the 256-column step (96, 288,
+    1056), every activation row against the oracle on the first, a middle and the last weight rows,
+    and exact homogeneity."""
+    from frink_amd import synth
+    print("gemm q8_0", rows, cols, batch, flush=True)
+    data = make_weights(fo.Q8_0, rows, cols, seed=rows + batch)
+    x = synth.activations(rows * 7 + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q8_0, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert got.shape == (batch, rows)
+    n = min(64, rows)
+    for row0 in sorted({0, (rows // 2) // 32 * 32 + 5 if rows > 128 else 0, rows - n}):
+        want = fo.gemm(fo.Q8_0, data, rows, cols, x, fo.INT_DOT, row0=row0, nrows=n)
+        assert_rows_close(got[:, row0:row0 + n], want, "gemm q8_0 %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
+    half = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
+    assert np.array_equal(bits(half), bits(got * np.float32(0.5)))
+    w.release()
+
+
+def test_gemm_q8_0_keeps_scales_below_the_f16_normal_range(fa):
+    """Block scales under 2^-14 are subnormal f16 values: weights of size 2e-4 give such weight scales,
+    activations of size 1e-3 such activation scales.  The scale product must not flush them."""
+    from frink_amd import synth
+    rows, cols, batch = 96, 512, 40
+    data = make_weights(fo.Q8_0, rows, cols, seed=77, sigma=2e-4)
+    d_bits = np.frombuffer(data, np.uint8).reshape(rows, cols // 32, 34)[:, :, :2].copy().view(np.uint16)
+    assert ((d_bits & 0x7c00) == 0).all() and (d_bits & 0x3ff).any(), "the weight scales are meant to be subnormal"
+    w = fa.Weights.from_host(fo.Q8_0, data, rows, cols)
+    x = synth.activations(78, batch, cols, outlier_frac=0.0)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert_rows_close(got, fo.gemm(fo.Q8_0, data, rows, cols, x, fo.INT_DOT), "subnormal weight scales")
+    assert np.abs(got).max() > 0
+    w.release()
+    data = make_weights(fo.Q8_0, rows, cols, seed=79)
+    w = fa.Weights.from_host(fo.Q8_0, data, rows, cols)
+    x = (x * np.float32(1e-3)).astype(np.float32)
+    _, d = fo.quantize_q8_0(x.reshape(-1))
+    assert (d < 2.0 ** -14).all() and (d > 0).any(), "the activation scales are meant to be subnormal"
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert_rows_close(got, fo.gemm(fo.Q8_0, data, rows, cols, x, fo.INT_DOT), "subnormal activation scales")
+    assert np.abs(got).max() > 0
     w.release()
 
 
