@@ -11,16 +11,21 @@
 // outer product is a second, tiny matrix product, and the f16 matrix cores compute it exactly (both
 // factors are f16 values, their product has 22 significant bits): v_mfma_f32_32x32x8_f16 with da in
 // k = 0 of A, dw in k = 0 of B and zeros elsewhere returns the scales in the very register layout of
-// the integer sums.  Left to the vector ALU are a conversion and a fused multiply-add per sum -- 32
-// instructions a block, which is what bounds the kernel (an MFMA pair takes about 50 clocks, the 32
-// instructions 128).
+// the integer sums.  Left to the vector ALU are a conversion and a fused multiply-add per sum: 32
+// instructions a block.
 //
 // A workgroup of TT x RT wavefronts owns 32*TT tokens x 32*RT rows, one tile per wavefront, and walks
-// the columns 256 (8 blocks) at a time: quants go global -> registers -> LDS (rows padded to 272
-// bytes so that the 32 rows of a fragment read fall in different banks), the next chunk's loads are
-// in flight while the current one is multiplied.  A wavefront reads its own rows' 8 scales of the
-// chunk straight from global memory, one chunk ahead as well.
+// the columns 256 (8 blocks) at a time: quants go global -> registers -> LDS, two chunks ahead of
+// the multiplication.  An LDS row is 272 bytes -- 256 of quants, so that the 32 rows of a fragment
+// read fall in different banks, and the row's eight f16 scales of the chunk in the 16 behind them.
+//
+// Measured at 4096 x 14336, M = 512 (128-token x 64-row workgroups, one per CU): 120 us.  With the
+// float step taken out it is 95 us, with the multiplication taken out 63 us: the 688 MB that the 256
+// workgroups pull out of L2 (every chunk of a tile is 48 KB for 4.2 M multiply-adds) cost as much as
+// the vector instructions do, and the two overlap only in part.
 #include "frk_device.hpp"
+
+#include <type_traits>
 
 namespace frk {
 
@@ -34,7 +39,7 @@ struct Q8GemmArgs {
     const uint8_t *W;   // resident rows: quants [nb][32], then the f16 scales [nb]
     size_t row_stride, off_d;
     const int8_t *aq;   // [M][cols]
-    const float *ad;    // [M][nb], every value an f16 value
+    const uint16_t *ad; // [M][nb rounded up to 8] f16 bits, zeros in the padding
     float *y;           // [M][rows]
     int rows, nb, M;
 };
@@ -58,6 +63,46 @@ __device__ __forceinline__ q8_v4h q8_as_k0(uint32_t h) {  // {h, 0, 0, 0}
     return v;
 }
 
+// quantize_activations_q8, Avx form (crates/frink-quant/src/act_quant.rs:157-189), for the GEMM: the
+// same quants as frk_quant.hip's kernel; the block scales leave as the f16 values they are, a token's
+// scales padded with zeros to a multiple of eight so that the GEMM reads any chunk's eight in one load.
+// Eight lanes per 32-value block.
+__global__ __launch_bounds__(256) void quantize_q8_0_gemm_kernel(const float *__restrict__ x, size_t n_blocks, int nb,
+                                                                 int8_t *__restrict__ q, uint16_t *__restrict__ d) {
+    const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t b = t >> 3;
+    const bool live = b < n_blocks;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) v = reinterpret_cast<const float4 *>(x)[t];
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+    if (!live) return;
+    const float scale = __fdiv_rn(amax, 127.0f);
+    const float inv = amax != 0.0f ? __fdiv_rn(127.0f, amax) : 0.0f;
+    auto quant = [&](float e) {
+        float r = rintf(e * inv);
+        r = fminf(fmaxf(r, -127.0f), 127.0f);
+        return (r != r) ? 0 : (int)r;
+    };
+    const int q0 = quant(v.x), q1 = quant(v.y), q2 = quant(v.z), q3 = quant(v.w);
+    reinterpret_cast<uint32_t *>(q)[t] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) |
+                                         ((uint32_t)(q2 & 0xff) << 16) | ((uint32_t)(q3 & 0xff) << 24);
+    if ((t & 7) == 0) {
+        const int stride = (nb + 7) & ~7;
+        const size_t tok = b / (size_t)nb;
+        const int in_row = (int)(b % (size_t)nb);
+        d[tok * stride + in_row] = f2h_bits(scale);
+        if (in_row == nb - 1)
+            for (int i = nb; i < stride; i++) d[tok * stride + i] = 0;
+    }
+}
+
+template <int AP, int WP>
+struct Q8Stage {  // one chunk's share of a thread on its way from global memory to LDS
+    q8_v4i a[AP], w[WP];  // 16-byte pieces of the activation and weight tiles
+    q8_v4i s;             // the eight f16 scales of one weight row or token (the first wavefronts only)
+};
+
 template <int TT, int RT>
 __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs g) {
     constexpr int NT = 64 * TT * RT;
@@ -76,13 +121,16 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     const uint8_t *a_src = (const uint8_t *)g.aq;
     const uint8_t *w_src = g.W;
     const int stage_dst = r0 * Q8_LDS_ROW + p * 16;
-    // the wavefront's own tile: token and weight row of this lane's operand fragments and scales
-    const int my_tok = min(tok0 + tt * 32 + (lane & 31), g.M - 1);
-    const int my_row = min(row0 + rt * 32 + (lane & 31), g.rows - 1);
-    const float *da_src = g.ad + (size_t)my_tok * g.nb;
-    const uint8_t *dw_src = g.W + (size_t)my_row * g.row_stride + g.off_d;
+    // The scales ride in the 16 bytes behind a row's quants in LDS.  Thread i of the first
+    // (RT + TT) / 2 wavefronts stages those of weight row i, or of token i - 32 * RT, of the tile.
+    const bool stages_scales = wave < (RT + TT) / 2;
+    const bool stages_weight_scales = tid < 32 * RT;
+    const uint8_t *s_src = stages_weight_scales
+                               ? g.W + (size_t)min(row0 + tid, g.rows - 1) * g.row_stride + g.off_d
+                               : (const uint8_t *)(g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * ((g.nb + 7) & ~7));
+    uint8_t *s_dst = stages_weight_scales ? lds_w + tid * Q8_LDS_ROW + 256 : lds_a + (tid - 32 * RT) * Q8_LDS_ROW + 256;
     const bool low_half = lane < 32;
-    const bool da_vec = (g.nb & 3) == 0;  // a token's scales then start 16-byte aligned
+    const int n_full = g.nb / Q8_CHUNK_BLOCKS;  // chunks of eight whole blocks
 
     q8_v16f acc;
 #pragma unroll
@@ -93,87 +141,111 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     const uint8_t *frag_a = lds_a + (tt * 32 + (lane & 31)) * Q8_LDS_ROW + (lane >> 5) * 16;
     const uint8_t *frag_w = lds_w + (rt * 32 + (lane & 31)) * Q8_LDS_ROW + (lane >> 5) * 16;
 
-    Q8Scales sa = {0u, 0u, 0u, 0u}, sw = {0u, 0u, 0u, 0u};
-    // round c multiplies chunk c while chunk c + 1 is on its way into registers; round -1 only fetches
-    for (int c = -1; c < n_chunks; c++) {
-        const bool more = c + 1 < n_chunks;
-        // vector values, not structs (a struct picked by a condition goes through memory), and nothing
-        // here may look at what a load returns: that would wait for it before the multiplication
-        q8_v4i a_reg[AP], w_reg[WP], dw_raw = {0, 0, 0, 0};
-        q8_v4f da_lo = {0.f, 0.f, 0.f, 0.f}, da_hi = {0.f, 0.f, 0.f, 0.f};
-        if (more) {
-            const int blk0 = (c + 1) * Q8_CHUNK_BLOCKS;
+    Q8Scales sa, sw;
+    // Round c asks for chunk c + 2 (into the registers `in`), multiplies chunk c out of LDS and then
+    // moves chunk c + 1 (the registers `out`, asked for a round earlier) into LDS: a load has two
+    // rounds to arrive.  Nothing may look at `in` within the round -- that would wait for its loads.
+    // In the steady rounds (steady_tag) every condition is known to hold and is not tested: a branch
+    // around the loads would make the waits in front of the LDS writes count as if none were issued.
+    auto round = [&](auto steady_tag, int c, Q8Stage<AP, WP> &out, Q8Stage<AP, WP> &in) {
+        constexpr bool STEADY = decltype(steady_tag)::value;
+        if (STEADY || c + 2 < n_chunks) {
+            const int blk0 = (c + 2) * Q8_CHUNK_BLOCKS;
             // Rows past the end repeat the last row, and pieces past the row's end its first piece:
             // every load is inside the operand.  What they return meets a zero scale or an
             // output that is not stored.
-            const size_t piece = blk0 + (p >> 1) < g.nb ? (size_t)blk0 * 32 + p * 16 : 0;
+            const size_t piece = STEADY || blk0 + (p >> 1) < g.nb ? (size_t)blk0 * 32 + p * 16 : 0;
 #pragma unroll
             for (int j = 0; j < AP; j++) {
                 const int tok = min(tok0 + r0 + j * (NT / 16), g.M - 1);
-                a_reg[j] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
+                in.a[j] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
             }
 #pragma unroll
             for (int j = 0; j < WP; j++) {
                 const int row = min(row0 + r0 + j * (NT / 16), g.rows - 1);
-                w_reg[j] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
+                in.w[j] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
             }
-            // scales: blocks past the end count as zero
-            if (blk0 + 8 <= g.nb) {
-                if (da_vec) {
-                    da_lo = *reinterpret_cast<const q8_v4f *>(da_src + blk0);
-                    da_hi = *reinterpret_cast<const q8_v4f *>(da_src + blk0 + 4);
-                } else {
+            if (stages_scales) {
+                if (STEADY || !stages_weight_scales || blk0 + 8 <= g.nb) {
+                    // (a token's scales are padded with zeros to whole chunks)
+                    in.s = *reinterpret_cast<const q8_v4i *>(s_src + (size_t)blk0 * 2);
+                } else {  // a weight row's last chunk when it is not a multiple of 256 columns
+                    const uint16_t *dh = reinterpret_cast<const uint16_t *>(s_src);
+                    auto wgt = [&](int b) { return blk0 + b < g.nb ? (int)dh[blk0 + b] : 0; };
 #pragma unroll
-                    for (int b = 0; b < 4; b++) da_lo[b] = da_src[blk0 + b], da_hi[b] = da_src[blk0 + 4 + b];
-                }
-                dw_raw = *reinterpret_cast<const q8_v4i *>(dw_src + (size_t)blk0 * 2);
-            } else {  // the last chunk of a row that is not a multiple of 256 columns
-                const uint16_t *dh = reinterpret_cast<const uint16_t *>(dw_src);
-                auto act = [&](int b) { return blk0 + b < g.nb ? da_src[blk0 + b] : 0.0f; };
-                auto wgt = [&](int b) { return blk0 + b < g.nb ? (int)dh[blk0 + b] : 0; };
-#pragma unroll
-                for (int b = 0; b < 4; b++) {
-                    da_lo[b] = act(b), da_hi[b] = act(4 + b);
-                    dw_raw[b] = wgt(2 * b) | (wgt(2 * b + 1) << 16);
+                    for (int b = 0; b < 4; b++) in.s[b] = wgt(2 * b) | (wgt(2 * b + 1) << 16);
                 }
             }
         }
-        if (c >= 0) {
-            // the matrix cores run one block ahead of the float step
-            auto products = [&](int b, q8_v16i &isum, q8_v16f &scale) {
-                const q8_v4i qa = *reinterpret_cast<const q8_v4i *>(frag_a + b * 32);
-                const q8_v4i qw = *reinterpret_cast<const q8_v4i *>(frag_w + b * 32);
+        if (STEADY || (c >= 0 && c < n_chunks)) {
+            // A three-stage pipeline over the blocks: the LDS reads of block b + 2, the matrix products
+            // of block b + 1 and the float step of block b are issued in that order, so that reads
+            // and products run in the shadow of the 32 vector instructions.
+            auto frags = [&](int b, q8_v4i &qa, q8_v4i &qw) {
+                qa = *reinterpret_cast<const q8_v4i *>(frag_a + b * 32);
+                qw = *reinterpret_cast<const q8_v4i *>(frag_w + b * 32);
+            };
+            auto products = [&](int b, const q8_v4i &qa, const q8_v4i &qw, q8_v16i &isum, q8_v16f &scale) {
                 isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa, qw, zero_i, 0, 0, 0);
                 scale = __builtin_amdgcn_mfma_f32_32x32x8f16(q8_as_k0(q8_pick(sa, b)), q8_as_k0(q8_pick(sw, b)), zero_f, 0, 0, 0);
             };
+            {
+                const q8_v4i va = *reinterpret_cast<const q8_v4i *>(frag_a - (lane >> 5) * 16 + 256);
+                const q8_v4i vw = *reinterpret_cast<const q8_v4i *>(frag_w - (lane >> 5) * 16 + 256);
+                sa = Q8Scales{low_half ? (uint32_t)va[0] : 0u, low_half ? (uint32_t)va[1] : 0u, low_half ? (uint32_t)va[2] : 0u,
+                              low_half ? (uint32_t)va[3] : 0u};
+                sw = Q8Scales{low_half ? (uint32_t)vw[0] : 0u, low_half ? (uint32_t)vw[1] : 0u, low_half ? (uint32_t)vw[2] : 0u,
+                              low_half ? (uint32_t)vw[3] : 0u};
+            }
+            q8_v4i qa1, qw1, qa2, qw2;
             q8_v16i isum_next;
             q8_v16f scale_next;
-            products(0, isum_next, scale_next);
+            frags(0, qa1, qw1);
+            frags(1, qa2, qw2);
+            products(0, qa1, qw1, isum_next, scale_next);
+            qa1 = qa2, qw1 = qw2;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int b = 0; b < Q8_CHUNK_BLOCKS; b++) {
                 const q8_v16i isum = isum_next;
                 const q8_v16f scale = scale_next;
-                if (b + 1 < Q8_CHUNK_BLOCKS) products(b + 1, isum_next, scale_next);
+                if (b + 2 < Q8_CHUNK_BLOCKS) frags(b + 2, qa2, qw2);
+                if (b + 1 < Q8_CHUNK_BLOCKS) products(b + 1, qa1, qw1, isum_next, scale_next);
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[r] = __builtin_fmaf(scale[r], (float)isum[r], acc[r]);
+                if (b + 2 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
+                if (b + 1 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMAs
+                __builtin_amdgcn_sched_group_barrier(0x002, 40, 0);                               // vector ALU
                 // keeps the float step here: sunk towards the loop's end it would leave every
                 // block's matrix results alive at once
                 asm volatile("" : "+v"(acc));
                 __builtin_amdgcn_sched_barrier(0);
+                qa1 = qa2, qw1 = qw2;
             }
         }
-        if (!more) break;
-        __syncthreads();  // every wavefront has read the chunk in LDS
+        if (STEADY || (c + 1 >= 0 && c + 1 < n_chunks)) {
+            lds_barrier();  // every wavefront has read the chunk in LDS (no wait for the loads on their way)
 #pragma unroll
-        for (int j = 0; j < AP; j++) *reinterpret_cast<q8_v4i *>(lds_a + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = a_reg[j];
+            for (int j = 0; j < AP; j++) *reinterpret_cast<q8_v4i *>(lds_a + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.a[j];
 #pragma unroll
-        for (int j = 0; j < WP; j++) *reinterpret_cast<q8_v4i *>(lds_w + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = w_reg[j];
-        auto pair = [](float lo, float hi) { return (uint32_t)f2h_bits(lo) | ((uint32_t)f2h_bits(hi) << 16); };
-        sa = Q8Scales{low_half ? pair(da_lo[0], da_lo[1]) : 0u, low_half ? pair(da_lo[2], da_lo[3]) : 0u,
-                      low_half ? pair(da_hi[0], da_hi[1]) : 0u, low_half ? pair(da_hi[2], da_hi[3]) : 0u};
-        sw = Q8Scales{low_half ? (uint32_t)dw_raw[0] : 0u, low_half ? (uint32_t)dw_raw[1] : 0u,
-                      low_half ? (uint32_t)dw_raw[2] : 0u, low_half ? (uint32_t)dw_raw[3] : 0u};
-        __syncthreads();
+            for (int j = 0; j < WP; j++) *reinterpret_cast<q8_v4i *>(lds_w + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.w[j];
+            if (stages_scales) *reinterpret_cast<q8_v4i *>(s_dst) = out.s;
+            lds_barrier();
+        }
+    };
+    Q8Stage<AP, WP> even, odd;  // the chunks of either parity on their way
+    const std::false_type any;
+    const std::true_type steady;
+    round(any, -2, odd, even);
+    round(any, -1, even, odd);
+    int c = 0;
+    for (; c + 3 < n_full; c += 2) {  // the chunks these rounds ask for, c + 2 and c + 3, are whole
+        round(steady, c, odd, even);
+        round(steady, c + 1, even, odd);
+    }
+    for (; c < n_chunks; c += 2) {
+        round(any, c, odd, even);
+        round(any, c + 1, even, odd);
     }
 
     // D register r of lane l is token 8*(r/4) + 4*(l/32) + r%4, weight row l%32 of the tile
@@ -194,16 +266,18 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     } while (0)
 
 size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols) {
-    return round_up(M * cols, 256) + round_up(M * (cols / 32) * 4, 256);
+    return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256);
 }
 
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     if (M > (size_t)1 << 30 || w->rows > (size_t)1 << 30)
         return set_error(FRK_ERR_SHAPE, "gemm_q8_0: %zu activation rows x %zu weight rows is too many", M, w->rows);
     int8_t *aq = (int8_t *)ws;
-    float *ad = (float *)((char *)ws + round_up(M * w->cols, 256));
-    int rc = launch_quantize_q8_0(x, M * w->cols, aq, ad, s);
-    if (rc) return rc;
+    uint16_t *ad = (uint16_t *)((char *)ws + round_up(M * w->cols, 256));
+    const size_t n_blocks = M * (w->cols / 32);
+    hipLaunchKernelGGL(quantize_q8_0_gemm_kernel, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, s, x, n_blocks,
+                       (int)(w->cols / 32), aq, ad);
+    FRK_LAUNCH_CHECK("quantize_q8_0_gemm");
     Q8GemmArgs g;
     g.W = w->dev;
     g.row_stride = w->layout.row_stride;

@@ -94,16 +94,22 @@ int main(int argc, char **argv) {
         for (size_t r = 0; r < rows; r++) exact = exact && y->value()[r] == std::ldexp((float)isum, -(int)r);
     CHECK(exact, "launch_matvec(Q8_0) equals the closed form exactly");
 
-    // the batched entry point is batch-major and equals per-row matvecs
+    // The batched entry point is batch-major.  A Q8_0 batch is quantized to Q8_0 activation blocks
+    // first: with one value of 127*(t+1) in every block of token t the block scale is t+1 and the
+    // quants are the values themselves, so the closed form is exact here too.
+    std::vector<float> base(xv);
+    base[0] = base[32] = 127.0f;
+    long bsum = 0;
+    for (size_t i = 0; i < cols; i++) bsum += ((long)(i % 7) - 3) * (long)base[i];
     std::vector<float> xb(3 * cols);
     for (size_t t = 0; t < 3; t++)
-        for (size_t i = 0; i < cols; i++) xb[t * cols + i] = xv[i] * (float)(t + 1);
+        for (size_t i = 0; i < cols; i++) xb[t * cols + i] = base[i] * (float)(t + 1);
     auto yb = launch_mul_mm(QuantKind::Q8_0, w8.data(), w8.size(), xb.data(), xb.size(), rows, cols, 3, nb * 34);
     bool major = yb.is_ok();
     if (major)
         for (size_t t = 0; t < 3; t++)
             for (size_t r = 0; r < rows; r++)
-                major = major && yb.value()[t * rows + r] == std::ldexp((float)(isum * (long)(t + 1)), -(int)r);
+                major = major && yb.value()[t * rows + r] == std::ldexp((float)(bsum * (long)(t + 1)), -(int)r);
     CHECK(major, "launch_mul_mm output is out[token*n_rows + row]");
 
     std::printf("%d failure(s)\n", failures);
