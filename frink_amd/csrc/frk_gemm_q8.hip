@@ -16,13 +16,14 @@
 //
 // A workgroup of TT x RT wavefronts owns 32*TT tokens x 32*RT rows, one tile per wavefront, and walks
 // the columns 256 (8 blocks) at a time: quants go global -> registers -> LDS, two chunks ahead of
-// the multiplication.  An LDS row is 272 bytes -- 256 of quants, so that the 32 rows of a fragment
-// read fall in different banks, and the row's eight f16 scales of the chunk in the 16 behind them.
+// the multiplication; LDS holds the chunks of even and of odd number, so a round needs one barrier.
+// An LDS row is 272 bytes -- 256 of quants, so that the 32 rows of a fragment read fall in different
+// banks, and the row's eight f16 scales of the chunk in the 16 behind them.
 //
-// Measured at 4096 x 14336, M = 512 (128-token x 64-row workgroups, one per CU): 120 us.  With the
+// Measured at 4096 x 14336, M = 512 (128-token x 64-row workgroups, one per CU): 115 us.  With the
 // float step taken out it is 95 us, with the multiplication taken out 63 us: the 688 MB that the 256
-// workgroups pull out of L2 (every chunk of a tile is 48 KB for 4.2 M multiply-adds) cost as much as
-// the vector instructions do, and the two overlap only in part.
+// workgroups pull out of L2 (every chunk of a tile is 48 KB for 4.2 M multiply-adds) cost about as
+// much as the vector instructions do, and the two overlap only in part.
 #include "frk_device.hpp"
 
 #include <type_traits>
@@ -107,8 +108,10 @@ template <int TT, int RT>
 __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs g) {
     constexpr int NT = 64 * TT * RT;
     constexpr int AP = TT * 512 / NT, WP = RT * 512 / NT;  // 16-byte pieces a thread stages per chunk
-    __shared__ __align__(16) uint8_t lds_a[TT * 32 * Q8_LDS_ROW];
-    __shared__ __align__(16) uint8_t lds_w[RT * 32 * Q8_LDS_ROW];
+    // two copies of the tiles' chunk: the chunks of even and of odd number
+    constexpr int LDS_A = TT * 32 * Q8_LDS_ROW, LDS_COPY = (TT + RT) * 32 * Q8_LDS_ROW;
+    extern __shared__ __align__(16) uint8_t q8_lds[];
+    uint8_t *const lds_a = q8_lds, *const lds_w = q8_lds + LDS_A;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tt = wave % TT, rt = wave / TT;
@@ -142,56 +145,61 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     const uint8_t *frag_w = lds_w + (rt * 32 + (lane & 31)) * Q8_LDS_ROW + (lane >> 5) * 16;
 
     Q8Scales sa, sw;
+    // The loads of a chunk: quant piece i < AP + WP, or (i == AP + WP) the scales.  `whole` says that the
+    // chunk is known to be eight whole blocks.
+    auto fetch = [&](int i, int chunk, bool whole, Q8Stage<AP, WP> &in) {
+        const int blk0 = chunk * Q8_CHUNK_BLOCKS;
+        // Rows past the end repeat the last row, and pieces past the row's end its first piece:
+        // every load is inside the operand.  What they return meets a zero scale or an output
+        // that is not stored.
+        const size_t piece = whole || blk0 + (p >> 1) < g.nb ? (size_t)blk0 * 32 + p * 16 : 0;
+        if (i < AP) {
+            const int tok = min(tok0 + r0 + i * (NT / 16), g.M - 1);
+            in.a[i] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
+        } else if (i < AP + WP) {
+            const int row = min(row0 + r0 + (i - AP) * (NT / 16), g.rows - 1);
+            in.w[i - AP] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
+        } else if (stages_scales) {
+            if (whole || !stages_weight_scales || blk0 + 8 <= g.nb) {
+                // (a token's scales are padded with zeros to whole chunks)
+                in.s = *reinterpret_cast<const q8_v4i *>(s_src + (size_t)blk0 * 2);
+            } else {  // a weight row's last chunk when it is not a multiple of 256 columns
+                const uint16_t *dh = reinterpret_cast<const uint16_t *>(s_src);
+                auto wgt = [&](int b) { return blk0 + b < g.nb ? (int)dh[blk0 + b] : 0; };
+#pragma unroll
+                for (int b = 0; b < 4; b++) in.s[b] = wgt(2 * b) | (wgt(2 * b + 1) << 16);
+            }
+        }
+    };
     // Round c asks for chunk c + 2 (into the registers `in`), multiplies chunk c out of LDS and then
     // moves chunk c + 1 (the registers `out`, asked for a round earlier) into LDS: a load has two
     // rounds to arrive.  Nothing may look at `in` within the round -- that would wait for its loads.
-    // In the steady rounds (steady_tag) every condition is known to hold and is not tested: a branch
-    // around the loads would make the waits in front of the LDS writes count as if none were issued.
+    constexpr int LOADS = AP + WP + 1, LOADS_A_BLOCK = (LOADS + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS;
+    // In the steady rounds (steady_tag) every condition is known to hold and is not tested (a branch
+    // around the loads would make the waits in front of the LDS writes count as if none were issued),
+    // and the loads are spread over the blocks of the multiplication: issued together, the eight
+    // wavefronts' loads fill the CU's queue and hold up the wavefronts behind them.
     auto round = [&](auto steady_tag, int c, Q8Stage<AP, WP> &out, Q8Stage<AP, WP> &in) {
         constexpr bool STEADY = decltype(steady_tag)::value;
-        if (STEADY || c + 2 < n_chunks) {
-            const int blk0 = (c + 2) * Q8_CHUNK_BLOCKS;
-            // Rows past the end repeat the last row, and pieces past the row's end its first piece:
-            // every load is inside the operand.  What they return meets a zero scale or an
-            // output that is not stored.
-            const size_t piece = STEADY || blk0 + (p >> 1) < g.nb ? (size_t)blk0 * 32 + p * 16 : 0;
+        if (!STEADY && c + 2 < n_chunks) {
 #pragma unroll
-            for (int j = 0; j < AP; j++) {
-                const int tok = min(tok0 + r0 + j * (NT / 16), g.M - 1);
-                in.a[j] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
-            }
-#pragma unroll
-            for (int j = 0; j < WP; j++) {
-                const int row = min(row0 + r0 + j * (NT / 16), g.rows - 1);
-                in.w[j] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
-            }
-            if (stages_scales) {
-                if (STEADY || !stages_weight_scales || blk0 + 8 <= g.nb) {
-                    // (a token's scales are padded with zeros to whole chunks)
-                    in.s = *reinterpret_cast<const q8_v4i *>(s_src + (size_t)blk0 * 2);
-                } else {  // a weight row's last chunk when it is not a multiple of 256 columns
-                    const uint16_t *dh = reinterpret_cast<const uint16_t *>(s_src);
-                    auto wgt = [&](int b) { return blk0 + b < g.nb ? (int)dh[blk0 + b] : 0; };
-#pragma unroll
-                    for (int b = 0; b < 4; b++) in.s[b] = wgt(2 * b) | (wgt(2 * b + 1) << 16);
-                }
-            }
+            for (int i = 0; i < LOADS; i++) fetch(i, c + 2, false, in);
         }
         if (STEADY || (c >= 0 && c < n_chunks)) {
             // A three-stage pipeline over the blocks: the LDS reads of block b + 2, the matrix products
             // of block b + 1 and the float step of block b are issued in that order, so that reads
             // and products run in the shadow of the 32 vector instructions.
             auto frags = [&](int b, q8_v4i &qa, q8_v4i &qw) {
-                qa = *reinterpret_cast<const q8_v4i *>(frag_a + b * 32);
-                qw = *reinterpret_cast<const q8_v4i *>(frag_w + b * 32);
+                qa = *reinterpret_cast<const q8_v4i *>(frag_a + (c & 1) * LDS_COPY + b * 32);
+                qw = *reinterpret_cast<const q8_v4i *>(frag_w + (c & 1) * LDS_COPY + b * 32);
             };
             auto products = [&](int b, const q8_v4i &qa, const q8_v4i &qw, q8_v16i &isum, q8_v16f &scale) {
                 isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa, qw, zero_i, 0, 0, 0);
                 scale = __builtin_amdgcn_mfma_f32_32x32x8f16(q8_as_k0(q8_pick(sa, b)), q8_as_k0(q8_pick(sw, b)), zero_f, 0, 0, 0);
             };
             {
-                const q8_v4i va = *reinterpret_cast<const q8_v4i *>(frag_a - (lane >> 5) * 16 + 256);
-                const q8_v4i vw = *reinterpret_cast<const q8_v4i *>(frag_w - (lane >> 5) * 16 + 256);
+                const q8_v4i va = *reinterpret_cast<const q8_v4i *>(frag_a + (c & 1) * LDS_COPY - (lane >> 5) * 16 + 256);
+                const q8_v4i vw = *reinterpret_cast<const q8_v4i *>(frag_w + (c & 1) * LDS_COPY - (lane >> 5) * 16 + 256);
                 sa = Q8Scales{low_half ? (uint32_t)va[0] : 0u, low_half ? (uint32_t)va[1] : 0u, low_half ? (uint32_t)va[2] : 0u,
                               low_half ? (uint32_t)va[3] : 0u};
                 sw = Q8Scales{low_half ? (uint32_t)vw[0] : 0u, low_half ? (uint32_t)vw[1] : 0u, low_half ? (uint32_t)vw[2] : 0u,
@@ -211,11 +219,14 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
                 const q8_v16f scale = scale_next;
                 if (b + 2 < Q8_CHUNK_BLOCKS) frags(b + 2, qa2, qw2);
                 if (b + 1 < Q8_CHUNK_BLOCKS) products(b + 1, qa1, qw1, isum_next, scale_next);
+                if (STEADY) {
+#pragma unroll
+                    for (int i = b * LOADS_A_BLOCK; i < (b + 1) * LOADS_A_BLOCK && i < LOADS; i++) fetch(i, c + 2, true, in);
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[r] = __builtin_fmaf(scale[r], (float)isum[r], acc[r]);
                 if (b + 2 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
                 if (b + 1 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMAs
-                __builtin_amdgcn_sched_group_barrier(0x002, 40, 0);                               // vector ALU
                 // keeps the float step here: sunk towards the loop's end it would leave every
                 // block's matrix results alive at once
                 asm volatile("" : "+v"(acc));
@@ -224,14 +235,16 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
             }
         }
         if (STEADY || (c + 1 >= 0 && c + 1 < n_chunks)) {
-            lds_barrier();  // every wavefront has read the chunk in LDS (no wait for the loads on their way)
+            // chunk c + 1 goes into the copy that chunk c - 1 was read from: every wavefront finished
+            // with that before the barrier that ended the last round
+            const int to = ((c + 1) & 1) * LDS_COPY;
 #pragma unroll
-            for (int j = 0; j < AP; j++) *reinterpret_cast<q8_v4i *>(lds_a + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.a[j];
+            for (int j = 0; j < AP; j++) *reinterpret_cast<q8_v4i *>(lds_a + to + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.a[j];
 #pragma unroll
-            for (int j = 0; j < WP; j++) *reinterpret_cast<q8_v4i *>(lds_w + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.w[j];
-            if (stages_scales) *reinterpret_cast<q8_v4i *>(s_dst) = out.s;
-            lds_barrier();
+            for (int j = 0; j < WP; j++) *reinterpret_cast<q8_v4i *>(lds_w + to + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.w[j];
+            if (stages_scales) *reinterpret_cast<q8_v4i *>(s_dst + to) = out.s;
         }
+        lds_barrier();  // one barrier a round (it does not wait for the loads on their way)
     };
     Q8Stage<AP, WP> even, odd;  // the chunks of either parity on their way
     const std::false_type any;
@@ -290,15 +303,26 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
     g.M = (int)M;
     // the widest token tile the batch fills; two row tiles per workgroup with it, one wavefront a
     // workgroup for the thinnest batches, whose grids are small
+    auto lds_bytes = [](int tt, int rt) { return (size_t)2 * (tt + rt) * 32 * Q8_LDS_ROW; };
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(4, 2));
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2, 2));
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", lds_bytes(4, 2), hipGetErrorString(e));
+        sized = true;
+    }
     if (M > 64) {
         const dim3 grid((unsigned)((w->rows + 63) / 64), (unsigned)((M + 127) / 128));
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2>), grid, dim3(512), 0, s, g);
+        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2>), grid, dim3(512), lds_bytes(4, 2), s, g);
     } else if (M > 32) {
         const dim3 grid((unsigned)((w->rows + 63) / 64), 1u);
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2>), grid, dim3(256), 0, s, g);
+        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2>), grid, dim3(256), lds_bytes(2, 2), s, g);
     } else {
         const dim3 grid((unsigned)((w->rows + 31) / 32), 1u);
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1>), grid, dim3(64), 0, s, g);
+        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1>), grid, dim3(64), lds_bytes(1, 1), s, g);
     }
     FRK_LAUNCH_CHECK("gemm_q8_0_mfma");
     return FRK_OK;
