@@ -412,9 +412,8 @@ __global__ __launch_bounds__(256) void q6_zero_kernel(float4 *p, size_t n4) {
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
-#ifndef Q6_NARROW_BELOW
-#define Q6_NARROW_BELOW 200
-#endif
+// fewer 256-row workgroups than this leave too many CUs idle: split the blocks, or take 128-row ones
+constexpr size_t Q6_NARROW_BELOW = 200;
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
 
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
