@@ -13,11 +13,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libfrink_oracle.so")
 
-Q8_0, Q4_K, Q6_K = 8, 12, 14
+Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
 FORM_NEON, FORM_AVX, FORM_SCALAR = 0, 1, 2
 F32_DOT, INT_DOT = 0, 1
 
-BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256)}
+BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
 
 
 def build(force=False):
@@ -45,19 +45,23 @@ def lib():
             "fo_f32_to_f16": (C.c_uint16, [C.c_float]),
             "fo_dequant": (C.c_int, [C.c_int, u8p, sz, f32p]),
             "fo_q4_k_element": (C.c_float, [u8p, C.c_int]),
+            "fo_q5_k_element": (C.c_float, [u8p, C.c_int]),
             "fo_q6_k_element": (C.c_float, [u8p, C.c_int]),
             "fo_dot_q8_0_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q4_k_f32": (C.c_float, [u8p, sz, f32p]),
+            "fo_dot_q5_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q6_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_quantize_q8_k": (None, [f32p, sz, i8p, f32p, i16p]),
             "fo_quantize_q8_0": (None, [f32p, sz, C.c_int, i8p, f32p]),
             "fo_dot_q8_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
             "fo_dot_q4_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
+            "fo_dot_q5_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
             "fo_dot_q6_k_q8k": (C.c_float, [u8p, sz, i8p, f32p]),
             "fo_nearest_int": (C.c_int, [C.c_float]),
             "fo_make_qx_quants": (C.c_float, [C.c_int, C.c_int, f32p, i8p, C.c_int]),
             "fo_encode_row_q8_0": (C.c_int, [f32p, sz, u8p]),
             "fo_encode_row_q4_k": (C.c_int, [f32p, sz, u8p]),
+            "fo_encode_row_q5_k": (C.c_int, [f32p, sz, u8p]),
             "fo_encode_row_q6_k": (C.c_int, [f32p, sz, u8p]),
             "fo_encode_matrix": (C.c_int, [C.c_int, f32p, sz, sz, u8p, C.c_int]),
             "fo_gemm": (C.c_int, [C.c_int, u8p, sz, sz, f32p, sz, f32p, C.c_int, C.c_int]),
@@ -111,13 +115,14 @@ def dequant(kind, data):
 
 def element(kind, block, i):
     block = _u8(block)
-    fn = lib().fo_q4_k_element if kind == Q4_K else lib().fo_q6_k_element
+    fn = {Q4_K: lib().fo_q4_k_element, Q5_K: lib().fo_q5_k_element, Q6_K: lib().fo_q6_k_element}[kind]
     return fn(_p(block, C.c_uint8), i)
 
 
 def dot_f32(kind, row, x):
     row, x = _u8(row), _f32(x)
-    fn = {Q8_0: lib().fo_dot_q8_0_f32, Q4_K: lib().fo_dot_q4_k_f32, Q6_K: lib().fo_dot_q6_k_f32}[kind]
+    fn = {Q8_0: lib().fo_dot_q8_0_f32, Q4_K: lib().fo_dot_q4_k_f32, Q5_K: lib().fo_dot_q5_k_f32,
+          Q6_K: lib().fo_dot_q6_k_f32}[kind]
     return fn(_p(row, C.c_uint8), row.size, _p(x, C.c_float))
 
 
@@ -146,9 +151,9 @@ def dot_int(kind, row, acts):
         q, d = acts
         return lib().fo_dot_q8_0_q8(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
     q, d, bs = acts
-    if kind == Q4_K:
-        return lib().fo_dot_q4_k_q8k(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float),
-                                     _p(bs, C.c_int16))
+    if kind in (Q4_K, Q5_K):
+        fn = lib().fo_dot_q4_k_q8k if kind == Q4_K else lib().fo_dot_q5_k_q8k
+        return fn(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float), _p(bs, C.c_int16))
     return lib().fo_dot_q6_k_q8k(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
 
 
@@ -168,7 +173,8 @@ def encode_row(kind, x):
     x = _f32(x).ravel()
     bb, be = BLOCK[kind]
     out = np.empty(x.size // be * bb, np.uint8)
-    fn = {Q8_0: lib().fo_encode_row_q8_0, Q4_K: lib().fo_encode_row_q4_k, Q6_K: lib().fo_encode_row_q6_k}[kind]
+    fn = {Q8_0: lib().fo_encode_row_q8_0, Q4_K: lib().fo_encode_row_q4_k, Q5_K: lib().fo_encode_row_q5_k,
+          Q6_K: lib().fo_encode_row_q6_k}[kind]
     if fn(_p(x, C.c_float), x.size, _p(out, C.c_uint8)):
         return None
     return out

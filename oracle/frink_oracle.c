@@ -30,6 +30,7 @@
 #define Q8_0_BYTES 34
 #define Q8_0_ELEMS 32
 #define Q4_K_BYTES 144
+#define Q5_K_BYTES 176
 #define Q6_K_BYTES 210
 #define QK_K 256
 
@@ -38,6 +39,7 @@ int fo_block_bytes(int kind) {
     switch (kind) {
     case FO_KIND_Q8_0: return Q8_0_BYTES;
     case FO_KIND_Q4_K: return Q4_K_BYTES;
+    case FO_KIND_Q5_K: return Q5_K_BYTES;
     case FO_KIND_Q6_K: return Q6_K_BYTES;
     }
     return 0;
@@ -45,7 +47,7 @@ int fo_block_bytes(int kind) {
 int fo_block_elems(int kind) {
     switch (kind) {
     case FO_KIND_Q8_0: return Q8_0_ELEMS;
-    case FO_KIND_Q4_K: case FO_KIND_Q6_K: return QK_K;
+    case FO_KIND_Q4_K: case FO_KIND_Q5_K: case FO_KIND_Q6_K: return QK_K;
     }
     return 0;
 }
@@ -150,6 +152,41 @@ int fo_dequant_q4_k(const uint8_t *src, size_t nbytes, float *out) {
     return 0;
 }
 
+/* src/lib.rs:424-459: Q4_K's walk, each code's fifth bit from the qh plane (bytes 16..48), whose
+ * byte l serves elements l, l+32, l+64, ... of the block through bits 0, 1, 2, ... */
+int fo_dequant_q5_k(const uint8_t *src, size_t nbytes, float *out) {
+    if (nbytes % Q5_K_BYTES) return -1;
+    size_t nb = nbytes / Q5_K_BYTES;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = src + b * Q5_K_BYTES;
+        float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        float *y = out + b * QK_K;
+        int is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int oi = 0; oi < 4; oi++) {
+            uint8_t sc1, m1, sc2, m2;
+            fo_q4_k_scale_min(is, scales, &sc1, &m1);
+            fo_q4_k_scale_min(is + 1, scales, &sc2, &m2);
+            float d1 = d * (float)sc1, min1 = dmin * (float)m1;
+            float d2 = d * (float)sc2, min2 = dmin * (float)m2;
+            const uint8_t *ql = qs + oi * 32;
+            for (int l = 0; l < 32; l++) {
+                uint8_t hi = (qh[l] & u1) ? 16 : 0;
+                *y++ = d1 * (float)(uint8_t)((ql[l] & 0x0F) + hi) - min1;
+            }
+            for (int l = 0; l < 32; l++) {
+                uint8_t hi = (qh[l] & u2) ? 16 : 0;
+                *y++ = d2 * (float)(uint8_t)((ql[l] >> 4) + hi) - min2;
+            }
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+    }
+    return 0;
+}
+
 /* src/lib.rs:519-552 */
 int fo_dequant_q6_k(const uint8_t *src, size_t nbytes, float *out) {
     if (nbytes % Q6_K_BYTES) return -1;
@@ -181,6 +218,7 @@ int fo_dequant(int kind, const uint8_t *src, size_t nbytes, float *out) {
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dequant_q8_0(src, nbytes, out);
     case FO_KIND_Q4_K: return fo_dequant_q4_k(src, nbytes, out);
+    case FO_KIND_Q5_K: return fo_dequant_q5_k(src, nbytes, out);
     case FO_KIND_Q6_K: return fo_dequant_q6_k(src, nbytes, out);
     }
     return -2;
@@ -198,6 +236,16 @@ float fo_q4_k_element(const uint8_t *blk, int i) {
     fo_q4_k_scale_min(sub, blk + 4, &sc, &m);
     float d = rd_f16(blk), dmin = rd_f16(blk + 2);
     return (d * (float)sc) * (float)nib - dmin * (float)m;
+}
+float fo_q5_k_element(const uint8_t *blk, int i) {
+    int sub = i >> 5, within = i & 31;
+    int byte = 48 + (sub >> 1) * 32 + within;
+    int nib = (sub & 1) ? (blk[byte] >> 4) : (blk[byte] & 15);
+    int fifth = (blk[16 + within] >> sub) & 1;  /* bit `sub` of qh[within] */
+    uint8_t sc, m;
+    fo_q4_k_scale_min(sub, blk + 4, &sc, &m);
+    float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+    return (d * (float)sc) * (float)(nib + 16 * fifth) - dmin * (float)m;
 }
 float fo_q6_k_element(const uint8_t *blk, int i) {
     int half = i >> 7, r = i & 127, quarter = r >> 5, l = r & 31;
@@ -248,6 +296,41 @@ float fo_dot_q4_k_f32(const uint8_t *row, size_t row_bytes, const float *x) {
             q_off += 32;
             base += 64;
             is += 2;
+        }
+    }
+    return acc;
+}
+
+/* src/lib.rs:481-515 */
+float fo_dot_q5_k_f32(const uint8_t *row, size_t row_bytes, const float *x) {
+    size_t nb = row_bytes / Q5_K_BYTES;
+    float acc = 0.0f;
+    size_t base = 0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * Q5_K_BYTES;
+        float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        int is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int oi = 0; oi < 4; oi++) {
+            uint8_t sc1, m1, sc2, m2;
+            fo_q4_k_scale_min(is, scales, &sc1, &m1);
+            fo_q4_k_scale_min(is + 1, scales, &sc2, &m2);
+            float d1 = d * (float)sc1, min1 = dmin * (float)m1;
+            float d2 = d * (float)sc2, min2 = dmin * (float)m2;
+            const uint8_t *ql = qs + oi * 32;
+            for (int l = 0; l < 32; l++) {
+                uint8_t hi = (qh[l] & u1) ? 16 : 0;
+                acc += (d1 * (float)(uint8_t)((ql[l] & 0x0F) + hi) - min1) * x[base + l];
+            }
+            for (int l = 0; l < 32; l++) {
+                uint8_t hi = (qh[l] & u2) ? 16 : 0;
+                acc += (d2 * (float)(uint8_t)((ql[l] >> 4) + hi) - min2) * x[base + 32 + l];
+            }
+            base += 64;
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
         }
     }
     return acc;
@@ -386,6 +469,53 @@ float fo_dot_q4_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, con
             q_off += 32;
             base += 64;
             is += 2;
+        }
+    }
+    return acc;
+}
+
+/* src/lib.rs:886-938 */
+float fo_dot_q5_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *dact,
+                      const int16_t *bsums_all) {
+    size_t nb = row_bytes / Q5_K_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * Q5_K_BYTES;
+        float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+        float da = dact[b];
+        const int8_t *q8 = q + b * QK_K;
+        const int16_t *bsums = bsums_all + b * 16;
+
+        int32_t sum_min = 0;
+        for (int i = 0; i < 8; i++) {
+            uint8_t sc, m;
+            fo_q4_k_scale_min(i, scales, &sc, &m);
+            sum_min += (int32_t)m * ((int32_t)bsums[2 * i] + (int32_t)bsums[2 * i + 1]);
+        }
+        acc -= dmin * da * (float)sum_min;
+
+        int q_off = 0, base = 0, is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int p = 0; p < 4; p++) {
+            uint8_t sc1, sc2, m_;
+            fo_q4_k_scale_min(is, scales, &sc1, &m_);
+            fo_q4_k_scale_min(is + 1, scales, &sc2, &m_);
+            int32_t isum1 = 0, isum2 = 0;
+            for (int l = 0; l < 32; l++) {
+                int32_t hi = (qh[l] & u1) ? 16 : 0;
+                isum1 += ((int32_t)(qs[q_off + l] & 0x0F) + hi) * (int32_t)q8[base + l];
+            }
+            for (int l = 0; l < 32; l++) {
+                int32_t hi = (qh[l] & u2) ? 16 : 0;
+                isum2 += ((int32_t)(qs[q_off + l] >> 4) + hi) * (int32_t)q8[base + 32 + l];
+            }
+            acc += d * da * ((float)sc1 * (float)isum1 + (float)sc2 * (float)isum2);
+            q_off += 32;
+            base += 64;
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
         }
     }
     return acc;
@@ -611,12 +741,15 @@ static void pack_scale_min(uint8_t *packed, int j, uint8_t ls, uint8_t lm) {
     }
 }
 
-/* src/encode/fit.rs:416-571 (plain path, Q4_K_FIT = {15, -1.0, 0.1, 20} from
- * src/encode/q4_k.rs:42-48) and the nibble packing of src/encode/q4_k.rs:83-102 */
-static void encode_block_q4_k(const float *block, uint8_t *out) {
-    uint8_t l[QK_K], laux[32];
+/* fit_qk_super_block, src/encode/fit.rs:416-571 (plain path): the fit Q4_K and Q5_K share, with
+ * QkFit's numbers as arguments -- Q4_K_FIT = {15, -1.0, 0.1, 20} (src/encode/q4_k.rs:42-48),
+ * Q5_K_FIT = {31, -0.5, 0.1, 15} (src/encode/q5_k.rs:38-44).  Leaves the codes in l, the packed
+ * 6-bit scales and mins, and the two f16 fields. */
+static void fit_qk_super_block(const float *block, int nmax, float rmin, float rdelta, int nstep, uint8_t *l,
+                               uint8_t *packed, uint16_t *dh_out, uint16_t *dminh_out) {
+    uint8_t laux[32];
     float weights[32], mins[8], scales[8];
-    memset(l, 0, sizeof l);
+    memset(l, 0, QK_K);
     float max_scale = 0.0f, max_min = 0.0f;
     for (int j = 0; j < 8; j++) {
         const float *xs = block + 32 * j;
@@ -626,14 +759,13 @@ static void encode_block_q4_k(const float *block, uint8_t *out) {
         float av_x = sqrtf(sum_x2 / 32.0f);
         for (int i = 0; i < 32; i++) weights[i] = av_x + fabsf(xs[i]);
         float mn;
-        float sc = fo_make_qkx2_quants(32, 15, xs, weights, l + 32 * j, &mn, laux, -1.0f, 0.1f, 20, 0);
+        float sc = fo_make_qkx2_quants(32, nmax, xs, weights, l + 32 * j, &mn, laux, rmin, rdelta, nstep, 0);
         scales[j] = sc;
         mins[j] = mn;
         if (sc > max_scale) max_scale = sc;
         if (mn > max_min) max_min = mn;
     }
-    uint8_t packed[12];
-    memset(packed, 0, sizeof packed);
+    memset(packed, 0, 12);
     float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
     float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
     for (int j = 0; j < 8; j++) {
@@ -654,9 +786,18 @@ static void encode_block_q4_k(const float *block, uint8_t *out) {
         float dm = dmin * (float)m;
         for (int ii = 0; ii < 32; ii++) {
             int idx = 32 * j + ii;
-            l[idx] = (uint8_t)clampi(fo_nearest_int((block[idx] + dm) / dj), 0, 15);
+            l[idx] = (uint8_t)clampi(fo_nearest_int((block[idx] + dm) / dj), 0, nmax);
         }
     }
+    *dh_out = dh;
+    *dminh_out = dminh;
+}
+
+/* the nibble packing of src/encode/q4_k.rs:83-102 */
+static void encode_block_q4_k(const float *block, uint8_t *out) {
+    uint8_t l[QK_K], packed[12];
+    uint16_t dh, dminh;
+    fit_qk_super_block(block, 15, -1.0f, 0.1f, 20, l, packed, &dh, &dminh);
     out[0] = dh & 0xff; out[1] = dh >> 8;
     out[2] = dminh & 0xff; out[3] = dminh >> 8;
     memcpy(out + 4, packed, 12);
@@ -665,10 +806,41 @@ static void encode_block_q4_k(const float *block, uint8_t *out) {
         for (int i = 0; i < 32; i++) *qs++ = (uint8_t)(l[j + i] | (l[j + i + 32] << 4));
 }
 
+/* src/encode/q5_k.rs:55-100: the fifth bit of a code goes to the qh plane, bit 2g of qh[j] for
+ * element 64g + j and bit 2g + 1 for element 64g + 32 + j */
+static void encode_block_q5_k(const float *block, uint8_t *out) {
+    uint8_t l[QK_K], packed[12];
+    uint16_t dh, dminh;
+    fit_qk_super_block(block, 31, -0.5f, 0.1f, 15, l, packed, &dh, &dminh);
+    out[0] = dh & 0xff; out[1] = dh >> 8;
+    out[2] = dminh & 0xff; out[3] = dminh >> 8;
+    memcpy(out + 4, packed, 12);
+    uint8_t *qh = out + 16, *ql = out + 48;
+    memset(qh, 0, 32);
+    uint8_t m1 = 1, m2 = 2;
+    for (int g = 0; g < 4; g++) {
+        for (int j = 0; j < 32; j++) {
+            uint8_t l1 = l[64 * g + j], l2 = l[64 * g + j + 32];
+            if (l1 > 15) { l1 -= 16; qh[j] |= m1; }
+            if (l2 > 15) { l2 -= 16; qh[j] |= m2; }
+            ql[32 * g + j] = (uint8_t)(l1 | (l2 << 4));
+        }
+        m1 = (uint8_t)(m1 << 2);
+        m2 = (uint8_t)(m2 << 2);
+    }
+}
+
 /* src/encode/q4_k.rs:120-131 */
 int fo_encode_row_q4_k(const float *src, size_t n, uint8_t *out) {
     if (n % QK_K) return -1;
     for (size_t b = 0; b < n / QK_K; b++) encode_block_q4_k(src + b * QK_K, out + b * Q4_K_BYTES);
+    return 0;
+}
+
+/* src/encode/q5_k.rs:118-130 */
+int fo_encode_row_q5_k(const float *src, size_t n, uint8_t *out) {
+    if (n % QK_K) return -1;
+    for (size_t b = 0; b < n / QK_K; b++) encode_block_q5_k(src + b * QK_K, out + b * Q5_K_BYTES);
     return 0;
 }
 
@@ -756,6 +928,7 @@ int fo_encode_matrix(int kind, const float *src, size_t rows, size_t cols, uint8
         uint8_t *o = out + (size_t)r * row_bytes;
         int e = kind == FO_KIND_Q8_0 ? fo_encode_row_q8_0(s, cols, o)
               : kind == FO_KIND_Q4_K ? fo_encode_row_q4_k(s, cols, o)
+              : kind == FO_KIND_Q5_K ? fo_encode_row_q5_k(s, cols, o)
                                      : fo_encode_row_q6_k(s, cols, o);
         if (e) rc = e;
     }
@@ -801,6 +974,7 @@ static inline float row_dot_int(int kind, const uint8_t *row, size_t row_bytes, 
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_q8(row, row_bytes, q, d);
     case FO_KIND_Q4_K: return fo_dot_q4_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
+    case FO_KIND_Q5_K: return fo_dot_q5_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
     default: return fo_dot_q6_k_q8k(row, row_bytes, q, d);
     }
 }
@@ -808,6 +982,7 @@ static inline float row_dot_f32(int kind, const uint8_t *row, size_t row_bytes, 
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_f32(row, row_bytes, x);
     case FO_KIND_Q4_K: return fo_dot_q4_k_f32(row, row_bytes, x);
+    case FO_KIND_Q5_K: return fo_dot_q5_k_f32(row, row_bytes, x);
     default: return fo_dot_q6_k_f32(row, row_bytes, x);
     }
 }

@@ -14,9 +14,10 @@ Sources (paths relative to the reference root):
 
 * crates/frink-quant/src/encode.rs            Q8_0 encoder goldens, tie block
 * crates/frink-quant/src/encode/q4_k.rs       llama.cpp Q4_K bytes for the k-quant fixture
+* crates/frink-quant/src/encode/q5_k.rs       llama.cpp Q5_K bytes for the k-quant fixture
 * crates/frink-quant/src/encode/q6_k.rs       llama.cpp Q6_K bytes for the k-quant fixture
 * crates/frink-quant/src/encode/testdata.rs   8 real-weight super-blocks (f16 bits)
-* crates/frink-quant/src/lib.rs               Q4_K / Q6_K dequant test blocks + goldens
+* crates/frink-quant/src/lib.rs               Q4_K / Q5_K / Q6_K dequant test blocks + goldens
 """
 import json
 import os
@@ -58,6 +59,8 @@ def main():
 
     q4 = open(os.path.join(QUANT, "encode", "q4_k.rs")).read()
     out["q4_k_encode_golden"] = bytes(ints(q4, "LLAMA_CPP_Q4_K_GOLDEN")).hex()
+    q5 = open(os.path.join(QUANT, "encode", "q5_k.rs")).read()
+    out["q5_k_encode_golden"] = bytes(ints(q5, "LLAMA_CPP_Q5_K_GOLDEN")).hex()
     q6 = open(os.path.join(QUANT, "encode", "q6_k.rs")).read()
     out["q6_k_encode_golden"] = bytes(ints(q6, "LLAMA_CPP_Q6_K_GOLDEN")).hex()
 
@@ -67,6 +70,7 @@ def main():
     lib = open(os.path.join(QUANT, "lib.rs")).read()
     for blk, gold in [
         ("Q4_K_TEST_BLOCK", "Q4_K_GOLDEN"),
+        ("Q5_K_TEST_BLOCK", "Q5_K_GOLDEN"),
         ("Q6_K_TEST_BLOCK", "Q6_K_GOLDEN"),
         ("Q6_K_SIGNED_SCALES_TEST_BLOCK", "Q6_K_SIGNED_SCALES_GOLDEN"),
         ("Q6_K_SIGNED_TEST_BLOCK", "Q6_K_SIGNED_GOLDEN"),
@@ -76,7 +80,7 @@ def main():
 
     sizes = {
         "q8_0_encode_golden": 2 * 34, "q8_0_tie_block_f16_bits": 32, "q8_0_tie_block_golden": 34,
-        "q4_k_encode_golden": 12 * 144, "q6_k_encode_golden": 12 * 210,
+        "q4_k_encode_golden": 12 * 144, "q5_k_encode_golden": 12 * 176, "q6_k_encode_golden": 12 * 210,
         "real_weight_blocks_f16_bits": 8 * 256,
         "q4_k_test_block": 144, "q4_k_golden": 256,
         "q6_k_test_block": 210, "q6_k_golden": 256,

@@ -67,7 +67,7 @@ def test_q8_0_all_zero_block_is_34_zero_bytes():
 
 
 @pytest.mark.parametrize("kind,ragged", [(fo.Q8_0, 33), (fo.Q8_0, 1), (fo.Q4_K, 257), (fo.Q4_K, 32),
-                                         (fo.Q6_K, 257), (fo.Q6_K, 16)])
+                                         (fo.Q5_K, 257), (fo.Q5_K, 32), (fo.Q6_K, 257), (fo.Q6_K, 16)])
 def test_a_ragged_row_is_refused_and_an_empty_one_accepted(kind, ragged):
     assert fo.encode_row(kind, np.full(ragged, 0.5, np.float32)) is None
     assert fo.encode_row(kind, np.zeros(0, np.float32)).size == 0
@@ -95,6 +95,16 @@ def test_q4_k_matches_llama_cpp_quantize_row_q4_k_ref(vectors, kfix):
     gold = hexbytes(vectors["q4_k_encode_golden"]).reshape(12, 144)
     for b in range(12):
         assert got[b].tobytes() == gold[b].tobytes(), "super-block %d disagrees with llama.cpp" % b
+
+
+# crates/frink-quant/src/encode/q5_k.rs:144-305
+def test_q5_k_matches_llama_cpp_quantize_row_q5_k_ref(vectors, kfix):
+    got = fo.encode_row(fo.Q5_K, kfix).reshape(12, 176)
+    gold = hexbytes(vectors["q5_k_encode_golden"]).reshape(12, 176)
+    for b in range(12):
+        assert got[b].tobytes() == gold[b].tobytes(), "super-block %d disagrees with llama.cpp" % b
+    # the fixture uses the fifth bit: some codes are above 15
+    assert gold[:, 16:48].any()
 
 
 def test_q6_k_matches_llama_cpp_quantize_row_q6_k_ref(vectors, kfix):
@@ -173,6 +183,7 @@ def test_make_qx_quants_zero_group_and_sign_convention():
 
 @pytest.mark.parametrize("kind,blk,gold", [
     (fo.Q4_K, "q4_k_test_block", "q4_k_golden"),
+    (fo.Q5_K, "q5_k_test_block", "q5_k_golden"),
     (fo.Q6_K, "q6_k_test_block", "q6_k_golden"),
     (fo.Q6_K, "q6_k_signed_scales_test_block", "q6_k_signed_scales_golden"),
     (fo.Q6_K, "q6_k_signed_test_block", "q6_k_signed_golden"),
@@ -184,13 +195,13 @@ def test_dequant_matches_independent_python_reference(vectors, kind, blk, gold):
     assert np.abs(got - want).max() < 1e-3
 
 
-@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K])
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K])
 def test_block_walk_and_index_formula_decoders_agree_bit_for_bit(kind):
     bb, be = fo.BLOCK[kind]
     for _ in range(64):
         blk = RNG.integers(0, 256, bb, dtype=np.uint8)
         # keep the f16 super-scales finite
-        for off in ((0, 2) if kind == fo.Q4_K else (208,)):
+        for off in ((208,) if kind == fo.Q6_K else (0, 2)):
             blk[off:off + 2] = np.frombuffer(np.float16(RNG.uniform(-0.01, 0.01)).tobytes(), np.uint8)
         walk = fo.dequant(kind, blk)
         elem = np.array([fo.element(kind, blk, i) for i in range(be)], np.float32)
@@ -206,7 +217,7 @@ def test_q8_0_dequant_is_q_times_f16_scale():
 
 
 def test_misaligned_buffers_are_refused():
-    for kind in (fo.Q8_0, fo.Q4_K, fo.Q6_K):
+    for kind in (fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K):
         with pytest.raises(ValueError):
             fo.dequant(kind, np.zeros(5, np.uint8))
 
@@ -214,6 +225,7 @@ def test_misaligned_buffers_are_refused():
 # fused dot == dequant-then-dot (crates/frink-quant/src/lib.rs:6544-6577, 7170-7246)
 @pytest.mark.parametrize("kind,blk,freq,fn", [
     (fo.Q4_K, "q4_k_test_block", 0.017, np.sin),
+    (fo.Q5_K, "q5_k_test_block", 0.019, np.cos),
     (fo.Q6_K, "q6_k_test_block", 0.021, np.cos),
     (fo.Q6_K, "q6_k_signed_test_block", 0.023, np.sin),
     (fo.Q6_K, "q6_k_signed_scales_test_block", 0.023, np.sin),
@@ -232,20 +244,21 @@ def test_q6_k_scalar_dot_matches_python_golden_with_negative_scales(vectors):
     assert abs(got - expected) < 1e-2
 
 
-def _python_order_dot_q4_k(row, x):
-    """dot_q4_k_f32_scalar's summation order in numpy float32, one op at a time."""
+def _python_order_dot(kind, row, x):
+    """dot_q4_k_f32_scalar's / dot_q5_k_f32_scalar's summation order in numpy float32, one op at a time."""
     acc = np.float32(0)
-    w = fo.dequant(fo.Q4_K, row)
+    w = fo.dequant(kind, row)
     for wi, xi in zip(w, x):
         acc = np.float32(acc + np.float32(wi * xi))
     return acc
 
 
-def test_q4_k_f32_dot_is_the_sequential_sum_of_dequantized_products(vectors):
-    row = np.tile(hexbytes(vectors["q4_k_test_block"]), 3)
+@pytest.mark.parametrize("kind,blk", [(fo.Q4_K, "q4_k_test_block"), (fo.Q5_K, "q5_k_test_block")])
+def test_f32_dot_is_the_sequential_sum_of_dequantized_products(vectors, kind, blk):
+    row = np.tile(hexbytes(vectors[blk]), 3)
     x = RNG.standard_normal(768).astype(np.float32)
-    got = np.float32(fo.dot_f32(fo.Q4_K, row, x))
-    assert got.view(np.uint32) == _python_order_dot_q4_k(row, x).view(np.uint32)
+    got = np.float32(fo.dot_f32(kind, row, x))
+    assert got.view(np.uint32) == _python_order_dot(kind, row, x).view(np.uint32)
 
 
 # ---------------------------------------------------------------- activation quantizers
@@ -328,7 +341,7 @@ def _weights(kind, rows, cols, sigma=0.02):
     return fo.encode_matrix(kind, w)
 
 
-@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q6_K])
+@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K])
 def test_int_dot_equals_dequant_dot_in_exact_arithmetic(kind):
     rows, cols = 6, 1024
     bb, be = fo.BLOCK[kind]
@@ -344,6 +357,8 @@ def test_int_dot_equals_dequant_dot_in_exact_arithmetic(kind):
         # dequantizer but not in the int dot, so rebuild the unrounded weights for Q4_K
         if kind == fo.Q4_K:
             wq = _q4_k_exact(row)
+        elif kind == fo.Q5_K:
+            wq = _q5_k_exact(row)
         else:
             wq = fo.dequant(kind, row).astype(np.float64)
             if kind == fo.Q6_K:
@@ -374,6 +389,25 @@ def _q4_k_exact(row):
     return np.concatenate(out)
 
 
+def _q5_k_exact(row):
+    out = []
+    for blk in row.reshape(-1, 176):
+        d = float(blk[0:2].view(np.float16)[0])
+        dmin = float(blk[2:4].view(np.float16)[0])
+        s = blk[4:16].astype(int)
+        qh = blk[16:48].astype(int)
+        for j in range(8):
+            if j < 4:
+                sc, m = s[j] & 63, s[j + 4] & 63
+            else:
+                sc = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4)
+                m = (s[j + 4] >> 4) | ((s[j] >> 6) << 4)
+            qs = blk[48 + (j // 2) * 32:48 + (j // 2) * 32 + 32].astype(int)
+            code = ((qs >> 4) if j & 1 else (qs & 15)) + 16 * ((qh >> j) & 1)
+            out.append(d * sc * code - dmin * m)
+    return np.concatenate(out)
+
+
 def _q6_k_exact(row):
     out = np.empty(row.size // 210 * 256)
     for b, blk in enumerate(row.reshape(-1, 210)):
@@ -391,7 +425,7 @@ def _q6_k_exact(row):
 
 def test_exact_rebuilds_agree_with_the_dequantizers():
     # the float64 rebuilds above are themselves checked against the pinned dequantizers
-    for kind, fn in ((fo.Q4_K, _q4_k_exact), (fo.Q6_K, _q6_k_exact)):
+    for kind, fn in ((fo.Q4_K, _q4_k_exact), (fo.Q5_K, _q5_k_exact), (fo.Q6_K, _q6_k_exact)):
         data = _weights(kind, 2, 512)
         assert np.abs(fn(data) - fo.dequant(kind, data)).max() < 1e-6
 
@@ -399,7 +433,7 @@ def test_exact_rebuilds_agree_with_the_dequantizers():
 # ---------------------------------------------------------------- dispatch level
 # crates/frink-core/src/weight_matrix.rs:4747-5350: apply_batch == N x apply; out is [batch][rows]
 
-@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q6_K])
+@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K])
 @pytest.mark.parametrize("mode", [fo.F32_DOT, fo.INT_DOT])
 def test_gemm_is_batch_times_gemv_and_output_is_batch_major(kind, mode):
     rows, cols, batch = 24, 512, 5
