@@ -11,11 +11,13 @@ namespace frk {
 // ------------------------------------------------------------------ Q4_K x Q8_K
 // dot_q4_k_q8 (crates/frink-quant/src/lib.rs:822-869).  Unit = (block b, pair p): the 32 bytes
 // qs[32p..32p+32] hold sub-block 2p in their low nibbles and 2p+1 in their high nibbles.
-template <int LPR>
-__global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows,
-                                                        int nb, const int8_t *__restrict__ aq,
-                                                        const float *__restrict__ ad,
-                                                        const int16_t *__restrict__ absums, float *__restrict__ y) {
+// Q5_K (dot_q5_k_q8, lib.rs:886-938) is the same walk: 176-byte blocks whose two words behind the
+// header hold the codes' fifth bits -- byte l of them serves weight l of every sub-block, sub-block
+// j through bit j -- and whose nibbles start at word 3.
+template <int LPR, bool Q5>
+__device__ __forceinline__ void gemv_q45_k(const uint8_t *__restrict__ W, size_t row_stride, int rows, int nb,
+                                           const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                           const int16_t *__restrict__ absums, float *__restrict__ y) {
     extern __shared__ uint4 smem[];
     int8_t *sq = reinterpret_cast<int8_t *>(smem);      // nb*256 activation quants
     int *sbs = reinterpret_cast<int *>(sq + nb * 256);  // nb*8 sums over 32
@@ -37,9 +39,21 @@ __global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restric
             const uint8_t *row = W + (size_t)r * row_stride;
             for (int u = l; u < units; u += LPR) {
                 const int b = u >> 2, p = u & 3;
-                const uint4 *blk = reinterpret_cast<const uint4 *>(row + (size_t)b * Q4_K_BYTES);
+                const uint4 *blk = reinterpret_cast<const uint4 *>(row + (size_t)b * (Q5 ? Q5_K_BYTES : Q4_K_BYTES));
                 const uint4 h = blk[0];
-                const uint4 qa = blk[1 + 2 * p], qb = blk[2 + 2 * p];
+                const uint4 qa = blk[(Q5 ? 3 : 1) + 2 * p], qb = blk[(Q5 ? 4 : 2) + 2 * p];
+                // Q5_K: the words of fifth bits that belong to qa (weights 0..15 of a sub-block) and qb
+                const uint4 fa = Q5 ? blk[1] : make_uint4(0u, 0u, 0u, 0u), fb = Q5 ? blk[2] : make_uint4(0u, 0u, 0u, 0u);
+                auto lo_codes = [&](uint32_t q, uint32_t f) {  // sub-block 2p
+                    uint32_t c = q & 0x0f0f0f0fu;
+                    if (Q5) c |= ((f >> (2 * p)) & 0x01010101u) << 4;
+                    return c;
+                };
+                auto hi_codes = [&](uint32_t q, uint32_t f) {  // sub-block 2p + 1
+                    uint32_t c = (q >> 4) & 0x0f0f0f0fu;
+                    if (Q5) c |= ((f >> (2 * p + 1)) & 0x01010101u) << 4;
+                    return c;
+                };
                 const uint4 *a = reinterpret_cast<const uint4 *>(sq + b * 256 + p * 64);
                 const uint4 a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];
                 // 6-bit scales and mins of sub-blocks 2p and 2p+1 (q4_k_scale_min, lib.rs:321-330)
@@ -55,22 +69,22 @@ __global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restric
                 const int sc1 = (scw >> sh) & 0xff, sc2 = (scw >> (sh + 8)) & 0xff;
                 const int m1 = (mw >> sh) & 0xff, m2 = (mw >> (sh + 8)) & 0xff;
                 int is1 = 0, is2 = 0;
-                is1 = dot4(qa.x & 0x0f0f0f0fu, a0.x, is1);
-                is1 = dot4(qa.y & 0x0f0f0f0fu, a0.y, is1);
-                is1 = dot4(qa.z & 0x0f0f0f0fu, a0.z, is1);
-                is1 = dot4(qa.w & 0x0f0f0f0fu, a0.w, is1);
-                is1 = dot4(qb.x & 0x0f0f0f0fu, a1.x, is1);
-                is1 = dot4(qb.y & 0x0f0f0f0fu, a1.y, is1);
-                is1 = dot4(qb.z & 0x0f0f0f0fu, a1.z, is1);
-                is1 = dot4(qb.w & 0x0f0f0f0fu, a1.w, is1);
-                is2 = dot4((qa.x >> 4) & 0x0f0f0f0fu, a2.x, is2);
-                is2 = dot4((qa.y >> 4) & 0x0f0f0f0fu, a2.y, is2);
-                is2 = dot4((qa.z >> 4) & 0x0f0f0f0fu, a2.z, is2);
-                is2 = dot4((qa.w >> 4) & 0x0f0f0f0fu, a2.w, is2);
-                is2 = dot4((qb.x >> 4) & 0x0f0f0f0fu, a3.x, is2);
-                is2 = dot4((qb.y >> 4) & 0x0f0f0f0fu, a3.y, is2);
-                is2 = dot4((qb.z >> 4) & 0x0f0f0f0fu, a3.z, is2);
-                is2 = dot4((qb.w >> 4) & 0x0f0f0f0fu, a3.w, is2);
+                is1 = dot4(lo_codes(qa.x, fa.x), a0.x, is1);
+                is1 = dot4(lo_codes(qa.y, fa.y), a0.y, is1);
+                is1 = dot4(lo_codes(qa.z, fa.z), a0.z, is1);
+                is1 = dot4(lo_codes(qa.w, fa.w), a0.w, is1);
+                is1 = dot4(lo_codes(qb.x, fb.x), a1.x, is1);
+                is1 = dot4(lo_codes(qb.y, fb.y), a1.y, is1);
+                is1 = dot4(lo_codes(qb.z, fb.z), a1.z, is1);
+                is1 = dot4(lo_codes(qb.w, fb.w), a1.w, is1);
+                is2 = dot4(hi_codes(qa.x, fa.x), a2.x, is2);
+                is2 = dot4(hi_codes(qa.y, fa.y), a2.y, is2);
+                is2 = dot4(hi_codes(qa.z, fa.z), a2.z, is2);
+                is2 = dot4(hi_codes(qa.w, fa.w), a2.w, is2);
+                is2 = dot4(hi_codes(qb.x, fb.x), a3.x, is2);
+                is2 = dot4(hi_codes(qb.y, fb.y), a3.y, is2);
+                is2 = dot4(hi_codes(qb.z, fb.z), a3.z, is2);
+                is2 = dot4(hi_codes(qb.w, fb.w), a3.w, is2);
                 const int s1 = sc1 * is1 + sc2 * is2;
                 const int s2 = m1 * sbs[b * 8 + 2 * p] + m2 * sbs[b * 8 + 2 * p + 1];
                 const float da = sd[b];
@@ -81,6 +95,21 @@ __global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restric
         acc = part_sum<LPR>(acc);
         if (l == 0 && r < rows) y[r] = acc;
     }
+}
+
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows,
+                                                        int nb, const int8_t *__restrict__ aq,
+                                                        const float *__restrict__ ad,
+                                                        const int16_t *__restrict__ absums, float *__restrict__ y) {
+    gemv_q45_k<LPR, false>(W, row_stride, rows, nb, aq, ad, absums, y);
+}
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q5_k_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows,
+                                                        int nb, const int8_t *__restrict__ aq,
+                                                        const float *__restrict__ ad,
+                                                        const int16_t *__restrict__ absums, float *__restrict__ y) {
+    gemv_q45_k<LPR, true>(W, row_stride, rows, nb, aq, ad, absums, y);
 }
 
 // ------------------------------------------------------------------ Q6_K x Q8_K
@@ -270,6 +299,16 @@ int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
     FRK_DISPATCH_LPR(lpr, gemv_q4_k_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout.row_stride,
                      (int)w->rows, nb, a.q, a.d, a.bsums, y);
     FRK_LAUNCH_CHECK("gemv_q4_k");
+    return FRK_OK;
+}
+
+int launch_gemv_q5_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    const int lpr = lanes_per_row(nb * 4);
+    const size_t shmem = (size_t)nb * (256 + 8 * 4 + 4);
+    FRK_DISPATCH_LPR(lpr, gemv_q5_k_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout.row_stride,
+                     (int)w->rows, nb, a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("gemv_q5_k");
     return FRK_OK;
 }
 

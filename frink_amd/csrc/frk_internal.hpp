@@ -28,19 +28,22 @@ void clear_error();
 constexpr int QK_K = 256;
 constexpr int Q8_0_BYTES = 34, Q8_0_ELEMS = 32;
 constexpr int Q4_K_BYTES = 144;
+constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
 
 inline int block_bytes(int kind) {
     return kind == FRK_KIND_Q8_0 ? Q8_0_BYTES : kind == FRK_KIND_Q4_K ? Q4_K_BYTES
-         : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : 0;
+         : kind == FRK_KIND_Q5_K ? Q5_K_BYTES : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : 0;
 }
 inline int block_elems(int kind) {
-    return kind == FRK_KIND_Q8_0 ? Q8_0_ELEMS : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K) ? QK_K : 0;
+    return kind == FRK_KIND_Q8_0 ? Q8_0_ELEMS
+         : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K) ? QK_K : 0;
 }
 
 // ---- resident layouts ----
 // Q4_K stays verbatim: a 144-byte block is nine 16-byte words (header + 8 words of nibbles)
-// and every row starts 16-byte aligned.
+// and every row starts 16-byte aligned.  So does Q5_K: 176 bytes are eleven words (header, two of
+// fifth bits, eight of nibbles).
 // Q6_K (210-byte blocks, 2-byte aligned) and Q8_0 (34-byte blocks) are permuted per row into
 // planes so every load is a 16-byte word:
 //   Q6_K row of nb blocks: ql[nb][128] | qh[nb][64] | sc[nb][16] | d[nb] f16, padded to 16
@@ -60,6 +63,8 @@ inline Layout layout_for(int kind, size_t cols) {
     size_t nb = cols / (size_t)block_elems(kind);
     if (kind == FRK_KIND_Q4_K) {
         l.row_stride = nb * Q4_K_BYTES;
+    } else if (kind == FRK_KIND_Q5_K) {
+        l.row_stride = nb * Q5_K_BYTES;
     } else if (kind == FRK_KIND_Q6_K) {
         l.off_a = nb * 128;
         l.off_b = l.off_a + nb * 64;
@@ -114,6 +119,7 @@ struct Q8KActs {  // Q8_K activations in HBM, struct-of-arrays per activation ro
     const int16_t *bsums; // [batch][cols/16]
 };
 int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+int launch_gemv_q5_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 // one-launch kernels (activation quantized inside the GEMV); cols <= 16384
 // rows of at most this many columns have a one-launch Q4_K GEMV

@@ -134,6 +134,33 @@ __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t *__rest
     out[i] = d1 * (float)nib - min1;
 }
 
+// dequant_q5_k (crates/frink-quant/src/lib.rs:424-459): Q4_K's arithmetic on a five-bit code, whose
+// top bit is bit `sub` of qh[within] (the 32 bytes behind the header)
+__global__ __launch_bounds__(256) void dequant_q5_k_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
+                                                           size_t row_stride, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * cols) return;
+    const size_t r = i / cols, c = i % cols;
+    const uint8_t *blk = w + r * row_stride + (c / QK_K) * Q5_K_BYTES;
+    const int e = (int)(c % QK_K), sub = e >> 5, within = e & 31;
+    const uint8_t *s = blk + 4;
+    int sc, m;
+    if (sub < 4) {
+        sc = s[sub] & 63;
+        m = s[sub + 4] & 63;
+    } else {
+        sc = (s[sub + 4] & 0x0F) | ((s[sub - 4] >> 6) << 4);
+        m = (s[sub + 4] >> 4) | ((s[sub] >> 6) << 4);
+    }
+    const float d = f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+    const float dmin = f16_bits_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+    const uint8_t byte = blk[48 + (sub >> 1) * 32 + within];
+    const int code = ((sub & 1) ? (byte >> 4) : (byte & 15)) + 16 * ((blk[16 + within] >> sub) & 1);
+    const float d1 = d * (float)sc;
+    const float min1 = dmin * (float)m;
+    out[i] = d1 * (float)code - min1;
+}
+
 // dequant_q6_k (crates/frink-quant/src/lib.rs:519-552)
 __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
                                                            Layout l, float *__restrict__ out) {
@@ -214,7 +241,7 @@ int launch_quantize_q8_0(const float *x, size_t n, int8_t *q, float *d, hipStrea
 int launch_repack(int kind, const uint8_t *src, uint8_t *dst, size_t rows, size_t cols, const Layout &l,
                   hipStream_t s) {
     const size_t src_row_bytes = cols / (size_t)block_elems(kind) * (size_t)block_bytes(kind);
-    if (kind == FRK_KIND_Q4_K) {
+    if (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K) {
         hipError_t e = hipMemcpyAsync(dst, src, rows * src_row_bytes, hipMemcpyDeviceToDevice, s);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipMemcpyAsync(weights): %s", hipGetErrorString(e));
         return FRK_OK;
@@ -234,6 +261,10 @@ int launch_dequant(const frk_weights *w, float *out, hipStream_t s) {
     switch (w->kind) {
     case FRK_KIND_Q4_K:
         hipLaunchKernelGGL(dequant_q4_k_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols,
+                           w->layout.row_stride, out);
+        break;
+    case FRK_KIND_Q5_K:
+        hipLaunchKernelGGL(dequant_q5_k_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols,
                            w->layout.row_stride, out);
         break;
     case FRK_KIND_Q6_K:

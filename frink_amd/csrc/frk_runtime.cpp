@@ -184,6 +184,7 @@ const char *frk_hip_matvec_kernel(int kind) {
     switch (kind) {
     case FRK_KIND_Q8_0: return "Q8_0";
     case FRK_KIND_Q4_K: return "Q4_K";
+    case FRK_KIND_Q5_K: return "Q5_K";
     case FRK_KIND_Q6_K: return "Q6_K";
     }
     return nullptr;
@@ -343,12 +344,14 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q4_K:
         if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
         [[fallthrough]];
+    case FRK_KIND_Q5_K:
     case FRK_KIND_Q6_K: {
         if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, &a);
         if (rc) return rc;
         if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, s);
+        if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, s);
         return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, s) : launch_gemv_q6_k(w, a, y, s);
     }
     case FRK_KIND_Q8_0: {
@@ -376,10 +379,11 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     if (w->kind == FRK_KIND_Q4_K)
         return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
                                   : launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
+    if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, (hipStream_t)stream);
     if (w->kind == FRK_KIND_Q6_K)
         return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, (hipStream_t)stream)
                                    : launch_gemv_q6_k(w, a, y, (hipStream_t)stream);
-    return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K and Q6_K weights only (kind %d)", w->kind);
+    return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d)", w->kind);
 }
 
 int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *y, void *stream) {
@@ -425,6 +429,20 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         }
         return FRK_OK;
     }
+    // Q5_K has no batched kernel (gemm_supported says so): the batch is quantized once and every row
+    // takes the decode kernel
+    if (w->kind == FRK_KIND_Q5_K) {
+        Q8KActs a;
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
+        if (rc) return rc;
+        const size_t nb = w->cols / QK_K;
+        for (size_t b = 0; b < batch; b++) {
+            Q8KActs c = {a.q + b * w->cols, a.d + b * nb, a.bsums + b * nb * 16};
+            rc = launch_gemv_q5_k(w, c, y + b * w->rows, (hipStream_t)stream);
+            if (rc) return rc;
+        }
+        return FRK_OK;
+    }
     // otherwise one matvec per activation row (the reference's own path below its GEMM threshold,
     // crates/frink-core/src/weight_matrix.rs:2636-2652)
     for (size_t b = 0; b < batch; b++) {
@@ -445,7 +463,7 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
         if (ws[i]->cols != ws[0]->cols)
             return set_error(FRK_ERR_SHAPE, "matrix %zu has %zu columns, matrix 0 has %zu: they share one activation", i,
                              ws[i]->cols, ws[0]->cols);
-        any_k = any_k || ws[i]->kind == FRK_KIND_Q4_K || ws[i]->kind == FRK_KIND_Q6_K;
+        any_k = any_k || ws[i]->kind == FRK_KIND_Q4_K || ws[i]->kind == FRK_KIND_Q5_K || ws[i]->kind == FRK_KIND_Q6_K;
     }
     // Where every matrix has a one-launch GEMV that quantizes the activation inside the kernel (in
     // the shadow of its first weight loads), sharing a quantization launch is slower than not having

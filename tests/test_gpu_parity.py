@@ -53,6 +53,7 @@ def assert_rows_close(got, want, what):
 
 @pytest.mark.parametrize("kind,rows,cols", [
     (fo.Q4_K, 33, 4096), (fo.Q4_K, 5, 256), (fo.Q4_K, 7, 768),
+    (fo.Q5_K, 33, 4096), (fo.Q5_K, 5, 256), (fo.Q5_K, 7, 768),
     (fo.Q6_K, 9, 14336), (fo.Q6_K, 5, 256), (fo.Q6_K, 3, 768),
     (fo.Q8_0, 17, 4096), (fo.Q8_0, 4, 32), (fo.Q8_0, 3, 96),
 ])
@@ -68,7 +69,7 @@ def test_dequant_is_bit_exact(fa, kind, rows, cols):
 def test_dequant_of_arbitrary_block_bytes_is_bit_exact(fa):
     # any byte pattern is a structurally valid block; only the f16 super-scales are kept finite
     rng = np.random.default_rng(7)
-    for kind, offs in ((fo.Q4_K, (0, 2)), (fo.Q6_K, (208,)), (fo.Q8_0, (0,))):
+    for kind, offs in ((fo.Q4_K, (0, 2)), (fo.Q5_K, (0, 2)), (fo.Q6_K, (208,)), (fo.Q8_0, (0,))):
         bb, be = fo.BLOCK[kind]
         rows, nb = 6, 4
         data = rng.integers(0, 256, rows * nb * bb, dtype=np.uint8).reshape(rows * nb, bb)
@@ -82,7 +83,8 @@ def test_dequant_of_arbitrary_block_bytes_is_bit_exact(fa):
 
 
 def test_dequant_of_the_reference_golden_blocks(fa, vectors):
-    for kind, blk, gold in ((fo.Q4_K, "q4_k_test_block", "q4_k_golden"), (fo.Q6_K, "q6_k_test_block", "q6_k_golden"),
+    for kind, blk, gold in ((fo.Q4_K, "q4_k_test_block", "q4_k_golden"), (fo.Q5_K, "q5_k_test_block", "q5_k_golden"),
+                            (fo.Q6_K, "q6_k_test_block", "q6_k_golden"),
                             (fo.Q6_K, "q6_k_signed_scales_test_block", "q6_k_signed_scales_golden"),
                             (fo.Q6_K, "q6_k_signed_test_block", "q6_k_signed_golden")):
         data = np.frombuffer(bytes.fromhex(vectors[blk]), np.uint8)
@@ -154,6 +156,7 @@ def test_quantize_q8_0_is_bit_exact(fa):
 GEMV_SHAPES = [
     (fo.Q4_K, 64, 4096), (fo.Q4_K, 37, 4096), (fo.Q4_K, 19, 2048), (fo.Q4_K, 21, 768), (fo.Q4_K, 9, 256),
     (fo.Q4_K, 6, 14336),
+    (fo.Q5_K, 64, 4096), (fo.Q5_K, 37, 4096), (fo.Q5_K, 19, 2048), (fo.Q5_K, 21, 768), (fo.Q5_K, 9, 256), (fo.Q5_K, 6, 14336),
     (fo.Q6_K, 48, 14336), (fo.Q6_K, 13, 4096), (fo.Q6_K, 11, 768), (fo.Q6_K, 9, 256), (fo.Q6_K, 5, 2048),
     (fo.Q8_0, 64, 4096), (fo.Q8_0, 7, 32), (fo.Q8_0, 9, 544), (fo.Q8_0, 5, 2048),
 ]
@@ -189,7 +192,7 @@ def test_gemv_outliers_and_zero_activation(fa):
     assert not w.gemv(to_dev(z)).cpu().numpy().any()
 
 
-@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K, fo.Q8_0])
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q8_0])
 def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
     from frink_amd import synth
     rows, cols = 24, 1024
@@ -206,6 +209,41 @@ def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
     got2 = fa.launch_matvec(kind, data, x, rows, cols // be * bb)
     want2 = fo.gemv(kind, data2, rows, cols, x, fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT)
     assert_rows_close(got2[None], want2[None], "launch_matvec after the host bytes changed")
+
+
+def test_q5_k_decode_at_full_size_and_its_batches(fa):
+    """Q5_K (Q4_K's scale packing, a fifth bit per code from a separate plane) has a decode kernel: the
+    FFN shape against the oracle on slices of rows, the whole output against dequantized weights in
+    float64, arbitrary block bytes (every bit pattern of the fifth-bit plane), and a batch -- one
+    quantization, the decode kernel per row -- equal to the single rows bit for bit."""
+    from frink_amd import synth
+    rows, cols = 14336, 4096
+    data = _random_q5_k(rows, cols, 41)
+    w = fa.Weights.from_host(fo.Q5_K, data, rows, cols)
+    x = synth.activations(42, 3, cols, outlier_frac=0.01)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert got.shape == (3, rows)
+    for row0 in (0, 7000, rows - 64):
+        want = fo.gemm(fo.Q5_K, data, rows, cols, x, row0=row0, nrows=64)
+        assert_rows_close(got[:, row0:row0 + 64], want, "q5_k rows %d.." % row0)
+    for b in range(3):
+        one = w.gemv(to_dev(x[b])).cpu().numpy()
+        assert np.array_equal(bits(one), bits(got[b]))
+    wd = w.dequant().cpu().numpy().astype(np.float64)
+    q, d, _ = fo.quantize_q8_k(x[0])
+    xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), 256)
+    ref = wd @ xa
+    assert np.abs(got[0] - ref).max() <= 1e-3 * np.abs(ref).max()
+    w.release()
+
+
+def _random_q5_k(rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    nb = rows * cols // 256
+    data = rng.integers(0, 256, nb * 176, dtype=np.uint8).reshape(nb, 176)
+    data[:, 0:2] = rng.uniform(1e-4, 1e-3, nb).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    data[:, 2:4] = rng.uniform(1e-4, 1e-3, nb).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return data.ravel()
 
 
 def test_gemm_entry_point_is_batch_major(fa):
@@ -657,7 +695,7 @@ def _ffn_oracle(gate, up, down, ffn, hidden, x):
 def test_gemv_multi_shares_one_quantized_activation(fa):
     from frink_amd import synth
     hidden = 1024
-    shapes = [(fo.Q4_K, 96), (fo.Q6_K, 40), (fo.Q8_0, 72), (fo.Q4_K, 33)]
+    shapes = [(fo.Q4_K, 96), (fo.Q6_K, 40), (fo.Q8_0, 72), (fo.Q5_K, 24), (fo.Q4_K, 33)]
     datas = [make_weights(k, r, hidden, seed=300 + i) for i, (k, r) in enumerate(shapes)]
     ws = [fa.Weights.from_host(k, d, r, hidden) for (k, r), d in zip(shapes, datas)]
     x = synth.activations(301, 1, hidden, outlier_frac=0.01)[0]
