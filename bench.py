@@ -45,7 +45,7 @@ def random_blocks(kind, rows, cols, seed):
 
     def f16(lo, hi):
         return rng.uniform(lo, hi, nb).astype(np.float16).view(np.uint8).reshape(nb, 2)
-    if kind == 12:      # Q4_K: d, dmin
+    if kind in (12, 13):  # Q4_K, Q5_K: d, dmin
         data[:, 0:2] = f16(1e-4, 3e-4)
         data[:, 2:4] = f16(1e-3, 3e-3)
     elif kind == 14:    # Q6_K: d
@@ -202,7 +202,8 @@ def main():
         extra["copy_33MB_read_plus_write_GBs"] = round(2 * wbytes / (t / 800) / 1e9, 1)
         del src, dst
         for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
-                                 ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096)):
+                                 ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
+                                 ("Q5_K GEMV 14336x4096 (quantization + decode kernel)", fa.Q5_K, 14336, 4096)):
             d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
             n_copies = COPIES if k2 != fa.Q8_0 else 32
             w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]
