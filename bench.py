@@ -304,12 +304,15 @@ def main():
         h8 = torch.from_numpy(synth.activations(10, 8, rows)).to(dev)
         y8 = torch.empty((8, rows), dtype=torch.float32, device=dev)
         z8 = torch.empty((8, cols), dtype=torch.float32, device=dev)
+        d5 = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=80)).to(dev)
+        q5 = [fa.Weights.from_device(fa.Q5_K, d5, rows, cols) for _ in range(8)]
         for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096", g8, x8, y8),
-                                      ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8)):
+                                      ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8),
+                                      ("Q5_K thin GEMM M=8 14336x4096", q5, x8, y8)):
             def step5(i, mats=mats, xin=xin, yout=yout):
                 mats[i % 8].gemm(xin, out=yout)
             _, t = time_graph(torch, step5, 400, 200)
-            wb = mats[0].rows * (mats[0].cols // 256) * (144 if mats[0].kind == kind else 210)
+            wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
             extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
                            "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
         yf = torch.empty(cols, dtype=torch.float32, device=dev)
@@ -321,7 +324,7 @@ def main():
         extra["decode FFN 4096->14336->4096 (gate, up Q4_K; down Q6_K)"] = {
             "us_per_step": round(t / 400 * 1e6, 2), "GBs": round(fb / (t / 400) / 1e9, 1),
             "frac_of_hbm_peak": round(fb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
-        for w in g8 + u8 + dn:
+        for w in g8 + u8 + dn + q5:
             w.release()
         # q/k/v of a Llama-3-8B layer (4096, 1024 and 1024 rows of 4096): one launch for the three;
         # 40 sets of weights in turn (566 MB > the 256 MB Infinity Cache)

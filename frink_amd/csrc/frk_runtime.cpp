@@ -190,7 +190,9 @@ const char *frk_hip_matvec_kernel(int kind) {
     return nullptr;
 }
 int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
-int frk_hip_gemm_supported(int kind) { return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0; }
+int frk_hip_gemm_supported(int kind) {
+    return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0;
+}
 int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
 int frk_hip_block_elems(int kind) { return block_elems(kind); }
 int frk_hip_worth_a_gemm(size_t batch) { return batch >= 2; }
@@ -413,7 +415,8 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
-    const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q6_K) && batch >= 2 ? thin_gemm_max_batch(w) : 0;
+    const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K) && batch >= 2
+                         ? thin_gemm_max_batch(w) : 0;
     if (thin >= 2) {
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
@@ -429,8 +432,8 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         }
         return FRK_OK;
     }
-    // Q5_K has no batched kernel (gemm_supported says so): the batch is quantized once and every row
-    // takes the decode kernel
+    // Q5_K rows too long for the thin kernel's LDS: the batch is quantized once and every row takes the
+    // decode kernel
     if (w->kind == FRK_KIND_Q5_K) {
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);

@@ -338,18 +338,22 @@ typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
 
 constexpr int TM_WAVES = 8;
 constexpr int TM_AHEAD = 4;                    // blocks of a wavefront in flight
-constexpr int TM_WBLOCK = 16 * Q4_K_BYTES;     // 2304: one block of 16 rows
+// one block of 16 rows: 2304 bytes of Q4_K, 2816 of Q5_K
+__host__ __device__ constexpr int tm_wblock(bool q5) { return 16 * (q5 ? Q5_K_BYTES : Q4_K_BYTES); }
 // LDS rows of the activations are padded so that the 16 rows a read touches fall in different banks
 __host__ __device__ constexpr int tm_q_stride(int cols) { return cols + 16; }
 __host__ __device__ constexpr int tm_bs_stride(int cols) { return cols / 8 + 8; }  // f16 sums, bytes
-__host__ __device__ inline size_t tm_lds_bytes(int acts, int cols) {
+__host__ __device__ inline size_t tm_lds_bytes(int acts, int cols, bool q5) {
     return (size_t)acts * (tm_q_stride(cols) + tm_bs_stride(cols)) + (size_t)(cols / QK_K) * 64 +
-           (size_t)TM_WAVES * TM_WBLOCK;
+           (size_t)TM_WAVES * tm_wblock(q5);
 }
 
 // (at most 4 wavefronts per SIMD: without the bound the compiler aims for 7, with 72 registers,
 // and keeps the ring in scratch memory)
-template <int RG, int ACTS>
+// Q5: the weights are Q5_K -- the same super-block with 32 bytes of fifth bits between the header and
+// the nibbles (11 sixteen-byte pieces a row instead of 9); byte l of them serves weight l of every
+// sub-block, sub-block j through bit j (dot_q5_k_q8, crates/frink-quant/src/lib.rs:886-938).
+template <int RG, int ACTS, bool Q5>
 __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2, 4))) void thin_mfma_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride,
                                                                         int rows, int nb, int batch,
                                                                         const int8_t *__restrict__ aq,
@@ -357,6 +361,10 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
                                                                         const int16_t *__restrict__ absums,
                                                                         float *__restrict__ y) {
     constexpr int KS = TM_WAVES / RG;
+    constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES;  // bytes of a block
+    constexpr int PR = BB / 16, NP = 16 * PR;         // 16-byte pieces of a row's block, of 16 rows' blocks
+    constexpr int QS = Q5 ? 48 : 16;                  // where the nibbles start
+    constexpr int WBLOCK = tm_wblock(Q5);
     extern __shared__ uint4 smem[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
     const int cols = nb * QK_K;
@@ -364,7 +372,7 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     uint8_t *lds_q = lds;                                     // [ACTS][q_stride]
     uint8_t *lds_bs = lds_q + (size_t)ACTS * q_stride;        // [ACTS][bs_stride] f16
     float *lds_d = reinterpret_cast<float *>(lds_bs + (size_t)ACTS * bs_stride);  // [nb][16]
-    uint8_t *lds_w = reinterpret_cast<uint8_t *>(lds_d + (size_t)nb * 16);        // [wave][2304]
+    uint8_t *lds_w = reinterpret_cast<uint8_t *>(lds_d + (size_t)nb * 16);        // [wave][WBLOCK]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int j = lane & 15, g = lane >> 4;
@@ -372,22 +380,22 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     const int row0 = (blockIdx.x * RG + rgrp) * 16;
     const int my_blocks = nb > ksp ? (nb - ksp + KS - 1) / KS : 0;
 
-    // ---- this wavefront's weight stream: piece p = 64*c + lane of chunk c is row p/9, piece p%9 ----
+    // ---- this wavefront's weight stream: piece p = 64*c + lane of chunk c is row p/PR, piece p%PR ----
     const uint8_t *w_src[3];
 #pragma unroll
     for (int c = 0; c < 3; c++) {
-        const int p = min(64 * c + lane, 143);
-        w_src[c] = W + (size_t)min(row0 + p / 9, rows - 1) * row_stride + (p % 9) * 16 + (size_t)ksp * Q4_K_BYTES;
+        const int p = min(64 * c + lane, NP - 1);
+        w_src[c] = W + (size_t)min(row0 + p / PR, rows - 1) * row_stride + (p % PR) * 16 + (size_t)ksp * BB;
     }
     struct Raw {
         uint4 a, b, c;
     };
     auto fetch_block = [&](int i) {  // (past the last block: the last one again, never used)
-        const size_t off = (size_t)KS * max(min(i, my_blocks - 1), 0) * Q4_K_BYTES;
+        const size_t off = (size_t)KS * max(min(i, my_blocks - 1), 0) * BB;
         Raw R;
         R.a = *reinterpret_cast<const uint4 *>(w_src[0] + off);
         R.b = *reinterpret_cast<const uint4 *>(w_src[1] + off);
-        R.c = *reinterpret_cast<const uint4 *>(w_src[2] + off);  // lanes 16.. repeat piece 143
+        R.c = *reinterpret_cast<const uint4 *>(w_src[2] + off);  // lanes NP-128.. repeat the last piece
         return R;
     };
     static_assert(TM_AHEAD == 4, "the ring is four named buffers");
@@ -465,15 +473,15 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     const uint8_t *a_q = lds_q + (size_t)act * q_stride + 8 * g;
     const uint8_t *a_bs = lds_bs + (size_t)act * bs_stride + 8 * g;
     const float *a_d = lds_d + 4 * g;
-    uint8_t *area = lds_w + (size_t)wave * TM_WBLOCK;
-    const uint8_t *a_w = area + j * Q4_K_BYTES;
+    uint8_t *area = lds_w + (size_t)wave * WBLOCK;
+    const uint8_t *a_w = area + j * BB;
     auto as_long = [](uint2 v) { return (long)(((unsigned long)v.y << 32) | v.x); };
     v4f_t acc = {0.f, 0.f, 0.f, 0.f};
     auto multiply_block = [&](int i, Raw R) {  // returns the block that takes this one's place in the ring
         const int kb = ksp + KS * i;
         reinterpret_cast<uint4 *>(area)[lane] = R.a;
         reinterpret_cast<uint4 *>(area)[64 + lane] = R.b;
-        if (lane < 16) reinterpret_cast<uint4 *>(area)[128 + lane] = R.c;
+        if (lane < NP - 128) reinterpret_cast<uint4 *>(area)[128 + lane] = R.c;
         R = fetch_block(i + TM_AHEAD);  // the registers are free again
         const uint4 h = *reinterpret_cast<const uint4 *>(a_w);
         // 6-bit scales and mins (q4_k_scale_min, lib.rs:321-330): bytes of sc_lo/m_lo are sub-blocks
@@ -484,15 +492,21 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
         v4i_t s1 = {0, 0, 0, 0};
         const v4i_t zero = {0, 0, 0, 0};
         const uint8_t *aq_k = a_q + (size_t)kb * QK_K;
+        // Q5_K: the fifth bits of this lane's eight weights, of every sub-block
+        const uint2 f = Q5 ? *reinterpret_cast<const uint2 *>(a_w + 16 + 8 * g) : make_uint2(0u, 0u);
 #pragma unroll
         for (int c = 0; c < 4; c++) {  // sub-blocks 2c (low nibbles) and 2c+1 (high)
-            const uint2 q = *reinterpret_cast<const uint2 *>(a_w + 16 + 32 * c + 8 * g);
+            const uint2 q = *reinterpret_cast<const uint2 *>(a_w + QS + 32 * c + 8 * g);
             const uint2 alo = *reinterpret_cast<const uint2 *>(aq_k + 64 * c);
             const uint2 ahi = *reinterpret_cast<const uint2 *>(aq_k + 64 * c + 32);
             const uint32_t scw = (c < 2 ? sc_lo : sc_hi) >> (16 * (c & 1));
             const int sc0 = scw & 0xff, sc1 = (scw >> 8) & 0xff;
-            const uint2 lo = make_uint2(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu);
-            const uint2 hi = make_uint2((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu);
+            uint2 lo = make_uint2(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu);
+            uint2 hi = make_uint2((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu);
+            if (Q5) {
+                lo.x |= ((f.x >> (2 * c)) & 0x01010101u) << 4, lo.y |= ((f.y >> (2 * c)) & 0x01010101u) << 4;
+                hi.x |= ((f.x >> (2 * c + 1)) & 0x01010101u) << 4, hi.y |= ((f.y >> (2 * c + 1)) & 0x01010101u) << 4;
+            }
             const v4i_t t0 = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(alo), as_long(lo), zero, 0, 0, 0);
             const v4i_t t1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(ahi), as_long(hi), zero, 0, 0, 0);
 #pragma unroll
@@ -797,26 +811,31 @@ static int launch_thin_nb(const frk_weights *w, int batch, Q8KActs a, float *y, 
 
 constexpr size_t TM_LDS_LIMIT = 160 * 1024;
 
-template <int RG, int ACTS>
-static int launch_thin_mfma(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
-    const size_t shmem = tm_lds_bytes(ACTS, (int)w->cols);
+template <int RG, int ACTS, bool Q5>
+static int launch_thin_mfma_kind(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t shmem = tm_lds_bytes(ACTS, (int)w->cols, Q5);
     static bool sized = false;
     if (!sized) {
-        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_mfma_q4_k_kernel<RG, ACTS>),
+        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_mfma_q4_k_kernel<RG, ACTS, Q5>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)TM_LDS_LIMIT));
         sized = true;
     }
     const size_t groups = (w->rows + 15) / 16;
-    hipLaunchKernelGGL((thin_mfma_q4_k_kernel<RG, ACTS>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
+    hipLaunchKernelGGL((thin_mfma_q4_k_kernel<RG, ACTS, Q5>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
                        shmem, s, w->dev, w->layout.row_stride, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d,
                        a.bsums, y);
     FRK_LAUNCH_CHECK("thin mfma gemm");
     return FRK_OK;
 }
-// rows of activations the matrix-core kernel can stage for this matrix (16, 8, 4 or 0)
+template <int RG, int ACTS>
+static int launch_thin_mfma(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    return w->kind == FRK_KIND_Q5_K ? launch_thin_mfma_kind<RG, ACTS, true>(w, batch, a, y, s)
+                                    : launch_thin_mfma_kind<RG, ACTS, false>(w, batch, a, y, s);
+}
+// rows of activations the matrix-core kernel can stage for this Q4_K or Q5_K matrix (16, 8, 4 or 0)
 static int thin_mfma_acts(const frk_weights *w) {
     for (int acts = 16; acts >= 4; acts /= 2)
-        if (tm_lds_bytes(acts, (int)w->cols) <= TM_LDS_LIMIT) return acts;
+        if (tm_lds_bytes(acts, (int)w->cols, w->kind == FRK_KIND_Q5_K) <= TM_LDS_LIMIT) return acts;
     return 0;
 }
 template <int ACTS>
@@ -872,7 +891,8 @@ static int launch_thin_mfma6_rg(const frk_weights *w, int batch, Q8KActs a, floa
 // Largest number of activation rows one launch can take for this matrix: up to 16 on the
 // matrix-core path (Q4_K), else what fits LDS, at most 8.
 int thin_gemm_max_batch(const frk_weights *w) {
-    if (w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0) return thin_mfma_acts(w);
+    if ((w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K) && thin_mfma_acts(w) > 0) return thin_mfma_acts(w);
+    if (w->kind == FRK_KIND_Q5_K) return 0;  // (no other batched kernel for Q5_K)
     const size_t per_row = (w->cols / QK_K) * (256 + (w->kind == FRK_KIND_Q4_K ? 8 : 16) * 4 + 4);
     for (int nbatch = 8; nbatch >= 2; nbatch /= 2)
         if (per_row * nbatch <= THIN_LDS_LIMIT) return nbatch;
@@ -890,7 +910,8 @@ int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, 
 
 // y[batch][rows] for 1 <= batch <= thin_gemm_max_batch(w) quantized activation rows (K-quants).
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
-    if (w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0 && batch > 2) {  // (two rows: the dot4 kernel is still ahead)
+    // (two rows of Q4_K: the dot4 kernel is still ahead)
+    if ((w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0 && batch > 2) || w->kind == FRK_KIND_Q5_K) {
         // the fewest staged rows that hold the batch
         if (batch <= 4) return launch_thin_mfma_rg<4>(w, batch, a, y, s);
         if (batch <= 8) return launch_thin_mfma_rg<8>(w, batch, a, y, s);

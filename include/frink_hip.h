@@ -175,8 +175,7 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
 
 /* y[batch][rows] = x[batch][cols] W^T (WeightMatrix::apply_batch_with_acts,
  * crates/frink-core/src/weight_matrix.rs:2481).  Any batch >= 1.  Q4_K and Q6_K multiply Q8_K
- * activations at every batch size; so does Q5_K, which has a decode kernel only (gemm_supported is
- * false for it): its batch is quantized once and takes that kernel row by row.  Q8_0 follows the reference's host: one row is the f32 dot of its
+ * activations at every batch size, and so does Q5_K (16 rows per launch of its batched kernel).  Q8_0 follows the reference's host: one row is the f32 dot of its
  * decode path (FRK_ACT_F32), two or more rows are quantized to Q8_0 activation blocks and multiplied
  * as integers (weight_matrix.rs:2701-2829, the arithmetic of FRK_ACT_Q8). */
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,

@@ -211,29 +211,40 @@ def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
     assert_rows_close(got2[None], want2[None], "launch_matvec after the host bytes changed")
 
 
-def test_q5_k_decode_at_full_size_and_its_batches(fa):
-    """Q5_K (Q4_K's scale packing, a fifth bit per code from a separate plane) has a decode kernel: the
-    FFN shape against the oracle on slices of rows, the whole output against dequantized weights in
-    float64, arbitrary block bytes (every bit pattern of the fifth-bit plane), and a batch -- one
-    quantization, the decode kernel per row -- equal to the single rows bit for bit."""
+def test_q5_k_decode_and_batches_at_full_size(fa):
+    """Q5_K (Q4_K's scale packing, a fifth bit per code from a separate plane): the FFN shape with
+    arbitrary block bytes (every bit pattern of the fifth-bit plane) against the oracle on slices of
+    rows, for one row (the decode kernel), 3, 16 and 17 rows (the thin matrix-core kernel, 16 rows a
+    launch), and the whole output of a row against dequantized weights in float64."""
     from frink_amd import synth
     rows, cols = 14336, 4096
     data = _random_q5_k(rows, cols, 41)
     w = fa.Weights.from_host(fo.Q5_K, data, rows, cols)
-    x = synth.activations(42, 3, cols, outlier_frac=0.01)
-    got = w.gemm(to_dev(x)).cpu().numpy()
-    assert got.shape == (3, rows)
-    for row0 in (0, 7000, rows - 64):
-        want = fo.gemm(fo.Q5_K, data, rows, cols, x, row0=row0, nrows=64)
-        assert_rows_close(got[:, row0:row0 + 64], want, "q5_k rows %d.." % row0)
-    for b in range(3):
-        one = w.gemv(to_dev(x[b])).cpu().numpy()
-        assert np.array_equal(bits(one), bits(got[b]))
+    x = synth.activations(42, 17, cols, outlier_frac=0.01)
+    for batch in (1, 3, 16, 17):
+        print("q5_k batch", batch, flush=True)
+        got = w.gemm(to_dev(x[:batch])).cpu().numpy()
+        assert got.shape == (batch, rows)
+        for row0 in (0, 7000, rows - 64):
+            want = fo.gemm(fo.Q5_K, data, rows, cols, x[:batch], row0=row0, nrows=64)
+            assert_rows_close(got[:, row0:row0 + 64], want, "q5_k batch %d rows %d.." % (batch, row0))
+    one = w.gemv(to_dev(x[0])).cpu().numpy()
     wd = w.dequant().cpu().numpy().astype(np.float64)
     q, d, _ = fo.quantize_q8_k(x[0])
     xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), 256)
     ref = wd @ xa
-    assert np.abs(got[0] - ref).max() <= 1e-3 * np.abs(ref).max()
+    assert np.abs(one - ref).max() <= 1e-3 * np.abs(ref).max()
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(72, 512, 2), (33, 768, 5), (100, 256, 16), (50, 2048, 9), (20, 14336, 4)])
+def test_q5_k_thin_batches_on_ragged_shapes(fa, rows, cols, batch):
+    from frink_amd import synth
+    data = make_weights(fo.Q5_K, rows, cols, seed=rows + cols)
+    w = fa.Weights.from_host(fo.Q5_K, data, rows, cols)
+    x = synth.activations(rows, batch, cols, outlier_frac=0.01)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert_rows_close(got, fo.gemm(fo.Q5_K, data, rows, cols, x), "q5_k thin %dx%d batch %d" % (rows, cols, batch))
     w.release()
 
 
@@ -553,7 +564,7 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
     w.release()
 
 
-@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K, fo.Q8_0])
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q8_0])
 def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
     """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
     the matrix cores; wider: 8-row groups, or the MFMA GEMM from 17 rows (Q4_K) or 112 (Q6_K); Q8_0:
