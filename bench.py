@@ -50,7 +50,7 @@ def random_blocks(kind, rows, cols, seed):
         data[:, 2:4] = f16(1e-3, 3e-3)
     elif kind == 14:    # Q6_K: d
         data[:, 208:210] = f16(2e-5, 6e-5)
-    else:               # Q8_0: d
+    else:               # Q8_0, Q4_0: d
         data[:, 0:2] = f16(3e-4, 6e-4)
     return data.reshape(-1)
 
@@ -203,7 +203,8 @@ def main():
         del src, dst
         for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
                                  ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
-                                 ("Q5_K GEMV 14336x4096 (quantization + decode kernel)", fa.Q5_K, 14336, 4096)):
+                                 ("Q5_K GEMV 14336x4096 (quantization + decode kernel)", fa.Q5_K, 14336, 4096),
+                                 ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096)):
             d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
             n_copies = COPIES if k2 != fa.Q8_0 else 32
             w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]

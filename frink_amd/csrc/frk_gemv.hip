@@ -263,6 +263,103 @@ __global__ __launch_bounds__(256) void gemv_q8_0_q8_kernel(const uint8_t *__rest
     }
 }
 
+// ------------------------------------------------------------------ Q4_0
+// Unit = one 32-weight block: 16 bytes of nibbles (byte i: element i low, element i + 16 high) from the
+// quant plane and the block's f16 scale from the scale plane.
+// dot_q4_0_f32 (crates/frink-quant/src/lib.rs:4253-4276): the block's sum of (nibble - 8) * x, then
+// times the scale.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q4_0_f32_kernel(const uint8_t *__restrict__ W, Layout lay, int rows,
+                                                            int nb, const float *__restrict__ x, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    float *sx = reinterpret_cast<float *>(smem);
+    for (int i = threadIdx.x; i < nb * 8; i += 256) smem[i] = reinterpret_cast<const uint4 *>(x)[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * lay.row_stride;
+            for (int u = l; u < nb; u += LPR) {
+                const uint4 qv = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+                const float scale = h2f(*reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)u * 2));
+                const float4 *xv = reinterpret_cast<const float4 *>(sx + u * 32);
+                float s = 0.0f;
+#define FRK_Q4_STEP(c, k)                                                        \
+    {                                                                            \
+        const float4 lo = xv[k], hi = xv[4 + k];                                 \
+        s = fmaf((float)((int)(qv.c & 15) - 8), lo.x, s);                        \
+        s = fmaf((float)((int)((qv.c >> 4) & 15) - 8), hi.x, s);                 \
+        s = fmaf((float)((int)((qv.c >> 8) & 15) - 8), lo.y, s);                 \
+        s = fmaf((float)((int)((qv.c >> 12) & 15) - 8), hi.y, s);                \
+        s = fmaf((float)((int)((qv.c >> 16) & 15) - 8), lo.z, s);                \
+        s = fmaf((float)((int)((qv.c >> 20) & 15) - 8), hi.z, s);                \
+        s = fmaf((float)((int)((qv.c >> 24) & 15) - 8), lo.w, s);                \
+        s = fmaf((float)((int)(qv.c >> 28) - 8), hi.w, s);                       \
+    }
+                FRK_Q4_STEP(x, 0)
+                FRK_Q4_STEP(y, 1)
+                FRK_Q4_STEP(z, 2)
+                FRK_Q4_STEP(w, 3)
+#undef FRK_Q4_STEP
+                acc = fmaf(s, scale, acc);
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
+// dot_q4_0_q8 (crates/frink-quant/src/lib.rs:772-796) against Q8_0 activation blocks: the exact integer
+// sum of (nibble - 8) * qa -- as the dots of the raw nibbles minus eight times the sum of the
+// activation quants -- then acc += (dw * da) * isum.
+template <int LPR>
+__global__ __launch_bounds__(256) void gemv_q4_0_q8_kernel(const uint8_t *__restrict__ W, Layout lay, int rows,
+                                                           int nb, const int8_t *__restrict__ aq,
+                                                           const float *__restrict__ ad, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    float *sd = reinterpret_cast<float *>(smem + nb * 2);
+    for (int i = threadIdx.x; i < nb * 2; i += 256) smem[i] = reinterpret_cast<const uint4 *>(aq)[i];
+    for (int i = threadIdx.x; i < nb; i += 256) sd[i] = ad[i];
+    __syncthreads();
+
+    constexpr int PARTS = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int part = lane / LPR, l = lane % LPR;
+    const long n_waves = (long)gridDim.x * 4;
+    for (long r0 = ((long)blockIdx.x * 4 + (threadIdx.x >> 6)) * PARTS; r0 < rows; r0 += n_waves * PARTS) {
+        const long r = r0 + part;
+        float acc = 0.0f;
+        if (r < rows) {
+            const uint8_t *row = W + (size_t)r * lay.row_stride;
+            for (int u = l; u < nb; u += LPR) {
+                const uint4 qv = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+                const float dw = h2f(*reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)u * 2));
+                const uint4 lo = smem[2 * u], hi = smem[2 * u + 1];  // activation quants 0..15 and 16..31
+                int isum = 0, asum = 0;
+#define FRK_Q4_STEP(c)                                              \
+    isum = dot4(qv.c & 0x0f0f0f0fu, lo.c, isum);                    \
+    isum = dot4((qv.c >> 4) & 0x0f0f0f0fu, hi.c, isum);             \
+    asum = dot4(0x01010101u, lo.c, asum);                           \
+    asum = dot4(0x01010101u, hi.c, asum);
+                FRK_Q4_STEP(x)
+                FRK_Q4_STEP(y)
+                FRK_Q4_STEP(z)
+                FRK_Q4_STEP(w)
+#undef FRK_Q4_STEP
+                acc += (dw * sd[u]) * (float)(isum - 8 * asum);
+            }
+        }
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && r < rows) y[r] = acc;
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 static int lanes_per_row(int units) { return units > 32 ? 64 : units > 16 ? 32 : 16; }
@@ -339,6 +436,26 @@ int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, f
     FRK_DISPATCH_LPR(lpr, gemv_q8_0_q8_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
                      nb, q, d, y);
     FRK_LAUNCH_CHECK("gemv_q8_0_q8");
+    return FRK_OK;
+}
+
+int launch_gemv_q4_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS);
+    const int lpr = lanes_per_row(nb);
+    const size_t shmem = (size_t)nb * 32 * 4;
+    FRK_DISPATCH_LPR(lpr, gemv_q4_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+                     nb, x, y);
+    FRK_LAUNCH_CHECK("gemv_q4_0_f32");
+    return FRK_OK;
+}
+
+int launch_gemv_q4_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS);
+    const int lpr = lanes_per_row(nb);
+    const size_t shmem = (size_t)nb * (32 + 4);
+    FRK_DISPATCH_LPR(lpr, gemv_q4_0_q8_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+                     nb, q, d, y);
+    FRK_LAUNCH_CHECK("gemv_q4_0_q8");
     return FRK_OK;
 }
 

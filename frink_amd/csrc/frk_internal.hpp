@@ -27,16 +27,17 @@ void clear_error();
 // ---- block geometry ----
 constexpr int QK_K = 256;
 constexpr int Q8_0_BYTES = 34, Q8_0_ELEMS = 32;
+constexpr int Q4_0_BYTES = 18;  // 32 weights, like Q8_0
 constexpr int Q4_K_BYTES = 144;
 constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
 
 inline int block_bytes(int kind) {
-    return kind == FRK_KIND_Q8_0 ? Q8_0_BYTES : kind == FRK_KIND_Q4_K ? Q4_K_BYTES
+    return kind == FRK_KIND_Q8_0 ? Q8_0_BYTES : kind == FRK_KIND_Q4_0 ? Q4_0_BYTES : kind == FRK_KIND_Q4_K ? Q4_K_BYTES
          : kind == FRK_KIND_Q5_K ? Q5_K_BYTES : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : 0;
 }
 inline int block_elems(int kind) {
-    return kind == FRK_KIND_Q8_0 ? Q8_0_ELEMS
+    return (kind == FRK_KIND_Q8_0 || kind == FRK_KIND_Q4_0) ? Q8_0_ELEMS
          : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K) ? QK_K : 0;
 }
 
@@ -48,10 +49,11 @@ inline int block_elems(int kind) {
 // planes so every load is a 16-byte word:
 //   Q6_K row of nb blocks: ql[nb][128] | qh[nb][64] | sc[nb][16] | d[nb] f16, padded to 16
 //   Q8_0 row of nb blocks: qs[nb][32] | d[nb] f16, padded to 16
+//   Q4_0 row of nb blocks (18-byte blocks): qs[nb][16] | d[nb] f16, padded to 16
 // Same bytes, same count per block; only their order changes.
 struct Layout {
     size_t row_stride = 0;  // bytes between resident rows
-    size_t off_a = 0;       // Q6_K: qh plane offset in a row; Q8_0: d plane offset
+    size_t off_a = 0;       // Q6_K: qh plane offset in a row; Q8_0, Q4_0: d plane offset
     size_t off_b = 0;       // Q6_K: sc plane offset
     size_t off_c = 0;       // Q6_K: d plane offset
 };
@@ -72,6 +74,9 @@ inline Layout layout_for(int kind, size_t cols) {
         l.row_stride = round_up(l.off_c + nb * 2, 16);
     } else if (kind == FRK_KIND_Q8_0) {
         l.off_a = nb * 32;
+        l.row_stride = round_up(l.off_a + nb * 2, 16);
+    } else if (kind == FRK_KIND_Q4_0) {
+        l.off_a = nb * 16;
         l.row_stride = round_up(l.off_a + nb * 2, 16);
     }
     return l;
@@ -196,5 +201,7 @@ int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, 
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
+int launch_gemv_q4_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_q4_0_q8(const frk_weights *w, const int8_t *q, const float *d, float *y, hipStream_t s);
 
 }  // namespace frk

@@ -101,6 +101,9 @@ __global__ __launch_bounds__(256) void repack_kernel(int kind, const uint8_t *__
     } else if (kind == FRK_KIND_Q8_0) {
         const size_t blk = o / Q8_0_BYTES, w = o % Q8_0_BYTES;
         to = w < 2 ? l.off_a + blk * 2 + w : blk * 32 + (w - 2);
+    } else if (kind == FRK_KIND_Q4_0) {
+        const size_t blk = o / Q4_0_BYTES, w = o % Q4_0_BYTES;
+        to = w < 2 ? l.off_a + blk * 2 + w : blk * 16 + (w - 2);
     } else {
         to = o;
     }
@@ -191,6 +194,22 @@ __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t *__rest
     out[i] = (float)(int8_t)row[c] * scale;
 }
 
+// dequant_q4_0 (crates/frink-quant/src/lib.rs:291-310): byte i of a block holds element i in its low
+// nibble and element i + 16 in its high one
+__global__ __launch_bounds__(256) void dequant_q4_0_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
+                                                           Layout l, float *__restrict__ out) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * cols) return;
+    const size_t r = i / cols, c = i % cols, b = c / Q8_0_ELEMS;
+    const int e = (int)(c % Q8_0_ELEMS);
+    const uint8_t *row = w + r * l.row_stride;
+    const uint8_t *dp = row + l.off_a + b * 2;
+    const float scale = f16_bits_to_f32((uint16_t)(dp[0] | (dp[1] << 8)));
+    const uint8_t byte = row[b * 16 + (e & 15)];
+    const int nib = e < 16 ? (byte & 15) : (byte >> 4);
+    out[i] = (float)(nib - 8) * scale;
+}
+
 // ---- bandwidth calibration kernels ----
 __global__ __launch_bounds__(256) void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
     const size_t stride = (size_t)gridDim.x * 256;
@@ -272,6 +291,9 @@ int launch_dequant(const frk_weights *w, float *out, hipStream_t s) {
         break;
     case FRK_KIND_Q8_0:
         hipLaunchKernelGGL(dequant_q8_0_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols, w->layout, out);
+        break;
+    case FRK_KIND_Q4_0:
+        hipLaunchKernelGGL(dequant_q4_0_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols, w->layout, out);
         break;
     default:
         return set_error(FRK_ERR_UNSUPPORTED, "no dequantizer for quant kind %d", w->kind);

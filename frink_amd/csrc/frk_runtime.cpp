@@ -182,6 +182,7 @@ int frk_hip_dense_enabled(void) {
 
 const char *frk_hip_matvec_kernel(int kind) {
     switch (kind) {
+    case FRK_KIND_Q4_0: return "Q4_0";
     case FRK_KIND_Q8_0: return "Q8_0";
     case FRK_KIND_Q4_K: return "Q4_K";
     case FRK_KIND_Q5_K: return "Q5_K";
@@ -356,9 +357,12 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
         if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, s);
         return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, s) : launch_gemv_q6_k(w, a, y, s);
     }
+    case FRK_KIND_Q4_0:
     case FRK_KIND_Q8_0: {
-        if (act_mode == FRK_ACT_F32)
+        if (act_mode == FRK_ACT_F32) {
+            if (w->kind == FRK_KIND_Q4_0) return launch_gemv_q4_0_f32(w, x, y, s);
             return direct_gemv_fits(w) ? launch_gemv_q8_0_f32_direct(w, x, y, s) : launch_gemv_q8_0_f32(w, x, y, s);
+        }
         size_t n = w->cols;
         void *ws = nullptr;
         int rc = workspace(round_up(n, 256) + n / 32 * 4, s, &ws);
@@ -367,7 +371,7 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
         float *d = (float *)((char *)ws + round_up(n, 256));
         rc = launch_quantize_q8_0(x, n, q, d, s);
         if (rc) return rc;
-        return launch_gemv_q8_0_q8(w, q, d, y, s);
+        return w->kind == FRK_KIND_Q4_0 ? launch_gemv_q4_0_q8(w, q, d, y, s) : launch_gemv_q8_0_q8(w, q, d, y, s);
     }
     }
     return set_error(FRK_ERR_UNSUPPORTED, "no matvec kernel for quant kind %d", w->kind);
@@ -475,7 +479,8 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     for (size_t i = 0; i < n; i++) {
         const frk_weights *w = ws[i];
         all_fused = all_fused && ((w->kind == FRK_KIND_Q4_K && fused_gemv_fits(w)) ||
-                                  (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) || w->kind == FRK_KIND_Q8_0);
+                                  (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) || w->kind == FRK_KIND_Q8_0 ||
+                                  w->kind == FRK_KIND_Q4_0);
     }
     if (all_fused) {
         // Q4_K neighbours go out in one launch, four at most: the kernel walks their rows as one list
@@ -503,7 +508,8 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     }
     for (size_t i = 0; i < n; i++) {
         int rc;
-        if (ws[i]->kind == FRK_KIND_Q8_0) rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
+        if (ws[i]->kind == FRK_KIND_Q8_0 || ws[i]->kind == FRK_KIND_Q4_0)
+            rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
         else rc = frk_hip_gemv_q8k_dev(ws[i], a.q, a.d, a.bsums, ys[i], stream);
         if (rc) return rc;
     }

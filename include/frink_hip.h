@@ -46,7 +46,7 @@ enum {
 
 /* Quant kinds, numbered by ggml type id (crates/frink-gguf/src/lib.rs:236-242).
  * Names are QuantKind::name() (crates/frink-core/src/weight_matrix.rs:264-290). */
-enum { FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q5_K = 13, FRK_KIND_Q6_K = 14 };
+enum { FRK_KIND_Q4_0 = 2, FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q5_K = 13, FRK_KIND_Q6_K = 14 };
 
 /* Q8_0 GEMV arithmetic.  F32 multiplies dequantized weights by the f32
  * activation (dot_q8_0_f32, crates/frink-quant/src/lib.rs:663-686); INT8

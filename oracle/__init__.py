@@ -13,11 +13,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libfrink_oracle.so")
 
-Q8_0, Q4_K, Q5_K, Q6_K = 8, 12, 13, 14
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
 FORM_NEON, FORM_AVX, FORM_SCALAR = 0, 1, 2
 F32_DOT, INT_DOT = 0, 1
 
-BLOCK = {Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
 
 
 def build(force=False):
@@ -48,12 +48,14 @@ def lib():
             "fo_q5_k_element": (C.c_float, [u8p, C.c_int]),
             "fo_q6_k_element": (C.c_float, [u8p, C.c_int]),
             "fo_dot_q8_0_f32": (C.c_float, [u8p, sz, f32p]),
+            "fo_dot_q4_0_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q4_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q5_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q6_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_quantize_q8_k": (None, [f32p, sz, i8p, f32p, i16p]),
             "fo_quantize_q8_0": (None, [f32p, sz, C.c_int, i8p, f32p]),
             "fo_dot_q8_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
+            "fo_dot_q4_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
             "fo_dot_q4_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
             "fo_dot_q5_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
             "fo_dot_q6_k_q8k": (C.c_float, [u8p, sz, i8p, f32p]),
@@ -121,7 +123,7 @@ def element(kind, block, i):
 
 def dot_f32(kind, row, x):
     row, x = _u8(row), _f32(x)
-    fn = {Q8_0: lib().fo_dot_q8_0_f32, Q4_K: lib().fo_dot_q4_k_f32, Q5_K: lib().fo_dot_q5_k_f32,
+    fn = {Q4_0: lib().fo_dot_q4_0_f32, Q8_0: lib().fo_dot_q8_0_f32, Q4_K: lib().fo_dot_q4_k_f32, Q5_K: lib().fo_dot_q5_k_f32,
           Q6_K: lib().fo_dot_q6_k_f32}[kind]
     return fn(_p(row, C.c_uint8), row.size, _p(x, C.c_float))
 
@@ -147,9 +149,10 @@ def quantize_q8_0(x, form=FORM_AVX):
 
 def dot_int(kind, row, acts):
     row = _u8(row)
-    if kind == Q8_0:
+    if kind in (Q8_0, Q4_0):
         q, d = acts
-        return lib().fo_dot_q8_0_q8(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
+        fn = lib().fo_dot_q8_0_q8 if kind == Q8_0 else lib().fo_dot_q4_0_q8
+        return fn(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
     q, d, bs = acts
     if kind in (Q4_K, Q5_K):
         fn = lib().fo_dot_q4_k_q8k if kind == Q4_K else lib().fo_dot_q5_k_q8k

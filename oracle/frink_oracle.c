@@ -28,6 +28,7 @@
 #endif
 
 #define Q8_0_BYTES 34
+#define Q4_0_BYTES 18
 #define Q8_0_ELEMS 32
 #define Q4_K_BYTES 144
 #define Q5_K_BYTES 176
@@ -38,6 +39,7 @@
 int fo_block_bytes(int kind) {
     switch (kind) {
     case FO_KIND_Q8_0: return Q8_0_BYTES;
+    case FO_KIND_Q4_0: return Q4_0_BYTES;
     case FO_KIND_Q4_K: return Q4_K_BYTES;
     case FO_KIND_Q5_K: return Q5_K_BYTES;
     case FO_KIND_Q6_K: return Q6_K_BYTES;
@@ -46,7 +48,7 @@ int fo_block_bytes(int kind) {
 }
 int fo_block_elems(int kind) {
     switch (kind) {
-    case FO_KIND_Q8_0: return Q8_0_ELEMS;
+    case FO_KIND_Q8_0: case FO_KIND_Q4_0: return Q8_0_ELEMS;
     case FO_KIND_Q4_K: case FO_KIND_Q5_K: case FO_KIND_Q6_K: return QK_K;
     }
     return 0;
@@ -125,6 +127,23 @@ void fo_q4_k_scale_min(int j, const uint8_t *s, uint8_t *sc, uint8_t *m) {
         *sc = (uint8_t)((s[j + 4] & 0x0F) | ((s[j - 4] >> 6) << 4));
         *m = (uint8_t)((s[j + 4] >> 4) | ((s[j] >> 6) << 4));
     }
+}
+
+/* src/lib.rs:291-310: block = [d:f16][16 bytes]; byte i holds element i in its low nibble and
+ * element i + 16 in its high nibble; y = (nibble - 8) * d */
+int fo_dequant_q4_0(const uint8_t *src, size_t nbytes, float *out) {
+    if (nbytes % Q4_0_BYTES) return -1;
+    size_t nb = nbytes / Q4_0_BYTES;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = src + b * Q4_0_BYTES;
+        float scale = rd_f16(blk);
+        for (int i = 0; i < 16; i++) {
+            int lo = (int)(blk[2 + i] & 0x0F) - 8, hi = (int)(blk[2 + i] >> 4) - 8;
+            out[b * 32 + i] = (float)lo * scale;
+            out[b * 32 + i + 16] = (float)hi * scale;
+        }
+    }
+    return 0;
 }
 
 /* src/lib.rs:334-364 */
@@ -217,6 +236,7 @@ int fo_dequant_q6_k(const uint8_t *src, size_t nbytes, float *out) {
 int fo_dequant(int kind, const uint8_t *src, size_t nbytes, float *out) {
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dequant_q8_0(src, nbytes, out);
+    case FO_KIND_Q4_0: return fo_dequant_q4_0(src, nbytes, out);
     case FO_KIND_Q4_K: return fo_dequant_q4_k(src, nbytes, out);
     case FO_KIND_Q5_K: return fo_dequant_q5_k(src, nbytes, out);
     case FO_KIND_Q6_K: return fo_dequant_q6_k(src, nbytes, out);
@@ -268,6 +288,24 @@ float fo_dot_q8_0_f32(const uint8_t *row, size_t row_bytes, const float *x) {
         float scale = rd_f16(blk);
         float block_acc = 0.0f;
         for (int i = 0; i < 32; i++) block_acc += (float)(int8_t)blk[2 + i] * x[b * 32 + i];
+        acc += block_acc * scale;
+    }
+    return acc;
+}
+
+/* src/lib.rs:4253-4276 */
+float fo_dot_q4_0_f32(const uint8_t *row, size_t row_bytes, const float *x) {
+    size_t nb = row_bytes / Q4_0_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * Q4_0_BYTES;
+        float scale = rd_f16(blk);
+        float block_acc = 0.0f;
+        for (int i = 0; i < 16; i++) {
+            int lo = (int)(blk[2 + i] & 0x0F) - 8, hi = (int)(blk[2 + i] >> 4) - 8;
+            block_acc += (float)lo * x[b * 32 + i];
+            block_acc += (float)hi * x[b * 32 + i + 16];
+        }
         acc += block_acc * scale;
     }
     return acc;
@@ -431,6 +469,24 @@ float fo_dot_q8_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, cons
         float dw = rd_f16(blk);
         int32_t isum = 0;
         for (int i = 0; i < 32; i++) isum += (int32_t)(int8_t)blk[2 + i] * (int32_t)q[b * 32 + i];
+        acc += dw * d[b] * (float)isum;
+    }
+    return acc;
+}
+
+/* src/lib.rs:772-796: against Q8_0 activation blocks */
+float fo_dot_q4_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d) {
+    size_t nb = row_bytes / Q4_0_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * Q4_0_BYTES;
+        float dw = rd_f16(blk);
+        int32_t isum = 0;
+        for (int i = 0; i < 16; i++) {
+            int32_t q0 = (int32_t)(blk[2 + i] & 0x0F) - 8, q1 = (int32_t)(blk[2 + i] >> 4) - 8;
+            isum += q0 * (int32_t)q[b * 32 + i];
+            isum += q1 * (int32_t)q[b * 32 + 16 + i];
+        }
         acc += dw * d[b] * (float)isum;
     }
     return acc;
@@ -950,15 +1006,16 @@ static int acts_alloc(acts_t *a, int kind, size_t cols, size_t batch) {
     size_t be = (size_t)fo_block_elems(kind);
     a->q = (int8_t *)malloc(batch * cols);
     a->d = (float *)malloc(batch * (cols / be) * sizeof(float));
-    a->bsums = kind == FO_KIND_Q8_0 ? NULL : (int16_t *)malloc(batch * (cols / 16) * sizeof(int16_t));
-    return a->q && a->d && (kind == FO_KIND_Q8_0 || a->bsums) ? 0 : -1;
+    int q8_0_acts = kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0;
+    a->bsums = q8_0_acts ? NULL : (int16_t *)malloc(batch * (cols / 16) * sizeof(int16_t));
+    return a->q && a->d && (q8_0_acts || a->bsums) ? 0 : -1;
 }
 static void acts_free(acts_t *a) { free(a->q); free(a->d); free(a->bsums); }
 
 static void acts_quantize(acts_t *a, int kind, const float *x, size_t cols, size_t batch) {
     size_t be = (size_t)fo_block_elems(kind);
     for (size_t b = 0; b < batch; b++) {
-        if (kind == FO_KIND_Q8_0)
+        if (kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0)
             fo_quantize_q8_0(x + b * cols, cols, FO_Q8_0_FORM_AVX, a->q + b * cols, a->d + b * (cols / be));
         else
             fo_quantize_q8_k(x + b * cols, cols, a->q + b * cols, a->d + b * (cols / be),
@@ -973,6 +1030,7 @@ static inline float row_dot_int(int kind, const uint8_t *row, size_t row_bytes, 
     const float *d = a->d + b * (cols / be);
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_q8(row, row_bytes, q, d);
+    case FO_KIND_Q4_0: return fo_dot_q4_0_q8(row, row_bytes, q, d);
     case FO_KIND_Q4_K: return fo_dot_q4_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
     case FO_KIND_Q5_K: return fo_dot_q5_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
     default: return fo_dot_q6_k_q8k(row, row_bytes, q, d);
@@ -981,6 +1039,7 @@ static inline float row_dot_int(int kind, const uint8_t *row, size_t row_bytes, 
 static inline float row_dot_f32(int kind, const uint8_t *row, size_t row_bytes, const float *x) {
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_f32(row, row_bytes, x);
+    case FO_KIND_Q4_0: return fo_dot_q4_0_f32(row, row_bytes, x);
     case FO_KIND_Q4_K: return fo_dot_q4_k_f32(row, row_bytes, x);
     case FO_KIND_Q5_K: return fo_dot_q5_k_f32(row, row_bytes, x);
     default: return fo_dot_q6_k_f32(row, row_bytes, x);

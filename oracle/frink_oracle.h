@@ -22,7 +22,7 @@ extern "C" {
 
 /* quant kinds; the numbers are the ggml type ids the reference maps from
  * (crates/frink-gguf/src/lib.rs:236-242). */
-enum { FO_KIND_Q8_0 = 8, FO_KIND_Q4_K = 12, FO_KIND_Q5_K = 13, FO_KIND_Q6_K = 14 };
+enum { FO_KIND_Q4_0 = 2, FO_KIND_Q8_0 = 8, FO_KIND_Q4_K = 12, FO_KIND_Q5_K = 13, FO_KIND_Q6_K = 14 };
 
 /* Q8_0 activation forms (crates/frink-quant/src/act_quant.rs:121-127). */
 enum { FO_Q8_0_FORM_NEON = 0, FO_Q8_0_FORM_AVX = 1, FO_Q8_0_FORM_SCALAR = 2 };
@@ -38,6 +38,7 @@ uint16_t fo_f32_to_f16(float f);
 
 /* dequantizers: return 0, or -1 when nbytes is not a whole number of blocks */
 int fo_dequant_q8_0(const uint8_t *src, size_t nbytes, float *out);
+int fo_dequant_q4_0(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q4_k(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q5_k(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q6_k(const uint8_t *src, size_t nbytes, float *out);
@@ -50,6 +51,7 @@ void  fo_q4_k_scale_min(int j, const uint8_t *scales12, uint8_t *sc, uint8_t *m)
 
 /* fused f32 dots (scalar twins) */
 float fo_dot_q8_0_f32(const uint8_t *row, size_t row_bytes, const float *x);
+float fo_dot_q4_0_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q4_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q5_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q6_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
@@ -60,6 +62,7 @@ void fo_quantize_q8_0(const float *x, size_t n, int form, int8_t *q, float *d);
 
 /* integer dots against quantized activations */
 float fo_dot_q8_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
+float fo_dot_q4_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
 float fo_dot_q4_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d,
                       const int16_t *bsums);
 float fo_dot_q5_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d,

@@ -43,11 +43,12 @@ def test_every_kind_the_backend_claims_can_be_launched():
         else:
             assert name is None and fa.lib().frk_hip_block_bytes(kind) == 0
     assert all(fa.lib().frk_hip_gemm_supported(k) for k in (fa.Q4_K, fa.Q5_K, fa.Q6_K, fa.Q8_0))
+    assert not fa.lib().frk_hip_gemm_supported(fa.Q4_0)  # decode kernels only
     assert not fa.lib().frk_hip_worth_a_gemm(1) and fa.lib().frk_hip_worth_a_gemm(2)
 
 
 def test_an_unknown_kind_is_the_none_answer_not_an_error():
-    assert fa.launch_matvec(2, np.zeros(18, np.uint8), np.zeros(32, np.float32), 1, 18) is None
+    assert fa.launch_matvec(3, np.zeros(20, np.uint8), np.zeros(32, np.float32), 1, 20) is None  # Q4_1
 
 
 # crates/frink-core/src/weight_matrix/gpu_backend.rs:1342-1670: a mismatched shape is an error value, never a crash

@@ -248,6 +248,43 @@ def test_q5_k_thin_batches_on_ragged_shapes(fa, rows, cols, batch):
     w.release()
 
 
+def _random_q4_0(rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    nb = rows * cols // 32
+    data = rng.integers(0, 256, nb * 18, dtype=np.uint8).reshape(nb, 18)
+    data[:, 0:2] = rng.uniform(-2e-3, 2e-3, nb).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    return data.ravel()
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (37, 4096), (7, 32), (9, 544), (5, 2048), (4096, 4096)])
+def test_q4_0_dequant_and_decode(fa, rows, cols):
+    """Q4_0 (18-byte blocks: an f16 scale and 16 bytes of nibbles, value (nibble - 8) * d) is kept as a
+    plane of nibbles and a plane of scales.  The reference holds no encoder for it, so the blocks are
+    arbitrary bytes with finite scales: dequantization bit-exact, the f32 dot (decode on an x86 host)
+    and the integer dot against Q8_0 activation blocks within the tolerance, batches row by row."""
+    from frink_amd import synth
+    print("q4_0", rows, cols, flush=True)
+    data = _random_q4_0(rows, cols, rows + cols)
+    w = fa.Weights.from_host(fo.Q4_0, data, rows, cols)
+    assert np.array_equal(bits(w.dequant().cpu().numpy()), bits(fo.dequant(fo.Q4_0, data).reshape(rows, cols)))
+    x = synth.activations(rows * 3 + cols, 3, cols, outlier_frac=0.01)
+    n = min(rows, 64)
+    for row0 in sorted({0, rows - n}):
+        got = w.gemv(to_dev(x[0]), act_mode=fa.ACT_F32).cpu().numpy()
+        want = fo.gemm(fo.Q4_0, data, rows, cols, x[:1], fo.F32_DOT, row0=row0, nrows=n)
+        assert_rows_close(got[None, row0:row0 + n], want, "q4_0 f32 dot")
+        got_i = w.gemv(to_dev(x[0]), act_mode=fa.ACT_INT8).cpu().numpy()
+        want_i = fo.gemm(fo.Q4_0, data, rows, cols, x[:1], fo.INT_DOT, row0=row0, nrows=n)
+        assert_rows_close(got_i[None, row0:row0 + n], want_i, "q4_0 integer dot")
+    yb = w.gemm(to_dev(x)).cpu().numpy()
+    for b in range(3):
+        assert np.array_equal(bits(yb[b]), bits(w.gemv(to_dev(x[b])).cpu().numpy()))
+    bb = fo.BLOCK[fo.Q4_0][0]
+    host = fa.launch_matvec(fo.Q4_0, data, x[0], rows, cols // 32 * bb)
+    assert np.array_equal(bits(host), bits(yb[0]))
+    w.release()
+
+
 def _random_q5_k(rows, cols, seed):
     rng = np.random.default_rng(seed)
     nb = rows * cols // 256

@@ -216,8 +216,47 @@ def test_q8_0_dequant_is_q_times_f16_scale():
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+# crates/frink-quant/src/lib.rs:291-310, 5855-5864, 6277-6295: Q4_0 has no vector in the reference beyond closed forms
+def test_q4_0_dequant_is_nibble_minus_eight_times_f16_scale():
+    blk = np.concatenate([np.frombuffer(np.float16(1.0).tobytes(), np.uint8), np.zeros(16, np.uint8)])
+    assert (fo.dequant(fo.Q4_0, blk) == -8.0).all()  # the reference's own case: nibble 0 is -8 * scale
+    data = RNG.integers(0, 256, 18 * 7, dtype=np.uint8).reshape(7, 18)
+    data[:, 0:2] = np.frombuffer(np.float16([0.01, -0.5, 1.0, 6e-6, 0.0, 3.0, 0.125]).tobytes(), np.uint8).reshape(7, 2)
+    got = fo.dequant(fo.Q4_0, data.ravel()).reshape(7, 32)
+    d = data[:, 0:2].copy().view(np.float16).astype(np.float32)
+    lo = (data[:, 2:] & 15).astype(np.float32) - 8
+    hi = (data[:, 2:] >> 4).astype(np.float32) - 8
+    want = np.concatenate([lo, hi], axis=1) * d  # element i from byte i's low nibble, i + 16 from its high one
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_q4_0_dots_follow_the_dequantized_row():
+    nb = 12
+    data = RNG.integers(0, 256, 18 * nb, dtype=np.uint8).reshape(nb, 18)
+    data[:, 0:2] = RNG.uniform(-0.05, 0.05, nb).astype(np.float16).view(np.uint8).reshape(nb, 2)
+    row = data.ravel()
+    x = RNG.standard_normal(32 * nb).astype(np.float32)
+    w = fo.dequant(fo.Q4_0, row).astype(np.float64)
+    assert abs(fo.dot_f32(fo.Q4_0, row, x) - float(np.dot(w, x.astype(np.float64)))) < 1e-4
+    # f32 order: per block the sum of (nibble - 8) * x, elements i and i + 16 alternating, then times the scale
+    acc = np.float32(0)
+    for b in range(nb):
+        blk = data[b]
+        ba = np.float32(0)
+        for i in range(16):
+            ba = np.float32(ba + np.float32(np.float32(int(blk[2 + i] & 15) - 8) * x[32 * b + i]))
+            ba = np.float32(ba + np.float32(np.float32(int(blk[2 + i] >> 4) - 8) * x[32 * b + i + 16]))
+        acc = np.float32(acc + np.float32(ba * np.float32(blk[0:2].view(np.float16)[0])))
+    assert np.float32(fo.dot_f32(fo.Q4_0, row, x)).view(np.uint32) == acc.view(np.uint32)
+    # integer dot: exact integers times dw * da, in block order
+    q, d = fo.quantize_q8_0(x)
+    xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), 32)
+    want = float(np.dot(w, xa))
+    assert abs(fo.dot_int(fo.Q4_0, row, (q, d)) - want) <= 2e-6 * float(np.abs(w * xa).sum())
+
+
 def test_misaligned_buffers_are_refused():
-    for kind in (fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K):
+    for kind in (fo.Q4_0, fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K):
         with pytest.raises(ValueError):
             fo.dequant(kind, np.zeros(5, np.uint8))
 
