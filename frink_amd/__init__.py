@@ -31,6 +31,7 @@ EXPORTS = [
     "frk_hip_gemm_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
+    "frk_hip_get_rows_dev", "frk_hip_get_rows",
     "frk_hip_copy_dev", "frk_hip_read_dev",
 ]
 
@@ -92,6 +93,8 @@ def lib():
             "frk_hip_quantize_q8_k_dev": (i, [vp, sz, vp, vp, vp, vp]),
             "frk_hip_quantize_q8_0_dev": (i, [vp, sz, vp, vp, vp]),
             "frk_hip_dequant_dev": (i, [vp, vp, vp]),
+            "frk_hip_get_rows_dev": (i, [vp, vp, C.c_size_t, vp, vp]),
+            "frk_hip_get_rows": (i, [vp, vp, C.c_size_t, vp]),
             "frk_hip_copy_dev": (i, [vp, vp, sz, vp]),
             "frk_hip_read_dev": (i, [vp, sz, vp, vp]),
         }
@@ -204,6 +207,29 @@ class Weights:
         out = torch.empty((self.rows, self.cols), dtype=torch.float32, device="cuda")
         check(lib().frk_hip_dequant_dev(self.handle, C.c_void_p(out.data_ptr()), _stream()))
         return out
+
+
+def _get_rows_dev(self, ids):
+    """The embedding gather on device ids (int32 tensor): [len(ids)][cols] f32."""
+    import torch
+    assert ids.dtype == torch.int32 and ids.is_cuda and ids.is_contiguous()
+    out = torch.empty((ids.numel(), self.cols), dtype=torch.float32, device=ids.device)
+    check(lib().frk_hip_get_rows_dev(self.handle, C.c_void_p(ids.data_ptr()), ids.numel(), C.c_void_p(out.data_ptr()),
+                                     _stream()))
+    return out
+
+
+def _get_rows_host(self, ids):
+    """The embedding gather on host ids, every id checked against the table: numpy [len(ids)][cols] f32."""
+    import numpy as np
+    ids = np.ascontiguousarray(ids, np.int32)
+    out = np.empty((ids.size, self.cols), np.float32)
+    check(lib().frk_hip_get_rows(self.handle, _np_ptr(ids), ids.size, _np_ptr(out)))
+    return out
+
+
+Weights.get_rows = _get_rows_dev
+Weights.get_rows_host = _get_rows_host
 
 
 def quantize_q8_k(x):

@@ -113,6 +113,7 @@ hipStream_t own_stream();  // the stream host-buffer entry points run on
 int launch_quantize_q8_k(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s);
 int launch_quantize_q8_0(const float *x, size_t n, int8_t *q, float *d, hipStream_t s);
 int launch_dequant(const frk_weights *w, float *out, hipStream_t s);
+int launch_dequant_rows(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s);
 int launch_repack(int kind, const uint8_t *src, uint8_t *dst, size_t rows, size_t cols, const Layout &l,
                   hipStream_t s);
 int launch_copy(const void *src, void *dst, size_t bytes, hipStream_t s);

@@ -111,12 +111,21 @@ __global__ __launch_bounds__(256) void repack_kernel(int kind, const uint8_t *__
 }
 
 // ---- dequantizers, one thread per element, reading the resident layout ----
+// With a list of row numbers they are the embedding gather (get_rows, crates/frink-cuda/src/get_rows.rs:
+// output row r is the dequantized row ids[r], bit for bit what the dequantizer gives); a number outside
+// the table reads its nearest row instead of faulting (the host-side entry point refuses such lists).
+__device__ __forceinline__ size_t source_row(size_t r, const int32_t *ids, size_t table_rows) {
+    if (!ids) return r;
+    const int32_t id = ids[r];
+    return id < 0 ? 0 : (size_t)id >= table_rows ? table_rows - 1 : (size_t)id;
+}
 // dequant_q4_k (crates/frink-quant/src/lib.rs:334-364)
 __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
-                                                           size_t row_stride, float *__restrict__ out) {
+                                                           size_t row_stride, const int32_t *__restrict__ ids, size_t table_rows,
+                                                           float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * cols) return;
-    const size_t r = i / cols, c = i % cols;
+    const size_t r = source_row(i / cols, ids, table_rows), c = i % cols;
     const uint8_t *blk = w + r * row_stride + (c / QK_K) * Q4_K_BYTES;
     const int e = (int)(c % QK_K), sub = e >> 5, within = e & 31;
     const uint8_t *s = blk + 4;
@@ -140,10 +149,11 @@ __global__ __launch_bounds__(256) void dequant_q4_k_kernel(const uint8_t *__rest
 // dequant_q5_k (crates/frink-quant/src/lib.rs:424-459): Q4_K's arithmetic on a five-bit code, whose
 // top bit is bit `sub` of qh[within] (the 32 bytes behind the header)
 __global__ __launch_bounds__(256) void dequant_q5_k_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
-                                                           size_t row_stride, float *__restrict__ out) {
+                                                           size_t row_stride, const int32_t *__restrict__ ids, size_t table_rows,
+                                                           float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * cols) return;
-    const size_t r = i / cols, c = i % cols;
+    const size_t r = source_row(i / cols, ids, table_rows), c = i % cols;
     const uint8_t *blk = w + r * row_stride + (c / QK_K) * Q5_K_BYTES;
     const int e = (int)(c % QK_K), sub = e >> 5, within = e & 31;
     const uint8_t *s = blk + 4;
@@ -166,10 +176,11 @@ __global__ __launch_bounds__(256) void dequant_q5_k_kernel(const uint8_t *__rest
 
 // dequant_q6_k (crates/frink-quant/src/lib.rs:519-552)
 __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
-                                                           Layout l, float *__restrict__ out) {
+                                                           Layout l, const int32_t *__restrict__ ids, size_t table_rows,
+                                                           float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * cols) return;
-    const size_t r = i / cols, c = i % cols, b = c / QK_K;
+    const size_t r = source_row(i / cols, ids, table_rows), c = i % cols, b = c / QK_K;
     const uint8_t *row = w + r * l.row_stride;
     const int e = (int)(c % QK_K), half = e >> 7, rem = e & 127, quarter = rem >> 5, ll = rem & 31;
     const int qlb = row[b * 128 + half * 64 + (quarter & 1) * 32 + ll];
@@ -184,10 +195,11 @@ __global__ __launch_bounds__(256) void dequant_q6_k_kernel(const uint8_t *__rest
 
 // dequant_q8_0 (crates/frink-quant/src/lib.rs:271-286)
 __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
-                                                           Layout l, float *__restrict__ out) {
+                                                           Layout l, const int32_t *__restrict__ ids, size_t table_rows,
+                                                           float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * cols) return;
-    const size_t r = i / cols, c = i % cols, b = c / Q8_0_ELEMS;
+    const size_t r = source_row(i / cols, ids, table_rows), c = i % cols, b = c / Q8_0_ELEMS;
     const uint8_t *row = w + r * l.row_stride;
     const uint8_t *dp = row + l.off_a + b * 2;
     const float scale = f16_bits_to_f32((uint16_t)(dp[0] | (dp[1] << 8)));
@@ -197,10 +209,11 @@ __global__ __launch_bounds__(256) void dequant_q8_0_kernel(const uint8_t *__rest
 // dequant_q4_0 (crates/frink-quant/src/lib.rs:291-310): byte i of a block holds element i in its low
 // nibble and element i + 16 in its high one
 __global__ __launch_bounds__(256) void dequant_q4_0_kernel(const uint8_t *__restrict__ w, size_t rows, size_t cols,
-                                                           Layout l, float *__restrict__ out) {
+                                                           Layout l, const int32_t *__restrict__ ids, size_t table_rows,
+                                                           float *__restrict__ out) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= rows * cols) return;
-    const size_t r = i / cols, c = i % cols, b = c / Q8_0_ELEMS;
+    const size_t r = source_row(i / cols, ids, table_rows), c = i % cols, b = c / Q8_0_ELEMS;
     const int e = (int)(c % Q8_0_ELEMS);
     const uint8_t *row = w + r * l.row_stride;
     const uint8_t *dp = row + l.off_a + b * 2;
@@ -275,25 +288,27 @@ int launch_repack(int kind, const uint8_t *src, uint8_t *dst, size_t rows, size_
     return FRK_OK;
 }
 
-int launch_dequant(const frk_weights *w, float *out, hipStream_t s) {
-    const unsigned g = blocks_for(w->rows * w->cols, 256);
+// out[n_out][cols]: every row of the matrix (ids == nullptr, n_out == rows) or the rows ids[0..n_out)
+int launch_dequant_rows(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s) {
+    if (n_out == 0) return FRK_OK;
+    const unsigned g = blocks_for(n_out * w->cols, 256);
     switch (w->kind) {
     case FRK_KIND_Q4_K:
-        hipLaunchKernelGGL(dequant_q4_k_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols,
-                           w->layout.row_stride, out);
+        hipLaunchKernelGGL(dequant_q4_k_kernel, dim3(g), dim3(256), 0, s, w->dev, n_out, w->cols, w->layout.row_stride, ids,
+                           w->rows, out);
         break;
     case FRK_KIND_Q5_K:
-        hipLaunchKernelGGL(dequant_q5_k_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols,
-                           w->layout.row_stride, out);
+        hipLaunchKernelGGL(dequant_q5_k_kernel, dim3(g), dim3(256), 0, s, w->dev, n_out, w->cols, w->layout.row_stride, ids,
+                           w->rows, out);
         break;
     case FRK_KIND_Q6_K:
-        hipLaunchKernelGGL(dequant_q6_k_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols, w->layout, out);
+        hipLaunchKernelGGL(dequant_q6_k_kernel, dim3(g), dim3(256), 0, s, w->dev, n_out, w->cols, w->layout, ids, w->rows, out);
         break;
     case FRK_KIND_Q8_0:
-        hipLaunchKernelGGL(dequant_q8_0_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols, w->layout, out);
+        hipLaunchKernelGGL(dequant_q8_0_kernel, dim3(g), dim3(256), 0, s, w->dev, n_out, w->cols, w->layout, ids, w->rows, out);
         break;
     case FRK_KIND_Q4_0:
-        hipLaunchKernelGGL(dequant_q4_0_kernel, dim3(g), dim3(256), 0, s, w->dev, w->rows, w->cols, w->layout, out);
+        hipLaunchKernelGGL(dequant_q4_0_kernel, dim3(g), dim3(256), 0, s, w->dev, n_out, w->cols, w->layout, ids, w->rows, out);
         break;
     default:
         return set_error(FRK_ERR_UNSUPPORTED, "no dequantizer for quant kind %d", w->kind);
@@ -301,6 +316,8 @@ int launch_dequant(const frk_weights *w, float *out, hipStream_t s) {
     FRK_LAUNCH_CHECK("dequant");
     return FRK_OK;
 }
+
+int launch_dequant(const frk_weights *w, float *out, hipStream_t s) { return launch_dequant_rows(w, nullptr, w->rows, out, s); }
 
 int launch_copy(const void *src, void *dst, size_t bytes, hipStream_t s) {
     const size_t n = bytes / 16;

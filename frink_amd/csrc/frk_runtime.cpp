@@ -307,6 +307,12 @@ int frk_hip_dequant_dev(const frk_weights *w, float *out, void *stream) {
     return launch_dequant(w, out, (hipStream_t)stream);
 }
 
+int frk_hip_get_rows_dev(const frk_weights *w, const int32_t *ids, size_t n_ids, float *out, void *stream) {
+    clear_error();
+    if (!w || (n_ids && (!ids || !out))) return set_error(FRK_ERR_ARG, "frk_hip_get_rows_dev: null argument");
+    return launch_dequant_rows(w, ids, n_ids, out, (hipStream_t)stream);
+}
+
 int frk_hip_copy_dev(const void *src, void *dst, size_t bytes, void *stream) {
     clear_error();
     if (!src || !dst) return set_error(FRK_ERR_ARG, "frk_hip_copy_dev: null argument");
@@ -656,6 +662,31 @@ static int host_launch(int kind, const uint8_t *weights, size_t weights_len, con
     memcpy(keep, g_err, sizeof keep);
     frk_hip_weights_release(w);
     memcpy(g_err, keep, sizeof keep);
+    return rc;
+}
+
+int frk_hip_get_rows(const frk_weights *w, const int32_t *ids, size_t n_ids, float *out) {
+    clear_error();
+    if (!w || (n_ids && (!ids || !out))) return set_error(FRK_ERR_ARG, "frk_hip_get_rows: null argument");
+    for (size_t i = 0; i < n_ids; i++)
+        if (ids[i] < 0 || (size_t)ids[i] >= w->rows)
+            return set_error(FRK_ERR_SHAPE, "id %zu is %d, the table has %zu rows", i, ids[i], w->rows);
+    if (n_ids == 0) return FRK_OK;
+    std::lock_guard<std::mutex> lk(g_launch_mu);
+    const size_t ib = n_ids * sizeof(int32_t), ob = n_ids * w->cols * sizeof(float);
+    int rc = stage_buffers(ib, ob);
+    hipStream_t s = g_dev.stream;
+    if (!rc) {
+        hipError_t e = hipMemcpyAsync(g_dev.x_dev, ids, ib, hipMemcpyHostToDevice, s);
+        if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(ids): %s", hipGetErrorString(e));
+    }
+    if (!rc) rc = launch_dequant_rows(w, (const int32_t *)g_dev.x_dev, n_ids, (float *)g_dev.y_dev, s);
+    if (!rc) {
+        hipError_t e = hipMemcpyAsync(out, g_dev.y_dev, ob, hipMemcpyDeviceToHost, s);
+        if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemcpyAsync(rows): %s", hipGetErrorString(e));
+    }
+    hipError_t e = hipStreamSynchronize(s);
+    if (!rc && e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipStreamSynchronize: %s", hipGetErrorString(e));
     return rc;
 }
 

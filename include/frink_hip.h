@@ -216,8 +216,17 @@ int frk_hip_quantize_q8_k_dev(const float *x_dev, size_t n, int8_t *q_dev, float
 int frk_hip_quantize_q8_0_dev(const float *x_dev, size_t n, int8_t *q_dev, float *d_dev,
                               void *stream);
 /* dequant_q8_0 / dequant_q4_k / dequant_q6_k (crates/frink-quant/src/lib.rs:271-286, 334-364,
- * 519-552) from the resident (possibly permuted) copy: out[rows*cols] f32. */
+ * 519-552; dequant_q5_k :424-459, dequant_q4_0 :291-310) from the resident (possibly permuted)
+ * copy: out[rows*cols] f32. */
 int frk_hip_dequant_dev(const frk_weights *w, float *out_dev, void *stream);
+/* The embedding gather (get_rows, crates/frink-cuda/src/get_rows.rs:1-60; WeightMatrix::dequant_row):
+ * out[n_ids][cols] f32, row r the dequantized row ids[r] of the table, bit for bit what the
+ * dequantizer gives.  The host form checks every id against the table and returns FRK_ERR_SHAPE for
+ * one outside it, as the reference validates before a launch; the device form cannot, and reads the
+ * nearest row for such an id. */
+int frk_hip_get_rows_dev(const frk_weights *w, const int32_t *ids_dev, size_t n_ids, float *out_dev,
+                         void *stream);
+int frk_hip_get_rows(const frk_weights *w, const int32_t *ids_host, size_t n_ids, float *out_host);
 
 /* Plain device copy of `bytes` (multiple of 16), used to calibrate HBM counters and as the
  * practical bandwidth ceiling a streaming kernel of the same size can reach. */

@@ -94,6 +94,35 @@ def test_dequant_of_the_reference_golden_blocks(fa, vectors):
         w.release()
 
 
+@pytest.mark.parametrize("kind", [fo.Q4_0, fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K])
+def test_get_rows_is_the_dequantized_row_bit_for_bit(fa, kind):
+    """The embedding gather (crates/frink-cuda/src/get_rows.rs): row r of the output is the dequantized
+    row ids[r] of the table -- repeated ids, the first and last rows, an empty list; the host form
+    refuses an id outside the table, the device form reads the nearest row for it."""
+    import torch
+    rows, cols = 300, 768
+    bb, be = fo.BLOCK[kind]
+    rng = np.random.default_rng(kind)
+    data = rng.integers(0, 256, rows * cols // be * bb, dtype=np.uint8).reshape(-1, bb)
+    for off in {fo.Q6_K: (208,), fo.Q4_0: (0,), fo.Q8_0: (0,)}.get(kind, (0, 2)):
+        data[:, off:off + 2] = rng.uniform(-0.05, 0.05, data.shape[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    data = data.ravel()
+    table = fo.dequant(kind, data).reshape(rows, cols)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    ids = np.array([0, 299, 17, 17, 150, 1, 298, 0], np.int32)
+    got = w.get_rows(torch.from_numpy(ids).cuda()).cpu().numpy()
+    assert np.array_equal(bits(got), bits(table[ids]))
+    assert np.array_equal(bits(w.get_rows_host(ids)), bits(table[ids]))
+    assert w.get_rows_host(np.zeros(0, np.int32)).shape == (0, cols)
+    for bad in (300, -1):
+        with pytest.raises(fa.BackendError) as e:
+            w.get_rows_host(np.array([3, bad], np.int32))
+        assert e.value.code == fa.ERR_SHAPE and "300 rows" in str(e.value)
+    near = w.get_rows(torch.tensor([300, -5, 1 << 30], dtype=torch.int32).cuda()).cpu().numpy()
+    assert np.array_equal(bits(near), bits(table[[299, 0, 299]]))
+    w.release()
+
+
 def test_weights_from_device_bytes_match_from_host(fa):
     data = make_weights(fo.Q6_K, 8, 512, seed=5)
     a = fa.Weights.from_host(fo.Q6_K, data, 8, 512)
