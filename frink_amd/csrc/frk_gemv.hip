@@ -179,14 +179,18 @@ __global__ __launch_bounds__(256) void gemv_q6_k_kernel(const uint8_t *__restric
 
 // ------------------------------------------------------------------ Q8_0 x f32
 // dot_q8_0_f32 (crates/frink-quant/src/lib.rs:663-686) over the planar resident layout.
-// Unit = 16 quants (half a block); the f32 activation is staged in LDS.
+// Unit = 16 quants (half a block); the f32 activation is staged in LDS, a unit's 16 floats every 20:
+// a lane owns a unit, so neighbouring lanes' 16-byte reads would otherwise be 64 bytes apart and
+// share banks four ways.
+constexpr int Q8_X_STRIDE = 20;
 template <int LPR>
 __global__ __launch_bounds__(256) void gemv_q8_0_f32_kernel(const uint8_t *__restrict__ W, Layout lay, int rows,
                                                             int nb, const float *__restrict__ x,
                                                             float *__restrict__ y) {
     extern __shared__ uint4 smem[];
     float *sx = reinterpret_cast<float *>(smem);
-    for (int i = threadIdx.x; i < nb * 8; i += 256) smem[i] = reinterpret_cast<const uint4 *>(x)[i];
+    for (int i = threadIdx.x; i < nb * 8; i += 256)
+        *reinterpret_cast<uint4 *>(sx + (i >> 2) * Q8_X_STRIDE + (i & 3) * 4) = reinterpret_cast<const uint4 *>(x)[i];
     __syncthreads();
 
     constexpr int PARTS = 64 / LPR;
@@ -202,7 +206,7 @@ __global__ __launch_bounds__(256) void gemv_q8_0_f32_kernel(const uint8_t *__res
             for (int u = l; u < units; u += LPR) {
                 const uint4 qv = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
                 const float scale = h2f(*reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2));
-                const float4 *xv = reinterpret_cast<const float4 *>(sx + u * 16);
+                const float4 *xv = reinterpret_cast<const float4 *>(sx + u * Q8_X_STRIDE);
                 float s = 0.0f;
 #define FRK_Q8_STEP(c, k)                                                  \
     {                                                                      \
@@ -404,6 +408,29 @@ static unsigned gemv_grid(size_t rows, int lpr) {
         else hipLaunchKernelGGL(KERNEL<16>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__);              \
     } while (0)
 
+// The same for kernels that may ask for more than 64 KB of LDS (long rows of f32 activation): the limit
+// is raised once per instantiation.
+constexpr size_t GEMV_LDS_LIMIT = 160 * 1024;
+#define FRK_DISPATCH_LPR_BIG(lpr, KERNEL, grid, shmem, s, ...)                                          \
+    do {                                                                                                \
+        if ((shmem) > GEMV_LDS_LIMIT)                                                                   \
+            return set_error(FRK_ERR_SHAPE, "activation of this width needs %zu bytes of LDS (limit %zu)", \
+                             (size_t)(shmem), GEMV_LDS_LIMIT);                                          \
+        static bool sized = false;                                                                      \
+        if (!sized) {                                                                                   \
+            FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&KERNEL<64>),                \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMV_LDS_LIMIT)); \
+            FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&KERNEL<32>),                \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMV_LDS_LIMIT)); \
+            FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&KERNEL<16>),                \
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)GEMV_LDS_LIMIT)); \
+            sized = true;                                                                               \
+        }                                                                                               \
+        if (lpr == 64) hipLaunchKernelGGL(KERNEL<64>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__);    \
+        else if (lpr == 32) hipLaunchKernelGGL(KERNEL<32>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__); \
+        else hipLaunchKernelGGL(KERNEL<16>, dim3(grid), dim3(256), shmem, s, __VA_ARGS__);              \
+    } while (0)
+
 int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / QK_K);
     const int lpr = lanes_per_row(nb * 4);
@@ -437,8 +464,8 @@ int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
 int launch_gemv_q8_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / Q8_0_ELEMS);
     const int lpr = lanes_per_row(nb * 2);
-    const size_t shmem = (size_t)nb * 32 * 4;
-    FRK_DISPATCH_LPR(lpr, gemv_q8_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+    const size_t shmem = (size_t)nb * 2 * Q8_X_STRIDE * 4;
+    FRK_DISPATCH_LPR_BIG(lpr, gemv_q8_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
                      nb, x, y);
     FRK_LAUNCH_CHECK("gemv_q8_0_f32");
     return FRK_OK;
@@ -457,9 +484,9 @@ int launch_gemv_q8_0_q8(const frk_weights *w, const int8_t *q, const float *d, f
 int launch_gemv_q4_0_f32(const frk_weights *w, const float *x, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / Q8_0_ELEMS);
     const int lpr = lanes_per_row(nb);
-    const int xs = (size_t)nb * (36 + 1) * 4 <= 64 * 1024 ? 36 : 32;
+    const int xs = (size_t)nb * (36 + 1) * 4 <= GEMV_LDS_LIMIT ? 36 : 32;
     const size_t shmem = (size_t)nb * (xs + 1) * 4;
-    FRK_DISPATCH_LPR(lpr, gemv_q4_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
+    FRK_DISPATCH_LPR_BIG(lpr, gemv_q4_0_f32_kernel, gemv_grid(w->rows, lpr), shmem, s, w->dev, w->layout, (int)w->rows,
                      nb, xs, x, y);
     FRK_LAUNCH_CHECK("gemv_q4_0_f32");
     return FRK_OK;
