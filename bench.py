@@ -260,6 +260,18 @@ def main():
                                                "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
         for w in w8:
             w.release()
+        # the same kernel on Q4_0 weights (nibbles turned into signed bytes while they are staged)
+        d40 = torch.from_numpy(random_blocks(fa.Q4_0, cols, rows, seed=81)).to(dev)
+        w40 = [fa.Weights.from_device(fa.Q4_0, d40, cols, rows) for _ in range(4)]
+
+        def step3d(i):
+            w40[i % 4].gemm(xb6, out=yb6)
+        _, t = time_graph(torch, step3d, 100, 50)
+        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+        extra["Q4_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        for w in w40:
+            w.release()
         # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
         E, K, H, F, T = 128, 8, 2048, 768, 512
         experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)

@@ -37,7 +37,7 @@ typedef _Float16 q8_v4h __attribute__((ext_vector_type(4)));
 typedef float q8_v4f __attribute__((ext_vector_type(4)));
 
 struct Q8GemmArgs {
-    const uint8_t *W;   // resident rows: quants [nb][32], then the f16 scales [nb]
+    const uint8_t *W;   // resident rows: quants [nb][32] (Q4_0: nibbles [nb][16]), then the f16 scales [nb]
     size_t row_stride, off_d;
     const int8_t *aq;   // [M][cols]
     const uint16_t *ad; // [M][nb rounded up to 8] f16 bits, zeros in the padding
@@ -104,10 +104,22 @@ struct Q8Stage {  // one chunk's share of a thread on its way from global memory
     q8_v4i s;             // the eight f16 scales of one weight row or token (the first wavefronts only)
 };
 
-template <int TT, int RT>
+// Four nibbles of Q4_0 (one per byte of t, already XOR-ed with 8) as the signed bytes nibble - 8:
+// n - 8 is the four-bit two's complement value n ^ 8, so bit 3 is copied into bits 4..7 -- 0xF0 per
+// byte that has it, as (m << 5) - (m << 1) of the mask m (no byte's 0xF0 reaches its neighbour).
+__device__ __forceinline__ int q4_0_bytes(uint32_t t) {
+    const uint32_t m = t & 0x08080808u;
+    return (int)(t | ((m << 5) - (m << 1)));
+}
+
+// Q4: the weights are Q4_0 (dot_q4_0_q8, crates/frink-quant/src/lib.rs:772-796) -- 16 bytes of nibbles a
+// block, byte i holding element i low and element i + 16 high -- and become the same signed bytes
+// nibble - 8 on their way from the staging registers to LDS; everything behind that is the Q8_0 kernel.
+template <int TT, int RT, bool Q4>
 __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs g) {
     constexpr int NT = 64 * TT * RT;
-    constexpr int AP = TT * 512 / NT, WP = RT * 512 / NT;  // 16-byte pieces a thread stages per chunk
+    // 16-byte pieces a thread stages per chunk (a piece of Q4_0 nibbles is a whole block)
+    constexpr int AP = TT * 512 / NT, WP = (Q4 ? RT * 256 : RT * 512) / NT;
     // two copies of the tiles' chunk: the chunks of even and of odd number
     constexpr int LDS_A = TT * 32 * Q8_LDS_ROW, LDS_COPY = (TT + RT) * 32 * Q8_LDS_ROW;
     extern __shared__ __align__(16) uint8_t q8_lds[];
@@ -121,6 +133,7 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
 
     // The 16-byte pieces this thread stages: piece j is byte 16*p of row r0 + j*NT/16 of either tile.
     const int r0 = tid >> 4, p = tid & 15;
+    const int rq = tid >> 3, pq = tid & 7;  // Q4_0: piece j is block pq of row rq + j*NT/8
     const uint8_t *a_src = (const uint8_t *)g.aq;
     const uint8_t *w_src = g.W;
     const int stage_dst = r0 * Q8_LDS_ROW + p * 16;
@@ -157,8 +170,14 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
             const int tok = min(tok0 + r0 + i * (NT / 16), g.M - 1);
             in.a[i] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
         } else if (i < AP + WP) {
-            const int row = min(row0 + r0 + (i - AP) * (NT / 16), g.rows - 1);
-            in.w[i - AP] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
+            if (Q4) {
+                const int row = min(row0 + rq + (i - AP) * (NT / 8), g.rows - 1);
+                const size_t nibbles = whole || blk0 + pq < g.nb ? (size_t)(blk0 + pq) * 16 : 0;
+                in.w[i - AP] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + nibbles);
+            } else {
+                const int row = min(row0 + r0 + (i - AP) * (NT / 16), g.rows - 1);
+                in.w[i - AP] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
+            }
         } else if (stages_scales) {
             if (whole || !stages_weight_scales || blk0 + 8 <= g.nb) {
                 // (a token's scales are padded with zeros to whole chunks)
@@ -241,7 +260,23 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
 #pragma unroll
             for (int j = 0; j < AP; j++) *reinterpret_cast<q8_v4i *>(lds_a + to + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.a[j];
 #pragma unroll
-            for (int j = 0; j < WP; j++) *reinterpret_cast<q8_v4i *>(lds_w + to + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.w[j];
+            for (int j = 0; j < WP; j++) {
+                if (Q4) {
+                    const q8_v4i v = out.w[j];
+                    q8_v4i lo, hi;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const uint32_t wv = (uint32_t)v[k];
+                        lo[k] = q4_0_bytes((wv & 0x0f0f0f0fu) ^ 0x08080808u);
+                        hi[k] = q4_0_bytes(((wv >> 4) & 0x0f0f0f0fu) ^ 0x08080808u);
+                    }
+                    uint8_t *dst = lds_w + to + (rq + j * (NT / 8)) * Q8_LDS_ROW + pq * 32;
+                    *reinterpret_cast<q8_v4i *>(dst) = lo;
+                    *reinterpret_cast<q8_v4i *>(dst + 16) = hi;
+                } else {
+                    *reinterpret_cast<q8_v4i *>(lds_w + to + stage_dst + j * (NT / 16) * Q8_LDS_ROW) = out.w[j];
+                }
+            }
             if (stages_scales) *reinterpret_cast<q8_v4i *>(s_dst + to) = out.s;
         }
         lds_barrier();  // one barrier a round (it does not wait for the loads on their way)
@@ -306,23 +341,30 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
     auto lds_bytes = [](int tt, int rt) { return (size_t)2 * (tt + rt) * 32 * Q8_LDS_ROW; };
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(4, 2));
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(2, 2));
-        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", lds_bytes(4, 2), hipGetErrorString(e));
+        const void *big[4] = {reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, false>),
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, true>),
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, false>),
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, true>)};
+        for (int i = 0; i < 4; i++) {
+            hipError_t e = hipFuncSetAttribute(big[i], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(4, 2));
+            if (e != hipSuccess)
+                return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", lds_bytes(4, 2), hipGetErrorString(e));
+        }
         sized = true;
     }
+    const bool q4 = w->kind == FRK_KIND_Q4_0;
     if (M > 64) {
         const dim3 grid((unsigned)((w->rows + 63) / 64), (unsigned)((M + 127) / 128));
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2>), grid, dim3(512), lds_bytes(4, 2), s, g);
+        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, true>), grid, dim3(512), lds_bytes(4, 2), s, g);
+        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, false>), grid, dim3(512), lds_bytes(4, 2), s, g);
     } else if (M > 32) {
         const dim3 grid((unsigned)((w->rows + 63) / 64), 1u);
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2>), grid, dim3(256), lds_bytes(2, 2), s, g);
+        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, true>), grid, dim3(256), lds_bytes(2, 2), s, g);
+        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, false>), grid, dim3(256), lds_bytes(2, 2), s, g);
     } else {
         const dim3 grid((unsigned)((w->rows + 31) / 32), 1u);
-        hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1>), grid, dim3(64), lds_bytes(1, 1), s, g);
+        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, true>), grid, dim3(64), lds_bytes(1, 1), s, g);
+        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, false>), grid, dim3(64), lds_bytes(1, 1), s, g);
     }
     FRK_LAUNCH_CHECK("gemm_q8_0_mfma");
     return FRK_OK;

@@ -192,7 +192,8 @@ const char *frk_hip_matvec_kernel(int kind) {
 }
 int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
 int frk_hip_gemm_supported(int kind) {
-    return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0;
+    return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0 ||
+           kind == FRK_KIND_Q4_0;
 }
 int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
 int frk_hip_block_elems(int kind) { return block_elems(kind); }
@@ -418,7 +419,7 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     }
     // Q8_0: a batch is the integer path, as in the reference (Q8_0 activation blocks and dot_q8_0_q8,
     // crates/frink-core/src/weight_matrix.rs:2701-2829); a single row keeps the f32 dot of its decode path
-    if (w->kind == FRK_KIND_Q8_0 && batch >= 2) {
+    if ((w->kind == FRK_KIND_Q8_0 || w->kind == FRK_KIND_Q4_0) && batch >= 2) {  // (Q4_0: the same kernel, dot_q4_0_q8)
         void *ws = nullptr;
         int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
         if (rc) return rc;

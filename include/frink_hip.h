@@ -177,7 +177,7 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
  * crates/frink-core/src/weight_matrix.rs:2481).  Any batch >= 1.  Q4_K and Q6_K multiply Q8_K
  * activations at every batch size, and so does Q5_K (16 rows per launch of its batched kernel).  Q8_0 follows the reference's host: one row is the f32 dot of its
  * decode path (FRK_ACT_F32), two or more rows are quantized to Q8_0 activation blocks and multiplied
- * as integers (weight_matrix.rs:2701-2829, the arithmetic of FRK_ACT_Q8). */
+ * as integers (weight_matrix.rs:2701-2829, the arithmetic of FRK_ACT_Q8); Q4_0 does the same. */
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
                      void *stream);
 

@@ -38,9 +38,8 @@ int main(int argc, char **argv) {
     }
     CHECK(agree, "matvec_kernel(kind) agrees with has_launch(kind) over all 23 kinds and names the kind");
     CHECK(claimed == 5 && Hip::has_launch(QuantKind::Q8_0) && Hip::has_launch(QuantKind::Q4K) &&
-              Hip::has_launch(QuantKind::Q5K) && Hip::has_launch(QuantKind::Q6K) && Hip::has_launch(QuantKind::Q4_0) &&
-              !Hip::gemm_supported(QuantKind::Q4_0),
-          "the five kinds of this path have kernels (Q4_0 decode kernels only)");
+              Hip::has_launch(QuantKind::Q5K) && Hip::has_launch(QuantKind::Q6K) && Hip::has_launch(QuantKind::Q4_0),
+          "the five kinds of this path have kernels");
 
     // None vs Some(Err)
     std::vector<uint8_t> w(34 * 4, 0);

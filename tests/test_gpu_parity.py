@@ -290,7 +290,7 @@ def test_q4_0_dequant_and_decode(fa, rows, cols):
     """Q4_0 (18-byte blocks: an f16 scale and 16 bytes of nibbles, value (nibble - 8) * d) is kept as a
     plane of nibbles and a plane of scales.  The reference holds no encoder for it, so the blocks are
     arbitrary bytes with finite scales: dequantization bit-exact, the f32 dot (decode on an x86 host)
-    and the integer dot against Q8_0 activation blocks within the tolerance, batches row by row."""
+    and the integer dot against Q8_0 activation blocks within the tolerance."""
     from frink_amd import synth
     print("q4_0", rows, cols, flush=True)
     data = _random_q4_0(rows, cols, rows + cols)
@@ -305,12 +305,31 @@ def test_q4_0_dequant_and_decode(fa, rows, cols):
         got_i = w.gemv(to_dev(x[0]), act_mode=fa.ACT_INT8).cpu().numpy()
         want_i = fo.gemm(fo.Q4_0, data, rows, cols, x[:1], fo.INT_DOT, row0=row0, nrows=n)
         assert_rows_close(got_i[None, row0:row0 + n], want_i, "q4_0 integer dot")
-    yb = w.gemm(to_dev(x)).cpu().numpy()
-    for b in range(3):
-        assert np.array_equal(bits(yb[b]), bits(w.gemv(to_dev(x[b])).cpu().numpy()))
     bb = fo.BLOCK[fo.Q4_0][0]
     host = fa.launch_matvec(fo.Q4_0, data, x[0], rows, cols // 32 * bb)
-    assert np.array_equal(bits(host), bits(yb[0]))
+    assert np.array_equal(bits(host), bits(w.gemv(to_dev(x[0])).cpu().numpy()))
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols,batch", [(72, 512, 5), (100, 96, 33), (33, 288, 70), (64, 4096, 129),
+                                             (1000, 1056, 300), (4096, 4096, 512)])
+def test_gemm_q4_0_on_the_matrix_cores(fa, rows, cols, batch):
+    """A Q4_0 batch is the Q8_0 GEMM kernel with the nibbles turned into signed bytes on their way to
+    LDS (dot_q4_0_q8: Q8_0 activation blocks, exact integer sums): the three workgroup shapes, ragged
+    tiles and rows that are not whole 256-column steps, arbitrary block bytes, against the oracle."""
+    from frink_amd import synth
+    print("gemm q4_0", rows, cols, batch, flush=True)
+    data = _random_q4_0(rows, cols, rows + batch)
+    x = synth.activations(rows * 11 + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.Q4_0, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert got.shape == (batch, rows)
+    n = min(64, rows)
+    for row0 in sorted({0, (rows // 2) // 32 * 32 + 5 if rows > 128 else 0, rows - n}):
+        want = fo.gemm(fo.Q4_0, data, rows, cols, x, fo.INT_DOT, row0=row0, nrows=n)
+        assert_rows_close(got[:, row0:row0 + n], want, "gemm q4_0 %dx%d batch %d rows %d.." % (rows, cols, batch, row0))
+    half = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
+    assert np.array_equal(bits(half), bits(got * np.float32(0.5)))
     w.release()
 
 
