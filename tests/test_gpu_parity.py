@@ -652,13 +652,13 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
 @pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q8_0])
 def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
     """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
-    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 17 rows (Q4_K) or 112 (Q6_K); Q8_0:
+    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 33 or 49 rows (Q4_K, by the matrix's size) or 112 (Q6_K); Q8_0:
     the MFMA GEMM from two rows, its token tile growing at 33 and 65): every size on either side of a threshold, on a ragged matrix, against the oracle."""
     from frink_amd import synth
     rows, cols = 72, 512
     data = make_weights(kind, rows, cols, seed=900 + kind)
     w = fa.Weights.from_host(kind, data, rows, cols)
-    for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 64, 65, 111, 112, 113, 129):
+    for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65, 111, 112, 113, 129):
         print("gemm boundary", kind, batch, flush=True)
         x = synth.activations(901 + batch, batch, cols, outlier_frac=0.01)
         got = w.gemm(to_dev(x)).cpu().numpy()
