@@ -44,7 +44,8 @@ struct Q6GemmArgs {
     Q8KTiled a;
     float *y;
     int row_tiles, tok_tiles;
-    int k_split;  // 1, or 2: blockIdx.y takes half of the blocks and the results are added into a zeroed y
+    int k_split;     // 1, or 2/4/8: blockIdx.y takes that share of the blocks and writes its sums to `partial`
+    float *partial;  // [k_split][M][rows], added up in order by q6_reduce_kernel
 };
 
 struct Q6Lds {
@@ -231,9 +232,8 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
     const int tok0 = (in_grp >> 3) * (32 * L::MT);
     const int row0 = row_tile * (32 * RGS) + rgrp * 32;  // this wavefront's first weight row
     const int nb = g.nb;  // blocks of a row (strides); this workgroup multiplies blocks kb_begin .. kb_end - 1
-    const int per_part = (nb + g.k_split - 1) / g.k_split;
-    const int kb_begin = blockIdx.y * per_part, kb_end = min(nb, kb_begin + per_part);
-    if (kb_begin >= kb_end) return;  // uniform per workgroup
+    const int kb_begin = nb * (int)blockIdx.y / g.k_split, kb_end = nb * ((int)blockIdx.y + 1) / g.k_split;
+    // (never empty: the launcher splits no finer than four blocks a part)
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
     auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
         int l = lane;
@@ -387,23 +387,24 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 
     // store: a lane holds one weight row and 16 tokens per tile
     const int row = row0 + li;
+    float *const dst = g.k_split > 1 ? g.partial + (size_t)blockIdx.y * g.M * g.rows : g.y;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tile_first + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) {
-                float *out = g.y + (size_t)tok * g.rows + row;
-                // two parts: both add into the zeroed output (two addends: the order does not matter)
-                if (g.k_split > 1) unsafeAtomicAdd(out, accF[mt][r]);
-                else *out = accF[mt][r];
-            }
+            if (row < g.rows && tok < g.M) dst[(size_t)tok * g.rows + row] = accF[mt][r];
         }
 }
 
-__global__ __launch_bounds__(256) void q6_zero_kernel(float4 *p, size_t n4) {
+// y = the parts' sums added in the order of the parts: the same bits on every run
+__global__ __launch_bounds__(256) void q6_reduce_kernel(const float *__restrict__ partial, int parts, size_t n,
+                                                        float *__restrict__ y) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n4) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i >= n) return;
+    float acc = partial[i];
+    for (int p = 1; p < parts; p++) acc += partial[(size_t)p * n + i];
+    y[i] = acc;
 }
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -414,7 +415,11 @@ __global__ __launch_bounds__(256) void q6_zero_kernel(float4 *p, size_t n4) {
 
 // fewer 256-row workgroups than this leave too many CUs idle: split the blocks, or take 128-row ones
 constexpr size_t Q6_NARROW_BELOW = 200;
-size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
+constexpr int Q6_MAX_SPLIT = 8;
+// the tiled activations, then room for the parts' sums
+size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
+    return round_up(q8k_tiled_bytes(M, cols), 256) + (size_t)Q6_MAX_SPLIT * M * rows * sizeof(float);
+}
 
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     // the kernel addresses the weights and the tiled activations with 32-bit byte offsets
@@ -436,13 +441,17 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.y = y;
     g.tok_tiles = (int)((M + 63) / 64);
     // 256 weight rows per workgroup (a block is unpacked once for two tiles) when that gives about
-    // every CU one; for a short and wide matrix the same with the blocks split between two workgroups
-    // that add into a zeroed output; 128 rows for what is left
+    // every CU one.  For a short and wide matrix, or a batch of few token tiles, the blocks are split
+    // between 2, 4 or 8 workgroups (no finer than four blocks each) whose sums a second kernel adds
+    // up in order; 128 rows where even that leaves most CUs idle.
     const size_t wgs256 = ((w->rows + 255) / 256) * (size_t)g.tok_tiles;
-    const bool split = wgs256 < Q6_NARROW_BELOW && 2 * wgs256 >= 128 && g.nb >= 8 && (M * w->rows) % 4 == 0;
+    int ks = 1;
+    while (ks < Q6_MAX_SPLIT && wgs256 < Q6_NARROW_BELOW && wgs256 * ks * 2 <= 256 && g.nb / (ks * 2) >= 4) ks *= 2;
+    const bool split = ks > 1;
     const bool narrow = wgs256 < Q6_NARROW_BELOW && !split;
     const int rows_wg = narrow ? 128 : 256;
-    g.k_split = split ? 2 : 1;
+    g.k_split = ks;
+    g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
     g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
     const dim3 grid((unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles), (unsigned)g.k_split);
     static bool sized = false;  // a benign race: every thread sets the same attribute
@@ -455,13 +464,14 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", Q6Lds::BYTES, hipGetErrorString(e));
         sized = true;
     }
-    if (split) {
-        const size_t n4 = M * w->rows / 4;
-        hipLaunchKernelGGL(q6_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, reinterpret_cast<float4 *>(y), n4);
-    }
     if (narrow) hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<2>, grid, dim3(512), Q6Lds::BYTES, s, g);
     else hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, grid, dim3(512), Q6Lds::BYTES, s, g);
     FRK_LAUNCH_CHECK("gemm_q6_k_mfma");
+    if (split) {
+        const size_t n = M * w->rows;
+        hipLaunchKernelGGL(q6_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g.partial, ks, n, y);
+        FRK_LAUNCH_CHECK("gemm_q6_k reduce");
+    }
     return FRK_OK;
 }
 

@@ -161,7 +161,7 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // the same for Q6_K (frk_gemm_q6.hip)
-size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols);
+size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // and for Q8_0 (frk_gemm_q8.hip), over activations quantized 32 at a time
 size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols);

@@ -413,11 +413,13 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
-    // Q6_K: from about a hundred rows on the matrix-core GEMM (whose time hardly depends on the batch
-    // up to 512 rows: 230 us at 4096x14336) is ahead of the thin kernel's 8-row groups (15 us each)
-    if (w->kind == FRK_KIND_Q6_K && batch >= 112) {
+    // Q6_K: the matrix-core GEMM (with its blocks split between workgroups for small batches: 53 us at
+    // 4096x14336 and 31 us at 4096x4096 up to 64 rows) is ahead of the thin kernel's 8-row groups (15 us
+    // and 6 us each) from four groups on for large matrices and from six on for small ones
+    const size_t q6k_gemm_from = w->rows * w->cols > (size_t)2 * 4096 * 4096 ? 25 : 41;
+    if (w->kind == FRK_KIND_Q6_K && batch >= q6k_gemm_from) {
         void *ws = nullptr;
-        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q6_k(w, x, batch, y, ws, (hipStream_t)stream);
     }

@@ -652,13 +652,13 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
 @pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q8_0])
 def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
     """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
-    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 33 or 49 rows (Q4_K, by the matrix's size) or 112 (Q6_K); Q8_0:
+    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 33 or 49 rows (Q4_K, by the matrix's size) or from 25 or 41 (Q6_K); Q8_0:
     the MFMA GEMM from two rows, its token tile growing at 33 and 65): every size on either side of a threshold, on a ragged matrix, against the oracle."""
     from frink_amd import synth
     rows, cols = 72, 512
     data = make_weights(kind, rows, cols, seed=900 + kind)
     w = fa.Weights.from_host(kind, data, rows, cols)
-    for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65, 111, 112, 113, 129):
+    for batch in (1, 2, 3, 4, 5, 8, 9, 16, 17, 24, 25, 31, 32, 33, 40, 41, 47, 48, 49, 64, 65, 111, 112, 113, 129):
         print("gemm boundary", kind, batch, flush=True)
         x = synth.activations(901 + batch, batch, cols, outlier_frac=0.01)
         got = w.gemm(to_dev(x)).cpu().numpy()
@@ -688,11 +688,13 @@ def test_wide_q6_k_batch_is_one_launch_of_row_groups(fa, rows, cols, batch):
 
 
 @pytest.mark.parametrize("rows,cols,batch", [(300, 768, 130), (64, 256, 112), (13000, 512, 500), (257, 1024, 200),
-                                             (4096, 14336, 512)])
+                                             (4096, 14336, 512), (4096, 14336, 41), (4096, 14336, 128),
+                                             (4096, 4096, 64), (500, 8192, 256), (96, 2048, 45)])
 def test_gemm_q6_k_on_the_matrix_cores(fa, rows, cols, batch):
-    """Q6_K batches of 112 rows and more take the int8 MFMA kernel (four pre-scaled planes per
-    16-weight group): both workgroup shapes (256 weight rows at 13000x512, 128 elsewhere), ragged last
-    row and token tiles, every activation row against the oracle on the first, a middle and the last
+    """Q6_K batches from 25 rows on (41 for small matrices) take the int8 MFMA kernel (four pre-scaled
+    planes per 16-weight group): both workgroup shapes (256 weight rows at 13000x512, 128 elsewhere),
+    the blocks split between 2, 4 and 8 workgroups whose sums are added in order, ragged last row and
+    token tiles, every activation row against the oracle on the first, a middle and the last
     weight rows, and exact homogeneity."""
     from frink_amd import synth
     print("gemm q6_k", rows, cols, batch, flush=True)
