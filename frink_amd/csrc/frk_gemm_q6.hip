@@ -45,7 +45,7 @@ struct Q6GemmArgs {
     float *y;
     int row_tiles, tok_tiles;
     int k_split;     // 1, or 2/4/8: blockIdx.y takes that share of the blocks and writes its sums to `partial`
-    float *partial;  // [k_split][M][rows], added up in order by q6_reduce_kernel
+    float *partial;  // [k_split][M][rows], added up in order by sum_parts_kernel
 };
 
 struct Q6Lds {
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 }
 
 // y = the parts' sums added in the order of the parts: the same bits on every run
-__global__ __launch_bounds__(256) void q6_reduce_kernel(const float *__restrict__ partial, int parts, size_t n,
+__global__ __launch_bounds__(256) void sum_parts_kernel(const float *__restrict__ partial, int parts, size_t n,
                                                         float *__restrict__ y) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
@@ -412,6 +412,12 @@ __global__ __launch_bounds__(256) void q6_reduce_kernel(const float *__restrict_
         hipError_t e_ = hipGetLastError();                                                              \
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
+
+int launch_sum_parts(const float *partial, int parts, size_t n, float *y, hipStream_t s) {
+    hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, partial, parts, n, y);
+    FRK_LAUNCH_CHECK("sum of the split GEMM's parts");
+    return FRK_OK;
+}
 
 // fewer 256-row workgroups than this leave too many CUs idle: split the blocks, or take 128-row ones
 constexpr size_t Q6_NARROW_BELOW = 200;
@@ -467,11 +473,7 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     if (narrow) hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<2>, grid, dim3(512), Q6Lds::BYTES, s, g);
     else hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, grid, dim3(512), Q6Lds::BYTES, s, g);
     FRK_LAUNCH_CHECK("gemm_q6_k_mfma");
-    if (split) {
-        const size_t n = M * w->rows;
-        hipLaunchKernelGGL(q6_reduce_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g.partial, ks, n, y);
-        FRK_LAUNCH_CHECK("gemm_q6_k reduce");
-    }
+    if (split) return launch_sum_parts(g.partial, ks, M * w->rows, y, s);
     return FRK_OK;
 }
 

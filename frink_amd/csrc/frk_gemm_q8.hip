@@ -43,6 +43,8 @@ struct Q8GemmArgs {
     const uint16_t *ad; // [M][nb rounded up to 8] f16 bits, zeros in the padding
     float *y;           // [M][rows]
     int rows, nb, M;
+    int k_split;     // 1, or 2/4/8: blockIdx.z takes that share of the 256-column chunks (whole pairs of them)
+    float *partial;  // [k_split][M][rows], added up in order afterwards
 };
 
 constexpr int Q8_CHUNK_BLOCKS = 8;   // 256 columns a step
@@ -130,6 +132,10 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     const int tok0 = blockIdx.y * (32 * TT), row0 = blockIdx.x * (32 * RT);
     const size_t cols = (size_t)g.nb * 32;
     const int n_chunks = (g.nb + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS;
+    // this workgroup's chunks c0 .. c1 - 1; c0 is even, so that the chunks of even number are the same
+    // everywhere
+    const int pairs = (n_chunks + 1) / 2;
+    const int c0 = 2 * (pairs * (int)blockIdx.z / g.k_split), c1 = min(n_chunks, 2 * (pairs * ((int)blockIdx.z + 1) / g.k_split));
 
     // The 16-byte pieces this thread stages: piece j is byte 16*p of row r0 + j*NT/16 of either tile.
     const int r0 = tid >> 4, p = tid & 15;
@@ -200,11 +206,11 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     // wavefronts' loads fill the CU's queue and hold up the wavefronts behind them.
     auto round = [&](auto steady_tag, int c, Q8Stage<AP, WP> &out, Q8Stage<AP, WP> &in) {
         constexpr bool STEADY = decltype(steady_tag)::value;
-        if (!STEADY && c + 2 < n_chunks) {
+        if (!STEADY && c + 2 < c1) {
 #pragma unroll
             for (int i = 0; i < LOADS; i++) fetch(i, c + 2, false, in);
         }
-        if (STEADY || (c >= 0 && c < n_chunks)) {
+        if (STEADY || (c >= c0 && c < c1)) {
             // A three-stage pipeline over the blocks: the LDS reads of block b + 2, the matrix products
             // of block b + 1 and the float step of block b are issued in that order, so that reads
             // and products run in the shadow of the 32 vector instructions.
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
                 qa1 = qa2, qw1 = qw2;
             }
         }
-        if (STEADY || (c + 1 >= 0 && c + 1 < n_chunks)) {
+        if (STEADY || (c + 1 >= c0 && c + 1 < c1)) {
             // chunk c + 1 goes into the copy that chunk c - 1 was read from: every wavefront finished
             // with that before the barrier that ended the last round
             const int to = ((c + 1) & 1) * LDS_COPY;
@@ -284,25 +290,26 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     Q8Stage<AP, WP> even, odd;  // the chunks of either parity on their way
     const std::false_type any;
     const std::true_type steady;
-    round(any, -2, odd, even);
-    round(any, -1, even, odd);
-    int c = 0;
-    for (; c + 3 < n_full; c += 2) {  // the chunks these rounds ask for, c + 2 and c + 3, are whole
+    round(any, c0 - 2, odd, even);
+    round(any, c0 - 1, even, odd);
+    int c = c0;
+    for (; c + 3 < min(n_full, c1); c += 2) {  // the chunks these rounds ask for, c + 2 and c + 3, are whole and ours
         round(steady, c, odd, even);
         round(steady, c + 1, even, odd);
     }
-    for (; c < n_chunks; c += 2) {
+    for (; c < c1; c += 2) {
         round(any, c, odd, even);
         round(any, c + 1, even, odd);
     }
 
     // D register r of lane l is token 8*(r/4) + 4*(l/32) + r%4, weight row l%32 of the tile
     const int row = row0 + rt * 32 + (lane & 31);
+    float *const dst = g.k_split > 1 ? g.partial + (size_t)blockIdx.z * g.M * g.rows : g.y;
     if (row < g.rows) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + tt * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (tok < g.M) g.y[(size_t)tok * g.rows + row] = acc[r];
+            if (tok < g.M) dst[(size_t)tok * g.rows + row] = acc[r];
         }
     }
 }
@@ -313,8 +320,10 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
-size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols) {
-    return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256);
+constexpr int Q8_MAX_SPLIT = 8;
+// the quantized activations, their scales, and room for the parts' sums
+size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows) {
+    return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256) + (size_t)Q8_MAX_SPLIT * M * rows * sizeof(float);
 }
 
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
@@ -353,20 +362,31 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
         sized = true;
     }
     const bool q4 = w->kind == FRK_KIND_Q4_0;
+    // A small grid (few token tiles, a short matrix) splits the chunks of a row between 2, 4 or 8
+    // workgroups, no finer than two pairs of chunks each; their sums are added in order afterwards.
+    const size_t wgs = M > 32 ? ((w->rows + 63) / 64) * ((M + 127) / 128) : (w->rows + 31) / 32;
+    const int pairs = ((g.nb + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS + 1) / 2;
+    int ks = 1;
+    const size_t fill = M > 32 ? 256 : 1024;  // (the one-wavefront workgroups of the thinnest batches: four per CU)
+    while (ks < Q8_MAX_SPLIT && wgs * ks * 2 <= fill && pairs / (ks * 2) >= 2) ks *= 2;
+    g.k_split = ks;
+    g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));
+    const unsigned kz = (unsigned)ks;
     if (M > 64) {
-        const dim3 grid((unsigned)((w->rows + 63) / 64), (unsigned)((M + 127) / 128));
+        const dim3 grid((unsigned)((w->rows + 63) / 64), (unsigned)((M + 127) / 128), kz);
         if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, true>), grid, dim3(512), lds_bytes(4, 2), s, g);
         else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, false>), grid, dim3(512), lds_bytes(4, 2), s, g);
     } else if (M > 32) {
-        const dim3 grid((unsigned)((w->rows + 63) / 64), 1u);
+        const dim3 grid((unsigned)((w->rows + 63) / 64), 1u, kz);
         if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, true>), grid, dim3(256), lds_bytes(2, 2), s, g);
         else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, false>), grid, dim3(256), lds_bytes(2, 2), s, g);
     } else {
-        const dim3 grid((unsigned)((w->rows + 31) / 32), 1u);
+        const dim3 grid((unsigned)((w->rows + 31) / 32), 1u, kz);
         if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, true>), grid, dim3(64), lds_bytes(1, 1), s, g);
         else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, false>), grid, dim3(64), lds_bytes(1, 1), s, g);
     }
     FRK_LAUNCH_CHECK("gemm_q8_0_mfma");
+    if (ks > 1) return launch_sum_parts(g.partial, ks, M * w->rows, y, s);
     return FRK_OK;
 }
 

@@ -164,7 +164,9 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // and for Q8_0 (frk_gemm_q8.hip), over activations quantized 32 at a time
-size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols);
+size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows);
+// y[n] = partial[0][n] + partial[1][n] + ... in that order (the split GEMMs' second step; frk_gemm_q6.hip)
+int launch_sum_parts(const float *partial, int parts, size_t n, float *y, hipStream_t s);
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
 // tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the

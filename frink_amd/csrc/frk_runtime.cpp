@@ -427,7 +427,7 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     // crates/frink-core/src/weight_matrix.rs:2701-2829); a single row keeps the f32 dot of its decode path
     if ((w->kind == FRK_KIND_Q8_0 || w->kind == FRK_KIND_Q4_0) && batch >= 2) {  // (Q4_0: the same kernel, dot_q4_0_q8)
         void *ws = nullptr;
-        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
