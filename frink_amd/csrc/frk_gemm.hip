@@ -65,6 +65,8 @@ struct GemmArgs {
     Q8KTiled a;  // ceil(M / 32) tiles
     float *y;    // [M][rows]
     int row_tiles, tok_tiles;
+    int k_split;     // 1, or 2/4: blockIdx.y takes that share of a row's blocks and writes its sums to `partial`
+    float *partial;  // [k_split][M][rows], added up in order afterwards (launch_sum_parts)
 };
 
 // The grouped form: work items (tile, matrix, row group of 256 rows) streamed by persistent workgroups.
@@ -417,7 +419,8 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     const int tok0 = (in_grp >> 3) * TM;
     const int row0 = row_tile * ROWS + rgrp * 32;  // this wavefront's first weight row
     const int row = row0 + li;
-    const int nb = g.nb;
+    const int nb = g.nb;  // blocks of a row (strides); this workgroup multiplies blocks kb0 .. kb1 - 1
+    const int kb0 = nb * (int)blockIdx.y / g.k_split, kb1 = nb * ((int)blockIdx.y + 1) / g.k_split;
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
 
     // ---- what this lane fetches ----
@@ -500,20 +503,23 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     const int pf_tile = __builtin_amdgcn_readfirstlane(wave >= NW / 2 ? MT / 2 : 0);
 
     // prologue: weights of blocks 0..WD-1, activations of block 0; the last weights may stay in flight
-    issue_weights(0);
-    issue_acts(0);
+    issue_weights(kb0);
+    issue_acts(kb0);
 #pragma unroll
     for (int i = 1; i < WD; i++)
-        if (i < nb) issue_weights(i);
-    if (WS == 4 && nb > 2) wait_vm<C_W>();
+        if (kb0 + i < kb1) issue_weights(kb0 + i);
+    if (WS == 4 && kb1 - kb0 > 2) wait_vm<C_W>();
     else wait_vm<0>();
     lds_barrier();
-    read_raw(R, lds_wv, lds_wv + 16 * lg);
+    {
+        const uint32_t first = lds_wv + (kb0 % WS) * L::W_STAGE;
+        read_raw(R, first, first + 16 * lg);
+    }
     wait_raw<0>(R);
     unpack_block(R, lg, B);
     fold_mins(B);
 
-    for (int kb = 0; kb < nb; kb++) {
+    for (int kb = kb0; kb < kb1; kb++) {
         // The first tile's operands are requested before anything else: they travel from LDS while
         // the prefetch below is issued.  In the same way every later tile's operands are requested
         // before the epilogue of the tile before it.
@@ -530,9 +536,9 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
         // stalled the other has the matrix core.  With one tile per wavefront there is no such choice.
         auto prefetch_part = [&](int j, v16i &) {
             if (j < N_A + 2) {
-                if (kb + 1 < nb) act_part(j, kb + 1);
+                if (kb + 1 < kb1) act_part(j, kb + 1);
             } else if (j < N_DMA) {
-                if (kb + WD < nb) weight_part(j - (N_A + 2), kb + WD);
+                if (kb + WD < kb1) weight_part(j - (N_A + 2), kb + WD);
             }
         };
         if (MT == 1) {
@@ -566,7 +572,7 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
             // epilogues of all tiles to the end of this one, every tile's MFMA result alive until then)
             asm volatile("" : "+v"(accF[mt]));
         }
-        if (kb + 1 < nb) {
+        if (kb + 1 < kb1) {
             // the next block's raw weights landed during iteration kb-1
             read_raw(R, wa, wa + 16 * lg);
             wait_raw<0>(R);
@@ -574,19 +580,20 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
             fold_mins(B);
             // activations of block kb+1 and weights of block kb+2 must have landed; with four weight
             // stages the weights requested above (younger than both) may stay in flight
-            if (WS == 4 && kb + WD < nb) wait_vm<C_W>();
+            if (WS == 4 && kb + WD < kb1) wait_vm<C_W>();
             else wait_vm<0>();
         }
         lds_barrier();
     }
 
     // store: a lane holds one weight row and 16 tokens per tile
+    float *const dst = g.k_split > 1 ? g.partial + (size_t)blockIdx.y * g.M * g.rows : g.y;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tgrp * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) g.y[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < g.M) dst[(size_t)tok * g.rows + row] = accF[mt][r];
         }
 }
 
@@ -897,8 +904,9 @@ static int launch_variant(const GemmArgs &g, unsigned grid, hipStream_t s) {
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS>), dim3(grid), dim3(64 * RG * WT), shmem, s, g);
+    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS>), dim3(grid, (unsigned)g.k_split), dim3(64 * RG * WT), shmem, s, g);
     FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
+    if (g.k_split > 1) return launch_sum_parts(g.partial, g.k_split, (size_t)g.M * g.rows, g.y, s);
     return FRK_OK;
 }
 
@@ -938,7 +946,11 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
                          : launch_quantize_records<4>(x, 0, nb, gather, n_rec, out, s);
 }
 
-size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols) { return q8k_tiled_bytes(M, cols); }
+constexpr int Q4K_MAX_SPLIT = 4;
+// the tiled activations, then room for the parts' sums
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
+    return round_up(q8k_tiled_bytes(M, cols), 256) + (size_t)Q4K_MAX_SPLIT * M * rows * sizeof(float);
+}
 
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     // the kernel addresses the weights and the tiled activations with 32-bit byte offsets
@@ -955,6 +967,8 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.nb = (int)(w->cols / QK_K);
     g.M = (int)M;
     g.y = y;
+    g.k_split = 1;
+    g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
     // shape of a workgroup's tile: 256 rows x 128 or 64 tokens when that still gives (about) every CU a
     // workgroup, else 128 rows x 64 or 32 tokens
     auto grid_for = [&](int rows_wg, int tm) {
@@ -965,8 +979,12 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     const size_t wgs_big = ((w->rows + 255) / 256) * ((M + 63) / 64);
     if (M > 64 && ((w->rows + 255) / 256) * ((M + 127) / 128) >= 200) return launch_variant<8, 1, 4, 2>(g, grid_for(256, 128), s);
     if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2>(g, grid_for(256, 64), s);
-    if (M > 32) return launch_variant<4, 2, 1, 4>(g, grid_for(128, 64), s);
-    return launch_variant<4, 1, 1, 2>(g, grid_for(128, 32), s);
+    // The small tiles of a batch that fills few of the CUs: a row's blocks are split between 2 or 4
+    // workgroups (no finer than four blocks each) whose sums are added in order afterwards.
+    const unsigned grid = M > 32 ? grid_for(128, 64) : grid_for(128, 32);
+    while (g.k_split < Q4K_MAX_SPLIT && (size_t)grid * g.k_split * 2 <= 256 && g.nb / (g.k_split * 2) >= 4) g.k_split *= 2;
+    if (M > 32) return launch_variant<4, 2, 1, 4>(g, grid, s);
+    return launch_variant<4, 1, 1, 2>(g, grid, s);
 }
 
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,

@@ -158,7 +158,7 @@ int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTile
 int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, size_t max_rows, Q8KTiled out,
                                 hipStream_t s);
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
-size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols);
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // the same for Q6_K (frk_gemm_q6.hip)
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);

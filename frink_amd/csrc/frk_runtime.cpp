@@ -403,13 +403,13 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     clear_error();
     if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
     if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
-    // Q4_K: up to two launches of the thin kernel (16 rows each, 15 us at 14336x4096) are ahead of the
-    // matrix-core GEMM, whose time hardly depends on the batch below 128 rows (37 us there); three for a
-    // matrix of at most 4096x4096, where a thin launch is 10 us and the GEMM 35
-    const size_t q4k_thin_rows = w->rows * w->cols <= (size_t)4096 * 4096 ? 48 : 32;
+    // Q4_K: up to two launches of the thin kernel (16 rows each: 15 us at 14336x4096, 10 us at 4096x4096)
+    // are ahead of the matrix-core GEMM (28 us and 18 us there for 33..64 rows, its blocks split between
+    // workgroups)
+    const size_t q4k_thin_rows = 32;
     if (w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16)) {
         void *ws = nullptr;
-        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols), (hipStream_t)stream, &ws);
+        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }

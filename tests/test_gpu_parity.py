@@ -652,7 +652,7 @@ def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
 @pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q8_0])
 def test_gemm_at_every_batch_size_where_the_kernel_changes(fa, kind):
     """frk_hip_gemm_dev picks a kernel by the batch size (one row: the GEMV; 2: dot4; 3..16: thin on
-    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 33 or 49 rows (Q4_K, by the matrix's size) or from 25 or 41 (Q6_K); Q8_0:
+    the matrix cores; wider: 8-row groups, or the MFMA GEMM from 33 rows (Q4_K) or from 25 or 41 (Q6_K, by the matrix's size); Q8_0:
     the MFMA GEMM from two rows, its token tile growing at 33 and 65): every size on either side of a threshold, on a ragged matrix, against the oracle."""
     from frink_amd import synth
     rows, cols = 72, 512
