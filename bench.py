@@ -305,6 +305,26 @@ def main():
         extra["MoE layer 128x top-8, 2048/768, 1 token (decode)"] = {
             "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok_bytes / (t / 800) / 1e9, 1),
             "frac_of_hbm_peak": round(tok_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+        # the same layer with its down experts in Q6_K (a Q4_K_M file keeps some layers' that way), 512 tokens and 1
+        down6 = fa.Weights.from_device(fa.Q6_K, torch.from_numpy(random_blocks(fa.Q6_K, E * H, F, seed=83)).to(dev), E * H, F)
+
+        def step4c(i):
+            fa.moe_ffn(experts[0], experts[1], down6, E, xm, ids, wts, out=ym)
+        _, t = time_graph(torch, step4c, 100, 50)
+        moe6_bytes = E * F * H // 256 * (2 * 144 + 210) + 2 * T * H * 4 + 2 * T * K * 4
+        extra["MoE layer 128x top-8, 2048/768, 512 tokens, down experts Q6_K"] = {
+            "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
+            "algorithmic_GBs": round(moe6_bytes / (t / 100) / 1e9, 1),
+            "frac_of_hbm_peak": round(moe6_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4)}
+
+        def step4d(i):
+            fa.moe_ffn(experts[0], experts[1], down6, E, x1, ids1[i % 16], w1, out=y1)
+        _, t = time_graph(torch, step4d, 800, 400)
+        tok6_bytes = K * F * H // 256 * (2 * 144 + 210)
+        extra["MoE layer 128x top-8, 2048/768, 1 token (decode), down experts Q6_K"] = {
+            "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok6_bytes / (t / 800) / 1e9, 1),
+            "frac_of_hbm_peak": round(tok6_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+        down6.release()
         for w in experts:
             w.release()
         # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call

@@ -46,6 +46,11 @@ struct Q6GemmArgs {
     int row_tiles, tok_tiles;
     int k_split;     // 1, or 2/4/8: blockIdx.y takes that share of the blocks and writes its sums to `partial`
     float *partial;  // [k_split][M][rows], added up in order by sum_parts_kernel
+    // The grouped (per-expert) form: token tile t (64 rows of the activations and of y) belongs to expert
+    // tiles[t].x, whose `rows` weight rows start at row tiles[t].x * rows of W, and has tiles[t].z rows in
+    // use; tiles past *n_tiles do nothing.  Null for one matrix.
+    const int4 *tiles;
+    const int *n_tiles;
 };
 
 struct Q6Lds {
@@ -235,12 +240,21 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
     const int kb_begin = nb * (int)blockIdx.y / g.k_split, kb_end = nb * ((int)blockIdx.y + 1) / g.k_split;
     // (never empty: the launcher splits no finer than four blocks a part)
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
+    uint32_t expert_base = 0;  // byte offset of the expert's first weight row
+    int tok_end = g.M;         // first activation row that is not stored
+    if (g.tiles) {             // (uniform per workgroup)
+        const int t = in_grp >> 3;
+        if (t >= *g.n_tiles) return;
+        const int4 ti = g.tiles[t];
+        expert_base = (uint32_t)ti.x * (uint32_t)g.rows * g.row_stride;
+        tok_end = ti.y + ti.z;
+    }
     auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
         int l = lane;
         asm volatile("" : "+v"(l));
         return l;
     };
-    auto row_offset = [&](int r) { return (uint32_t)min(row0 + r, g.rows - 1) * g.row_stride; };  // rows past the end repeat the last
+    auto row_offset = [&](int r) { return expert_base + (uint32_t)min(row0 + r, g.rows - 1) * g.row_stride; };  // rows past the end repeat the last
 
     // ---- the prefetch ----
     const uint8_t *Qb = reinterpret_cast<const uint8_t *>(g.a.q);
@@ -393,7 +407,7 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tile_first + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) dst[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < tok_end) dst[(size_t)tok * g.rows + row] = accF[mt][r];
         }
 }
 
@@ -456,6 +470,8 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     const bool split = ks > 1;
     const bool narrow = wgs256 < Q6_NARROW_BELOW && !split;
     const int rows_wg = narrow ? 128 : 256;
+    g.tiles = nullptr;
+    g.n_tiles = nullptr;
     g.k_split = ks;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
     g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
@@ -474,6 +490,45 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     else hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, grid, dim3(512), Q6Lds::BYTES, s, g);
     FRK_LAUNCH_CHECK("gemm_q6_k_mfma");
     if (split) return launch_sum_parts(g.partial, ks, M * w->rows, y, s);
+    return FRK_OK;
+}
+
+// The grouped form for the MoE down projection: `a` holds max_tiles tiles of 64 activation rows in the
+// grouped order, y is [64 * max_tiles][rows_e]; w stacks the experts' rows_e x cols matrices.
+int launch_gemm_q6_k_grouped(const frk_weights *w, size_t rows_e, Q8KTiled a, const int4 *tiles, const int *n_tiles,
+                             int max_tiles, float *y, hipStream_t s) {
+    if ((uint64_t)w->rows * w->layout.row_stride >= (1ull << 32) ||
+        (uint64_t)q8k_tiled_bytes((size_t)max_tiles * 64, w->cols) >= (1ull << 32))
+        return set_error(FRK_ERR_SHAPE, "grouped gemm_q6_k: %zu x %zu weights with %d tiles exceed 4 GiB per operand", w->rows,
+                         w->cols, max_tiles);
+    if (max_tiles <= 0) return FRK_OK;
+    Q6GemmArgs g;
+    g.a = a;
+    g.W = w->dev;
+    g.row_stride = (uint32_t)w->layout.row_stride;
+    g.off_qh = (uint32_t)w->layout.off_a;
+    g.off_sc = (uint32_t)w->layout.off_b;
+    g.off_d = (uint32_t)w->layout.off_c;
+    g.rows = (int)rows_e;
+    g.nb = (int)(w->cols / QK_K);
+    g.M = max_tiles * 64;
+    g.y = y;
+    g.tok_tiles = max_tiles;
+    g.row_tiles = (int)((rows_e + 255) / 256);
+    g.k_split = 1;
+    g.partial = nullptr;
+    g.tiles = tiles;
+    g.n_tiles = n_tiles;
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6_k_mfma_kernel<1>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)Q6Lds::BYTES);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", Q6Lds::BYTES, hipGetErrorString(e));
+        sized = true;
+    }
+    const dim3 grid((unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles), 1u);
+    hipLaunchKernelGGL(gemm_q6_k_mfma_kernel<1>, grid, dim3(512), Q6Lds::BYTES, s, g);
+    FRK_LAUNCH_CHECK("gemm_q6_k_mfma (grouped)");
     return FRK_OK;
 }
 

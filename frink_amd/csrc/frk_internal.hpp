@@ -163,6 +163,10 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
 // the same for Q6_K (frk_gemm_q6.hip)
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+// its grouped (per-expert) form: tile t = rows [64*t, 64*t+64) of the activations and of y, tiles[t] =
+// {expert, 64*t, rows in use, 0}, tiles past *n_tiles idle; expert e owns rows [e*rows_e, (e+1)*rows_e) of w
+int launch_gemm_q6_k_grouped(const frk_weights *w, size_t rows_e, Q8KTiled a, const int4 *tiles, const int *n_tiles,
+                             int max_tiles, float *y, hipStream_t s);
 // and for Q8_0 (frk_gemm_q8.hip), over activations quantized 32 at a time
 size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows);
 // y[n] = partial[0][n] + partial[1][n] + ... in that order (the split GEMMs' second step; frk_gemm_q6.hip)
@@ -178,7 +182,7 @@ constexpr int MOE_TILE = 64;
 // on the 128-expert, top-8, 2048/768 layer: 8 tokens 47 us against 94 us on the grouped path, 16
 // tokens 79 against 123, 32 tokens 146 against 140.
 constexpr size_t MOE_PER_TOKEN_MAX_BATCH = 16;
-bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn);
+bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind);
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
                             const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,
                             hipStream_t s);

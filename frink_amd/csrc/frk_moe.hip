@@ -389,8 +389,10 @@ int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hid
 // slot) pair reads its expert's three matrices alone, so the layer is three launches of decode
 // kernels -- gate, up and silu(g)*u of all pairs; down of all pairs, each quantizing its own
 // intermediate; the weighted sum in ascending expert id -- instead of the six of the grouped path.
-bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn) {
-    return batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS && ffn <= FUSED_GEMV_MAX_COLS;
+// (Q4_K experts throughout: a Q6_K down projection has the grouped kernel only)
+bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind) {
+    return down_kind == FRK_KIND_Q4_K && batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS &&
+           ffn <= FUSED_GEMV_MAX_COLS;
 }
 static int launch_moe_ffn_per_token(const frk_weights *gate, const frk_weights *up, const frk_weights *down,
                                     int n_experts, const float *x, size_t batch, const int32_t *ids,
@@ -415,7 +417,7 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts);
     const MoeScratch m = moe_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
     const int max_tiles = (int)(rows / MOE_TILE);
-    if (moe_takes_per_token_path(batch, (size_t)hidden, (size_t)ffn))
+    if (moe_takes_per_token_path(batch, (size_t)hidden, (size_t)ffn, down->kind))
         return launch_moe_ffn_per_token(gate, up, down, n_experts, x, batch, ids, weights, k, out, m, s);
 
     static bool sized = false;  // a benign race: every thread sets the same attribute
@@ -436,7 +438,10 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(256), 0, s, m.gate_out,
                        m.up_out, ffn / QK_K, m.gather, m.act);
     FRK_LAUNCH_CHECK("swiglu_quantize");
-    rc = launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
+    // (a Q4_K_M checkpoint keeps some layers' down experts in Q6_K: the matrix-core Q6_K kernel, by tile)
+    rc = down->kind == FRK_KIND_Q6_K
+             ? launch_gemm_q6_k_grouped(down, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, s)
+             : launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights, m.pos_of, k,
                        hidden, out);

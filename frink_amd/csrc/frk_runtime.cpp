@@ -585,8 +585,9 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
         return set_error(FRK_ERR_SHAPE, "empty shape: batch=%zu experts=%zu k=%zu", batch, n_experts, k);
     if (n_experts > 1024 || k > 64 || k > n_experts)
         return set_error(FRK_ERR_SHAPE, "experts=%zu (max 1024), k=%zu (max 64, at most the expert count)", n_experts, k);
-    if (gate->kind != FRK_KIND_Q4_K || up->kind != FRK_KIND_Q4_K || down->kind != FRK_KIND_Q4_K)
-        return set_error(FRK_ERR_UNSUPPORTED, "the grouped expert GEMM takes Q4_K experts (got kinds %d/%d/%d)", gate->kind,
+    if (gate->kind != FRK_KIND_Q4_K || up->kind != FRK_KIND_Q4_K || (down->kind != FRK_KIND_Q4_K && down->kind != FRK_KIND_Q6_K))
+        return set_error(FRK_ERR_UNSUPPORTED,
+                         "the expert GEMMs take Q4_K gate and up and Q4_K or Q6_K down experts (got kinds %d/%d/%d)", gate->kind,
                          up->kind, down->kind);
     if (gate->rows % n_experts || down->rows % n_experts)
         return set_error(FRK_ERR_SHAPE, "stacked rows %zu/%zu do not divide into %zu experts", gate->rows, down->rows,
@@ -609,7 +610,8 @@ int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size
     clear_error();
     if (batch == 0 || k == 0 || n_experts == 0 || hidden == 0 || ffn == 0)
         return set_error(FRK_ERR_SHAPE, "frk_hip_moe_intermediates_dev: empty shape");
-    if (moe_takes_per_token_path(batch, hidden, ffn))
+    // (the hook does not know the experts' kinds: it refuses what Q4_K experts would have run per token)
+    if (moe_takes_per_token_path(batch, hidden, ffn, FRK_KIND_Q4_K))
         return set_error(FRK_ERR_UNSUPPORTED, "a batch of %zu runs per token and keeps no grouped intermediates", batch);
     void *ws = nullptr;
     int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);

@@ -192,7 +192,8 @@ int frk_hip_route_top_k_softmax_dev(const float *logits_dev, size_t batch, size_
  * (frink_moe::run_expert, crates/frink-moe/src/lib.rs:1068-1165): out[batch][hidden] =
  * sum over each token's k routed experts, in ascending expert id, of
  * weights * down_e(silu(gate_e x) * up_e x).  gate/up/down hold the experts stacked row-wise
- * (expert e = rows [e*ffn, (e+1)*ffn) of gate and up, [e*hidden, (e+1)*hidden) of down), Q4_K.
+ * (expert e = rows [e*ffn, (e+1)*ffn) of gate and up, [e*hidden, (e+1)*hidden) of down); gate and up
+ * are Q4_K, down is Q4_K or Q6_K (other kinds: FRK_ERR_UNSUPPORTED).
  * ids[batch][k] / weights[batch][k] are a RoutingDecision per token (lib.rs:112-115); an id outside
  * [0, n_experts) contributes nothing. */
 int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down,

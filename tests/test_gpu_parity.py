@@ -482,7 +482,28 @@ def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False):
     return out
 
 
-def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, ids_override=None):
+def _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w):
+    """moe_ffn_batch with the down experts in another kind than gate and up (a Q4_K_M checkpoint keeps
+    some layers' down experts in Q6_K): the oracle's own GEMMs and SwiGLU per expert bucket, summed per
+    token in ascending expert id like fo_moe_ffn_batch does."""
+    if down_kind == fo.Q4_K:
+        return fo.moe_ffn_batch(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
+    out = np.zeros((x.shape[0], hidden), np.float32)
+    for e in range(n_experts):
+        toks, slots = np.nonzero(ids == e)
+        if toks.size == 0:
+            continue
+        g = fo.gemm(fo.Q4_K, gb[e], ffn, hidden, x[toks])
+        u = fo.gemm(fo.Q4_K, ub[e], ffn, hidden, x[toks])
+        act = fo.swiglu(g.ravel(), u.ravel()).reshape(toks.size, ffn)
+        y = fo.gemm(down_kind, db[e], hidden, ffn, act)
+        for i, (t, sl) in enumerate(zip(toks, slots)):
+            out[t] += w[t, sl] * y[i]
+    return out
+
+
+def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, ids_override=None, down_kind=None):
     """The quantizer between the two GEMMs is a step function, so a last-bit difference in a
     gate/up output can move one intermediate value to the next int8 level and shift a whole output
     row by d_act*|w|: the end-to-end comparison alone cannot hold 1e-3 on every row for any
@@ -495,6 +516,9 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     from frink_amd import synth
     print("moe", n_experts, k, hidden, ffn, batch, flush=True)
     gate, up, down = _stacked_experts(n_experts, hidden, ffn, seed, random_blocks)
+    down_kind = fo.Q4_K if down_kind is None else down_kind
+    if down_kind != fo.Q4_K:
+        down = make_weights(down_kind, n_experts * hidden, ffn, seed=seed + 2, sigma=0.05)
     x = synth.activations(seed + 10, batch, hidden)
     logits = synth.normal(seed + 11, batch * n_experts).reshape(batch, n_experts)
     ids, w = _route(logits, k)
@@ -503,12 +527,19 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     ids = ids.astype(np.int32)
     wg = fa.Weights.from_host(fo.Q4_K, gate, n_experts * ffn, hidden)
     wu = fa.Weights.from_host(fo.Q4_K, up, n_experts * ffn, hidden)
-    wd = fa.Weights.from_host(fo.Q4_K, down, n_experts * hidden, ffn)
+    wd = fa.Weights.from_host(down_kind, down, n_experts * hidden, ffn)
     got = fa.moe_ffn(wg, wu, wd, n_experts, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
-    if batch <= fa.MOE_PER_TOKEN_MAX_BATCH:
+    if batch <= fa.MOE_PER_TOKEN_MAX_BATCH and down_kind == fo.Q4_K:
         for h in (wg, wu, wd):
             h.release()
         return _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, batch, x, ids, w)
+    if batch <= fa.MOE_PER_TOKEN_MAX_BATCH:  # grouped all the same, but the hook keeps no record of so few tokens
+        for h in (wg, wu, wd):
+            h.release()
+        want = _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+        rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
+        assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, rel.max()
+        return got, want
     g_out, u_out, act_q, act_d, pos = (t.cpu().numpy() for t in fa.moe_intermediates(batch, k, n_experts, hidden, ffn))
     for h in (wg, wu, wd):
         h.release()
@@ -527,7 +558,7 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
             continue
         assert_rows_close(g_out[rows], fo.gemm(fo.Q4_K, gb[e], ffn, hidden, x[toks]), "gate of expert %d" % e)
         assert_rows_close(u_out[rows], fo.gemm(fo.Q4_K, ub[e], ffn, hidden, x[toks]), "up of expert %d" % e)
-        want_down[rows] = fo.gemm(fo.Q4_K, db[e], hidden, ffn, act[rows])
+        want_down[rows] = fo.gemm(down_kind, db[e], hidden, ffn, act[rows])
     q, d, _ = fo.quantize_q8_k(act.ravel())
     assert np.array_equal(act_q.ravel(), q) and np.array_equal(bits(act_d.ravel()), bits(d))
     chained = np.zeros((batch, hidden), np.float32)
@@ -535,7 +566,7 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
         chained[t] += w[t, s] * want_down[pos[t, s]]
     assert_rows_close(got, chained, "down+combine E=%d k=%d batch=%d" % (n_experts, k, batch))
 
-    want = fo.moe_ffn_batch(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    want = _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w)
     rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
     print("moe end-to-end: rows over 1e-3: %d of %d, worst %.3g" % ((rel > TOL).sum(), batch, rel.max()), flush=True)
     assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, rel.max()
@@ -591,6 +622,25 @@ def test_moe_ffn_of_a_few_tokens_runs_per_token(fa, n_experts, k, hidden, ffn, b
 ])
 def test_moe_ffn_matches_the_oracle(fa, n_experts, k, hidden, ffn, batch):
     _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 100 + batch)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_experts,k,hidden,ffn,batch", [(8, 2, 256, 512, 40), (4, 2, 768, 256, 3), (16, 4, 512, 768, 130),
+                                                         (32, 4, 256, 256, 200)])
+def test_moe_ffn_with_q6_k_down_experts(fa, n_experts, k, hidden, ffn, batch):
+    """Q4_K gate and up, Q6_K down: the down projection runs on the Q6_K matrix-core kernel by token tile
+    (batch 3: grouped although so few tokens)."""
+    _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 7 + batch, down_kind=fo.Q6_K)
+
+
+def test_moe_ffn_refuses_other_expert_kinds(fa):
+    w4 = fa.Weights.from_host(fo.Q4_K, make_weights(fo.Q4_K, 2 * 256, 256, seed=1), 2 * 256, 256)
+    w8 = fa.Weights.from_host(fo.Q8_0, make_weights(fo.Q8_0, 2 * 256, 256, seed=2), 2 * 256, 256)
+    x, ids, w = to_dev(np.zeros((20, 256), np.float32)), to_dev(np.zeros((20, 1), np.int32)), to_dev(np.ones((20, 1), np.float32))
+    for gate, up, down in ((w4, w4, w8), (w8, w4, w4)):
+        with pytest.raises(fa.BackendError) as e:
+            fa.moe_ffn(gate, up, down, 2, x, ids, w)
+        assert e.value.code == fa.ERR_UNSUPPORTED
 
 
 def test_moe_ffn_with_idle_experts_and_one_hot_routing(fa):
