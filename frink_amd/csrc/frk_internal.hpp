@@ -103,10 +103,30 @@ struct frk_weights {
 
 namespace frk {
 
-// ---- per-device scratch the library owns (quantized activations etc.) ----
-// Returns a buffer of at least `bytes` on the current device, growing it if needed.
-// Grown with the stream idle (hipStreamSynchronize) so no kernel still reads the old one.
-int workspace(size_t bytes, hipStream_t stream, void **out);
+// ---- scratch the library owns (quantized activations, intermediates) ----
+// One buffer per caller stream.  A lease holds the stream's buffer for as long as one entry point is
+// enqueueing its launches (a recursive lock: entry points call each other), so calls made on one stream
+// from several threads go out whole, one after the other, and stream order keeps their use of the buffer
+// apart; calls on different streams have different buffers.  A buffer that is too small is replaced, never
+// freed in place: the old one is kept until the outermost lease ends, then retired behind an event on the
+// stream and handed out again (to any stream) once that event has passed.  A stream that is being captured
+// cannot grow its buffer (the caller runs the shape once before capturing).
+struct StreamWorkspace;
+class WorkspaceLease {
+  public:
+    WorkspaceLease() = default;
+    ~WorkspaceLease();
+    WorkspaceLease(const WorkspaceLease &) = delete;
+    WorkspaceLease &operator=(const WorkspaceLease &) = delete;
+    void *ptr = nullptr;
+
+  private:
+    friend int workspace(size_t, hipStream_t, WorkspaceLease &);
+    StreamWorkspace *held_ = nullptr;
+    hipStream_t stream_ = nullptr;
+};
+// Leases at least `bytes` of the stream's buffer (the same start address for nested leases).
+int workspace(size_t bytes, hipStream_t stream, WorkspaceLease &lease);
 hipStream_t own_stream();  // the stream host-buffer entry points run on
 
 // ---- launchers (each validates nothing: callers have checked shapes) ----
@@ -182,6 +202,9 @@ constexpr int MOE_TILE = 64;
 // on the 128-expert, top-8, 2048/768 layer: 8 tokens 47 us against 94 us on the grouped path, 16
 // tokens 79 against 123, 32 tokens 146 against 140.
 constexpr size_t MOE_PER_TOKEN_MAX_BATCH = 16;
+// From this many tokens on the reference buckets a batch by expert (ffn_batch.rs:355) and a token's experts
+// add up in ascending expert id; smaller batches run per position and add up in routing order.
+constexpr size_t MOE_BUCKET_ORDER_FROM = 32;
 bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind);
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
                             const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,

@@ -2,7 +2,7 @@
 // (crates/frink-models/src/decoder/ffn_batch.rs:343-434):
 //   bucket (token, slot) pairs by expert  ->  gate/up grouped GEMM over gathered token rows
 //   ->  silu(gate)*up, quantized to Q8_K  ->  down grouped GEMM  ->  out[tok] = sum_e w * down
-// with each token's experts added in ascending expert id, as the reference's expert loop does.
+// with each token's experts added in the order the reference adds them (moe_combine_kernel).
 #include "frk_device.hpp"
 
 namespace frk {
@@ -253,23 +253,30 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
 
 int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s);
 
-// out[tok] = sum over the token's slots, ascending expert id, of w * down[pos]: the order of the
-// reference's expert loop (ffn_batch.rs:388-423), each term a separate multiply and add.
+// out[tok] = sum over the token's slots of w * down[pos], each term a separate multiply and add, in the
+// order the reference adds them for a batch of this size: its bucket path (32 tokens and more,
+// ffn_batch.rs:355, 388-423) walks the experts in ascending id; below that every position runs alone and
+// combine_expert_outputs (crates/frink-moe/src/lib.rs:1246-1263) adds the slots in routing order.
+// A slot whose id is outside [0, n_experts) contributes nothing.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ down, const int32_t *__restrict__ ids,
                                                           const float *__restrict__ weights,
                                                           const int *__restrict__ pos_of, int k, int hidden,
-                                                          float *__restrict__ out) {
+                                                          int n_experts, int by_expert_id, float *__restrict__ out) {
     __shared__ int s_pos[64];
     __shared__ float s_w[64];
     __shared__ int s_id[64];
     const int tok = blockIdx.x, tid = threadIdx.x;
     if (tid < k) s_id[tid] = ids[(size_t)tok * k + tid];
     __syncthreads();
-    if (tid < k) {  // place in the ascending order of expert ids, equal ids in slot order
+    if (tid < k) {
         const int mine = s_id[tid];
-        int rank = 0;
-        for (int j = 0; j < k; j++) rank += (s_id[j] < mine) || (s_id[j] == mine && j < tid);
-        s_pos[rank] = pos_of ? pos_of[(size_t)tok * k + tid] : tok * k + tid;  // (no map: rows in pair order)
+        int rank = tid;
+        if (by_expert_id) {  // place in the ascending order of expert ids, equal ids in slot order
+            rank = 0;
+            for (int j = 0; j < k; j++) rank += (s_id[j] < mine) || (s_id[j] == mine && j < tid);
+        }
+        const int pos = pos_of ? pos_of[(size_t)tok * k + tid] : tok * k + tid;  // (no map: rows in pair order)
+        s_pos[rank] = (mine >= 0 && mine < n_experts) ? pos : -1;
         s_w[rank] = weights[(size_t)tok * k + tid];
     }
     __syncthreads();
@@ -388,7 +395,7 @@ int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hid
 // moe_host.rs:102-203, crates/frink-moe/src/lib.rs:1068-1165): with a token or a few, every (token,
 // slot) pair reads its expert's three matrices alone, so the layer is three launches of decode
 // kernels -- gate, up and silu(g)*u of all pairs; down of all pairs, each quantizing its own
-// intermediate; the weighted sum in ascending expert id -- instead of the six of the grouped path.
+// intermediate; the weighted sum in routing order -- instead of the six of the grouped path.
 // (Q4_K experts throughout: a Q6_K down projection has the grouped kernel only)
 bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind) {
     return down_kind == FRK_KIND_Q4_K && batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS &&
@@ -405,7 +412,7 @@ static int launch_moe_ffn_per_token(const frk_weights *gate, const frk_weights *
                                   m.down_out, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights,
-                       (const int *)nullptr, k, hidden, out);
+                       (const int *)nullptr, k, hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);
     FRK_LAUNCH_CHECK("moe_combine");
     return FRK_OK;
 }
@@ -444,7 +451,7 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
              : launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights, m.pos_of, k,
-                       hidden, out);
+                       hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);
     FRK_LAUNCH_CHECK("moe_combine");
     return FRK_OK;
 }

@@ -30,8 +30,6 @@ struct DeviceState {
     bool probed = false;
     int device_count = 0;
     hipStream_t stream = nullptr;  // for host-buffer entry points
-    void *ws = nullptr;
-    size_t ws_bytes = 0;
     // host staging for the host-buffer entry points
     void *x_dev = nullptr, *y_dev = nullptr;
     size_t x_bytes = 0, y_bytes = 0;
@@ -58,22 +56,110 @@ static int ensure_device_locked() {
 
 hipStream_t own_stream() { return g_dev.stream; }
 
-int workspace(size_t bytes, hipStream_t stream, void **out) {
-    std::lock_guard<std::mutex> lk(g_dev.mu);
-    if (bytes > g_dev.ws_bytes) {
-        if (g_dev.ws) {
-            FRK_HIP_TRY(hipDeviceSynchronize());
-            FRK_HIP_TRY(hipFree(g_dev.ws));
-            g_dev.ws = nullptr;
-            g_dev.ws_bytes = 0;
+struct StreamWorkspace {
+    std::recursive_mutex mu;  // held by the thread whose entry point is enqueueing on the stream
+    void *ptr = nullptr;
+    size_t bytes = 0;
+    int depth = 0;                 // nested leases of the holder
+    std::vector<std::pair<void *, size_t>> outgrown;  // replaced under a lease; retired when the outermost ends
+};
+struct RetiredBuffer {
+    void *ptr;
+    size_t bytes;
+    hipEvent_t passed;  // recorded on the stream that used the buffer last
+};
+static std::map<hipStream_t, StreamWorkspace *> g_ws;  // under g_dev.mu; entries live until the process ends
+static std::vector<RetiredBuffer> g_retired;           // under g_dev.mu
+
+// A retired buffer of at least `bytes` whose last use has passed, or a fresh allocation.  Retired
+// buffers that are idle and too small are given back to the driver here, where an allocation is
+// being paid for anyway.
+static int take_buffer_locked(size_t bytes, void **ptr, size_t *got) {
+    size_t best = g_retired.size();
+    for (size_t i = 0; i < g_retired.size(); i++) {
+        if (hipEventQuery(g_retired[i].passed) != hipSuccess) {
+            (void)hipGetLastError();  // not ready is not an error
+            continue;
         }
-        size_t want = std::max<size_t>(round_up(bytes, 1 << 20), 4u << 20);
-        FRK_HIP_TRY(hipMalloc(&g_dev.ws, want));
-        g_dev.ws_bytes = want;
+        if (g_retired[i].bytes >= bytes && (best == g_retired.size() || g_retired[i].bytes < g_retired[best].bytes)) best = i;
     }
-    (void)stream;
-    *out = g_dev.ws;
+    if (best < g_retired.size()) {
+        *ptr = g_retired[best].ptr;
+        *got = g_retired[best].bytes;
+        (void)hipEventDestroy(g_retired[best].passed);
+        g_retired.erase(g_retired.begin() + (long)best);
+        return FRK_OK;
+    }
+    for (size_t i = 0; i < g_retired.size();) {
+        if (hipEventQuery(g_retired[i].passed) == hipSuccess) {
+            (void)hipFree(g_retired[i].ptr);
+            (void)hipEventDestroy(g_retired[i].passed);
+            g_retired.erase(g_retired.begin() + (long)i);
+        } else {
+            (void)hipGetLastError();
+            i++;
+        }
+    }
+    const size_t want = std::max<size_t>(round_up(bytes, 1 << 20), 4u << 20);
+    FRK_HIP_TRY(hipMalloc(ptr, want));
+    *got = want;
     return FRK_OK;
+}
+
+int workspace(size_t bytes, hipStream_t stream, WorkspaceLease &lease) {
+    StreamWorkspace *w = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_dev.mu);
+        auto it = g_ws.find(stream);
+        if (it == g_ws.end()) it = g_ws.emplace(stream, new StreamWorkspace()).first;
+        w = it->second;
+    }
+    w->mu.lock();
+    w->depth++;
+    lease.held_ = w;
+    lease.stream_ = stream;
+    if (bytes > w->bytes) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cs) != hipSuccess) (void)hipGetLastError();
+        if (cs != hipStreamCaptureStatusNone)
+            return set_error(FRK_ERR_HIP,
+                             "the stream's scratch buffer holds %zu bytes and this call needs %zu: it cannot grow while the "
+                             "stream is being captured (run the shape once before capturing)", w->bytes, bytes);
+        void *fresh = nullptr;
+        size_t got = 0;
+        {
+            std::lock_guard<std::mutex> lk(g_dev.mu);
+            int rc = take_buffer_locked(bytes, &fresh, &got);
+            if (rc) return rc;
+        }
+        if (w->ptr) w->outgrown.emplace_back(w->ptr, w->bytes);
+        w->ptr = fresh;
+        w->bytes = got;
+    }
+    lease.ptr = w->ptr;
+    return FRK_OK;
+}
+
+WorkspaceLease::~WorkspaceLease() {
+    StreamWorkspace *w = held_;
+    if (!w) return;
+    if (--w->depth == 0 && !w->outgrown.empty()) {
+        // kernels enqueued under this lease may still read a replaced buffer: it is free once the
+        // stream has passed this point
+        std::lock_guard<std::mutex> lk(g_dev.mu);
+        for (auto &b : w->outgrown) {
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) == hipSuccess && hipEventRecord(ev, stream_) == hipSuccess) {
+                g_retired.push_back({b.first, b.second, ev});
+            } else {
+                (void)hipGetLastError();
+                if (ev) (void)hipEventDestroy(ev);
+                // without an event the buffer cannot be shown idle: it is kept until the process ends
+            }
+        }
+        w->outgrown.clear();
+    }
+    w->mu.unlock();
 }
 
 static void fingerprint_of(const uint8_t *bytes, size_t len, uint8_t out[192]) {
@@ -114,8 +200,9 @@ static int make_resident(int kind, const uint8_t *src_dev, size_t rows, size_t c
     (void)hipGetDevice(&w->device);
     hipError_t e = hipMalloc((void **)&w->dev, w->dev_bytes);
     if (e != hipSuccess) {
+        const size_t wanted = w->dev_bytes;
         delete w;
-        return set_error(FRK_ERR_OOM, "hipMalloc(%zu) for resident weights: %s", w->dev_bytes, hipGetErrorString(e));
+        return set_error(FRK_ERR_OOM, "hipMalloc(%zu) for resident weights: %s", wanted, hipGetErrorString(e));
     }
     int rc = launch_repack(kind, src_dev, w->dev, rows, cols, w->layout, s);
     if (rc == FRK_OK) {
@@ -329,12 +416,14 @@ int frk_hip_read_dev(const void *src, size_t bytes, void *sink, void *stream) {
 }
 
 // Quantizes `batch` activation rows of w->cols values to Q8_K in the workspace.
-static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch, hipStream_t s, Q8KActs *a) {
+// (the lease must outlive the launches that read `a`)
+static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch, hipStream_t s, WorkspaceLease &lease,
+                              Q8KActs *a) {
     size_t n = batch * w->cols;
     size_t q_bytes = round_up(n, 256), d_bytes = round_up(n / QK_K * 4, 256), b_bytes = round_up(n / 16 * 2, 256);
-    void *ws = nullptr;
-    int rc = workspace(q_bytes + d_bytes + b_bytes, s, &ws);
+    int rc = workspace(q_bytes + d_bytes + b_bytes, s, lease);
     if (rc) return rc;
+    void *ws = lease.ptr;
     int8_t *q = (int8_t *)ws;
     float *d = (float *)((char *)ws + q_bytes);
     int16_t *b = (int16_t *)((char *)ws + q_bytes + d_bytes);
@@ -358,7 +447,8 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q6_K: {
         if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
         Q8KActs a;
-        int rc = quantize_acts_q8_k(w, x, 1, s, &a);
+        WorkspaceLease lease;
+        int rc = quantize_acts_q8_k(w, x, 1, s, lease, &a);
         if (rc) return rc;
         if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, s);
         if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, s);
@@ -371,9 +461,10 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
             return direct_gemv_fits(w) ? launch_gemv_q8_0_f32_direct(w, x, y, s) : launch_gemv_q8_0_f32(w, x, y, s);
         }
         size_t n = w->cols;
-        void *ws = nullptr;
-        int rc = workspace(round_up(n, 256) + n / 32 * 4, s, &ws);
+        WorkspaceLease lease;
+        int rc = workspace(round_up(n, 256) + n / 32 * 4, s, lease);
         if (rc) return rc;
+        void *ws = lease.ptr;
         int8_t *q = (int8_t *)ws;
         float *d = (float *)((char *)ws + round_up(n, 256));
         rc = launch_quantize_q8_0(x, n, q, d, s);
@@ -408,35 +499,36 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     // workgroups)
     const size_t q4k_thin_rows = 32;
     if (w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16)) {
-        void *ws = nullptr;
-        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
+        WorkspaceLease lease;
+        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
         if (rc) return rc;
-        return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
+        return launch_gemm_q4_k(w, x, batch, y, lease.ptr, (hipStream_t)stream);
     }
     // Q6_K: the matrix-core GEMM (with its blocks split between workgroups for small batches: 53 us at
     // 4096x14336 and 31 us at 4096x4096 up to 64 rows) is ahead of the thin kernel's 8-row groups (15 us
     // and 6 us each) from four groups on for large matrices and from six on for small ones
     const size_t q6k_gemm_from = w->rows * w->cols > (size_t)2 * 4096 * 4096 ? 25 : 41;
     if (w->kind == FRK_KIND_Q6_K && batch >= q6k_gemm_from) {
-        void *ws = nullptr;
-        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
+        WorkspaceLease lease;
+        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
         if (rc) return rc;
-        return launch_gemm_q6_k(w, x, batch, y, ws, (hipStream_t)stream);
+        return launch_gemm_q6_k(w, x, batch, y, lease.ptr, (hipStream_t)stream);
     }
     // Q8_0: a batch is the integer path, as in the reference (Q8_0 activation blocks and dot_q8_0_q8,
     // crates/frink-core/src/weight_matrix.rs:2701-2829); a single row keeps the f32 dot of its decode path
     if ((w->kind == FRK_KIND_Q8_0 || w->kind == FRK_KIND_Q4_0) && batch >= 2) {  // (Q4_0: the same kernel, dot_q4_0_q8)
-        void *ws = nullptr;
-        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
+        WorkspaceLease lease;
+        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
         if (rc) return rc;
-        return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
+        return launch_gemm_q8_0(w, x, batch, y, lease.ptr, (hipStream_t)stream);
     }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K) && batch >= 2
                          ? thin_gemm_max_batch(w) : 0;
     if (thin >= 2) {
         Q8KActs a;
-        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
+        WorkspaceLease lease;
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, lease, &a);
         if (rc) return rc;
         const size_t nb = w->cols / QK_K;
         if (batch > (size_t)thin && batch <= (size_t)thin_gemm_wide_rows(w))
@@ -453,7 +545,8 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     // decode kernel
     if (w->kind == FRK_KIND_Q5_K) {
         Q8KActs a;
-        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, &a);
+        WorkspaceLease lease;
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, lease, &a);
         if (rc) return rc;
         const size_t nb = w->cols / QK_K;
         for (size_t b = 0; b < batch; b++) {
@@ -515,8 +608,9 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     }
     // otherwise one Q8_K quantization for every K-quant matrix of the group
     Q8KActs a = {nullptr, nullptr, nullptr};
+    WorkspaceLease lease;
     if (any_k) {
-        int rc = quantize_acts_q8_k(ws[0], x, 1, s, &a);
+        int rc = quantize_acts_q8_k(ws[0], x, 1, s, lease, &a);
         if (rc) return rc;
     }
     for (size_t i = 0; i < n; i++) {
@@ -541,9 +635,10 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
     // scratch for gate(x), up(x) and silu(gate)*up behind the quantized activation
     const size_t q_cols = std::max(gate->cols, down->cols);  // either projection may quantize its input here
     const size_t q_area = round_up(q_cols, 256) + round_up(q_cols / 32 * 4, 256) + round_up(q_cols / 8, 256);
-    void *ws = nullptr;
-    int rc = workspace(q_area + 3 * round_up(ffn * 4, 256), s, &ws);
+    WorkspaceLease lease;
+    int rc = workspace(q_area + 3 * round_up(ffn * 4, 256), s, lease);
     if (rc) return rc;
+    void *ws = lease.ptr;
     float *g_out = (float *)((char *)ws + q_area), *u_out = g_out + round_up(ffn * 4, 256) / 4,
           *act = u_out + round_up(ffn * 4, 256) / 4;
     if (gate->kind == FRK_KIND_Q4_K && up->kind == FRK_KIND_Q4_K && fused_gemv_fits(gate) &&
@@ -598,10 +693,10 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
                          "expert shapes disagree: gate %zux%zu up %zux%zu down %zux%zu over %zu experts (hidden %zu, ffn %zu)",
                          gate->rows, gate->cols, up->rows, up->cols, down->rows, down->cols, n_experts, hidden, ffn);
     if (batch * k > (size_t)1 << 30) return set_error(FRK_ERR_SHAPE, "batch*k = %zu pairs is too many", batch * k);
-    void *ws = nullptr;
-    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);
+    WorkspaceLease lease;
+    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, lease);
     if (rc) return rc;
-    return launch_moe_ffn(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, ws, (hipStream_t)stream);
+    return launch_moe_ffn(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, lease.ptr, (hipStream_t)stream);
 }
 
 int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size_t hidden, size_t ffn,
@@ -613,10 +708,10 @@ int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size
     // (the hook does not know the experts' kinds: it refuses what Q4_K experts would have run per token)
     if (moe_takes_per_token_path(batch, hidden, ffn, FRK_KIND_Q4_K))
         return set_error(FRK_ERR_UNSUPPORTED, "a batch of %zu runs per token and keeps no grouped intermediates", batch);
-    void *ws = nullptr;
-    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, &ws);
+    WorkspaceLease lease;
+    int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, lease);
     if (rc) return rc;
-    return moe_copy_intermediates(ws, batch, (int)k, (int)n_experts, (int)hidden, (int)ffn, gate_out, up_out, act_q,
+    return moe_copy_intermediates(lease.ptr, batch, (int)k, (int)n_experts, (int)hidden, (int)ffn, gate_out, up_out, act_q,
                                   act_d, pos_of, (hipStream_t)stream);
 }
 

@@ -149,7 +149,14 @@ int frk_hip_launch_dense_ffn_swiglu(const frk_matvec_launch *gate, const frk_mat
                                     const frk_matvec_launch *down, const float *x, size_t x_len,
                                     float *out);
 
-/* ---- device-pointer entry points (asynchronous on `stream`, a hipStream_t or NULL) ---- */
+/* ---- device-pointer entry points (asynchronous on `stream`, a hipStream_t or NULL) ----
+ * Scratch memory (quantized activations, intermediates) is one library-owned buffer PER STREAM, held by
+ * the calling thread while it enqueues a call's launches: calls on different streams never share
+ * scratch, calls on one stream from several threads go out one after the other (as the reference's
+ * rayon workers call the seam, gpu_backend.rs:722-725).  A buffer that is too small is replaced, not
+ * freed in place, and nothing in these calls waits for the device.  While a stream is being captured
+ * into a graph its buffer cannot grow: run each shape once before capturing it (a call that would need
+ * to grow returns FRK_ERR_HIP and launches nothing). */
 
 /* y[rows] = W x for one activation vector in HBM.  K-quants: x is quantized to Q8_K
  * on the device first (bit-exact with quantize_activations_q8_k,
@@ -190,8 +197,10 @@ int frk_hip_route_top_k_softmax_dev(const float *logits_dev, size_t batch, size_
 
 /* Decoder::moe_ffn_batch (crates/frink-models/src/decoder/ffn_batch.rs:343-434) with SwiGLU experts
  * (frink_moe::run_expert, crates/frink-moe/src/lib.rs:1068-1165): out[batch][hidden] =
- * sum over each token's k routed experts, in ascending expert id, of
- * weights * down_e(silu(gate_e x) * up_e x).  gate/up/down hold the experts stacked row-wise
+ * sum over each token's k routed experts of weights * down_e(silu(gate_e x) * up_e x), added in the
+ * reference's order for a batch of this size: ascending expert id from 32 tokens on (its bucket path,
+ * ffn_batch.rs:355), routing order below (the per-position path's combine_expert_outputs,
+ * crates/frink-moe/src/lib.rs:1246-1263).  gate/up/down hold the experts stacked row-wise
  * (expert e = rows [e*ffn, (e+1)*ffn) of gate and up, [e*hidden, (e+1)*hidden) of down); gate and up
  * are Q4_K, down is Q4_K or Q6_K (other kinds: FRK_ERR_UNSUPPORTED).
  * ids[batch][k] / weights[batch][k] are a RoutingDecision per token (lib.rs:112-115); an id outside
@@ -201,7 +210,8 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
                         const float *weights_dev, size_t k, float *out_dev, void *stream);
 
 /* Test hooks for the bit-exact gates. */
-/* What the last frk_hip_moe_ffn_dev call of this shape on this stream left behind, copied out
+/* What the last frk_hip_moe_ffn_dev call of this shape on this stream left behind in the stream's
+ * scratch buffer (valid only if no other call on that stream came between), copied out
  * (null = skip): the gate and up projections [batch*k][ffn], silu(gate)*up quantized to Q8_K
  * (act_q [batch*k][ffn] i8, act_d [batch*k][ffn/256] f32), rows in grouped order, and
  * pos_of[tok*k + slot] = the row of a (token, slot) pair (the reference's bucket order,

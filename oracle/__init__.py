@@ -73,6 +73,8 @@ def lib():
             "fo_route_top_k_softmax": (None, [f32p, C.c_int, C.c_int, C.c_int, i32p, f32p]),
             "fo_moe_ffn_batch": (C.c_int, [C.c_int, u8p, u8p, u8p, C.c_int, C.c_int, C.c_int, f32p,
                                            C.c_int, i32p, f32p, C.c_int, f32p, C.c_int]),
+            "fo_moe_ffn_per_position": (C.c_int, [C.c_int, u8p, u8p, u8p, C.c_int, C.c_int, C.c_int, f32p,
+                                                  C.c_int, i32p, f32p, C.c_int, f32p, C.c_int]),
             "fo_have_avx2": (C.c_int, []),
         }
         for name, (res, args) in sig.items():
@@ -232,7 +234,23 @@ def route_top_k_softmax(logits, k, norm_topk_prob=True):
     return ids, w
 
 
-def moe_ffn_batch(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads=0):
+MOE_BUCKET_FROM = 32  # ffn_batch.rs:355: smaller batches run per position
+
+
+def moe_ffn(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads=0):
+    """The MoE layer the way the reference runs a batch of this size: bucketed by expert from 32
+    tokens on (experts added in ascending id), per position below (slots added in routing order)."""
+    batch = _f32(x).reshape(-1, hidden).shape[0]
+    fn = moe_ffn_batch if batch >= MOE_BUCKET_FROM else moe_ffn_per_position
+    return fn(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads)
+
+
+def moe_ffn_per_position(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads=0):
+    return moe_ffn_batch(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads,
+                         _fn="fo_moe_ffn_per_position")
+
+
+def moe_ffn_batch(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights, threads=0, _fn="fo_moe_ffn_batch"):
     gate, up, down = _u8(gate), _u8(up), _u8(down)
     x = _f32(x).reshape(-1, hidden)
     batch = x.shape[0]
@@ -240,11 +258,11 @@ def moe_ffn_batch(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights,
     weights = _f32(weights).reshape(batch, -1)
     k = ids.shape[1]
     out = np.empty((batch, hidden), np.float32)
-    rc = lib().fo_moe_ffn_batch(kind, _p(gate, C.c_uint8), _p(up, C.c_uint8), _p(down, C.c_uint8),
+    rc = getattr(lib(), _fn)(kind, _p(gate, C.c_uint8), _p(up, C.c_uint8), _p(down, C.c_uint8),
                                 n_experts, hidden, ffn, _p(x, C.c_float), batch, _p(ids, C.c_int32),
                                 _p(weights, C.c_float), k, _p(out, C.c_float), threads)
     if rc:
-        raise ValueError("fo_moe_ffn_batch rc=%d" % rc)
+        raise ValueError("%s rc=%d" % (_fn, rc))
     return out
 
 

@@ -1121,12 +1121,50 @@ void fo_route_top_k_softmax(const float *logits, int n, int k, int norm, int32_t
     free(taken);
 }
 
-/* frink-moe/src/lib.rs:1246-1263 (routed part) */
+/* frink-moe/src/lib.rs:1246-1263 (routed part): the slots of one token in the order given */
 void fo_combine_expert_outputs(const float *const *expert_out, const float *weights, int n,
                                int hidden, float *out) {
     for (int i = 0; i < hidden; i++) out[i] = 0.0f;
     for (int e = 0; e < n; e++)
         for (int i = 0; i < hidden; i++) out[i] += expert_out[e][i] * weights[e];
+}
+
+/* The path of a batch below 32 tokens (ffn_batch.rs:355 returns None, the caller then runs every
+ * position alone): per token, run_expert (frink-moe/src/lib.rs:1068-1165: gate and up over one
+ * quantization of the token, SwiGLU, down over a quantization of its own) for each routed slot,
+ * then combine_expert_outputs over the slots in routing order.  A slot whose id is outside
+ * [0, n_experts) is left out. */
+int fo_moe_ffn_per_position(int kind, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                            int n_experts, int hidden, int ffn, const float *x, int batch,
+                            const int32_t *ids, const float *weights, int k, float *out, int threads) {
+    int be = fo_block_elems(kind), bb = fo_block_bytes(kind);
+    if (!be || hidden % be || ffn % be) return -1;
+    size_t gu_bytes = (size_t)ffn * ((size_t)hidden / (size_t)be) * (size_t)bb;
+    size_t dn_bytes = (size_t)hidden * ((size_t)ffn / (size_t)be) * (size_t)bb;
+    float *g = (float *)malloc((size_t)ffn * sizeof(float));
+    float *u = (float *)malloc((size_t)ffn * sizeof(float));
+    float *outs = (float *)malloc((size_t)k * (size_t)hidden * sizeof(float));
+    const float **ptrs = (const float **)malloc((size_t)k * sizeof(float *));
+    float *w = (float *)malloc((size_t)k * sizeof(float));
+    for (int b = 0; b < batch; b++) {
+        const float *xb = x + (size_t)b * hidden;
+        int n = 0;
+        for (int s = 0; s < k; s++) {
+            int e = ids[b * k + s];
+            if (e < 0 || e >= n_experts) continue;
+            fo_gemv(kind, gate + (size_t)e * gu_bytes, (size_t)ffn, (size_t)hidden, xb, g, FO_MODE_INT_DOT, threads);
+            fo_gemv(kind, up + (size_t)e * gu_bytes, (size_t)ffn, (size_t)hidden, xb, u, FO_MODE_INT_DOT, threads);
+            fo_swiglu(g, u, (size_t)ffn, g);
+            fo_gemv(kind, down + (size_t)e * dn_bytes, (size_t)hidden, (size_t)ffn, g, outs + (size_t)n * hidden,
+                    FO_MODE_INT_DOT, threads);
+            ptrs[n] = outs + (size_t)n * hidden;
+            w[n] = weights[b * k + s];
+            n++;
+        }
+        fo_combine_expert_outputs(ptrs, w, n, hidden, out + (size_t)b * hidden);
+    }
+    free(g); free(u); free(outs); free((void *)ptrs); free(w);
+    return 0;
 }
 
 /* frink-models/src/decoder/ffn_batch.rs:343-434: bucket tokens by expert (token-major fill),

@@ -105,6 +105,11 @@ int fo_moe_ffn_batch(int kind, const uint8_t *gate, const uint8_t *up, const uin
                      int n_experts, int hidden, int ffn, const float *x, int batch,
                      const int32_t *ids, const float *weights, int k, float *out, int threads);
 
+/* The same layer the way a batch below 32 tokens runs it: per position, slots in routing order. */
+int fo_moe_ffn_per_position(int kind, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                            int n_experts, int hidden, int ffn, const float *x, int batch,
+                            const int32_t *ids, const float *weights, int k, float *out, int threads);
+
 /* CPU baseline: AVX2 dot where the host has it; returns 1 if AVX2 was used */
 int fo_have_avx2(void);
 

@@ -41,6 +41,15 @@ def make_weights(kind, rows, cols, seed, sigma=0.02):
     return fo.encode_matrix(kind, synth.weights(seed, rows, cols, sigma))
 
 
+def record(what, value):
+    """Measured worst-row figures survive `pytest -q` in a file (when the folder for run outputs exists)."""
+    import os
+    d = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    if os.path.isdir(d):
+        with open(os.path.join(d, "parity_worst_rows.txt"), "a") as f:
+            f.write("%s\t%.6g\n" % (what, value))
+
+
 def assert_rows_close(got, want, what):
     got = np.asarray(got, np.float32).reshape(want.shape)
     for b in range(want.shape[0]):
@@ -464,12 +473,18 @@ def test_route_top_k_softmax_matches_the_oracle(fa):
     assert ids.cpu().numpy().tolist() == [[1, 3]]
 
 
-def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False):
+def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False, sigma=0.05):
     """gate/up [E*ffn][hidden] and down [E*hidden][ffn] as Q4_K bytes."""
     shapes = ((n_experts * ffn, hidden), (n_experts * ffn, hidden), (n_experts * hidden, ffn))
     out = []
     for i, (rows, cols) in enumerate(shapes):
-        if random_blocks:
+        if random_blocks == "encoded":
+            # N(0, sigma) from numpy's generator (the documented splitmix generator takes minutes for
+            # 600 M values), encoded by the oracle's threaded Q4_K encoder
+            w = np.random.default_rng(seed + i).standard_normal((rows, cols), dtype=np.float32) * np.float32(sigma)
+            out.append(fo.encode_matrix(fo.Q4_K, w))
+            del w
+        elif random_blocks:
             # any bytes are a valid block; keep the two f16 super-scales small and finite
             rng = np.random.default_rng(seed + i)
             nblk = rows * cols // 256
@@ -478,18 +493,29 @@ def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False):
             data[:, 2:4] = rng.uniform(0.0005, 0.004, nblk).astype(np.float16).view(np.uint8).reshape(-1, 2)
             out.append(data.ravel())
         else:
-            out.append(make_weights(fo.Q4_K, rows, cols, seed=seed + i, sigma=0.05))
+            out.append(make_weights(fo.Q4_K, rows, cols, seed=seed + i, sigma=sigma))
     return out
 
 
+def _slot_order(ids_row, batch):
+    """The order in which the reference adds a token's routed slots: ascending expert id on its bucket
+    path (32 tokens and more, ffn_batch.rs:355, 388-423), routing order below that
+    (combine_expert_outputs, crates/frink-moe/src/lib.rs:1246-1263)."""
+    k = len(ids_row)
+    if batch >= fo.MOE_BUCKET_FROM:
+        return sorted(range(k), key=lambda s: (int(ids_row[s]), s))
+    return list(range(k))
+
+
 def _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w):
-    """moe_ffn_batch with the down experts in another kind than gate and up (a Q4_K_M checkpoint keeps
-    some layers' down experts in Q6_K): the oracle's own GEMMs and SwiGLU per expert bucket, summed per
-    token in ascending expert id like fo_moe_ffn_batch does."""
+    """The layer as the reference runs a batch of this size (fo.moe_ffn); with the down experts in
+    another kind than gate and up (a Q4_K_M checkpoint keeps some layers' down experts in Q6_K) from the
+    oracle's own GEMMs and SwiGLU per expert, added per token in the same order."""
     if down_kind == fo.Q4_K:
-        return fo.moe_ffn_batch(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+        return fo.moe_ffn(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
     gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
-    out = np.zeros((x.shape[0], hidden), np.float32)
+    batch, k = ids.shape
+    pair_out = np.zeros((batch, k, hidden), np.float32)
     for e in range(n_experts):
         toks, slots = np.nonzero(ids == e)
         if toks.size == 0:
@@ -497,26 +523,61 @@ def _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w):
         g = fo.gemm(fo.Q4_K, gb[e], ffn, hidden, x[toks])
         u = fo.gemm(fo.Q4_K, ub[e], ffn, hidden, x[toks])
         act = fo.swiglu(g.ravel(), u.ravel()).reshape(toks.size, ffn)
-        y = fo.gemm(down_kind, db[e], hidden, ffn, act)
-        for i, (t, sl) in enumerate(zip(toks, slots)):
-            out[t] += w[t, sl] * y[i]
+        pair_out[toks, slots] = fo.gemm(down_kind, db[e], hidden, ffn, act)
+    out = np.zeros((batch, hidden), np.float32)
+    for t in range(batch):
+        for sl in _slot_order(ids[t], batch):
+            if 0 <= ids[t, sl] < n_experts:
+                out[t] += w[t, sl] * pair_out[t, sl]
     return out
 
 
-def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, ids_override=None, down_kind=None):
+def _end_to_end_gate(got, want, what, strict):
+    """The Q8_K quantizer between the two GEMMs is a step function: a last-bit difference in a gate
+    output (any implementation that adds in another order than the oracle has them) can move an
+    intermediate to the next int8 level, which shifts that output row by d_act*|w|, and the fewer
+    columns the down projection has the larger that is against ||y||inf.  So the stage-by-stage gates
+    are the strict ones, and end to end a full-size layer (strict) must hold the tolerance on at least
+    99 % of its rows and twice the tolerance on every row (measured on the 128-expert layer of 2048/768:
+    1 row of 512 at 1.3e-3, the rest below 5e-7 apart from such flips), the small test shapes on 90 % of
+    the rows and ten times the tolerance on every row."""
+    rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
+    print("%s end-to-end: rows over 1e-3: %d of %d, worst %.3g" % (what, (rel > TOL).sum(), rel.size, rel.max()), flush=True)
+    record(what, rel.max())
+    if strict:
+        assert (rel <= TOL).mean() >= 0.99 and rel.max() <= 2 * TOL, "%s: worst row %.3g of ||y||inf" % (what, rel.max())
+    else:
+        assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, "%s: worst row %.3g" % (what, rel.max())
+
+
+def _swiglu_rounded_once(g, u):
+    """silu(g) * u with exp evaluated in double and rounded once to f32 -- the correctly rounded expf,
+    which is how the device evaluates it.  A host libm's expf (the oracle's, and the reference's scalar
+    build) returns the same value except for rare last-bit cases, and the reference's SIMD build uses a
+    polynomial a few ulp off, so the bit-exact gate on the quantized intermediate is stated on this
+    definition; the caller checks that it stays within a few ulp of the oracle's."""
+    g = np.asarray(g, np.float32)
+    with np.errstate(over="ignore"):  # exp(-g) of a very negative g is inf in f32, as on the device
+        e = np.exp(-g.astype(np.float64)).astype(np.float32)
+    return (g / (np.float32(1.0) + e)) * np.asarray(u, np.float32)
+
+
+def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, ids_override=None, down_kind=None,
+              sigma=0.05, strict=False):
     """The quantizer between the two GEMMs is a step function, so a last-bit difference in a
     gate/up output can move one intermediate value to the next int8 level and shift a whole output
     row by d_act*|w|: the end-to-end comparison alone cannot hold 1e-3 on every row for any
     implementation that sums in another order than the oracle.  The layer is therefore gated as a
     chain in which each link starts from the device's own previous result:
       1. gate/up grouped GEMM outputs (row of every (token, slot) pair) vs the oracle's GEMM  [tolerance]
-      2. silu(gate)*up and its Q8_K quantization, from the device's gate/up                   [bit-exact]
+      2. silu(gate)*up (exp rounded once, _swiglu_rounded_once) and its Q8_K quantization, from the device's gate/up  [bit-exact]
       3. down GEMM + weighted combine, from that same intermediate                            [tolerance]
-    and end to end against moe_ffn_batch: most rows inside the tolerance, all inside 10x."""
+    and end to end against the oracle's layer (_end_to_end_gate)."""
     from frink_amd import synth
     print("moe", n_experts, k, hidden, ffn, batch, flush=True)
-    gate, up, down = _stacked_experts(n_experts, hidden, ffn, seed, random_blocks)
+    gate, up, down = _stacked_experts(n_experts, hidden, ffn, seed, random_blocks, sigma)
     down_kind = fo.Q4_K if down_kind is None else down_kind
+    what = "moe E=%d k=%d %d/%d batch=%d down=%d" % (n_experts, k, hidden, ffn, batch, down_kind)
     if down_kind != fo.Q4_K:
         down = make_weights(down_kind, n_experts * hidden, ffn, seed=seed + 2, sigma=0.05)
     x = synth.activations(seed + 10, batch, hidden)
@@ -537,8 +598,7 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
         for h in (wg, wu, wd):
             h.release()
         want = _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w)
-        rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
-        assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, rel.max()
+        _end_to_end_gate(got, want, what, strict)
         return got, want
     g_out, u_out, act_q, act_d, pos = (t.cpu().numpy() for t in fa.moe_intermediates(batch, k, n_experts, hidden, ffn))
     for h in (wg, wu, wd):
@@ -550,7 +610,9 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
 
     gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
     want_down = np.zeros((batch * k, hidden), np.float32)
-    act = fo.swiglu(g_out.ravel(), u_out.ravel()).reshape(batch * k, ffn)
+    act = _swiglu_rounded_once(g_out, u_out).reshape(batch * k, ffn)
+    lib_act = fo.swiglu(g_out.ravel(), u_out.ravel()).reshape(batch * k, ffn)
+    assert (np.abs(act - lib_act) <= 4.8e-7 * np.abs(lib_act)).all()  # a few ulp: 1 in exp, then 1 + e, the quotient and the product
     for e in range(n_experts):
         rows = np.array([int(pos[t, s]) for ee, t, s in order if ee == e], dtype=np.int64)
         toks = np.array([t for ee, t, s in order if ee == e], dtype=np.int64)
@@ -562,23 +624,23 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     q, d, _ = fo.quantize_q8_k(act.ravel())
     assert np.array_equal(act_q.ravel(), q) and np.array_equal(bits(act_d.ravel()), bits(d))
     chained = np.zeros((batch, hidden), np.float32)
-    for e, t, s in order:  # ascending expert id per token: the reference's accumulation order
-        chained[t] += w[t, s] * want_down[pos[t, s]]
+    for t in range(batch):  # the reference's accumulation order for a batch of this size
+        for s in _slot_order(ids[t], batch):
+            chained[t] += w[t, s] * want_down[pos[t, s]]
     assert_rows_close(got, chained, "down+combine E=%d k=%d batch=%d" % (n_experts, k, batch))
 
     want = _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w)
-    rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
-    print("moe end-to-end: rows over 1e-3: %d of %d, worst %.3g" % ((rel > TOL).sum(), batch, rel.max()), flush=True)
-    assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, rel.max()
+    _end_to_end_gate(got, want, what, strict)
     return got, want
 
 
 def _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, batch, x, ids, w):
     """A token or a few run per (token, slot) pair on the decode kernels.  Each pair is then the dense
     SwiGLU FFN of its expert's three matrices -- the very kernels, so the layer must equal, bit for
-    bit, the library's own frk_hip_ffn_swiglu_dev on the expert's slices summed in ascending expert id
-    (that FFN is gated against the oracle in test_dense_ffn_swiglu and the GEMV tests) -- and end to
-    end it must agree with moe_ffn_batch like the grouped path."""
+    bit, the library's own frk_hip_ffn_swiglu_dev on the expert's slices added in routing order, as the
+    reference's per-position path adds them (that FFN is gated against the oracle in
+    test_dense_ffn_swiglu and the GEMV tests) -- and end to end it must agree with the oracle's
+    per-position layer."""
     with pytest.raises(fa.BackendError) as e:
         fa.moe_intermediates(batch, k, n_experts, hidden, ffn)
     assert e.value.code == fa.ERR_UNSUPPORTED
@@ -587,7 +649,7 @@ def _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, ba
     cache = {}
     for t in range(batch):
         xd = to_dev(x[t])
-        for s in sorted(range(k), key=lambda s: (int(ids[t, s]), s)):
+        for s in range(k):  # routing order (combine_expert_outputs, crates/frink-moe/src/lib.rs:1246-1263)
             ex = int(ids[t, s])
             if ex not in cache:
                 cache[ex] = (fa.Weights.from_host(fo.Q4_K, gb[ex], ffn, hidden), fa.Weights.from_host(fo.Q4_K, ub[ex], ffn, hidden),
@@ -599,10 +661,9 @@ def _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, ba
         for h in hs:
             h.release()
     assert np.array_equal(bits(got), bits(composed)), np.abs(got - composed).max()
-    want = fo.moe_ffn_batch(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
-    rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
-    print("moe per token end-to-end: worst %.3g" % rel.max(), flush=True)
-    assert (rel <= TOL).mean() >= 0.5 and rel.max() <= 10 * TOL, rel.max()
+    want = fo.moe_ffn(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    _end_to_end_gate(got, want, "moe per token E=%d k=%d %d/%d batch=%d" % (n_experts, k, hidden, ffn, batch),
+                     strict=hidden >= 2048)
     return got, want
 
 
@@ -649,11 +710,45 @@ def test_moe_ffn_with_idle_experts_and_one_hot_routing(fa):
 
 
 def test_moe_ffn_full_size_layer(fa):
-    """128 experts, top-8, hidden 2048, ffn 768, 512 tokens: every token row against the oracle.
-    Weights are random block bytes with small positive super-scales (encoding 600 M weights on the
-    CPU would take minutes); the expert arithmetic does not care where the bytes came from."""
+    """The MoE configuration itself: 128 experts, top-8, hidden 2048, ffn 768, all Q4_K encoded from
+    N(0, 0.02), 512 tokens N(0, 1): every stage and every token row against the oracle, and the whole
+    layer end to end (_end_to_end_gate, strict)."""
+    got, want = _moe_case(fa, 128, 8, 2048, 768, 512, seed=5, random_blocks="encoded", sigma=0.02, strict=True)
+    assert np.isfinite(got).all()
+
+
+def test_moe_ffn_full_size_layer_arbitrary_block_bytes(fa):
+    """The same shape over arbitrary block bytes (every scale, min and nibble pattern): stage gates
+    strict as always; end to end the larger cancellation of such weights leaves the relaxed gate."""
     got, want = _moe_case(fa, 128, 8, 2048, 768, 512, seed=5, random_blocks=True)
     assert np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("batch", [3, 40])
+def test_moe_ffn_leaves_out_ids_outside_the_experts(fa, batch):
+    """An id outside [0, n_experts) contributes nothing, on the per-token path (batch 3) and on the grouped
+    path (batch 40) alike: the oracle with those slots dropped."""
+    def spoil(ids):
+        ids = ids.copy()
+        ids[0, 0] = -1
+        ids[1, 1] = 8
+        ids[batch - 1, :] = np.array([8, -1], np.int32)  # a token with no valid slot: zeros
+        return ids
+    n_experts, k, hidden, ffn = 8, 2, 256, 256
+    from frink_amd import synth
+    gate, up, down = _stacked_experts(n_experts, hidden, ffn, 4242)
+    x = synth.activations(4250, batch, hidden)
+    ids, w = _route(synth.normal(4251, batch * n_experts).reshape(batch, n_experts), k)
+    ids = spoil(ids.astype(np.int32))
+    hs = [fa.Weights.from_host(fo.Q4_K, m, r, c) for m, r, c in ((gate, n_experts * ffn, hidden), (up, n_experts * ffn, hidden),
+                                                                 (down, n_experts * hidden, ffn))]
+    got = fa.moe_ffn(hs[0], hs[1], hs[2], n_experts, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    for h in hs:
+        h.release()
+    want = fo.moe_ffn(fo.Q4_K, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    assert not got[batch - 1].any() and not want[batch - 1].any()
+    rel = np.abs(got[:-1] - want[:-1]).max(axis=1) / np.abs(want[:-1]).max(axis=1)
+    assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, rel.max()
 
 
 # ------------------------------------------------------------------ the C++ host mirror
@@ -910,7 +1005,10 @@ def test_dense_ffn_swiglu(fa, hidden, ffn):
     e2e = fo.gemv(fo.Q6_K, down, hidden, ffn, fo.swiglu(g, u))
     rel = np.abs(y - e2e).max() / np.abs(e2e).max()
     print("ffn end to end: %.3g of ||y||inf" % rel, flush=True)
-    assert rel <= 10 * TOL
+    record("dense ffn %dx%d end to end" % (hidden, ffn), rel)
+    # the full-size FFN holds the tolerance itself; the small one only ten times it (the quantizer
+    # between the projections is a step function, see _end_to_end_gate)
+    assert rel <= (TOL if hidden >= 4096 else 10 * TOL), rel
     if hidden == 512:  # the host-buffer form (launch_dense_ffn_swiglu)
         out = fa.launch_dense_ffn_swiglu(fa.MatvecLaunch.of(fo.Q4_K, gate, ffn, hidden // 256 * 144),
                                          fa.MatvecLaunch.of(fo.Q4_K, up, ffn, hidden // 256 * 144),
@@ -918,3 +1016,63 @@ def test_dense_ffn_swiglu(fa, hidden, ffn):
         assert np.array_equal(bits(out), bits(y))
     for w in (wg, wu, wd):
         w.release()
+
+
+# ------------------------------------------------------------------ scratch memory per stream
+
+def test_dev_calls_on_two_streams_from_two_threads(fa):
+    """Two threads, each on a stream of its own, enqueue calls of different shapes that all use the
+    library's scratch memory (quantized activations, split-K parts, MoE intermediates), a small shape
+    first and a larger one after it, so that each stream's buffer is replaced while the other stream is
+    busy.  Every result must be the one the same call gives alone, and agree with the oracle."""
+    import threading
+    import torch
+    from frink_amd import synth
+    shapes = {"a": (fo.Q4_K, 384, 1024, (40, 130)), "b": (fo.Q6_K, 256, 2048, (48, 200))}
+    mats, xs, alone = {}, {}, {}
+    for name, (kind, rows, cols, batches) in shapes.items():
+        data = make_weights(kind, rows, cols, seed=900 + kind)
+        mats[name] = (data, fa.Weights.from_host(kind, data, rows, cols))
+        xs[name] = [to_dev(synth.activations(910 + b, b, cols)) for b in batches]
+        alone[name] = [mats[name][1].gemm(x).cpu().numpy() for x in xs[name]]
+    # a MoE layer on stream "a" as well (its intermediates live in the same scratch buffer)
+    E, k, hidden, ffn, batch = 8, 2, 256, 256, 40
+    gate, up, down = _stacked_experts(E, hidden, ffn, 930)
+    hs = [fa.Weights.from_host(fo.Q4_K, m, r, c) for m, r, c in ((gate, E * ffn, hidden), (up, E * ffn, hidden), (down, E * hidden, ffn))]
+    xm = to_dev(synth.activations(931, batch, hidden))
+    ids, wts = _route(synth.normal(932, batch * E).reshape(batch, E), k)
+    ids_d, wts_d = to_dev(ids.astype(np.int32)), to_dev(wts)
+    moe_alone = fa.moe_ffn(hs[0], hs[1], hs[2], E, xm, ids_d, wts_d).cpu().numpy()
+    torch.cuda.synchronize()
+
+    results, errors = {}, []
+
+    def work(name):
+        try:
+            stream = torch.cuda.Stream()  # default priority
+            with torch.cuda.stream(stream):
+                last = None
+                for rep in range(12):
+                    outs = [mats[name][1].gemm(x) for x in xs[name]]
+                    if name == "a":
+                        last = fa.moe_ffn(hs[0], hs[1], hs[2], E, xm, ids_d, wts_d)
+                stream.synchronize()
+            results[name] = [o.cpu().numpy() for o in outs] + ([last.cpu().numpy()] if last is not None else [])
+        except Exception as e:  # noqa: BLE001 - reported in the main thread
+            errors.append((name, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(n,)) for n in shapes]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not errors, errors
+    for name, (kind, rows, cols, batches) in shapes.items():
+        for got, want_alone, x in zip(results[name], alone[name], xs[name]):
+            assert np.array_equal(bits(got), bits(want_alone)), "%s: differs from the same call alone" % name
+            assert_rows_close(got, fo.gemm(kind, mats[name][0], rows, cols, x.cpu().numpy()), "two streams, %s" % name)
+    assert np.array_equal(bits(results["a"][-1]), bits(moe_alone))
+    for _, w in mats.values():
+        w.release()
+    for h in hs:
+        h.release()

@@ -540,3 +540,42 @@ def test_moe_batch_equals_per_token_experts_combined():
             o = fo.gemv(fo.Q4_K, down[e * dn:(e + 1) * dn], hidden, ffn, fo.swiglu(g, u))
             acc = acc + we * o
         assert np.array_equal(got[b].view(np.uint32), acc.view(np.uint32))
+
+
+def test_moe_per_position_adds_the_slots_in_routing_order():
+    """Below 32 tokens the reference runs every position alone (ffn_batch.rs:355) and
+    combine_expert_outputs (frink-moe/src/lib.rs:1246-1263) adds the routed slots in routing order;
+    the batch path adds them in ascending expert id.  So the two paths agree bit for bit on a token
+    whose routing order is ascending, and to rounding otherwise -- and a slot with an id outside the
+    experts is left out of both."""
+    E, k, hidden, ffn, batch = 8, 3, 256, 256, 7
+    gate = _weights(fo.Q4_K, E * ffn, hidden)
+    up = _weights(fo.Q4_K, E * ffn, hidden)
+    down = _weights(fo.Q4_K, E * hidden, ffn)
+    x = RNG.standard_normal((batch, hidden)).astype(np.float32)
+    logits = RNG.standard_normal((batch, E)).astype(np.float32)
+    routed = [fo.route_top_k_softmax(l, k, True) for l in logits]
+    ids = np.stack([r[0] for r in routed]).astype(np.int32)
+    w = np.stack([r[1] for r in routed])
+    ids[0] = np.sort(ids[0])           # ascending routing order: both paths add in the same order
+    ids[1] = np.sort(ids[1])[::-1]     # descending: the orders differ
+    ids[2, 1] = E                      # an id outside the experts
+    ids[3, 0] = -1
+    per_pos = fo.moe_ffn_per_position(fo.Q4_K, gate, up, down, E, hidden, ffn, x, ids, w)
+    bucket = fo.moe_ffn_batch(fo.Q4_K, gate, up, down, E, hidden, ffn, x, ids, w)
+    assert np.array_equal(per_pos[0].view(np.uint32), bucket[0].view(np.uint32))
+    assert np.abs(per_pos - bucket).max() <= 2e-6 * np.abs(bucket).max()
+    gu, dn = ffn * (hidden // 256) * 144, hidden * (ffn // 256) * 144
+    for b in range(batch):
+        acc = np.zeros(hidden, np.float32)
+        for s in range(k):  # routing order
+            e = int(ids[b, s])
+            if not 0 <= e < E:
+                continue
+            g = fo.gemv(fo.Q4_K, gate[e * gu:(e + 1) * gu], ffn, hidden, x[b])
+            u = fo.gemv(fo.Q4_K, up[e * gu:(e + 1) * gu], ffn, hidden, x[b])
+            o = fo.gemv(fo.Q4_K, down[e * dn:(e + 1) * dn], hidden, ffn, fo.swiglu(g, u))
+            acc = acc + o * w[b, s]
+        assert np.array_equal(per_pos[b].view(np.uint32), acc.view(np.uint32)), b
+    # the dispatcher follows the reference's threshold
+    assert np.array_equal(fo.moe_ffn(fo.Q4_K, gate, up, down, E, hidden, ffn, x, ids, w), per_pos)
