@@ -947,9 +947,26 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 }
 
 constexpr int Q4K_MAX_SPLIT = 4;
-// the tiled activations, then room for the parts' sums
+// The workgroup tile of a batch: 256 rows x 128 or 64 tokens when that still gives (about) every CU a
+// workgroup, else 128 rows x 64 or 32 tokens -- and with those small tiles, when the grid fills few of
+// the CUs, a row's blocks split between 2 or 4 workgroups (no finer than four blocks each) whose sums
+// are added in order afterwards.
+struct Q4KPlan {
+    int rows_wg, tok_wg, k_split;
+};
+static Q4KPlan q4_k_plan(size_t rows, size_t M, size_t nb) {
+    if (M > 64 && ((rows + 255) / 256) * ((M + 127) / 128) >= 200) return {256, 128, 1};
+    if (M > 64 && ((rows + 255) / 256) * ((M + 63) / 64) >= 256) return {256, 64, 1};
+    const int tm = M > 32 ? 64 : 32;
+    const size_t grid = (((rows + 127) / 128 + 7) / 8 * 8) * ((M + (size_t)tm - 1) / (size_t)tm);
+    int ks = 1;
+    while (ks < Q4K_MAX_SPLIT && grid * (size_t)ks * 2 <= 256 && nb / (size_t)(ks * 2) >= 4) ks *= 2;
+    return {128, tm, ks};
+}
+// the tiled activations, then room for the parts' sums where the blocks are split
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
-    return round_up(q8k_tiled_bytes(M, cols), 256) + (size_t)Q4K_MAX_SPLIT * M * rows * sizeof(float);
+    const Q4KPlan p = q4_k_plan(rows, M, cols / QK_K);
+    return round_up(q8k_tiled_bytes(M, cols), 256) + (p.k_split > 1 ? (size_t)p.k_split * M * rows * sizeof(float) : 0);
 }
 
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
@@ -969,21 +986,13 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.y = y;
     g.k_split = 1;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
-    // shape of a workgroup's tile: 256 rows x 128 or 64 tokens when that still gives (about) every CU a
-    // workgroup, else 128 rows x 64 or 32 tokens
-    auto grid_for = [&](int rows_wg, int tm) {
-        g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
-        g.tok_tiles = (int)((M + tm - 1) / tm);
-        return (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
-    };
-    const size_t wgs_big = ((w->rows + 255) / 256) * ((M + 63) / 64);
-    if (M > 64 && ((w->rows + 255) / 256) * ((M + 127) / 128) >= 200) return launch_variant<8, 1, 4, 2>(g, grid_for(256, 128), s);
-    if (M > 64 && wgs_big >= 256) return launch_variant<8, 1, 2, 2>(g, grid_for(256, 64), s);
-    // The small tiles of a batch that fills few of the CUs: a row's blocks are split between 2 or 4
-    // workgroups (no finer than four blocks each) whose sums are added in order afterwards.
-    const unsigned grid = M > 32 ? grid_for(128, 64) : grid_for(128, 32);
-    while (g.k_split < Q4K_MAX_SPLIT && (size_t)grid * g.k_split * 2 <= 256 && g.nb / (g.k_split * 2) >= 4) g.k_split *= 2;
-    if (M > 32) return launch_variant<4, 2, 1, 4>(g, grid, s);
+    const Q4KPlan p = q4_k_plan(w->rows, M, (size_t)g.nb);
+    g.row_tiles = (int)((w->rows + p.rows_wg - 1) / p.rows_wg);
+    g.tok_tiles = (int)((M + p.tok_wg - 1) / p.tok_wg);
+    g.k_split = p.k_split;
+    const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
+    if (p.rows_wg == 256) return p.tok_wg == 128 ? launch_variant<8, 1, 4, 2>(g, grid, s) : launch_variant<8, 1, 2, 2>(g, grid, s);
+    if (p.tok_wg == 64) return launch_variant<4, 2, 1, 4>(g, grid, s);
     return launch_variant<4, 1, 1, 2>(g, grid, s);
 }
 

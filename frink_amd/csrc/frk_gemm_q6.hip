@@ -436,9 +436,19 @@ int launch_sum_parts(const float *partial, int parts, size_t n, float *y, hipStr
 // fewer 256-row workgroups than this leave too many CUs idle: split the blocks, or take 128-row ones
 constexpr size_t Q6_NARROW_BELOW = 200;
 constexpr int Q6_MAX_SPLIT = 8;
-// the tiled activations, then room for the parts' sums
+// 256 weight rows per workgroup (a block is unpacked once for two tiles) when that gives about every
+// CU one.  For a short and wide matrix, or a batch of few token tiles, the blocks are split between 2,
+// 4 or 8 workgroups (no finer than four blocks each) whose sums a second kernel adds up in order.
+static int q6_k_split(size_t rows, size_t M, size_t nb) {
+    const size_t wgs256 = ((rows + 255) / 256) * ((M + 63) / 64);
+    int ks = 1;
+    while (ks < Q6_MAX_SPLIT && wgs256 < Q6_NARROW_BELOW && wgs256 * ks * 2 <= 256 && nb / (size_t)(ks * 2) >= 4) ks *= 2;
+    return ks;
+}
+// the tiled activations, then room for the parts' sums where the blocks are split
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
-    return round_up(q8k_tiled_bytes(M, cols), 256) + (size_t)Q6_MAX_SPLIT * M * rows * sizeof(float);
+    const int ks = q6_k_split(rows, M, cols / QK_K);
+    return round_up(q8k_tiled_bytes(M, cols), 256) + (ks > 1 ? (size_t)ks * M * rows * sizeof(float) : 0);
 }
 
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
@@ -460,13 +470,10 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.M = (int)M;
     g.y = y;
     g.tok_tiles = (int)((M + 63) / 64);
-    // 256 weight rows per workgroup (a block is unpacked once for two tiles) when that gives about
-    // every CU one.  For a short and wide matrix, or a batch of few token tiles, the blocks are split
-    // between 2, 4 or 8 workgroups (no finer than four blocks each) whose sums a second kernel adds
-    // up in order; 128 rows where even that leaves most CUs idle.
+    // the blocks split between workgroups (q6_k_split), or 128 rows per workgroup where even that
+    // leaves most CUs idle
     const size_t wgs256 = ((w->rows + 255) / 256) * (size_t)g.tok_tiles;
-    int ks = 1;
-    while (ks < Q6_MAX_SPLIT && wgs256 < Q6_NARROW_BELOW && wgs256 * ks * 2 <= 256 && g.nb / (ks * 2) >= 4) ks *= 2;
+    const int ks = q6_k_split(w->rows, M, (size_t)g.nb);
     const bool split = ks > 1;
     const bool narrow = wgs256 < Q6_NARROW_BELOW && !split;
     const int rows_wg = narrow ? 128 : 256;

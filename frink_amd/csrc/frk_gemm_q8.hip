@@ -321,9 +321,20 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     } while (0)
 
 constexpr int Q8_MAX_SPLIT = 8;
-// the quantized activations, their scales, and room for the parts' sums
+// A small grid (few token tiles, a short matrix) splits the chunks of a row between 2, 4 or 8
+// workgroups, no finer than two pairs of chunks each; their sums are added in order afterwards.
+static int q8_0_split(size_t rows, size_t M, size_t nb32) {
+    const size_t wgs = M > 32 ? ((rows + 63) / 64) * ((M + 127) / 128) : (rows + 31) / 32;
+    const size_t pairs = ((nb32 + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS + 1) / 2;
+    int ks = 1;
+    const size_t fill = M > 32 ? 256 : 1024;  // (the one-wavefront workgroups of the thinnest batches: four per CU)
+    while (ks < Q8_MAX_SPLIT && wgs * ks * 2 <= fill && pairs / (size_t)(ks * 2) >= 2) ks *= 2;
+    return ks;
+}
+// the quantized activations, their scales, and room for the parts' sums where the chunks are split
 size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows) {
-    return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256) + (size_t)Q8_MAX_SPLIT * M * rows * sizeof(float);
+    const int ks = q8_0_split(rows, M, cols / 32);
+    return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256) + (ks > 1 ? (size_t)ks * M * rows * sizeof(float) : 0);
 }
 
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
@@ -362,13 +373,7 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
         sized = true;
     }
     const bool q4 = w->kind == FRK_KIND_Q4_0;
-    // A small grid (few token tiles, a short matrix) splits the chunks of a row between 2, 4 or 8
-    // workgroups, no finer than two pairs of chunks each; their sums are added in order afterwards.
-    const size_t wgs = M > 32 ? ((w->rows + 63) / 64) * ((M + 127) / 128) : (w->rows + 31) / 32;
-    const int pairs = ((g.nb + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS + 1) / 2;
-    int ks = 1;
-    const size_t fill = M > 32 ? 256 : 1024;  // (the one-wavefront workgroups of the thinnest batches: four per CU)
-    while (ks < Q8_MAX_SPLIT && wgs * ks * 2 <= fill && pairs / (ks * 2) >= 2) ks *= 2;
+    const int ks = q8_0_split(w->rows, M, (size_t)g.nb);
     g.k_split = ks;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));
     const unsigned kz = (unsigned)ks;
