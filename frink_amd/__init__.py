@@ -28,7 +28,7 @@ EXPORTS = [
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
     "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
-    "frk_hip_gemm_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
+    "frk_hip_gemm_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
@@ -87,6 +87,7 @@ def lib():
             "frk_hip_gemv_dev": (i, [vp, vp, vp, i, vp]),
             "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
+            "frk_hip_gemm_noalloc_dev": (i, [vp, vp, sz, vp, vp]),
             "frk_hip_route_top_k_softmax_dev": (i, [vp, sz, sz, sz, i, vp, vp, vp]),
             "frk_hip_moe_ffn_dev": (i, [vp, vp, vp, sz, vp, sz, vp, vp, sz, vp, vp]),
             "frk_hip_moe_intermediates_dev": (i, [sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
@@ -201,6 +202,16 @@ class Weights:
         check(lib().frk_hip_gemm_dev(self.handle, C.c_void_p(x.data_ptr()), batch, C.c_void_p(y.data_ptr()),
                                      _stream()))
         return y
+
+    def gemm_noalloc(self, x, out):
+        """frk_hip_gemm_noalloc_dev: the caller brings the output; the call allocates nothing."""
+        import torch
+        assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.shape[-1] == self.cols
+        batch = x.numel() // self.cols
+        assert out.dtype == torch.float32 and out.is_cuda and out.is_contiguous() and out.numel() == batch * self.rows
+        check(lib().frk_hip_gemm_noalloc_dev(self.handle, C.c_void_p(x.data_ptr()), batch, C.c_void_p(out.data_ptr()),
+                                             _stream()))
+        return out
 
     def dequant(self):
         import torch

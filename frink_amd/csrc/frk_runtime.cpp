@@ -114,10 +114,12 @@ int workspace(size_t bytes, hipStream_t stream, WorkspaceLease &lease) {
         if (it == g_ws.end()) it = g_ws.emplace(stream, new StreamWorkspace()).first;
         w = it->second;
     }
-    w->mu.lock();
-    w->depth++;
-    lease.held_ = w;
-    lease.stream_ = stream;
+    if (lease.held_ != w) {  // (a lease asked again, by a later step of the same call, keeps its one hold)
+        w->mu.lock();
+        w->depth++;
+        lease.held_ = w;
+        lease.stream_ = stream;
+    }
     if (bytes > w->bytes) {
         hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
         if (hipStreamIsCapturing(stream, &cs) != hipSuccess) (void)hipGetLastError();
@@ -415,15 +417,37 @@ int frk_hip_read_dev(const void *src, size_t bytes, void *sink, void *stream) {
     return launch_read(src, bytes, sink, (hipStream_t)stream);
 }
 
-// Quantizes `batch` activation rows of w->cols values to Q8_K in the workspace.
-// (the lease must outlive the launches that read `a`)
-static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch, hipStream_t s, WorkspaceLease &lease,
+// Where one call's scratch memory comes from: the stream's leased buffer (grown on demand), or a fixed
+// region that has to suffice (the entry point that allocates nothing).  It must outlive the launches that
+// use the memory; nested requests of one call get the same start address, as with the lease.
+struct Scratch {
+    WorkspaceLease lease;
+    void *fixed = nullptr;
+    size_t fixed_bytes = 0;
+    Scratch() = default;
+    Scratch(void *region, size_t bytes) : fixed(region), fixed_bytes(bytes) {}
+    int get(size_t bytes, hipStream_t s, void **out) {
+        if (fixed) {
+            if (bytes > fixed_bytes)
+                return set_error(FRK_ERR_SHAPE, "this shape needs %zu bytes of scratch memory, the entry point that allocates nothing has %zu",
+                                 bytes, fixed_bytes);
+            *out = fixed;
+            return FRK_OK;
+        }
+        int rc = workspace(bytes, s, lease);
+        *out = lease.ptr;
+        return rc;
+    }
+};
+
+// Quantizes `batch` activation rows of w->cols values to Q8_K in the call's scratch memory.
+static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch, hipStream_t s, Scratch &scratch,
                               Q8KActs *a) {
     size_t n = batch * w->cols;
     size_t q_bytes = round_up(n, 256), d_bytes = round_up(n / QK_K * 4, 256), b_bytes = round_up(n / 16 * 2, 256);
-    int rc = workspace(q_bytes + d_bytes + b_bytes, s, lease);
+    void *ws = nullptr;
+    int rc = scratch.get(q_bytes + d_bytes + b_bytes, s, &ws);
     if (rc) return rc;
-    void *ws = lease.ptr;
     int8_t *q = (int8_t *)ws;
     float *d = (float *)((char *)ws + q_bytes);
     int16_t *b = (int16_t *)((char *)ws + q_bytes + d_bytes);
@@ -435,10 +459,7 @@ static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch
     return FRK_OK;
 }
 
-int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mode, void *stream) {
-    clear_error();
-    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_dev: null argument");
-    hipStream_t s = (hipStream_t)stream;
+static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mode, hipStream_t s, Scratch &scratch) {
     switch (w->kind) {
     case FRK_KIND_Q4_K:
         if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
@@ -447,8 +468,7 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q6_K: {
         if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
         Q8KActs a;
-        WorkspaceLease lease;
-        int rc = quantize_acts_q8_k(w, x, 1, s, lease, &a);
+        int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
         if (rc) return rc;
         if (w->kind == FRK_KIND_Q4_K) return launch_gemv_q4_k(w, a, y, s);
         if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, s);
@@ -461,10 +481,9 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
             return direct_gemv_fits(w) ? launch_gemv_q8_0_f32_direct(w, x, y, s) : launch_gemv_q8_0_f32(w, x, y, s);
         }
         size_t n = w->cols;
-        WorkspaceLease lease;
-        int rc = workspace(round_up(n, 256) + n / 32 * 4, s, lease);
+        void *ws = nullptr;
+        int rc = scratch.get(round_up(n, 256) + n / 32 * 4, s, &ws);
         if (rc) return rc;
-        void *ws = lease.ptr;
         int8_t *q = (int8_t *)ws;
         float *d = (float *)((char *)ws + round_up(n, 256));
         rc = launch_quantize_q8_0(x, n, q, d, s);
@@ -473,6 +492,13 @@ int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mod
     }
     }
     return set_error(FRK_ERR_UNSUPPORTED, "no matvec kernel for quant kind %d", w->kind);
+}
+
+int frk_hip_gemv_dev(const frk_weights *w, const float *x, float *y, int act_mode, void *stream) {
+    clear_error();
+    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_dev: null argument");
+    Scratch scratch;
+    return gemv_impl(w, x, y, act_mode, (hipStream_t)stream, scratch);
 }
 
 int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, const int16_t *bsums, float *y,
@@ -490,45 +516,41 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d)", w->kind);
 }
 
-int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *y, void *stream) {
-    clear_error();
-    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
-    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
     // Q4_K: up to two launches of the thin kernel (16 rows each: 15 us at 14336x4096, 10 us at 4096x4096)
     // are ahead of the matrix-core GEMM (28 us and 18 us there for 33..64 rows, its blocks split between
     // workgroups)
     const size_t q4k_thin_rows = 32;
     if (w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16)) {
-        WorkspaceLease lease;
-        int rc = workspace(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
+        void *ws = nullptr;
+        int rc = scratch.get(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
-        return launch_gemm_q4_k(w, x, batch, y, lease.ptr, (hipStream_t)stream);
+        return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // Q6_K: the matrix-core GEMM (with its blocks split between workgroups for small batches: 53 us at
     // 4096x14336 and 31 us at 4096x4096 up to 64 rows) is ahead of the thin kernel's 8-row groups (15 us
     // and 6 us each) from four groups on for large matrices and from six on for small ones
     const size_t q6k_gemm_from = w->rows * w->cols > (size_t)2 * 4096 * 4096 ? 25 : 41;
     if (w->kind == FRK_KIND_Q6_K && batch >= q6k_gemm_from) {
-        WorkspaceLease lease;
-        int rc = workspace(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
+        void *ws = nullptr;
+        int rc = scratch.get(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
-        return launch_gemm_q6_k(w, x, batch, y, lease.ptr, (hipStream_t)stream);
+        return launch_gemm_q6_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // Q8_0: a batch is the integer path, as in the reference (Q8_0 activation blocks and dot_q8_0_q8,
     // crates/frink-core/src/weight_matrix.rs:2701-2829); a single row keeps the f32 dot of its decode path
     if ((w->kind == FRK_KIND_Q8_0 || w->kind == FRK_KIND_Q4_0) && batch >= 2) {  // (Q4_0: the same kernel, dot_q4_0_q8)
-        WorkspaceLease lease;
-        int rc = workspace(gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, lease);
+        void *ws = nullptr;
+        int rc = scratch.get(gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
-        return launch_gemm_q8_0(w, x, batch, y, lease.ptr, (hipStream_t)stream);
+        return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K) && batch >= 2
                          ? thin_gemm_max_batch(w) : 0;
     if (thin >= 2) {
         Q8KActs a;
-        WorkspaceLease lease;
-        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, lease, &a);
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, scratch, &a);
         if (rc) return rc;
         const size_t nb = w->cols / QK_K;
         if (batch > (size_t)thin && batch <= (size_t)thin_gemm_wide_rows(w))
@@ -545,8 +567,7 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     // decode kernel
     if (w->kind == FRK_KIND_Q5_K) {
         Q8KActs a;
-        WorkspaceLease lease;
-        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, lease, &a);
+        int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, scratch, &a);
         if (rc) return rc;
         const size_t nb = w->cols / QK_K;
         for (size_t b = 0; b < batch; b++) {
@@ -559,10 +580,53 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     // otherwise one matvec per activation row (the reference's own path below its GEMM threshold,
     // crates/frink-core/src/weight_matrix.rs:2636-2652)
     for (size_t b = 0; b < batch; b++) {
-        int rc = frk_hip_gemv_dev(w, x + b * w->cols, y + b * w->rows, FRK_ACT_F32, stream);
+        int rc = gemv_impl(w, x + b * w->cols, y + b * w->rows, FRK_ACT_F32, (hipStream_t)stream, scratch);
         if (rc) return rc;
     }
     return FRK_OK;
+}
+
+int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *y, void *stream) {
+    clear_error();
+    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_dev: null argument");
+    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+    Scratch scratch;
+    return gemm_impl(w, x, batch, y, stream, scratch);
+}
+
+// ---- the entry point that allocates nothing ----
+// Its scratch memory is this array in the library's device image: every GPU the library runs on holds
+// its own copy, at its own address, until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress; what the kernels get is the address looked up once per device.
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)FRK_NOALLOC_SCRATCH_MIB << 20;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static void *g_scratch_addr[NOALLOC_MAX_DEVICES] = {nullptr};  // under g_dev.mu
+
+static int noalloc_scratch(void **out) {
+    int dev = -1;
+    FRK_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return set_error(FRK_ERR_NO_DEVICE, "device %d: at most %d devices", dev, NOALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    if (!g_scratch_addr[dev]) {  // first call on this device, which is the current one
+        void *ptr = nullptr;
+        FRK_HIP_TRY(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return set_error(FRK_ERR_HIP, "hipGetSymbolAddress gave no address for the scratch array");
+        g_scratch_addr[dev] = ptr;
+    }
+    *out = g_scratch_addr[dev];
+    return FRK_OK;
+}
+
+int frk_hip_gemm_noalloc_dev(const frk_weights *w, const float *x, size_t batch, float *y, void *stream) {
+    clear_error();
+    if (!w || !x || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_noalloc_dev: null argument");
+    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+    void *region = nullptr;
+    int rc = noalloc_scratch(&region);
+    if (rc) return rc;
+    Scratch fixed(region, NOALLOC_SCRATCH_BYTES);
+    return gemm_impl(w, x, batch, y, stream, fixed);
 }
 
 int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *x, float *const *ys, void *stream) {
@@ -608,9 +672,9 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     }
     // otherwise one Q8_K quantization for every K-quant matrix of the group
     Q8KActs a = {nullptr, nullptr, nullptr};
-    WorkspaceLease lease;
+    Scratch scratch;
     if (any_k) {
-        int rc = quantize_acts_q8_k(ws[0], x, 1, s, lease, &a);
+        int rc = quantize_acts_q8_k(ws[0], x, 1, s, scratch, &a);
         if (rc) return rc;
     }
     for (size_t i = 0; i < n; i++) {

@@ -188,6 +188,19 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
                      void *stream);
 
+/* frk_hip_gemm_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same
+ * kernels and bit for bit the same y, but the scratch memory (quantized activations, the parts of a
+ * split GEMM) is a fixed array of FRK_NOALLOC_SCRATCH_MIB MiB inside the library's device image, looked
+ * up on the first call on a device; the call never allocates or frees.  A shape whose scratch does not
+ * fit returns FRK_ERR_SHAPE and launches nothing (it fits every batch of up to 64 rows of matrices up to
+ * 16384 columns, and prefill batches of 512 rows of 4096 columns that need no split).  Every call on a
+ * GPU shares that GPU's array: calls that overlap on one GPU (two streams, two threads) race -- enqueue
+ * them on one stream. */
+#define FRK_NOALLOC_SCRATCH_MIB 16
+int frk_hip_gemm_noalloc_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
+                             void *stream);
+
 /* frink_moe::route_top_k_softmax (crates/frink-moe/src/lib.rs:567-589) for a batch of tokens:
  * logits[batch][n_experts] -> ids[batch][k] (probability descending), weights[batch][k]
  * (probs[ids], divided by their sum when norm != 0).  Equal probabilities, which the reference's
