@@ -288,8 +288,8 @@ __device__ __forceinline__ void tile_mfmas_as_they_land(TileOperands &T, const B
     X.s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
 }
 
-// The dense kernel's form of a tile, one accumulator less: the mins' MFMA adds onto the converted
-// integer sums instead of into registers of its own.  With d' = d / (-dmin):
+// The dense kernel's form of a tile's float step, one accumulator less: the mins' MFMA adds onto the
+// converted integer sums instead of into registers of its own.  With d' = d / (-dmin):
 //     d * S1 - dmin * S2 = (-dmin) * (d' * S1 + S2),
 // so the f16 MFMA takes d' * S1 as its C operand and the epilogue multiplies by -dmin (and the token's
 // scale).  A row whose dmin is zero keeps d and a factor of one, and zero mins.  (Not the same
@@ -300,115 +300,203 @@ __device__ __forceinline__ void fold_mins(BPlanes &B) {
     B.ndmin = z ? 1.0f : B.ndmin;
     if (z) B.m = v8h{0, 0, 0, 0, 0, 0, 0, 0};
 }
-template <class Between = NothingBetween>
-__device__ __forceinline__ v16f tile_mfmas_folded(TileOperands &T, const BPlanes &B, Between between = Between()) {
-    const v16i zi = {0};
-    asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(T.a0));
-    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
-    between(0, acc);
-    FRK_WAIT_LGKM(7, T.a1, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
-    between(1, acc);
-    FRK_WAIT_LGKM(6, T.a2, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
-    between(2, acc);
-    FRK_WAIT_LGKM(5, T.a3, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
-    between(3, acc);
-    FRK_WAIT_LGKM(4, T.a4, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
-    between(4, acc);
-    FRK_WAIT_LGKM(3, T.a5, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
-    between(5, acc);
-    FRK_WAIT_LGKM(2, T.a6, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
-    between(6, acc);
-    FRK_WAIT_LGKM(1, T.a7, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
-    between(7, acc);
-    acc = acc << 3;
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
-    between(8, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
-    between(9, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
-    between(10, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
-    between(11, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
-    between(12, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
-    between(13, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
-    between(14, acc);
-    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
-    FRK_WAIT_LGKM(0, T.bs, acc);
-    v16f c;
-#pragma unroll
-    for (int r = 0; r < 16; r++) c[r] = B.d * (float)acc[r];
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(T.bs, B.m, c, 0, 0, 0);
-}
-__device__ __forceinline__ void tile_epilogue_folded(const v16f &c, const TileScales &S, const BPlanes &B, v16f &acc) {
-    const v4f dav[4] = {S.da0, S.da1, S.da2, S.da3};
-#pragma unroll
-    for (int q = 0; q < 4; q++)
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int r = q * 4 + e;
-            acc[r] = fmaf(dav[q][e] * B.ndmin, c[r], acc[r]);
-        }
-}
-
-// A workgroup = RG*WT wavefronts = RG row groups of 32 weight rows x WT token groups of MT 32-token
-// tiles.  A wavefront keeps the current block of its 32 rows in registers as MFMA B operands and
-// runs its MT tiles against them, so a block of a row is unpacked once per MT tiles.  A SIMD holds
-// two wavefronts: while one issues a tile's MFMAs the other does its vector work (unpack,
-// epilogue), which is how the matrix cores and the vector ALU overlap here.
+// ---------------------------------------------------------------------------------------------
+// The dense kernel in its pipelined form.
 //
-// What bounds the tile shape: every block moves (32*RG*144 + 32*NT*292) bytes from L2 into LDS for
-// 2*32*RG*32*NT*256 operations, and a CU's address unit takes roughly 40 cycles per kilobyte of such
-// loads (whether they write LDS directly or go through registers), so more rows and tokens per
-// workgroup is better -- until the registers run out: 256 rows x 128 tokens (8 wavefronts, four
-// tiles each) fits two wavefronts per SIMD (256 registers per lane) without spills, and a spill is
-// fatal here because scratch reloads wait on the same counter as the prefetch.  What keeps the
-// registers down: the prefetch writes LDS directly, its addresses are recomputed from the lane
-// number at every use (made opaque, or the compiler keeps them all), the mins' term shares the
-// integer sums' accumulator (tile_mfmas_folded) and every tile's epilogue is pinned to its tile.
+// What bounds a SIMD here is its one issue port, not the matrix core alone: measured on this part, a
+// v_mfma_i32_32x32x32_i8 keeps the matrix core 32 clocks but costs the SIMD about 20 clocks in which no
+// vector instruction issues, and every vector instruction another 2.6 -- whichever wavefront they come
+// from.  About five vector instructions fit between two MFMAs for free; a tile (16 + 1 MFMAs) has ~80
+// of epilogue.  So the epilogue of tile t-1 is cut into sixteen pieces that ride in the gaps of tile
+// t's chain of MFMAs, the address arithmetic of the prefetch is scalar (global_load_lds with a scalar
+// base and lane offsets that are computed once), and what stays exposed is the unpacking of the
+// next block and the last tile's epilogue.
 //
-// LDS rings.  Activations, 2 stages:
-//     quants [NT][8 k-slices][1 KB] | bsums f16 [NT][1 KB] | scales f32 [NT*32],  NT = MT*WT tiles
-// weights, WS stages of [RG][32 rows][144 B] raw blocks; block kb+1 is unpacked at the end of
-// iteration kb, so with WS = 2 a stage is refilled two blocks ahead, with WS = 4 three.
-template <int RG, int WT, int MT, int WS>
-struct GemmLds {
-    static constexpr int NT = WT * MT;
+// A workgroup = 8 wavefronts = RG row groups of 32 weight rows x KS shares of the blocks; a wavefront
+// runs MT 32-token tiles against its rows' current block.  KS = 2 (small matrices: 128 rows x 64 tokens
+// per workgroup fill the chip where 256 x 128 would not) halves the blocks between two wavefronts whose
+// sums are added through LDS at the end, always the first half's plus the second half's.
+//
+// LDS: activations in a ring of 3 stages (requested two steps ahead), their scales in a ring of 4
+// (they are read by an epilogue that may run a step later), the raw weights in ONE slot per
+// wavefront: a block leaves its slot for registers at the end of the step before it is multiplied,
+// and the slot is refilled at once.  One barrier per step.
+template <int RG, int KS, int MT>
+struct PipeLds {
+    static constexpr int NW = RG * KS;
+    static constexpr int NT = KS * MT;  // tile slots of a stage
     static constexpr int OFF_BS = NT * 8192;
-    static constexpr int OFF_DA = NT * 9216;
-    static constexpr int A_STAGE = OFF_DA + ((NT + 1) / 2) * 256;
-    static constexpr int W_GROUP = 32 * Q4_K_BYTES;  // 4608
-    static constexpr int W_STAGE = RG * W_GROUP;
-    static constexpr size_t BYTES = (size_t)2 * A_STAGE + (size_t)WS * W_STAGE;
+    static constexpr int A_STAGE = NT * 9216;  // quants [NT][8 slices][1 KB] | sums f16 [NT][1 KB]
+    static constexpr int A_STAGES = 3;
+    static constexpr int OFF_DA = A_STAGES * A_STAGE;
+    static constexpr int DA_STAGE = NT * 128, DA_STAGES = 4;
+    static constexpr int OFF_W = OFF_DA + DA_STAGES * DA_STAGE;
+    static constexpr int W_SLOT = 32 * Q4_K_BYTES;
+    static constexpr size_t BYTES = (size_t)OFF_W + (size_t)NW * W_SLOT;
 };
 
-template <int RG, int WT, int MT, int WS>
-__global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g) {
-    using L = GemmLds<RG, WT, MT, WS>;
-    constexpr int NW = RG * WT, NT = L::NT, TM = 32 * NT, ROWS = 32 * RG;
-    constexpr int N_DA = (NT + 1) / 2;
-    static_assert(NW == 4 || NW == 8, "the k-slice to wavefront map assumes 4 or 8 wavefronts");
-    static_assert(WS == 2 || WS == 4, "weight ring of 2 or 4 stages");
-    static_assert(WT == 1 || WT == 2, "one or two token groups");
-    constexpr int WD = WS == 4 ? 3 : 2;  // weights are requested WD blocks ahead
-    // global_load_lds instructions per wavefront for one block of weights
-    constexpr int C_W = WT == 1 ? 5 : 3;
+// global_load_lds from a wavefront-uniform base (scalar registers) plus a 32-bit lane offset; the 64
+// lanes' pieces land at lds_uniform + 16 (or 4) * lane.  Counted by vmcnt.
+// (readfirstlane costs nothing on a value the compiler already keeps in scalar registers and makes the
+// operands scalar where its uniformity analysis gives up)
+__device__ __forceinline__ const void *scalar_pointer(const void *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma16(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
+                 : "memory");
+}
+__device__ __forceinline__ void dma4(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
+                 : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void ds_read16(v4i &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void ds_read16(v8h &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+template <int OFF>
+__device__ __forceinline__ void ds_read16(v4f &dst, uint32_t addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
+}
+// tile slot SLOT of a stage: its eight k-slices and its sums (nine reads, in this order)
+template <int SLOT>
+__device__ __forceinline__ void read_tile(TileOperands &T, uint32_t qa, uint32_t ba) {
+    ds_read16<SLOT * 8192 + 0>(T.a0, qa);
+    ds_read16<SLOT * 8192 + 1024>(T.a1, qa);
+    ds_read16<SLOT * 8192 + 2048>(T.a2, qa);
+    ds_read16<SLOT * 8192 + 3072>(T.a3, qa);
+    ds_read16<SLOT * 8192 + 4096>(T.a4, qa);
+    ds_read16<SLOT * 8192 + 5120>(T.a5, qa);
+    ds_read16<SLOT * 8192 + 6144>(T.a6, qa);
+    ds_read16<SLOT * 8192 + 7168>(T.a7, qa);
+    ds_read16<SLOT * 1024>(T.bs, ba);
+}
+// operand J (0..7) of tile slot SLOT
+template <int SLOT, int J>
+__device__ __forceinline__ void read_tile_operand(TileOperands &T, uint32_t qa) {
+    v4i &dst = J == 0 ? T.a0 : J == 1 ? T.a1 : J == 2 ? T.a2 : J == 3 ? T.a3 : J == 4 ? T.a4 : J == 5 ? T.a5 : J == 6 ? T.a6 : T.a7;
+    ds_read16<SLOT * 8192 + J * 1024>(dst, qa);
+}
+template <int SLOT>
+__device__ __forceinline__ void read_tile_sums(TileOperands &T, uint32_t ba) {
+    ds_read16<SLOT * 1024>(T.bs, ba);
+}
+template <int SLOT>
+__device__ __forceinline__ void read_tile_scales(TileScales &S, uint32_t sa) {
+    ds_read16<SLOT * 128 + 0>(S.da0, sa);
+    ds_read16<SLOT * 128 + 32>(S.da1, sa);
+    ds_read16<SLOT * 128 + 64>(S.da2, sa);
+    ds_read16<SLOT * 128 + 96>(S.da3, sa);
+}
+
+// The sixteen integer MFMAs of a tile.  Its operands were requested in the order a0..a7, sums, and then
+// EXTRA more LDS reads; each MFMA waits only for its own operand.  between(i) runs after MFMA i has been
+// issued; from MFMA 8 on operand a(i-8) has been read for the last time, and next(i-8) may request the
+// next tile's into its place.
+template <int N, class V>
+__device__ __forceinline__ void wait_lgkm(V &reg, v16i &acc) {
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(reg), "+v"(acc) : "n"(N));
+}
+template <int EXTRA, class Between, class Next>
+__device__ __forceinline__ v16i tile_chain(TileOperands &T, const BPlanes &B, Between between, Next next) {
+    const v16i zi = {0};
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(T.a0) : "n"(8 + EXTRA));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    between(0);
+    wait_lgkm<7 + EXTRA>(T.a1, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    between(1);
+    wait_lgkm<6 + EXTRA>(T.a2, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    between(2);
+    wait_lgkm<5 + EXTRA>(T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    between(3);
+    wait_lgkm<4 + EXTRA>(T.a4, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    between(4);
+    wait_lgkm<3 + EXTRA>(T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    between(5);
+    wait_lgkm<2 + EXTRA>(T.a6, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    between(6);
+    wait_lgkm<1 + EXTRA>(T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    between(7);
+    wait_lgkm<0>(T.bs, acc);  // (and the EXTRA reads behind the sums)
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    next(0);
+    between(8);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    next(1);
+    between(9);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    next(2);
+    between(10);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    next(3);
+    between(11);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    next(4);
+    between(12);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    next(5);
+    between(13);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    next(6);
+    between(14);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+    next(7);
+    between(15);
+    return acc;
+}
+
+// A finished tile's way into the float sums (the arithmetic fold_mins prepares), in sixteen pieces:
+//   pieces 0..7   c[r] = d' * float(S1[r]) for two results each,
+//   piece  7      then the mins' MFMA adds S2 onto c,
+//   pieces 8..15  sum[r] += (da[r] * -dmin) * c[r] for two results each.
+struct TileTail {
+    v16i s1;      // the integer sums
+    v16f c;       // d' * S1, then + S2
+    v8h bs;       // the tile's 16-wide activation sums
+    TileScales S; // the tile's activation scales
+};
+__device__ __forceinline__ void tail_piece(int i, TileTail &E, const BPlanes &B, v16f &sum) {
+    if (i < 8) {
+        E.c[2 * i] = B.d * (float)E.s1[2 * i];
+        E.c[2 * i + 1] = B.d * (float)E.s1[2 * i + 1];
+        if (i == 7) E.c = __builtin_amdgcn_mfma_f32_32x32x16_f16(E.bs, B.m, E.c, 0, 0, 0);
+    } else {
+        const v4f dav[4] = {E.S.da0, E.S.da1, E.S.da2, E.S.da3};
+#pragma unroll
+        for (int r = 2 * (i - 8); r < 2 * (i - 8) + 2; r++) sum[r] = fmaf(dav[r >> 2][r & 3] * B.ndmin, E.c[r], sum[r]);
+    }
+}
+
+template <int RG, int KS, int MT>
+__global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
+    using L = PipeLds<RG, KS, MT>;
+    constexpr int NW = L::NW, NT = L::NT, ROWS = 32 * RG, TM = 32 * MT;
+    static_assert(NW == 8 && NT == 4, "eight wavefronts share the four tile slots of a stage");
     extern __shared__ uint4 smem_gemm[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
-    uint8_t *lds_w = lds + 2 * L::A_STAGE;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t lds0 = lds_address(lds);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lg = lane >> 5;
-    const int rgrp = wave % RG, tgrp = wave / RG;
+    const int rg = wave % RG, ks = wave / RG;
 
     // workgroups that share weight rows (different token tiles) sit on one XCD (block id mod 8)
     const int bid = blockIdx.x;
@@ -417,183 +505,184 @@ __global__ __launch_bounds__(64 * RG * WT) void gemm_q4_k_mfma_kernel(GemmArgs g
     const int row_tile = grp * 8 + (in_grp & 7);
     if (row_tile >= g.row_tiles) return;  // uniform per workgroup
     const int tok0 = (in_grp >> 3) * TM;
-    const int row0 = row_tile * ROWS + rgrp * 32;  // this wavefront's first weight row
-    const int row = row0 + li;
-    const int nb = g.nb;  // blocks of a row (strides); this workgroup multiplies blocks kb0 .. kb1 - 1
+    const int nb = g.nb;
+    // this workgroup multiplies blocks kb0 .. kb1 - 1, its KS shares `steps` consecutive ones each (a
+    // share that runs out of blocks idles through its last steps)
     const int kb0 = nb * (int)blockIdx.y / g.k_split, kb1 = nb * ((int)blockIdx.y + 1) / g.k_split;
+    const int steps = (kb1 - kb0 + KS - 1) / KS;
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
+    auto block_of = [&](int share, int i) { return min(kb0 + share * steps + i, kb1 - 1); };  // uniform
+    auto tile_of = [&](int slot) { return min(tile0 + slot % MT, last_tile); };               // uniform
 
-    // ---- what this lane fetches ----
-    // Only 32-bit offsets of the first piece are kept in registers; everything else is uniform or is
-    // recomputed from them where it is used.
-    // activations: the tiled form is the LDS image, so chunk (tile t, slice ks) is 1 KB of consecutive
-    // memory and lane j brings its bytes 16*j..; same for the sums.  Tiles past the last one repeat it.
-    // (offsets from the quants: the three arrays of the tiled form are carved from one allocation,
-    // quants first)
+    // ---- what this wavefront fetches per step (all bases scalar, all lane offsets fixed) ----
+    // quants: the four consecutive k-slices (4 KB) (wave & 1) * 4 .. of tile slot wave / 2
     const uint8_t *Qb = reinterpret_cast<const uint8_t *>(g.a.q);
-    const uint32_t bs_base = (uint32_t)(reinterpret_cast<const uint8_t *>(g.a.bs) - Qb);
-    const uint32_t d_base = (uint32_t)(reinterpret_cast<const uint8_t *>(g.a.d) - Qb);
-    auto tile_rec = [&](int t) { return (uint32_t)min(tile0 + t, last_tile) * (uint32_t)nb; };  // uniform
-    // with fewer chunks than wavefronts some fetch a chunk twice, into the same place
-    const int bs_tile = wave % NT, da_chunk = wave % N_DA;
-    // weights: a row group's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of chunk c, so that
-    // LDS holds the rows back to back (144 bytes each) and consecutive lanes read consecutive memory:
-    // chunk c is 7c rows further down and c pieces to the right of chunk 0, modulo the nine of a row.
-    // Offsets past the matrix are pulled back to its last 16 bytes (such rows are never stored).
-    // With WT = 2 the two wavefronts of a row group split the five chunks (3 + 2, one fetched twice).
-    const uint8_t *Wb = g.W;
+    const uint8_t *Sb = reinterpret_cast<const uint8_t *>(g.a.bs);
+    const uint8_t *Db = reinterpret_cast<const uint8_t *>(g.a.d);
+    const int slot_q = wave >> 1, slice_q = (wave & 1) * 4;
+    const int slot_s = wave & 3;                // sums of one tile slot (the second four wavefronts repeat the first)
+    const int slot_d = (wave & 1) * 2;          // scales of two tile slots, one per lane half
+    const uint32_t lane16 = (uint32_t)lane * 16;
+    const uint32_t lane_d = (uint32_t)(lane & 31) * 4 +
+                            (lane >= 32 ? (uint32_t)(tile_of(slot_d + 1) - tile_of(slot_d)) * (uint32_t)nb * 128u : 0u);
+    // weights: this wavefront's 32 rows x 9 sixteen-byte pieces, piece p = 64 * c + lane of chunk c, so
+    // that LDS holds the rows back to back (144 bytes each).  Rows past the matrix read its last row.
     const uint32_t stride = (uint32_t)g.row_stride;
-    const uint32_t w_last = (uint32_t)g.rows * stride - 16;
-    const int wc0 = (WT == 1) ? 0 : (tgrp == 0 ? 0 : 3);
-    auto chunk_of = [&](int i) { return min(wc0 + i, 4) - ((WT == 2 && tgrp == 1 && i == 2) ? 1 : 0); };  // tgrp 1: 3, 4, 3
-    auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
-        int l = lane;
-        asm volatile("" : "+v"(l));
-        return l;
-    };
+    const int row_base = min(row_tile * ROWS + rg * 32, g.rows - 1);
+    uint32_t w_off[5];
+#pragma unroll
+    for (int c = 0; c < 5; c++) {
+        const int p = 64 * c + lane;
+        const int r = min(p / 9, g.rows - 1 - row_base);
+        w_off[c] = (uint32_t)r * stride + (uint32_t)(p % 9) * 16;
+    }
+    const uint8_t *Wrow = g.W + (size_t)row_base * stride;
+    const uint32_t lds_w = lds0 + L::OFF_W + wave * L::W_SLOT;
 
-    // the prefetch of one block, as N_A + 2 + C_W separate loads so that they can be issued one by one
-    constexpr int N_A = NT * (8 / NW), N_DMA = N_A + 2 + C_W;
-    auto act_part = [&](int j, int kb) {  // j = 0 .. N_A + 1
-        asm volatile("" : "+s"(kb));  // (seen as the loop counter, every address becomes a pointer of its own)
-        uint8_t *st = lds + (kb & 1) * L::A_STAGE;
-        const uint32_t l = (uint32_t)opaque_lane();
-        if (j < N_A) {
-            const int t = j / (8 / NW), i = j % (8 / NW);
-            const int ks = ((wave + t) % NW) + NW * i;
-            load_to_lds16(Qb + ((tile_rec(t) + kb) * 8192 + ks * 1024 + l * 16), st + (t * 8 + ks) * 1024);
-        } else if (j == N_A) {
-            load_to_lds16(Qb + (bs_base + (tile_rec(bs_tile) + kb) * 1024 + l * 16), st + L::OFF_BS + bs_tile * 1024);
+    auto fetch_acts_part = [&](int j, int i) {  // j = 0..5: request part j of step i's activations
+        const uint32_t st = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE;
+        if (j < 4) {
+            const size_t rec = (size_t)tile_of(slot_q) * nb + block_of(slot_q / MT, i);
+            dma16(st + slot_q * 8192 + (slice_q + j) * 1024, Qb + rec * 8192 + (size_t)(slice_q + j) * 1024, lane16);
+        } else if (j == 4) {
+            const size_t rec = (size_t)tile_of(slot_s) * nb + block_of(slot_s / MT, i);
+            dma16(st + L::OFF_BS + slot_s * 1024, Sb + rec * 1024, lane16);
         } else {
-            load_to_lds4(Qb + (d_base + (tile_rec(2 * da_chunk + (l >> 5)) + kb) * 128 + (l & 31) * 4),
-                         st + L::OFF_DA + da_chunk * 256);
+            const size_t rec = (size_t)tile_of(slot_d) * nb + block_of(slot_d / MT, i);
+            dma4(lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + slot_d * 128, Db + rec * 128, lane_d);
         }
     };
-    auto weight_part = [&](int i, int kb) {  // i = 0 .. C_W - 1
-        asm volatile("" : "+s"(kb));
-        uint8_t *st = lds_w + (kb % WS) * L::W_STAGE + rgrp * L::W_GROUP;
-        const uint32_t l = (uint32_t)opaque_lane();
-        const uint32_t pc0 = l % 9;
-        const uint32_t off0 = ((uint32_t)(row_tile * ROWS + rgrp * 32) + l / 9) * stride + pc0 * 16 + (uint32_t)kb * Q4_K_BYTES;
-        const int c = chunk_of(i);
-        const uint32_t v = pc0 + c, wrap = v >= 9 ? 1u : 0u;  // c <= 4: at most one wrap
-        const uint32_t off = off0 + (uint32_t)(7 * c) * stride + wrap * (stride - 144) + c * 16;
-        // chunk 4 is half a chunk: 32 pieces
-        if (c < 4 || l < 32) load_to_lds16(Wb + min(off, w_last), st + c * 1024);
-    };
-    auto issue_acts = [&](int kb) {
+    auto fetch_weights = [&](int i) {  // five requests
+        const uint8_t *src = Wrow + (size_t)block_of(ks, i) * Q4_K_BYTES;
 #pragma unroll
-        for (int j = 0; j < N_A + 2; j++) act_part(j, kb);
-    };
-    auto issue_weights = [&](int kb) {
-#pragma unroll
-        for (int i = 0; i < C_W; i++) weight_part(i, kb);
+        for (int c = 0; c < 4; c++) dma16(lds_w + c * 1024, src, w_off[c]);
+        if (lane < 32) dma16(lds_w + 4096, src, w_off[4]);
     };
 
-    const uint32_t lds_a = lds_address(lds);
-    const uint32_t lds_wv = lds_address(lds_w) + rgrp * L::W_GROUP + li * Q4_K_BYTES;
-
-    v16f accF[MT];
+    v16f sum[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) accF[mt] = v16f{0.0f};
-
+    for (int mt = 0; mt < MT; mt++) sum[mt] = v16f{0.0f};
     BPlanes B;
     RawBlock R;
-    v16i accI0 = {0};  // (an argument the prefetch does not use)
-    const int pf_tile = __builtin_amdgcn_readfirstlane(wave >= NW / 2 ? MT / 2 : 0);
 
-    // prologue: weights of blocks 0..WD-1, activations of block 0; the last weights may stay in flight
-    issue_weights(kb0);
-    issue_acts(kb0);
+    // prologue: activations of steps 0 and 1, weights of step 0; then the weights of step 1
 #pragma unroll
-    for (int i = 1; i < WD; i++)
-        if (kb0 + i < kb1) issue_weights(kb0 + i);
-    if (WS == 4 && kb1 - kb0 > 2) wait_vm<C_W>();
-    else wait_vm<0>();
+    for (int j = 0; j < 6; j++) fetch_acts_part(j, 0);
+    fetch_weights(0);
+    if (steps > 1) {
+#pragma unroll
+        for (int j = 0; j < 6; j++) fetch_acts_part(j, 1);
+    }
+    wait_vm<0>();
     lds_barrier();
     {
-        const uint32_t first = lds_wv + (kb0 % WS) * L::W_STAGE;
-        read_raw(R, first, first + 16 * lg);
+        const uint32_t wa = lds_w + li * Q4_K_BYTES;
+        read_raw(R, wa, wa + 16 * lg);
+        wait_raw<0>(R);
+        if (steps > 1) fetch_weights(1);
+        unpack_block(R, lg, B);
+        fold_mins(B);
     }
-    wait_raw<0>(R);
-    unpack_block(R, lg, B);
-    fold_mins(B);
 
-    for (int kb = kb0; kb < kb1; kb++) {
-        // The first tile's operands are requested before anything else: they travel from LDS while
-        // the prefetch below is issued.  In the same way every later tile's operands are requested
-        // before the epilogue of the tile before it.
-        const uint32_t st = lds_a + (kb & 1) * L::A_STAGE;
-        const uint32_t qa = st + lane * 16, ba = st + L::OFF_BS + lane * 16, sa = st + L::OFF_DA + lg * 16;
-        const uint32_t wa = lds_wv + ((kb + 1) % WS) * L::W_STAGE;
-        TileOperands T;
-        read_ops(T, qa + (tgrp * MT) * 8192, ba + (tgrp * MT) * 1024);
-        // The prefetch (the stages refilled were last read in iteration kb-1, which every wavefront
-        // has left).  A wavefront is stalled while its loads wait for the CU's one address unit, and
-        // a block's loads keep that unit busy for about as long as half the block's MFMAs take: so the
-        // two wavefronts of a SIMD (w and w + NW/2) issue theirs at different times, from inside the
-        // chain of MFMAs of their first and of their middle tile, one load per gap; while one is
-        // stalled the other has the matrix core.  With one tile per wavefront there is no such choice.
-        auto prefetch_part = [&](int j, v16i &) {
-            if (j < N_A + 2) {
-                if (kb + 1 < kb1) act_part(j, kb + 1);
-            } else if (j < N_DMA) {
-                if (kb + WD < kb1) weight_part(j - (N_A + 2), kb + WD);
-            }
-        };
-        if (MT == 1) {
+    for (int i = 0; i < steps; i++) {
+        const bool active = kb0 + ks * steps + i < kb1;  // uniform per wavefront
+        const uint32_t st = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + (uint32_t)(ks * MT) * 8192;
+        const uint32_t qa = st + lane16;
+        const uint32_t ba = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + L::OFF_BS + (uint32_t)(ks * MT) * 1024 + lane16;
+        const uint32_t sa = lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + (uint32_t)(ks * MT) * 128 + lg * 16;
+        const bool more_acts = i + 2 < steps;
+        if (active) {
+            TileOperands T, Tn;
+            TileTail E;
+            read_tile<0>(T, qa, ba);
+            // One tile after the other; the second half of a tile's chain requests the next tile's operands
+            // into the registers it has read for the last time, and carries the tail of the tile before.
+            auto run_tile = [&](auto mt_c) {
+                constexpr int mt = decltype(mt_c)::value;
+                auto between = [&](int j) {
+                    if (mt == 0) {
+                        if (j < 6 && more_acts) fetch_acts_part(j, i + 2);
+                    } else {
+                        tail_piece(j, E, B, sum[mt > 0 ? mt - 1 : 0]);
+                    }
+                };
+                auto next = [&](int j) {
+                    if (mt + 1 < MT) {
+                        constexpr int nx = mt + 1 < MT ? mt + 1 : mt;
+                        if (j == 0) read_tile_operand<nx, 0>(Tn, qa);
+                        if (j == 1) read_tile_operand<nx, 1>(Tn, qa);
+                        if (j == 2) read_tile_operand<nx, 2>(Tn, qa);
+                        if (j == 3) read_tile_operand<nx, 3>(Tn, qa);
+                        if (j == 4) read_tile_operand<nx, 4>(Tn, qa);
+                        if (j == 5) read_tile_operand<nx, 5>(Tn, qa);
+                        if (j == 6) read_tile_operand<nx, 6>(Tn, qa);
+                        if (j == 7) read_tile_operand<nx, 7>(Tn, qa);
+                    }
+                };
+                // (a tile after the first finds four more reads behind its sums: the scales of the tile before)
+                const v16i s1 = tile_chain<(mt > 0 ? 4 : 0)>(T, B, between, next);
+                E.s1 = s1;
+                E.bs = T.bs;
+                if (mt + 1 < MT) {
+                    constexpr int nx = mt + 1 < MT ? mt + 1 : mt;
+                    read_tile_sums<nx>(Tn, ba);
+                }
+                read_tile_scales<mt>(E.S, sa);
+                if (mt + 1 < MT) T = Tn;
+            };
+            run_tile(std::integral_constant<int, 0>());
+            if (MT > 1) run_tile(std::integral_constant<int, 1 < MT ? 1 : 0>());
+            if (MT > 2) run_tile(std::integral_constant<int, 2 < MT ? 2 : 0>());
+            if (MT > 3) run_tile(std::integral_constant<int, 3 < MT ? 3 : 0>());
+            // the last tile's tail is exposed
+            wait_scales<0>(E.S);
 #pragma unroll
-            for (int j = 0; j < N_DMA; j++) prefetch_part(j, accI0);
-        }
+            for (int j = 0; j < 16; j++) tail_piece(j, E, B, sum[MT - 1]);
+        } else if (more_acts) {
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            const int t = tgrp * MT + mt;
-            TileScales S;
-            v16f c;
-            if (MT > 1 && (mt == 0 || mt == MT / 2)) {
-                // (one chain for both cases, the choice made per load: two copies of the chain behind
-                // a branch would meet in register copies of the operands, which the compiler, blind
-                // to the hand-placed waits, is free to put in front of them)
-                c = tile_mfmas_folded(T, B, [&](int j, v16i &a) {
-                    if (mt == pf_tile) prefetch_part(j, a);
-                });
-            } else {
-                c = tile_mfmas_folded(T, B);
-            }
-            read_scales(S, sa + t * 128);
-            if (mt + 1 < MT) {
-                read_ops(T, qa + (t + 1) * 8192, ba + (t + 1) * 1024);
-                wait_scales<9>(S);
-            } else {
-                wait_scales<0>(S);
-            }
-            tile_epilogue_folded(c, S, B, accF[mt]);
-            // (the sums are next used in the following iteration, which lets the compiler sink the
-            // epilogues of all tiles to the end of this one, every tile's MFMA result alive until then)
-            asm volatile("" : "+v"(accF[mt]));
+            for (int j = 0; j < 6; j++) fetch_acts_part(j, i + 2);
         }
-        if (kb + 1 < kb1) {
-            // the next block's raw weights landed during iteration kb-1
+        if (i + 1 < steps) {
+            // step i+1's raw weights (requested a step ago) leave their slot, which is refilled at once;
+            // the activations of step i+2, younger than they, may stay in flight
+            if (more_acts) wait_vm<6>();
+            else wait_vm<0>();
+            const uint32_t wa = lds_w + li * Q4_K_BYTES;
             read_raw(R, wa, wa + 16 * lg);
             wait_raw<0>(R);
+            if (more_acts) fetch_weights(i + 2);
             unpack_block(R, lg, B);
             fold_mins(B);
-            // activations of block kb+1 and weights of block kb+2 must have landed; with four weight
-            // stages the weights requested above (younger than both) may stay in flight
-            if (WS == 4 && kb + WD < kb1) wait_vm<C_W>();
-            else wait_vm<0>();
         }
         lds_barrier();
     }
 
+    // two shares of the blocks: the second half's sums go through LDS and are added onto the first's
+    if (KS == 2) {
+        float *xch = reinterpret_cast<float *>(lds) + (size_t)rg * MT * 16 * 64;
+        if (ks == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) xch[(mt * 16 + r) * 64 + lane] = sum[mt][r];
+        }
+        __syncthreads();
+        if (ks == 1) return;
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) sum[mt][r] += xch[(mt * 16 + r) * 64 + lane];
+    }
     // store: a lane holds one weight row and 16 tokens per tile
+    const int row = row_tile * ROWS + rg * 32 + li;
     float *const dst = g.k_split > 1 ? g.partial + (size_t)blockIdx.y * g.M * g.rows : g.y;
+    const int rows_lim = g.rows;
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int tok = tok0 + (tgrp * MT + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < g.M) dst[(size_t)tok * g.rows + row] = accF[mt][r];
+            const int tok = tok0 + mt * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
+            if (row < rows_lim && tok < g.M) dst[(size_t)tok * g.rows + row] = sum[mt][r];
         }
 }
 
@@ -893,19 +982,19 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
-template <int RG, int WT, int MT, int WS>
-static int launch_variant(const GemmArgs &g, unsigned grid, hipStream_t s) {
-    constexpr size_t shmem = GemmLds<RG, WT, MT, WS>::BYTES;
+template <int RG, int KS, int MT>
+static int launch_pipe(const GemmArgs &g, unsigned grid, hipStream_t s) {
+    constexpr size_t shmem = PipeLds<RG, KS, MT>::BYTES;
     static_assert(shmem <= 160 * 1024, "LDS of a CU");
     static bool sized = false;  // a benign race: every thread sets the same attribute
-    if (shmem > 65536 && !sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_mfma_kernel<RG, WT, MT, WS>),
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_pipe_kernel<RG, KS, MT>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemm_q4_k_mfma_kernel<RG, WT, MT, WS>), dim3(grid, (unsigned)g.k_split), dim3(64 * RG * WT), shmem, s, g);
-    FRK_LAUNCH_CHECK("gemm_q4_k_mfma");
+    hipLaunchKernelGGL((gemm_q4_k_pipe_kernel<RG, KS, MT>), dim3(grid, (unsigned)g.k_split), dim3(512), shmem, s, g);
+    FRK_LAUNCH_CHECK("gemm_q4_k_pipe");
     if (g.k_split > 1) return launch_sum_parts(g.partial, g.k_split, (size_t)g.M * g.rows, g.y, s);
     return FRK_OK;
 }
@@ -947,21 +1036,19 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 }
 
 constexpr int Q4K_MAX_SPLIT = 4;
-// The workgroup tile of a batch: 256 rows x 128 or 64 tokens when that still gives (about) every CU a
-// workgroup, else 128 rows x 64 or 32 tokens -- and with those small tiles, when the grid fills few of
-// the CUs, a row's blocks split between 2 or 4 workgroups (no finer than four blocks each) whose sums
-// are added in order afterwards.
+// The workgroup tile of a batch: 256 rows x 128 tokens when that gives (about) every CU a workgroup,
+// else 128 rows x 64 tokens with each row's blocks shared between two wavefronts -- and with those,
+// when the grid still fills few of the CUs, a row's blocks split between 2 or 4 workgroups (no finer
+// than four blocks each) whose sums are added in order afterwards.
 struct Q4KPlan {
     int rows_wg, tok_wg, k_split;
 };
 static Q4KPlan q4_k_plan(size_t rows, size_t M, size_t nb) {
     if (M > 64 && ((rows + 255) / 256) * ((M + 127) / 128) >= 200) return {256, 128, 1};
-    if (M > 64 && ((rows + 255) / 256) * ((M + 63) / 64) >= 256) return {256, 64, 1};
-    const int tm = M > 32 ? 64 : 32;
-    const size_t grid = (((rows + 127) / 128 + 7) / 8 * 8) * ((M + (size_t)tm - 1) / (size_t)tm);
+    const size_t grid = (((rows + 127) / 128 + 7) / 8 * 8) * ((M + 63) / 64);
     int ks = 1;
     while (ks < Q4K_MAX_SPLIT && grid * (size_t)ks * 2 <= 256 && nb / (size_t)(ks * 2) >= 4) ks *= 2;
-    return {128, tm, ks};
+    return {128, 64, ks};
 }
 // the tiled activations, then room for the parts' sums where the blocks are split
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
@@ -970,10 +1057,10 @@ size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
 }
 
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
-    // the kernel addresses the weights and the tiled activations with 32-bit byte offsets
-    if ((uint64_t)w->rows * w->layout.row_stride >= (1ull << 32) || (uint64_t)q8k_tiled_bytes(M, w->cols) >= (1ull << 32))
-        return set_error(FRK_ERR_SHAPE, "gemm_q4_k: %zu x %zu weights with %zu activation rows exceed 4 GiB per operand", w->rows,
-                         w->cols, M);
+    // the kernel addresses the tiled activations with 32-bit lane offsets and a row group's weights likewise
+    if ((uint64_t)w->layout.row_stride * 64 >= (1ull << 32) || (uint64_t)q8k_tiled_bytes(M, w->cols) >= (1ull << 40))
+        return set_error(FRK_ERR_SHAPE, "gemm_q4_k: rows of %zu bytes or %zu activation rows are beyond the kernel's offsets",
+                         w->layout.row_stride, M);
     GemmArgs g;
     g.a = q8k_tiled_carve(ws, M, w->cols);
     int rc = launch_quantize_q8_k_tiled(x, M, w->cols, g.a, s);
@@ -984,16 +1071,13 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.nb = (int)(w->cols / QK_K);
     g.M = (int)M;
     g.y = y;
-    g.k_split = 1;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
     const Q4KPlan p = q4_k_plan(w->rows, M, (size_t)g.nb);
     g.row_tiles = (int)((w->rows + p.rows_wg - 1) / p.rows_wg);
     g.tok_tiles = (int)((M + p.tok_wg - 1) / p.tok_wg);
     g.k_split = p.k_split;
     const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
-    if (p.rows_wg == 256) return p.tok_wg == 128 ? launch_variant<8, 1, 4, 2>(g, grid, s) : launch_variant<8, 1, 2, 2>(g, grid, s);
-    if (p.tok_wg == 64) return launch_variant<4, 2, 1, 4>(g, grid, s);
-    return launch_variant<4, 1, 1, 2>(g, grid, s);
+    return p.rows_wg == 256 ? launch_pipe<8, 1, 4>(g, grid, s) : launch_pipe<4, 2, 2>(g, grid, s);
 }
 
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,

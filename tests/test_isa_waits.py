@@ -20,7 +20,7 @@ def _assembly(tmp_path, name):
 def test_no_use_of_lds_reads_before_their_waits(tmp_path):
     asm = _assembly(tmp_path, "frk_gemm.hip")
     names = isa_wait_lint.kernels(asm)
-    assert sum("gemm_q4_k" in k for k in names) >= 5, names  # the dense variants and the streaming kernel
+    assert sum("gemm_q4_k" in k for k in names) >= 3, names  # the two dense forms and the streaming kernel
     for k in names:
         assert isa_wait_lint.violations(asm, k) == [], k
     asm = _assembly(tmp_path, "frk_gemm_q6.hip")
