@@ -573,6 +573,14 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < 6; j++) fetch_acts_part(j, 1);
     }
+    // where step i's first tile slot of this wavefront's share sits in LDS: quants and sums (lane offsets in)
+    auto quants_of = [&](int i) { return lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + (uint32_t)(ks * MT) * 8192 + lane16; };
+    auto sums_of = [&](int i) {
+        return lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + L::OFF_BS + (uint32_t)(ks * MT) * 1024 + lane16;
+    };
+    auto is_active = [&](int i) { return kb0 + ks * steps + i < kb1; };  // uniform per wavefront
+    TileOperands T;  // the first tile's operands of the step about to run: requested behind the barrier, so that
+                     // they travel while the block is unpacked
     wait_vm<0>();
     lds_barrier();
     {
@@ -580,21 +588,19 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
         read_raw(R, wa, wa + 16 * lg);
         wait_raw<0>(R);
         if (steps > 1) fetch_weights(1);
+        if (is_active(0)) read_tile<0>(T, quants_of(0), sums_of(0));
         unpack_block(R, lg, B);
         fold_mins(B);
     }
 
     for (int i = 0; i < steps; i++) {
-        const bool active = kb0 + ks * steps + i < kb1;  // uniform per wavefront
-        const uint32_t st = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + (uint32_t)(ks * MT) * 8192;
-        const uint32_t qa = st + lane16;
-        const uint32_t ba = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + L::OFF_BS + (uint32_t)(ks * MT) * 1024 + lane16;
+        const bool active = is_active(i);
+        const uint32_t qa = quants_of(i), ba = sums_of(i);
         const uint32_t sa = lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + (uint32_t)(ks * MT) * 128 + lg * 16;
         const bool more_acts = i + 2 < steps;
         if (active) {
-            TileOperands T, Tn;
+            TileOperands Tn;
             TileTail E;
-            read_tile<0>(T, qa, ba);
             // One tile after the other; the second half of a tile's chain requests the next tile's operands
             // into the registers it has read for the last time, and carries the tail of the tile before.
             auto run_tile = [&](auto mt_c) {
@@ -651,10 +657,13 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
             read_raw(R, wa, wa + 16 * lg);
             wait_raw<0>(R);
             if (more_acts) fetch_weights(i + 2);
+            lds_barrier();
+            if (is_active(i + 1)) read_tile<0>(T, quants_of(i + 1), sums_of(i + 1));
             unpack_block(R, lg, B);
             fold_mins(B);
+        } else {
+            lds_barrier();
         }
-        lds_barrier();
     }
 
     // two shares of the blocks: the second half's sums go through LDS and are added onto the first's
