@@ -28,7 +28,7 @@ EXPORTS = [
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
     "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
-    "frk_hip_gemm_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
+    "frk_hip_gemm_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
@@ -88,6 +88,7 @@ def lib():
             "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
             "frk_hip_gemm_noalloc_dev": (i, [vp, vp, sz, vp, vp]),
+            "frk_hip_gemm_pair_dev": (i, [vp, vp, vp, sz, vp, vp, vp]),
             "frk_hip_route_top_k_softmax_dev": (i, [vp, sz, sz, sz, i, vp, vp, vp]),
             "frk_hip_moe_ffn_dev": (i, [vp, vp, vp, sz, vp, sz, vp, vp, sz, vp, vp]),
             "frk_hip_moe_intermediates_dev": (i, [sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
@@ -241,6 +242,17 @@ def _get_rows_host(self, ids):
 
 Weights.get_rows = _get_rows_dev
 Weights.get_rows_host = _get_rows_host
+
+
+def gemm_pair(w0, w1, x, outs=None):
+    """frk_hip_gemm_pair_dev: (x W0^T, x W1^T) over one quantization of the batch x[batch][cols]."""
+    import torch
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.shape[-1] == w0.cols == w1.cols
+    batch = x.numel() // w0.cols
+    y0, y1 = outs if outs is not None else (torch.empty((batch, w.rows), dtype=torch.float32, device=x.device) for w in (w0, w1))
+    check(lib().frk_hip_gemm_pair_dev(w0.handle, w1.handle, C.c_void_p(x.data_ptr()), batch, C.c_void_p(y0.data_ptr()),
+                                      C.c_void_p(y1.data_ptr()), _stream()))
+    return y0, y1
 
 
 def quantize_q8_k(x):

@@ -56,6 +56,27 @@ __device__ __forceinline__ void load_to_lds4(const void *src, void *lds_chunk) {
 #endif
 }
 
+// global_load_lds from a wavefront-uniform base (scalar registers) plus a 32-bit lane offset; the 64
+// lanes' pieces land at lds_uniform + 16 (or 4) * lane.  Counted by vmcnt.
+// (readfirstlane costs nothing on a value the compiler already keeps in scalar registers and makes the
+// operands scalar where its uniformity analysis gives up)
+__device__ __forceinline__ const void *scalar_pointer(const void *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ void dma16(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
+                 : "memory");
+}
+__device__ __forceinline__ void dma4(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
+                 : "memory");
+}
 // the 32-bit LDS address of a pointer into shared memory, for LDS instructions written as inline assembly
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -65,18 +86,28 @@ __device__ __forceinline__ uint32_t lds_address(const void *p) {
 #endif
 }
 
+// a 32-bit LDS store the compiler does not see (its LDS address from lds_address)
+__device__ __forceinline__ void lds_store32(uint32_t addr, uint32_t value) {
+    asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(value) : "memory");
+}
+
+typedef uint32_t lds_u4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_store128(uint32_t addr, lds_u4 value) {
+    asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"(value) : "memory");
+}
+
 constexpr int DPP_QUAD_XOR1 = 0xB1;     // quad_perm [1,0,3,2]
 constexpr int DPP_QUAD_XOR2 = 0x4E;     // quad_perm [2,3,0,1]
 constexpr int DPP_HALF_MIRROR = 0x141;  // lane i <- lane 7-i of its group of 8
 constexpr int DPP_ROW_MIRROR = 0x140;   // lane i <- lane 15-i of its row of 16
 
-// Sum over the LPR lanes (16, 32 or 64) that share a row; every lane ends with the total.
+// Sum over the LPR lanes (8, 16, 32 or 64) that share a row; every lane ends with the total.
 template <int LPR>
 __device__ __forceinline__ float part_sum(float v) {
     v += dpp_f<DPP_QUAD_XOR1>(v);
     v += dpp_f<DPP_QUAD_XOR2>(v);
     v += dpp_f<DPP_HALF_MIRROR>(v);
-    v += dpp_f<DPP_ROW_MIRROR>(v);
+    if (LPR >= 16) v += dpp_f<DPP_ROW_MIRROR>(v);
     if (LPR >= 32) v += __shfl_xor(v, 16);
     if (LPR >= 64) v += __shfl_xor(v, 32);
     return v;

@@ -335,27 +335,6 @@ struct PipeLds {
     static constexpr size_t BYTES = (size_t)OFF_W + (size_t)NW * W_SLOT;
 };
 
-// global_load_lds from a wavefront-uniform base (scalar registers) plus a 32-bit lane offset; the 64
-// lanes' pieces land at lds_uniform + 16 (or 4) * lane.  Counted by vmcnt.
-// (readfirstlane costs nothing on a value the compiler already keeps in scalar registers and makes the
-// operands scalar where its uniformity analysis gives up)
-__device__ __forceinline__ const void *scalar_pointer(const void *p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const void *>(((uint64_t)hi << 32) | lo);
-}
-__device__ __forceinline__ void dma16(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
-                 : "memory");
-}
-__device__ __forceinline__ void dma4(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
-                 : "memory");
-}
 template <int OFF>
 __device__ __forceinline__ void ds_read16(v4i &dst, uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(OFF));
@@ -609,6 +588,10 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
                     if (mt == 0) {
                         if (j < 6 && more_acts) fetch_acts_part(j, i + 2);
                     } else {
+                        // the scales of the tile before were the last reads requested ahead of this chain:
+                        // they have landed once the chain has waited for everything, in front of MFMA 8, and
+                        // only from here on may the compiler touch them
+                        if (j == 8) wait_scales<0>(E.S);
                         tail_piece(j, E, B, sum[mt > 0 ? mt - 1 : 0]);
                     }
                 };
@@ -1065,28 +1048,33 @@ size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
     return round_up(q8k_tiled_bytes(M, cols), 256) + (p.k_split > 1 ? (size_t)p.k_split * M * rows * sizeof(float) : 0);
 }
 
-int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
-    // the kernel addresses the tiled activations with 32-bit lane offsets and a row group's weights likewise
-    if ((uint64_t)w->layout.row_stride * 64 >= (1ull << 32) || (uint64_t)q8k_tiled_bytes(M, w->cols) >= (1ull << 40))
-        return set_error(FRK_ERR_SHAPE, "gemm_q4_k: rows of %zu bytes or %zu activation rows are beyond the kernel's offsets",
-                         w->layout.row_stride, M);
+// the GEMM proper, over activations already in the tiled form (`partial`: room for the parts' sums)
+int launch_gemm_q4_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *y, float *partial, hipStream_t s) {
+    // the kernel addresses a row group's weights with 32-bit lane offsets
+    if ((uint64_t)w->layout.row_stride * 64 >= (1ull << 32))
+        return set_error(FRK_ERR_SHAPE, "gemm_q4_k: rows of %zu bytes are beyond the kernel's offsets", w->layout.row_stride);
     GemmArgs g;
-    g.a = q8k_tiled_carve(ws, M, w->cols);
-    int rc = launch_quantize_q8_k_tiled(x, M, w->cols, g.a, s);
-    if (rc) return rc;
+    g.a = acts;
     g.W = w->dev;
     g.row_stride = w->layout.row_stride;
     g.rows = (int)w->rows;
     g.nb = (int)(w->cols / QK_K);
     g.M = (int)M;
     g.y = y;
-    g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
+    g.partial = partial;
     const Q4KPlan p = q4_k_plan(w->rows, M, (size_t)g.nb);
     g.row_tiles = (int)((w->rows + p.rows_wg - 1) / p.rows_wg);
     g.tok_tiles = (int)((M + p.tok_wg - 1) / p.tok_wg);
     g.k_split = p.k_split;
     const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
     return p.rows_wg == 256 ? launch_pipe<8, 1, 4>(g, grid, s) : launch_pipe<4, 2, 2>(g, grid, s);
+}
+
+int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
+    const Q8KTiled acts = q8k_tiled_carve(ws, M, w->cols);
+    int rc = launch_quantize_q8_k_tiled(x, M, w->cols, acts, s);
+    if (rc) return rc;
+    return launch_gemm_q4_k_acts(w, acts, M, y, reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256)), s);
 }
 
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,

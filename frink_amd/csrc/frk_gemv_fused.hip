@@ -321,6 +321,173 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
     }
 }
 
+// ------------------------------------------------------------------ whole cache lines
+// The same product for rows whose block count divides 64 (row lengths 2048 .. 16384 in powers of two),
+// read the way a plain copy reads memory.  The kernel above gives every lane its own half block, so
+// one load instruction touches some three dozen cache lines and the five loads of a block revisit
+// them: its 33 MB cost the CU's L1 six times the line look-ups of a linear read.  Here a wavefront
+// owns 64 consecutive blocks (9216 contiguous bytes = 64/NB whole rows, rows being stored back to
+// back) and moves them into LDS with nine global_load_lds of 1 KB -- eight full lines per
+// instruction, nothing staged in registers.  From there lane l reads block l of the span (nine
+// 16-byte reads 144 bytes apart: conflict-free) and multiplies the whole block: dot_q4_k_q8's
+// integers and its per-block float expression (crates/frink-quant/src/lib.rs:822-869), the blocks
+// of a row then added by its NB lanes with DPP.  The activation's blocks sit 272 bytes apart in LDS,
+// so that the lanes of a wavefront, which read NB different blocks at once, hit different banks.
+constexpr int LINES_ACT_STRIDE = QK_K + 16;
+template <int NB, int MODE, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8_t *__restrict__ W, int rows,
+                                                                    const float *__restrict__ x,
+                                                                    const int8_t *__restrict__ aq,
+                                                                    const float *__restrict__ ad,
+                                                                    const int16_t *__restrict__ absums,
+                                                                    float *__restrict__ y) {
+    constexpr int RPS = 64 / NB;  // rows of a wavefront's span
+    static_assert(64 % NB == 0 && NB >= 8, "a span of 64 blocks is a whole number of rows of at least 8 blocks");
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    int8_t *sq = reinterpret_cast<int8_t *>(lds);                          // NB blocks of quants, 272 bytes apart
+    int *sbs = reinterpret_cast<int *>(lds + NB * LINES_ACT_STRIDE);       // NB x 8 sums over 32
+    float *sd = reinterpret_cast<float *>(lds + NB * LINES_ACT_STRIDE + NB * 32);
+    uint8_t *sw = lds + NB * LINES_ACT_STRIDE + NB * 32 + NB * 4;          // WAVES spans of 9216 bytes (16-byte aligned)
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const size_t span = (size_t)blockIdx.x * WAVES + wave;
+    const size_t bytes = (size_t)rows * NB * Q4_K_BYTES;
+    const bool has_rows = span * 9216 < bytes;  // (a wavefront past the matrix still quantizes its share)
+
+    // ---- the activation's loads first (a wavefront's loads return in order), then the span ----
+    typedef float xv_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t uq_t __attribute__((ext_vector_type(4)));
+    xv_t xv[(NB + WAVES - 1) / WAVES];
+    uq_t qv = {0u, 0u, 0u, 0u}, qv2 = {0u, 0u, 0u, 0u};
+    uint32_t bv = 0;
+    float dv = 0.0f;
+    // (All of this kernel's global loads are issued from assembly and waited for by hand: the compiler
+    // waits for every load in flight, the span's included, before it touches a register an older load
+    // fills when loads that write LDS are among the younger ones.)
+    if (MODE == MODE_FUSED) {
+#pragma unroll
+        for (int i = 0; i < (NB + WAVES - 1) / WAVES; i++) {
+            const int b = min(wave + i * WAVES, NB - 1);
+            const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K) + lane;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xv[i]) : "v"(src) : "memory");
+        }
+    } else {
+        // quants: NB*16 words over 64*WAVES threads (NB <= 64, WAVES = 8: at most two each); sums and scales.
+        // Every lane loads (a clamped index where it has no word of its own) and the stores are masked.
+        const int t = threadIdx.x;
+        const uq_t *q_src = reinterpret_cast<const uq_t *>(aq);
+        const uq_t *s0 = q_src + min(t, NB * 16 - 1), *s1 = q_src + min(t + 64 * WAVES, NB * 16 - 1);
+        const uint32_t *s2 = reinterpret_cast<const uint32_t *>(absums) + min(t, NB * 8 - 1);
+        const float *s3 = ad + min(t, NB - 1);
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv) : "v"(s0) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv2) : "v"(s1) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(bv) : "v"(s2) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(dv) : "v"(s3) : "memory");
+    }
+    // (a wavefront past the matrix fetches the last span and stores nothing)
+    {
+        const size_t span_c = min(span, (bytes - 1) / 9216);
+        const uint8_t *src = W + span_c * 9216;
+        const uint32_t left = (uint32_t)min((size_t)9216, bytes - span_c * 9216);  // (the last span may be short)
+        const uint32_t slot = lds_address(sw) + (uint32_t)wave * 9216;
+#pragma unroll
+        for (int c = 0; c < 9; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+    }
+
+    // ---- the activation into LDS ----
+    if (MODE == MODE_FUSED) {
+        // the activation's loads are older than the span's nine
+        // (one wait that names them all, so that the blocks' quantizations can be interleaved)
+        constexpr int XB = (NB + WAVES - 1) / WAVES;
+        if (XB == 1) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]));
+        else if (XB == 2) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]));
+        else if (XB == 4)
+            asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]));
+        else
+            asm volatile("s_waitcnt vmcnt(9)"
+                         : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
+                           "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0]), "+v"(xv[XB > 7 ? 7 : 0]));
+#pragma unroll
+        for (int i = 0; i < XB; i++) {
+            const int b = wave + i * WAVES;
+            float d;
+            int bs;
+            const uint32_t packed = quantize_q8_k_lane(make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w), d, bs);
+            // a lane's 16-wide sum is in all four lanes of its quad: pairs of them make the 32-wide sums
+            const int bs32 = bs + __shfl_xor(bs, 4);
+            if (b < NB) {  // uniform across the wavefront
+                // (stored from assembly: a store the compiler sees makes it wait for the span's loads
+                // first, which write LDS too -- and the quantization would no longer run in their shadow)
+                lds_store32(lds_address(sq + b * LINES_ACT_STRIDE) + lane * 4, packed);
+                if ((lane & 7) == 0) lds_store32(lds_address(sbs + b * 8) + (lane >> 3) * 4, (uint32_t)bs32);
+                if (lane == 0) lds_store32(lds_address(sd + b), __float_as_uint(d));
+            }
+        }
+    } else {
+        asm volatile("s_waitcnt vmcnt(9)" : "+v"(qv), "+v"(qv2), "+v"(bv), "+v"(dv));  // (older than the span's nine)
+        auto put = [&](int t, uq_t v) {  // word t of the quants: block t / 16, word t % 16 of it
+            if (t < NB * 16) lds_store128(lds_address(sq + (t >> 4) * LINES_ACT_STRIDE + (t & 15) * 16), v);
+        };
+        put(threadIdx.x, qv);
+        if (NB * 16 > 64 * WAVES) put(threadIdx.x + 64 * WAVES, qv2);
+        if ((int)threadIdx.x < NB * 8)
+            lds_store32(lds_address(sbs + threadIdx.x), (uint32_t)((int)(int16_t)(bv & 0xffff) + (int)(int16_t)(bv >> 16)));
+        if ((int)threadIdx.x < NB) lds_store32(lds_address(sd + threadIdx.x), __float_as_uint(dv));
+    }
+    // Only the activation is shared: the barrier comes before the wait for the span, so that a wavefront
+    // starts multiplying when ITS blocks have landed, whatever the others' have done.
+    lds_barrier();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the span has landed (in this wavefront's own slot)
+    if (!has_rows) return;
+
+    // ---- lane l multiplies block l of the span ----
+    const int b = lane % NB;
+    const uint4 *blk = reinterpret_cast<const uint4 *>(sw + wave * 9216 + lane * Q4_K_BYTES);
+    const uint4 hd = blk[0];
+    const uint32_t sc_lo = hd.y & 0x3f3f3f3fu, m_lo = hd.z & 0x3f3f3f3fu;
+    const uint32_t sc_hi = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
+    const uint32_t m_hi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
+    const uint4 *ap = reinterpret_cast<const uint4 *>(sq + b * LINES_ACT_STRIDE);
+    int s1 = 0;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {  // the 32 bytes qs[32p..]: sub-block 2p in their low nibbles, 2p+1 in their high ones
+        const uint4 qa = blk[1 + 2 * p], qb = blk[2 + 2 * p];
+        const uint4 a0 = ap[4 * p], a1 = ap[4 * p + 1], a2 = ap[4 * p + 2], a3 = ap[4 * p + 3];
+        int lo = 0, hi = 0;
+        lo = dot4(qa.x & 0x0f0f0f0fu, a0.x, lo);
+        lo = dot4(qa.y & 0x0f0f0f0fu, a0.y, lo);
+        lo = dot4(qa.z & 0x0f0f0f0fu, a0.z, lo);
+        lo = dot4(qa.w & 0x0f0f0f0fu, a0.w, lo);
+        lo = dot4(qb.x & 0x0f0f0f0fu, a1.x, lo);
+        lo = dot4(qb.y & 0x0f0f0f0fu, a1.y, lo);
+        lo = dot4(qb.z & 0x0f0f0f0fu, a1.z, lo);
+        lo = dot4(qb.w & 0x0f0f0f0fu, a1.w, lo);
+        hi = dot4((qa.x >> 4) & 0x0f0f0f0fu, a2.x, hi);
+        hi = dot4((qa.y >> 4) & 0x0f0f0f0fu, a2.y, hi);
+        hi = dot4((qa.z >> 4) & 0x0f0f0f0fu, a2.z, hi);
+        hi = dot4((qa.w >> 4) & 0x0f0f0f0fu, a2.w, hi);
+        hi = dot4((qb.x >> 4) & 0x0f0f0f0fu, a3.x, hi);
+        hi = dot4((qb.y >> 4) & 0x0f0f0f0fu, a3.y, hi);
+        hi = dot4((qb.z >> 4) & 0x0f0f0f0fu, a3.z, hi);
+        hi = dot4((qb.w >> 4) & 0x0f0f0f0fu, a3.w, hi);
+        const uint32_t scw = (p < 2 ? sc_lo : sc_hi) >> ((p & 1) * 16);
+        s1 += __mul24((int)(scw & 0xff), lo) + __mul24((int)((scw >> 8) & 0xff), hi);
+    }
+    const int4 bsa = *reinterpret_cast<const int4 *>(sbs + b * 8), bsb = *reinterpret_cast<const int4 *>(sbs + b * 8 + 4);
+    int s2 = __mul24((int)(m_lo & 0xff), bsa.x) + __mul24((int)((m_lo >> 8) & 0xff), bsa.y) +
+             __mul24((int)((m_lo >> 16) & 0xff), bsa.z) + __mul24((int)(m_lo >> 24), bsa.w);
+    s2 += __mul24((int)(m_hi & 0xff), bsb.x) + __mul24((int)((m_hi >> 8) & 0xff), bsb.y) +
+          __mul24((int)((m_hi >> 16) & 0xff), bsb.z) + __mul24((int)(m_hi >> 24), bsb.w);
+    const float da = sd[b];
+    const float d = h2f(hd.x & 0xffffu), dmin = h2f(hd.x >> 16);
+    float v = (d * da) * (float)s1 - (dmin * da) * (float)s2;
+    const size_t row = span * RPS + lane / NB;
+    if (row >= (size_t)rows) v = 0.0f;  // (a short last span: this lane's block is not there)
+    v = part_sum<NB>(v);
+    if (lane % NB == 0 && row < (size_t)rows) y[row] = v;
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -409,10 +576,47 @@ bool fused_gemv_fits(const frk_weights *w) {
     return w->cols <= FUSED_GEMV_MAX_COLS;
 }
 
+// rows stored back to back whose block count divides 64
+static bool lines_kernel_fits(const frk_weights *w) {
+    const size_t nb = w->cols / QK_K;
+    return (nb == 8 || nb == 16 || nb == 32 || nb == 64) && w->layout.row_stride == nb * Q4_K_BYTES;
+}
+template <int NB, int MODE, int WAVES>
+static int launch_q4_k_lines_as(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+    constexpr size_t shmem = (size_t)NB * (LINES_ACT_STRIDE + 32 + 4) + (size_t)WAVES * 9216;
+    static_assert(shmem <= 160 * 1024, "LDS of a CU");
+    const size_t spans = (w->rows * (size_t)NB + 63) / 64;
+    const unsigned grid = (unsigned)((spans + WAVES - 1) / WAVES);
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_lines_kernel<NB, MODE, WAVES>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv lines, LDS %zu): %s", shmem, hipGetErrorString(e));
+        sized = true;
+    }
+    hipLaunchKernelGGL((gemv_q4_k_lines_kernel<NB, MODE, WAVES>), dim3(grid), dim3(64 * WAVES), shmem, s, w->dev, (int)w->rows, x,
+                       a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("gemv_q4_k_lines");
+    return FRK_OK;
+}
+// (Eight wavefronts to a workgroup: sixteen, which halve the activation's repeated quantization in the
+// one-launch form, measured slower -- 8.5 us against 8.2 at 14336x4096, one workgroup per CU instead of two.)
+template <int MODE>
+static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    constexpr int WIDE = 8;
+    if (nb == 8) return launch_q4_k_lines_as<8, MODE, WIDE>(w, x, a, y, s);
+    if (nb == 16) return launch_q4_k_lines_as<16, MODE, WIDE>(w, x, a, y, s);
+    if (nb == 32) return launch_q4_k_lines_as<32, MODE, WIDE>(w, x, a, y, s);
+    return launch_q4_k_lines_as<64, MODE, 8>(w, x, a, y, s);
+}
+
 int launch_gemv_q4_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    if (lines_kernel_fits(w)) return launch_q4_k_lines<MODE_FUSED>(w, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
     return launch_q4_k_fused<MODE_FUSED>(w, nullptr, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
 }
 int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    if (lines_kernel_fits(w)) return launch_q4_k_lines<MODE_PREQ_LDS>(w, nullptr, a, y, s);
     if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, nullptr, a, y, s);
     return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, nullptr, a, y, s);
 }

@@ -180,6 +180,8 @@ int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, 
 // batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
 size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+// the same over activations already quantized into the tiled form; `partial` holds the parts' sums of a split
+int launch_gemm_q4_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *y, float *partial, hipStream_t s);
 // the same for Q6_K (frk_gemm_q6.hip)
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);

@@ -516,12 +516,16 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d)", w->kind);
 }
 
-static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
-    // Q4_K: up to two launches of the thin kernel (16 rows each: 15 us at 14336x4096, 10 us at 4096x4096)
-    // are ahead of the matrix-core GEMM (28 us and 18 us there for 33..64 rows, its blocks split between
-    // workgroups)
+// Q4_K: up to two launches of the thin kernel (16 rows each: 15 us at 14336x4096, 10 us at 4096x4096)
+// are ahead of the matrix-core GEMM (28 us and 18 us there for 33..64 rows, its blocks split between
+// workgroups)
+static bool q4_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
     const size_t q4k_thin_rows = 32;
-    if (w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16)) {
+    return w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16);
+}
+
+static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
+    if (q4_k_takes_the_matrix_cores(w, batch)) {
         void *ws = nullptr;
         int rc = scratch.get(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
@@ -592,6 +596,36 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
     Scratch scratch;
     return gemm_impl(w, x, batch, y, stream, scratch);
+}
+
+int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const float *x, size_t batch, float *y0, float *y1,
+                          void *stream) {
+    clear_error();
+    if (!w0 || !w1 || !x || !y0 || !y1) return set_error(FRK_ERR_ARG, "frk_hip_gemm_pair_dev: null argument");
+    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+    if (w0->cols != w1->cols)
+        return set_error(FRK_ERR_SHAPE, "the matrices have %zu and %zu columns: they share one batch of activations", w0->cols, w1->cols);
+    hipStream_t s = (hipStream_t)stream;
+    Scratch scratch;
+    if (q4_k_takes_the_matrix_cores(w0, batch) && q4_k_takes_the_matrix_cores(w1, batch)) {
+        // one quantization into the tiled form, then the two GEMMs (each with its own room for a split's parts)
+        const size_t acts_bytes = round_up(q8k_tiled_bytes(batch, w0->cols), 256);
+        const size_t part0 = gemm_q4_k_workspace_bytes(batch, w0->cols, w0->rows) - acts_bytes;
+        const size_t part1 = gemm_q4_k_workspace_bytes(batch, w1->cols, w1->rows) - acts_bytes;
+        void *ws = nullptr;
+        int rc = scratch.get(acts_bytes + round_up(part0, 256) + part1, s, &ws);
+        if (rc) return rc;
+        const Q8KTiled acts = q8k_tiled_carve(ws, batch, w0->cols);
+        rc = launch_quantize_q8_k_tiled(x, batch, w0->cols, acts, s);
+        if (rc) return rc;
+        rc = launch_gemm_q4_k_acts(w0, acts, batch, y0, reinterpret_cast<float *>((char *)ws + acts_bytes), s);
+        if (rc) return rc;
+        return launch_gemm_q4_k_acts(w1, acts, batch, y1, reinterpret_cast<float *>((char *)ws + acts_bytes + round_up(part0, 256)), s);
+    }
+    // otherwise each matrix takes the path frk_hip_gemm_dev gives it (the same results, two quantizations)
+    int rc = gemm_impl(w0, x, batch, y0, stream, scratch);
+    if (rc) return rc;
+    return gemm_impl(w1, x, batch, y1, stream, scratch);
 }
 
 // ---- the entry point that allocates nothing ----

@@ -188,6 +188,12 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
                      void *stream);
 
+/* WeightMatrix::apply_batch_pair_with_acts (crates/frink-core/src/weight_matrix.rs:2447-2479) with
+ * BatchActs::Q8K (:757-768): two matrices of one column count over ONE quantization of the batch -- gate
+ * and up of a prefill FFN.  y0 and y1 are bit for bit what two frk_hip_gemm_dev calls give. */
+int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const float *x_dev, size_t batch,
+                          float *y0_dev, float *y1_dev, void *stream);
+
 /* frk_hip_gemm_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same
  * kernels and bit for bit the same y, but the scratch memory (quantized activations, the parts of a

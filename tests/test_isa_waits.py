@@ -28,11 +28,12 @@ def test_no_use_of_lds_reads_before_their_waits(tmp_path):
     assert sum("gemm_q6_k" in k for k in names) == 2, names
     for k in names:
         assert isa_wait_lint.violations(asm, k) == [], k
-    asm = _assembly(tmp_path, "frk_gemv_direct.hip")
-    names = isa_wait_lint.kernels(asm)
-    assert names
-    for k in names:
-        assert isa_wait_lint.violations(asm, k) == [], k
+    for name in ("frk_gemv_direct.hip", "frk_gemv_fused.hip"):
+        asm = _assembly(tmp_path, name)
+        names = isa_wait_lint.kernels(asm)
+        assert names
+        for k in names:
+            assert isa_wait_lint.violations(asm, k) == [], k
 
 
 def test_lint_sees_an_early_copy():
@@ -50,3 +51,45 @@ def test_lint_sees_an_early_copy():
     ])
     got = isa_wait_lint.violations(asm, "k")
     assert len(got) == 2 and "line 4" in got[0] and "line 7" in got[1], got
+
+
+def test_lint_follows_branches_and_loops():
+    # a read that a loop's back edge leaves in flight is seen by the loop head's first instruction;
+    # the block behind an unconditional branch is not reached from above
+    asm = "\n".join([
+        "k:",
+        "\tv_mov_b32_e32 v4, 0",
+        ".LBB0_1:",
+        "\tv_add_u32_e32 v30, v4, v5",
+        "\ts_waitcnt lgkmcnt(0)",
+        "\tds_read_b128 v[4:7], v1 offset:0",
+        "\ts_cbranch_scc1 .LBB0_1",
+        "\ts_branch .LBB0_3",
+        ".LBB0_2:",
+        "\tv_add_u32_e32 v31, v6, v5",
+        ".LBB0_3:",
+        "\ts_waitcnt lgkmcnt(0)",
+        "\tv_add_u32_e32 v31, v7, v5",
+        "\ts_endpgm",
+        ".Lfunc_end0:",
+    ])
+    got = isa_wait_lint.violations(asm, "k")
+    assert len(got) == 1 and "line 4" in got[0] and "since line 6" in got[0], got
+
+
+def test_lint_counts_memory_loads_and_loads_into_lds():
+    # vmcnt counts a load into LDS like any other; the register load in front of it is released by
+    # vmcnt(1), not before
+    asm = "\n".join([
+        "k:",
+        "\tglobal_load_dwordx4 v[4:7], v[2:3], off",
+        "\tglobal_load_lds_dwordx4 v1, s[2:3]",
+        "\tv_add_u32_e32 v30, v4, v9",
+        "\ts_waitcnt vmcnt(1)",
+        "\tv_add_u32_e32 v30, v4, v9",
+        "\tglobal_store_dword v[2:3], v30, off",
+        "\ts_endpgm",
+        ".Lfunc_end0:",
+    ])
+    got = isa_wait_lint.violations(asm, "k")
+    assert len(got) == 1 and "line 4" in got[0] and "since line 2" in got[0], got
