@@ -8,7 +8,12 @@ COPIES weight copies (COPIES x 33 MB > the 256 MB Infinity Cache), so the weight
 and not from cache.  The metric is the reference's: quantized weight bytes / seconds per step
 (crates/frink-cuda/examples/matvec_bench.rs:56-61), in GB/s.
 
-Prints ONE JSON line (see the fields at the bottom).
+The timed region is K steps captured in HIP graphs of at most GRAPH_STEPS steps and replayed
+(config.graph says how many steps one replay held: a replay starts with a few microseconds of
+nothing, which 400 steps dilute and 20 do not).
+
+Prints ONE JSON line (see the fields at the bottom).  `--read-sweep` prints, instead, the time of a
+read-only stream against its size (cache-cold), the floor under any kernel that reads that much.
 """
 import argparse
 import json
@@ -29,9 +34,11 @@ COPIES = 16
 # replay starts with a few microseconds of nothing, which 400 steps dilute and 16 would not
 GRAPH_STEPS = 400
 # HBM bytes per launch of the roofline kernel at 14336x4096, from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE 16163.5, WRITE_SIZE 56.0 per dispatch), each scaled by what the same counter
-# reads for copy_kernel over 32,256 KiB (FETCH_SIZE 16138.0 -> x1.9988, WRITE_SIZE 32256.0 -> x1.0).
-GEMV_TRAFFIC_BYTES = int((16163.5 * 32256.0 / 16138.0 + 56.0) * 1024)
+# script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter reads for
+# copy_kernel over 32,256 KiB: see profiles/bench_kernels_hbm_traffic_pmc.txt
+GEMV_FETCH_KIB, GEMV_WRITE_KIB = 16230.5, 56.0
+COPY_FETCH_KIB, COPY_WRITE_KIB, COPY_KIB = 16138.0, 32256.0, 32256.0
+GEMV_TRAFFIC_BYTES = int((GEMV_FETCH_KIB * COPY_KIB / COPY_FETCH_KIB + GEMV_WRITE_KIB * COPY_KIB / COPY_WRITE_KIB) * 1024)
 
 
 def random_blocks(kind, rows, cols, seed):
@@ -74,12 +81,15 @@ def time_graph(torch, fn_steps, n_steps, copies):
             graphs.append((g, count))
         g_full = graphs[0][0] if full else None
         g_rem = graphs[-1][0] if rem else None
-        # one untimed replay of each
+        # one untimed replay of each, then a synchronization; a second untimed replay goes out right in
+        # front of the timed ones with no synchronization between, so that the timed steps start on a
+        # GPU that is already running steps (the state of a decode loop) and not on an idle one
         for g, _ in graphs:
             g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        graphs[0][0].replay()
         e0.record()
         for _ in range(full):
             g_full.replay()
@@ -88,29 +98,102 @@ def time_graph(torch, fn_steps, n_steps, copies):
         e1.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-    return wall, e0.elapsed_time(e1) * 1e-3
+    # (the host's clock also saw the untimed replay in front: scaled to the timed steps' share)
+    return wall * n_steps / (n_steps + graphs[0][1]), e0.elapsed_time(e1) * 1e-3
 
 
-def cpu_baseline(kind, data, rows, cols, x, y_gpu, budget_s=8.0):
-    """Times the CPU oracle (a C restatement of Frink's integer-dot CPU path, row-parallel over
-    OpenMP threads) on the same weights and activation, and checks the GPU result against it."""
-    import oracle as fo
-    threads = min(16, os.cpu_count() or 1)
-    want = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads)
-    reps, spent = 0, 0.0
-    best = float("inf")
-    while spent < budget_s and reps < 200:
+def host_cpu():
+    """Model name, logical CPUs this process may use, physical cores among them (distinct
+    thread_siblings_list entries, as crates/frink-core/src/threads.rs sizes the reference's pool) and
+    whether AVX2 and FMA are there."""
+    model, flags = "unknown", ""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name") and model == "unknown":
+                model = line.split(":", 1)[1].strip()
+            elif line.startswith("flags") and not flags:
+                flags = line.split(":", 1)[1]
+    except OSError:
+        pass
+    cpus = sorted(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else list(range(os.cpu_count() or 1))
+    cores = set()
+    for c in cpus:
+        try:
+            cores.add(open("/sys/devices/system/cpu/cpu%d/topology/thread_siblings_list" % c).read().strip())
+        except OSError:
+            cores.add("cpu%d" % c)
+    words = flags.split()
+    return {"cpu_model": model, "logical_cpus": len(cpus), "physical_cores": len(cores),
+            "avx2_fma": "avx2" in words and "fma" in words}
+
+
+def best_of(fn, budget_s, max_reps=50):
+    reps, spent, best = 0, 0.0, float("inf")
+    while reps < 1 or (spent < budget_s and reps < max_reps):
         t = time.perf_counter()
-        fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads)
+        fn()
         dt = time.perf_counter() - t
         best = min(best, dt)
         spent += dt
         reps += 1
+    return best, reps
+
+
+def cpu_baseline(kind, data, rows, cols, x, y_gpu, xb):
+    """Times the CPU forms of the same work on this host's physical cores (rows over OpenMP threads,
+    as the reference partitions them): the decode GEMV as the reference's x86 default runs it (AVX2+FMA
+    f32 dot), as its integer path runs it (Q8_K + AVX2 integer dot) and as the scalar oracle computes
+    it; and the M=512 GEMM as integer dots with the weight row outermost.  Checks the GPU's GEMV
+    against the scalar oracle on the way."""
+    import oracle as fo
+    host = host_cpu()
+    threads = max(1, host["physical_cores"])
+    want = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads)
     err = float(np.abs(y_gpu - want).max() / np.abs(want).max())
-    return {"value": round(data.size / best / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": "the whole workload (Q8_K activation quantization + %dx%d Q4_K integer dots), best of %d "
-                      "repetitions, scalar C restatement of dot_q4_k_q8 with OpenMP row partition" % (rows, cols, reps),
-            "gpu_vs_cpu_max_err_over_ninf": err}
+    legs = {}
+    t, n = best_of(lambda: fo.gemv(kind, data, rows, cols, x, fo.INT_DOT, threads), 3.0)
+    legs["decode_int_dot_scalar_GBs"] = round(data.size / t / 1e9, 2)
+    simd = host["avx2_fma"] and fo.have_avx2()
+    if simd:
+        t, n = best_of(lambda: fo.avx2_gemv_q4_k_f32(data, rows, cols, x, threads), 4.0)
+        legs["decode_f32_dot_avx2_GBs"] = round(data.size / t / 1e9, 2)
+        headline, what = data.size / t / 1e9, "AVX2+FMA f32 dot (the reference's x86 decode default), best of %d" % n
+        t, n = best_of(lambda: fo.avx2_gemm_q4_k_q8k(data, rows, cols, x, threads), 4.0)
+        legs["decode_int_dot_avx2_GBs"] = round(data.size / t / 1e9, 2)
+        t, n = best_of(lambda: fo.avx2_gemm_q4_k_q8k(data, rows, cols, xb, threads), 8.0, 5)
+        legs["gemm_m512_int_dot_avx2_TOPS"] = round(2.0 * xb.shape[0] * rows * cols / t / 1e12, 4)
+        legs["gemm_m512_ms"] = round(t * 1e3, 1)
+    else:
+        headline, what = legs["decode_int_dot_scalar_GBs"], "scalar integer dot (this host has no AVX2+FMA)"
+    out = {"value": round(headline, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+           "sample": "the whole workload (%dx%d Q4_K decode GEMV) as %s; legs: the same GEMV on the integer path "
+                     "(Q8_K quantization + AVX2 integer dot, and the scalar oracle), and the whole M=512 GEMM as "
+                     "AVX2 integer dots with the weight row outermost; %d OpenMP threads = physical cores"
+                     % (rows, cols, what, threads),
+           "legs": legs, "gpu_vs_cpu_max_err_over_ninf": err}
+    out.update(host)
+    return out
+
+
+def read_sweep(torch, fa):
+    """time of a read-only stream against its size, every launch reading memory no earlier launch of
+    the last 512 MB touched"""
+    import ctypes as C
+    dev = torch.device("cuda:0")
+    pool = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_()
+    sink = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+    L = fa.lib()
+    print("# read-only stream (frk_hip_read_dev), cache-cold: bytes, us per launch, GB/s")
+    for mb in (8, 16, 33, 66, 132, 264):
+        nbytes = mb * 1000 * 1000 // 4096 * 4096
+        slots = max(2, (1 << 30) // nbytes)
+
+        def rd(i):
+            fa.check(L.frk_hip_read_dev(C.c_void_p(pool.data_ptr() + (i % slots) * nbytes), nbytes,
+                                        C.c_void_p(sink.data_ptr()), fa._stream()))
+        n = 4 * slots if mb >= 132 else 400
+        _, t = time_graph(torch, rd, n, min(n, 400))
+        print("%10d  %7.2f  %7.1f" % (nbytes, t / n * 1e6, nbytes / (t / n) / 1e9), flush=True)
 
 
 def main():
@@ -120,6 +203,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--read-sweep", action="store_true", help="only: time of a read-only stream against its size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
@@ -129,6 +213,9 @@ def main():
     import torch
     import frink_amd as fa
 
+    if args.read_sweep:
+        read_sweep(torch, fa)
+        return
     info = fa.probe()
     dev = torch.device("cuda:0")
     rows, cols, kind = 14336, 4096, fa.Q4_K
@@ -153,7 +240,12 @@ def main():
     wbytes = data.size
     value = wbytes / sec_per_step / 1e9
 
-    # ---- roofline of the dominant kernel: GEMV alone, activation already quantized ----
+    # ---- roofline of the dominant kernel = the one kernel a step launches (quantization inside it):
+    # its launch duration is the step's, measured above with events on the stream it runs on ----
+    alg_bytes = wbytes + cols * 4 + rows * 4  # W + x + y
+    achieved = alg_bytes / sec_per_step / 1e9
+    y_gpu = y.cpu().numpy()
+    # the same product from an activation quantized beforehand (what a fused producer would hand over)
     acts = fa.quantize_q8_k(xd)
 
     def gemv_only(i):
@@ -162,9 +254,6 @@ def main():
     n_k = max(COPIES * 8, min(args.steps, 4000))
     _, ev_k = time_graph(torch, gemv_only, n_k, GRAPH_STEPS)
     k_sec = ev_k / n_k
-    alg_bytes = wbytes + cols + cols // 256 * 4 + cols // 16 * 2 + rows * 4  # W + Q8_K activation + y
-    achieved = alg_bytes / k_sec / 1e9
-    y_gpu = y.cpu().numpy()
 
     out = {
         "metric": "Q4_K GEMV HBM GB/s", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
@@ -172,13 +261,20 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "Q4_K decode GEMV, rows=14336 cols=4096 batch=1 (Llama-3-8B FFN gate/up): Q8_K "
-                               "activation quantization + GEMV per step, %d weight copies rotated (cache-cold)" % COPIES,
+                               "activation quantization + GEMV per step (one kernel), %d weight copies rotated "
+                               "(cache-cold)" % COPIES,
+                   "graph": "%d steps timed with HIP events as replays of a HIP graph of %d steps, behind one untimed "
+                            "replay with no synchronization between" % (args.steps, min(args.steps, GRAPH_STEPS)),
                    "weight_bytes": int(wbytes), "device": info["name"], "arch": info["gcn_arch"],
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_fused_kernel<32, 1, 1, 1, 2, 512, false, false, false>", "algorithmic_bytes": int(alg_bytes),
-                     "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k},
+                     "kernel": "gemv_q4_k_lines_kernel<16, 0, 8>", "algorithmic_bytes": int(alg_bytes),
+                     "avg_launch_us": round(sec_per_step * 1e6, 3), "launches": args.steps,
+                     "prequantized_form": {"kernel": "gemv_q4_k_lines_kernel<16, 1, 8>",
+                                           "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k,
+                                           "frac": round((wbytes + cols + cols // 256 * 4 + cols // 16 * 2 + rows * 4)
+                                                         / k_sec / 1e9 / HBM_PEAK_GBS, 4)}},
     }
 
     if not args.no_extra:
@@ -218,22 +314,38 @@ def main():
                            "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
             for w in w2:
                 w.release()
-        # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step
-        # (activation quantization is inside the step)
+        # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step.  The step is
+        # the activations' quantization + the GEMM kernel; the kernel alone is what a second matrix over
+        # the same quantized activations adds (frk_hip_gemm_pair_dev: one quantization, two GEMM launches).
         xb = torch.from_numpy(synth.activations(6, 512, cols, outlier_frac=0.01)).to(dev)
-        for name, r2 in (("Q4_K GEMM M=512 4096x4096", 4096), ("Q4_K GEMM M=512 14336x4096", 14336)):
+        gemm_records = []
+        for name, r2, kname in (("Q4_K GEMM M=512 4096x4096", 4096, "gemm_q4_k_pipe_kernel<4, 2, 2>"),
+                                ("Q4_K GEMM M=512 14336x4096", 14336, "gemm_q4_k_pipe_kernel<8, 1, 4>")):
             d2 = torch.from_numpy(random_blocks(kind, r2, cols, seed=78)).to(dev)
-            w2 = [fa.Weights.from_device(kind, d2, r2, cols) for _ in range(4)]
+            w2 = [fa.Weights.from_device(kind, d2, r2, cols) for _ in range(8)]
             yb = torch.empty((512, r2), dtype=torch.float32, device=dev)
+            yb2 = torch.empty((512, r2), dtype=torch.float32, device=dev)
 
             def step3(i):
-                w2[i % 4].gemm(xb, out=yb)
+                w2[i % 8].gemm(xb, out=yb)
+
+            def step3p(i):
+                fa.gemm_pair(w2[(2 * i) % 8], w2[(2 * i + 1) % 8], xb, outs=(yb, yb2))
             _, t = time_graph(torch, step3, 200, 100)
-            tops = 2.0 * 512 * r2 * cols / (t / 200) / 1e12
+            _, tp = time_graph(torch, step3p, 200, 100)
+            ops = 2.0 * 512 * r2 * cols
+            tops = ops / (t / 200) / 1e12
+            k_us = (tp - t) / 200 * 1e6
             extra[name] = {"TOPS": round(tops, 1), "us_per_step": round(t / 200 * 1e6, 2),
                            "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            gemm_records.append({"bound": "mfma", "workload": name, "kernel": kname, "achieved": round(ops / k_us / 1e6, 1),
+                                 "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops / k_us / 1e6 / INT8_PEAK_TOPS, 4),
+                                 "ops": ops, "avg_launch_us": round(k_us, 2), "launches": 200,
+                                 "how": "pair step (one quantization + two GEMM launches) minus single step, HIP events",
+                                 "step_us_with_quantization": round(t / 200 * 1e6, 2)})
             for w in w2:
                 w.release()
+        out["roofline_gemm"] = gemm_records
         # the FFN down projection of a Q4_K_M model at M=512: Q6_K on the matrix cores
         d6g = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=78)).to(dev)
         w6 = [fa.Weights.from_device(fa.Q6_K, d6g, cols, rows) for _ in range(4)]
@@ -379,7 +491,7 @@ def main():
         out["extra"] = extra
 
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(kind, data, rows, cols, x, y_gpu)
+        out["cpu_baseline"] = cpu_baseline(kind, data, rows, cols, x, y_gpu, synth.activations(6, 512, cols, outlier_frac=0.01))
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -402,6 +402,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
         constexpr int XB = (NB + WAVES - 1) / WAVES;
         if (XB == 1) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]));
         else if (XB == 2) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]));
+        else if (XB == 3) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]));
         else if (XB == 4)
             asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]));
         else
@@ -599,8 +600,9 @@ static int launch_q4_k_lines_as(const frk_weights *w, const float *x, Q8KActs a,
     FRK_LAUNCH_CHECK("gemv_q4_k_lines");
     return FRK_OK;
 }
-// (Eight wavefronts to a workgroup: sixteen, which halve the activation's repeated quantization in the
-// one-launch form, measured slower -- 8.5 us against 8.2 at 14336x4096, one workgroup per CU instead of two.)
+// (Eight wavefronts to a workgroup, two workgroups to a CU.  Measured at 14336x4096, one-launch form /
+// pre-quantized form in us: 8 wavefronts 8.1 / 7.5; 7 (which spreads the 3584 spans evenly, 14 per CU)
+// 8.7 / 7.7; 14 in one workgroup per CU 9.2 / 8.7; 4 9.0 / 8.3; 2 12.1 / 8.3.)
 template <int MODE>
 static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / QK_K);

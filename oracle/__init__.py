@@ -76,6 +76,8 @@ def lib():
             "fo_moe_ffn_per_position": (C.c_int, [C.c_int, u8p, u8p, u8p, C.c_int, C.c_int, C.c_int, f32p,
                                                   C.c_int, i32p, f32p, C.c_int, f32p, C.c_int]),
             "fo_have_avx2": (C.c_int, []),
+            "fo_avx2_gemv_q4_k_f32": (C.c_int, [u8p, sz, sz, f32p, f32p, C.c_int]),
+            "fo_avx2_gemm_q4_k_q8k": (C.c_int, [u8p, sz, sz, f32p, sz, f32p, C.c_int]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -268,3 +270,23 @@ def moe_ffn_batch(kind, gate, up, down, n_experts, hidden, ffn, x, ids, weights,
 
 def have_avx2():
     return bool(lib().fo_have_avx2())
+
+
+def avx2_gemv_q4_k_f32(w, rows, cols, x, threads=1):
+    """The reference's x86 decode default (AVX2+FMA f32 dot), for the timed CPU baseline."""
+    w, x = _u8(w), _f32(x).ravel()
+    y = np.empty(rows, np.float32)
+    rc = lib().fo_avx2_gemv_q4_k_f32(_p(w, C.c_uint8), rows, cols, _p(x, C.c_float), _p(y, C.c_float), threads)
+    if rc:
+        raise RuntimeError("fo_avx2_gemv_q4_k_f32 rc=%d (no AVX2+FMA on this host?)" % rc)
+    return y
+
+
+def avx2_gemm_q4_k_q8k(w, rows, cols, x, threads=1):
+    """x: [batch][cols] -> [batch][rows]: Q8_K quantization + AVX2 integer dots, weight row outermost."""
+    w, x = _u8(w), _f32(x).reshape(-1, cols)
+    y = np.empty((x.shape[0], rows), np.float32)
+    rc = lib().fo_avx2_gemm_q4_k_q8k(_p(w, C.c_uint8), rows, cols, _p(x, C.c_float), x.shape[0], _p(y, C.c_float), threads)
+    if rc:
+        raise RuntimeError("fo_avx2_gemm_q4_k_q8k rc=%d (no AVX2+FMA on this host?)" % rc)
+    return y

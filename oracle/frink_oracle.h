@@ -113,6 +113,13 @@ int fo_moe_ffn_per_position(int kind, const uint8_t *gate, const uint8_t *up, co
 /* CPU baseline: AVX2 dot where the host has it; returns 1 if AVX2 was used */
 int fo_have_avx2(void);
 
+/* The x86 forms the reference runs, for the timed CPU baseline only (cpu_baseline_avx2.c):
+ * AVX2+FMA f32 decode dot and AVX2 integer dot (Q8_K activations, `batch` rows of them, weight row
+ * outermost), rows over `threads` OpenMP threads.  -1 on a host without AVX2 and FMA. */
+int fo_avx2_gemv_q4_k_f32(const uint8_t *w, size_t rows, size_t cols, const float *x, float *y, int threads);
+int fo_avx2_gemm_q4_k_q8k(const uint8_t *w, size_t rows, size_t cols, const float *x, size_t batch, float *y,
+                          int threads);
+
 #ifdef __cplusplus
 }
 #endif

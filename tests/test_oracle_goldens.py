@@ -579,3 +579,29 @@ def test_moe_per_position_adds_the_slots_in_routing_order():
         assert np.array_equal(per_pos[b].view(np.uint32), acc.view(np.uint32)), b
     # the dispatcher follows the reference's threshold
     assert np.array_equal(fo.moe_ffn(fo.Q4_K, gate, up, down, E, hidden, ffn, x, ids, w), per_pos)
+
+
+def test_cpu_baseline_legs_agree_with_the_scalar_oracle():
+    """The AVX2 forms bench.py times beside the GPU: the integer dot must equal the scalar oracle's bit
+    for bit (exact integers, the same float expression); the f32 dot keeps eight partial sums a
+    sub-block where the scalar form keeps one, so it is held to fp32 reassociation only (no vector of
+    the reference pins it: it is timed, never used as a checker)."""
+    if not fo.have_avx2():
+        pytest.skip("no AVX2+FMA on this host")
+    rng = np.random.default_rng(5)
+    rows, cols = 96, 1024
+    w = fo.encode_matrix(fo.Q4_K, (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32))
+    x = rng.standard_normal((7, cols)).astype(np.float32)
+    x[3] = 0.0
+    got = fo.avx2_gemm_q4_k_q8k(w, rows, cols, x, threads=3)
+    want = fo.gemm(fo.Q4_K, w, rows, cols, x, fo.INT_DOT, 2)
+    assert np.array_equal(got, want)
+    f = fo.avx2_gemv_q4_k_f32(w, rows, cols, x[0], threads=2)
+    wf = fo.gemv(fo.Q4_K, w, rows, cols, x[0], fo.F32_DOT, 1)
+    assert np.abs(f - wf).max() <= 2e-6 * np.abs(wf).max()
+
+
+def test_bench_reads_the_host_cpu():
+    import bench
+    h = bench.host_cpu()
+    assert 1 <= h["physical_cores"] <= h["logical_cpus"] and isinstance(h["cpu_model"], str)
