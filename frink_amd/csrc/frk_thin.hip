@@ -752,6 +752,175 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
     }
 }
 
+// ------------------------------------------------------------------ thin GEMM over whole spans (Q4_K)
+//
+// The kernel above walks a row group's blocks one after the other, four in flight: at 14336x4096 a
+// wavefront's sixteen blocks are a chain of sixteen round trips, and its 144-byte pieces of sixteen
+// rows cost the CU's L1 two line look-ups for every line of data.  Here a wavefront owns 16 rows x 4
+// blocks = 16 contiguous pieces of 576 bytes, requests them all at once and into LDS without passing
+// registers (ten global_load_lds: a row's 36 sixteen-byte pieces back to back and a 37th of padding,
+// so that rows, 592 bytes apart, fall in different banks for the MFMA's reads), and multiplies when
+// they have landed.  The quantized activations come in slices of four blocks (a KB a row, with the
+// slice's sums and scales), moved by global_load_lds as well.  The arithmetic is the kernel's above,
+// block by block, all LDS reads and MFMAs of the four blocks issued before the first integer multiply.
+// A workgroup is one row group, its wavefronts the row's groups of four blocks (rows of up to 32
+// blocks); all slices of the activations are staged, and the wavefronts' sums are added in the order
+// of the blocks through LDS.  Small workgroups, two to a CU: one streams while the other multiplies.
+// Measured at 14336x4096, 8 rows: 12.0 us against the kernel above's 12.1 (the data movement alone
+// takes 7.5 us: what is left is the multiplication, which two workgroups a CU overlap too little);
+// at 4096x4096 6.0 us against 6.9.  (Rows split between workgroups, one slice each, with the
+// partial sums added by whichever workgroup finishes last, were tried for longer rows: the three
+// trips to memory at the end cost 3 us, more than the split gains.)
+constexpr int TS_ROW_PIECES = 37;
+constexpr int TS_ROW_BYTES = TS_ROW_PIECES * 16;   // 592
+constexpr int TS_SLOT = 16 * TS_ROW_BYTES;         // 9472
+constexpr int TS_Q_STRIDE = 1024 + 16;             // a row of an activation slice (padded: 16 rows, 16 banks apart)
+template <int ACTS>
+struct SpanLds {
+    static constexpr int OFF_BS = ACTS * TS_Q_STRIDE;  // int16 sums [ACTS][4 blocks][16]
+    static constexpr int OFF_D = OFF_BS + ACTS * 128;  // f32 scales [4 blocks][16 rows]
+    static constexpr int SLICE = OFF_D + 256;
+    static constexpr size_t bytes(int slices, int waves) { return (size_t)slices * SLICE + (size_t)waves * TS_SLOT; }
+};
+
+template <int ACTS>
+__global__ __launch_bounds__(512) void thin_span_q4_k_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int nb,
+                                                            int batch, const int8_t *__restrict__ aq,
+                                                            const float *__restrict__ ad, const int16_t *__restrict__ absums,
+                                                            float *__restrict__ y) {
+    using L = SpanLds<ACTS>;
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    const uint32_t lds0 = lds_address(lds);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = (int)blockDim.x >> 6;
+    const int kg = wave, slices = waves;  // a wavefront per group of four blocks
+    const int row0 = (int)blockIdx.x * 16;
+    const int cols = nb * QK_K;
+    uint8_t *const lds_w = lds + slices * L::SLICE;
+
+    // ---- the activations' slices, their pieces dealt to the wavefronts ----
+    for (int t = wave; t < slices * (ACTS + 2); t += waves) {  // (uniform per wavefront)
+        const int sl = t / (ACTS + 2), piece = t % (ACTS + 2);
+        const int k = sl;
+        const uint32_t base = lds0 + (uint32_t)sl * L::SLICE;
+        if (piece < ACTS) {
+            dma16(base + piece * TS_Q_STRIDE, aq + (size_t)min(piece, batch - 1) * cols + (size_t)k * 1024, (uint32_t)lane * 16);
+        } else if (piece == ACTS) {  // the 64 sums of a row's slice are 128 bytes: eight rows an instruction
+#pragma unroll
+            for (int h = 0; h < ACTS / 8; h++) {
+                const int tok = min(h * 8 + (lane >> 3), batch - 1);
+                dma16(base + L::OFF_BS + h * 1024, reinterpret_cast<const uint8_t *>(absums) + (size_t)k * 128,
+                      (uint32_t)tok * (uint32_t)nb * 32u + (uint32_t)(lane & 7) * 16u);
+            }
+        } else {  // the scales, [block][row]
+            const int tok = min(lane & 15, batch - 1);
+            dma4(base + L::OFF_D, ad + (size_t)k * 4, ((uint32_t)tok * (uint32_t)nb + (uint32_t)(lane >> 4)) * 4u);
+        }
+    }
+    // ---- this wavefront's 16 rows x 4 blocks: slot piece s = 64 c + lane is row s / 37, piece s % 37 ----
+    {
+        const int rbase = min(row0, rows - 1);  // (a wavefront past the matrix reads its last row and stores nothing)
+        const uint8_t *src = W + (size_t)rbase * row_stride + (size_t)kg * 576;
+        const uint32_t slot = lds_address(lds_w) + (uint32_t)wave * TS_SLOT;
+#pragma unroll
+        for (int c = 0; c < 10; c++) {
+            const int sl = 64 * c + lane;
+            const int r = min(sl / TS_ROW_PIECES, 15), q = min(sl % TS_ROW_PIECES, 35);  // (the 37th piece: the 36th again)
+            const uint32_t off = (uint32_t)(min(row0 + r, rows - 1) - rbase) * (uint32_t)row_stride + (uint32_t)q * 16u;
+            if (c < 9) dma16(slot + c * 1024, src, off);
+            else if (lane < 16 * TS_ROW_PIECES - 576) dma16(slot + 9 * 1024, src, off);
+        }
+    }
+    // the activations' pieces are older than the span's ten; only they are shared, so the barrier comes
+    // before the wait for the span and a wavefront multiplies as soon as ITS rows have landed
+    asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+    lds_barrier();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    const int j = lane & 15, g = lane >> 4;
+    const int act = min(j, ACTS - 1);  // (rows past the staged ones repeat the last; their results are not stored)
+    const uint8_t *slice = lds + wave * L::SLICE;
+    const uint8_t *a_q = slice + act * TS_Q_STRIDE + 8 * g;
+    const uint8_t *a_bs = slice + L::OFF_BS + act * 128 + 8 * g;
+    const float *a_d = reinterpret_cast<const float *>(slice + L::OFF_D) + 4 * g;
+    uint8_t *const my_slot = lds_w + wave * TS_SLOT;
+    const uint8_t *a_w = my_slot + j * TS_ROW_BYTES;
+    auto as_long = [](uint2 v) { return (long)(((unsigned long)v.y << 32) | v.x); };
+    v4f_t acc = {0.f, 0.f, 0.f, 0.f};
+    // Everything the four blocks need is read from LDS first: with two wavefronts to a SIMD there is nothing
+    // else to hide a block's chain of LDS reads, MFMAs and integer multiplies behind but the other blocks.
+    uint4 hd[4];
+    uint2 wq[4][4], alo[4][4], ahi[4][4], bsw[4];
+    v4f_t da[4];
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) {
+        hd[blk] = *reinterpret_cast<const uint4 *>(a_w + blk * Q4_K_BYTES);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            wq[blk][c] = *reinterpret_cast<const uint2 *>(a_w + blk * Q4_K_BYTES + 16 + 32 * c + 8 * g);
+            alo[blk][c] = *reinterpret_cast<const uint2 *>(a_q + blk * QK_K + 64 * c);
+            ahi[blk][c] = *reinterpret_cast<const uint2 *>(a_q + blk * QK_K + 64 * c + 32);
+        }
+        bsw[blk] = *reinterpret_cast<const uint2 *>(a_bs + blk * 32);
+        da[blk] = *reinterpret_cast<const v4f_t *>(a_d + blk * 16);
+    }
+    const v4i_t zero = {0, 0, 0, 0};
+    v4i_t t0[4][4], t1[4][4];
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {  // sub-blocks 2c (low nibbles) and 2c+1 (high)
+            const uint2 q = wq[blk][c];
+            const uint2 lo = make_uint2(q.x & 0x0f0f0f0fu, q.y & 0x0f0f0f0fu);
+            const uint2 hi = make_uint2((q.x >> 4) & 0x0f0f0f0fu, (q.y >> 4) & 0x0f0f0f0fu);
+            t0[blk][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(alo[blk][c]), as_long(lo), zero, 0, 0, 0);
+            t1[blk][c] = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(ahi[blk][c]), as_long(hi), zero, 0, 0, 0);
+        }
+#pragma unroll
+    for (int blk = 0; blk < 4; blk++) {
+        const uint4 h = hd[blk];
+        const uint32_t sc_lo = h.y & 0x3f3f3f3fu, m_lo = h.z & 0x3f3f3f3fu;
+        const uint32_t sc_hi = (h.w & 0x0f0f0f0fu) | (((h.y >> 6) & 0x03030303u) << 4);
+        const uint32_t m_hi = ((h.w >> 4) & 0x0f0f0f0fu) | (((h.z >> 6) & 0x03030303u) << 4);
+        v4i_t s1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t scw = (c < 2 ? sc_lo : sc_hi) >> (16 * (c & 1));
+            const int sc0 = scw & 0xff, sc1 = (scw >> 8) & 0xff;
+#pragma unroll
+            for (int r = 0; r < 4; r++) s1[r] += __mul24(sc0, t0[blk][c][r]) + __mul24(sc1, t1[blk][c][r]);
+        }
+        const uint32_t mw = (g < 2 ? m_lo : m_hi) >> (16 * (g & 1));
+        const _Float16 m0 = (_Float16)(int)(mw & 0xff), m1 = (_Float16)(int)((mw >> 8) & 0xff);
+        const v4h_t mh = {m0, m0, m1, m1};
+        const v4h_t bh = {(_Float16)(int)(int16_t)(bsw[blk].x & 0xffff), (_Float16)(int)(int16_t)(bsw[blk].x >> 16),
+                          (_Float16)(int)(int16_t)(bsw[blk].y & 0xffff), (_Float16)(int)(int16_t)(bsw[blk].y >> 16)};
+        const v4f_t zf = {0.f, 0.f, 0.f, 0.f};
+        const v4f_t s2 = __builtin_amdgcn_mfma_f32_16x16x16f16(bh, mh, zf, 0, 0, 0);
+        const float d = h2f(h.x & 0xffffu), ndmin = -h2f(h.x >> 16);
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[r] = fmaf(da[blk][r], fmaf(ndmin, s2[r], d * (float)s1[r]), acc[r]);
+    }
+
+    const int row = row0 + j;
+    // the row's groups of four blocks meet in LDS (every wavefront's own slot, which it has read for the
+    // last time) and the first wavefront adds them in their order
+    if (waves > 1) {
+        if (wave > 0) *reinterpret_cast<v4f_t *>(my_slot + lane * 16) = acc;
+        __syncthreads();
+        if (wave > 0) return;
+        for (int k = 1; k < waves; k++) {
+            const v4f_t o = *reinterpret_cast<const v4f_t *>(lds_w + k * TS_SLOT + lane * 16);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += o[r];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        if (4 * g + r < batch && row < rows) y[(size_t)(4 * g + r) * rows + row] = acc[r];
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -810,6 +979,7 @@ static int launch_thin_nb(const frk_weights *w, int batch, Q8KActs a, float *y, 
 }
 
 constexpr size_t TM_LDS_LIMIT = 160 * 1024;
+
 
 template <int RG, int ACTS, bool Q5>
 static int launch_thin_mfma_kind(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
@@ -888,6 +1058,31 @@ static int launch_thin_mfma6_rg(const frk_weights *w, int batch, Q8KActs a, floa
     }
 }
 
+// ---- the span kernel: Q4_K rows of 4, 8, .. 32 blocks (a wavefront per four), up to 16 activation rows ----
+static bool thin_span_fits(const frk_weights *w, int batch) {
+    const size_t nb = w->cols / QK_K, n_kg = nb / 4;
+    if (w->kind != FRK_KIND_Q4_K || nb % 4 || n_kg > 8 || batch < 1 || batch > 16) return false;
+    if (nb * Q4_K_BYTES > w->layout.row_stride) return false;
+    const size_t lds = batch > 8 ? SpanLds<16>::bytes((int)n_kg, (int)n_kg) : SpanLds<8>::bytes((int)n_kg, (int)n_kg);
+    return lds <= TM_LDS_LIMIT;
+}
+template <int ACTS>
+static int launch_thin_span(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t groups = (w->rows + 15) / 16;
+    const int waves = (int)(w->cols / QK_K / 4);
+    const size_t shmem = SpanLds<ACTS>::bytes(waves, waves);
+    static bool sized = false;
+    if (!sized) {
+        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_span_q4_k_kernel<ACTS>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)TM_LDS_LIMIT));
+        sized = true;
+    }
+    hipLaunchKernelGGL((thin_span_q4_k_kernel<ACTS>), dim3((unsigned)groups), dim3(64 * waves), shmem, s, w->dev,
+                       w->layout.row_stride, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("thin span gemm");
+    return FRK_OK;
+}
+
 // Largest number of activation rows one launch can take for this matrix: up to 16 on the
 // matrix-core path (Q4_K), else what fits LDS, at most 8.
 int thin_gemm_max_batch(const frk_weights *w) {
@@ -910,6 +1105,8 @@ int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, 
 
 // y[batch][rows] for 1 <= batch <= thin_gemm_max_batch(w) quantized activation rows (K-quants).
 int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    if (batch > 2 && thin_span_fits(w, batch))
+        return batch > 8 ? launch_thin_span<16>(w, batch, a, y, s) : launch_thin_span<8>(w, batch, a, y, s);
     // (two rows of Q4_K: the dot4 kernel is still ahead)
     if ((w->kind == FRK_KIND_Q4_K && thin_mfma_acts(w) > 0 && batch > 2) || w->kind == FRK_KIND_Q5_K) {
         // the fewest staged rows that hold the batch
