@@ -135,6 +135,98 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void gemv_q6_k_direct_kernel(
     if (lane == 0 && store) y[r] = acc;
 }
 
+// ------------------------------------------------------------------ Q6_K experts, one job per (token, slot)
+// The decode form of a mixture-of-experts down projection whose experts are Q6_K (run_expert,
+// crates/frink-moe/src/lib.rs:1068-1165): job j multiplies expert ids[j]'s rows_e rows (the experts'
+// matrices are stacked) by ITS activation x + j * x_stride, which the workgroup quantizes to Q8_K in
+// LDS first (bit-exact with quantize_activations_q8_k).  Expert rows are short (768 columns = 12
+// units in the usual case), so LPR lanes share a row and a wavefront takes 64 / LPR rows at a time,
+// STEPS times, all of a lane's weight loads in flight before the activation is quantized.
+// The arithmetic is dot_q6_k_q8's, as in the kernel above.  An id outside [0, n_experts) computes on
+// expert 0 (the weighted sum leaves such a slot out).
+template <int LPR, int STEPS>
+__global__ __launch_bounds__(256) void gemv_q6_k_experts_kernel(const uint8_t *__restrict__ W, Layout lay, int rows_e, int nb,
+                                                               int n_experts, const int32_t *__restrict__ ids,
+                                                               const float *__restrict__ x, int x_stride,
+                                                               float *__restrict__ y) {
+    constexpr int PARTS = 64 / LPR, ROWS_WG = 4 * PARTS * STEPS;
+    extern __shared__ uint4 smem_direct[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int part = lane / LPR, l = lane % LPR;
+    const int job = blockIdx.y;
+    int e = ids[job];
+    if (e < 0 || e >= n_experts) e = 0;
+    const int units = nb * 4;
+    const int u = min(l, units - 1);  // (a lane past the row's units repeats the last, unused)
+    const int b = u >> 2, h = (u >> 1) & 1, t = u & 1;
+    const float *xj = x + (size_t)job * x_stride;
+
+    constexpr int XB = 4;  // blocks of the activation a wavefront quantizes (nb <= 16)
+    float4 xv[XB];
+#pragma unroll
+    for (int i = 0; i < XB; i++) xv[i] = reinterpret_cast<const float4 *>(xj + (size_t)min(wave + 4 * i, nb - 1) * QK_K)[lane];
+    uint4 qla[STEPS], qlb[STEPS], qh[STEPS];
+    uint2 scv[STEPS];
+    uint32_t dbits[STEPS];
+    int rr[STEPS];
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+        rr[st] = (int)blockIdx.x * ROWS_WG + (st * 4 + wave) * PARTS + part;
+        const uint8_t *row = W + ((size_t)e * rows_e + min(rr[st], rows_e - 1)) * lay.row_stride;
+        qla[st] = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + t * 16);
+        qlb[st] = *reinterpret_cast<const uint4 *>(row + (size_t)b * 128 + h * 64 + 32 + t * 16);
+        qh[st] = *reinterpret_cast<const uint4 *>(row + lay.off_a + (size_t)b * 64 + h * 32 + t * 16);
+        scv[st] = *reinterpret_cast<const uint2 *>(row + lay.off_b + (size_t)b * 16 + h * 8);
+        dbits[st] = *reinterpret_cast<const uint16_t *>(row + lay.off_c + (size_t)b * 2);
+    }
+    int8_t *sq = reinterpret_cast<int8_t *>(smem_direct);
+    int16_t *sbs = reinterpret_cast<int16_t *>(sq + (size_t)nb * 256);
+    float *sd = reinterpret_cast<float *>(sbs + (size_t)nb * 16);
+#pragma unroll
+    for (int i = 0; i < XB; i++) {
+        const int bq = wave + 4 * i;
+        float d;
+        int s16;
+        const uint32_t packed = quantize_q8_k_lane(xv[i], d, s16);
+        if (bq < nb) {  // uniform across the wavefront
+            reinterpret_cast<uint32_t *>(sq + bq * QK_K)[lane] = packed;
+            if ((lane & 3) == 0) sbs[bq * 16 + (lane >> 2)] = (int16_t)s16;
+            if (lane == 0) sd[bq] = d;
+        }
+    }
+    lds_barrier();  // publishes LDS, does not wait for the weight loads
+
+    const int8_t *abase = sq + b * 256 + h * 128 + t * 16;
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(abase), a1 = *reinterpret_cast<const uint4 *>(abase + 32);
+    const uint4 a2 = *reinterpret_cast<const uint4 *>(abase + 64), a3 = *reinterpret_cast<const uint4 *>(abase + 96);
+    const uint4 bs = *reinterpret_cast<const uint4 *>(sbs + b * 16 + h * 8);
+    const float da = sd[b];
+    const int sh = 16 * t;
+    const int b1 = (int)(int16_t)(bs.x >> sh), b2 = (int)(int16_t)(bs.y >> sh);
+    const int b3 = (int)(int16_t)(bs.z >> sh), b4 = (int)(int16_t)(bs.w >> sh);
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+        int d1 = 0, d2 = 0, d3 = 0, d4 = 0;
+#define FRK_Q6_STEP(c)                                                                                     \
+    d1 = dot4((qla[st].c & 0x0f0f0f0fu) | ((qh[st].c << 4) & 0x30303030u), a0.c, d1);                       \
+    d2 = dot4((qlb[st].c & 0x0f0f0f0fu) | ((qh[st].c << 2) & 0x30303030u), a1.c, d2);                       \
+    d3 = dot4(((qla[st].c >> 4) & 0x0f0f0f0fu) | (qh[st].c & 0x30303030u), a2.c, d3);                       \
+    d4 = dot4(((qlb[st].c >> 4) & 0x0f0f0f0fu) | ((qh[st].c >> 2) & 0x30303030u), a3.c, d4);
+        FRK_Q6_STEP(x)
+        FRK_Q6_STEP(y)
+        FRK_Q6_STEP(z)
+        FRK_Q6_STEP(w)
+#undef FRK_Q6_STEP
+        const uint32_t slo = t ? (scv[st].x >> 8) : scv[st].x, shi = t ? (scv[st].y >> 8) : scv[st].y;
+        const int s1 = (int)(int8_t)(slo & 0xff), s2 = (int)(int8_t)((slo >> 16) & 0xff);
+        const int s3 = (int)(int8_t)(shi & 0xff), s4 = (int)(int8_t)((shi >> 16) & 0xff);
+        const int isum = s1 * (d1 - 32 * b1) + s2 * (d2 - 32 * b2) + s3 * (d3 - 32 * b3) + s4 * (d4 - 32 * b4);
+        float acc = l < units ? (h2f(dbits[st]) * da) * (float)isum : 0.0f;
+        acc = part_sum<LPR>(acc);
+        if (l == 0 && rr[st] < rows_e) y[(size_t)job * rows_e + rr[st]] = acc;
+    }
+}
+
 // ------------------------------------------------------------------ Q8_0 x f32
 // dot_q8_0_f32 (crates/frink-quant/src/lib.rs:663-686) over the planar resident layout.
 // Unit = 16 quants (half a block).
@@ -299,6 +391,29 @@ int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipSt
     else FRK_GO(4, 4);              // nb <= 64
 #undef FRK_GO
     FRK_LAUNCH_CHECK("gemv_q6_k_fused");
+    return FRK_OK;
+}
+
+// expert rows of at most 64 units (4096 columns), at most 16 blocks for the workgroup to quantize
+bool q6_k_experts_gemv_fits(const frk_weights *w) {
+    return w->kind == FRK_KIND_Q6_K && w->cols / QK_K * 4 <= 64;
+}
+// y[j][rows_e] = (rows of expert ids[j]) . (x + j * x_stride) for j < jobs
+int launch_gemv_q6_k_experts(const frk_weights *w, int n_experts, size_t rows_e, const float *x, size_t x_stride,
+                             const int32_t *ids, size_t jobs, float *y, hipStream_t s) {
+    if (jobs > 65535) return set_error(FRK_ERR_SHAPE, "%zu expert jobs exceed the grid", jobs);
+    const int nb = (int)(w->cols / QK_K), units = nb * 4;
+    const size_t shmem = (size_t)nb * (256 + 32 + 4);
+    constexpr int STEPS = 4;
+#define FRK_GO(LPR)                                                                                                    \
+    hipLaunchKernelGGL((gemv_q6_k_experts_kernel<LPR, STEPS>),                                                         \
+                       dim3((unsigned)((rows_e + 4 * (64 / LPR) * STEPS - 1) / (4 * (64 / LPR) * STEPS)), (unsigned)jobs), \
+                       dim3(256), shmem, s, w->dev, w->layout, (int)rows_e, nb, n_experts, ids, x, (int)x_stride, y)
+    if (units <= 16) FRK_GO(16);
+    else if (units <= 32) FRK_GO(32);
+    else FRK_GO(64);
+#undef FRK_GO
+    FRK_LAUNCH_CHECK("gemv_q6_k_experts");
     return FRK_OK;
 }
 

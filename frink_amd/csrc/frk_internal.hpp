@@ -225,6 +225,10 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
 bool direct_gemv_fits(const frk_weights *w);
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+// Q6_K experts stacked in w, one job per (token, slot): y[j][rows_e] = expert ids[j] times x + j * x_stride
+bool q6_k_experts_gemv_fits(const frk_weights *w);
+int launch_gemv_q6_k_experts(const frk_weights *w, int n_experts, size_t rows_e, const float *x, size_t x_stride,
+                             const int32_t *ids, size_t jobs, float *y, hipStream_t s);
 int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // thin batched GEMM of the K-quants: 1 <= batch <= thin_gemm_max_batch(w) rows per launch (0: does not fit)
 int thin_gemm_max_batch(const frk_weights *w);

@@ -396,10 +396,10 @@ int moe_copy_intermediates(void *ws, size_t batch, int k, int n_experts, int hid
 // slot) pair reads its expert's three matrices alone, so the layer is three launches of decode
 // kernels -- gate, up and silu(g)*u of all pairs; down of all pairs, each quantizing its own
 // intermediate; the weighted sum in routing order -- instead of the six of the grouped path.
-// (Q4_K experts throughout: a Q6_K down projection has the grouped kernel only)
+// (Q4_K gate and up experts; the down experts Q4_K, or Q6_K with rows of at most 4096 columns)
 bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind) {
-    return down_kind == FRK_KIND_Q4_K && batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS &&
-           ffn <= FUSED_GEMV_MAX_COLS;
+    const bool down_ok = down_kind == FRK_KIND_Q4_K || (down_kind == FRK_KIND_Q6_K && ffn <= 4096);
+    return down_ok && batch <= MOE_PER_TOKEN_MAX_BATCH && hidden <= FUSED_GEMV_MAX_COLS && ffn <= FUSED_GEMV_MAX_COLS;
 }
 static int launch_moe_ffn_per_token(const frk_weights *gate, const frk_weights *up, const frk_weights *down,
                                     int n_experts, const float *x, size_t batch, const int32_t *ids,
@@ -408,8 +408,10 @@ static int launch_moe_ffn_per_token(const frk_weights *gate, const frk_weights *
     float *act = m.gate_out;  // [batch*k][ffn]
     int rc = launch_gemv_q4_k_experts(gate, up, n_experts, (size_t)ffn, x, (size_t)hidden, ids, batch, (size_t)k, act, s);
     if (rc) return rc;
-    rc = launch_gemv_q4_k_experts(down, nullptr, n_experts, (size_t)hidden, act, (size_t)ffn, ids, batch * (size_t)k, 1,
-                                  m.down_out, s);
+    rc = down->kind == FRK_KIND_Q6_K
+             ? launch_gemv_q6_k_experts(down, n_experts, (size_t)hidden, act, (size_t)ffn, ids, batch * (size_t)k, m.down_out, s)
+             : launch_gemv_q4_k_experts(down, nullptr, n_experts, (size_t)hidden, act, (size_t)ffn, ids, batch * (size_t)k, 1,
+                                        m.down_out, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights,
                        (const int *)nullptr, k, hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);

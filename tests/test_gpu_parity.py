@@ -707,10 +707,12 @@ def test_moe_ffn_matches_the_oracle(fa, n_experts, k, hidden, ffn, batch):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("n_experts,k,hidden,ffn,batch", [(8, 2, 256, 512, 40), (4, 2, 768, 256, 3), (16, 4, 512, 768, 130),
-                                                         (32, 4, 256, 256, 200)])
+                                                         (32, 4, 256, 256, 200), (128, 8, 2048, 768, 1), (16, 4, 512, 768, 16),
+                                                         (8, 2, 256, 4096, 2), (8, 2, 256, 2048, 5)])
 def test_moe_ffn_with_q6_k_down_experts(fa, n_experts, k, hidden, ffn, batch):
-    """Q4_K gate and up, Q6_K down: the down projection runs on the Q6_K matrix-core kernel by token tile
-    (batch 3: grouped although so few tokens)."""
+    """Q4_K gate and up, Q6_K down: the down projection runs on the Q6_K matrix-core kernel by token tile,
+    and for up to 16 tokens as one decode job per (token, slot) on the expert-indexed Q6_K kernel (16, 32 or
+    64 lanes to a row, by the row's length)."""
     _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 7 + batch, down_kind=fo.Q6_K)
 
 
