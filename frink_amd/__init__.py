@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfrink_hip.so")
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
 KIND_NAME = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
 BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}  # (block_bytes, block_elems)
-ACT_F32, ACT_INT8 = 0, 1
+ACT_F32, ACT_INT8, ACT_F32_DOT = 0, 1, 2
 
 OK, ERR_NO_DEVICE, ERR_UNSUPPORTED, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_OOM = 0, -1, -2, -3, -4, -5, -6
 

@@ -225,6 +225,9 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
 bool direct_gemv_fits(const frk_weights *w);
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+// K-quant GEMV on dequantized weights and the f32 activation (the reference's default x86 decode numerics)
+bool kquant_f32_gemv_fits(const frk_weights *w);
+int launch_gemv_kquant_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // Q6_K experts stacked in w, one job per (token, slot): y[j][rows_e] = expert ids[j] times x + j * x_stride
 bool q6_k_experts_gemv_fits(const frk_weights *w);
 int launch_gemv_q6_k_experts(const frk_weights *w, int n_experts, size_t rows_e, const float *x, size_t x_stride,

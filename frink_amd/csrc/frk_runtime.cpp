@@ -460,6 +460,12 @@ static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch
 }
 
 static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mode, hipStream_t s, Scratch &scratch) {
+    if (act_mode == FRK_ACT_F32_DOT && (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K)) {
+        if (!kquant_f32_gemv_fits(w))
+            return set_error(FRK_ERR_UNSUPPORTED, "the f32-dot GEMV of the K-quants takes rows of at most 16384 columns (%zu)", w->cols);
+        return launch_gemv_kquant_f32(w, x, y, s);
+    }
+    if (act_mode == FRK_ACT_F32_DOT) act_mode = FRK_ACT_F32;  // (Q8_0 and Q4_0: their FRK_ACT_F32 is the f32 dot)
     switch (w->kind) {
     case FRK_KIND_Q4_K:
         if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);

@@ -54,7 +54,12 @@ enum { FRK_KIND_Q4_0 = 2, FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q5_K =
  * activation form Avx of crates/frink-quant/src/act_quant.rs:157-189).  The
  * K-quants always take the integer path against Q8_K activations
  * (dot_q4_k_q8 lib.rs:822-869, dot_q6_k_q8 lib.rs:1069-1110). */
-enum { FRK_ACT_F32 = 0, FRK_ACT_INT8 = 1 };
+enum { FRK_ACT_F32 = 0, FRK_ACT_INT8 = 1, FRK_ACT_F32_DOT = 2 };
+/* FRK_ACT_F32_DOT (frk_hip_gemv_dev only): the K-quants multiply their dequantized weights by the f32
+ * activation, the numerics of the reference's default x86 decode path (WeightMatrix::dot,
+ * crates/frink-core/src/weight_matrix.rs:2044-2048; dot_q4_k_f32, dot_q5_k_f32, dot_q6_k_f32,
+ * crates/frink-quant/src/lib.rs:370-415, 461-515, 558-605), within float summation order; rows of at
+ * most 16384 columns.  For Q8_0 and Q4_0 it is FRK_ACT_F32. */
 
 typedef struct frk_weights frk_weights; /* opaque: one weight matrix resident in HBM */
 

@@ -789,6 +789,44 @@ def test_cpp_host_mirror_launches(fa):
     assert r.returncode == 0 and "FAIL" not in r.stdout, r.stdout + r.stderr
 
 
+# ------------------------------------------------------------------ the K-quants' f32 dot (the reference's x86 decode default)
+
+@pytest.mark.parametrize("kind,rows,cols", [
+    (fo.Q4_K, 70, 1024), (fo.Q4_K, 9, 256), (fo.Q4_K, 300, 4096), (fo.Q4_K, 17, 16384),
+    (fo.Q5_K, 70, 1024), (fo.Q5_K, 33, 768), (fo.Q5_K, 128, 4096),
+    (fo.Q6_K, 70, 1024), (fo.Q6_K, 5, 256), (fo.Q6_K, 64, 14336), (fo.Q6_K, 257, 2048),
+])
+def test_k_quant_f32_dot_gemv(fa, kind, rows, cols):
+    """FRK_ACT_F32_DOT: dequantized weights times the f32 activation (dot_q4_k_f32 / dot_q5_k_f32 / dot_q6_k_f32).
+    Against the oracle's f32 dot within the tolerance, and -- what tells it from the integer path, whose
+    activation is rounded to eight bits -- against the product of the dequantized matrix in float64 to
+    within float32 summation error."""
+    from frink_amd import synth
+    print("f32 dot", kind, rows, cols, flush=True)
+    data = make_weights(kind, rows, cols, seed=kind * 31 + rows)
+    x = synth.activations(rows + cols, 1, cols, outlier_frac=0.01)[0]
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    got = w.gemv(to_dev(x), act_mode=fa.ACT_F32_DOT).cpu().numpy()
+    want = fo.gemv(kind, data, rows, cols, x, fo.F32_DOT)
+    assert_rows_close(got[None], want[None], "f32 dot kind %d" % kind)
+    deq = fo.dequant(kind, data).reshape(rows, cols).astype(np.float64)
+    exact = deq @ x.astype(np.float64)
+    bound = 4e-6 * (np.abs(deq) @ np.abs(x).astype(np.float64))
+    assert (np.abs(got - exact) <= bound).all(), float((np.abs(got - exact) / bound).max())
+    ints = w.gemv(to_dev(x)).cpu().numpy()
+    assert (np.abs(ints - exact) > bound).any(), "the integer path is not expected to be this close"
+    w.release()
+
+
+def test_k_quant_f32_dot_refuses_long_rows(fa):
+    data = make_weights(fo.Q4_K, 2, 32768, seed=3)
+    w = fa.Weights.from_host(fo.Q4_K, data, 2, 32768)
+    with pytest.raises(fa.BackendError) as e:
+        w.gemv(to_dev(np.zeros(32768, np.float32)), act_mode=fa.ACT_F32_DOT)
+    assert e.value.code == fa.ERR_UNSUPPORTED
+    w.release()
+
+
 # ------------------------------------------------------------------ thin batched GEMM (batched decode)
 
 @pytest.mark.parametrize("kind,rows,cols,batch", [
