@@ -5,7 +5,7 @@ The compiler does not know that the registers such an instruction names are fill
 it puts between the request and the hand-written s_waitcnt that releases them (a register copy where
 two branches meet, a spill, a multiply it hoisted) reads or overwrites them too early, silently.
 This walks a kernel's assembly along its control flow, keeps two queues of what is in flight
-according to the s_waitcnt bookkeeping -- lgkmcnt for LDS reads, vmcnt for global/buffer/scratch
+according to the s_waitcnt bookkeeping -- lgkmcnt for LDS operations (reads, writes, lane permutes), vmcnt for global/buffer/scratch
 loads, stores and loads that land in LDS (each queue completes in order on this target) -- and
 reports every instruction that touches a register still in flight.  Test infrastructure: nothing in
 the library uses it."""
@@ -98,11 +98,13 @@ def violations(asm_text, kernel):
                 continue
             parts = args.split(",")
             is_vm = op.startswith(_VM_OPS)
-            fills = op.startswith("ds_read") or (is_vm and "_load" in op and "_lds" not in op)
+            is_lds = op.startswith("ds_")  # every LDS operation counts in lgkmcnt, writes and lane permutes included
+            lds_fills = is_lds and any(k in op for k in ("read", "permute", "swizzle", "_rtn", "consume", "append"))
+            fills = lds_fills or (is_vm and "_load" in op and "_lds" not in op)
             writes_first = fills or op.startswith("v_")
             read = _regs(",".join(parts[1:]) if writes_first else args)
             written = _regs(parts[0]) if writes_first else set()
-            own = lds if op.startswith("ds_read") else vm if fills else None
+            own = lds if lds_fills else vm if fills else None
             for queue in (lds, vm):
                 for regs, since in queue:
                     if regs & read:
@@ -110,8 +112,9 @@ def violations(asm_text, kernel):
                     # (a second fill of a register from the same queue lands after the first: in order)
                     if regs & written and queue is not own:
                         found.append("line %d: `%s` overwrites v%d, in flight since line %d" % (n, text, min(regs & written), since))
-            if op.startswith("ds_read"):
-                lds.append((frozenset(written), n))
+            if is_lds:
+                lds.append((frozenset(written), n) if lds_fills else (frozenset(), 0))
+                del lds[:-15]  # (the hardware's counter holds 4 bits)
             elif is_vm:
                 # (what fills no register only counts: its line is left out, so that states that differ
                 # in nothing else are one state; the hardware's counter holds 6 bits)

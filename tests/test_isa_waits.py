@@ -93,3 +93,22 @@ def test_lint_counts_memory_loads_and_loads_into_lds():
     ])
     got = isa_wait_lint.violations(asm, "k")
     assert len(got) == 1 and "line 4" in got[0] and "since line 2" in got[0], got
+
+
+def test_lint_counts_lds_writes_and_permutes():
+    # lgkmcnt(1) behind a read and a write releases the read: the write is the younger operation
+    asm = "\n".join([
+        "k:",
+        "\tds_read_b128 v[4:7], v1 offset:0",
+        "\tds_write_b32 v2, v3",
+        "\ts_waitcnt lgkmcnt(1)",
+        "\tv_add_u32_e32 v30, v4, v9",
+        "\tds_read_b128 v[4:7], v1 offset:0",
+        "\tds_bpermute_b32 v8, v2, v3",
+        "\ts_waitcnt lgkmcnt(1)",
+        "\tv_add_u32_e32 v30, v4, v8",
+        "\ts_endpgm",
+        ".Lfunc_end0:",
+    ])
+    got = isa_wait_lint.violations(asm, "k")
+    assert len(got) == 1 and "line 9" in got[0] and "reads v8" in got[0], got
