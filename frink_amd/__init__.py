@@ -15,8 +15,10 @@ LIB_PATH = os.path.join(_HERE, "lib", "libfrink_hip.so")
 
 # quant kinds (ggml type ids) and their QuantKind::name()
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
-KIND_NAME = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K"}
-BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}  # (block_bytes, block_elems)
+Q5_0, IQ4_XS, MXFP4 = 6, 23, 39
+KIND_NAME = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q5_0: "Q5_0", IQ4_XS: "IQ4_XS", MXFP4: "MXFP4"}
+BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256),
+         Q5_0: (22, 32), IQ4_XS: (136, 256), MXFP4: (17, 32)}  # (block_bytes, block_elems)
 ACT_F32, ACT_INT8, ACT_F32_DOT = 0, 1, 2
 
 OK, ERR_NO_DEVICE, ERR_UNSUPPORTED, ERR_SHAPE, ERR_ARG, ERR_HIP, ERR_OOM = 0, -1, -2, -3, -4, -5, -6

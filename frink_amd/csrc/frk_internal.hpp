@@ -31,14 +31,16 @@ constexpr int Q4_0_BYTES = 18;  // 32 weights, like Q8_0
 constexpr int Q4_K_BYTES = 144;
 constexpr int Q5_K_BYTES = 176;
 constexpr int Q6_K_BYTES = 210;
+constexpr int Q5_0_BYTES = 22, IQ4_XS_BYTES = 136, MXFP4_BYTES = 17;  // 32, 256 and 32 weights
 
 inline int block_bytes(int kind) {
     return kind == FRK_KIND_Q8_0 ? Q8_0_BYTES : kind == FRK_KIND_Q4_0 ? Q4_0_BYTES : kind == FRK_KIND_Q4_K ? Q4_K_BYTES
-         : kind == FRK_KIND_Q5_K ? Q5_K_BYTES : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : 0;
+         : kind == FRK_KIND_Q5_K ? Q5_K_BYTES : kind == FRK_KIND_Q6_K ? Q6_K_BYTES : kind == FRK_KIND_Q5_0 ? Q5_0_BYTES
+         : kind == FRK_KIND_IQ4_XS ? IQ4_XS_BYTES : kind == FRK_KIND_MXFP4 ? MXFP4_BYTES : 0;
 }
 inline int block_elems(int kind) {
-    return (kind == FRK_KIND_Q8_0 || kind == FRK_KIND_Q4_0) ? Q8_0_ELEMS
-         : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K) ? QK_K : 0;
+    return (kind == FRK_KIND_Q8_0 || kind == FRK_KIND_Q4_0 || kind == FRK_KIND_Q5_0 || kind == FRK_KIND_MXFP4) ? Q8_0_ELEMS
+         : (kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_IQ4_XS) ? QK_K : 0;
 }
 
 // ---- resident layouts ----
@@ -78,6 +80,8 @@ inline Layout layout_for(int kind, size_t cols) {
     } else if (kind == FRK_KIND_Q4_0) {
         l.off_a = nb * 16;
         l.row_stride = round_up(l.off_a + nb * 2, 16);
+    } else {  // Q5_0, IQ4_XS, MXFP4: the GGUF bytes in place, rows 16-byte aligned
+        l.row_stride = round_up(nb * (size_t)block_bytes(kind), 16);
     }
     return l;
 }
@@ -225,6 +229,10 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
 bool direct_gemv_fits(const frk_weights *w);
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+// Q5_0, IQ4_XS, MXFP4: dequantizer / row gather and the f32-dot decode GEMV
+bool is_unit_kind(int kind);
+int launch_dequant_units(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s);
+int launch_gemv_units_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // K-quant GEMV on dequantized weights and the f32 activation (the reference's default x86 decode numerics)
 bool kquant_f32_gemv_fits(const frk_weights *w);
 int launch_gemv_kquant_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);

@@ -293,6 +293,7 @@ int launch_repack(int kind, const uint8_t *src, uint8_t *dst, size_t rows, size_
 // out[n_out][cols]: every row of the matrix (ids == nullptr, n_out == rows) or the rows ids[0..n_out)
 int launch_dequant_rows(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s) {
     if (n_out == 0) return FRK_OK;
+    if (is_unit_kind(w->kind)) return launch_dequant_units(w, ids, n_out, out, s);
     const unsigned g = blocks_for(n_out * w->cols, 256);
     switch (w->kind) {
     case FRK_KIND_Q4_K:

@@ -272,6 +272,9 @@ int frk_hip_dense_enabled(void) {
 const char *frk_hip_matvec_kernel(int kind) {
     switch (kind) {
     case FRK_KIND_Q4_0: return "Q4_0";
+    case FRK_KIND_Q5_0: return "Q5_0";
+    case FRK_KIND_IQ4_XS: return "IQ4_XS";
+    case FRK_KIND_MXFP4: return "MXFP4";
     case FRK_KIND_Q8_0: return "Q8_0";
     case FRK_KIND_Q4_K: return "Q4_K";
     case FRK_KIND_Q5_K: return "Q5_K";
@@ -466,6 +469,11 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
         return launch_gemv_kquant_f32(w, x, y, s);
     }
     if (act_mode == FRK_ACT_F32_DOT) act_mode = FRK_ACT_F32;  // (Q8_0 and Q4_0: their FRK_ACT_F32 is the f32 dot)
+    if (is_unit_kind(w->kind)) {
+        if (act_mode != FRK_ACT_F32)
+            return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has the f32-dot GEMV only", w->kind);
+        return launch_gemv_units_f32(w, x, y, s);
+    }
     switch (w->kind) {
     case FRK_KIND_Q4_K:
         if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);

@@ -46,7 +46,12 @@ enum {
 
 /* Quant kinds, numbered by ggml type id (crates/frink-gguf/src/lib.rs:236-242).
  * Names are QuantKind::name() (crates/frink-core/src/weight_matrix.rs:264-290). */
-enum { FRK_KIND_Q4_0 = 2, FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q5_K = 13, FRK_KIND_Q6_K = 14 };
+enum { FRK_KIND_Q4_0 = 2, FRK_KIND_Q5_0 = 6, FRK_KIND_Q8_0 = 8, FRK_KIND_Q4_K = 12, FRK_KIND_Q5_K = 13, FRK_KIND_Q6_K = 14,
+       FRK_KIND_IQ4_XS = 23, FRK_KIND_MXFP4 = 39 };
+/* Q5_0, IQ4_XS and MXFP4 (the 17-byte GGUF block form) have the dequantizer / row gather and the
+ * decode GEMV on the f32 activation (dot_q5_0_f32, dot_iq4_xs_f32, dot_mxfp4_gguf_f32,
+ * crates/frink-quant/src/lib.rs:4380-4418, 4894-4934, 5506); a batch is one such GEMV per row, the
+ * reference's own path below its GEMM threshold (crates/frink-core/src/weight_matrix.rs:2636-2652). */
 
 /* Q8_0 GEMV arithmetic.  F32 multiplies dequantized weights by the f32
  * activation (dot_q8_0_f32, crates/frink-quant/src/lib.rs:663-686); INT8

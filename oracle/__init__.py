@@ -14,10 +14,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libfrink_oracle.so")
 
 Q4_0, Q8_0, Q4_K, Q5_K, Q6_K = 2, 8, 12, 13, 14
+Q5_0, IQ4_XS, MXFP4 = 6, 23, 39  # (dequantizers and f32 dots only)
 FORM_NEON, FORM_AVX, FORM_SCALAR = 0, 1, 2
 F32_DOT, INT_DOT = 0, 1
 
-BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256)}
+BLOCK = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q5_K: (176, 256), Q6_K: (210, 256),
+         Q5_0: (22, 32), IQ4_XS: (136, 256), MXFP4: (17, 32)}
 
 
 def build(force=False):
@@ -76,6 +78,7 @@ def lib():
             "fo_moe_ffn_per_position": (C.c_int, [C.c_int, u8p, u8p, u8p, C.c_int, C.c_int, C.c_int, f32p,
                                                   C.c_int, i32p, f32p, C.c_int, f32p, C.c_int]),
             "fo_have_avx2": (C.c_int, []),
+            "fo_e8m0_scale": (C.c_float, [C.c_uint8]),
             "fo_avx2_gemv_q4_k_f32": (C.c_int, [u8p, sz, sz, f32p, f32p, C.c_int]),
             "fo_avx2_gemm_q4_k_q8k": (C.c_int, [u8p, sz, sz, f32p, sz, f32p, C.c_int]),
         }

@@ -34,6 +34,9 @@
 #define Q5_K_BYTES 176
 #define Q6_K_BYTES 210
 #define QK_K 256
+#define Q5_0_BYTES 22
+#define IQ4_XS_BYTES 136
+#define MXFP4_BYTES 17
 
 /* src/lib.rs:74-75, 180-182, 196-197 */
 int fo_block_bytes(int kind) {
@@ -43,13 +46,16 @@ int fo_block_bytes(int kind) {
     case FO_KIND_Q4_K: return Q4_K_BYTES;
     case FO_KIND_Q5_K: return Q5_K_BYTES;
     case FO_KIND_Q6_K: return Q6_K_BYTES;
+    case FO_KIND_Q5_0: return Q5_0_BYTES;
+    case FO_KIND_IQ4_XS: return IQ4_XS_BYTES;
+    case FO_KIND_MXFP4: return MXFP4_BYTES;
     }
     return 0;
 }
 int fo_block_elems(int kind) {
     switch (kind) {
-    case FO_KIND_Q8_0: case FO_KIND_Q4_0: return Q8_0_ELEMS;
-    case FO_KIND_Q4_K: case FO_KIND_Q5_K: case FO_KIND_Q6_K: return QK_K;
+    case FO_KIND_Q8_0: case FO_KIND_Q4_0: case FO_KIND_Q5_0: case FO_KIND_MXFP4: return Q8_0_ELEMS;
+    case FO_KIND_Q4_K: case FO_KIND_Q5_K: case FO_KIND_Q6_K: case FO_KIND_IQ4_XS: return QK_K;
     }
     return 0;
 }
@@ -233,6 +239,139 @@ int fo_dequant_q6_k(const uint8_t *src, size_t nbytes, float *out) {
     return 0;
 }
 
+/* ---- Q5_0, IQ4_XS, MXFP4 (GGUF block form): dequantizers and f32 dots ---- */
+
+/* src/lib.rs:4346-4350: the fifth bits of elements j and j + 16 of a Q5_0 block, at bit 4 */
+static void q5_fifth_bits(uint32_t qh, int j, uint8_t *xh0, uint8_t *xh1) {
+    *xh0 = (uint8_t)((qh >> j) << 4) & 0x10;
+    *xh1 = (uint8_t)(qh >> (j + 12)) & 0x10;
+}
+/* src/lib.rs:4356-4376: block = [d:f16][qh:u32][16 bytes]; y = (q - 16) * d */
+int fo_dequant_q5_0(const uint8_t *src, size_t nbytes, float *out) {
+    if (nbytes % Q5_0_BYTES) return -1;
+    size_t nb = nbytes / Q5_0_BYTES;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = src + b * Q5_0_BYTES;
+        float d = rd_f16(blk);
+        uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        const uint8_t *qs = blk + 6;
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh0, xh1;
+            q5_fifth_bits(qh, j, &xh0, &xh1);
+            int x0 = (int)((qs[j] & 0x0F) | xh0) - 16, x1 = (int)((qs[j] >> 4) | xh1) - 16;
+            out[b * 32 + j] = (float)x0 * d;
+            out[b * 32 + j + 16] = (float)x1 * d;
+        }
+    }
+    return 0;
+}
+/* src/lib.rs:4396-4418 */
+float fo_dot_q5_0_f32(const uint8_t *row, size_t row_bytes, const float *x) {
+    size_t nb = row_bytes / Q5_0_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * Q5_0_BYTES;
+        float d = rd_f16(blk);
+        uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        const uint8_t *qs = blk + 6;
+        for (int j = 0; j < 16; j++) {
+            uint8_t xh0, xh1;
+            q5_fifth_bits(qh, j, &xh0, &xh1);
+            int x0 = (int)((qs[j] & 0x0F) | xh0) - 16, x1 = (int)((qs[j] >> 4) | xh1) - 16;
+            acc += ((float)x0 * d) * x[b * 32 + j];
+            acc += ((float)x1 * d) * x[b * 32 + j + 16];
+        }
+    }
+    return acc;
+}
+
+/* src/lib.rs:4801-4803 (ggml's kvalues_iq4nl) */
+static const int8_t KVALUES_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+/* src/lib.rs:4860-4890: block = [d:f16][scales_h:u16][scales_l:4][qs:128]; eight sub-blocks of 32, each with a
+ * 6-bit scale ls: y = d * (ls - 32) * kvalues[nibble], low nibbles first then high */
+int fo_dequant_iq4_xs(const uint8_t *src, size_t nbytes, float *out) {
+    if (nbytes % IQ4_XS_BYTES) return -1;
+    size_t nb = nbytes / IQ4_XS_BYTES;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = src + b * IQ4_XS_BYTES;
+        float d = rd_f16(blk);
+        unsigned scales_h = (unsigned)blk[2] | ((unsigned)blk[3] << 8);
+        const uint8_t *scales_l = blk + 4, *qs = blk + 8;
+        for (int ib = 0; ib < 8; ib++) {
+            uint8_t ls = (uint8_t)(((scales_l[ib / 2] >> (4 * (ib % 2))) & 0xf) | (uint8_t)(((scales_h >> (2 * ib)) & 3) << 4));
+            float dl = d * ((float)ls - 32.0f);
+            for (int j = 0; j < 16; j++) {
+                uint8_t byte = qs[ib * 16 + j];
+                out[b * QK_K + ib * 32 + j] = dl * (float)KVALUES_IQ4NL[byte & 0xf];
+                out[b * QK_K + ib * 32 + 16 + j] = dl * (float)KVALUES_IQ4NL[byte >> 4];
+            }
+        }
+    }
+    return 0;
+}
+/* src/lib.rs:4910-4934 */
+float fo_dot_iq4_xs_f32(const uint8_t *row, size_t row_bytes, const float *x) {
+    size_t nb = row_bytes / IQ4_XS_BYTES;
+    float acc = 0.0f;
+    size_t x_base = 0;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * IQ4_XS_BYTES;
+        float d = rd_f16(blk);
+        unsigned scales_h = (unsigned)blk[2] | ((unsigned)blk[3] << 8);
+        const uint8_t *scales_l = blk + 4, *qs = blk + 8;
+        for (int ib = 0; ib < 8; ib++) {
+            uint8_t ls = (uint8_t)(((scales_l[ib / 2] >> (4 * (ib % 2))) & 0xf) | (uint8_t)(((scales_h >> (2 * ib)) & 3) << 4));
+            float dl = d * ((float)ls - 32.0f);
+            for (int j = 0; j < 16; j++) {
+                uint8_t byte = qs[ib * 16 + j];
+                acc += (dl * (float)KVALUES_IQ4NL[byte & 0xf]) * x[x_base + j];
+                acc += (dl * (float)KVALUES_IQ4NL[byte >> 4]) * x[x_base + 16 + j];
+            }
+            x_base += 32;
+        }
+    }
+    return acc;
+}
+
+/* src/lib.rs:4947-4949 (E2M1) and :4960-4966 (E8M0: 2^(e-127), e = 0 the subnormal 2^-127) */
+static const float KVALUES_MXFP4[16] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f,
+                                        -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+float fo_e8m0_scale(uint8_t e) {
+    uint32_t bits = e == 0 ? 0x00400000u : (uint32_t)e << 23;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+/* GGUF block form, src/lib.rs:5560-5570: block = [e:E8M0][16 bytes], low nibble -> element j, high -> j + 16;
+ * the arithmetic of dequant_mxfp4_row (:4980-5003) */
+int fo_dequant_mxfp4(const uint8_t *src, size_t nbytes, float *out) {
+    if (nbytes % MXFP4_BYTES) return -1;
+    size_t nb = nbytes / MXFP4_BYTES;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = src + b * MXFP4_BYTES;
+        float d = fo_e8m0_scale(blk[0]);
+        for (int j = 0; j < 16; j++) {
+            out[b * 32 + j] = d * KVALUES_MXFP4[blk[1 + j] & 0xf];
+            out[b * 32 + 16 + j] = d * KVALUES_MXFP4[blk[1 + j] >> 4];
+        }
+    }
+    return 0;
+}
+/* src/lib.rs:5025-5040, over GGUF blocks */
+float fo_dot_mxfp4_f32(const uint8_t *row, size_t row_bytes, const float *x) {
+    size_t nb = row_bytes / MXFP4_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * MXFP4_BYTES;
+        float d = fo_e8m0_scale(blk[0]);
+        for (int j = 0; j < 16; j++) {
+            acc += (d * KVALUES_MXFP4[blk[1 + j] & 0xf]) * x[b * 32 + j];
+            acc += (d * KVALUES_MXFP4[blk[1 + j] >> 4]) * x[b * 32 + 16 + j];
+        }
+    }
+    return acc;
+}
+
 int fo_dequant(int kind, const uint8_t *src, size_t nbytes, float *out) {
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dequant_q8_0(src, nbytes, out);
@@ -240,6 +379,9 @@ int fo_dequant(int kind, const uint8_t *src, size_t nbytes, float *out) {
     case FO_KIND_Q4_K: return fo_dequant_q4_k(src, nbytes, out);
     case FO_KIND_Q5_K: return fo_dequant_q5_k(src, nbytes, out);
     case FO_KIND_Q6_K: return fo_dequant_q6_k(src, nbytes, out);
+    case FO_KIND_Q5_0: return fo_dequant_q5_0(src, nbytes, out);
+    case FO_KIND_IQ4_XS: return fo_dequant_iq4_xs(src, nbytes, out);
+    case FO_KIND_MXFP4: return fo_dequant_mxfp4(src, nbytes, out);
     }
     return -2;
 }
@@ -1040,6 +1182,9 @@ static inline float row_dot_f32(int kind, const uint8_t *row, size_t row_bytes, 
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_f32(row, row_bytes, x);
     case FO_KIND_Q4_0: return fo_dot_q4_0_f32(row, row_bytes, x);
+    case FO_KIND_Q5_0: return fo_dot_q5_0_f32(row, row_bytes, x);
+    case FO_KIND_IQ4_XS: return fo_dot_iq4_xs_f32(row, row_bytes, x);
+    case FO_KIND_MXFP4: return fo_dot_mxfp4_f32(row, row_bytes, x);
     case FO_KIND_Q4_K: return fo_dot_q4_k_f32(row, row_bytes, x);
     case FO_KIND_Q5_K: return fo_dot_q5_k_f32(row, row_bytes, x);
     default: return fo_dot_q6_k_f32(row, row_bytes, x);
@@ -1052,6 +1197,8 @@ int fo_gemm_rows(int kind, const uint8_t *w, size_t rows, size_t cols, size_t ro
     if (!be || cols == 0 || cols % (size_t)be || row0 + nrows > rows) return -1;
     size_t row_bytes = cols / (size_t)be * (size_t)bb;
     threads = pick_threads(threads);
+    /* (the integer tier of these kinds, crates/frink-quant/src/legacy_q8.rs and iq4_xs_q8.rs, is not restated) */
+    if (mode == FO_MODE_INT_DOT && (kind == FO_KIND_Q5_0 || kind == FO_KIND_IQ4_XS || kind == FO_KIND_MXFP4)) return -4;
     acts_t a = {0, 0, 0};
     if (mode == FO_MODE_INT_DOT) {
         if (acts_alloc(&a, kind, cols, batch)) { acts_free(&a); return -3; }

@@ -22,7 +22,8 @@ extern "C" {
 
 /* quant kinds; the numbers are the ggml type ids the reference maps from
  * (crates/frink-gguf/src/lib.rs:236-242). */
-enum { FO_KIND_Q4_0 = 2, FO_KIND_Q8_0 = 8, FO_KIND_Q4_K = 12, FO_KIND_Q5_K = 13, FO_KIND_Q6_K = 14 };
+enum { FO_KIND_Q4_0 = 2, FO_KIND_Q5_0 = 6, FO_KIND_Q8_0 = 8, FO_KIND_Q4_K = 12, FO_KIND_Q5_K = 13, FO_KIND_Q6_K = 14,
+       FO_KIND_IQ4_XS = 23, FO_KIND_MXFP4 = 39 };
 
 /* Q8_0 activation forms (crates/frink-quant/src/act_quant.rs:121-127). */
 enum { FO_Q8_0_FORM_NEON = 0, FO_Q8_0_FORM_AVX = 1, FO_Q8_0_FORM_SCALAR = 2 };
@@ -42,6 +43,10 @@ int fo_dequant_q4_0(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q4_k(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q5_k(const uint8_t *src, size_t nbytes, float *out);
 int fo_dequant_q6_k(const uint8_t *src, size_t nbytes, float *out);
+int fo_dequant_q5_0(const uint8_t *src, size_t nbytes, float *out);
+int fo_dequant_iq4_xs(const uint8_t *src, size_t nbytes, float *out);
+int fo_dequant_mxfp4(const uint8_t *src, size_t nbytes, float *out); /* GGUF block form: [E8M0][16 nibble bytes] */
+float fo_e8m0_scale(uint8_t e);
 int fo_dequant(int kind, const uint8_t *src, size_t nbytes, float *out);
 /* independent per-element decoders (index formula, not a block walk) */
 float fo_q4_k_element(const uint8_t *block, int i);
@@ -55,6 +60,9 @@ float fo_dot_q4_0_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q4_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q5_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
 float fo_dot_q6_k_f32(const uint8_t *row, size_t row_bytes, const float *x);
+float fo_dot_q5_0_f32(const uint8_t *row, size_t row_bytes, const float *x);
+float fo_dot_iq4_xs_f32(const uint8_t *row, size_t row_bytes, const float *x);
+float fo_dot_mxfp4_f32(const uint8_t *row, size_t row_bytes, const float *x);
 
 /* activation quantizers */
 void fo_quantize_q8_k(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums);

@@ -17,7 +17,9 @@ Sources (paths relative to the reference root):
 * crates/frink-quant/src/encode/q5_k.rs       llama.cpp Q5_K bytes for the k-quant fixture
 * crates/frink-quant/src/encode/q6_k.rs       llama.cpp Q6_K bytes for the k-quant fixture
 * crates/frink-quant/src/encode/testdata.rs   8 real-weight super-blocks (f16 bits)
-* crates/frink-quant/src/lib.rs               Q4_K / Q5_K / Q6_K dequant test blocks + goldens
+* crates/frink-quant/src/lib.rs               Q4_K / Q5_K / Q6_K dequant test blocks + goldens;
+                                              IQ4_XS and MXFP4 (GGUF block form and two-buffer form) test
+                                              blocks + goldens
 """
 import json
 import os
@@ -78,7 +80,16 @@ def main():
         out[blk.lower()] = bytes(ints(lib, blk)).hex()
         out[gold.lower()] = floats(lib, gold)
 
+    for blk, gold in [("IQ4_XS_TEST_BLOCK", "IQ4_XS_GOLDEN"), ("MXFP4_GGUF_TEST_BLOCKS", "MXFP4_GGUF_GOLDEN")]:
+        out[blk.lower()] = bytes(ints(lib, blk)).hex()
+        out[gold.lower()] = floats(lib, gold)
+    out["mxfp4_test_packed"] = bytes(ints(lib, "MXFP4_TEST_PACKED")).hex()
+    out["mxfp4_test_scales"] = bytes(ints(lib, "MXFP4_TEST_SCALES")).hex()
+    out["mxfp4_golden"] = floats(lib, "MXFP4_GOLDEN")
+
     sizes = {
+        "iq4_xs_test_block": 136, "iq4_xs_golden": 256, "mxfp4_gguf_test_blocks": 68, "mxfp4_gguf_golden": 128,
+        "mxfp4_test_packed": 32, "mxfp4_test_scales": 2, "mxfp4_golden": 64,
         "q8_0_encode_golden": 2 * 34, "q8_0_tie_block_f16_bits": 32, "q8_0_tie_block_golden": 34,
         "q4_k_encode_golden": 12 * 144, "q5_k_encode_golden": 12 * 176, "q6_k_encode_golden": 12 * 210,
         "real_weight_blocks_f16_bits": 8 * 256,

@@ -37,14 +37,15 @@ int main(int argc, char **argv) {
         if (Hip::gemm_supported(k)) agree = agree && Hip::has_launch(k);
     }
     CHECK(agree, "matvec_kernel(kind) agrees with has_launch(kind) over all 23 kinds and names the kind");
-    CHECK(claimed == 5 && Hip::has_launch(QuantKind::Q8_0) && Hip::has_launch(QuantKind::Q4K) &&
-              Hip::has_launch(QuantKind::Q5K) && Hip::has_launch(QuantKind::Q6K) && Hip::has_launch(QuantKind::Q4_0),
-          "the five kinds of this path have kernels");
+    CHECK(claimed == 8 && Hip::has_launch(QuantKind::Q8_0) && Hip::has_launch(QuantKind::Q4K) &&
+              Hip::has_launch(QuantKind::Q5K) && Hip::has_launch(QuantKind::Q6K) && Hip::has_launch(QuantKind::Q4_0) &&
+              Hip::has_launch(QuantKind::Q5_0) && Hip::has_launch(QuantKind::IQ4XS) && Hip::has_launch(QuantKind::Mxfp4Gguf),
+          "the eight kinds of this path have kernels");
 
     // None vs Some(Err)
     std::vector<uint8_t> w(34 * 4, 0);
     std::vector<float> x(32, 1.0f);
-    CHECK(!Hip::launch_matvec(QuantKind::Q5_0, w.data(), w.size(), x.data(), x.size(), 4, 34).has_value(),
+    CHECK(!Hip::launch_matvec(QuantKind::Q5_1, w.data(), w.size(), x.data(), x.size(), 4, 34).has_value(),
           "a kind without a kernel is None, not an error");
     auto bad = Hip::launch_matvec(QuantKind::Q8_0, w.data(), w.size(), x.data(), x.size(), 4, 35);
     CHECK(bad.has_value() && bad->is_err() && bad->error().status == FRK_ERR_SHAPE && !bad->error().message.empty(),

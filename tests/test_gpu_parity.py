@@ -789,6 +789,60 @@ def test_cpp_host_mirror_launches(fa):
     assert r.returncode == 0 and "FAIL" not in r.stdout, r.stdout + r.stderr
 
 
+# ------------------------------------------------------------------ Q5_0, IQ4_XS, MXFP4 (GGUF block form)
+
+def _other_kind_blocks(kind, rows, cols, seed):
+    """valid blocks with finite scales and every code value in play (these kinds have no encoder here)"""
+    bb, be = fo.BLOCK[kind]
+    n = rows * cols // be
+    rng = np.random.default_rng(seed)
+    blocks = rng.integers(0, 256, (n, bb), dtype=np.uint8)
+    if kind == fo.MXFP4:
+        blocks[:, 0] = rng.integers(100, 140, n)
+        blocks[0, 0], blocks[1 % n, 0] = 0, 1  # the subnormal scales 2^-127 and 2^-126
+    else:
+        blocks[:, 0:2] = rng.uniform(-0.05, 0.05, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+    return blocks.ravel()
+
+
+@pytest.mark.parametrize("kind,rows,cols", [
+    (fo.Q5_0, 33, 4096), (fo.Q5_0, 5, 32), (fo.Q5_0, 7, 96), (fo.IQ4_XS, 33, 4096), (fo.IQ4_XS, 5, 256), (fo.IQ4_XS, 3, 768),
+    (fo.MXFP4, 33, 4096), (fo.MXFP4, 5, 32), (fo.MXFP4, 9, 2880),
+])
+def test_other_kinds_dequant_and_get_rows_are_bit_exact(fa, kind, rows, cols):
+    import torch
+    data = _other_kind_blocks(kind, rows, cols, seed=kind + rows)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    want = fo.dequant(kind, data).reshape(rows, cols)
+    assert np.array_equal(bits(w.dequant().cpu().numpy()), bits(want))
+    ids = np.array([rows - 1, 0, rows // 2, 0], np.int32)
+    assert np.array_equal(bits(w.get_rows(torch.from_numpy(ids).cuda()).cpu().numpy()), bits(want[ids]))
+    w.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols,batch", [
+    (fo.Q5_0, 70, 1024, 1), (fo.Q5_0, 300, 4096, 3), (fo.IQ4_XS, 70, 1024, 1), (fo.IQ4_XS, 130, 4096, 2), (fo.IQ4_XS, 9, 16384, 1),
+    (fo.MXFP4, 70, 1024, 1), (fo.MXFP4, 64, 2880, 4),
+])
+def test_other_kinds_gemv_matches_the_oracle(fa, kind, rows, cols, batch):
+    """The decode GEMV of Q5_0 / IQ4_XS / MXFP4 is the f32 dot of the reference's decode path; a batch is a GEMV per row."""
+    from frink_amd import synth
+    print("other kinds", kind, rows, cols, batch, flush=True)
+    data = _other_kind_blocks(kind, rows, cols, seed=kind * 3 + rows)
+    x = synth.activations(rows + cols, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy() if batch > 1 else w.gemv(to_dev(x[0])).cpu().numpy()[None]
+    want = fo.gemm(kind, data, rows, cols, x, fo.F32_DOT)
+    assert_rows_close(got, want, "kind %d" % kind)
+    deq = fo.dequant(kind, data).reshape(rows, cols).astype(np.float64)
+    bound = 4e-6 * (np.abs(deq) @ np.abs(x.T).astype(np.float64)).T
+    assert (np.abs(got - (deq @ x.T.astype(np.float64)).T) <= bound).all()
+    with pytest.raises(fa.BackendError) as e:
+        w.gemv(to_dev(x[0]), act_mode=fa.ACT_INT8)
+    assert e.value.code == fa.ERR_UNSUPPORTED
+    w.release()
+
+
 # ------------------------------------------------------------------ the K-quants' f32 dot (the reference's x86 decode default)
 
 @pytest.mark.parametrize("kind,rows,cols", [

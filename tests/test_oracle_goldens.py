@@ -605,3 +605,91 @@ def test_bench_reads_the_host_cpu():
     import bench
     h = bench.host_cpu()
     assert 1 <= h["physical_cores"] <= h["logical_cpus"] and isinstance(h["cpu_model"], str)
+
+
+# ---------------------------------------------------------------- Q5_0, IQ4_XS, MXFP4
+
+def _vectors():
+    import json
+    import os
+    return json.load(open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "frink_quant_vectors.json")))
+
+
+def _random_blocks(kind, n, seed):
+    """valid blocks of Q5_0 / IQ4_XS / MXFP4 with finite scales, all code values in play"""
+    bb, _ = fo.BLOCK[kind]
+    rng = np.random.default_rng(seed)
+    blocks = rng.integers(0, 256, (n, bb), dtype=np.uint8)
+    if kind == fo.MXFP4:
+        blocks[:, 0] = rng.integers(100, 140, n)  # 2^-27 .. 2^12
+    else:
+        blocks[:, 0:2] = rng.uniform(-0.1, 0.1, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+    return blocks
+
+
+def test_iq4_xs_dequant_matches_the_reference_golden():
+    # iq4_xs_dequant_matches_independent_python_reference (crates/frink-quant/src/lib.rs:7480-7490); the golden is
+    # printed to six digits
+    v = _vectors()
+    got = fo.dequant(fo.IQ4_XS, hexbytes(v["iq4_xs_test_block"]))
+    want = np.array(v["iq4_xs_golden"], np.float32)
+    assert np.abs(got - want).max() <= 6e-6 * np.abs(want).max() and np.abs(want).max() > 100
+
+
+def test_mxfp4_dequant_matches_the_reference_goldens():
+    # mxfp4_gguf_dequant_matches_independent_python_reference (lib.rs:7056-7066): powers of two, exact
+    v = _vectors()
+    got = fo.dequant(fo.MXFP4, hexbytes(v["mxfp4_gguf_test_blocks"]))
+    assert np.array_equal(got, np.array(v["mxfp4_gguf_golden"], np.float32))
+    # the two-buffer form's vectors (mxfp4_dequant_matches_independent_python_reference, lib.rs:7588-7599) through the block
+    # form: scale bytes 0x00 (the subnormal 2^-127) and 0x82
+    packed, scales = hexbytes(v["mxfp4_test_packed"]).reshape(2, 16), hexbytes(v["mxfp4_test_scales"])
+    blocks = np.concatenate([np.concatenate([[scales[i]], packed[i]]) for i in range(2)]).astype(np.uint8)
+    got = fo.dequant(fo.MXFP4, blocks)
+    want = np.array(v["mxfp4_golden"], np.float64)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max() and np.abs(got[:32]).max() < 1e-37
+    # mxfp4_scale_byte_zero_and_max_match_the_e8m0_formula (lib.rs:7613-7620)
+    assert fo.lib().fo_e8m0_scale(0) == 2.0 ** -127 and fo.lib().fo_e8m0_scale(127) == 1.0 and fo.lib().fo_e8m0_scale(254) == 2.0 ** 127
+
+
+def test_q5_0_known_answers():
+    # q5_0_fifth_bit_extends_range_past_a_plain_nibble (lib.rs:5886-5910)
+    blk = np.zeros(22, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blk[2] = 1
+    blk[6] = 0x0F
+    out = fo.dequant(fo.Q5_0, blk)
+    assert out[0] == 15.0 and (out[1:] == -16.0).all()
+    # every element from the published layout by index arithmetic: q = nibble | bit (j or j + 16) of qh << 4
+    blocks = _random_blocks(fo.Q5_0, 50, 5)
+    got = fo.dequant(fo.Q5_0, blocks.ravel()).reshape(50, 32)
+    for b in range(50):
+        d = np.float32(blocks[b, 0:2].copy().view(np.float16)[0])
+        qh = int(blocks[b, 2:6].copy().view(np.uint32)[0])
+        for i in range(32):
+            nib = (blocks[b, 6 + i % 16] >> (4 * (i // 16))) & 15
+            q = int(nib) | (((qh >> i) & 1) << 4)
+            assert got[b, i] == np.float32(q - 16) * d
+
+
+@pytest.mark.parametrize("kind", [fo.Q5_0, fo.IQ4_XS, fo.MXFP4])
+def test_f32_dots_of_the_other_kinds_are_the_dequantized_dot(kind):
+    # (the reference's *_fused_dot_matches_dequant_then_dot tests, lib.rs:7068-7082, 7492-7502): the fused dot adds the
+    # same products left to right, so it equals the dequantized row's sequential f32 dot bit for bit
+    bb, be = fo.BLOCK[kind]
+    cols = 1024
+    blocks = _random_blocks(kind, 6 * cols // be, 11 + kind)
+    x = np.random.default_rng(kind).standard_normal(cols).astype(np.float32)
+    got = fo.gemv(kind, blocks.ravel(), 6, cols, x, fo.F32_DOT, 1)
+    deq = fo.dequant(kind, blocks.ravel()).reshape(6, cols)
+    for r in range(6):
+        acc = np.float32(0)
+        if kind == fo.Q5_0 or kind == fo.MXFP4 or kind == fo.IQ4_XS:
+            # element pairs (j, j + 16) of each group of 32, in that order
+            for g in range(cols // 32):
+                for j in range(16):
+                    acc = np.float32(acc + deq[r, 32 * g + j] * x[32 * g + j])
+                    acc = np.float32(acc + deq[r, 32 * g + 16 + j] * x[32 * g + 16 + j])
+        assert got[r] == acc
+    with pytest.raises(ValueError):
+        fo.gemv(kind, blocks.ravel(), 6, cols, x, fo.INT_DOT, 1)
