@@ -346,6 +346,20 @@ def main():
             for w in w2:
                 w.release()
         out["roofline_gemm"] = gemm_records
+        # Q5_K at M=512: the thin matrix-core kernel as a grid of 16-row groups, one launch
+        d5g = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=84)).to(dev)
+        w5 = [fa.Weights.from_device(fa.Q5_K, d5g, rows, cols) for _ in range(4)]
+        yb5 = torch.empty((512, rows), dtype=torch.float32, device=dev)
+
+        def step3e(i):
+            w5[i % 4].gemm(xb, out=yb5)
+        _, t = time_graph(torch, step3e, 40, 20)
+        tops = 2.0 * 512 * rows * cols / (t / 40) / 1e12
+        extra["Q5_K GEMM M=512 14336x4096 (16-row groups, one launch)"] = {
+            "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        for w in w5:
+            w.release()
+        del d5g, yb5
         # the FFN down projection of a Q4_K_M model at M=512: Q6_K on the matrix cores
         d6g = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=78)).to(dev)
         w6 = [fa.Weights.from_device(fa.Q6_K, d6g, cols, rows) for _ in range(4)]

@@ -361,6 +361,13 @@ __global__ __launch_bounds__(64 * TM_WAVES) __attribute__((amdgpu_waves_per_eu(2
                                                                         const int16_t *__restrict__ absums,
                                                                         float *__restrict__ y) {
     constexpr int KS = TM_WAVES / RG;
+    // a batch wider than ACTS is a grid of groups of ACTS activation rows: blockIdx.y picks the group
+    // (every group streams the weights again, out of L2 after the first)
+    aq += (size_t)blockIdx.y * ACTS * nb * QK_K;
+    ad += (size_t)blockIdx.y * ACTS * nb;
+    absums += (size_t)blockIdx.y * ACTS * nb * 16;
+    y += (size_t)blockIdx.y * ACTS * rows;
+    batch = min(ACTS, batch - (int)blockIdx.y * ACTS);
     constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES;  // bytes of a block
     constexpr int PR = BB / 16, NP = 16 * PR;         // 16-byte pieces of a row's block, of 16 rows' blocks
     constexpr int QS = Q5 ? 48 : 16;                  // where the nibbles start
@@ -991,7 +998,8 @@ static int launch_thin_mfma_kind(const frk_weights *w, int batch, Q8KActs a, flo
         sized = true;
     }
     const size_t groups = (w->rows + 15) / 16;
-    hipLaunchKernelGGL((thin_mfma_q4_k_kernel<RG, ACTS, Q5>), dim3((unsigned)((groups + RG - 1) / RG)), dim3(64 * TM_WAVES),
+    hipLaunchKernelGGL((thin_mfma_q4_k_kernel<RG, ACTS, Q5>), dim3((unsigned)((groups + RG - 1) / RG), (unsigned)((batch + ACTS - 1) / ACTS)),
+                       dim3(64 * TM_WAVES),
                        shmem, s, w->dev, w->layout.row_stride, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d,
                        a.bsums, y);
     FRK_LAUNCH_CHECK("thin mfma gemm");
@@ -1094,12 +1102,15 @@ int thin_gemm_max_batch(const frk_weights *w) {
     return 0;
 }
 
-// A batch of any width in one launch, where the kind has a kernel that takes one (Q6_K on the matrix
-// cores: a grid of 8-row groups); 0 rows = no such kernel for this matrix.
+// A batch of any width in one launch, where the kind has a kernel that takes one (Q6_K and Q5_K on the
+// matrix cores: a grid of 8- and 16-row groups); 0 rows = no such kernel for this matrix.
 int thin_gemm_wide_rows(const frk_weights *w) {
+    if (w->kind == FRK_KIND_Q5_K && thin_mfma_acts(w) >= 16) return 65535 * 16;  // (groups of 16 rows)
     return (w->kind == FRK_KIND_Q6_K && thin_mfma6_acts(w) >= 8) ? 65535 * 8 : 0;
 }
 int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    // Q5_K: many groups of activation rows fill the chip whatever the matrix, so a workgroup takes eight row groups
+    if (w->kind == FRK_KIND_Q5_K) return launch_thin_mfma<8, 16>(w, batch, a, y, s);
     return launch_thin_mfma6_rg<8>(w, batch, a, y, s);
 }
 

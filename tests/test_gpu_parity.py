@@ -272,14 +272,15 @@ def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
 def test_q5_k_decode_and_batches_at_full_size(fa):
     """Q5_K (Q4_K's scale packing, a fifth bit per code from a separate plane): the FFN shape with
     arbitrary block bytes (every bit pattern of the fifth-bit plane) against the oracle on slices of
-    rows, for one row (the decode kernel), 3, 16 and 17 rows (the thin matrix-core kernel, 16 rows a
-    launch), and the whole output of a row against dequantized weights in float64."""
+    rows, for one row (the decode kernel), 3, 16, 17 and 70 rows (the thin matrix-core kernel: 16 rows
+    a workgroup, wider batches as a grid of 16-row groups in one launch, the last group ragged), and the
+    whole output of a row against dequantized weights in float64."""
     from frink_amd import synth
     rows, cols = 14336, 4096
     data = _random_q5_k(rows, cols, 41)
     w = fa.Weights.from_host(fo.Q5_K, data, rows, cols)
-    x = synth.activations(42, 17, cols, outlier_frac=0.01)
-    for batch in (1, 3, 16, 17):
+    x = synth.activations(42, 70, cols, outlier_frac=0.01)
+    for batch in (1, 3, 16, 17, 70):
         print("q5_k batch", batch, flush=True)
         got = w.gemm(to_dev(x[:batch])).cpu().numpy()
         assert got.shape == (batch, rows)
@@ -295,7 +296,8 @@ def test_q5_k_decode_and_batches_at_full_size(fa):
     w.release()
 
 
-@pytest.mark.parametrize("rows,cols,batch", [(72, 512, 2), (33, 768, 5), (100, 256, 16), (50, 2048, 9), (20, 14336, 4)])
+@pytest.mark.parametrize("rows,cols,batch", [(72, 512, 2), (33, 768, 5), (100, 256, 16), (50, 2048, 9), (20, 14336, 4),
+                                             (72, 512, 33), (40, 1024, 130)])
 def test_q5_k_thin_batches_on_ragged_shapes(fa, rows, cols, batch):
     from frink_amd import synth
     data = make_weights(fo.Q5_K, rows, cols, seed=rows + cols)
