@@ -286,20 +286,22 @@ __global__ __launch_bounds__(256) void gemv_q8_0_f32_direct_kernel(const uint8_t
 // consecutive; LDS reads are inline assembly so that the compiler does not wait for the weight
 // loads in front of them (it cannot tell the two apart from the global_load_lds).
 typedef float v4f_t __attribute__((ext_vector_type(4)));
-template <int U>
-__global__ __launch_bounds__(1024) void gemv_q8_0_f32_shared_kernel(const uint8_t *__restrict__ W, Layout lay,
-                                                                    int rows, int nb, const float *__restrict__ x,
-                                                                    float *__restrict__ y) {
+template <int U, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_q8_0_f32_shared_kernel(const uint8_t *__restrict__ W, Layout lay,
+                                                                          int rows, int nb, const float *__restrict__ x,
+                                                                          float *__restrict__ y) {
     extern __shared__ uint4 smem_direct[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = min((int)blockIdx.x * 16 + wave, rows - 1);
-    const bool store = (int)blockIdx.x * 16 + wave < rows;
+    const int r = min((int)blockIdx.x * WAVES + wave, rows - 1);
+    const bool store = (int)blockIdx.x * WAVES + wave < rows;
     const uint8_t *row = W + (size_t)r * lay.row_stride;
     const int units = nb * 2;
-    {
-        const int slot = min(wave * 64 + lane, 4 * units - 1);  // wavefronts past the end repeat the last slot
+#pragma unroll
+    for (int i = 0; i < (4 * U + WAVES - 1) / WAVES; i++) {  // the activation's 4 U KB at most: a KB a wavefront and round
+        const int chunk = min(wave + i * WAVES, 4 * U - 1);  // (a wavefront past the end repeats the last chunk)
+        const int slot = min(chunk * 64 + lane, 4 * units - 1);  // slots past the end repeat the last slot
         const int k = slot / units, u = slot - k * units;
-        load_to_lds16(x + (size_t)(4 * u + k) * 4, reinterpret_cast<uint8_t *>(smem_direct) + wave * 1024);
+        load_to_lds16(x + (size_t)(4 * u + k) * 4, reinterpret_cast<uint8_t *>(smem_direct) + chunk * 1024);
     }
     asm volatile("" ::: "memory");  // the weight loads below are issued after it: the wait counts on that
     uint4 qv[U];
@@ -357,7 +359,8 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_f32_shared_kernel(const uint8_
 // rows of at most 64*4 units, and long enough that a wavefront per row is not mostly idle lanes
 bool direct_gemv_fits(const frk_weights *w) {
     const size_t units = w->kind == FRK_KIND_Q6_K ? w->cols / QK_K * 4 : w->cols / Q8_0_ELEMS * 2;
-    return (w->kind == FRK_KIND_Q6_K || w->kind == FRK_KIND_Q8_0) && units > 32 && units <= 256;
+    // (Q8_0: up to eight units a lane, 8192 columns)
+    return (w->kind == FRK_KIND_Q6_K || w->kind == FRK_KIND_Q8_0) && units > 32 && units <= (w->kind == FRK_KIND_Q8_0 ? 512u : 256u);
 }
 
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
@@ -420,15 +423,18 @@ int launch_gemv_q6_k_experts(const frk_weights *w, int n_experts, size_t rows_e,
 int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / Q8_0_ELEMS);
     const int u = (nb * 2 + 63) / 64;
-    if (w->rows >= 1024) {  // enough rows that 16-row workgroups still cover the CUs
-        const dim3 grid((unsigned)((w->rows + 15) / 16)), block(1024);
+    if (w->rows >= 1024) {  // enough rows that these workgroups still cover the CUs
+        constexpr int WAVES = 8;  // (two workgroups to a CU: 5.75 us at 4096x4096 against 6.1 with sixteen wavefronts and 5.96 with four)
+        const dim3 grid((unsigned)((w->rows + WAVES - 1) / WAVES)), block(64 * WAVES);
 #define FRK_GO(UU)                                                                                                \
-    hipLaunchKernelGGL(gemv_q8_0_f32_shared_kernel<UU>, grid, block, 16384, s, w->dev, w->layout, (int)w->rows, nb, \
+    hipLaunchKernelGGL((gemv_q8_0_f32_shared_kernel<UU, WAVES>), grid, block, 4096 * UU, s, w->dev, w->layout, (int)w->rows, nb, \
                        x, y)
         if (u == 1) FRK_GO(1);
         else if (u == 2) FRK_GO(2);
         else if (u == 3) FRK_GO(3);
-        else FRK_GO(4);
+        else if (u == 4) FRK_GO(4);
+        else if (u <= 6) FRK_GO(6);
+        else FRK_GO(8);
 #undef FRK_GO
         FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");
         return FRK_OK;
@@ -439,7 +445,9 @@ int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, 
     if (u == 1) FRK_GO(1);
     else if (u == 2) FRK_GO(2);
     else if (u == 3) FRK_GO(3);
-    else FRK_GO(4);
+    else if (u == 4) FRK_GO(4);
+    else if (u <= 6) FRK_GO(6);
+    else FRK_GO(8);
 #undef FRK_GO
     FRK_LAUNCH_CHECK("gemv_q8_0_f32_direct");
     return FRK_OK;

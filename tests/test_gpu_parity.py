@@ -197,6 +197,8 @@ GEMV_SHAPES = [
     (fo.Q5_K, 64, 4096), (fo.Q5_K, 37, 4096), (fo.Q5_K, 19, 2048), (fo.Q5_K, 21, 768), (fo.Q5_K, 9, 256), (fo.Q5_K, 6, 14336),
     (fo.Q6_K, 48, 14336), (fo.Q6_K, 13, 4096), (fo.Q6_K, 11, 768), (fo.Q6_K, 9, 256), (fo.Q6_K, 5, 2048),
     (fo.Q8_0, 64, 4096), (fo.Q8_0, 7, 32), (fo.Q8_0, 9, 544), (fo.Q8_0, 5, 2048),
+    (fo.Q8_0, 1030, 4096), (fo.Q8_0, 1025, 8192), (fo.Q8_0, 40, 8192), (fo.Q8_0, 1100, 5120), (fo.Q8_0, 33, 6144),
+    (fo.Q8_0, 12, 16384),
 ]
 
 
