@@ -94,6 +94,16 @@ struct BPlanes {
 struct RawBlock {  // header + the lane's 16-byte half of each 32-byte nibble pair, as read from LDS
     v4i wh, q0, q1, q2, q3;
 };
+// Q5_K: the same block with a fifth bit per weight -- byte l of the 32 bytes behind the header holds weight l of
+// every sub-block, sub-block j in bit j (dot_q5_k_q8, crates/frink-quant/src/lib.rs:886-938); fh is the lane's
+// 16-byte half of them.  With q5 = q4 + 16 * bit the scaled weight is sc * q5 = 8 * H + L + 16 * P for a third
+// int8 plane P = sc * bit (0 .. 63): three chains of MFMAs, S1 = 8 * (2 * acc_P + acc_H) + acc_L.
+struct FifthBits {
+    v4i fh;
+};
+struct PPlanes {
+    v4i P0, P1, P2, P3, P4, P5, P6, P7;
+};
 struct TileOperands {  // one 32-token tile of a block: 8 k-slices of quants and the bsums
     v4i a0, a1, a2, a3, a4, a5, a6, a7;
     v8h bs;
@@ -146,6 +156,11 @@ __device__ __forceinline__ void wait_scales(TileScales &S) {
 template <int N>
 __device__ __forceinline__ void wait_raw(RawBlock &R) {
     asm volatile("s_waitcnt lgkmcnt(%5)" : "+v"(R.wh), "+v"(R.q0), "+v"(R.q1), "+v"(R.q2), "+v"(R.q3) : "n"(N));
+}
+__device__ __forceinline__ void read_fifth(FifthBits &F, uint32_t addr) { FRK_DS_READ(F.fh, addr, 0); }
+template <int N>
+__device__ __forceinline__ void wait_raw5(RawBlock &R, FifthBits &F) {
+    asm volatile("s_waitcnt lgkmcnt(%6)" : "+v"(R.wh), "+v"(R.q0), "+v"(R.q1), "+v"(R.q2), "+v"(R.q3), "+v"(F.fh) : "n"(N));
 }
 template <int N>
 __device__ __forceinline__ void wait_vm() {
@@ -214,6 +229,29 @@ __device__ __forceinline__ void unpack_block(const RawBlock &R, int lg, BPlanes 
     unpack_pair(R.q2, s.sc_hi, B.H4, B.L4, B.H5, B.L5);
     unpack_pair(R.q3, s.sc_hi >> 16, B.H6, B.L6, B.H7, B.L7);
     unpack_rest(R, s, lg, B);
+}
+
+// the third plane of Q5_K: sub-block j's scale where the weight's fifth bit is set (bytes 0 or sc <= 63)
+__device__ __forceinline__ void unpack_fifth(const RawBlock &R, const FifthBits &F, PPlanes &P) {
+    const BlockScales s = block_scales(R);
+    auto plane = [&](int j) {
+        const unsigned short sc = (unsigned short)(((j < 4 ? s.sc_lo : s.sc_hi) >> (8 * (j & 3))) & 0xff);
+        const us2 scs = {sc, sc};
+        v4i o;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t bits = ((uint32_t)F.fh[c] >> j) & 0x01010101u;
+            us2 b;
+            __builtin_memcpy(&b, &bits, 4);
+            const us2 r = b * scs;  // 0x0101 * sc: both bytes sc, no carry between them
+            int ri;
+            __builtin_memcpy(&ri, &r, 4);
+            o[c] = ri;
+        }
+        return o;
+    };
+    P.P0 = plane(0), P.P1 = plane(1), P.P2 = plane(2), P.P3 = plane(3);
+    P.P4 = plane(4), P.P5 = plane(5), P.P6 = plane(6), P.P7 = plane(7);
 }
 
 __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales &S, const BPlanes &B, v16f &acc) {
@@ -321,8 +359,9 @@ __device__ __forceinline__ void fold_mins(BPlanes &B) {
 // (they are read by an epilogue that may run a step later), the raw weights in ONE slot per
 // wavefront: a block leaves its slot for registers at the end of the step before it is multiplied,
 // and the slot is refilled at once.  One barrier per step.
-template <int RG, int KS, int MT>
+template <int RG, int KS, int MT, bool Q5 = false>
 struct PipeLds {
+    static constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES;  // bytes of a weight block
     static constexpr int NW = RG * KS;
     static constexpr int NT = KS * MT;  // tile slots of a stage
     static constexpr int OFF_BS = NT * 8192;
@@ -331,7 +370,7 @@ struct PipeLds {
     static constexpr int OFF_DA = A_STAGES * A_STAGE;
     static constexpr int DA_STAGE = NT * 128, DA_STAGES = 4;
     static constexpr int OFF_W = OFF_DA + DA_STAGES * DA_STAGE;
-    static constexpr int W_SLOT = 32 * Q4_K_BYTES;
+    static constexpr int W_SLOT = 32 * BB;
     static constexpr size_t BYTES = (size_t)OFF_W + (size_t)NW * W_SLOT;
 };
 
@@ -386,10 +425,35 @@ template <int N, class V>
 __device__ __forceinline__ void wait_lgkm(V &reg, v16i &acc) {
     asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(reg), "+v"(acc) : "n"(N));
 }
-template <int EXTRA, class Between, class Next>
-__device__ __forceinline__ v16i tile_chain(TileOperands &T, const BPlanes &B, Between between, Next next) {
+// (Q5_K: the chain of the fifth bits' plane runs first, each of its MFMAs waiting for its operand; the sum is
+// doubled and the two chains below follow with every operand there.)
+template <int EXTRA>
+__device__ __forceinline__ v16i fifth_chain(TileOperands &T, const PPlanes &P) {
     const v16i zi = {0};
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(T.a0) : "n"(8 + EXTRA));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, P.P0, zi, 0, 0, 0);
+    wait_lgkm<7 + EXTRA>(T.a1, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, P.P1, acc, 0, 0, 0);
+    wait_lgkm<6 + EXTRA>(T.a2, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, P.P2, acc, 0, 0, 0);
+    wait_lgkm<5 + EXTRA>(T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, P.P3, acc, 0, 0, 0);
+    wait_lgkm<4 + EXTRA>(T.a4, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, P.P4, acc, 0, 0, 0);
+    wait_lgkm<3 + EXTRA>(T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, P.P5, acc, 0, 0, 0);
+    wait_lgkm<2 + EXTRA>(T.a6, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, P.P6, acc, 0, 0, 0);
+    wait_lgkm<1 + EXTRA>(T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, P.P7, acc, 0, 0, 0);
+    return acc << 1;
+}
+// SEEDED: the running sum starts from `seed` (the doubled sum of the fifth bits' chain) and every operand has
+// landed already.
+template <int EXTRA, bool SEEDED = false, class Between, class Next>
+__device__ __forceinline__ v16i tile_chain(TileOperands &T, const BPlanes &B, Between between, Next next, v16i seed = v16i{0}) {
+    const v16i zi = seed;
+    if (!SEEDED) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(T.a0) : "n"(8 + EXTRA));
     v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
     between(0);
     wait_lgkm<7 + EXTRA>(T.a1, acc);
@@ -464,9 +528,12 @@ __device__ __forceinline__ void tail_piece(int i, TileTail &E, const BPlanes &B,
     }
 }
 
-template <int RG, int KS, int MT>
+template <int RG, int KS, int MT, bool Q5 = false>
 __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
-    using L = PipeLds<RG, KS, MT>;
+    using L = PipeLds<RG, KS, MT, Q5>;
+    constexpr int BB = L::BB, PR = BB / 16;          // bytes of a block, its 16-byte pieces
+    constexpr int NC = (32 * PR + 63) / 64;          // requests that move a wavefront's 32 rows of a block (the last: half)
+    static_assert(32 * PR == 64 * (NC - 1) + 32, "the last request of a block is 32 lanes wide");
     constexpr int NW = L::NW, NT = L::NT, ROWS = 32 * RG, TM = 32 * MT;
     static_assert(NW == 8 && NT == 4, "eight wavefronts share the four tile slots of a stage");
     extern __shared__ uint4 smem_gemm[];
@@ -508,12 +575,12 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
     // that LDS holds the rows back to back (144 bytes each).  Rows past the matrix read its last row.
     const uint32_t stride = (uint32_t)g.row_stride;
     const int row_base = min(row_tile * ROWS + rg * 32, g.rows - 1);
-    uint32_t w_off[5];
+    uint32_t w_off[NC];
 #pragma unroll
-    for (int c = 0; c < 5; c++) {
+    for (int c = 0; c < NC; c++) {
         const int p = 64 * c + lane;
-        const int r = min(p / 9, g.rows - 1 - row_base);
-        w_off[c] = (uint32_t)r * stride + (uint32_t)(p % 9) * 16;
+        const int r = min(p / PR, g.rows - 1 - row_base);
+        w_off[c] = (uint32_t)r * stride + (uint32_t)(p % PR) * 16;
     }
     const uint8_t *Wrow = g.W + (size_t)row_base * stride;
     const uint32_t lds_w = lds0 + L::OFF_W + wave * L::W_SLOT;
@@ -531,18 +598,36 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
             dma4(lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + slot_d * 128, Db + rec * 128, lane_d);
         }
     };
-    auto fetch_weights = [&](int i) {  // five requests
-        const uint8_t *src = Wrow + (size_t)block_of(ks, i) * Q4_K_BYTES;
+    auto fetch_weights = [&](int i) {  // NC requests
+        const uint8_t *src = Wrow + (size_t)block_of(ks, i) * BB;
 #pragma unroll
-        for (int c = 0; c < 4; c++) dma16(lds_w + c * 1024, src, w_off[c]);
-        if (lane < 32) dma16(lds_w + 4096, src, w_off[4]);
+        for (int c = 0; c < NC - 1; c++) dma16(lds_w + c * 1024, src, w_off[c]);
+        if (lane < 32) dma16(lds_w + (NC - 1) * 1024, src, w_off[NC - 1]);
     };
 
     v16f sum[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) sum[mt] = v16f{0.0f};
     BPlanes B;
+    PPlanes P;  // (Q5_K only)
     RawBlock R;
+    FifthBits F;
+    // a raw block leaves this wavefront's slot for registers (Q5_K: the nibbles sit behind the 32 bytes of fifth bits)
+    auto read_block = [&]() {
+        const uint32_t wa = lds_w + li * BB;
+        read_raw(R, wa, wa + (Q5 ? 32 : 0) + 16 * lg);
+        if (Q5) {
+            read_fifth(F, wa + 16 + 16 * lg);
+            wait_raw5<0>(R, F);
+        } else {
+            wait_raw<0>(R);
+        }
+    };
+    auto unpack = [&]() {
+        unpack_block(R, lg, B);
+        if (Q5) unpack_fifth(R, F, P);
+        fold_mins(B);
+    };
 
     // prologue: activations of steps 0 and 1, weights of step 0; then the weights of step 1
 #pragma unroll
@@ -563,13 +648,10 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
     wait_vm<0>();
     lds_barrier();
     {
-        const uint32_t wa = lds_w + li * Q4_K_BYTES;
-        read_raw(R, wa, wa + 16 * lg);
-        wait_raw<0>(R);
+        read_block();
         if (steps > 1) fetch_weights(1);
         if (is_active(0)) read_tile<0>(T, quants_of(0), sums_of(0));
-        unpack_block(R, lg, B);
-        fold_mins(B);
+        unpack();
     }
 
     for (int i = 0; i < steps; i++) {
@@ -609,7 +691,10 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
                     }
                 };
                 // (a tile after the first finds four more reads behind its sums: the scales of the tile before)
-                const v16i s1 = tile_chain<(mt > 0 ? 4 : 0)>(T, B, between, next);
+                constexpr int EXTRA = mt > 0 ? 4 : 0;
+                v16i s1;
+                if constexpr (Q5) s1 = tile_chain<EXTRA, true>(T, B, between, next, fifth_chain<EXTRA>(T, P));
+                else s1 = tile_chain<EXTRA>(T, B, between, next);
                 E.s1 = s1;
                 E.bs = T.bs;
                 if (mt + 1 < MT) {
@@ -636,14 +721,11 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
             // the activations of step i+2, younger than they, may stay in flight
             if (more_acts) wait_vm<6>();
             else wait_vm<0>();
-            const uint32_t wa = lds_w + li * Q4_K_BYTES;
-            read_raw(R, wa, wa + 16 * lg);
-            wait_raw<0>(R);
+            read_block();
             if (more_acts) fetch_weights(i + 2);
             lds_barrier();
             if (is_active(i + 1)) read_tile<0>(T, quants_of(i + 1), sums_of(i + 1));
-            unpack_block(R, lg, B);
-            fold_mins(B);
+            unpack();
         } else {
             lds_barrier();
         }
@@ -974,18 +1056,18 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         if (e_ != hipSuccess) return set_error(FRK_ERR_HIP, what " launch: %s", hipGetErrorString(e_)); \
     } while (0)
 
-template <int RG, int KS, int MT>
+template <int RG, int KS, int MT, bool Q5 = false>
 static int launch_pipe(const GemmArgs &g, unsigned grid, hipStream_t s) {
-    constexpr size_t shmem = PipeLds<RG, KS, MT>::BYTES;
+    constexpr size_t shmem = PipeLds<RG, KS, MT, Q5>::BYTES;
     static_assert(shmem <= 160 * 1024, "LDS of a CU");
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_pipe_kernel<RG, KS, MT>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_pipe_kernel<RG, KS, MT, Q5>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemm_q4_k_pipe_kernel<RG, KS, MT>), dim3(grid, (unsigned)g.k_split), dim3(512), shmem, s, g);
+    hipLaunchKernelGGL((gemm_q4_k_pipe_kernel<RG, KS, MT, Q5>), dim3(grid, (unsigned)g.k_split), dim3(512), shmem, s, g);
     FRK_LAUNCH_CHECK("gemm_q4_k_pipe");
     if (g.k_split > 1) return launch_sum_parts(g.partial, g.k_split, (size_t)g.M * g.rows, g.y, s);
     return FRK_OK;
@@ -1035,16 +1117,17 @@ constexpr int Q4K_MAX_SPLIT = 4;
 struct Q4KPlan {
     int rows_wg, tok_wg, k_split;
 };
-static Q4KPlan q4_k_plan(size_t rows, size_t M, size_t nb) {
-    if (M > 64 && ((rows + 255) / 256) * ((M + 127) / 128) >= 200) return {256, 128, 1};
+static Q4KPlan q4_k_plan(size_t rows, size_t M, size_t nb, bool q5 = false) {
+    // (Q5_K: the third plane's 32 registers fit the 128 x 64 form only)
+    if (!q5 && M > 64 && ((rows + 255) / 256) * ((M + 127) / 128) >= 200) return {256, 128, 1};
     const size_t grid = (((rows + 127) / 128 + 7) / 8 * 8) * ((M + 63) / 64);
     int ks = 1;
     while (ks < Q4K_MAX_SPLIT && grid * (size_t)ks * 2 <= 256 && nb / (size_t)(ks * 2) >= 4) ks *= 2;
     return {128, 64, ks};
 }
 // the tiled activations, then room for the parts' sums where the blocks are split
-size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
-    const Q4KPlan p = q4_k_plan(rows, M, cols / QK_K);
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows, bool q5) {
+    const Q4KPlan p = q4_k_plan(rows, M, cols / QK_K, q5);
     return round_up(q8k_tiled_bytes(M, cols), 256) + (p.k_split > 1 ? (size_t)p.k_split * M * rows * sizeof(float) : 0);
 }
 
@@ -1062,11 +1145,13 @@ int launch_gemm_q4_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *
     g.M = (int)M;
     g.y = y;
     g.partial = partial;
-    const Q4KPlan p = q4_k_plan(w->rows, M, (size_t)g.nb);
+    const bool q5 = w->kind == FRK_KIND_Q5_K;
+    const Q4KPlan p = q4_k_plan(w->rows, M, (size_t)g.nb, q5);
     g.row_tiles = (int)((w->rows + p.rows_wg - 1) / p.rows_wg);
     g.tok_tiles = (int)((M + p.tok_wg - 1) / p.tok_wg);
     g.k_split = p.k_split;
     const unsigned grid = (unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles);
+    if (q5) return launch_pipe<4, 2, 2, true>(g, grid, s);
     return p.rows_wg == 256 ? launch_pipe<8, 1, 4>(g, grid, s) : launch_pipe<4, 2, 2>(g, grid, s);
 }
 
@@ -1076,6 +1161,7 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
     if (rc) return rc;
     return launch_gemm_q4_k_acts(w, acts, M, y, reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256)), s);
 }
+// (Q5_K weights take the same entry points: launch_gemm_q4_k_acts looks at the kind)
 
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
                             const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,

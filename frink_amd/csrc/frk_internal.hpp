@@ -181,8 +181,9 @@ int launch_quantize_q8_k_tiled(const float *x, size_t rows, size_t cols, Q8KTile
 // max_rows rows whose first entry is not negative
 int launch_quantize_q8_k_gather(const float *x, size_t cols, const int *gather, size_t max_rows, Q8KTiled out,
                                 hipStream_t s);
-// batched GEMM on the int8 matrix cores (Q4_K); ws must hold gemm_q4_k_workspace_bytes(M, cols)
-size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows);
+// batched GEMM on the int8 matrix cores (Q4_K, and Q5_K with q5 set: its fifth bits are a third plane of
+// the same kernel); ws must hold gemm_q4_k_workspace_bytes(M, cols, rows, kind is Q5_K)
+size_t gemm_q4_k_workspace_bytes(size_t M, size_t cols, size_t rows, bool q5 = false);
 int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 // the same over activations already quantized into the tiled form; `partial` holds the parts' sums of a split
 int launch_gemm_q4_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *y, float *partial, hipStream_t s);

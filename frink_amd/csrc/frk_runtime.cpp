@@ -537,11 +537,18 @@ static bool q4_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
     const size_t q4k_thin_rows = 32;
     return w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16);
 }
+// Q5_K: the same kernel with a third plane for the fifth bits, from the batch on where it is ahead of the
+// thin kernel's 16-row groups
+static bool q5_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
+    const size_t q5k_thin_rows = 32;
+    return w->kind == FRK_KIND_Q5_K && batch > q5k_thin_rows;
+}
 
 static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
-    if (q4_k_takes_the_matrix_cores(w, batch)) {
+    if (q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch)) {  // (frk_hip_gemm_pair_dev: the same test)
         void *ws = nullptr;
-        int rc = scratch.get(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
+        int rc = scratch.get(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows, w->kind == FRK_KIND_Q5_K),
+                             (hipStream_t)stream, &ws);
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
@@ -621,11 +628,12 @@ int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const fl
         return set_error(FRK_ERR_SHAPE, "the matrices have %zu and %zu columns: they share one batch of activations", w0->cols, w1->cols);
     hipStream_t s = (hipStream_t)stream;
     Scratch scratch;
-    if (q4_k_takes_the_matrix_cores(w0, batch) && q4_k_takes_the_matrix_cores(w1, batch)) {
+    auto tiled = [&](const frk_weights *w) { return q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch); };
+    if (tiled(w0) && tiled(w1)) {
         // one quantization into the tiled form, then the two GEMMs (each with its own room for a split's parts)
         const size_t acts_bytes = round_up(q8k_tiled_bytes(batch, w0->cols), 256);
-        const size_t part0 = gemm_q4_k_workspace_bytes(batch, w0->cols, w0->rows) - acts_bytes;
-        const size_t part1 = gemm_q4_k_workspace_bytes(batch, w1->cols, w1->rows) - acts_bytes;
+        const size_t part0 = gemm_q4_k_workspace_bytes(batch, w0->cols, w0->rows, w0->kind == FRK_KIND_Q5_K) - acts_bytes;
+        const size_t part1 = gemm_q4_k_workspace_bytes(batch, w1->cols, w1->rows, w1->kind == FRK_KIND_Q5_K) - acts_bytes;
         void *ws = nullptr;
         int rc = scratch.get(acts_bytes + round_up(part0, 256) + part1, s, &ws);
         if (rc) return rc;

@@ -274,15 +274,16 @@ def test_host_buffer_launch_matvec_is_the_drop_in(fa, kind):
 def test_q5_k_decode_and_batches_at_full_size(fa):
     """Q5_K (Q4_K's scale packing, a fifth bit per code from a separate plane): the FFN shape with
     arbitrary block bytes (every bit pattern of the fifth-bit plane) against the oracle on slices of
-    rows, for one row (the decode kernel), 3, 16, 17 and 70 rows (the thin matrix-core kernel: 16 rows
-    a workgroup, wider batches as a grid of 16-row groups in one launch, the last group ragged), and the
-    whole output of a row against dequantized weights in float64."""
+    rows, for one row (the decode kernel), 3, 16, 17 and 32 rows (the thin matrix-core kernel: 16 rows
+    a workgroup, wider batches as a grid of 16-row groups in one launch), 33, 70 and 512 rows (the tiled
+    matrix-core kernel with the fifth bits as a third int8 plane, its blocks split between workgroups for
+    the small batches), and the whole output of a row against dequantized weights in float64."""
     from frink_amd import synth
     rows, cols = 14336, 4096
     data = _random_q5_k(rows, cols, 41)
     w = fa.Weights.from_host(fo.Q5_K, data, rows, cols)
-    x = synth.activations(42, 70, cols, outlier_frac=0.01)
-    for batch in (1, 3, 16, 17, 70):
+    x = synth.activations(42, 512, cols, outlier_frac=0.01)
+    for batch in (1, 3, 16, 17, 32, 33, 70, 512):
         print("q5_k batch", batch, flush=True)
         got = w.gemm(to_dev(x[:batch])).cpu().numpy()
         assert got.shape == (batch, rows)
@@ -299,7 +300,8 @@ def test_q5_k_decode_and_batches_at_full_size(fa):
 
 
 @pytest.mark.parametrize("rows,cols,batch", [(72, 512, 2), (33, 768, 5), (100, 256, 16), (50, 2048, 9), (20, 14336, 4),
-                                             (72, 512, 33), (40, 1024, 130)])
+                                             (72, 512, 33), (40, 1024, 130), (200, 768, 130), (257, 1024, 200),
+                                             (13000, 512, 300), (129, 256, 65)])
 def test_q5_k_thin_batches_on_ragged_shapes(fa, rows, cols, batch):
     from frink_amd import synth
     data = make_weights(fo.Q5_K, rows, cols, seed=rows + cols)
@@ -1205,6 +1207,8 @@ def test_dev_calls_on_two_streams_from_two_threads(fa):
     ((fo.Q4_K, fo.Q4_K), (96, 256), 2048, 40),     # the blocks split between workgroups: each GEMM its own parts
     ((fo.Q4_K, fo.Q4_K), (64, 64), 512, 8),        # thin kernel
     ((fo.Q4_K, fo.Q6_K), (128, 96), 1024, 64),     # kinds that do not share a quantized form
+    ((fo.Q5_K, fo.Q4_K), (200, 136), 1024, 70),    # Q5_K's three planes beside Q4_K's two, one quantization
+    ((fo.Q5_K, fo.Q5_K), (96, 160), 2048, 40),     # both with their blocks split
 ])
 def test_gemm_pair_is_two_gemms_over_one_quantization(fa, kinds, rows, cols, batch):
     """frk_hip_gemm_pair_dev (apply_batch_pair_with_acts, weight_matrix.rs:2447-2479): bit for bit the two
