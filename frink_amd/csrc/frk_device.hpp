@@ -124,6 +124,46 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// expf the way glibc computes it (2.28 and later, every architecture: sysdeps/ieee754/flt-32/e_expf.c, the
+// algorithm of ARM's optimized routines): in double, exp(x) = 2^(k/32) * 2^(r/32) with k = round(32 x / ln 2),
+// 2^(k/32) from a table of 32 correctly rounded values (the exponent added to the table entry's bits) and a
+// cubic for the rest, rounded to f32 once.  Rust's f32::exp is the platform's expf (the reference's silu:
+// crates/frink-core/src/matmul.rs:634-650), so this returns a Linux host's bits (a build of glibc that fuses
+// the cubic's multiply-adds differs in the double's last bits, which reaches the f32 in about one value in
+// 2^29) at a third of the instructions of a correctly rounded double exp.  Outside |x| < 88 (where glibc
+// handles overflow, underflow and NaN separately) the double exp rounds to the same values.
+__constant__ const uint64_t EXPF_TABLE[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+// (`table`: EXPF_TABLE or a copy of it, e.g. in LDS for a kernel that evaluates many)
+__device__ __forceinline__ float expf_as_libm(float x, const uint64_t *table = EXPF_TABLE) {
+    if (!(fabsf(x) < 88.0f)) return (float)exp((double)x);
+    constexpr double N = 32.0;
+    constexpr double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
+    constexpr double INV_LN2_N = 0x1.71547652b82fep+0 * N, SHIFT = 0x1.8p+52;
+    const double z = INV_LN2_N * (double)x;
+    double kd = z + SHIFT;  // the integer nearest to z sits in the low bits
+    const uint64_t ki = (uint64_t)__double_as_longlong(kd);
+    kd -= SHIFT;
+    const double r = z - kd;
+    const double s = __longlong_as_double((long long)(table[ki & 31] + (ki << 47)));
+    const double p = C0 * r + C1;
+    const double r2 = r * r;
+    double y = C2 * r + 1.0;
+    y = p * r2 + y;
+    return (float)(y * s);
+}
+// x * sigmoid(x) as the reference's hosts compute it: x / (1 + expf(-x)), each step rounded to f32
+__device__ __forceinline__ float silu_as_host(float x, const uint64_t *table = EXPF_TABLE) {
+    return __fdiv_rn(x, 1.0f + expf_as_libm(-x, table));
+}
+
 // quantize_activations_q8_k (crates/frink-quant/src/act_quant.rs:69-104) for one 256-value block
 // held four consecutive values per lane by one wavefront.  Returns the lane's four quants packed
 // little-endian; d_out is the block scale (same in every lane); bsum16 is the sum of the 16-wide
@@ -155,7 +195,7 @@ __device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, i
 }
 
 // One record of the tiled Q8_K form (32 rows x one 256-wide block) by a workgroup of WAVES wavefronts
-// (4 or 16): wavefront w quantizes rows 32/WAVES * w .. (`load(r)` returns this lane's four values of
+// (4, 8 or 16): wavefront w quantizes rows 32/WAVES * w .. (`load(r)` returns this lane's four values of
 // row r, zeros for a row that does not exist; all of a wavefront's loads are in flight before its
 // first row is quantized), the record is put together in LDS and leaves as three contiguous copies
 // -- quantizing straight into the tiled form would write it in 4-byte pieces.  These kernels are

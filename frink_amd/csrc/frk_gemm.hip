@@ -80,6 +80,10 @@ struct StreamArgs {
     const int4 *tiles;  // {expert, 32 * t, rows in use, 0}
     const int *n_tiles;
     int row_tiles;  // ceil(rows / 256)
+    // the gathering form: the activations are the source rows' Q8_K, quantized once each, and row r of the
+    // grouped order is source row gather[r] (negative: a row not in use)
+    Q8KRows src;
+    const int *gather;
 };
 
 // One block of a lane's weight row as MFMA B operands: the two pre-scaled planes of the 8 sub-blocks,
@@ -773,6 +777,11 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
 // times, one before its MFMAs and one after: a wavefront is stalled while its loads wait for the
 // CU's address unit, and this way the other one has the matrix core meanwhile.
 // Items of a tile sit on one XCD (block id mod 8), whose L2 then serves the tile's activations.
+// GATHER: a tile's activation rows are fetched from where their source rows were quantized (plain rows,
+// each quantized once however many tiles it is part of) instead of from a record of the grouped order: a
+// lane's piece of a record is 16 bytes of one row in either form, so only the lane offsets differ -- the
+// source row times the row length, looked up per item from a table in LDS.
+template <bool GATHER>
 struct StreamLds {
     static constexpr int RG = 8;
     static constexpr int W_WAVE = 32 * Q4_K_BYTES;  // a wavefront's 32 rows of one block
@@ -787,12 +796,17 @@ struct StreamLds {
     // item change costs no global load (whose completion would count in vmcnt, in the middle of the
     // prefetch bookkeeping)
     static constexpr int OFF_ITEMS = OFF_A + A_STAGES * A_STAGE;
-    static constexpr int MAX_ITEMS = 128;
-    static constexpr size_t BYTES = (size_t)OFF_ITEMS + MAX_ITEMS * 8;
+    static constexpr int MAX_ITEMS = GATHER ? 64 : 128;
+    // GATHER: the source rows of each item's tile, row r of the first half in the low 16 bits of word r and
+    // row 32 + r in the high ones
+    static constexpr int OFF_SRC = OFF_ITEMS + MAX_ITEMS * 8;
+    static constexpr size_t BYTES = (size_t)OFF_SRC + (GATHER ? MAX_ITEMS * 128 : 0);
+    static_assert(BYTES <= 160 * 1024, "LDS of a CU");
 };
 
-__global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(StreamArgs g) {
-    using L = StreamLds;
+template <bool GATHER>
+__global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
+    using L = StreamLds<GATHER>;
     extern __shared__ uint4 smem_gemm[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -825,6 +839,14 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
             const int4 ti = g.tiles[xcd + 8 * ((slot + i * per_xcd) / per_tile)];
             table[i] = make_int2(ti.x, ti.z);
         }
+        if (GATHER) {
+            uint32_t *src_rows = reinterpret_cast<uint32_t *>(lds + L::OFF_SRC);
+            for (int i = tid; i < my_items * 32; i += 64 * L::RG) {
+                const int t = xcd + 8 * ((slot + (i >> 5) * per_xcd) / per_tile), r = i & 31;
+                const int a = g.gather[t * MOE_TILE + r], b = g.gather[t * MOE_TILE + 32 + r];
+                src_rows[i] = (uint32_t)max(a, 0) | ((uint32_t)max(b, 0) << 16);  // (a row not in use: any row will do)
+            }
+        }
         __syncthreads();
     }
     const uint32_t lds_items = lds_address(lds + L::OFF_ITEMS);
@@ -853,6 +875,8 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
     };
     const uint8_t *f_w, *f_x;
     const int8_t *f_q;
+    uint32_t f_src = 0;  // GATHER: this lane's source rows of the cursor's tile (row lane % 32 of either half)
+    const uint32_t lds_src = lds_address(lds + L::OFF_SRC);
     int f_ord = 0, f_kb = 0, f_step = 0;
     bool f_two = false;  // the cursor's tile has rows in its second half
     int issued = 0;      // loads of the fetch most recently issued by this wavefront
@@ -864,14 +888,40 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         const int l = opaque_lane();
         w_off0 = (uint32_t)(rg * (32 * L::RG) + wave * 32 + l / 9) * (uint32_t)g.row_stride + (uint32_t)(l % 9) * 16;
         f_two = count > 32;
-        const size_t rec = (size_t)(2 * t + (wave >> 1 & 1)) * nb;  // the small piece's half
-        f_q = g.a.q + (size_t)2 * t * nb * 8192;
-        f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.a.bs + rec * 512)
-                     : reinterpret_cast<const uint8_t *>(g.a.d + rec * 32);
+        if (GATHER) {
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(f_src) : "v"(lds_src + ord * 128 + (l & 31) * 4));
+            f_q = g.src.q;
+            f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.src.bs) : reinterpret_cast<const uint8_t *>(g.src.d);
+        } else {
+            const size_t rec = (size_t)(2 * t + (wave >> 1 & 1)) * nb;  // the small piece's half
+            f_q = g.a.q + (size_t)2 * t * nb * 8192;
+            f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.a.bs + rec * 512)
+                         : reinterpret_cast<const uint8_t *>(g.a.d + rec * 32);
+        }
     };
     auto fetch_acts = [&]() {  // of the cursor's step
         uint8_t *st = lds + L::OFF_A + (f_step & 3) * L::A_STAGE;
         const int l = opaque_lane();
+        if (GATHER) {
+            // piece (row, 16-byte half hk) of quant slice `wave`: bytes 32 * wave + 16 * hk of the row's block;
+            // of the sums: 16 * hk of the block's 32 bytes; the scale: the block's 4 bytes
+            const uint32_t row_a = f_src & 0xffffu, row_b = f_src >> 16, hk = (uint32_t)(l >> 5) * 16;
+            const uint32_t cols = (uint32_t)nb * QK_K;
+            load_to_lds16(f_q + (row_a * cols + (uint32_t)wave * 32 + hk), st + wave * 1024);
+            issued = 1;
+            if (f_two) {
+                load_to_lds16(f_q + (row_b * cols + (uint32_t)wave * 32 + hk), st + L::A_HALF + wave * 1024);
+                issued = 2;
+            }
+            if (wave < 2 || (wave < 4 && f_two)) {
+                uint8_t *half = st + (wave >> 1) * L::A_HALF;
+                const uint32_t row = (wave >> 1) ? row_b : row_a;
+                if (x_sums) load_to_lds16(f_x + (row * (uint32_t)nb * 32 + hk), half + L::A_BS);
+                else load_to_lds4(f_x + row * (uint32_t)nb * 4, half + L::A_DA);
+                issued++;
+            }
+            return;
+        }
         const uint32_t q_off = (uint32_t)(wave * 1024 + l * 16);
         const uint32_t x_off = x_sums ? (uint32_t)l * 16 : (uint32_t)(l & 31) * 4;
         load_to_lds16(f_q + q_off, st + wave * 1024);
@@ -901,8 +951,8 @@ __global__ __launch_bounds__(64 * StreamLds::RG) void gemm_q4_k_stream_kernel(St
         issued += 5;
         f_step++;
         f_w += Q4_K_BYTES;
-        f_q += 8192;
-        f_x += x_sums ? 1024 : 128;
+        f_q += GATHER ? QK_K : 8192;
+        f_x += GATHER ? (x_sums ? 32 : 4) : (x_sums ? 1024 : 128);
         if (++f_kb == nb) {
             f_kb = 0;
             if (++f_ord < my_items) point_at(f_ord);
@@ -1163,9 +1213,39 @@ int launch_gemm_q4_k(const frk_weights *w, const float *x, size_t M, float *y, v
 }
 // (Q5_K weights take the same entry points: launch_gemm_q4_k_acts looks at the kind)
 
+template <bool GATHER>
+static int launch_stream(const StreamArgs &g, int max_tiles, hipStream_t s) {
+    using L = StreamLds<GATHER>;
+    static int grid = 0;
+    if (grid == 0) {
+        int dev = 0, cus = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_stream_kernel<GATHER>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)L::BYTES);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "gemm_q4_k_stream setup: %s", hipGetErrorString(e));
+        grid = cus < 8 ? 8 : cus / 8 * 8;  // one workgroup per CU, a multiple of the 8 XCDs
+    }
+    // more workgroups than CUs when a workgroup's share of the largest possible list would not fit
+    // its item table
+    const size_t most_items = ((size_t)max_tiles + 7) / 8 * g.n_mat * g.row_tiles;
+    const unsigned rounds = (unsigned)((most_items + (size_t)(grid / 8) * L::MAX_ITEMS - 1) /
+                                       ((size_t)(grid / 8) * L::MAX_ITEMS));
+    hipLaunchKernelGGL(gemm_q4_k_stream_kernel<GATHER>, dim3((unsigned)grid * (rounds ? rounds : 1)), dim3(64 * L::RG),
+                       L::BYTES, s, g);
+    FRK_LAUNCH_CHECK("gemm_q4_k_stream");
+    return FRK_OK;
+}
+
+bool gemm_q4_k_stream_gathers(size_t src_rows, size_t cols) {
+    // a source row is a 16-bit entry of the kernel's table, a row's place a 32-bit lane offset
+    return src_rows <= 65535 && src_rows * cols < (1ull << 32);
+}
+
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
-                            const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,
-                            hipStream_t s) {
+                            const Q8KRows *src, const int *gather, const int4 *tiles, const int *n_tiles,
+                            int max_tiles, float *y0, float *y1, hipStream_t s) {
     StreamArgs g;
     g.W[0] = w0->dev;
     g.W[1] = w1 ? w1->dev : w0->dev;
@@ -1179,26 +1259,9 @@ int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t
     g.tiles = tiles;
     g.n_tiles = n_tiles;
     g.row_tiles = (int)((rows_e + 255) / 256);
-    static int grid = 0;
-    if (grid == 0) {
-        int dev = 0, cus = 0;
-        hipError_t e = hipGetDevice(&dev);
-        if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-        if (e == hipSuccess)
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4_k_stream_kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)StreamLds::BYTES);
-        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "gemm_q4_k_stream setup: %s", hipGetErrorString(e));
-        grid = cus < 8 ? 8 : cus / 8 * 8;  // one workgroup per CU, a multiple of the 8 XCDs
-    }
-    // more workgroups than CUs when a workgroup's share of the largest possible list would not fit
-    // its item table
-    const size_t most_items = ((size_t)max_tiles + 7) / 8 * g.n_mat * g.row_tiles;
-    const unsigned rounds = (unsigned)((most_items + (size_t)(grid / 8) * StreamLds::MAX_ITEMS - 1) /
-                                       ((size_t)(grid / 8) * StreamLds::MAX_ITEMS));
-    hipLaunchKernelGGL(gemm_q4_k_stream_kernel, dim3((unsigned)grid * (rounds ? rounds : 1)), dim3(64 * StreamLds::RG),
-                       StreamLds::BYTES, s, g);
-    FRK_LAUNCH_CHECK("gemm_q4_k_stream");
-    return FRK_OK;
+    g.src = src ? *src : Q8KRows{nullptr, nullptr, nullptr};
+    g.gather = gather;
+    return src ? launch_stream<true>(g, max_tiles, s) : launch_stream<false>(g, max_tiles, s);
 }
 
 }  // namespace frk

@@ -303,9 +303,7 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
 #pragma unroll
                 for (int j = 0; j < J2; j++) up += q4_k_unit_dot(vh[k][j], v0[k][j], v1[k][j], v2[k][j], v3[k][j], U[j]);
                 up = part_sum<LPR>(up);
-                // exp in double, rounded once: what a host libm's expf returns in all but a vanishing
-                // share of cases, so a quantizer downstream sees the same input as the reference's
-                acc = __fdiv_rn(acc, 1.0f + (float)exp(-(double)acc)) * up;
+                acc = silu_as_host(acc) * up;  // (a host's bits: a quantizer downstream sees the reference's input)
             }
             if (MULTI) {
                 float *out = ma.y[0];

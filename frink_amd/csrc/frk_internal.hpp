@@ -173,6 +173,13 @@ struct Q8KTiled {
     _Float16 *bs;
     float *d;
 };
+// Q8_K of plain rows, each quantized once: q [row][cols], bs [row][block][16] (the 16-wide sums as f16),
+// d [row][block]
+struct Q8KRows {
+    int8_t *q;
+    _Float16 *bs;
+    float *d;
+};
 size_t q8k_tiled_bytes(size_t rows, size_t cols);
 Q8KTiled q8k_tiled_carve(void *base, size_t rows, size_t cols);
 // out row r = x[r] quantized, r < rows; the rest of the last tile becomes zeros
@@ -213,9 +220,13 @@ constexpr size_t MOE_PER_TOKEN_MAX_BATCH = 16;
 // add up in ascending expert id; smaller batches run per position and add up in routing order.
 constexpr size_t MOE_BUCKET_ORDER_FROM = 32;
 bool moe_takes_per_token_path(size_t batch, size_t hidden, size_t ffn, int down_kind);
+// The grouped Q4_K GEMM over the tile list (one matrix, or two that share the activations).  The activations
+// are `a`, quantized in the grouped order, or -- with `src` -- the source rows' Q8_K and `gather`, the source
+// row of every row of the grouped order (gemm_q4_k_stream_gathers tells whether the kernel can address them).
+bool gemm_q4_k_stream_gathers(size_t src_rows, size_t cols);
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
-                            const int4 *tiles, const int *n_tiles, int max_tiles, float *y0, float *y1,
-                            hipStream_t s);
+                            const Q8KRows *src, const int *gather, const int4 *tiles, const int *n_tiles,
+                            int max_tiles, float *y0, float *y1, hipStream_t s);
 // MoE expert FFN over stacked Q4_K experts; ws must hold moe_workspace_bytes(...)
 size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);
 int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,

@@ -22,7 +22,7 @@ __global__ __launch_bounds__(64) void route_top_k_softmax_kernel(const float *__
     float mx = -INFINITY;
     for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, l[i]);
     mx = wave_max(mx);
-    for (int i = lane; i < n_experts; i += 64) prob[i] = expf(l[i] - mx);
+    for (int i = lane; i < n_experts; i += 64) prob[i] = expf_as_libm(l[i] - mx);  // (a host's bits, as the reference's f32::exp gives them)
     __syncthreads();
     if (lane == 0) {
         float sum = 0.0f;
@@ -111,11 +111,20 @@ struct GroupLds {
     int tile_big[1024], n_big[1024], tile_small[1024], seg_sum[1024];  // first heavy tile, their number, the light tile
     int wave_tot[16];
 };
-__global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restrict__ ids, int pairs, int k,
-                                                         int n_experts, int *__restrict__ group_off,
-                                                         int *__restrict__ gather, int *__restrict__ pos_of,
-                                                         int *__restrict__ cpos_of, int4 *__restrict__ tiles,
-                                                         int *__restrict__ n_tiles, int max_rows) {
+struct GroupArgs {
+    const int32_t *ids;
+    int pairs, k, n_experts;
+    int *group_off, *gather, *pos_of, *cpos_of;
+    int4 *tiles;
+    int *n_tiles;
+    int max_rows;
+};
+__device__ __forceinline__ void moe_group(const GroupArgs &a) {
+    const int32_t *__restrict__ ids = a.ids;
+    const int pairs = a.pairs, k = a.k, n_experts = a.n_experts, max_rows = a.max_rows;
+    int *__restrict__ group_off = a.group_off, *__restrict__ gather = a.gather, *__restrict__ pos_of = a.pos_of;
+    int *__restrict__ cpos_of = a.cpos_of, *__restrict__ n_tiles = a.n_tiles;
+    int4 *__restrict__ tiles = a.tiles;
     extern __shared__ uint4 smem_group[];
     GroupLds &L = *reinterpret_cast<GroupLds *>(smem_group);
     const int tid = threadIdx.x;
@@ -216,25 +225,55 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
         __syncthreads();
     }
 }
+__global__ __launch_bounds__(1024) void moe_group_kernel(GroupArgs a) { moe_group(a); }
+
+// The bucketing and the quantization of the token rows do not depend on each other: in one launch, workgroup
+// 0 buckets while the others quantize (quantize_activations_q8_k, crates/frink-quant/src/act_quant.rs:69-104;
+// a wavefront per 256-value block) every token row ONCE, into plain rows that the grouped GEMM gathers from
+// -- instead of a launch that waits for the bucketing and then quantizes every (token, slot) pair's copy.
+__global__ __launch_bounds__(1024) void moe_group_quantize_kernel(GroupArgs a, const float *__restrict__ x, int n_blocks,
+                                                                  Q8KRows out) {
+    if (blockIdx.x == 0) {
+        moe_group(a);
+        return;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int b = ((int)blockIdx.x - 1) * 16 + wave; b < n_blocks; b += ((int)gridDim.x - 1) * 16) {
+        const float4 v = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K)[lane];
+        float dd;
+        int bs;
+        const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
+        reinterpret_cast<uint32_t *>(out.q + (size_t)b * QK_K)[lane] = packed;
+        if ((lane & 3) == 0) out.bs[(size_t)b * 16 + (lane >> 2)] = (_Float16)bs;
+        if (lane == 0) out.d[b] = dd;
+    }
+}
 
 // GluAct::Swiglu (crates/frink-core/src/matmul.rs:634-650): act = gate / (1 + exp(-gate)) * up, quantized
 // straight to Q8_K in the tiled form -- the down projection quantizes its own input in the
 // reference too (ffn_batch.rs:405-415).  One workgroup per record (32 rows of the grouped order x
-// one block); rows in a gap become zeros, records without rows in use are skipped (a record's rows
-// in use come first, so its first row tells).
-__global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__restrict__ gate,
-                                                              const float *__restrict__ up, int nb,
-                                                              const int *__restrict__ gather, Q8KTiled out) {
+// one block), eight wavefronts of four rows each (measured at 512 tokens x top-8 of 128 experts, 2048/768:
+// 12.8 us; sixteen wavefronts 13.6, four 16.2 -- the kernel is about as long as one wavefront's chain of
+// tile entry -> loads -> exponentials -> record, times the rounds its workgroups need to become resident).
+// Rows past a tile's rows in use become zeros, records without rows in use are skipped.
+constexpr int SWIGLU_WAVES = 8;
+__global__ __launch_bounds__(64 * SWIGLU_WAVES) void swiglu_quantize_kernel(const float *__restrict__ gate,
+                                                                            const float *__restrict__ up, int nb,
+                                                                            const int4 *__restrict__ tiles,
+                                                                            const int *__restrict__ n_tiles, Q8KTiled out) {
     __shared__ Q8KRecordLds L;
     const int t32 = blockIdx.x / nb, kb = blockIdx.x % nb, lane = threadIdx.x & 63;
-    if (gather[t32 * 32] < 0) return;  // rows in use come first in a tile
-    // exp in double, rounded once to f32: the correctly rounded value, which is what a host libm's
-    // expf returns in all but a vanishing share of cases, so the quantizer sees the same input
-    auto silu = [](float x) { return __fdiv_rn(x, 1.0f + (float)exp(-(double)x)); };
-    quantize_q8k_record<4>(out, (size_t)t32 * nb + kb, L, [&](int r) {
-        const int row = t32 * 32 + r;
-        if (gather[row] < 0) return make_float4(0.f, 0.f, 0.f, 0.f);
-        const size_t src = ((size_t)row * nb + kb) * QK_K;
+    static_assert(MOE_TILE == 64, "a tile is two records");
+    const int4 tile = tiles[t32 >> 1];  // (the list is as long as the grid needs, entries past *n_tiles unwritten)
+    const int used = t32 >> 1 < *n_tiles ? tile.z - 32 * (t32 & 1) : 0;  // rows in use come first in a tile
+    if (used <= 0) return;
+    __shared__ uint64_t table[32];
+    if (threadIdx.x < 32) table[threadIdx.x] = EXPF_TABLE[threadIdx.x];
+    __syncthreads();
+    auto silu = [&](float x) { return silu_as_host(x, table); };  // (the quantizer sees a host's bits)
+    quantize_q8k_record<SWIGLU_WAVES>(out, (size_t)t32 * nb + kb, L, [&](int r) {
+        if (r >= used) return make_float4(0.f, 0.f, 0.f, 0.f);
+        const size_t src = ((size_t)(t32 * 32 + r) * nb + kb) * QK_K;
         const float4 gv = reinterpret_cast<const float4 *>(gate + src)[lane];
         const float4 uv = reinterpret_cast<const float4 *>(up + src)[lane];
         return make_float4(silu(gv.x) * uv.x, silu(gv.y) * uv.y, silu(gv.z) * uv.z, silu(gv.w) * uv.w);
@@ -248,7 +287,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const float g = gate[i];
-    act[i] = __fdiv_rn(g, 1.0f + (float)exp(-(double)g)) * up[i];
+    act[i] = silu_as_host(g) * up[i];
 }
 
 int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s);
@@ -266,18 +305,24 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     __shared__ float s_w[64];
     __shared__ int s_id[64];
     const int tok = blockIdx.x, tid = threadIdx.x;
-    if (tid < k) s_id[tid] = ids[(size_t)tok * k + tid];
+    // (the slot's three entries are asked for together: this kernel is as long as its chain of dependent loads)
+    int mine = 0, pos = 0;
+    float w = 0.0f;
+    if (tid < k) {
+        mine = ids[(size_t)tok * k + tid];
+        pos = pos_of ? pos_of[(size_t)tok * k + tid] : tok * k + tid;  // (no map: rows in pair order)
+        w = weights[(size_t)tok * k + tid];
+        s_id[tid] = mine;
+    }
     __syncthreads();
     if (tid < k) {
-        const int mine = s_id[tid];
         int rank = tid;
         if (by_expert_id) {  // place in the ascending order of expert ids, equal ids in slot order
             rank = 0;
             for (int j = 0; j < k; j++) rank += (s_id[j] < mine) || (s_id[j] == mine && j < tid);
         }
-        const int pos = pos_of ? pos_of[(size_t)tok * k + tid] : tok * k + tid;  // (no map: rows in pair order)
         s_pos[rank] = (mine >= 0 && mine < n_experts) ? pos : -1;
-        s_w[rank] = weights[(size_t)tok * k + tid];
+        s_w[rank] = w;
     }
     __syncthreads();
     for (int h = threadIdx.x * 4; h < hidden; h += blockDim.x * 4) {
@@ -319,6 +364,7 @@ struct MoeScratch {
     Q8KTiled xa;                          // the token rows in the grouped order, Q8_K
     float *gate_out, *up_out, *down_out;  // rows in the grouped order (with its gaps)
     Q8KTiled act;                         // Q8_K of silu(gate)*up
+    Q8KRows xr;                           // Q8_K of the token rows (the gathering form; shares xa's room)
     int *group_off, *gather, *pos_of, *cpos_of, *n_tiles;
     int4 *tiles;
 };
@@ -338,7 +384,16 @@ static MoeScratch moe_carve(void *base, size_t batch, int k, int n_experts, int 
         return r;
     };
     MoeScratch m;
-    m.xa = q8k_tiled_carve(take(q8k_tiled_bytes(rows, hidden)), rows, hidden);
+    {
+        // the token rows' Q8_K in one of two forms: gathered into the grouped order, or plain
+        const size_t nb = (size_t)hidden / QK_K;
+        const size_t plain = round_up(batch * hidden, 256) + round_up(batch * nb * 32, 256) + batch * nb * 4;
+        char *room = take(std::max(q8k_tiled_bytes(rows, hidden), plain));
+        m.xa = q8k_tiled_carve(room, rows, hidden);
+        m.xr.q = (int8_t *)room;
+        m.xr.bs = (_Float16 *)(room + round_up(batch * hidden, 256));
+        m.xr.d = (float *)(room + round_up(batch * hidden, 256) + round_up(batch * nb * 32, 256));
+    }
     m.gate_out = (float *)take(rows * ffn * 4);
     m.up_out = (float *)take(rows * ffn * 4);
     m.down_out = (float *)take(rows * hidden * 4);
@@ -433,24 +488,41 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
     if (!sized) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_group_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GroupLds));
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_group_quantize_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GroupLds));
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(moe_group): %s", hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ids, (int)pairs, k, n_experts,
-                       m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles, (int)rows);
-    FRK_LAUNCH_CHECK("moe_group");
-    // the token rows, gathered into the grouped order and quantized; gate and up share them
-    int rc = launch_quantize_q8_k_gather(x, (size_t)hidden, m.gather, rows, m.xa, s);
+    const GroupArgs ga{ids, (int)pairs, k, n_experts, m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles, (int)rows};
+    int rc;
+    if (gemm_q4_k_stream_gathers(batch, (size_t)hidden)) {
+        // every token row quantized once, beside the bucketing; the gate/up GEMM gathers its tiles' rows
+        const size_t n_blocks = batch * ((size_t)hidden / QK_K);
+        const unsigned quantizers = (unsigned)std::min<size_t>((n_blocks + 15) / 16, 512);
+        hipLaunchKernelGGL(moe_group_quantize_kernel, dim3(1 + quantizers), dim3(1024), sizeof(GroupLds), s, ga, x,
+                           (int)n_blocks, m.xr);
+        FRK_LAUNCH_CHECK("moe_group_quantize");
+        rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, &m.xr, m.gather, m.tiles, m.n_tiles, max_tiles, m.gate_out,
+                                     m.up_out, s);
+    } else {
+        hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ga);
+        FRK_LAUNCH_CHECK("moe_group");
+        // the token rows, gathered into the grouped order and quantized; gate and up share them
+        rc = launch_quantize_q8_k_gather(x, (size_t)hidden, m.gather, rows, m.xa, s);
+        if (rc) return rc;
+        rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, nullptr, nullptr, m.tiles, m.n_tiles, max_tiles, m.gate_out,
+                                     m.up_out, s);
+    }
     if (rc) return rc;
-    rc = launch_gemm_q4_k_stream(gate, up, (size_t)ffn, m.xa, m.tiles, m.n_tiles, max_tiles, m.gate_out, m.up_out, s);
-    if (rc) return rc;
-    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(256), 0, s, m.gate_out,
-                       m.up_out, ffn / QK_K, m.gather, m.act);
+    hipLaunchKernelGGL(swiglu_quantize_kernel, dim3((unsigned)(rows / 32 * (ffn / QK_K))), dim3(64 * SWIGLU_WAVES), 0, s,
+                       m.gate_out, m.up_out, ffn / QK_K, m.tiles, m.n_tiles, m.act);
     FRK_LAUNCH_CHECK("swiglu_quantize");
     // (a Q4_K_M checkpoint keeps some layers' down experts in Q6_K: the matrix-core Q6_K kernel, by tile)
     rc = down->kind == FRK_KIND_Q6_K
              ? launch_gemm_q6_k_grouped(down, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, s)
-             : launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, m.tiles, m.n_tiles, max_tiles, m.down_out, nullptr, s);
+             : launch_gemm_q4_k_stream(down, nullptr, (size_t)hidden, m.act, nullptr, nullptr, m.tiles, m.n_tiles, max_tiles,
+                                       m.down_out, nullptr, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch), dim3(256), 0, s, m.down_out, ids, weights, m.pos_of, k,
                        hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);

@@ -490,7 +490,8 @@ def test_route_top_k_softmax_matches_the_oracle(fa):
         ids, w = fa.route_top_k_softmax(to_dev(logits), 8, norm)
         want_ids, want_w = _route(logits, 8, norm)
         assert np.array_equal(ids.cpu().numpy(), want_ids)
-        np.testing.assert_allclose(w.cpu().numpy(), want_w, rtol=2e-6)
+        # bit for bit: the device evaluates expf the way the host's libm does, and adds in the oracle's order
+        assert np.array_equal(bits(w.cpu().numpy()), bits(want_w))
     # the reference's own known answers (crates/frink-moe/src/lib.rs:1345-1404)
     ids, w = fa.route_top_k_softmax(to_dev(np.arange(1, 9, dtype=np.float32)[None]), 3, False)
     assert ids.cpu().numpy().tolist() == [[7, 6, 5]]
@@ -576,18 +577,6 @@ def _end_to_end_gate(got, want, what, strict):
         assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, "%s: worst row %.3g" % (what, rel.max())
 
 
-def _swiglu_rounded_once(g, u):
-    """silu(g) * u with exp evaluated in double and rounded once to f32 -- the correctly rounded expf,
-    which is how the device evaluates it.  A host libm's expf (the oracle's, and the reference's scalar
-    build) returns the same value except for rare last-bit cases, and the reference's SIMD build uses a
-    polynomial a few ulp off, so the bit-exact gate on the quantized intermediate is stated on this
-    definition; the caller checks that it stays within a few ulp of the oracle's."""
-    g = np.asarray(g, np.float32)
-    with np.errstate(over="ignore"):  # exp(-g) of a very negative g is inf in f32, as on the device
-        e = np.exp(-g.astype(np.float64)).astype(np.float32)
-    return (g / (np.float32(1.0) + e)) * np.asarray(u, np.float32)
-
-
 def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, ids_override=None, down_kind=None,
               sigma=0.05, strict=False):
     """The quantizer between the two GEMMs is a step function, so a last-bit difference in a
@@ -596,7 +585,8 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     implementation that sums in another order than the oracle.  The layer is therefore gated as a
     chain in which each link starts from the device's own previous result:
       1. gate/up grouped GEMM outputs (row of every (token, slot) pair) vs the oracle's GEMM  [tolerance]
-      2. silu(gate)*up (exp rounded once, _swiglu_rounded_once) and its Q8_K quantization, from the device's gate/up  [bit-exact]
+      2. silu(gate)*up (the oracle's, whose expf is the host's: the device evaluates glibc's algorithm) and its
+         Q8_K quantization, from the device's gate/up                                          [bit-exact]
       3. down GEMM + weighted combine, from that same intermediate                            [tolerance]
     and end to end against the oracle's layer (_end_to_end_gate)."""
     from frink_amd import synth
@@ -636,9 +626,7 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
 
     gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
     want_down = np.zeros((batch * k, hidden), np.float32)
-    act = _swiglu_rounded_once(g_out, u_out).reshape(batch * k, ffn)
-    lib_act = fo.swiglu(g_out.ravel(), u_out.ravel()).reshape(batch * k, ffn)
-    assert (np.abs(act - lib_act) <= 4.8e-7 * np.abs(lib_act)).all()  # a few ulp: 1 in exp, then 1 + e, the quotient and the product
+    act = fo.swiglu(g_out.ravel(), u_out.ravel()).reshape(batch * k, ffn)
     for e in range(n_experts):
         rows = np.array([int(pos[t, s]) for ee, t, s in order if ee == e], dtype=np.int64)
         toks = np.array([t for ee, t, s in order if ee == e], dtype=np.int64)

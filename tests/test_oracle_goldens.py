@@ -517,6 +517,52 @@ def test_silu_and_swiglu_are_the_textbook_forms():
     assert fo.silu(0.0) == 0.0
 
 
+def _expf_table():
+    """2^(i/32) correctly rounded to double, i < 32, from integer arithmetic (the 32nd root of 2^(i + 32*400) by
+    five integer square roots), with i/32 taken off the exponent field: the table of glibc's expf."""
+    from math import isqrt
+    out = []
+    for i in range(32):
+        v = 1 << (i + 32 * 400)
+        for _ in range(5):
+            v = isqrt(v)
+        low = v & ((1 << 348) - 1)
+        assert abs(low - (1 << 347)) > (1 << 300)          # nowhere near a tie: the floors above cannot matter
+        m = (v + (1 << 347)) >> 348                         # 53 bits, the leading one included
+        out.append((1023 << 52) + (m - (1 << 52)) - ((i << 52) // 32))
+    return np.array(out, dtype=np.uint64)
+
+
+def expf_table_algorithm(x):
+    """expf as glibc >= 2.28 computes it (the algorithm the device kernels evaluate, restated in numpy's
+    IEEE double arithmetic), for |x| < 88."""
+    n = 32.0
+    c0, c1, c2 = float.fromhex("0x1.c6af84b912394p-5") / n / n / n, float.fromhex("0x1.ebfce50fac4f3p-3") / n / n, \
+        float.fromhex("0x1.62e42ff0c52d6p-1") / n
+    inv_ln2_n, shift = float.fromhex("0x1.71547652b82fep+0") * n, float.fromhex("0x1.8p+52")
+    z = inv_ln2_n * np.asarray(x, np.float32).astype(np.float64)
+    kd = z + shift
+    ki = kd.view(np.uint64)
+    r = z - (kd - shift)
+    s = (_expf_table()[(ki & np.uint64(31)).astype(np.int64)] + (ki << np.uint64(47))).view(np.float64)
+    y = (c0 * r + c1) * (r * r) + (c2 * r + 1.0)
+    return (y * s).astype(np.float32)
+
+
+def test_the_devices_expf_algorithm_is_the_hosts_expf():
+    """The device evaluates silu and the router's softmax with glibc's expf algorithm so that a quantizer
+    downstream sees a Linux host's bits (Rust's f32::exp is the platform's expf).  Its restatement above,
+    with a table derived here from integers, against the oracle's silu (x / (1 + expf(-x)) through this
+    host's libm) on four million values: bit for bit."""
+    x = np.concatenate([RNG.standard_normal(2_000_000).astype(np.float32) * 4,
+                        RNG.uniform(-87.9, 87.9, 2_000_000).astype(np.float32),
+                        np.array([0.0, -0.0, 1e-30, -1e-30, 87.99, -87.99, 1.0, -1.0], np.float32)])
+    with np.errstate(over="ignore"):
+        mine = x / (np.float32(1.0) + expf_table_algorithm(-x))
+    want = fo.swiglu(x, np.ones_like(x))
+    assert np.array_equal(mine.view(np.uint32), want.view(np.uint32))
+
+
 def test_moe_batch_equals_per_token_experts_combined():
     E, k, hidden, ffn, batch = 6, 2, 256, 512, 9
     gate = _weights(fo.Q4_K, E * ffn, hidden)
