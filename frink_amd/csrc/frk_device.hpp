@@ -130,8 +130,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // cubic for the rest, rounded to f32 once.  Rust's f32::exp is the platform's expf (the reference's silu:
 // crates/frink-core/src/matmul.rs:634-650), so this returns a Linux host's bits (a build of glibc that fuses
 // the cubic's multiply-adds differs in the double's last bits, which reaches the f32 in about one value in
-// 2^29) at a third of the instructions of a correctly rounded double exp.  Outside |x| < 88 (where glibc
-// handles overflow, underflow and NaN separately) the double exp rounds to the same values.
+// 2^29) at a third of the instructions of a correctly rounded double exp.
 __constant__ const uint64_t EXPF_TABLE[32] = {
     0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
     0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
@@ -141,23 +140,39 @@ __constant__ const uint64_t EXPF_TABLE[32] = {
     0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
     0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
-// (`table`: EXPF_TABLE or a copy of it, e.g. in LDS for a kernel that evaluates many)
-__device__ __forceinline__ float expf_as_libm(float x, const uint64_t *table = EXPF_TABLE) {
-    if (!(fabsf(x) < 88.0f)) return (float)exp((double)x);
-    constexpr double N = 32.0;
-    constexpr double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
-    constexpr double INV_LN2_N = 0x1.71547652b82fep+0 * N, SHIFT = 0x1.8p+52;
+// In two steps, so that a caller can fetch the table entries of several values at once: the reduction
+// (r and the integer k, whose low five bits select the entry) and the rest.  Outside the range where the
+// result is a finite, non-zero f32 glibc returns inf, 0 or (just above the underflow threshold, its "may
+// underflow" path) the smallest subnormal; a NaN comes out of the arithmetic as a NaN.
+struct ExpfReduced {
+    double r;
+    uint32_t k;
+};
+__device__ __forceinline__ ExpfReduced expf_reduce(float x) {
+    constexpr double INV_LN2_N = 0x1.71547652b82fep+0 * 32.0, SHIFT = 0x1.8p+52;
     const double z = INV_LN2_N * (double)x;
     double kd = z + SHIFT;  // the integer nearest to z sits in the low bits
-    const uint64_t ki = (uint64_t)__double_as_longlong(kd);
+    const uint32_t k = (uint32_t)__double_as_longlong(kd);
     kd -= SHIFT;
-    const double r = z - kd;
-    const double s = __longlong_as_double((long long)(table[ki & 31] + (ki << 47)));
-    const double p = C0 * r + C1;
-    const double r2 = r * r;
-    double y = C2 * r + 1.0;
+    return {z - kd, k};
+}
+__device__ __forceinline__ float expf_finish(float x, const ExpfReduced &a, uint64_t entry) {
+    constexpr double N = 32.0;
+    constexpr double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
+    const double s = __longlong_as_double((long long)(entry + ((uint64_t)a.k << 47)));
+    const double p = C0 * a.r + C1;
+    const double r2 = a.r * a.r;
+    double y = C2 * a.r + 1.0;
     y = p * r2 + y;
-    return (float)(y * s);
+    float e = (float)(y * s);
+    if (x > 0x1.62e42ep6f) e = INFINITY;
+    if (x < -0x1.9d1d9ep6f) e = x < -0x1.9fe368p6f ? 0.0f : 0x1p-149f;
+    return e;
+}
+// (`table`: EXPF_TABLE or a copy of it)
+__device__ __forceinline__ float expf_as_libm(float x, const uint64_t *table = EXPF_TABLE) {
+    const ExpfReduced a = expf_reduce(x);
+    return expf_finish(x, a, table[a.k & 31]);
 }
 // x * sigmoid(x) as the reference's hosts compute it: x / (1 + expf(-x)), each step rounded to f32
 __device__ __forceinline__ float silu_as_host(float x, const uint64_t *table = EXPF_TABLE) {

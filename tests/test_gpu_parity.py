@@ -492,6 +492,14 @@ def test_route_top_k_softmax_matches_the_oracle(fa):
         assert np.array_equal(ids.cpu().numpy(), want_ids)
         # bit for bit: the device evaluates expf the way the host's libm does, and adds in the oracle's order
         assert np.array_equal(bits(w.cpu().numpy()), bits(want_w))
+    # logits far below the row's maximum: expf down to its subnormal results, glibc's underflow value and zero
+    far = np.random.default_rng(5).uniform(-110, -80, (64, 16)).astype(np.float32)
+    far[:, 0] = 0.0
+    far[0, 1:6] = [-103.2, -103.3, -103.9, -104.0, -87.4]
+    ids, w = fa.route_top_k_softmax(to_dev(far), 4, False)
+    want_ids, want_w = _route(far, 4, False)
+    assert np.array_equal(bits(w.cpu().numpy()), bits(want_w))
+    assert np.array_equal(ids.cpu().numpy()[want_w > 0], want_ids[want_w > 0])  # (zeros tie: any order)
     # the reference's own known answers (crates/frink-moe/src/lib.rs:1345-1404)
     ids, w = fa.route_top_k_softmax(to_dev(np.arange(1, 9, dtype=np.float32)[None]), 3, False)
     assert ids.cpu().numpy().tolist() == [[7, 6, 5]]

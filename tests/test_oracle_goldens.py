@@ -535,18 +535,24 @@ def _expf_table():
 
 def expf_table_algorithm(x):
     """expf as glibc >= 2.28 computes it (the algorithm the device kernels evaluate, restated in numpy's
-    IEEE double arithmetic), for |x| < 88."""
+    IEEE double arithmetic), with its three results outside the range of a finite, non-zero f32."""
     n = 32.0
     c0, c1, c2 = float.fromhex("0x1.c6af84b912394p-5") / n / n / n, float.fromhex("0x1.ebfce50fac4f3p-3") / n / n, \
         float.fromhex("0x1.62e42ff0c52d6p-1") / n
     inv_ln2_n, shift = float.fromhex("0x1.71547652b82fep+0") * n, float.fromhex("0x1.8p+52")
-    z = inv_ln2_n * np.asarray(x, np.float32).astype(np.float64)
+    x = np.asarray(x, np.float32)
+    z = inv_ln2_n * x.astype(np.float64)
     kd = z + shift
     ki = kd.view(np.uint64)
     r = z - (kd - shift)
     s = (_expf_table()[(ki & np.uint64(31)).astype(np.int64)] + (ki << np.uint64(47))).view(np.float64)
     y = (c0 * r + c1) * (r * r) + (c2 * r + 1.0)
-    return (y * s).astype(np.float32)
+    with np.errstate(over="ignore", under="ignore", invalid="ignore"):
+        e = (y * s).astype(np.float32)
+    e = np.where(x > np.float32(float.fromhex("0x1.62e42ep6")), np.float32(np.inf), e)
+    e = np.where(x < np.float32(float.fromhex("-0x1.9d1d9ep6")), np.float32(2.0 ** -149), e)  # glibc's "may underflow" value
+    e = np.where(x < np.float32(float.fromhex("-0x1.9fe368p6")), np.float32(0.0), e)
+    return e.astype(np.float32)
 
 
 def test_the_devices_expf_algorithm_is_the_hosts_expf():
@@ -556,11 +562,20 @@ def test_the_devices_expf_algorithm_is_the_hosts_expf():
     host's libm) on four million values: bit for bit."""
     x = np.concatenate([RNG.standard_normal(2_000_000).astype(np.float32) * 4,
                         RNG.uniform(-87.9, 87.9, 2_000_000).astype(np.float32),
-                        np.array([0.0, -0.0, 1e-30, -1e-30, 87.99, -87.99, 1.0, -1.0], np.float32)])
-    with np.errstate(over="ignore"):
+                        RNG.uniform(-110, -86, 500_000).astype(np.float32), RNG.uniform(86, 92, 500_000).astype(np.float32),
+                        np.array([0.0, -0.0, 1e-30, -1e-30, 87.99, -87.99, 1.0, -1.0, 1e-42, 200.0, -200.0, np.inf, -np.inf],
+                                 np.float32)])
+    with np.errstate(over="ignore", invalid="ignore"):
         mine = x / (np.float32(1.0) + expf_table_algorithm(-x))
     want = fo.swiglu(x, np.ones_like(x))
     assert np.array_equal(mine.view(np.uint32), want.view(np.uint32))
+    # expf itself where silu hides it (1 + e rounds a small e away): softmax weights e(l) / (1 + e(l)) of two
+    # logits 0 and l <= 0 through the oracle's router, down to the underflow and past it
+    lo = np.concatenate([RNG.uniform(-110, -80, 20_000), RNG.uniform(-30, 0, 20_000)]).astype(np.float32)
+    e = expf_table_algorithm(lo)
+    for l, el in zip(lo[::40], e[::40]):
+        _, w = fo.route_top_k_softmax(np.array([0.0, l], np.float32), 2, False)
+        assert w[1].view(np.uint32) == (el / (np.float32(1.0) + el)).view(np.uint32)
 
 
 def test_moe_batch_equals_per_token_experts_combined():
