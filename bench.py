@@ -474,6 +474,18 @@ def main():
             wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
             extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
                            "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+        # the same M=8 batches from activations quantized beforehand (by the kernel that produced them, or
+        # shared with another projection): the multiplying launch alone
+        for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096, activations quantized beforehand", g8, x8, y8),
+                                      ("Q6_K thin GEMM M=8 4096x14336, activations quantized beforehand", dn, h8, z8)):
+            acts8 = fa.quantize_q8_k(xin)
+
+            def step5q(i, mats=mats, acts8=acts8, yout=yout):
+                mats[i % 8].gemm_q8k(acts8, 8, out=yout)
+            _, t = time_graph(torch, step5q, 400, 200)
+            wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
+            extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
+                           "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
         yf = torch.empty(cols, dtype=torch.float32, device=dev)
 
         def step6(i):

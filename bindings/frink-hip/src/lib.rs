@@ -86,6 +86,8 @@ extern "C" {
     fn frk_hip_ffn_swiglu_dev(gate: *const FrkWeights, up: *const FrkWeights, down: *const FrkWeights, x: *const f32,
                               y: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_gemm_dev(w: *const FrkWeights, x: *const f32, batch: usize, y: *mut f32, stream: *mut c_void) -> c_int;
+    fn frk_hip_gemm_q8k_dev(w: *const FrkWeights, q: *const i8, d: *const f32, bsums: *const i16, batch: usize,
+                            y: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_gemm_pair_dev(w0: *const FrkWeights, w1: *const FrkWeights, x: *const f32, batch: usize, y0: *mut f32,
                              y1: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_gemm_noalloc_dev(w: *const FrkWeights, x: *const f32, batch: usize, y: *mut f32,
@@ -306,6 +308,15 @@ pub mod dev {
     /// `x` holds `batch * w.cols()` floats, `y` room for `batch * w.rows()`.
     pub unsafe fn gemm(w: &Weights, x: *const f32, batch: usize, y: *mut f32, stream: *mut c_void) -> Result<(), HipError> {
         check(frk_hip_gemm_dev(w.0, x, batch, y, stream))
+    }
+    /// `apply_batch_with_acts` with `BatchActs::Q8K` (weight_matrix.rs:2481-2487, 757-768) for a thin batch: the
+    /// activations are Q8_K already (`q [batch][cols]`, `d [batch][cols/256]`, `bsums [batch][cols/16]`).
+    /// `Unsupported` beyond the rows the thin kernels take for the matrix.
+    /// # Safety
+    /// device pointers of those sizes; `y` has room for `batch * w.rows()` floats.
+    pub unsafe fn gemm_q8k(w: &Weights, q: *const i8, d: *const f32, bsums: *const i16, batch: usize, y: *mut f32,
+                           stream: *mut c_void) -> Result<(), HipError> {
+        check(frk_hip_gemm_q8k_dev(w.0, q, d, bsums, batch, y, stream))
     }
     /// `WeightMatrix::apply_batch_pair_with_acts` (weight_matrix.rs:2447-2479): gate and up of a prefill
     /// FFN over one quantization of the batch.

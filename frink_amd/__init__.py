@@ -30,7 +30,7 @@ EXPORTS = [
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
     "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
-    "frk_hip_gemm_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
+    "frk_hip_gemm_dev", "frk_hip_gemm_q8k_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
@@ -89,6 +89,7 @@ def lib():
             "frk_hip_gemv_dev": (i, [vp, vp, vp, i, vp]),
             "frk_hip_gemv_q8k_dev": (i, [vp, vp, vp, vp, vp, vp]),
             "frk_hip_gemm_dev": (i, [vp, vp, sz, vp, vp]),
+            "frk_hip_gemm_q8k_dev": (i, [vp, vp, vp, vp, sz, vp, vp]),
             "frk_hip_gemm_noalloc_dev": (i, [vp, vp, sz, vp, vp]),
             "frk_hip_gemm_pair_dev": (i, [vp, vp, vp, sz, vp, vp, vp]),
             "frk_hip_route_top_k_softmax_dev": (i, [vp, sz, sz, sz, i, vp, vp, vp]),
@@ -195,6 +196,15 @@ class Weights:
         y = out if out is not None else torch.empty(self.rows, dtype=torch.float32, device=q.device)
         check(lib().frk_hip_gemv_q8k_dev(self.handle, C.c_void_p(q.data_ptr()), C.c_void_p(d.data_ptr()),
                                          C.c_void_p(bs.data_ptr()), C.c_void_p(y.data_ptr()), _stream()))
+        return y
+
+    def gemm_q8k(self, acts, batch, out=None):
+        """A thin batch over activations quantized beforehand: acts = (q, d, bsums) of quantize_q8_k over the batch."""
+        import torch
+        q, d, bs = acts
+        y = out if out is not None else torch.empty((batch, self.rows), dtype=torch.float32, device=q.device)
+        check(lib().frk_hip_gemm_q8k_dev(self.handle, C.c_void_p(q.data_ptr()), C.c_void_p(d.data_ptr()),
+                                         C.c_void_p(bs.data_ptr()), batch, C.c_void_p(y.data_ptr()), _stream()))
         return y
 
     def gemm(self, x, out=None):

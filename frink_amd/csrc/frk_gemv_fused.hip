@@ -45,7 +45,7 @@ struct ActStage {
         }
     }
 
-    __device__ __forceinline__ void store(int nb, int8_t *sq, int16_t *sbs, float *sd) {
+    __device__ __forceinline__ void store(int nb, int8_t *sq, int16_t *sbs, float *sd, const int16_t *__restrict__ absums) {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
         if (MODE == MODE_PREQ_LDS) {
 #pragma unroll
@@ -54,6 +54,10 @@ struct ActStage {
                 if (idx < nb * 16) reinterpret_cast<uint4 *>(sq)[idx] = qv[i];
             }
             if ((int)threadIdx.x < nb * 8) reinterpret_cast<uint32_t *>(sbs)[threadIdx.x] = bv;
+            // (a workgroup of fewer threads than the row has pairs of sums -- few rows of many blocks -- fetches
+            // the rest here)
+            for (int i = (int)threadIdx.x + (int)blockDim.x; i < nb * 8; i += (int)blockDim.x)
+                reinterpret_cast<uint32_t *>(sbs)[i] = reinterpret_cast<const uint32_t *>(absums)[i];
             if ((int)threadIdx.x < nb) sd[threadIdx.x] = dv;
         } else if (MODE == MODE_FUSED) {
 #pragma unroll
@@ -269,7 +273,7 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
     issue(row_begin);
 
     if (MODE != MODE_PREQ_DIRECT) {
-        act.store(nb, sq, sbs, sd);
+        act.store(nb, sq, sbs, sd, absums);
         lds_barrier();
 #pragma unroll
         for (int j = 0; j < J; j++) {

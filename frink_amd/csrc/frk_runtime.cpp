@@ -544,6 +544,36 @@ static bool q5_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
     return w->kind == FRK_KIND_Q5_K && batch > q5k_thin_rows;
 }
 
+// Q6_K: the matrix-core GEMM (with its blocks split between workgroups for small batches: 53 us at
+// 4096x14336 and 31 us at 4096x4096 up to 64 rows) is ahead of the thin kernel's 8-row groups (15 us
+// and 6 us each) from four groups on for large matrices and from six on for small ones
+static bool q6_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
+    const size_t q6k_gemm_from = w->rows * w->cols > (size_t)2 * 4096 * 4096 ? 25 : 41;
+    return w->kind == FRK_KIND_Q6_K && batch >= q6k_gemm_from;
+}
+// whether a batch of this matrix multiplies on the thin kernels (over plain Q8_K rows)
+static bool batch_takes_the_thin_kernels(const frk_weights *w, size_t batch) {
+    const bool k_quant = w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K;
+    if (!k_quant || batch < 2) return false;
+    if (q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch) || q6_k_takes_the_matrix_cores(w, batch))
+        return false;
+    return thin_gemm_max_batch(w) >= 2;
+}
+
+// a thin batch over activations already in Q8_K: `thin` rows a launch (thin_gemm_max_batch), or one launch over a
+// grid of such groups where the kernel has that form
+static int thin_gemm_acts(const frk_weights *w, const Q8KActs &a, size_t batch, int thin, float *y, hipStream_t s) {
+    const size_t nb = w->cols / QK_K;
+    if (batch > (size_t)thin && batch <= (size_t)thin_gemm_wide_rows(w)) return launch_thin_gemm_wide(w, (int)batch, a, y, s);
+    for (size_t b0 = 0; b0 < batch; b0 += (size_t)thin) {
+        const int n = (int)std::min<size_t>((size_t)thin, batch - b0);
+        Q8KActs c = {a.q + b0 * w->cols, a.d + b0 * nb, a.bsums + b0 * nb * 16};
+        int rc = launch_thin_gemm(w, n, c, y + b0 * w->rows, s);
+        if (rc) return rc;
+    }
+    return FRK_OK;
+}
+
 static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
     if (q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch)) {  // (frk_hip_gemm_pair_dev: the same test)
         void *ws = nullptr;
@@ -552,11 +582,7 @@ static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *
         if (rc) return rc;
         return launch_gemm_q4_k(w, x, batch, y, ws, (hipStream_t)stream);
     }
-    // Q6_K: the matrix-core GEMM (with its blocks split between workgroups for small batches: 53 us at
-    // 4096x14336 and 31 us at 4096x4096 up to 64 rows) is ahead of the thin kernel's 8-row groups (15 us
-    // and 6 us each) from four groups on for large matrices and from six on for small ones
-    const size_t q6k_gemm_from = w->rows * w->cols > (size_t)2 * 4096 * 4096 ? 25 : 41;
-    if (w->kind == FRK_KIND_Q6_K && batch >= q6k_gemm_from) {
+    if (q6_k_takes_the_matrix_cores(w, batch)) {
         void *ws = nullptr;
         int rc = scratch.get(gemm_q6_k_workspace_bytes(batch, w->cols, w->rows), (hipStream_t)stream, &ws);
         if (rc) return rc;
@@ -571,22 +597,12 @@ static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *
         return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
-    const int thin = (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K) && batch >= 2
-                         ? thin_gemm_max_batch(w) : 0;
-    if (thin >= 2) {
+    if (batch_takes_the_thin_kernels(w, batch)) {
+        const int thin = thin_gemm_max_batch(w);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, batch, (hipStream_t)stream, scratch, &a);
         if (rc) return rc;
-        const size_t nb = w->cols / QK_K;
-        if (batch > (size_t)thin && batch <= (size_t)thin_gemm_wide_rows(w))
-            return launch_thin_gemm_wide(w, (int)batch, a, y, (hipStream_t)stream);
-        for (size_t b0 = 0; b0 < batch; b0 += (size_t)thin) {
-            const int n = (int)std::min<size_t>((size_t)thin, batch - b0);
-            Q8KActs c = {a.q + b0 * w->cols, a.d + b0 * nb, a.bsums + b0 * nb * 16};
-            rc = launch_thin_gemm(w, n, c, y + b0 * w->rows, (hipStream_t)stream);
-            if (rc) return rc;
-        }
-        return FRK_OK;
+        return thin_gemm_acts(w, a, batch, thin, y, (hipStream_t)stream);
     }
     // Q5_K rows too long for the thin kernel's LDS: the batch is quantized once and every row takes the
     // decode kernel
@@ -617,6 +633,22 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x, size_t batch, float *
     if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
     Scratch scratch;
     return gemm_impl(w, x, batch, y, stream, scratch);
+}
+
+int frk_hip_gemm_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, const int16_t *bsums, size_t batch, float *y,
+                         void *stream) {
+    clear_error();
+    if (!w || !q || !d || !bsums || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_q8k_dev: null argument");
+    if (batch == 0) return set_error(FRK_ERR_SHAPE, "empty shape: batch=0");
+    if (batch == 1) return frk_hip_gemv_q8k_dev(w, q, d, bsums, y, stream);
+    const bool k_quant = w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K;
+    if (!k_quant) return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d)", w->kind);
+    if (!batch_takes_the_thin_kernels(w, batch))
+        return set_error(FRK_ERR_UNSUPPORTED,
+                         "a batch of %zu rows of this matrix does not multiply on the thin kernels (the matrix-core GEMM "
+                         "quantizes into a tiled form of its own): frk_hip_gemm_dev / frk_hip_gemm_pair_dev", batch);
+    Q8KActs a{q, d, bsums};
+    return thin_gemm_acts(w, a, batch, thin_gemm_max_batch(w), y, (hipStream_t)stream);
 }
 
 int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const float *x, size_t batch, float *y0, float *y1,

@@ -198,6 +198,16 @@ int frk_hip_ffn_swiglu_dev(const frk_weights *gate, const frk_weights *up, const
 int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, float *y_dev,
                      void *stream);
 
+/* frk_hip_gemm_dev for a thin batch whose activations the caller (the kernel that produced them, or an earlier
+ * call over the same batch) has already quantized to Q8_K: q [batch][cols] i8, d [batch][cols/256] f32,
+ * bsums [batch][cols/16] i16, the layout frk_hip_quantize_q8_k_dev writes (BatchActs::Q8K,
+ * crates/frink-core/src/weight_matrix.rs:757-768, handed to apply_batch_with_acts, :2481-2487).  Bit for bit
+ * frk_hip_gemm_dev's result (one row: frk_hip_gemv_q8k_dev).  K-quants; the batches that frk_hip_gemm_dev multiplies on its thin kernels (up to 32
+ * rows for Q4_K and Q5_K, up to 24 or 40 for Q6_K by the matrix's size): FRK_ERR_UNSUPPORTED beyond, where the
+ * matrix-core GEMM quantizes into a tiled form of its own. */
+int frk_hip_gemm_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float *d_dev, const int16_t *bsums_dev,
+                         size_t batch, float *y_dev, void *stream);
+
 /* WeightMatrix::apply_batch_pair_with_acts (crates/frink-core/src/weight_matrix.rs:2447-2479) with
  * BatchActs::Q8K (:757-768): two matrices of one column count over ONE quantization of the batch -- gate
  * and up of a prefill FFN.  y0 and y1 are bit for bit what two frk_hip_gemm_dev calls give. */

@@ -242,6 +242,49 @@ def test_q4_k_gemv_over_whole_cache_lines(fa, rows, cols):
     w.release()
 
 
+@pytest.mark.parametrize("kind,rows,cols,batches", [
+    (fo.Q4_K, 200, 4096, (2, 8, 16, 17, 32)), (fo.Q4_K, 72, 512, (3, 9)), (fo.Q6_K, 136, 2048, (2, 8, 9, 24)),
+    (fo.Q5_K, 100, 1024, (2, 16, 17, 32)), (fo.Q4_K, 50, 14336, (8,)),
+])
+def test_thin_gemm_from_activations_quantized_beforehand(fa, kind, rows, cols, batches):
+    """frk_hip_gemm_q8k_dev (apply_batch_with_acts with BatchActs::Q8K, weight_matrix.rs:2481-2487, 757-768): a thin
+    batch over Q8_K activations that frk_hip_quantize_q8_k_dev (or the producing kernel) wrote -- bit for bit
+    frk_hip_gemm_dev's result (one row: frk_hip_gemv_q8k_dev's); a batch beyond the thin kernels' is refused with a
+    message that names the entry to call."""
+    from frink_amd import synth
+    data = make_weights(kind, rows, cols, seed=rows + cols)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    x = synth.activations(rows + 7, max(batches), cols, outlier_frac=0.01)
+    for batch in batches:
+        xd = to_dev(x[:batch])
+        want = w.gemm(xd).cpu().numpy()
+        got = w.gemm_q8k(fa.quantize_q8_k(xd), batch).cpu().numpy()
+        assert np.array_equal(bits(got), bits(want)), "batch %d" % batch
+    acts = fa.quantize_q8_k(to_dev(x[0]))  # one row is frk_hip_gemv_q8k_dev
+    assert np.array_equal(bits(w.gemm_q8k(acts, 1).cpu().numpy()[0]), bits(w.gemv_q8k(acts).cpu().numpy()))
+    if kind == fo.Q4_K:
+        xd = to_dev(synth.activations(3, 64, cols))
+        with pytest.raises(fa.BackendError) as err:
+            w.gemm_q8k(fa.quantize_q8_k(xd), 64)
+        assert err.value.code == fa.ERR_UNSUPPORTED and "frk_hip_gemm_dev" in str(err.value)
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols", [(50, 14336), (300, 12288), (1000, 8448), (7, 16128), (64, 8192), (40, 2304)])
+def test_q4_k_gemv_from_quantized_activation_at_rows_between_the_line_lengths(fa, rows, cols):
+    """frk_hip_gemv_q8k_dev for rows whose block count is not 8, 16, 32 or 64: above 8192 columns the activation
+    is staged in LDS by a workgroup of 256 threads -- fewer than a 14336-column row has pairs of 16-wide sums."""
+    from frink_amd import synth
+    data = make_weights(fo.Q4_K, rows, cols, seed=rows + cols)
+    x = synth.activations(rows + cols, 1, cols, outlier_frac=0.01)[0]
+    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    want = fo.gemv(fo.Q4_K, data, rows, cols, x)
+    pre = w.gemv_q8k(fa.quantize_q8_k(to_dev(x))).cpu().numpy()
+    assert_rows_close(pre[None], want[None], "gemv_q8k %dx%d" % (rows, cols))
+    assert_rows_close(w.gemv(to_dev(x)).cpu().numpy()[None], want[None], "gemv %dx%d" % (rows, cols))
+    w.release()
+
+
 def test_gemv_outliers_and_zero_activation(fa):
     from frink_amd import synth
     data = make_weights(fo.Q4_K, 32, 4096, seed=3)
