@@ -299,7 +299,7 @@ def main():
         del src, dst
         for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
                                  ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
-                                 ("Q5_K GEMV 14336x4096 (quantization + decode kernel)", fa.Q5_K, 14336, 4096),
+                                 ("Q5_K GEMV 14336x4096 (one launch)", fa.Q5_K, 14336, 4096),
                                  ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096)):
             d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
             n_copies = COPIES if k2 != fa.Q8_0 else 32

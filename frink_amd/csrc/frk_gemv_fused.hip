@@ -335,8 +335,11 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
 // integers and its per-block float expression (crates/frink-quant/src/lib.rs:822-869), the blocks
 // of a row then added by its NB lanes with DPP.  The activation's blocks sit 272 bytes apart in LDS,
 // so that the lanes of a wavefront, which read NB different blocks at once, hit different banks.
+// Q5: the same for Q5_K blocks (176 bytes: Q4_K's header, 32 bytes of fifth bits -- byte l holds weight l of
+// every sub-block, sub-block j in bit j --, the nibbles; dot_q5_k_q8, crates/frink-quant/src/lib.rs:886-938):
+// a span is 11 KB, and a weight's fifth bit is put over its nibble on the way into v_dot4.
 constexpr int LINES_ACT_STRIDE = QK_K + 16;
-template <int NB, int MODE, int WAVES>
+template <int NB, int MODE, int WAVES, bool Q5 = false>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8_t *__restrict__ W, int rows,
                                                                     const float *__restrict__ x,
                                                                     const int8_t *__restrict__ aq,
@@ -344,24 +347,26 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
                                                                     const int16_t *__restrict__ absums,
                                                                     float *__restrict__ y) {
     constexpr int RPS = 64 / NB;  // rows of a wavefront's span
+    constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES, SPAN = 64 * BB, PIECES = SPAN / 1024;  // 9 or 11 KB
     static_assert(64 % NB == 0 && NB >= 8, "a span of 64 blocks is a whole number of rows of at least 8 blocks");
+    static_assert(NB * 16 <= 3 * 64 * WAVES, "three 16-byte words of quantized activation a thread at most");
     extern __shared__ uint4 smem[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
     int8_t *sq = reinterpret_cast<int8_t *>(lds);                          // NB blocks of quants, 272 bytes apart
     int *sbs = reinterpret_cast<int *>(lds + NB * LINES_ACT_STRIDE);       // NB x 8 sums over 32
     float *sd = reinterpret_cast<float *>(lds + NB * LINES_ACT_STRIDE + NB * 32);
-    uint8_t *sw = lds + NB * LINES_ACT_STRIDE + NB * 32 + NB * 4;          // WAVES spans of 9216 bytes (16-byte aligned)
+    uint8_t *sw = lds + NB * LINES_ACT_STRIDE + NB * 32 + NB * 4;          // WAVES spans (16-byte aligned)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const size_t span = (size_t)blockIdx.x * WAVES + wave;
-    const size_t bytes = (size_t)rows * NB * Q4_K_BYTES;
-    const bool has_rows = span * 9216 < bytes;  // (a wavefront past the matrix still quantizes its share)
+    const size_t bytes = (size_t)rows * NB * BB;
+    const bool has_rows = span * SPAN < bytes;  // (a wavefront past the matrix still quantizes its share)
 
     // ---- the activation's loads first (a wavefront's loads return in order), then the span ----
     typedef float xv_t __attribute__((ext_vector_type(4)));
     typedef uint32_t uq_t __attribute__((ext_vector_type(4)));
     xv_t xv[(NB + WAVES - 1) / WAVES];
-    uq_t qv = {0u, 0u, 0u, 0u}, qv2 = {0u, 0u, 0u, 0u};
+    uq_t qv = {0u, 0u, 0u, 0u}, qv2 = {0u, 0u, 0u, 0u}, qv3 = {0u, 0u, 0u, 0u};
     uint32_t bv = 0;
     float dv = 0.0f;
     // (All of this kernel's global loads are issued from assembly and waited for by hand: the compiler
@@ -375,42 +380,65 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xv[i]) : "v"(src) : "memory");
         }
     } else {
-        // quants: NB*16 words over 64*WAVES threads (NB <= 64, WAVES = 8: at most two each); sums and scales.
+        // quants: NB*16 words over 64*WAVES threads (at most three each); sums and scales.
         // Every lane loads (a clamped index where it has no word of its own) and the stores are masked.
         const int t = threadIdx.x;
         const uq_t *q_src = reinterpret_cast<const uq_t *>(aq);
         const uq_t *s0 = q_src + min(t, NB * 16 - 1), *s1 = q_src + min(t + 64 * WAVES, NB * 16 - 1);
+        const uq_t *s1b = q_src + min(t + 128 * WAVES, NB * 16 - 1);
         const uint32_t *s2 = reinterpret_cast<const uint32_t *>(absums) + min(t, NB * 8 - 1);
         const float *s3 = ad + min(t, NB - 1);
         asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv) : "v"(s0) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv2) : "v"(s1) : "memory");
+        if (NB * 16 > 128 * WAVES) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv3) : "v"(s1b) : "memory");
         asm volatile("global_load_dword %0, %1, off" : "=v"(bv) : "v"(s2) : "memory");
         asm volatile("global_load_dword %0, %1, off" : "=v"(dv) : "v"(s3) : "memory");
     }
     // (a wavefront past the matrix fetches the last span and stores nothing)
     {
-        const size_t span_c = min(span, (bytes - 1) / 9216);
-        const uint8_t *src = W + span_c * 9216;
-        const uint32_t left = (uint32_t)min((size_t)9216, bytes - span_c * 9216);  // (the last span may be short)
-        const uint32_t slot = lds_address(sw) + (uint32_t)wave * 9216;
+        const size_t span_c = min(span, (bytes - 1) / SPAN);
+        const uint8_t *src = W + span_c * SPAN;
+        const uint32_t left = (uint32_t)min((size_t)SPAN, bytes - span_c * SPAN);  // (the last span may be short)
+        const uint32_t slot = lds_address(sw) + (uint32_t)wave * SPAN;
 #pragma unroll
-        for (int c = 0; c < 9; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+        for (int c = 0; c < PIECES; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
     }
 
     // ---- the activation into LDS ----
     if (MODE == MODE_FUSED) {
-        // the activation's loads are older than the span's nine
+        // the activation's loads are older than the span's nine (Q5_K: eleven)
         // (one wait that names them all, so that the blocks' quantizations can be interleaved)
         constexpr int XB = (NB + WAVES - 1) / WAVES;
-        if (XB == 1) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]));
-        else if (XB == 2) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]));
-        else if (XB == 3) asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]));
-        else if (XB == 4)
-            asm volatile("s_waitcnt vmcnt(9)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]));
-        else
-            asm volatile("s_waitcnt vmcnt(9)"
+        // (exactly the registers there are: an operand named twice would be copied in front of the wait)
+        static_assert(XB >= 1 && XB <= 8, "up to eight blocks of the activation a wavefront");
+        if constexpr (XB == 1) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xv[0]) : "n"(PIECES));
+        if constexpr (XB == 2) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]) : "n"(PIECES));
+        if constexpr (XB == 3)
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]) : "n"(PIECES));
+        if constexpr (XB == 4)
+            asm volatile("s_waitcnt vmcnt(%4)"
+                         : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0])
+                         : "n"(PIECES));
+        if constexpr (XB == 5)
+            asm volatile("s_waitcnt vmcnt(%5)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
-                           "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0]), "+v"(xv[XB > 7 ? 7 : 0]));
+                           "+v"(xv[XB > 4 ? 4 : 0])
+                         : "n"(PIECES));
+        if constexpr (XB == 6)
+            asm volatile("s_waitcnt vmcnt(%6)"
+                         : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
+                           "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0])
+                         : "n"(PIECES));
+        if constexpr (XB == 7)
+            asm volatile("s_waitcnt vmcnt(%7)"
+                         : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
+                           "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0])
+                         : "n"(PIECES));
+        if constexpr (XB == 8)
+            asm volatile("s_waitcnt vmcnt(%8)"
+                         : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
+                           "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0]), "+v"(xv[XB > 7 ? 7 : 0])
+                         : "n"(PIECES));
 #pragma unroll
         for (int i = 0; i < XB; i++) {
             const int b = wave + i * WAVES;
@@ -428,12 +456,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
             }
         }
     } else {
-        asm volatile("s_waitcnt vmcnt(9)" : "+v"(qv), "+v"(qv2), "+v"(bv), "+v"(dv));  // (older than the span's nine)
+        asm volatile("s_waitcnt vmcnt(%5)" : "+v"(qv), "+v"(qv2), "+v"(qv3), "+v"(bv), "+v"(dv) : "n"(PIECES));  // (older than the span's)
         auto put = [&](int t, uq_t v) {  // word t of the quants: block t / 16, word t % 16 of it
             if (t < NB * 16) lds_store128(lds_address(sq + (t >> 4) * LINES_ACT_STRIDE + (t & 15) * 16), v);
         };
         put(threadIdx.x, qv);
         if (NB * 16 > 64 * WAVES) put(threadIdx.x + 64 * WAVES, qv2);
+        if (NB * 16 > 128 * WAVES) put(threadIdx.x + 128 * WAVES, qv3);
         if ((int)threadIdx.x < NB * 8)
             lds_store32(lds_address(sbs + threadIdx.x), (uint32_t)((int)(int16_t)(bv & 0xffff) + (int)(int16_t)(bv >> 16)));
         if ((int)threadIdx.x < NB) lds_store32(lds_address(sd + threadIdx.x), __float_as_uint(dv));
@@ -446,8 +475,15 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
 
     // ---- lane l multiplies block l of the span ----
     const int b = lane % NB;
-    const uint4 *blk = reinterpret_cast<const uint4 *>(sw + wave * 9216 + lane * Q4_K_BYTES);
+    const uint4 *blk = reinterpret_cast<const uint4 *>(sw + wave * SPAN + lane * BB);
     const uint4 hd = blk[0];
+    const uint4 fa = Q5 ? blk[1] : make_uint4(0u, 0u, 0u, 0u), fb = Q5 ? blk[2] : make_uint4(0u, 0u, 0u, 0u);  // fifth bits
+    constexpr int QS = Q5 ? 3 : 1;  // where the nibbles start, in 16-byte words
+    // a word of nibbles (shifted down by 4 for the high ones) under the fifth bits of sub-block j
+    auto code = [&](uint32_t nib, uint32_t fifth, int j) {
+        const uint32_t q4 = nib & 0x0f0f0f0fu;
+        return Q5 ? (((fifth >> j) & 0x01010101u) << 4) | q4 : q4;
+    };
     const uint32_t sc_lo = hd.y & 0x3f3f3f3fu, m_lo = hd.z & 0x3f3f3f3fu;
     const uint32_t sc_hi = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
     const uint32_t m_hi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
@@ -455,25 +491,25 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
     int s1 = 0;
 #pragma unroll
     for (int p = 0; p < 4; p++) {  // the 32 bytes qs[32p..]: sub-block 2p in their low nibbles, 2p+1 in their high ones
-        const uint4 qa = blk[1 + 2 * p], qb = blk[2 + 2 * p];
+        const uint4 qa = blk[QS + 2 * p], qb = blk[QS + 1 + 2 * p];
         const uint4 a0 = ap[4 * p], a1 = ap[4 * p + 1], a2 = ap[4 * p + 2], a3 = ap[4 * p + 3];
         int lo = 0, hi = 0;
-        lo = dot4(qa.x & 0x0f0f0f0fu, a0.x, lo);
-        lo = dot4(qa.y & 0x0f0f0f0fu, a0.y, lo);
-        lo = dot4(qa.z & 0x0f0f0f0fu, a0.z, lo);
-        lo = dot4(qa.w & 0x0f0f0f0fu, a0.w, lo);
-        lo = dot4(qb.x & 0x0f0f0f0fu, a1.x, lo);
-        lo = dot4(qb.y & 0x0f0f0f0fu, a1.y, lo);
-        lo = dot4(qb.z & 0x0f0f0f0fu, a1.z, lo);
-        lo = dot4(qb.w & 0x0f0f0f0fu, a1.w, lo);
-        hi = dot4((qa.x >> 4) & 0x0f0f0f0fu, a2.x, hi);
-        hi = dot4((qa.y >> 4) & 0x0f0f0f0fu, a2.y, hi);
-        hi = dot4((qa.z >> 4) & 0x0f0f0f0fu, a2.z, hi);
-        hi = dot4((qa.w >> 4) & 0x0f0f0f0fu, a2.w, hi);
-        hi = dot4((qb.x >> 4) & 0x0f0f0f0fu, a3.x, hi);
-        hi = dot4((qb.y >> 4) & 0x0f0f0f0fu, a3.y, hi);
-        hi = dot4((qb.z >> 4) & 0x0f0f0f0fu, a3.z, hi);
-        hi = dot4((qb.w >> 4) & 0x0f0f0f0fu, a3.w, hi);
+        lo = dot4(code(qa.x, fa.x, 2 * p), a0.x, lo);
+        lo = dot4(code(qa.y, fa.y, 2 * p), a0.y, lo);
+        lo = dot4(code(qa.z, fa.z, 2 * p), a0.z, lo);
+        lo = dot4(code(qa.w, fa.w, 2 * p), a0.w, lo);
+        lo = dot4(code(qb.x, fb.x, 2 * p), a1.x, lo);
+        lo = dot4(code(qb.y, fb.y, 2 * p), a1.y, lo);
+        lo = dot4(code(qb.z, fb.z, 2 * p), a1.z, lo);
+        lo = dot4(code(qb.w, fb.w, 2 * p), a1.w, lo);
+        hi = dot4(code(qa.x >> 4, fa.x, 2 * p + 1), a2.x, hi);
+        hi = dot4(code(qa.y >> 4, fa.y, 2 * p + 1), a2.y, hi);
+        hi = dot4(code(qa.z >> 4, fa.z, 2 * p + 1), a2.z, hi);
+        hi = dot4(code(qa.w >> 4, fa.w, 2 * p + 1), a2.w, hi);
+        hi = dot4(code(qb.x >> 4, fb.x, 2 * p + 1), a3.x, hi);
+        hi = dot4(code(qb.y >> 4, fb.y, 2 * p + 1), a3.y, hi);
+        hi = dot4(code(qb.z >> 4, fb.z, 2 * p + 1), a3.z, hi);
+        hi = dot4(code(qb.w >> 4, fb.w, 2 * p + 1), a3.w, hi);
         const uint32_t scw = (p < 2 ? sc_lo : sc_hi) >> ((p & 1) * 16);
         s1 += __mul24((int)(scw & 0xff), lo) + __mul24((int)((scw >> 8) & 0xff), hi);
     }
@@ -582,22 +618,23 @@ bool fused_gemv_fits(const frk_weights *w) {
 // rows stored back to back whose block count divides 64
 static bool lines_kernel_fits(const frk_weights *w) {
     const size_t nb = w->cols / QK_K;
-    return (nb == 8 || nb == 16 || nb == 32 || nb == 64) && w->layout.row_stride == nb * Q4_K_BYTES;
+    const size_t bb = w->kind == FRK_KIND_Q5_K ? Q5_K_BYTES : Q4_K_BYTES;
+    return (nb == 8 || nb == 16 || nb == 32 || nb == 64) && w->layout.row_stride == nb * bb;
 }
-template <int NB, int MODE, int WAVES>
+template <int NB, int MODE, int WAVES, bool Q5 = false>
 static int launch_q4_k_lines_as(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
-    constexpr size_t shmem = (size_t)NB * (LINES_ACT_STRIDE + 32 + 4) + (size_t)WAVES * 9216;
+    constexpr size_t shmem = (size_t)NB * (LINES_ACT_STRIDE + 32 + 4) + (size_t)WAVES * 64 * (Q5 ? Q5_K_BYTES : Q4_K_BYTES);
     static_assert(shmem <= 160 * 1024, "LDS of a CU");
     const size_t spans = (w->rows * (size_t)NB + 63) / 64;
     const unsigned grid = (unsigned)((spans + WAVES - 1) / WAVES);
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_lines_kernel<NB, MODE, WAVES>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv lines, LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemv_q4_k_lines_kernel<NB, MODE, WAVES>), dim3(grid), dim3(64 * WAVES), shmem, s, w->dev, (int)w->rows, x,
+    hipLaunchKernelGGL((gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5>), dim3(grid), dim3(64 * WAVES), shmem, s, w->dev, (int)w->rows, x,
                        a.q, a.d, a.bsums, y);
     FRK_LAUNCH_CHECK("gemv_q4_k_lines");
     return FRK_OK;
@@ -623,6 +660,24 @@ int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t
     if (lines_kernel_fits(w)) return launch_q4_k_lines<MODE_PREQ_LDS>(w, nullptr, a, y, s);
     if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, nullptr, a, y, s);
     return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, nullptr, a, y, s);
+}
+// Q5_K rows of 8, 16, 32 or 64 blocks on the same kernel.  Wavefronts to a workgroup, measured (one-launch form,
+// us): 14336x4096 -- 4: 10.4, 5: 11.7, 6: 11.6, 7: 12.0, 8: 10.9; 4096x8192 -- 4: 9.0, 6: 10.9, 8: 7.3;
+// 8192x2048 -- 4: 4.1, 8: 4.6.  (An 11 KB span a wavefront: four wavefronts make three workgroups a CU.)
+bool q5_k_lines_gemv_fits(const frk_weights *w) { return w->kind == FRK_KIND_Q5_K && lines_kernel_fits(w); }
+template <int MODE>
+static int launch_q5_k_lines(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K);
+    if (nb == 8) return launch_q4_k_lines_as<8, MODE, 4, true>(w, x, a, y, s);
+    if (nb == 16) return launch_q4_k_lines_as<16, MODE, 4, true>(w, x, a, y, s);
+    if (nb == 32) return launch_q4_k_lines_as<32, MODE, 8, true>(w, x, a, y, s);
+    return launch_q4_k_lines_as<64, MODE, 8, true>(w, x, a, y, s);
+}
+int launch_gemv_q5_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    return launch_q5_k_lines<MODE_FUSED>(w, x, Q8KActs{nullptr, nullptr, nullptr}, y, s);
+}
+int launch_gemv_q5_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    return launch_q5_k_lines<MODE_PREQ_LDS>(w, nullptr, a, y, s);
 }
 // ys[i] = ws[i] . x for 2..4 Q4_K matrices of one row length (fused_gemv_fits), one launch
 int launch_gemv_q4_k_group(const frk_weights *const *ws, size_t n, const float *x, float *const *ys, hipStream_t s) {

@@ -150,6 +150,11 @@ struct Q8KActs {  // Q8_K activations in HBM, struct-of-arrays per activation ro
 };
 int launch_gemv_q4_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q5_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
+// Q5_K rows of 2048 / 4096 / 8192 / 16384 columns stored back to back: the whole-cache-line kernel, with the
+// activation's quantization inside the launch or from Q8_K activations (frk_gemv_fused.hip)
+bool q5_k_lines_gemv_fits(const frk_weights *w);
+int launch_gemv_q5_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_q5_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 // one-launch kernels (activation quantized inside the GEMV); cols <= 16384
 // rows of at most this many columns have a one-launch Q4_K GEMV

@@ -481,6 +481,7 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q5_K:
     case FRK_KIND_Q6_K: {
         if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
+        if (q5_k_lines_gemv_fits(w)) return launch_gemv_q5_k_fused(w, x, y, s);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
         if (rc) return rc;
@@ -523,7 +524,9 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     if (w->kind == FRK_KIND_Q4_K)
         return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
                                   : launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
-    if (w->kind == FRK_KIND_Q5_K) return launch_gemv_q5_k(w, a, y, (hipStream_t)stream);
+    if (w->kind == FRK_KIND_Q5_K)
+        return q5_k_lines_gemv_fits(w) ? launch_gemv_q5_k_preq(w, a, y, (hipStream_t)stream)
+                                       : launch_gemv_q5_k(w, a, y, (hipStream_t)stream);
     if (w->kind == FRK_KIND_Q6_K)
         return direct_gemv_fits(w) ? launch_gemv_q6_k_direct(w, a, y, (hipStream_t)stream)
                                    : launch_gemv_q6_k(w, a, y, (hipStream_t)stream);

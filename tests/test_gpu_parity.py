@@ -224,17 +224,19 @@ def test_gemv_matches_the_oracle(fa, kind, rows, cols):
 
 @pytest.mark.parametrize("rows,cols", [(5, 2048), (8, 2048), (100, 2048), (1, 4096), (4, 4096), (131, 4096), (3, 8192), (50, 8192),
                                        (1, 16384), (33, 16384)])
-def test_q4_k_gemv_over_whole_cache_lines(fa, rows, cols):
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K])
+def test_q4_k_gemv_over_whole_cache_lines(fa, kind, rows, cols):
     """Rows of 2048 .. 16384 columns take the kernel that gives a wavefront 64 consecutive blocks (8, 4, 2 or
     1 whole rows): row counts that fill a span, fall short of one, and leave a short last span -- with the
     quantization inside the launch and from activations quantized beforehand, which must agree bit for bit
-    (the same integers, the same float order)."""
+    (the same integers, the same float order).  Q5_K runs on the same kernel, the fifth bits put over the
+    nibbles on their way into the dot."""
     from frink_amd import synth
-    data = make_weights(fo.Q4_K, rows, cols, seed=rows + cols)
+    data = make_weights(kind, rows, cols, seed=rows + cols)
     x = synth.activations(rows * 3 + cols, 1, cols, outlier_frac=0.01)[0]
-    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    w = fa.Weights.from_host(kind, data, rows, cols)
     xd = to_dev(x)
-    want = fo.gemv(fo.Q4_K, data, rows, cols, x)
+    want = fo.gemv(kind, data, rows, cols, x)
     got = w.gemv(xd).cpu().numpy()
     assert_rows_close(got[None], want[None], "gemv over lines %dx%d" % (rows, cols))
     pre = w.gemv_q8k(fa.quantize_q8_k(xd)).cpu().numpy()
