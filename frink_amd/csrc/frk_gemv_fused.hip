@@ -339,6 +339,56 @@ __global__ __launch_bounds__(MAXT) void gemv_q4_k_fused_kernel(
 // every sub-block, sub-block j in bit j --, the nibbles; dot_q5_k_q8, crates/frink-quant/src/lib.rs:886-938):
 // a span is 11 KB, and a weight's fifth bit is put over its nibble on the way into v_dot4.
 constexpr int LINES_ACT_STRIDE = QK_K + 16;
+// One block of a row against the matching block of the activation, both in LDS: dot_q4_k_q8's (Q5: dot_q5_k_q8's)
+// integers and per-block float expression.  blk: the block's 16-byte words; ap: the activation block's quants;
+// bs32: its eight 32-wide sums; da: its scale.
+template <bool Q5>
+__device__ __forceinline__ float lines_block_dot(const uint4 *blk, const uint4 *ap, const int *bs32, float da) {
+    const uint4 hd = blk[0];
+    const uint4 fa = Q5 ? blk[1] : make_uint4(0u, 0u, 0u, 0u), fb = Q5 ? blk[2] : make_uint4(0u, 0u, 0u, 0u);  // fifth bits
+    constexpr int QS = Q5 ? 3 : 1;  // where the nibbles start, in 16-byte words
+    // a word of nibbles (shifted down by 4 for the high ones) under the fifth bits of sub-block j
+    auto code = [&](uint32_t nib, uint32_t fifth, int j) {
+        const uint32_t q4 = nib & 0x0f0f0f0fu;
+        return Q5 ? (((fifth >> j) & 0x01010101u) << 4) | q4 : q4;
+    };
+    const uint32_t sc_lo = hd.y & 0x3f3f3f3fu, m_lo = hd.z & 0x3f3f3f3fu;
+    const uint32_t sc_hi = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
+    const uint32_t m_hi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
+    int s1 = 0;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {  // the 32 bytes qs[32p..]: sub-block 2p in their low nibbles, 2p+1 in their high ones
+        const uint4 qa = blk[QS + 2 * p], qb = blk[QS + 1 + 2 * p];
+        const uint4 a0 = ap[4 * p], a1 = ap[4 * p + 1], a2 = ap[4 * p + 2], a3 = ap[4 * p + 3];
+        int lo = 0, hi = 0;
+        lo = dot4(code(qa.x, fa.x, 2 * p), a0.x, lo);
+        lo = dot4(code(qa.y, fa.y, 2 * p), a0.y, lo);
+        lo = dot4(code(qa.z, fa.z, 2 * p), a0.z, lo);
+        lo = dot4(code(qa.w, fa.w, 2 * p), a0.w, lo);
+        lo = dot4(code(qb.x, fb.x, 2 * p), a1.x, lo);
+        lo = dot4(code(qb.y, fb.y, 2 * p), a1.y, lo);
+        lo = dot4(code(qb.z, fb.z, 2 * p), a1.z, lo);
+        lo = dot4(code(qb.w, fb.w, 2 * p), a1.w, lo);
+        hi = dot4(code(qa.x >> 4, fa.x, 2 * p + 1), a2.x, hi);
+        hi = dot4(code(qa.y >> 4, fa.y, 2 * p + 1), a2.y, hi);
+        hi = dot4(code(qa.z >> 4, fa.z, 2 * p + 1), a2.z, hi);
+        hi = dot4(code(qa.w >> 4, fa.w, 2 * p + 1), a2.w, hi);
+        hi = dot4(code(qb.x >> 4, fb.x, 2 * p + 1), a3.x, hi);
+        hi = dot4(code(qb.y >> 4, fb.y, 2 * p + 1), a3.y, hi);
+        hi = dot4(code(qb.z >> 4, fb.z, 2 * p + 1), a3.z, hi);
+        hi = dot4(code(qb.w >> 4, fb.w, 2 * p + 1), a3.w, hi);
+        const uint32_t scw = (p < 2 ? sc_lo : sc_hi) >> ((p & 1) * 16);
+        s1 += __mul24((int)(scw & 0xff), lo) + __mul24((int)((scw >> 8) & 0xff), hi);
+    }
+    const int4 bsa = *reinterpret_cast<const int4 *>(bs32), bsb = *reinterpret_cast<const int4 *>(bs32 + 4);
+    int s2 = __mul24((int)(m_lo & 0xff), bsa.x) + __mul24((int)((m_lo >> 8) & 0xff), bsa.y) +
+             __mul24((int)((m_lo >> 16) & 0xff), bsa.z) + __mul24((int)(m_lo >> 24), bsa.w);
+    s2 += __mul24((int)(m_hi & 0xff), bsb.x) + __mul24((int)((m_hi >> 8) & 0xff), bsb.y) +
+          __mul24((int)((m_hi >> 16) & 0xff), bsb.z) + __mul24((int)(m_hi >> 24), bsb.w);
+    const float d = h2f(hd.x & 0xffffu), dmin = h2f(hd.x >> 16);
+    return (d * da) * (float)s1 - (dmin * da) * (float)s2;
+}
+
 template <int NB, int MODE, int WAVES, bool Q5 = false>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8_t *__restrict__ W, int rows,
                                                                     const float *__restrict__ x,
@@ -475,56 +525,128 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
 
     // ---- lane l multiplies block l of the span ----
     const int b = lane % NB;
-    const uint4 *blk = reinterpret_cast<const uint4 *>(sw + wave * SPAN + lane * BB);
-    const uint4 hd = blk[0];
-    const uint4 fa = Q5 ? blk[1] : make_uint4(0u, 0u, 0u, 0u), fb = Q5 ? blk[2] : make_uint4(0u, 0u, 0u, 0u);  // fifth bits
-    constexpr int QS = Q5 ? 3 : 1;  // where the nibbles start, in 16-byte words
-    // a word of nibbles (shifted down by 4 for the high ones) under the fifth bits of sub-block j
-    auto code = [&](uint32_t nib, uint32_t fifth, int j) {
-        const uint32_t q4 = nib & 0x0f0f0f0fu;
-        return Q5 ? (((fifth >> j) & 0x01010101u) << 4) | q4 : q4;
-    };
-    const uint32_t sc_lo = hd.y & 0x3f3f3f3fu, m_lo = hd.z & 0x3f3f3f3fu;
-    const uint32_t sc_hi = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
-    const uint32_t m_hi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
-    const uint4 *ap = reinterpret_cast<const uint4 *>(sq + b * LINES_ACT_STRIDE);
-    int s1 = 0;
-#pragma unroll
-    for (int p = 0; p < 4; p++) {  // the 32 bytes qs[32p..]: sub-block 2p in their low nibbles, 2p+1 in their high ones
-        const uint4 qa = blk[QS + 2 * p], qb = blk[QS + 1 + 2 * p];
-        const uint4 a0 = ap[4 * p], a1 = ap[4 * p + 1], a2 = ap[4 * p + 2], a3 = ap[4 * p + 3];
-        int lo = 0, hi = 0;
-        lo = dot4(code(qa.x, fa.x, 2 * p), a0.x, lo);
-        lo = dot4(code(qa.y, fa.y, 2 * p), a0.y, lo);
-        lo = dot4(code(qa.z, fa.z, 2 * p), a0.z, lo);
-        lo = dot4(code(qa.w, fa.w, 2 * p), a0.w, lo);
-        lo = dot4(code(qb.x, fb.x, 2 * p), a1.x, lo);
-        lo = dot4(code(qb.y, fb.y, 2 * p), a1.y, lo);
-        lo = dot4(code(qb.z, fb.z, 2 * p), a1.z, lo);
-        lo = dot4(code(qb.w, fb.w, 2 * p), a1.w, lo);
-        hi = dot4(code(qa.x >> 4, fa.x, 2 * p + 1), a2.x, hi);
-        hi = dot4(code(qa.y >> 4, fa.y, 2 * p + 1), a2.y, hi);
-        hi = dot4(code(qa.z >> 4, fa.z, 2 * p + 1), a2.z, hi);
-        hi = dot4(code(qa.w >> 4, fa.w, 2 * p + 1), a2.w, hi);
-        hi = dot4(code(qb.x >> 4, fb.x, 2 * p + 1), a3.x, hi);
-        hi = dot4(code(qb.y >> 4, fb.y, 2 * p + 1), a3.y, hi);
-        hi = dot4(code(qb.z >> 4, fb.z, 2 * p + 1), a3.z, hi);
-        hi = dot4(code(qb.w >> 4, fb.w, 2 * p + 1), a3.w, hi);
-        const uint32_t scw = (p < 2 ? sc_lo : sc_hi) >> ((p & 1) * 16);
-        s1 += __mul24((int)(scw & 0xff), lo) + __mul24((int)((scw >> 8) & 0xff), hi);
-    }
-    const int4 bsa = *reinterpret_cast<const int4 *>(sbs + b * 8), bsb = *reinterpret_cast<const int4 *>(sbs + b * 8 + 4);
-    int s2 = __mul24((int)(m_lo & 0xff), bsa.x) + __mul24((int)((m_lo >> 8) & 0xff), bsa.y) +
-             __mul24((int)((m_lo >> 16) & 0xff), bsa.z) + __mul24((int)(m_lo >> 24), bsa.w);
-    s2 += __mul24((int)(m_hi & 0xff), bsb.x) + __mul24((int)((m_hi >> 8) & 0xff), bsb.y) +
-          __mul24((int)((m_hi >> 16) & 0xff), bsb.z) + __mul24((int)(m_hi >> 24), bsb.w);
-    const float da = sd[b];
-    const float d = h2f(hd.x & 0xffffu), dmin = h2f(hd.x >> 16);
-    float v = (d * da) * (float)s1 - (dmin * da) * (float)s2;
+    float v = lines_block_dot<Q5>(reinterpret_cast<const uint4 *>(sw + wave * SPAN + lane * BB),
+                                  reinterpret_cast<const uint4 *>(sq + b * LINES_ACT_STRIDE), sbs + b * 8, sd[b]);
     const size_t row = span * RPS + lane / NB;
     if (row >= (size_t)rows) v = 0.0f;  // (a short last span: this lane's block is not there)
     v = part_sum<NB>(v);
     if (lane % NB == 0 && row < (size_t)rows) y[row] = v;
+}
+
+// The same for rows of ANY block count up to 64 (11008, 14336, 5120 ... columns): a wavefront's span is the
+// 64 / nb whole rows that fit 64 lanes -- contiguous bytes still, rows being stored back to back, though no
+// longer a whole number of kilobytes: the last of the nine (eleven) requests is clamped to the span's end
+// -- lanes past the span's blocks idle, and a row's blocks are added by a segmented shuffle in place of
+// the DPP butterfly (lane b of a row takes lane b + step's sum while that lane is in the row).  The
+// activation comes quantized (MODE_PREQ_LDS) or is quantized here, eight blocks a wavefront at most.
+template <int MODE, int WAVES, bool Q5 = false>
+__global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_rows_kernel(const uint8_t *__restrict__ W, int rows, int nb,
+                                                                   const float *__restrict__ x,
+                                                                   const int8_t *__restrict__ aq,
+                                                                   const float *__restrict__ ad,
+                                                                   const int16_t *__restrict__ absums,
+                                                                   float *__restrict__ y) {
+    constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES, SLOT = 64 * BB, PIECES = SLOT / 1024;
+    static_assert(WAVES >= 6 && (MODE != MODE_FUSED || WAVES >= 8), "64 blocks of activation: eight a wavefront, three words of quants a thread");
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    int8_t *sq = reinterpret_cast<int8_t *>(lds);                       // nb blocks of quants, 272 bytes apart
+    int *sbs = reinterpret_cast<int *>(lds + nb * LINES_ACT_STRIDE);    // nb x 8 sums over 32
+    float *sd = reinterpret_cast<float *>(lds + nb * LINES_ACT_STRIDE + nb * 32);
+    uint8_t *sw = lds + ((nb * (LINES_ACT_STRIDE + 32 + 4) + 15) & ~15);  // WAVES slots of 64 blocks
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rps = 64 / nb;  // rows of a span
+    const uint32_t span_bytes = (uint32_t)(rps * nb) * BB;
+    const size_t span = (size_t)blockIdx.x * WAVES + wave;
+    const size_t bytes = (size_t)rows * nb * BB;
+    const bool has_rows = span * span_bytes < bytes;
+
+    typedef float xv_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t uq_t __attribute__((ext_vector_type(4)));
+    xv_t xv[8];
+    uq_t qv = {0u, 0u, 0u, 0u}, qv2 = {0u, 0u, 0u, 0u}, qv3 = {0u, 0u, 0u, 0u};
+    uint32_t bv = 0, bv2 = 0;
+    float dv = 0.0f;
+    if (MODE == MODE_FUSED) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {  // (a block past the row's end: the last one again, not used)
+            const int b = min(wave + i * WAVES, nb - 1);
+            const float4 *src = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K) + lane;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xv[i]) : "v"(src) : "memory");
+        }
+    } else {
+        const int t = threadIdx.x;
+        const uq_t *q_src = reinterpret_cast<const uq_t *>(aq);
+        const uq_t *s0 = q_src + min(t, nb * 16 - 1), *s1 = q_src + min(t + 64 * WAVES, nb * 16 - 1);
+        const uq_t *s1b = q_src + min(t + 128 * WAVES, nb * 16 - 1);
+        // (nb * 8 <= 512 pairs of 16-wide sums over 64 * WAVES >= 384 threads: two a thread)
+        const uint32_t *s2 = reinterpret_cast<const uint32_t *>(absums) + min(t, nb * 8 - 1);
+        const uint32_t *s2b = reinterpret_cast<const uint32_t *>(absums) + min(t + 64 * WAVES, nb * 8 - 1);
+        const float *s3 = ad + min(t, nb - 1);
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv) : "v"(s0) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv2) : "v"(s1) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qv3) : "v"(s1b) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(bv) : "v"(s2) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(bv2) : "v"(s2b) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "=v"(dv) : "v"(s3) : "memory");
+    }
+    {
+        const size_t span_c = min(span, (bytes - 1) / span_bytes);
+        const uint8_t *src = W + span_c * span_bytes;
+        const uint32_t left = (uint32_t)min((size_t)span_bytes, bytes - span_c * span_bytes);
+        const uint32_t slot = lds_address(sw) + (uint32_t)wave * SLOT;
+#pragma unroll
+        for (int c = 0; c < PIECES; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+    }
+    if (MODE == MODE_FUSED) {
+        asm volatile("s_waitcnt vmcnt(%8)"
+                     : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]), "+v"(xv[4]), "+v"(xv[5]), "+v"(xv[6]), "+v"(xv[7])
+                     : "n"(PIECES));
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int b = wave + i * WAVES;
+            if (b < nb) {  // uniform across the wavefront
+                float d;
+                int bs;
+                const uint32_t packed = quantize_q8_k_lane(make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w), d, bs);
+                const int bs32 = bs + __shfl_xor(bs, 4);
+                lds_store32(lds_address(sq + b * LINES_ACT_STRIDE) + lane * 4, packed);
+                if ((lane & 7) == 0) lds_store32(lds_address(sbs + b * 8) + (lane >> 3) * 4, (uint32_t)bs32);
+                if (lane == 0) lds_store32(lds_address(sd + b), __float_as_uint(d));
+            }
+        }
+    } else {
+        asm volatile("s_waitcnt vmcnt(%6)" : "+v"(qv), "+v"(qv2), "+v"(qv3), "+v"(bv), "+v"(bv2), "+v"(dv) : "n"(PIECES));
+        auto put = [&](int t, uq_t v) {
+            if (t < nb * 16) lds_store128(lds_address(sq + (t >> 4) * LINES_ACT_STRIDE + (t & 15) * 16), v);
+        };
+        put(threadIdx.x, qv);
+        put(threadIdx.x + 64 * WAVES, qv2);
+        put(threadIdx.x + 128 * WAVES, qv3);
+        auto put_sum = [&](int t, uint32_t pair) {  // two 16-wide sums make a 32-wide one
+            if (t < nb * 8) lds_store32(lds_address(sbs + t), (uint32_t)((int)(int16_t)(pair & 0xffff) + (int)(int16_t)(pair >> 16)));
+        };
+        put_sum(threadIdx.x, bv);
+        put_sum(threadIdx.x + 64 * WAVES, bv2);
+        if ((int)threadIdx.x < nb) lds_store32(lds_address(sd + threadIdx.x), __float_as_uint(dv));
+    }
+    lds_barrier();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (!has_rows) return;
+
+    const int r_in = lane / nb, b_in = lane - r_in * nb;  // this lane's row of the span and block of the row
+    const bool live = r_in < rps;
+    const int b = live ? b_in : 0;
+    float v = lines_block_dot<Q5>(reinterpret_cast<const uint4 *>(sw + wave * SLOT + (live ? lane : 0) * BB),
+                                  reinterpret_cast<const uint4 *>(sq + b * LINES_ACT_STRIDE), sbs + b * 8, sd[b]);
+    const size_t row = span * rps + r_in;
+    if (!live || row >= (size_t)rows) v = 0.0f;
+    for (int step = 1; step < nb; step <<= 1) {  // (uniform bound)
+        const float o = __shfl_down(v, step);
+        if (b_in + step < nb) v += o;
+    }
+    if (live && b_in == 0 && row < (size_t)rows) y[row] = v;
 }
 
 // ------------------------------------------------------------------ launchers
@@ -661,6 +783,62 @@ int launch_gemv_q4_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t
     if (w->cols <= 8192) return launch_q4_k_fused<MODE_PREQ_DIRECT>(w, nullptr, nullptr, a, y, s);
     return launch_q4_k_fused<MODE_PREQ_LDS>(w, nullptr, nullptr, a, y, s);
 }
+// rows of any block count up to 64, stored back to back: whole rows to a wavefront (gemv_q4_k_rows_kernel)
+bool rows_gemv_fits(const frk_weights *w) {
+    const size_t nb = w->cols / QK_K;
+    const size_t bb = w->kind == FRK_KIND_Q5_K ? Q5_K_BYTES : Q4_K_BYTES;
+    return (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K) && nb >= 1 && nb <= 64 && w->layout.row_stride == nb * bb;
+}
+template <int MODE, bool Q5, int WAVES = 8>
+static int launch_rows_as(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
+    constexpr size_t slot = 64 * (Q5 ? Q5_K_BYTES : Q4_K_BYTES);
+    const int nb = (int)(w->cols / QK_K);
+    const size_t shmem = (((size_t)nb * (LINES_ACT_STRIDE + 32 + 4) + 15) & ~(size_t)15) + WAVES * slot;
+    const size_t spans = (w->rows + (size_t)(64 / nb) - 1) / (size_t)(64 / nb);
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        constexpr size_t most = ((64 * (LINES_ACT_STRIDE + 32 + 4) + 15) & ~15) + WAVES * slot;
+        static_assert(most <= 160 * 1024, "LDS of a CU");
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_rows_kernel<MODE, WAVES, Q5>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv rows): %s", hipGetErrorString(e));
+        sized = true;
+    }
+    hipLaunchKernelGGL((gemv_q4_k_rows_kernel<MODE, WAVES, Q5>), dim3((unsigned)((spans + WAVES - 1) / WAVES)), dim3(64 * WAVES),
+                       shmem, s, w->dev, (int)w->rows, nb, x, a.q, a.d, a.bsums, y);
+    FRK_LAUNCH_CHECK("gemv_q4_k_rows");
+    return FRK_OK;
+}
+int launch_gemv_rows_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const Q8KActs none{nullptr, nullptr, nullptr};
+    return w->kind == FRK_KIND_Q5_K ? launch_rows_as<MODE_FUSED, true>(w, x, none, y, s) : launch_rows_as<MODE_FUSED, false>(w, x, none, y, s);
+}
+// (six wavefronts to a workgroup: two workgroups' slots and activations fit a CU's LDS up to 64 blocks a row;
+// measured at 4096x14336 from quantized activations, kernel + the quantization launch: 6: 11.8 us, 7: 12.1,
+// 8: 12.6, 10: 13.9, 14: 15.4)
+int launch_gemv_rows_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
+    // (Q5_K's slots are 11 KB: six wavefronts would be alone on a CU, eight are more)
+    return w->kind == FRK_KIND_Q5_K ? launch_rows_as<MODE_PREQ_LDS, true, 8>(w, nullptr, a, y, s)
+                                    : launch_rows_as<MODE_PREQ_LDS, false, 6>(w, nullptr, a, y, s);
+}
+// Which form a decode GEMV of this matrix takes, by measurement (Q4_K, us; one launch with the quantization
+// inside on the per-lane kernel / on the whole-rows kernel / a quantization launch and the whole-rows kernel):
+//   4096x14336 15.3 / 15.3 / 11.8    4096x11008 13.6 / 13.2 / 11.0    5120x13824 19.0 / 21.2 / 13.6
+//   4096x16384 15.2 (whole lines) / 16.2 / 12.3 -- a workgroup quantizing 56 KB of activation for 74 KB of
+//   weights is what a long row costs in one launch;
+//   5120x5120 7.8 / 5.9 / 6.9    6144x6144 8.7 / 8.8 / 9.0    8192x3072 5.5 / 5.2 / 6.7    3072x3072 3.7 / 4.6 / 5.9
+//   2560x2560 3.4 / 4.5 / 5.8
+// Rows of 8, 16 and 32 blocks have the whole-cache-line kernel (14336x4096: 8.2 / 8.9 / 10.3).
+int rows_gemv_form(const frk_weights *w) {
+    if (!rows_gemv_fits(w)) return ROWS_FORM_NONE;
+    const size_t nb = w->cols / QK_K;
+    // (Q5_K rows of 64 blocks: the whole-cache-line kernel in one launch is ahead, 9.2 us against 12.2 at 2048x16384)
+    if (nb == 64 && w->kind == FRK_KIND_Q5_K) return ROWS_FORM_NONE;
+    if (nb > 32) return ROWS_FORM_QUANTIZED;
+    if (nb > 16 && nb < 32) return ROWS_FORM_ONE_LAUNCH;
+    return ROWS_FORM_NONE;
+}
+
 // Q5_K rows of 8, 16, 32 or 64 blocks on the same kernel.  Wavefronts to a workgroup, measured (one-launch form,
 // us): 14336x4096 -- 4: 10.4, 5: 11.7, 6: 11.6, 7: 12.0, 8: 10.9; 4096x8192 -- 4: 9.0, 6: 10.9, 8: 7.3;
 // 8192x2048 -- 4: 4.1, 8: 4.6.  (An 11 KB span a wavefront: four wavefronts make three workgroups a CU.)

@@ -153,6 +153,14 @@ int launch_gemv_q5_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 // Q5_K rows of 2048 / 4096 / 8192 / 16384 columns stored back to back: the whole-cache-line kernel, with the
 // activation's quantization inside the launch or from Q8_K activations (frk_gemv_fused.hip)
 bool q5_k_lines_gemv_fits(const frk_weights *w);
+// Q4_K / Q5_K rows of any block count up to 64 stored back to back: whole rows to a wavefront
+bool rows_gemv_fits(const frk_weights *w);
+// which form a decode GEMV of the matrix takes on that kernel: none (the other kernels are ahead), one launch
+// with the quantization inside, or a quantization launch and the kernel over Q8_K activations
+enum { ROWS_FORM_NONE = 0, ROWS_FORM_ONE_LAUNCH = 1, ROWS_FORM_QUANTIZED = 2 };
+int rows_gemv_form(const frk_weights *w);
+int launch_gemv_rows_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
+int launch_gemv_rows_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q5_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_q5_k_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);

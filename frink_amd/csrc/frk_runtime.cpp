@@ -476,12 +476,21 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     }
     switch (w->kind) {
     case FRK_KIND_Q4_K:
-        if (fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
+    case FRK_KIND_Q5_K: {
+        const int form = rows_gemv_form(w);  // rows of 17..31 and of 33..64 blocks: whole rows to a wavefront
+        if (form == ROWS_FORM_ONE_LAUNCH) return launch_gemv_rows_fused(w, x, y, s);
+        if (form == ROWS_FORM_QUANTIZED) {
+            Q8KActs a;
+            int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
+            if (rc) return rc;
+            return launch_gemv_rows_preq(w, a, y, s);
+        }
+        if (w->kind == FRK_KIND_Q4_K && fused_gemv_fits(w)) return launch_gemv_q4_k_fused(w, x, y, s);
+        if (q5_k_lines_gemv_fits(w)) return launch_gemv_q5_k_fused(w, x, y, s);
+    }
         [[fallthrough]];
-    case FRK_KIND_Q5_K:
     case FRK_KIND_Q6_K: {
         if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
-        if (q5_k_lines_gemv_fits(w)) return launch_gemv_q5_k_fused(w, x, y, s);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
         if (rc) return rc;
@@ -521,6 +530,8 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     clear_error();
     if (!w || !q || !d || !bsums || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_q8k_dev: null argument");
     Q8KActs a{q, d, bsums};
+    if ((w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K) && rows_gemv_form(w) == ROWS_FORM_QUANTIZED)
+        return launch_gemv_rows_preq(w, a, y, (hipStream_t)stream);
     if (w->kind == FRK_KIND_Q4_K)
         return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
                                   : launch_gemv_q4_k(w, a, y, (hipStream_t)stream);
