@@ -359,8 +359,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_0_f32_shared_kernel(const 
 // rows of at most 64*4 units, and long enough that a wavefront per row is not mostly idle lanes
 bool direct_gemv_fits(const frk_weights *w) {
     const size_t units = w->kind == FRK_KIND_Q6_K ? w->cols / QK_K * 4 : w->cols / Q8_0_ELEMS * 2;
-    // (Q8_0: up to eight units a lane, 8192 columns)
-    return (w->kind == FRK_KIND_Q6_K || w->kind == FRK_KIND_Q8_0) && units > 32 && units <= (w->kind == FRK_KIND_Q8_0 ? 512u : 256u);
+    // (Q8_0: up to eight units a lane, 8192 columns; sixteen, 16384 columns, where the rows are many enough for the
+    // kernel that shares the activation through LDS)
+    if (w->kind == FRK_KIND_Q8_0) return units > 32 && (units <= 512 || (units <= 1024 && w->rows >= 1024));
+    return w->kind == FRK_KIND_Q6_K && units > 32 && units <= 256;
 }
 
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s) {
@@ -429,12 +431,28 @@ int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, 
 #define FRK_GO(UU)                                                                                                \
     hipLaunchKernelGGL((gemv_q8_0_f32_shared_kernel<UU, WAVES>), grid, block, 4096 * UU, s, w->dev, w->layout, (int)w->rows, nb, \
                        x, y)
+// (more than 48 KB of LDS: the kernel is told once)
+#define FRK_GO_BIG(UU)                                                                                             \
+    do {                                                                                                           \
+        static bool sized = false;                                                                                 \
+        if (!sized) {                                                                                              \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q8_0_f32_shared_kernel<UU, WAVES>), \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * UU);             \
+            if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv q8_0, LDS): %s", hipGetErrorString(e)); \
+            sized = true;                                                                                          \
+        }                                                                                                          \
+        FRK_GO(UU);                                                                                                \
+    } while (0)
         if (u == 1) FRK_GO(1);
         else if (u == 2) FRK_GO(2);
         else if (u == 3) FRK_GO(3);
         else if (u == 4) FRK_GO(4);
         else if (u <= 6) FRK_GO(6);
-        else FRK_GO(8);
+        else if (u <= 8) FRK_GO(8);
+        else if (u <= 11) FRK_GO(11);
+        else if (u <= 14) FRK_GO_BIG(14);
+        else FRK_GO_BIG(16);
+#undef FRK_GO_BIG
 #undef FRK_GO
         FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");
         return FRK_OK;

@@ -199,6 +199,8 @@ GEMV_SHAPES = [
     (fo.Q8_0, 64, 4096), (fo.Q8_0, 7, 32), (fo.Q8_0, 9, 544), (fo.Q8_0, 5, 2048),
     (fo.Q8_0, 1030, 4096), (fo.Q8_0, 1025, 8192), (fo.Q8_0, 40, 8192), (fo.Q8_0, 1100, 5120), (fo.Q8_0, 33, 6144),
     (fo.Q8_0, 12, 16384),
+    # Q8_0 rows of 8224 .. 16384 columns with at least 1024 rows: the activation shared through LDS, 11 to 16 units a lane
+    (fo.Q8_0, 1024, 14336), (fo.Q8_0, 1500, 11008), (fo.Q8_0, 1027, 16384), (fo.Q8_0, 1100, 8704), (fo.Q8_0, 1030, 10240),
 ]
 
 
