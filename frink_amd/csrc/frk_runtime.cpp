@@ -544,11 +544,12 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d)", w->kind);
 }
 
-// Q4_K: up to two launches of the thin kernel (16 rows each: 15 us at 14336x4096, 10 us at 4096x4096)
-// are ahead of the matrix-core GEMM (28 us and 18 us there for 33..64 rows, its blocks split between
-// workgroups)
+// Q4_K: the thin kernel takes 16 rows a launch.  Measured (us; thin launches / the matrix-core GEMM, whose cost
+// is flat up to 64 rows): 4096x4096 8.8 at 16 rows, 14.5 at 32 / 17.6; 1024x4096 7.5, 12.9 / 15.0 -- two thin
+// launches are ahead for small matrices; 14336x4096 23.9, 44.9 / 24.9; 5120x5120 15.1, 26.8 / 20.4; 4096x11008
+// 25.3 at 16 rows / 23.7 -- from 20 M weights on a second thin launch is not.
 static bool q4_k_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
-    const size_t q4k_thin_rows = 32;
+    const size_t q4k_thin_rows = w->rows * w->cols > (size_t)20 << 20 ? 16 : 32;
     return w->kind == FRK_KIND_Q4_K && batch > 16 && (batch > q4k_thin_rows || thin_gemm_max_batch(w) < 16);
 }
 // Q5_K: the same kernel with a third plane for the fifth bits, from the batch on where it is ahead of the

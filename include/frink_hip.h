@@ -202,8 +202,8 @@ int frk_hip_gemm_dev(const frk_weights *w, const float *x_dev, size_t batch, flo
  * call over the same batch) has already quantized to Q8_K: q [batch][cols] i8, d [batch][cols/256] f32,
  * bsums [batch][cols/16] i16, the layout frk_hip_quantize_q8_k_dev writes (BatchActs::Q8K,
  * crates/frink-core/src/weight_matrix.rs:757-768, handed to apply_batch_with_acts, :2481-2487).  Bit for bit
- * frk_hip_gemm_dev's result (one row: frk_hip_gemv_q8k_dev).  K-quants; the batches that frk_hip_gemm_dev multiplies on its thin kernels (up to 32
- * rows for Q4_K and Q5_K, up to 24 or 40 for Q6_K by the matrix's size): FRK_ERR_UNSUPPORTED beyond, where the
+ * frk_hip_gemm_dev's result (one row: frk_hip_gemv_q8k_dev).  K-quants; the batches that frk_hip_gemm_dev multiplies on its thin kernels (up to 16
+ * or 32 rows for Q4_K and up to 24 or 40 for Q6_K by the matrix's size, 32 for Q5_K): FRK_ERR_UNSUPPORTED beyond, where the
  * matrix-core GEMM quantizes into a tiled form of its own. */
 int frk_hip_gemm_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float *d_dev, const int16_t *bsums_dev,
                          size_t batch, float *y_dev, void *stream);
