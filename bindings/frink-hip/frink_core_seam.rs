@@ -1,6 +1,6 @@
 // What crates/frink-core gains for the HIP backend, as the fragments a maintainer pastes where the
 // CUDA arms already are.  Not a compilation unit: each fragment names the file and the place it goes.
-// (Never compiled in the library's repository; see INTEGRATION.md.)
+// (Never compiled in the library's repository, whose image has no Rust toolchain.)
 
 // ---- crates/frink-core/Cargo.toml ----
 //   [dependencies]  frink-hip = { workspace = true, optional = true }

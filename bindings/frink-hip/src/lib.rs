@@ -272,7 +272,8 @@ impl Drop for Weights {
 }
 
 /// The device-pointer family.  Every pointer is a device pointer; calls are asynchronous on `stream`
-/// (a `hipStream_t` or null).  Scratch memory is per stream: see INTEGRATION.md, contract summary.
+/// (a `hipStream_t` or null).  Scratch memory is per stream (one library-owned buffer a stream, held by the calling thread while it
+/// enqueues a call's launches; see the comment in front of the device-pointer entry points in frink_hip.h).
 pub mod dev {
     use super::*;
 

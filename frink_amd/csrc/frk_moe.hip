@@ -203,7 +203,7 @@ __device__ __forceinline__ void moe_group(const GroupArgs &a) {
                     L.before[w * n_experts + e] = (unsigned short)run;
                     run += __popc(L.bits[w * n_experts + e]);
                 }
-                if (seg == segs - 1) L.cnt[e] = run;  // this round's pairs of the expert
+                if (seg == segs - 1) L.cnt[e] = run;  // this pass's pairs of the expert
             }
         }
         __syncthreads();
