@@ -361,7 +361,8 @@ bool direct_gemv_fits(const frk_weights *w) {
     const size_t units = w->kind == FRK_KIND_Q6_K ? w->cols / QK_K * 4 : w->cols / Q8_0_ELEMS * 2;
     // (Q8_0: up to eight units a lane, 8192 columns; sixteen, 16384 columns, where the rows are many enough for the
     // kernel that shares the activation through LDS)
-    if (w->kind == FRK_KIND_Q8_0) return units > 32 && (units <= 512 || (units <= 1024 && w->rows >= 1024));
+    // (... and twenty-eight, 28672 columns: 112 KB of activation in LDS, one workgroup a CU)
+    if (w->kind == FRK_KIND_Q8_0) return units > 32 && (units <= 512 || (units <= 1792 && w->rows >= 1024));
     return w->kind == FRK_KIND_Q6_K && units > 32 && units <= 256;
 }
 
@@ -451,7 +452,10 @@ int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, 
         else if (u <= 8) FRK_GO(8);
         else if (u <= 11) FRK_GO(11);
         else if (u <= 14) FRK_GO_BIG(14);
-        else FRK_GO_BIG(16);
+        else if (u <= 16) FRK_GO_BIG(16);
+        else if (u <= 20) FRK_GO_BIG(20);
+        else if (u <= 24) FRK_GO_BIG(24);
+        else FRK_GO_BIG(28);  // (2 * 28 loads in flight behind the activation's: vmcnt counts to 63)
 #undef FRK_GO_BIG
 #undef FRK_GO
         FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");

@@ -201,6 +201,7 @@ GEMV_SHAPES = [
     (fo.Q8_0, 12, 16384),
     # Q8_0 rows of 8224 .. 16384 columns with at least 1024 rows: the activation shared through LDS, 11 to 16 units a lane
     (fo.Q8_0, 1024, 14336), (fo.Q8_0, 1500, 11008), (fo.Q8_0, 1027, 16384), (fo.Q8_0, 1100, 8704), (fo.Q8_0, 1030, 10240),
+    (fo.Q8_0, 1025, 22016), (fo.Q8_0, 1030, 28672), (fo.Q8_0, 1024, 18432), (fo.Q8_0, 40, 28672), (fo.Q8_0, 1024, 28704),
 ]
 
 
