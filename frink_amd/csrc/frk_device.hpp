@@ -183,17 +183,21 @@ __device__ __forceinline__ float silu_as_host(float x, const uint64_t *table = E
 // held four consecutive values per lane by one wavefront.  Returns the lane's four quants packed
 // little-endian; d_out is the block scale (same in every lane); bsum16 is the sum of the 16-wide
 // group this lane belongs to (same in the four lanes of a quad).
+// BRANCHES false: an all-zero block is a select at the end instead of a branch around the arithmetic (the
+// same results: 127 / 0 is an infinity whose products are dropped by the select, and 1 / inf is the zero
+// scale), so that a wavefront quantizing several blocks can interleave their dependent chains.
+template <bool BRANCHES = true>
 __device__ __forceinline__ uint32_t quantize_q8_k_lane(float4 v, float &d_out, int &bsum16) {
-    // f32::max ignores a NaN operand, as fmaxf does
-    const float amax = wave_max(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    // f32::max ignores a NaN operand, as fmaxf does, and the fold starts from 0: a block of NaNs has the maximum 0
+    const float amax = wave_max(fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f));
     int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
     d_out = 0.0f;
-    if (amax != 0.0f) {  // uniform across the wavefront
+    if (!BRANCHES || amax != 0.0f) {  // uniform across the wavefront
         const float iscale = __fdiv_rn(127.0f, amax);
         auto quant = [&](float e) {
-            float r = rintf(iscale * e);  // round half to even
-            r = fminf(fmaxf(r, -127.0f), 127.0f);
-            return (r != r) ? 0 : (int)r;  // a NaN becomes 0, as Rust's `as i8` makes it
+            const float r = rintf(iscale * e);  // round half to even
+            // a NaN becomes 0: f32::clamp keeps it and `as i8` makes it 0 (fmaxf would turn it into -127)
+            return (r != r || (!BRANCHES && amax == 0.0f)) ? 0 : (int)fminf(fmaxf(r, -127.0f), 127.0f);
         };
         q0 = quant(v.x);
         q1 = quant(v.y);

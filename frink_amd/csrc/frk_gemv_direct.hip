@@ -135,6 +135,136 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void gemv_q6_k_direct_kernel(
     if (lane == 0 && store) y[r] = acc;
 }
 
+// ------------------------------------------------------------------ Q6_K x f32, one launch, no barrier before the dots
+// The same step -- quantize_activations_q8_k, then dot_q6_k_q8 per row -- with the work cut the other way:
+// a workgroup takes 4 * U rows and wavefront w the columns of blocks 4w .. 4w+3 of all of them, the very
+// blocks it quantizes itself.  A wavefront therefore waits for nobody before it multiplies: its slice of
+// the activation goes through a corner of LDS that only it touches (quantized four values a lane, read
+// back as this lane's 64 columns and kept in registers for every row), all its weight loads are in flight
+// from the start, and the one workgroup barrier stands at the very end, where the wavefronts' sixteen
+// partial sums a row meet.  (A barrier behind the weight loads, as in the kernel above, costs microseconds
+// on long rows: a wavefront reaches it only once the memory pipeline has taken all its loads.)
+// Round j of a wavefront covers rows 4j .. 4j+3 of the workgroup: lane = 16 * (row of the round) + unit,
+// unit = (block of the slice, half, 16-byte column) as above.
+constexpr int COLS_WAVE_LDS = 4 * (QK_K + 32 + 4);  // four blocks: quants, 16-wide sums, scale
+template <int U>
+__global__ __launch_bounds__(1024) void gemv_q6_k_cols_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
+                                                             const float *__restrict__ x, float *__restrict__ y) {
+    typedef float xv_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+    extern __shared__ uint4 smem_cols[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    uint8_t *mine = reinterpret_cast<uint8_t *>(smem_cols) + wave * COLS_WAVE_LDS;
+    float *parts = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(smem_cols) + waves * COLS_WAVE_LDS);
+    const int b0 = wave * 4, r0 = (int)blockIdx.x * 4 * U;
+
+    // the activation's loads first: a wavefront's loads return in issue order
+    xv_t xv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {  // (a block past the row's end: the last one again, not used)
+        const float *src = x + (size_t)min(b0 + i, nb - 1) * QK_K + lane * 4;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xv[i]) : "v"(src) : "memory");
+    }
+    const int ul = lane & 15, bl = ul >> 2, h = (ul >> 1) & 1, t = ul & 1;
+    const bool live = b0 + bl < nb;
+    const int b = min(b0 + bl, nb - 1);
+    u4_t qla[U], qlb[U], qh[U];
+    u2_t scv[U];
+    uint32_t dbits[U];
+    auto request = [&](int j) {
+        const int r = min(r0 + 4 * j + (lane >> 4), rows - 1);  // a row past the end: the last one again, not stored
+        const uint8_t *row = W + (size_t)r * lay.row_stride;
+        const uint8_t *p_l = row + (size_t)b * 128 + h * 64 + t * 16;
+        const uint8_t *p_h = row + lay.off_a + (size_t)b * 64 + h * 32 + t * 16;
+        const uint8_t *p_s = row + lay.off_b + (size_t)b * 16 + h * 8;
+        const uint8_t *p_d = row + lay.off_c + (size_t)b * 2;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qla[j]) : "v"(p_l) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(qlb[j]) : "v"(p_l) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qh[j]) : "v"(p_h) : "memory");
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(scv[j]) : "v"(p_s) : "memory");
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(dbits[j]) : "v"(p_d) : "memory");
+    };
+    request(0);
+
+    // ---- this wavefront's four blocks of the activation, through its own corner of LDS ----
+    // (the other rounds are requested once the activation is here: behind twenty weight loads of each of
+    // sixteen wavefronts, a late wavefront's activation came late)
+    asm volatile("s_waitcnt vmcnt(5)" : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]));
+#pragma unroll
+    for (int j = 1; j < U; j++) request(j);
+    uint32_t *sq = reinterpret_cast<uint32_t *>(mine);
+    int16_t *sbs = reinterpret_cast<int16_t *>(mine + 4 * QK_K);
+    float *sd = reinterpret_cast<float *>(mine + 4 * QK_K + 4 * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float d;
+        int s16;
+        const uint32_t packed = quantize_q8_k_lane<false>(make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w), d, s16);
+        sq[i * 64 + lane] = packed;
+        if ((lane & 3) == 0) sbs[i * 16 + (lane >> 2)] = (int16_t)s16;
+        if (lane == 0) sd[i] = d;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint8_t *abase = mine + bl * QK_K + h * 128 + t * 16;
+    const uint4 a0 = *reinterpret_cast<const uint4 *>(abase), a1 = *reinterpret_cast<const uint4 *>(abase + 32);
+    const uint4 a2 = *reinterpret_cast<const uint4 *>(abase + 64), a3 = *reinterpret_cast<const uint4 *>(abase + 96);
+    const uint4 bs = *reinterpret_cast<const uint4 *>(sbs + bl * 16 + h * 8);  // the half's eight 16-wide sums
+    const float da = sd[bl];
+    // sums of groups t, t+2, t+4, t+6 of the half: 16-bit fields t, t+2 (x, y) and t+4, t+6 (z, w)
+    const int sh = 16 * t;
+    const int b1 = 32 * (int)(int16_t)(bs.x >> sh), b2 = 32 * (int)(int16_t)(bs.y >> sh);
+    const int b3 = 32 * (int)(int16_t)(bs.z >> sh), b4 = 32 * (int)(int16_t)(bs.w >> sh);
+
+    auto round = [&](const u4_t la, const u4_t lb, const u4_t hh, const u2_t sc, const uint32_t dbit) {
+        int d1 = 0, d2 = 0, d3 = 0, d4 = 0;
+#define FRK_Q6_STEP(c)                                                                     \
+    d1 = dot4((la.c & 0x0f0f0f0fu) | ((hh.c << 4) & 0x30303030u), a0.c, d1);                \
+    d2 = dot4((lb.c & 0x0f0f0f0fu) | ((hh.c << 2) & 0x30303030u), a1.c, d2);                \
+    d3 = dot4(((la.c >> 4) & 0x0f0f0f0fu) | (hh.c & 0x30303030u), a2.c, d3);                \
+    d4 = dot4(((lb.c >> 4) & 0x0f0f0f0fu) | ((hh.c >> 2) & 0x30303030u), a3.c, d4);
+        FRK_Q6_STEP(x)
+        FRK_Q6_STEP(y)
+        FRK_Q6_STEP(z)
+        FRK_Q6_STEP(w)
+#undef FRK_Q6_STEP
+        const uint32_t slo = t ? (sc.x >> 8) : sc.x, shi = t ? (sc.y >> 8) : sc.y;
+        const int s1 = (int)(int8_t)(slo & 0xff), s2 = (int)(int8_t)((slo >> 16) & 0xff);
+        const int s3 = (int)(int8_t)(shi & 0xff), s4 = (int)(int8_t)((shi >> 16) & 0xff);
+        const int isum = s1 * (d1 - b1) + s2 * (d2 - b2) + s3 * (d3 - b3) + s4 * (d4 - b4);
+        const float term = (h2f(dbit) * da) * (float)isum;
+        return part_sum<16>(live ? term : 0.0f);
+    };
+    float sums[U];
+#define FRK_COLS_ROUND(j)                                                                                            \
+    if constexpr (U > j) {                                                                                           \
+        asm volatile("s_waitcnt vmcnt(%5)"                                                                           \
+                     : "+v"(qla[j]), "+v"(qlb[j]), "+v"(qh[j]), "+v"(scv[j]), "+v"(dbits[j])                         \
+                     : "n"(5 * (U - 1 - j)));                                                                        \
+        sums[j] = round(qla[j], qlb[j], qh[j], scv[j], dbits[j]);                                                    \
+    }
+    FRK_COLS_ROUND(0)
+    FRK_COLS_ROUND(1)
+    FRK_COLS_ROUND(2)
+    FRK_COLS_ROUND(3)
+    FRK_COLS_ROUND(4)
+    FRK_COLS_ROUND(5)
+#undef FRK_COLS_ROUND
+#pragma unroll
+    for (int j = 0; j < U; j++)
+        if (ul == 0) parts[wave * (4 * U) + 4 * j + (lane >> 4)] = sums[j];
+    lds_barrier();
+    // a row's partial sums, in the order of the columns
+    if ((int)threadIdx.x < 4 * U && r0 + (int)threadIdx.x < rows) {
+        float v = 0.0f;
+        for (int w = 0; w < waves; w++) v += parts[w * (4 * U) + threadIdx.x];
+        y[r0 + threadIdx.x] = v;
+    }
+}
+
 // ------------------------------------------------------------------ Q6_K experts, one job per (token, slot)
 // The decode form of a mixture-of-experts down projection whose experts are Q6_K (run_expert,
 // crates/frink-moe/src/lib.rs:1068-1165): job j multiplies expert ids[j]'s rows_e rows (the experts'
@@ -382,9 +512,50 @@ int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream
     return FRK_OK;
 }
 
+// Rows of 20 blocks and more, and rows too short for the kernel that gives a row to a wavefront: the column form.
+bool q6_k_cols_form(const frk_weights *w) {
+    const size_t nb = w->cols / QK_K;
+    return w->kind == FRK_KIND_Q6_K && nb <= 64 && (nb >= 20 || nb <= 8);
+}
+static int compute_units_direct() {
+    static const int n = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+            v = 256;
+        return v;
+    }();
+    return n;
+}
 // One launch: Q8_K quantization of x inside the kernel.  nb <= 64 (direct_gemv_fits).
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / QK_K);
+    if (q6_k_cols_form(w)) {  // the wavefronts split the columns, not the rows
+        const int waves = (nb + 3) / 4;
+        // Rows to a workgroup, 4 * U.  A CU's share of the launch costs about (its workgroups) x (4 * U rows + the
+        // quantization of the activation, as much as five rows): the U with the smallest product, the larger of
+        // equals.  (Measured at 1024 .. 32000 rows of 4 .. 56 blocks: within 4 % of the best U everywhere.)
+        const int cus = compute_units_direct();
+        int best_u = 1;
+        size_t best = SIZE_MAX;
+        for (int u = 1; u <= (waves == 1 ? 2 : 6); u++) {
+            const size_t wgs = (w->rows + 4 * u - 1) / (4 * u);
+            const size_t cost = (wgs + cus - 1) / cus * (4 * u + 5);
+            if (cost <= best) best = cost, best_u = u;
+        }
+        const size_t lds = (size_t)waves * (COLS_WAVE_LDS + 4 * best_u * 4);
+        const dim3 grid((unsigned)((w->rows + 4 * best_u - 1) / (4 * best_u))), block(64 * waves);
+#define FRK_GO_COLS(UU) \
+    hipLaunchKernelGGL((gemv_q6_k_cols_kernel<UU>), grid, block, lds, s, w->dev, w->layout, (int)w->rows, nb, x, y)
+        if (best_u == 1) FRK_GO_COLS(1);
+        else if (best_u == 2) FRK_GO_COLS(2);
+        else if (best_u == 3) FRK_GO_COLS(3);
+        else if (best_u == 4) FRK_GO_COLS(4);
+        else if (best_u == 5) FRK_GO_COLS(5);
+        else FRK_GO_COLS(6);
+#undef FRK_GO_COLS
+        FRK_LAUNCH_CHECK("gemv_q6_k_cols");
+        return FRK_OK;
+    }
     const int u = (nb * 4 + 63) / 64;
     const dim3 grid((unsigned)((w->rows + 15) / 16)), block(1024);
     const size_t shmem = (size_t)nb * (256 + 32 + 4);

@@ -389,7 +389,7 @@ __device__ __forceinline__ float lines_block_dot(const uint4 *blk, const uint4 *
     return (d * da) * (float)s1 - (dmin * da) * (float)s2;
 }
 
-template <int NB, int MODE, int WAVES, bool Q5 = false>
+template <int NB, int MODE, int WAVES, bool Q5 = false, int AHEAD = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8_t *__restrict__ W, int rows,
                                                                     const float *__restrict__ x,
                                                                     const int8_t *__restrict__ aq,
@@ -398,6 +398,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
                                                                     float *__restrict__ y) {
     constexpr int RPS = 64 / NB;  // rows of a wavefront's span
     constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES, SPAN = 64 * BB, PIECES = SPAN / 1024;  // 9 or 11 KB
+    // AHEAD > 0: only that many kilobytes of the span are requested before the activation is quantized, the
+    // rest behind the barrier.  For a launch whose workgroups all start at once (one round, the CUs full) the
+    // memory pipeline is then not yet full of weight requests when the activation's loads and the barrier
+    // want through: 8.0 against 8.55 us at 14336 x 4096 with four ahead (three 8.15, five 8.65).  A launch of
+    // several rounds, or of few workgroups, loses by it (4096 x 4096 5.05 against 4.7 us): AHEAD = 0 there.
+    constexpr int FIRST = AHEAD > 0 && MODE == MODE_FUSED ? AHEAD : PIECES;
     static_assert(64 % NB == 0 && NB >= 8, "a span of 64 blocks is a whole number of rows of at least 8 blocks");
     static_assert(NB * 16 <= 3 * 64 * WAVES, "three 16-byte words of quantized activation a thread at most");
     extern __shared__ uint4 smem[];
@@ -445,50 +451,48 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
         asm volatile("global_load_dword %0, %1, off" : "=v"(dv) : "v"(s3) : "memory");
     }
     // (a wavefront past the matrix fetches the last span and stores nothing)
-    {
-        const size_t span_c = min(span, (bytes - 1) / SPAN);
-        const uint8_t *src = W + span_c * SPAN;
-        const uint32_t left = (uint32_t)min((size_t)SPAN, bytes - span_c * SPAN);  // (the last span may be short)
-        const uint32_t slot = lds_address(sw) + (uint32_t)wave * SPAN;
+    const size_t span_c = min(span, (bytes - 1) / SPAN);
+    const uint8_t *span_src = W + span_c * SPAN;
+    const uint32_t left = (uint32_t)min((size_t)SPAN, bytes - span_c * SPAN);  // (the last span may be short)
+    const uint32_t slot = lds_address(sw) + (uint32_t)wave * SPAN;
 #pragma unroll
-        for (int c = 0; c < PIECES; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
-    }
+    for (int c = 0; c < FIRST; c++) dma16(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
 
     // ---- the activation into LDS ----
     if (MODE == MODE_FUSED) {
-        // the activation's loads are older than the span's nine (Q5_K: eleven)
+        // the activation's loads are older than the span's nine (Q5_K: eleven; AHEAD: those requested so far)
         // (one wait that names them all, so that the blocks' quantizations can be interleaved)
         constexpr int XB = (NB + WAVES - 1) / WAVES;
         // (exactly the registers there are: an operand named twice would be copied in front of the wait)
         static_assert(XB >= 1 && XB <= 8, "up to eight blocks of the activation a wavefront");
-        if constexpr (XB == 1) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xv[0]) : "n"(PIECES));
-        if constexpr (XB == 2) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]) : "n"(PIECES));
+        if constexpr (XB == 1) asm volatile("s_waitcnt vmcnt(%1)" : "+v"(xv[0]) : "n"(FIRST));
+        if constexpr (XB == 2) asm volatile("s_waitcnt vmcnt(%2)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]) : "n"(FIRST));
         if constexpr (XB == 3)
-            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]) : "n"(PIECES));
+            asm volatile("s_waitcnt vmcnt(%3)" : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]) : "n"(FIRST));
         if constexpr (XB == 4)
             asm volatile("s_waitcnt vmcnt(%4)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0])
-                         : "n"(PIECES));
+                         : "n"(FIRST));
         if constexpr (XB == 5)
             asm volatile("s_waitcnt vmcnt(%5)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
                            "+v"(xv[XB > 4 ? 4 : 0])
-                         : "n"(PIECES));
+                         : "n"(FIRST));
         if constexpr (XB == 6)
             asm volatile("s_waitcnt vmcnt(%6)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
                            "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0])
-                         : "n"(PIECES));
+                         : "n"(FIRST));
         if constexpr (XB == 7)
             asm volatile("s_waitcnt vmcnt(%7)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
                            "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0])
-                         : "n"(PIECES));
+                         : "n"(FIRST));
         if constexpr (XB == 8)
             asm volatile("s_waitcnt vmcnt(%8)"
                          : "+v"(xv[0]), "+v"(xv[XB > 1 ? 1 : 0]), "+v"(xv[XB > 2 ? 2 : 0]), "+v"(xv[XB > 3 ? 3 : 0]),
                            "+v"(xv[XB > 4 ? 4 : 0]), "+v"(xv[XB > 5 ? 5 : 0]), "+v"(xv[XB > 6 ? 6 : 0]), "+v"(xv[XB > 7 ? 7 : 0])
-                         : "n"(PIECES));
+                         : "n"(FIRST));
 #pragma unroll
         for (int i = 0; i < XB; i++) {
             const int b = wave + i * WAVES;
@@ -520,6 +524,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
     // Only the activation is shared: the barrier comes before the wait for the span, so that a wavefront
     // starts multiplying when ITS blocks have landed, whatever the others' have done.
     lds_barrier();
+#pragma unroll
+    for (int c = FIRST; c < PIECES; c++) dma16(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the span has landed (in this wavefront's own slot)
     if (!has_rows) return;
 
@@ -743,7 +749,7 @@ static bool lines_kernel_fits(const frk_weights *w) {
     const size_t bb = w->kind == FRK_KIND_Q5_K ? Q5_K_BYTES : Q4_K_BYTES;
     return (nb == 8 || nb == 16 || nb == 32 || nb == 64) && w->layout.row_stride == nb * bb;
 }
-template <int NB, int MODE, int WAVES, bool Q5 = false>
+template <int NB, int MODE, int WAVES, bool Q5 = false, int AHEAD = 0>
 static int launch_q4_k_lines_as(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
     constexpr size_t shmem = (size_t)NB * (LINES_ACT_STRIDE + 32 + 4) + (size_t)WAVES * 64 * (Q5 ? Q5_K_BYTES : Q4_K_BYTES);
     static_assert(shmem <= 160 * 1024, "LDS of a CU");
@@ -751,13 +757,13 @@ static int launch_q4_k_lines_as(const frk_weights *w, const float *x, Q8KActs a,
     const unsigned grid = (unsigned)((spans + WAVES - 1) / WAVES);
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5, AHEAD>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv lines, LDS %zu): %s", shmem, hipGetErrorString(e));
         sized = true;
     }
-    hipLaunchKernelGGL((gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5>), dim3(grid), dim3(64 * WAVES), shmem, s, w->dev, (int)w->rows, x,
-                       a.q, a.d, a.bsums, y);
+    hipLaunchKernelGGL((gemv_q4_k_lines_kernel<NB, MODE, WAVES, Q5, AHEAD>), dim3(grid), dim3(64 * WAVES), shmem, s, w->dev,
+                       (int)w->rows, x, a.q, a.d, a.bsums, y);
     FRK_LAUNCH_CHECK("gemv_q4_k_lines");
     return FRK_OK;
 }
@@ -769,7 +775,12 @@ static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, fl
     const int nb = (int)(w->cols / QK_K);
     constexpr int WIDE = 8;
     if (nb == 8) return launch_q4_k_lines_as<8, MODE, WIDE>(w, x, a, y, s);
-    if (nb == 16) return launch_q4_k_lines_as<16, MODE, WIDE>(w, x, a, y, s);
+    if (nb == 16) {
+        // one round of workgroups that fills the CUs (two workgroups each): part of the span behind the barrier
+        const size_t wgs = (w->rows * (size_t)16 / 64 + WIDE - 1) / WIDE, room = 2 * (size_t)compute_units();
+        if (MODE == MODE_FUSED && wgs <= room && 4 * wgs >= 3 * room) return launch_q4_k_lines_as<16, MODE, WIDE, false, 4>(w, x, a, y, s);
+        return launch_q4_k_lines_as<16, MODE, WIDE>(w, x, a, y, s);
+    }
     if (nb == 32) return launch_q4_k_lines_as<32, MODE, WIDE>(w, x, a, y, s);
     return launch_q4_k_lines_as<64, MODE, 8>(w, x, a, y, s);
 }

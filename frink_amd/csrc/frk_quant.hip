@@ -32,16 +32,16 @@ __global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restr
     if (b >= n_blocks) return;
     const float4 v = reinterpret_cast<const float4 *>(x + b * QK_K)[lane];
     // f32::max ignores a NaN operand, as fmaxf does; max is exact, so the fold order is free
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float amax = fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f);
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     int q0 = 0, q1 = 0, q2 = 0, q3 = 0;
     float dd = 0.0f;
     if (amax != 0.0f) {
         const float iscale = __fdiv_rn(127.0f, amax);
         auto quant = [&](float e) {
-            float r = rintf(iscale * e);  // round half to even
-            r = fminf(fmaxf(r, -127.0f), 127.0f);
-            return (r != r) ? 0 : (int)r;
+            const float r = rintf(iscale * e);  // round half to even
+            // (f32::clamp keeps a NaN, which `as i8` turns into 0; fmaxf would turn it into -127)
+            return (r != r) ? 0 : (int)fminf(fmaxf(r, -127.0f), 127.0f);
         };
         q0 = quant(v.x);
         q1 = quant(v.y);
@@ -68,15 +68,15 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const bool live = b < n_blocks;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = reinterpret_cast<const float4 *>(x)[t];
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float amax = fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f);
     for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     if (!live) return;
     const float scale = __fdiv_rn(amax, 127.0f);
     const float inv = amax != 0.0f ? __fdiv_rn(127.0f, amax) : 0.0f;
     auto quant = [&](float e) {
-        float r = rintf(e * inv);
-        r = fminf(fmaxf(r, -127.0f), 127.0f);
-        return (r != r) ? 0 : (int)r;
+        const float r = rintf(e * inv);
+        // (f32::clamp keeps a NaN, which `as i8` turns into 0; fmaxf would turn it into -127)
+        return (r != r) ? 0 : (int)fminf(fmaxf(r, -127.0f), 127.0f);
     };
     const int q0 = quant(v.x), q1 = quant(v.y), q2 = quant(v.z), q3 = quant(v.w);
     reinterpret_cast<uint32_t *>(q)[t] = (uint32_t)(q0 & 0xff) | ((uint32_t)(q1 & 0xff) << 8) |

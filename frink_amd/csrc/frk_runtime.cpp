@@ -490,7 +490,7 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     }
         [[fallthrough]];
     case FRK_KIND_Q6_K: {
-        if (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) return launch_gemv_q6_k_fused(w, x, y, s);
+        if (w->kind == FRK_KIND_Q6_K && (direct_gemv_fits(w) || q6_k_cols_form(w))) return launch_gemv_q6_k_fused(w, x, y, s);
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
         if (rc) return rc;
@@ -752,7 +752,7 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     for (size_t i = 0; i < n; i++) {
         const frk_weights *w = ws[i];
         all_fused = all_fused && ((w->kind == FRK_KIND_Q4_K && fused_gemv_fits(w)) ||
-                                  (w->kind == FRK_KIND_Q6_K && direct_gemv_fits(w)) || w->kind == FRK_KIND_Q8_0 ||
+                                  (w->kind == FRK_KIND_Q6_K && (direct_gemv_fits(w) || q6_k_cols_form(w))) || w->kind == FRK_KIND_Q8_0 ||
                                   w->kind == FRK_KIND_Q4_0);
     }
     if (all_fused) {

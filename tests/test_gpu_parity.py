@@ -155,7 +155,18 @@ def _q8k_cases():
         "tiny": synth.normal(13, 1024, 1e-30),
         "huge": synth.normal(14, 1024, 1e30),
         "wide": synth.activations(15, 2, 14336).ravel(),
+        # f32::clamp keeps a NaN and `as i8` makes it 0; an infinity makes the inverse scale 0 and the scale infinite
+        "nans": _with(synth.activations(16, 1, 2048).ravel(), {3: np.nan, 300: -np.nan, 511: np.nan, 1024: np.nan}),
+        "infinities": _with(synth.activations(17, 1, 1024).ravel(), {5: np.inf, 6: -np.inf, 700: np.inf, 701: np.nan}),
+        "all_nan": np.full(256, np.nan, np.float32),
     }
+
+
+def _with(x, values):
+    x = x.copy()
+    for i, v in values.items():
+        x[i] = v
+    return x
 
 
 def test_quantize_q8_k_is_bit_exact(fa):
@@ -181,7 +192,9 @@ def test_quantize_q8_0_is_bit_exact(fa):
     head = lambda h: np.concatenate([np.array(h, np.float32), np.zeros(32 - len(h), np.float32)])
     cases = [head([127.0, 2.5, -3.5, 0.5, 1.5]), head([1.0, 0.5]), np.zeros(32, np.float32),
              head([np.uint32(0x4013E709).view(np.float32), np.uint32(0x3CDF99C0).view(np.float32)]),
-             synth.activations(21, 4, 4096).ravel(), synth.normal(22, 320, 1e-6)]
+             synth.activations(21, 4, 4096).ravel(), synth.normal(22, 320, 1e-6),
+             _with(synth.activations(23, 1, 256).ravel(), {3: np.nan, 40: np.inf, 41: 1.0, 100: -np.nan}),
+             np.full(32, np.nan, np.float32)]
     for x in cases:
         q, d = fa.quantize_q8_0(to_dev(x))
         wq, wd = fo.quantize_q8_0(x, fo.FORM_AVX)
@@ -222,6 +235,43 @@ def test_gemv_matches_the_oracle(fa, kind, rows, cols):
         want_i = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT)
         got_i = w.gemv(to_dev(x), act_mode=fa.ACT_INT8).cpu().numpy()
         assert_rows_close(got_i[None], want_i[None], "gemv q8_0 int tier")
+    w.release()
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 6144), (16, 6144), (17, 8192), (100, 11008), (31, 13824), (64, 14336), (33, 16384),
+                                       (5, 6400), (40, 7168), (9, 256), (70, 1024), (33, 1792), (40, 2048), (21, 5120),
+                                       (4101, 6144), (10243, 6144), (12290, 6144), (5120, 13824)])
+def test_q6_k_gemv_with_the_columns_split_between_wavefronts(fa, rows, cols):
+    """Q6_K rows of 20 blocks and more (and of 8 and fewer), one launch: a wavefront takes four blocks of columns of
+    the workgroup's 4 .. 24 rows and quantizes exactly those blocks itself.  Row counts that fill a workgroup, fall
+    short and leave a short last one, at every number of rows to a workgroup the launch picks (the large row counts:
+    random block bytes, encoding that many rows takes too long); block counts that fill the last wavefront's four
+    and do not."""
+    from bench import random_blocks
+    from frink_amd import synth
+    data = random_blocks(fo.Q6_K, rows, cols, rows + cols) if rows > 2000 else make_weights(fo.Q6_K, rows, cols, seed=rows * 5 + cols)
+    x = synth.activations(rows + 2 * cols, 1, cols, outlier_frac=0.01)[0]
+    w = fa.Weights.from_host(fo.Q6_K, data, rows, cols)
+    want = fo.gemv(fo.Q6_K, data, rows, cols, x, fo.INT_DOT)
+    got = w.gemv(to_dev(x)).cpu().numpy()
+    assert_rows_close(got[None], want[None], "q6_k columns form %dx%d" % (rows, cols))
+    w.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols", [(fo.Q4_K, 40, 4096), (fo.Q4_K, 9, 1024), (fo.Q4_K, 20, 11008), (fo.Q5_K, 33, 4096),
+                                            (fo.Q6_K, 20, 4096), (fo.Q6_K, 20, 14336), (fo.Q6_K, 7, 768)])
+def test_gemv_quantizes_a_nan_to_zero_inside_the_launch(fa, kind, rows, cols):
+    """quantize_activations_q8_k makes a NaN activation a zero quant (f32::clamp keeps the NaN, `as i8` makes it 0)
+    and leaves it out of the block's maximum: the kernels that quantize inside the launch must do the same."""
+    from frink_amd import synth
+    data = make_weights(kind, rows, cols, seed=rows + cols)
+    x = synth.activations(rows + cols + 1, 1, cols)[0].copy()
+    x[[1, 77, 255, 256, cols - 1]] = np.nan
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    want = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT)
+    assert np.isfinite(want).all()
+    got = w.gemv(to_dev(x)).cpu().numpy()
+    assert_rows_close(got[None], want[None], "gemv with NaN activations, kind %d %dx%d" % (kind, rows, cols))
     w.release()
 
 
