@@ -806,9 +806,10 @@ __global__ __launch_bounds__(512) void thin_span_q4_k_kernel(const uint8_t *__re
     const int cols = nb * QK_K;
     uint8_t *const lds_w = lds + slices * L::SLICE;
 
-    // ---- the activations' slices, their pieces dealt to the wavefronts ----
-    for (int t = wave; t < slices * (ACTS + 2); t += waves) {  // (uniform per wavefront)
-        const int sl = t / (ACTS + 2), piece = t % (ACTS + 2);
+    // ---- the activations: a wavefront fetches the slice it multiplies, so that it waits for nobody ----
+#pragma unroll
+    for (int piece = 0; piece < ACTS + 2; piece++) {
+        const int sl = wave;
         const int k = sl;
         const uint32_t base = lds0 + (uint32_t)sl * L::SLICE;
         if (piece < ACTS) {
@@ -839,10 +840,9 @@ __global__ __launch_bounds__(512) void thin_span_q4_k_kernel(const uint8_t *__re
             else if (lane < 16 * TS_ROW_PIECES - 576) dma16(slot + 9 * 1024, src, off);
         }
     }
-    // the activations' pieces are older than the span's ten; only they are shared, so the barrier comes
-    // before the wait for the span and a wavefront multiplies as soon as ITS rows have landed
-    asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-    lds_barrier();
+    // Nothing is shared before the sums: a wavefront multiplies as soon as ITS slice and ITS rows have landed.
+    // (With the slices' pieces dealt round the wavefronts there was a barrier here, reached only once the
+    // memory pipeline had taken every wavefront's requests.)
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 
     const int j = lane & 15, g = lane >> 4;
