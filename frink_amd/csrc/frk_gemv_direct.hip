@@ -1,12 +1,14 @@
-// Decode GEMV for Q6_K and Q8_0 with every load of a row in flight at once.
+// Decode GEMV for Q6_K and Q8_0 with every load of a wavefront's share in flight at once.
 //
-// One wavefront owns one weight row; lane l owns units l, l+64, ... (a unit is 64 weights of Q6_K or
-// 16 of Q8_0, the same units as the looping kernels in frk_gemv.hip).  All of a lane's loads -- its
-// share of the activation first, because a wavefront's loads return in issue order and the
-// activation comes from L2, then its weights from HBM -- are issued before any arithmetic, so a CU
-// holds tens of kilobytes in flight instead of one loop iteration's worth.  No LDS, no barrier: the
-// quantized activation (a few kilobytes) is read by every lane straight from L2.
-// Rows longer than 64*U units fall back to the looping kernels.
+// Two ways of cutting a matrix between wavefronts.  Rows: one wavefront owns one weight row; lane l owns units
+// l, l+64, ... (a unit is 64 weights of Q6_K or 16 of Q8_0, the same units as the looping kernels in
+// frk_gemv.hip); the activation is shared by the rows of a workgroup through LDS, or read by every lane from L2.
+// Columns: a workgroup owns a few rows and wavefront w the same 64 units of every one of them, so that a lane's
+// slice of the activation is loaded (Q6_K: quantized) once and kept in registers -- nothing is shared before the
+// sums, and no barrier stands between the requests and the arithmetic.  All of a lane's loads -- its share of
+// the activation first, because a wavefront's loads return in issue order and the activation comes from L2,
+// then its weights from HBM -- are issued before any arithmetic, so a CU holds tens of kilobytes in flight
+// instead of one loop iteration's worth.  Rows too long for either fall back to the looping kernels.
 #include "frk_device.hpp"
 
 namespace frk {
@@ -360,58 +362,10 @@ __global__ __launch_bounds__(256) void gemv_q6_k_experts_kernel(const uint8_t *_
 // ------------------------------------------------------------------ Q8_0 x f32
 // dot_q8_0_f32 (crates/frink-quant/src/lib.rs:663-686) over the planar resident layout.
 // Unit = 16 quants (half a block).
-template <int U>
-__global__ __launch_bounds__(256) void gemv_q8_0_f32_direct_kernel(const uint8_t *__restrict__ W, Layout lay,
-                                                                   int rows, int nb, const float *__restrict__ x,
-                                                                   float *__restrict__ y) {
-    const int lane = threadIdx.x & 63;
-    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;  // uniform per wavefront
-    const uint8_t *row = W + (size_t)r * lay.row_stride;
-    const int units = nb * 2;
-
-    float4 x0[U], x1[U], x2[U], x3[U];
-    uint4 qv[U];
-    uint32_t dbits[U];
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-        const int u = min(lane + 64 * j, units - 1);
-        const float4 *xv = reinterpret_cast<const float4 *>(x + u * 16);
-        x0[j] = xv[0];
-        x1[j] = xv[1];
-        x2[j] = xv[2];
-        x3[j] = xv[3];
-    }
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-        const int u = min(lane + 64 * j, units - 1);
-        qv[j] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
-        dbits[j] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2);
-    }
-    float acc = 0.0f;
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-        float s = 0.0f;
-#define FRK_Q8_STEP(c, xx)                                         \
-    s = fmaf((float)(int8_t)(qv[j].c & 0xff), xx.x, s);            \
-    s = fmaf((float)(int8_t)((qv[j].c >> 8) & 0xff), xx.y, s);     \
-    s = fmaf((float)(int8_t)((qv[j].c >> 16) & 0xff), xx.z, s);    \
-    s = fmaf((float)(int8_t)(qv[j].c >> 24), xx.w, s);
-        FRK_Q8_STEP(x, x0[j])
-        FRK_Q8_STEP(y, x1[j])
-        FRK_Q8_STEP(z, x2[j])
-        FRK_Q8_STEP(w, x3[j])
-#undef FRK_Q8_STEP
-        const float term = s * h2f(dbits[j]);
-        acc += (lane + 64 * j < units) ? term : 0.0f;
-    }
-    acc = part_sum<64>(acc);
-    if (lane == 0) y[r] = acc;
-}
-
-// The same with the activation shared through LDS by the 16 rows of a 16-wavefront workgroup: a row
-// of 4096 Q8_0 weights is 4.3 KB but multiplies 16 KB of f32 activation, so per-lane activation
-// reads from L2 are four times the weight traffic.  The activation goes global -> LDS with one
+// A row to a wavefront, every load of the row in flight at once, the activation shared through LDS by the
+// rows of the workgroup (rows of more than 16384 columns): a row of Q8_0 weights is a quarter of the bytes of
+// the f32 activation it multiplies, so per-lane activation reads from L2 would be four times the weight
+// traffic.  The activation goes global -> LDS with one
 // global_load_lds per wavefront, laid out [piece k of a unit][unit] so that the lanes of a read are
 // consecutive; LDS reads are inline assembly so that the compiler does not wait for the weight
 // loads in front of them (it cannot tell the two apart from the global_load_lds).
@@ -478,6 +432,55 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_0_f32_shared_kernel(const 
     if (lane == 0 && store) y[r] = acc;
 }
 
+// The same product with the columns split between the wavefronts of a workgroup instead of the rows: wavefront w
+// takes units 64w .. 64w+63 (1024 columns) of the workgroup's R rows, so a lane multiplies the same sixteen
+// columns in every row and keeps its 64 bytes of the activation in registers, read straight from global memory
+// -- no copy in LDS, hence no barrier between the requests and the arithmetic; the wavefronts' partial sums of a
+// row meet in LDS at the end and are added in the order of the columns.
+template <int R>
+__global__ __launch_bounds__(1024) void gemv_q8_0_f32_cols_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
+                                                                 const float *__restrict__ x, float *__restrict__ y) {
+    extern __shared__ uint4 smem_direct[];
+    float *parts = reinterpret_cast<float *>(smem_direct);  // [wavefront][row]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int units = nb * 2;
+    const bool live = wave * 64 + lane < units;
+    const int u = min(wave * 64 + lane, units - 1);  // (a lane past the end: the last unit again, not added)
+    const int r0 = (int)blockIdx.x * R;
+    const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)u * 16);
+    const float4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+    uint4 qv[R];
+    uint32_t dbits[R];
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        const uint8_t *row = W + (size_t)min(r0 + k, rows - 1) * lay.row_stride;  // (a row past the end: the last again)
+        qv[k] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+        dbits[k] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2);
+    }
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        float s = 0.0f;
+#define FRK_Q8_STEP(c, xx)                                         \
+    s = fmaf((float)(int8_t)(qv[k].c & 0xff), xx.x, s);            \
+    s = fmaf((float)(int8_t)((qv[k].c >> 8) & 0xff), xx.y, s);     \
+    s = fmaf((float)(int8_t)((qv[k].c >> 16) & 0xff), xx.z, s);    \
+    s = fmaf((float)(int8_t)(qv[k].c >> 24), xx.w, s);
+        FRK_Q8_STEP(x, x0)
+        FRK_Q8_STEP(y, x1)
+        FRK_Q8_STEP(z, x2)
+        FRK_Q8_STEP(w, x3)
+#undef FRK_Q8_STEP
+        const float v = part_sum<64>(live ? s * h2f(dbits[k]) : 0.0f);
+        if (lane == 0) parts[wave * R + k] = v;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < R && r0 + (int)threadIdx.x < rows) {
+        float v = 0.0f;
+        for (int w = 0; w < waves; w++) v += parts[w * R + threadIdx.x];
+        y[r0 + threadIdx.x] = v;
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -489,10 +492,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_0_f32_shared_kernel(const 
 // rows of at most 64*4 units, and long enough that a wavefront per row is not mostly idle lanes
 bool direct_gemv_fits(const frk_weights *w) {
     const size_t units = w->kind == FRK_KIND_Q6_K ? w->cols / QK_K * 4 : w->cols / Q8_0_ELEMS * 2;
-    // (Q8_0: up to eight units a lane, 8192 columns; sixteen, 16384 columns, where the rows are many enough for the
-    // kernel that shares the activation through LDS)
-    // (... and twenty-eight, 28672 columns: 112 KB of activation in LDS, one workgroup a CU)
-    if (w->kind == FRK_KIND_Q8_0) return units > 32 && (units <= 512 || (units <= 1792 && w->rows >= 1024));
+    // (Q8_0: up to 16384 columns on the kernel whose wavefronts split the columns; up to 28672 -- 112 KB of activation
+    // in LDS, one workgroup a CU -- where the rows are many enough for the kernel that gives a row to a wavefront)
+    if (w->kind == FRK_KIND_Q8_0) return units > 32 && (units <= 1024 || (units <= 1792 && w->rows >= 1024));
     return w->kind == FRK_KIND_Q6_K && units > 32 && units <= 256;
 }
 
@@ -597,52 +599,43 @@ int launch_gemv_q6_k_experts(const frk_weights *w, int n_experts, size_t rows_e,
 int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / Q8_0_ELEMS);
     const int u = (nb * 2 + 63) / 64;
-    if (w->rows >= 1024) {  // enough rows that these workgroups still cover the CUs
-        constexpr int WAVES = 8;  // (two workgroups to a CU: 5.75 us at 4096x4096 against 6.1 with sixteen wavefronts and 5.96 with four)
-        const dim3 grid((unsigned)((w->rows + WAVES - 1) / WAVES)), block(64 * WAVES);
-#define FRK_GO(UU)                                                                                                \
-    hipLaunchKernelGGL((gemv_q8_0_f32_shared_kernel<UU, WAVES>), grid, block, 4096 * UU, s, w->dev, w->layout, (int)w->rows, nb, \
-                       x, y)
-// (more than 48 KB of LDS: the kernel is told once)
-#define FRK_GO_BIG(UU)                                                                                             \
-    do {                                                                                                           \
-        static bool sized = false;                                                                                 \
-        if (!sized) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q8_0_f32_shared_kernel<UU, WAVES>), \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * UU);             \
-            if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv q8_0, LDS): %s", hipGetErrorString(e)); \
-            sized = true;                                                                                          \
-        }                                                                                                          \
-        FRK_GO(UU);                                                                                                \
-    } while (0)
-        if (u == 1) FRK_GO(1);
-        else if (u == 2) FRK_GO(2);
-        else if (u == 3) FRK_GO(3);
-        else if (u == 4) FRK_GO(4);
-        else if (u <= 6) FRK_GO(6);
-        else if (u <= 8) FRK_GO(8);
-        else if (u <= 11) FRK_GO(11);
-        else if (u <= 14) FRK_GO_BIG(14);
-        else if (u <= 16) FRK_GO_BIG(16);
-        else if (u <= 20) FRK_GO_BIG(20);
-        else if (u <= 24) FRK_GO_BIG(24);
-        else FRK_GO_BIG(28);  // (2 * 28 loads in flight behind the activation's: vmcnt counts to 63)
-#undef FRK_GO_BIG
-#undef FRK_GO
-        FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");
+    if (u <= 16) {  // rows of up to 16384 columns: the wavefronts of a workgroup split the columns
+        // Eight rows to a workgroup; four where eight would leave a CU fewer than a dozen wavefronts.  (Measured
+        // against the kernel below, which shares the activation through LDS: 4096x4096 5.6 against 5.7 us,
+        // 14336x4096 13.2 / 14.0, 4096x8192 8.9 / 10.0, 4096x11008 11.3 / 12.9, 4096x14336 15.0 / 17.3; twelve and
+        // sixteen rows to a workgroup are slower everywhere.)
+        const bool four = (w->rows / 8) * (size_t)u < 12 * (size_t)compute_units_direct();
+#define FRK_GO_COLS(RR)                                                                                                              \
+    hipLaunchKernelGGL((gemv_q8_0_f32_cols_kernel<RR>), dim3((unsigned)((w->rows + RR - 1) / RR)), dim3(64 * u), (size_t)u * RR * 4, s, \
+                       w->dev, w->layout, (int)w->rows, nb, x, y)
+        if (four) FRK_GO_COLS(4);
+        else FRK_GO_COLS(8);
+#undef FRK_GO_COLS
+        FRK_LAUNCH_CHECK("gemv_q8_0_f32_cols");
         return FRK_OK;
     }
-    const dim3 grid((unsigned)((w->rows + 3) / 4)), block(256);
-#define FRK_GO(UU) \
-    hipLaunchKernelGGL(gemv_q8_0_f32_direct_kernel<UU>, grid, block, 0, s, w->dev, w->layout, (int)w->rows, nb, x, y)
-    if (u == 1) FRK_GO(1);
-    else if (u == 2) FRK_GO(2);
-    else if (u == 3) FRK_GO(3);
-    else if (u == 4) FRK_GO(4);
-    else if (u <= 6) FRK_GO(6);
-    else FRK_GO(8);
-#undef FRK_GO
-    FRK_LAUNCH_CHECK("gemv_q8_0_f32_direct");
+    // longer rows (direct_gemv_fits: up to 28672 columns, at least 1024 rows): a row to a wavefront, the activation
+    // through LDS, one workgroup to a CU
+    constexpr int WAVES = 8;
+    const dim3 grid((unsigned)((w->rows + WAVES - 1) / WAVES)), block(64 * WAVES);
+// (more than 48 KB of LDS: the kernel is told once)
+#define FRK_GO_BIG(UU)                                                                                                        \
+    do {                                                                                                                      \
+        static bool sized = false;                                                                                            \
+        if (!sized) {                                                                                                         \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_q8_0_f32_shared_kernel<UU, WAVES>),         \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * UU);                        \
+            if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv q8_0, LDS): %s", hipGetErrorString(e)); \
+            sized = true;                                                                                                     \
+        }                                                                                                                     \
+        hipLaunchKernelGGL((gemv_q8_0_f32_shared_kernel<UU, WAVES>), grid, block, 4096 * UU, s, w->dev, w->layout, (int)w->rows, \
+                           nb, x, y);                                                                                         \
+    } while (0)
+    if (u <= 20) FRK_GO_BIG(20);
+    else if (u <= 24) FRK_GO_BIG(24);
+    else FRK_GO_BIG(28);  // (2 * 28 loads in flight behind the activation's: vmcnt counts to 63)
+#undef FRK_GO_BIG
+    FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");
     return FRK_OK;
 }
 

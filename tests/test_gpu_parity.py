@@ -215,6 +215,8 @@ GEMV_SHAPES = [
     # Q8_0 rows of 8224 .. 16384 columns with at least 1024 rows: the activation shared through LDS, 11 to 16 units a lane
     (fo.Q8_0, 1024, 14336), (fo.Q8_0, 1500, 11008), (fo.Q8_0, 1027, 16384), (fo.Q8_0, 1100, 8704), (fo.Q8_0, 1030, 10240),
     (fo.Q8_0, 1025, 22016), (fo.Q8_0, 1030, 28672), (fo.Q8_0, 1024, 18432), (fo.Q8_0, 40, 28672), (fo.Q8_0, 1024, 28704),
+    # (the wavefronts split the columns: rows that fill a workgroup's four or eight and do not, a last wavefront short of units)
+    (fo.Q8_0, 1, 1056), (fo.Q8_0, 3, 16384), (fo.Q8_0, 4, 1088), (fo.Q8_0, 13, 3104), (fo.Q8_0, 9000, 2048), (fo.Q8_0, 8197, 4096),
 ]
 
 
