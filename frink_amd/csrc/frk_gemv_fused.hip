@@ -655,6 +655,113 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_rows_kernel(const uint8_
     if (live && b_in == 0 && row < (size_t)rows) y[row] = v;
 }
 
+// One launch for long rows of any block count, with the columns split between the wavefronts of a workgroup:
+// wavefront w takes blocks 4w .. 4w+3 of the workgroup's 8 * U rows, quantizes exactly those four blocks of the
+// activation (through a corner of LDS that only it touches) and keeps its lanes' slices of them in registers for
+// every row.  Nothing is shared before the sums, so no barrier stands between the requests and the arithmetic
+// (a barrier there is reached only once the memory pipeline has taken every wavefront's requests); the
+// wavefronts' partial sums of a row meet in LDS at the very end, added in the order of the columns.
+// Round j of a wavefront covers rows 8j .. 8j+7 of the workgroup: lane = 8 * (row of the round) + unit, a unit
+// being a half block as in gemv_q4_k_fused_kernel (the block's header and four of its eight 16-byte words).
+constexpr int COLS_WAVE_LDS = 4 * (QK_K + 32 + 4);  // four blocks: quants, 16-wide sums, scale
+template <int U>
+__global__ __launch_bounds__(1024) void gemv_q4_k_cols_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int nb,
+                                                             const float *__restrict__ x, float *__restrict__ y) {
+    typedef float xv_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+    extern __shared__ uint4 smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), waves = blockDim.x >> 6;
+    uint8_t *mine = reinterpret_cast<uint8_t *>(smem) + wave * COLS_WAVE_LDS;
+    float *parts = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(smem) + waves * COLS_WAVE_LDS);
+    const int b0 = wave * 4, r0 = (int)blockIdx.x * 8 * U;
+
+    // the activation's loads first: a wavefront's loads return in issue order
+    xv_t xv[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {  // (a block past the row's end: the last one again, not used)
+        const float *src = x + (size_t)min(b0 + i, nb - 1) * QK_K + lane * 4;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xv[i]) : "v"(src) : "memory");
+    }
+    const int ul = lane & 7, bl = ul >> 1, q = ul & 1;
+    const bool live = b0 + bl < nb;
+    const int b = min(b0 + bl, nb - 1);
+    u4_t wh[U], w0[U], w1[U], w2[U], w3[U];
+    auto request = [&](int j) {
+        const int r = min(r0 + 8 * j + (lane >> 3), rows - 1);  // a row past the end: the last one again, not stored
+        const uint8_t *blk = W + (size_t)r * row_stride + (size_t)b * Q4_K_BYTES;
+        const uint8_t *qs = blk + 16 + 32 * q;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(wh[j]) : "v"(blk) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(w0[j]) : "v"(qs) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(w1[j]) : "v"(qs) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=v"(w2[j]) : "v"(qs) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:80" : "=v"(w3[j]) : "v"(qs) : "memory");
+    };
+    request(0);
+    // (the other rounds are requested once the activation is here: behind every wavefront's later rounds a late
+    // wavefront's activation came late)
+    asm volatile("s_waitcnt vmcnt(5)" : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]));
+#pragma unroll
+    for (int j = 1; j < U; j++) request(j);
+
+    uint32_t *sq = reinterpret_cast<uint32_t *>(mine);
+    int16_t *sbs = reinterpret_cast<int16_t *>(mine + 4 * QK_K);
+    float *sd = reinterpret_cast<float *>(mine + 4 * QK_K + 4 * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float d;
+        int s16;
+        const uint32_t packed = quantize_q8_k_lane<false>(make_float4(xv[i].x, xv[i].y, xv[i].z, xv[i].w), d, s16);
+        sq[i * 64 + lane] = packed;
+        if ((lane & 3) == 0) sbs[i * 16 + (lane >> 2)] = (int16_t)s16;
+        if (lane == 0) sd[i] = d;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    Q4Unit unit;
+    {
+        const uint4 *ap = reinterpret_cast<const uint4 *>(mine + bl * QK_K + q * 64);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            unit.a[i] = ap[i];
+            unit.a[4 + i] = ap[8 + i];
+        }
+        const int16_t *bp = sbs + bl * 16 + q * 4;
+        unit.bs[0] = (int)bp[0] + (int)bp[1];
+        unit.bs[1] = (int)bp[2] + (int)bp[3];
+        unit.bs[2] = (int)bp[8] + (int)bp[9];
+        unit.bs[3] = (int)bp[10] + (int)bp[11];
+        unit.da = live ? sd[bl] : 0.0f;  // a lane past the end of the row contributes nothing
+        unit.sh = q * 16;
+    }
+    auto as4 = [](u4_t v) { return make_uint4(v.x, v.y, v.z, v.w); };
+    float sums[U];
+#define FRK_COLS_ROUND(j)                                                                                         \
+    if constexpr (U > j) {                                                                                        \
+        asm volatile("s_waitcnt vmcnt(%5)"                                                                        \
+                     : "+v"(wh[j]), "+v"(w0[j]), "+v"(w1[j]), "+v"(w2[j]), "+v"(w3[j])                            \
+                     : "n"(5 * (U - 1 - j)));                                                                     \
+        const float term = q4_k_unit_dot(as4(wh[j]), as4(w0[j]), as4(w1[j]), as4(w2[j]), as4(w3[j]), unit);       \
+        sums[j] = part_sum<8>(live ? term : 0.0f);                                                                \
+    }
+    FRK_COLS_ROUND(0)
+    FRK_COLS_ROUND(1)
+    FRK_COLS_ROUND(2)
+#undef FRK_COLS_ROUND
+    static_assert(U <= 3, "three rounds at most: a fourth does not fit the registers of sixteen wavefronts");
+#pragma unroll
+    for (int j = 0; j < U; j++)
+        if (ul == 0) parts[wave * (8 * U) + 8 * j + (lane >> 3)] = sums[j];
+    lds_barrier();
+    // a row's partial sums, in the order of the columns
+    if ((int)threadIdx.x < 8 * U && r0 + (int)threadIdx.x < rows) {
+        float v = 0.0f;
+        for (int w = 0; w < waves; w++) v += parts[w * (8 * U) + threadIdx.x];
+        y[r0 + threadIdx.x] = v;
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -840,14 +947,52 @@ int launch_gemv_rows_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t
 //   5120x5120 7.8 / 5.9 / 6.9    6144x6144 8.7 / 8.8 / 9.0    8192x3072 5.5 / 5.2 / 6.7    3072x3072 3.7 / 4.6 / 5.9
 //   2560x2560 3.4 / 4.5 / 5.8
 // Rows of 8, 16 and 32 blocks have the whole-cache-line kernel (14336x4096: 8.2 / 8.9 / 10.3).
+int launch_gemv_q4_k_cols(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / QK_K), waves = (nb + 3) / 4;
+    const int cus = compute_units();
+    int best_u = 1;
+    size_t best = SIZE_MAX;
+    // rows to a workgroup, 8 * U: the U with the least (workgroups of the busiest CU) x (8 * U rows + the quantization
+    // of the activation, about seven rows' worth), the larger of equals
+    for (int u = 1; u <= 3; u++) {
+        const size_t wgs = (w->rows + 8 * u - 1) / (8 * u);
+        const size_t cost = (wgs + cus - 1) / cus * (8 * u + 7);
+        if (cost <= best) best = cost, best_u = u;
+    }
+    const size_t lds = (size_t)waves * (COLS_WAVE_LDS + 8 * best_u * 4);
+    const dim3 grid((unsigned)((w->rows + 8 * best_u - 1) / (8 * best_u))), block(64 * waves);
+#define FRK_GO_COLS(UU) \
+    hipLaunchKernelGGL((gemv_q4_k_cols_kernel<UU>), grid, block, lds, s, w->dev, w->layout.row_stride, (int)w->rows, nb, x, y)
+    if (best_u == 1) FRK_GO_COLS(1);
+    else if (best_u == 2) FRK_GO_COLS(2);
+    else FRK_GO_COLS(3);  // (four rounds do not fit the registers of sixteen wavefronts)
+#undef FRK_GO_COLS
+    FRK_LAUNCH_CHECK("gemv_q4_k_cols");
+    return FRK_OK;
+}
+
+// Which kernel a one-launch GEMV of Q4_K / Q5_K rows of other lengths than 8 and 16 blocks takes.
 int rows_gemv_form(const frk_weights *w) {
     if (!rows_gemv_fits(w)) return ROWS_FORM_NONE;
     const size_t nb = w->cols / QK_K;
-    // (Q5_K rows of 64 blocks: the whole-cache-line kernel in one launch is ahead, 9.2 us against 12.2 at 2048x16384)
-    if (nb == 64 && w->kind == FRK_KIND_Q5_K) return ROWS_FORM_NONE;
-    if (nb > 32) return ROWS_FORM_QUANTIZED;
+    if (w->kind == FRK_KIND_Q4_K) {
+        // The column form, measured against what was there (us): 4096x14336 10.5 / 12.5, 4096x11008 9.2 / 11.5,
+        // 5120x13824 12.6 / 14.2, 8192x10240 14.1 / 17.3, 4096x6144 6.0 / 6.4, 2048x14336 7.0 / 8.8; against the
+        // whole-cache-line kernel at 64 blocks 4096x16384 11.2 / 12.9, 2048x16384 7.4 / 9.3, at 32 blocks
+        // 28672x8192 28.9 / 36.0, 14336x8192 17.1 / 21.0, 8192x8192 11.1 / 12.1, 1024x8192 4.8 / 5.3, but
+        // 4096x8192 7.2 / 6.8; rows of 20 blocks 5120x5120 6.3 / 6.0, of 16 blocks 14336x4096 10.5 / 8.1.
+        if (nb > 20 && nb != 32) return ROWS_FORM_COLUMNS;
+        if (nb == 32 && (w->rows <= 2048 || w->rows >= 6144)) return ROWS_FORM_COLUMNS;
+    }
     if (nb > 16 && nb < 32) return ROWS_FORM_ONE_LAUNCH;
+    if (rows_gemv_takes_quantized(w)) return ROWS_FORM_QUANTIZED;
     return ROWS_FORM_NONE;
+}
+// Rows of more than 32 blocks from activations quantized beforehand: whole rows to a wavefront.
+// (Q5_K rows of 64 blocks: the whole-cache-line kernel is ahead, 9.2 us against 12.2 at 2048x16384.)
+bool rows_gemv_takes_quantized(const frk_weights *w) {
+    const size_t nb = w->cols / QK_K;
+    return rows_gemv_fits(w) && nb > 32 && !(nb == 64 && w->kind == FRK_KIND_Q5_K);
 }
 
 // Q5_K rows of 8, 16, 32 or 64 blocks on the same kernel.  Wavefronts to a workgroup, measured (one-launch form,

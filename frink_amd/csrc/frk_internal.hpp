@@ -157,8 +157,10 @@ bool q5_k_lines_gemv_fits(const frk_weights *w);
 bool rows_gemv_fits(const frk_weights *w);
 // which form a decode GEMV of the matrix takes on that kernel: none (the other kernels are ahead), one launch
 // with the quantization inside, or a quantization launch and the kernel over Q8_K activations
-enum { ROWS_FORM_NONE = 0, ROWS_FORM_ONE_LAUNCH = 1, ROWS_FORM_QUANTIZED = 2 };
+enum { ROWS_FORM_NONE = 0, ROWS_FORM_ONE_LAUNCH = 1, ROWS_FORM_QUANTIZED = 2, ROWS_FORM_COLUMNS = 3 };
+int launch_gemv_q4_k_cols(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int rows_gemv_form(const frk_weights *w);
+bool rows_gemv_takes_quantized(const frk_weights *w);
 int launch_gemv_rows_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 int launch_gemv_rows_preq(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q5_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);

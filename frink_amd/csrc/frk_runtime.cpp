@@ -478,6 +478,7 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q4_K:
     case FRK_KIND_Q5_K: {
         const int form = rows_gemv_form(w);  // rows of 17..31 and of 33..64 blocks: whole rows to a wavefront
+        if (form == ROWS_FORM_COLUMNS) return launch_gemv_q4_k_cols(w, x, y, s);
         if (form == ROWS_FORM_ONE_LAUNCH) return launch_gemv_rows_fused(w, x, y, s);
         if (form == ROWS_FORM_QUANTIZED) {
             Q8KActs a;
@@ -530,7 +531,7 @@ int frk_hip_gemv_q8k_dev(const frk_weights *w, const int8_t *q, const float *d, 
     clear_error();
     if (!w || !q || !d || !bsums || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemv_q8k_dev: null argument");
     Q8KActs a{q, d, bsums};
-    if ((w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K) && rows_gemv_form(w) == ROWS_FORM_QUANTIZED)
+    if ((w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K) && rows_gemv_takes_quantized(w))
         return launch_gemv_rows_preq(w, a, y, (hipStream_t)stream);
     if (w->kind == FRK_KIND_Q4_K)
         return fused_gemv_fits(w) ? launch_gemv_q4_k_preq(w, a, y, (hipStream_t)stream)
