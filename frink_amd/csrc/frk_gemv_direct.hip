@@ -481,6 +481,67 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_f32_cols_kernel(const uint8_t 
     }
 }
 
+// Q4_0 x f32 the same way (dot_q4_0_f32, crates/frink-quant/src/lib.rs:4253-4276; blocks of 32 weights as 16 bytes of
+// nibbles -- byte i: element i low, element i + 16 high -- in the quant plane and an f16 scale in the scale plane):
+// wavefront w takes blocks 64w .. 64w+63 of the workgroup's R rows, a lane keeps its block's 32 activations and their
+// sum in registers.  The sum is taken over the raw nibbles and eight times the block's sum of x comes off afterwards,
+// as in gemv_q4_0_f32_kernel.
+template <int R>
+__global__ __launch_bounds__(1024) void gemv_q4_0_f32_cols_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
+                                                                 const float *__restrict__ x, float *__restrict__ y) {
+    extern __shared__ uint4 smem_direct[];
+    float *parts = reinterpret_cast<float *>(smem_direct);  // [wavefront][row]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const bool live = wave * 64 + lane < nb;
+    const int u = min(wave * 64 + lane, nb - 1);  // (a lane past the end: the last block again, not added)
+    const int r0 = (int)blockIdx.x * R;
+    const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)u * 32);
+    float4 xv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) xv[i] = xp[i];
+    uint4 qv[R];
+    uint32_t dbits[R];
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        const uint8_t *row = W + (size_t)min(r0 + k, rows - 1) * lay.row_stride;  // (a row past the end: the last again)
+        qv[k] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
+        dbits[k] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)u * 2);
+    }
+    float xsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; i++) xsum += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        float s = 0.0f;
+#define FRK_Q4_STEP(c, kk)                                                       \
+    {                                                                            \
+        const float4 lo = xv[kk], hi = xv[4 + kk];                               \
+        const uint32_t nl = qv[k].c & 0x0f0f0f0fu, nh = (qv[k].c >> 4) & 0x0f0f0f0fu; \
+        s = fmaf((float)(nl & 0xff), lo.x, s);                                   \
+        s = fmaf((float)(nh & 0xff), hi.x, s);                                   \
+        s = fmaf((float)((nl >> 8) & 0xff), lo.y, s);                            \
+        s = fmaf((float)((nh >> 8) & 0xff), hi.y, s);                            \
+        s = fmaf((float)((nl >> 16) & 0xff), lo.z, s);                           \
+        s = fmaf((float)((nh >> 16) & 0xff), hi.z, s);                           \
+        s = fmaf((float)(nl >> 24), lo.w, s);                                    \
+        s = fmaf((float)(nh >> 24), hi.w, s);                                    \
+    }
+        FRK_Q4_STEP(x, 0)
+        FRK_Q4_STEP(y, 1)
+        FRK_Q4_STEP(z, 2)
+        FRK_Q4_STEP(w, 3)
+#undef FRK_Q4_STEP
+        const float v = part_sum<64>(live ? fmaf(-8.0f, xsum, s) * h2f(dbits[k]) : 0.0f);
+        if (lane == 0) parts[wave * R + k] = v;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < R && r0 + (int)threadIdx.x < rows) {
+        float v = 0.0f;
+        for (int w = 0; w < waves; w++) v += parts[w * R + threadIdx.x];
+        y[r0 + threadIdx.x] = v;
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -636,6 +697,23 @@ int launch_gemv_q8_0_f32_direct(const frk_weights *w, const float *x, float *y, 
     else FRK_GO_BIG(28);  // (2 * 28 loads in flight behind the activation's: vmcnt counts to 63)
 #undef FRK_GO_BIG
     FRK_LAUNCH_CHECK("gemv_q8_0_f32_shared");
+    return FRK_OK;
+}
+
+// Q4_0 rows of up to 32768 columns (1024 blocks: sixteen wavefronts).  Against gemv_q4_0_f32_kernel, which stages the
+// activation in LDS behind a barrier (us): 4096x14336 12.3 / 18.5, 4096x11008 11.1 / 15.2, 4096x4096 5.3 / 5.9,
+// 1024x4096 3.8 / 5.5, 32000x4096 20.6 / 22.7, 14336x4096 12.0 / 12.0.
+bool q4_0_cols_form(const frk_weights *w) { return w->kind == FRK_KIND_Q4_0 && w->cols / Q8_0_ELEMS <= 1024; }
+int launch_gemv_q4_0_f32_cols(const frk_weights *w, const float *x, float *y, hipStream_t s) {
+    const int nb = (int)(w->cols / Q8_0_ELEMS), waves = (nb + 63) / 64;
+    const bool four = (w->rows / 8) * (size_t)waves < 12 * (size_t)compute_units_direct();
+#define FRK_GO_COLS(RR)                                                                                                       \
+    hipLaunchKernelGGL((gemv_q4_0_f32_cols_kernel<RR>), dim3((unsigned)((w->rows + RR - 1) / RR)), dim3(64 * waves),           \
+                       (size_t)waves * RR * 4, s, w->dev, w->layout, (int)w->rows, nb, x, y)
+    if (four) FRK_GO_COLS(4);
+    else FRK_GO_COLS(8);
+#undef FRK_GO_COLS
+    FRK_LAUNCH_CHECK("gemv_q4_0_f32_cols");
     return FRK_OK;
 }
 

@@ -254,6 +254,8 @@ int launch_route_top_k_softmax(const float *logits, int batch, int n_experts, in
                                float *weights, hipStream_t s);
 // prefetch-all GEMVs (one wavefront per row, no LDS) for rows of 33..256 units
 bool direct_gemv_fits(const frk_weights *w);
+bool q4_0_cols_form(const frk_weights *w);
+int launch_gemv_q4_0_f32_cols(const frk_weights *w, const float *x, float *y, hipStream_t s);
 bool q6_k_cols_form(const frk_weights *w);  // the one-launch Q6_K GEMV whose wavefronts split the columns
 int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream_t s);
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);

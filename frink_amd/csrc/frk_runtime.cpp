@@ -502,7 +502,7 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     case FRK_KIND_Q4_0:
     case FRK_KIND_Q8_0: {
         if (act_mode == FRK_ACT_F32) {
-            if (w->kind == FRK_KIND_Q4_0) return launch_gemv_q4_0_f32(w, x, y, s);
+            if (w->kind == FRK_KIND_Q4_0) return q4_0_cols_form(w) ? launch_gemv_q4_0_f32_cols(w, x, y, s) : launch_gemv_q4_0_f32(w, x, y, s);
             return direct_gemv_fits(w) ? launch_gemv_q8_0_f32_direct(w, x, y, s) : launch_gemv_q8_0_f32(w, x, y, s);
         }
         size_t n = w->cols;

@@ -460,7 +460,8 @@ def _random_q4_0(rows, cols, seed):
     return data.ravel()
 
 
-@pytest.mark.parametrize("rows,cols", [(64, 4096), (37, 4096), (7, 32), (9, 544), (5, 2048), (4096, 4096)])
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (37, 4096), (7, 32), (9, 544), (5, 2048), (4096, 4096), (1, 2080), (13, 14336),
+                                       (8200, 2048), (3, 32768), (10, 6176), (5, 34816)])
 def test_q4_0_dequant_and_decode(fa, rows, cols):
     """Q4_0 (18-byte blocks: an f16 scale and 16 bytes of nibbles, value (nibble - 8) * d) is kept as a
     plane of nibbles and a plane of scales.  The reference holds no encoder for it, so the blocks are
