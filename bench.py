@@ -269,9 +269,9 @@ def main():
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_lines_kernel<16, 0, 8, false, 4>", "algorithmic_bytes": int(alg_bytes),
+                     "kernel": "gemv_q4_k_lines_kernel<16, 0, 8, false, 4, false>", "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(sec_per_step * 1e6, 3), "launches": args.steps,
-                     "prequantized_form": {"kernel": "gemv_q4_k_lines_kernel<16, 1, 8, false, 0>",
+                     "prequantized_form": {"kernel": "gemv_q4_k_lines_kernel<16, 1, 8, false, 0, false>",
                                            "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k,
                                            "frac": round((wbytes + cols + cols // 256 * 4 + cols // 16 * 2 + rows * 4)
                                                          / k_sec / 1e9 / HBM_PEAK_GBS, 4)}},
