@@ -904,6 +904,9 @@ static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, fl
         // one round of workgroups that fills the CUs (two workgroups each): part of the span behind the barrier
         const size_t wgs = (w->rows * (size_t)16 / 64 + WIDE - 1) / WIDE, room = 2 * (size_t)compute_units();
         if (MODE == MODE_FUSED && wgs <= room && 4 * wgs >= 3 * room) return launch_q4_k_lines_as<16, MODE, WIDE, false, 4>(w, x, a, y, s);
+        // few workgroups: four wavefronts each, so that twice as many CUs take part (4096x4096 4.4 against 4.7 us,
+        // 1024x4096 from quantized activations 3.1 / 3.6; two wavefronts quantize eight blocks each: 5.6 at 1024x4096)
+        if (wgs <= (size_t)compute_units() / 2) return launch_q4_k_lines_as<16, MODE, 4>(w, x, a, y, s);
         return launch_q4_k_lines_as<16, MODE, WIDE>(w, x, a, y, s);
     }
     if (nb == 32) return launch_q4_k_lines_as<32, MODE, WIDE>(w, x, a, y, s);
