@@ -118,10 +118,18 @@ __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f<DPP_QUAD_XOR1>(v));
     v = fmaxf(v, dpp_f<DPP_QUAD_XOR2>(v));
     v = fmaxf(v, dpp_f<DPP_HALF_MIRROR>(v));
-    v = fmaxf(v, dpp_f<DPP_ROW_MIRROR>(v));
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
+    v = fmaxf(v, dpp_f<DPP_ROW_MIRROR>(v));  // every lane of a row of 16 holds its row's maximum
+    // across the rows without a trip through LDS: the row before's last lane into rows 1 and 3, lane 31 into rows 2
+    // and 3 (row_bcast15 / row_bcast31, other rows keep their value), and lane 63's total read out as a scalar
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int r1 = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x142, 0xa, 0xf, false);
+    v = fmaxf(v, __int_as_float(r1));
+    const int r2 = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x143, 0xc, 0xf, false);
+    v = fmaxf(v, __int_as_float(r2));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+#else
     return v;
+#endif
 }
 
 // expf the way glibc computes it (2.28 and later, every architecture: sysdeps/ieee754/flt-32/e_expf.c, the

@@ -16,53 +16,56 @@ __global__ __launch_bounds__(64) void route_top_k_softmax_kernel(const float *__
                                                                  int32_t *__restrict__ ids,
                                                                  float *__restrict__ weights) {
     __shared__ float prob[1024];
-    __shared__ float s_sum;
+    __shared__ uint64_t table[32];
     const int b = blockIdx.x, lane = threadIdx.x;
     const float *l = logits + (size_t)b * n_experts;
+    // This kernel is one wavefront and as long as its chain of dependent steps: the exponential's table is asked
+    // for beside the logits (not when the first exponent is known), a lane's candidates stay in registers (expert
+    // i lives in lane i % 64, register i / 64), and the ids leave in one store at the end.
+    const uint64_t entry = EXPF_TABLE[lane & 31];
+    float p[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) p[j] = lane + 64 * j < n_experts ? l[lane + 64 * j] : -INFINITY;
+    table[lane & 31] = entry;
     float mx = -INFINITY;
-    for (int i = lane; i < n_experts; i += 64) mx = fmaxf(mx, l[i]);
+#pragma unroll
+    for (int j = 0; j < 16; j++) mx = fmaxf(mx, p[j]);
     mx = wave_max(mx);
-    for (int i = lane; i < n_experts; i += 64) prob[i] = expf_as_libm(l[i] - mx);  // (a host's bits, as the reference's f32::exp gives them)
     __syncthreads();
-    if (lane == 0) {
-        float sum = 0.0f;
-        for (int i = 0; i < n_experts; i++) sum += prob[i];
-        s_sum = sum;
-    }
+#pragma unroll
+    for (int j = 0; j < 16; j++)
+        if (64 * j < n_experts) {  // uniform
+            p[j] = expf_as_libm(p[j] - mx, table);  // (a host's bits, as the reference's f32::exp gives them)
+            if (lane + 64 * j < n_experts) prob[lane + 64 * j] = p[j];
+        }
     __syncthreads();
-    const float sum = s_sum;
-    for (int i = lane; i < n_experts; i += 64) prob[i] = __fdiv_rn(prob[i], sum);
-    __syncthreads();
+    float sum = 0.0f;  // every lane adds all of them in index order, as the reference does: no broadcast afterwards
+    for (int i = 0; i < n_experts; i++) sum += prob[i];
+#pragma unroll
+    for (int j = 0; j < 16; j++) p[j] = lane + 64 * j < n_experts ? __fdiv_rn(p[j], sum) : -2.0f;  // (-2: no candidate)
     float top_sum = 0.0f, mine = 0.0f;  // lane s keeps the s-th weight
+    int mine_i = 0;
     for (int s = 0; s < k; s++) {
-        // wave argmax: larger probability, then smaller index
+        // argmax over the wavefront: larger probability, then smaller index
         float best = -1.0f;
         int best_i = 0x7fffffff;
-        for (int i = lane; i < n_experts; i += 64) {
-            const float p = prob[i];
-            if (p > best) {
-                best = p;
-                best_i = i;
-            }
-        }
 #pragma unroll
-        for (int m = 1; m < 64; m <<= 1) {
-            const float ob = __shfl_xor(best, m);
-            const int oi = __shfl_xor(best_i, m);
-            if (ob > best || (ob == best && oi < best_i)) {
-                best = ob;
-                best_i = oi;
-            }
-        }
-        if (lane == 0) {
-            ids[(size_t)b * k + s] = best_i;
-            prob[best_i] = -2.0f;  // taken
-        }
-        if (lane == s) mine = best;
-        top_sum += best;  // same order in every lane: the reference's sum over the k weights
-        __syncthreads();
+        for (int j = 0; j < 16; j++)
+            if (p[j] > best) best = p[j], best_i = lane + 64 * j;
+        // (two maxima, mostly DPP: the largest probability, then the smallest index among the lanes that hold it --
+        // an index up to 1024 is exact as a float)
+        const float top = wave_max(best);
+        best_i = n_experts - (int)wave_max(best == top ? (float)(n_experts - best_i) : -1.0f);
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+            if (best_i == lane + 64 * j) p[j] = -2.0f;  // taken
+        if (lane == s) mine = top, mine_i = best_i;
+        top_sum += top;  // same order in every lane: the reference's sum over the k weights
     }
-    if (lane < k) weights[(size_t)b * k + lane] = norm ? __fdiv_rn(mine, top_sum) : mine;
+    if (lane < k) {
+        ids[(size_t)b * k + lane] = mine_i;
+        weights[(size_t)b * k + lane] = norm ? __fdiv_rn(mine, top_sum) : mine;
+    }
 }
 
 // Exclusive scan over the workgroup's 1024 threads (16 wavefronts); `total` gets the sum.
