@@ -129,6 +129,44 @@ __device__ __forceinline__ float q4_k_unit_dot(const uint4 h, const uint4 w0, co
     return (d * U.da) * (float)s1 - (dmin * U.da) * (float)s2;
 }
 
+// dot_q5_k_q8 (crates/frink-quant/src/lib.rs:886-938) for one unit of one row: the same with every weight's fifth
+// bit put over its nibble (fa, fb: the block's 32 bytes of fifth bits, byte l holding weight l of every sub-block,
+// sub-block j in bit j; the unit's sub-blocks are 2q, 2q+1, 2q+4 and 2q+5).
+__device__ __forceinline__ float q5_k_unit_dot(const uint4 h, const uint4 fa, const uint4 fb, const uint4 w0, const uint4 w1,
+                                               const uint4 w2, const uint4 w3, const Q4Unit &U, int q) {
+    const uint32_t hy = h.y >> U.sh, hz = h.z >> U.sh, hw = h.w >> U.sh;  // bytes 0,1 are ours now
+    const uint32_t sc_lo = hy & 0x3f3fu, m_lo = hz & 0x3f3fu;
+    const uint32_t sc_hi = (hw & 0x0f0fu) | (((hy >> 6) & 0x0303u) << 4);
+    const uint32_t m_hi = ((hw >> 4) & 0x0f0fu) | (((hz >> 6) & 0x0303u) << 4);
+    auto code = [](uint32_t nib, uint32_t fifth, int j) { return (((fifth >> j) & 0x01010101u) << 4) | (nib & 0x0f0f0f0fu); };
+    int i0 = 0, i1 = 0, i2 = 0, i3 = 0;
+#define FRK_Q5(ACC, WW, FF, AV, SH, J)                       \
+    ACC = dot4(code(WW.x >> SH, FF.x, J), AV.x, ACC);        \
+    ACC = dot4(code(WW.y >> SH, FF.y, J), AV.y, ACC);        \
+    ACC = dot4(code(WW.z >> SH, FF.z, J), AV.z, ACC);        \
+    ACC = dot4(code(WW.w >> SH, FF.w, J), AV.w, ACC);
+    const int j = 2 * q;
+    FRK_Q5(i0, w0, fa, U.a[0], 0, j)
+    FRK_Q5(i0, w1, fb, U.a[1], 0, j)
+    FRK_Q5(i1, w0, fa, U.a[2], 4, j + 1)
+    FRK_Q5(i1, w1, fb, U.a[3], 4, j + 1)
+    FRK_Q5(i2, w2, fa, U.a[4], 0, j + 4)
+    FRK_Q5(i2, w3, fb, U.a[5], 0, j + 4)
+    FRK_Q5(i3, w2, fa, U.a[6], 4, j + 5)
+    FRK_Q5(i3, w3, fb, U.a[7], 4, j + 5)
+#undef FRK_Q5
+    int s1 = __mul24((int)(sc_lo & 0xff), i0);
+    s1 += __mul24((int)(sc_lo >> 8), i1);
+    s1 += __mul24((int)(sc_hi & 0xff), i2);
+    s1 += __mul24((int)(sc_hi >> 8), i3);
+    int s2 = __mul24((int)(m_lo & 0xff), U.bs[0]);
+    s2 += __mul24((int)(m_lo >> 8), U.bs[1]);
+    s2 += __mul24((int)(m_hi & 0xff), U.bs[2]);
+    s2 += __mul24((int)(m_hi >> 8), U.bs[3]);
+    const float d = h2f(h.x & 0xffffu), dmin = h2f(h.x >> 16);
+    return (d * U.da) * (float)s1 - (dmin * U.da) * (float)s2;
+}
+
 // LPR lanes share a row (a wavefront works on 64/LPR rows at once), a lane owns units
 // l, l+LPR, ... (J of them) and keeps RPW rounds of rows in flight.
 // GLU: two matrices of one shape (gate = W, up = W2) in one launch; row r of both is computed by the
@@ -678,7 +716,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_rows_kernel(const uint8_
 // Round j of a wavefront covers rows 8j .. 8j+7 of the workgroup: lane = 8 * (row of the round) + unit, a unit
 // being a half block as in gemv_q4_k_fused_kernel (the block's header and four of its eight 16-byte words).
 constexpr int COLS_WAVE_LDS = 4 * (QK_K + 32 + 4);  // four blocks: quants, 16-wide sums, scale
-template <int U>
+template <int U, bool Q5 = false>
 __global__ __launch_bounds__(1024) void gemv_q4_k_cols_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int nb,
                                                              const float *__restrict__ x, float *__restrict__ y) {
     typedef float xv_t __attribute__((ext_vector_type(4)));
@@ -700,12 +738,18 @@ __global__ __launch_bounds__(1024) void gemv_q4_k_cols_kernel(const uint8_t *__r
     const int ul = lane & 7, bl = ul >> 1, q = ul & 1;
     const bool live = b0 + bl < nb;
     const int b = min(b0 + bl, nb - 1);
-    u4_t wh[U], w0[U], w1[U], w2[U], w3[U];
+    // (Q5: Q5_K blocks, Q4_K's with 32 bytes of fifth bits between the header and the nibbles -- seven loads a round)
+    constexpr int BB = Q5 ? Q5_K_BYTES : Q4_K_BYTES, LOADS = Q5 ? 7 : 5;
+    u4_t wh[U], w0[U], w1[U], w2[U], w3[U], fa[Q5 ? U : 1], fb[Q5 ? U : 1];
     auto request = [&](int j) {
         const int r = min(r0 + 8 * j + (lane >> 3), rows - 1);  // a row past the end: the last one again, not stored
-        const uint8_t *blk = W + (size_t)r * row_stride + (size_t)b * Q4_K_BYTES;
-        const uint8_t *qs = blk + 16 + 32 * q;
+        const uint8_t *blk = W + (size_t)r * row_stride + (size_t)b * BB;
+        const uint8_t *qs = blk + (BB - 128) + 32 * q;
         asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(wh[j]) : "v"(blk) : "memory");
+        if constexpr (Q5) {
+            asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(fa[j]) : "v"(blk) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(fb[j]) : "v"(blk) : "memory");
+        }
         asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(w0[j]) : "v"(qs) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(w1[j]) : "v"(qs) : "memory");
         asm volatile("global_load_dwordx4 %0, %1, off offset:64" : "=v"(w2[j]) : "v"(qs) : "memory");
@@ -714,7 +758,7 @@ __global__ __launch_bounds__(1024) void gemv_q4_k_cols_kernel(const uint8_t *__r
     request(0);
     // (the other rounds are requested once the activation is here: behind every wavefront's later rounds a late
     // wavefront's activation came late)
-    asm volatile("s_waitcnt vmcnt(5)" : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]));
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(xv[0]), "+v"(xv[1]), "+v"(xv[2]), "+v"(xv[3]) : "n"(LOADS));
 #pragma unroll
     for (int j = 1; j < U; j++) request(j);
 
@@ -753,17 +797,25 @@ __global__ __launch_bounds__(1024) void gemv_q4_k_cols_kernel(const uint8_t *__r
     float sums[U];
 #define FRK_COLS_ROUND(j)                                                                                         \
     if constexpr (U > j) {                                                                                        \
-        asm volatile("s_waitcnt vmcnt(%5)"                                                                        \
-                     : "+v"(wh[j]), "+v"(w0[j]), "+v"(w1[j]), "+v"(w2[j]), "+v"(w3[j])                            \
-                     : "n"(5 * (U - 1 - j)));                                                                     \
-        const float term = q4_k_unit_dot(as4(wh[j]), as4(w0[j]), as4(w1[j]), as4(w2[j]), as4(w3[j]), unit);       \
+        float term;                                                                                               \
+        if constexpr (Q5) {                                                                                       \
+            asm volatile("s_waitcnt vmcnt(%7)"                                                                    \
+                         : "+v"(wh[j]), "+v"(fa[j]), "+v"(fb[j]), "+v"(w0[j]), "+v"(w1[j]), "+v"(w2[j]), "+v"(w3[j]) \
+                         : "n"(LOADS * (U - 1 - j)));                                                             \
+            term = q5_k_unit_dot(as4(wh[j]), as4(fa[j]), as4(fb[j]), as4(w0[j]), as4(w1[j]), as4(w2[j]), as4(w3[j]), unit, q); \
+        } else {                                                                                                  \
+            asm volatile("s_waitcnt vmcnt(%5)"                                                                    \
+                         : "+v"(wh[j]), "+v"(w0[j]), "+v"(w1[j]), "+v"(w2[j]), "+v"(w3[j])                        \
+                         : "n"(LOADS * (U - 1 - j)));                                                             \
+            term = q4_k_unit_dot(as4(wh[j]), as4(w0[j]), as4(w1[j]), as4(w2[j]), as4(w3[j]), unit);               \
+        }                                                                                                         \
         sums[j] = part_sum<8>(live ? term : 0.0f);                                                                \
     }
     FRK_COLS_ROUND(0)
     FRK_COLS_ROUND(1)
     FRK_COLS_ROUND(2)
 #undef FRK_COLS_ROUND
-    static_assert(U <= 3, "three rounds at most: a fourth does not fit the registers of sixteen wavefronts");
+    static_assert(U <= (Q5 ? 2 : 3), "three rounds at most (Q5_K: two): more do not fit the registers of sixteen wavefronts");
 #pragma unroll
     for (int j = 0; j < U; j++)
         if (ul == 0) parts[wave * (8 * U) + 8 * j + (lane >> 3)] = sums[j];
@@ -975,7 +1027,8 @@ int launch_gemv_q4_k_cols(const frk_weights *w, const float *x, float *y, hipStr
     size_t best = SIZE_MAX;
     // rows to a workgroup, 8 * U: the U with the least (workgroups of the busiest CU) x (8 * U rows + the quantization
     // of the activation, about seven rows' worth), the larger of equals
-    for (int u = 1; u <= 3; u++) {
+    const bool q5 = w->kind == FRK_KIND_Q5_K;
+    for (int u = 1; u <= (q5 ? 2 : 3); u++) {
         const size_t wgs = (w->rows + 8 * u - 1) / (8 * u);
         const size_t cost = (wgs + cus - 1) / cus * (8 * u + 7);
         if (cost <= best) best = cost, best_u = u;
@@ -984,9 +1037,14 @@ int launch_gemv_q4_k_cols(const frk_weights *w, const float *x, float *y, hipStr
     const dim3 grid((unsigned)((w->rows + 8 * best_u - 1) / (8 * best_u))), block(64 * waves);
 #define FRK_GO_COLS(UU) \
     hipLaunchKernelGGL((gemv_q4_k_cols_kernel<UU>), grid, block, lds, s, w->dev, w->layout.row_stride, (int)w->rows, nb, x, y)
-    if (best_u == 1) FRK_GO_COLS(1);
+#define FRK_GO_COLS5(UU) \
+    hipLaunchKernelGGL((gemv_q4_k_cols_kernel<UU, true>), grid, block, lds, s, w->dev, w->layout.row_stride, (int)w->rows, nb, x, y)
+    if (q5 && best_u == 1) FRK_GO_COLS5(1);
+    else if (q5) FRK_GO_COLS5(2);
+    else if (best_u == 1) FRK_GO_COLS(1);
     else if (best_u == 2) FRK_GO_COLS(2);
     else FRK_GO_COLS(3);  // (four rounds do not fit the registers of sixteen wavefronts)
+#undef FRK_GO_COLS5
 #undef FRK_GO_COLS
     FRK_LAUNCH_CHECK("gemv_q4_k_cols");
     return FRK_OK;
@@ -1005,6 +1063,9 @@ int rows_gemv_form(const frk_weights *w) {
         if (nb > 20 && nb != 32) return ROWS_FORM_COLUMNS;
         if (nb == 32 && (w->rows <= 2048 || w->rows >= 6144)) return ROWS_FORM_COLUMNS;
     }
+    // Q5_K on the same kernel (two rounds at most): 4096x14336 12.8 / 14.8, 4096x11008 10.4 / 13.7, 8192x10240 17.5 / 22.5,
+    // 4096x16384 13.3 / 16.8, 2048x16384 8.3 / 9.1; up to 32 blocks it is behind (5120x5120 7.6 / 6.8, 4096x8192 8.3 / 7.3)
+    if (w->kind == FRK_KIND_Q5_K && nb > 32) return ROWS_FORM_COLUMNS;
     if (nb > 16 && nb < 32) return ROWS_FORM_ONE_LAUNCH;
     if (rows_gemv_takes_quantized(w)) return ROWS_FORM_QUANTIZED;
     return ROWS_FORM_NONE;
