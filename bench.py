@@ -300,9 +300,12 @@ def main():
         for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
                                  ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
                                  ("Q5_K GEMV 14336x4096 (one launch)", fa.Q5_K, 14336, 4096),
-                                 ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096)):
+                                 ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096),
+                                 ("Q4_K GEMV 4096x14336 (a Q4_K down projection)", fa.Q4_K, 4096, 14336),
+                                 ("Q4_K GEMV 4096x4096 (attention projection)", fa.Q4_K, 4096, 4096),
+                                 ("Q8_0 GEMV 4096x14336", fa.Q8_0, 4096, 14336)):
             d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
-            n_copies = COPIES if k2 != fa.Q8_0 else 32
+            n_copies = max(COPIES, -(-560_000_000 // d2.numel()))  # (past the 256 MB Infinity Cache, like the headline's copies)
             w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]
             x2 = torch.from_numpy(synth.activations(5, 1, c2)[0]).to(dev)
             y2 = torch.empty(r2, dtype=torch.float32, device=dev)
