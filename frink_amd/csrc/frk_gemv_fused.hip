@@ -955,6 +955,11 @@ static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, fl
     if (nb == 16) {
         // one round of workgroups that fills the CUs (two workgroups each): part of the span behind the barrier
         const size_t wgs = (w->rows * (size_t)16 / 64 + WIDE - 1) / WIDE, room = 2 * (size_t)compute_units();
+        // between one and one and a half workgroups of eight a CU (10240, 11008 rows): six wavefronts to a workgroup
+        // spread the spans more evenly (11008x4096 7.5 against 7.8 us, from quantized activations 6.8 / 7.2; five
+        // and seven are behind six, and 12288 rows and more are best with eight)
+        if (2 * wgs > room && 4 * wgs < 3 * room)
+            return MODE == MODE_FUSED ? launch_q4_k_lines_as<16, MODE, 6, false, 4>(w, x, a, y, s) : launch_q4_k_lines_as<16, MODE, 6>(w, x, a, y, s);
         if (MODE == MODE_FUSED && wgs <= room && 4 * wgs >= 3 * room) return launch_q4_k_lines_as<16, MODE, WIDE, false, 4>(w, x, a, y, s);
         // few workgroups: four wavefronts each, so that twice as many CUs take part (4096x4096 4.4 against 4.7 us,
         // 1024x4096 from quantized activations 3.1 / 3.6; two wavefronts quantize eight blocks each: 5.6 at 1024x4096)

@@ -278,7 +278,7 @@ def test_gemv_quantizes_a_nan_to_zero_inside_the_launch(fa, kind, rows, cols):
 
 
 @pytest.mark.parametrize("rows,cols", [(5, 2048), (8, 2048), (100, 2048), (1, 4096), (4, 4096), (131, 4096), (3, 8192), (50, 8192),
-                                       (1, 16384), (33, 16384)])
+                                       (1, 16384), (33, 16384), (4100, 4096), (10301, 4096), (14336, 4096)])
 @pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K])
 def test_q4_k_gemv_over_whole_cache_lines(fa, kind, rows, cols):
     """Rows of 2048 .. 16384 columns take the kernel that gives a wavefront 64 consecutive blocks (8, 4, 2 or
@@ -286,8 +286,11 @@ def test_q4_k_gemv_over_whole_cache_lines(fa, kind, rows, cols):
     quantization inside the launch and from activations quantized beforehand, which must agree bit for bit
     (the same integers, the same float order).  Q5_K runs on the same kernel, the fifth bits put over the
     nibbles on their way into the dot."""
+    from bench import random_blocks
     from frink_amd import synth
-    data = make_weights(kind, rows, cols, seed=rows + cols)
+    # (the row counts at which the launch changes its workgroups -- four, six or eight wavefronts, part of the span
+    # behind the barrier -- need thousands of rows: random block bytes, encoding that many takes too long)
+    data = random_blocks(kind, rows, cols, rows + cols) if rows > 2000 else make_weights(kind, rows, cols, seed=rows + cols)
     x = synth.activations(rows * 3 + cols, 1, cols, outlier_frac=0.01)[0]
     w = fa.Weights.from_host(kind, data, rows, cols)
     xd = to_dev(x)
