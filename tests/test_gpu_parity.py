@@ -159,6 +159,9 @@ def _q8k_cases():
         "nans": _with(synth.activations(16, 1, 2048).ravel(), {3: np.nan, 300: -np.nan, 511: np.nan, 1024: np.nan}),
         "infinities": _with(synth.activations(17, 1, 1024).ravel(), {5: np.inf, 6: -np.inf, 700: np.inf, 701: np.nan}),
         "all_nan": np.full(256, np.nan, np.float32),
+        # a block of subnormal values: 127 / amax overflows to infinity, the clamp binds and the scale is zero
+        "subnormal": (synth.normal(18, 512, 1.0) * np.float32(1e-40)).astype(np.float32),
+        "smallest_normals": (synth.normal(19, 512, 1.0) * np.float32(3e-37)).astype(np.float32),
     }
 
 
@@ -194,7 +197,9 @@ def test_quantize_q8_0_is_bit_exact(fa):
              head([np.uint32(0x4013E709).view(np.float32), np.uint32(0x3CDF99C0).view(np.float32)]),
              synth.activations(21, 4, 4096).ravel(), synth.normal(22, 320, 1e-6),
              _with(synth.activations(23, 1, 256).ravel(), {3: np.nan, 40: np.inf, 41: 1.0, 100: -np.nan}),
-             np.full(32, np.nan, np.float32)]
+             np.full(32, np.nan, np.float32),
+             (synth.normal(24, 320, 1.0) * np.float32(1e-40)).astype(np.float32),
+             (synth.normal(25, 320, 1.0) * np.float32(3e-37)).astype(np.float32)]
     for x in cases:
         q, d = fa.quantize_q8_0(to_dev(x))
         wq, wd = fo.quantize_q8_0(x, fo.FORM_AVX)
