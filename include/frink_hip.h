@@ -281,8 +281,9 @@ int frk_hip_get_rows(const frk_weights *w, const int32_t *ids_host, size_t n_ids
 /* Plain device copy of `bytes` (multiple of 16), used to calibrate HBM counters and as the
  * practical bandwidth ceiling a streaming kernel of the same size can reach. */
 int frk_hip_copy_dev(const void *src_dev, void *dst_dev, size_t bytes, void *stream);
-/* Read-only stream over `bytes` (multiple of 16): every 16-byte word is loaded and folded
- * into 4 bytes per workgroup written to sink_dev (>= 64 KiB). */
+/* Read-only stream over `bytes` (multiple of 16): every 16-byte word is loaded and nothing is
+ * written -- a thread stores into sink_dev (>= 64 KiB) only if its words fold to one particular
+ * value, which is there to keep the loads alive. */
 int frk_hip_read_dev(const void *src_dev, size_t bytes, void *sink_dev, void *stream);
 
 #ifdef __cplusplus
