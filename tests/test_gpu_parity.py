@@ -997,7 +997,7 @@ def test_other_kinds_gemv_matches_the_oracle(fa, kind, rows, cols, batch):
 # ------------------------------------------------------------------ the K-quants' f32 dot (the reference's x86 decode default)
 
 @pytest.mark.parametrize("kind,rows,cols", [
-    (fo.Q4_K, 70, 1024), (fo.Q4_K, 9, 256), (fo.Q4_K, 300, 4096), (fo.Q4_K, 17, 16384),
+    (fo.Q4_K, 70, 1024), (fo.Q4_K, 9, 256), (fo.Q4_K, 300, 4096), (fo.Q4_K, 17, 16384), (fo.Q4_K, 3, 11008), (fo.Q4_K, 1, 6400),
     (fo.Q5_K, 70, 1024), (fo.Q5_K, 33, 768), (fo.Q5_K, 128, 4096),
     (fo.Q6_K, 70, 1024), (fo.Q6_K, 5, 256), (fo.Q6_K, 64, 14336), (fo.Q6_K, 257, 2048),
 ])
