@@ -951,7 +951,13 @@ template <int MODE>
 static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, float *y, hipStream_t s) {
     const int nb = (int)(w->cols / QK_K);
     constexpr int WIDE = 8;
-    if (nb == 8) return launch_q4_k_lines_as<8, MODE, WIDE>(w, x, a, y, s);
+    // (few workgroups -- fewer of eight wavefronts than half the CUs: four wavefronts each, twice as many CUs take part)
+    const size_t few = (size_t)compute_units() / 2;
+    if (nb == 8) {  // 4096x2048 3.5 against 4.0 us, 8192x2048 4.0 / 4.35
+        const size_t wgs8 = (w->rows * (size_t)8 / 64 + WIDE - 1) / WIDE;
+        if (wgs8 <= few) return launch_q4_k_lines_as<8, MODE, 4>(w, x, a, y, s);
+        return launch_q4_k_lines_as<8, MODE, WIDE>(w, x, a, y, s);
+    }
     if (nb == 16) {
         // one round of workgroups that fills the CUs (two workgroups each): part of the span behind the barrier
         const size_t wgs = (w->rows * (size_t)16 / 64 + WIDE - 1) / WIDE, room = 2 * (size_t)compute_units();
@@ -963,10 +969,14 @@ static int launch_q4_k_lines(const frk_weights *w, const float *x, Q8KActs a, fl
         if (MODE == MODE_FUSED && wgs <= room && 4 * wgs >= 3 * room) return launch_q4_k_lines_as<16, MODE, WIDE, false, 4>(w, x, a, y, s);
         // few workgroups: four wavefronts each, so that twice as many CUs take part (4096x4096 4.4 against 4.7 us,
         // 1024x4096 from quantized activations 3.1 / 3.6; two wavefronts quantize eight blocks each: 5.6 at 1024x4096)
-        if (wgs <= (size_t)compute_units() / 2) return launch_q4_k_lines_as<16, MODE, 4>(w, x, a, y, s);
+        if (wgs <= few) return launch_q4_k_lines_as<16, MODE, 4>(w, x, a, y, s);
         return launch_q4_k_lines_as<16, MODE, WIDE>(w, x, a, y, s);
     }
-    if (nb == 32) return launch_q4_k_lines_as<32, MODE, WIDE>(w, x, a, y, s);
+    if (nb == 32) {  // (from quantized activations: 2048x8192 4.0 against 4.25 us, 1024x8192 3.4 / 3.85)
+        const size_t wgs32 = (w->rows * (size_t)32 / 64 + WIDE - 1) / WIDE;
+        if (wgs32 <= few) return launch_q4_k_lines_as<32, MODE, 4>(w, x, a, y, s);
+        return launch_q4_k_lines_as<32, MODE, WIDE>(w, x, a, y, s);
+    }
     return launch_q4_k_lines_as<64, MODE, 8>(w, x, a, y, s);
 }
 
