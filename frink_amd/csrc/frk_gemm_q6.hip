@@ -452,14 +452,20 @@ size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows) {
 }
 
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
+    const Q8KTiled acts = q8k_tiled_carve(ws, M, w->cols);
+    int rc = launch_quantize_q8_k_tiled(x, M, w->cols, acts, s);
+    if (rc) return rc;
+    return launch_gemm_q6_k_acts(w, acts, M, y, reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256)), s);
+}
+
+// the GEMM proper, over activations already in the tiled form (`partial`: room for the parts' sums)
+int launch_gemm_q6_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *y, float *partial, hipStream_t s) {
     // the kernel addresses the weights and the tiled activations with 32-bit byte offsets
     if ((uint64_t)w->rows * w->layout.row_stride >= (1ull << 32) || (uint64_t)q8k_tiled_bytes(M, w->cols) >= (1ull << 32))
         return set_error(FRK_ERR_SHAPE, "gemm_q6_k: %zu x %zu weights with %zu activation rows exceed 4 GiB per operand", w->rows,
                          w->cols, M);
     Q6GemmArgs g;
-    g.a = q8k_tiled_carve(ws, M, w->cols);
-    int rc = launch_quantize_q8_k_tiled(x, M, w->cols, g.a, s);
-    if (rc) return rc;
+    g.a = acts;
     g.W = w->dev;
     g.row_stride = (uint32_t)w->layout.row_stride;
     g.off_qh = (uint32_t)w->layout.off_a;
@@ -480,7 +486,7 @@ int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, v
     g.tiles = nullptr;
     g.n_tiles = nullptr;
     g.k_split = ks;
-    g.partial = reinterpret_cast<float *>((char *)ws + round_up(q8k_tiled_bytes(M, w->cols), 256));
+    g.partial = partial;
     g.row_tiles = (int)((w->rows + rows_wg - 1) / rows_wg);
     const dim3 grid((unsigned)((g.row_tiles + 7) / 8 * 8 * g.tok_tiles), (unsigned)g.k_split);
     static bool sized = false;  // a benign race: every thread sets the same attribute

@@ -212,6 +212,7 @@ int launch_gemm_q4_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *
 // the same for Q6_K (frk_gemm_q6.hip)
 size_t gemm_q6_k_workspace_bytes(size_t M, size_t cols, size_t rows);
 int launch_gemm_q6_k(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+int launch_gemm_q6_k_acts(const frk_weights *w, Q8KTiled acts, size_t M, float *y, float *partial, hipStream_t s);
 // its grouped (per-expert) form: tile t = rows [64*t, 64*t+64) of the activations and of y, tiles[t] =
 // {expert, 64*t, rows in use, 0}, tiles past *n_tiles idle; expert e owns rows [e*rows_e, (e+1)*rows_e) of w
 int launch_gemm_q6_k_grouped(const frk_weights *w, size_t rows_e, Q8KTiled a, const int4 *tiles, const int *n_tiles,

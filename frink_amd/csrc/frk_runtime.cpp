@@ -60,6 +60,7 @@ struct StreamWorkspace {
     std::recursive_mutex mu;  // held by the thread whose entry point is enqueueing on the stream
     void *ptr = nullptr;
     size_t bytes = 0;
+    bool in_a_graph = false;  // a call was enqueued on it while the stream was being captured: a graph holds its address
     int depth = 0;                 // nested leases of the holder
     std::vector<std::pair<void *, size_t>> outgrown;  // replaced under a lease; retired when the outermost ends
 };
@@ -71,9 +72,10 @@ struct RetiredBuffer {
 static std::map<hipStream_t, StreamWorkspace *> g_ws;  // under g_dev.mu; entries live until the process ends
 static std::vector<RetiredBuffer> g_retired;           // under g_dev.mu
 
-// A retired buffer of at least `bytes` whose last use has passed, or a fresh allocation.  Retired
-// buffers that are idle and too small are given back to the driver here, where an allocation is
-// being paid for anyway.
+// A retired buffer of at least `bytes` whose last use has passed, or a fresh allocation.  Nothing is
+// given back to the driver here: hipFree waits for the whole device, which would stall every other
+// stream's calls from inside this one.  Idle retired buffers stay in the pool (a stream's buffer is
+// replaced only when a larger shape first runs on it, so the pool holds a handful of them).
 static int take_buffer_locked(size_t bytes, void **ptr, size_t *got) {
     size_t best = g_retired.size();
     for (size_t i = 0; i < g_retired.size(); i++) {
@@ -89,16 +91,6 @@ static int take_buffer_locked(size_t bytes, void **ptr, size_t *got) {
         (void)hipEventDestroy(g_retired[best].passed);
         g_retired.erase(g_retired.begin() + (long)best);
         return FRK_OK;
-    }
-    for (size_t i = 0; i < g_retired.size();) {
-        if (hipEventQuery(g_retired[i].passed) == hipSuccess) {
-            (void)hipFree(g_retired[i].ptr);
-            (void)hipEventDestroy(g_retired[i].passed);
-            g_retired.erase(g_retired.begin() + (long)i);
-        } else {
-            (void)hipGetLastError();
-            i++;
-        }
     }
     const size_t want = std::max<size_t>(round_up(bytes, 1 << 20), 4u << 20);
     FRK_HIP_TRY(hipMalloc(ptr, want));
@@ -120,9 +112,13 @@ int workspace(size_t bytes, hipStream_t stream, WorkspaceLease &lease) {
         lease.held_ = w;
         lease.stream_ = stream;
     }
+    // A graph captured from this stream replays the buffer's address for as long as the graph lives, which
+    // the library cannot see: a buffer that was current during a capture is never handed to another stream
+    // nor reused after a growth -- it stays allocated, untouched by later calls, until the process ends.
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cs) != hipSuccess) (void)hipGetLastError();
+    if (cs != hipStreamCaptureStatusNone && bytes <= w->bytes) w->in_a_graph = true;
     if (bytes > w->bytes) {
-        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &cs) != hipSuccess) (void)hipGetLastError();
         if (cs != hipStreamCaptureStatusNone)
             return set_error(FRK_ERR_HIP,
                              "the stream's scratch buffer holds %zu bytes and this call needs %zu: it cannot grow while the "
@@ -134,9 +130,10 @@ int workspace(size_t bytes, hipStream_t stream, WorkspaceLease &lease) {
             int rc = take_buffer_locked(bytes, &fresh, &got);
             if (rc) return rc;
         }
-        if (w->ptr) w->outgrown.emplace_back(w->ptr, w->bytes);
+        if (w->ptr && !w->in_a_graph) w->outgrown.emplace_back(w->ptr, w->bytes);  // (one a graph holds: kept, see above)
         w->ptr = fresh;
         w->bytes = got;
+        w->in_a_graph = false;
     }
     lease.ptr = w->ptr;
     return FRK_OK;
@@ -698,6 +695,126 @@ int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const fl
     return gemm_impl(w1, x, batch, y1, stream, scratch);
 }
 
+// ---- a batch's activations quantized once, for any number of matrices (BatchActs::Q8K) ----
+// The object owns room for both forms the K-quant kernels read: plain Q8_K rows (the decode and thin kernels)
+// and the tiled form (the matrix-core GEMMs).  Which of them a batch gets depends on its size alone, so that
+// the quantization does not need to know the matrices: plain rows up to ACTS_PLAIN_MAX_BATCH rows (the thin
+// kernels take at most 40), tiles from ACTS_TILED_MIN_BATCH rows on (no matrix-core GEMM starts below 17).
+constexpr size_t ACTS_PLAIN_MAX_BATCH = 64, ACTS_TILED_MIN_BATCH = 17;
+}  // extern "C"
+struct frk_batch_acts {
+    size_t max_batch = 0, cols = 0;
+    void *base = nullptr;       // one allocation: plain rows, then the tiled form
+    size_t tiled_off = 0;
+    size_t batch = 0;           // rows of the last quantization (0: none yet)
+    frk::Q8KActs plain{nullptr, nullptr, nullptr};
+};
+namespace {
+size_t acts_plain_bytes(size_t batch, size_t cols) {
+    const size_t n = batch * cols;
+    return frk::round_up(n, 256) + frk::round_up(n / frk::QK_K * 4, 256) + frk::round_up(n / 16 * 2, 256);
+}
+}  // namespace
+extern "C" {
+
+int frk_hip_batch_acts_create(size_t max_batch, size_t cols, frk_batch_acts **out) {
+    clear_error();
+    if (!out) return set_error(FRK_ERR_ARG, "frk_hip_batch_acts_create: null argument");
+    *out = nullptr;
+    if (max_batch == 0 || cols == 0 || cols % QK_K != 0)
+        return set_error(FRK_ERR_SHAPE, "batch activations: %zu rows of %zu columns (whole 256-column blocks, at least one row)", max_batch, cols);
+    {
+        std::lock_guard<std::mutex> lk(g_dev.mu);
+        int rc = ensure_device_locked();
+        if (rc) return rc;
+    }
+    frk_batch_acts *a = new frk_batch_acts();
+    a->max_batch = max_batch;
+    a->cols = cols;
+    a->tiled_off = round_up(acts_plain_bytes(std::min(max_batch, ACTS_PLAIN_MAX_BATCH), cols), 256);
+    const size_t bytes = a->tiled_off + (max_batch >= ACTS_TILED_MIN_BATCH ? round_up(q8k_tiled_bytes(max_batch, cols), 256) : 0);
+    hipError_t e = hipMalloc(&a->base, bytes);
+    if (e != hipSuccess) {
+        delete a;
+        return set_error(FRK_ERR_HIP, "hipMalloc(%zu) for batch activations: %s", bytes, hipGetErrorString(e));
+    }
+    *out = a;
+    return FRK_OK;
+}
+
+int frk_hip_batch_acts_release(frk_batch_acts *a) {
+    clear_error();
+    if (!a) return FRK_OK;
+    hipError_t e = hipFree(a->base);
+    delete a;
+    if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFree: %s", hipGetErrorString(e));
+    return FRK_OK;
+}
+
+int frk_hip_quantize_batch_acts_dev(frk_batch_acts *a, const float *x, size_t batch, void *stream) {
+    clear_error();
+    if (!a || !x) return set_error(FRK_ERR_ARG, "frk_hip_quantize_batch_acts_dev: null argument");
+    if (batch == 0 || batch > a->max_batch)
+        return set_error(FRK_ERR_SHAPE, "a batch of %zu rows in an object made for at most %zu", batch, a->max_batch);
+    hipStream_t s = (hipStream_t)stream;
+    a->batch = 0;
+    if (batch <= ACTS_PLAIN_MAX_BATCH) {
+        const size_t n = batch * a->cols;
+        int8_t *q = (int8_t *)a->base;
+        float *d = (float *)((char *)a->base + round_up(n, 256));
+        int16_t *b = (int16_t *)((char *)a->base + round_up(n, 256) + round_up(n / QK_K * 4, 256));
+        int rc = launch_quantize_q8_k(x, n, q, d, b, s);
+        if (rc) return rc;
+        a->plain = Q8KActs{q, d, b};
+    }
+    if (batch >= ACTS_TILED_MIN_BATCH) {
+        int rc = launch_quantize_q8_k_tiled(x, batch, a->cols, q8k_tiled_carve((char *)a->base + a->tiled_off, batch, a->cols), s);
+        if (rc) return rc;
+    }
+    a->batch = batch;
+    return FRK_OK;
+}
+
+int frk_hip_gemm_acts_dev(const frk_weights *w, const frk_batch_acts *a, float *y, void *stream) {
+    clear_error();
+    if (!w || !a || !y) return set_error(FRK_ERR_ARG, "frk_hip_gemm_acts_dev: null argument");
+    if (a->batch == 0) return set_error(FRK_ERR_ARG, "frk_hip_gemm_acts_dev: the activations hold no quantized batch");
+    if (w->cols != a->cols)
+        return set_error(FRK_ERR_SHAPE, "the matrix has %zu columns, the quantized activations %zu", w->cols, a->cols);
+    const bool k_quant = w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K;
+    if (!k_quant)
+        return set_error(FRK_ERR_UNSUPPORTED, "Q8_K activations feed Q4_K, Q5_K and Q6_K weights only (kind %d): frk_hip_gemm_dev", w->kind);
+    const size_t batch = a->batch;
+    hipStream_t s = (hipStream_t)stream;
+    const bool q45 = q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch);
+    if (q45 || q6_k_takes_the_matrix_cores(w, batch)) {
+        const Q8KTiled acts = q8k_tiled_carve((char *)a->base + a->tiled_off, batch, a->cols);
+        const size_t acts_bytes = round_up(q8k_tiled_bytes(batch, w->cols), 256);
+        const size_t need = q45 ? gemm_q4_k_workspace_bytes(batch, w->cols, w->rows, w->kind == FRK_KIND_Q5_K)
+                                : gemm_q6_k_workspace_bytes(batch, w->cols, w->rows);
+        float *partial = nullptr;
+        Scratch scratch;
+        if (need > acts_bytes) {  // a split of the blocks between workgroups: room for the parts' sums
+            void *ws = nullptr;
+            int rc = scratch.get(need - acts_bytes, s, &ws);
+            if (rc) return rc;
+            partial = (float *)ws;
+        }
+        return q45 ? launch_gemm_q4_k_acts(w, acts, batch, y, partial, s) : launch_gemm_q6_k_acts(w, acts, batch, y, partial, s);
+    }
+    // (below the matrix-core GEMMs' batches the plain rows are there: ACTS_PLAIN_MAX_BATCH covers every such batch)
+    if (batch > ACTS_PLAIN_MAX_BATCH)
+        return set_error(FRK_ERR_UNSUPPORTED, "a batch of %zu rows of this matrix has no kernel over quantized activations", batch);
+    if (batch == 1) return frk_hip_gemv_q8k_dev(w, a->plain.q, a->plain.d, a->plain.bsums, y, stream);
+    if (batch_takes_the_thin_kernels(w, batch)) return thin_gemm_acts(w, a->plain, batch, thin_gemm_max_batch(w), y, s);
+    const size_t nb = w->cols / QK_K;  // rows too long for the thin kernels: a decode launch per row
+    for (size_t b = 0; b < batch; b++) {
+        int rc = frk_hip_gemv_q8k_dev(w, a->plain.q + b * w->cols, a->plain.d + b * nb, a->plain.bsums + b * nb * 16, y + b * w->rows, stream);
+        if (rc) return rc;
+    }
+    return FRK_OK;
+}
+
 // ---- the entry point that allocates nothing ----
 // Its scratch memory is this array in the library's device image: every GPU the library runs on holds
 // its own copy, at its own address, until the process ends.  In host code the array's name is only a
@@ -783,8 +900,8 @@ int frk_hip_gemv_multi_dev(const frk_weights *const *ws, size_t n, const float *
     }
     for (size_t i = 0; i < n; i++) {
         int rc;
-        if (ws[i]->kind == FRK_KIND_Q8_0 || ws[i]->kind == FRK_KIND_Q4_0)
-            rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);
+        if (ws[i]->kind == FRK_KIND_Q8_0 || ws[i]->kind == FRK_KIND_Q4_0 || is_unit_kind(ws[i]->kind))
+            rc = frk_hip_gemv_dev(ws[i], x, ys[i], FRK_ACT_F32, stream);  // (these kinds multiply the f32 activation itself)
         else rc = frk_hip_gemv_q8k_dev(ws[i], a.q, a.d, a.bsums, ys[i], stream);
         if (rc) return rc;
     }

@@ -25,15 +25,27 @@ def splitmix64(seed, start, count):
 
 
 def normal(seed, count, sigma=1.0, start=0):
-    """`count` float32 values N(0, sigma) for counters start .. start+count."""
+    """`count` float32 values N(0, sigma) for counters start .. start+count.  (Large counts are generated in
+    chunks by a few threads: element i depends on (seed, i) only, so the result does not depend on how.)"""
     out = np.empty(count, np.float32)
-    step = 1 << 22
-    for lo in range(0, count, step):
+    step = 1 << 20
+
+    def chunk(lo):
         n = min(step, count - lo)
         z = splitmix64(seed, start + lo, n)
         u1 = ((z >> np.uint64(40)).astype(np.float64) + 1.0) / 16777216.0
         u2 = ((z >> np.uint64(16)) & np.uint64(0xFFFFFF)).astype(np.float64) / 16777216.0
         out[lo:lo + n] = (np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2) * sigma).astype(np.float32)
+
+    starts = range(0, count, step)
+    if count <= 4 * step:
+        for lo in starts:
+            chunk(lo)
+    else:
+        import os
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 1)) as pool:
+            list(pool.map(chunk, starts))
     return out
 
 

@@ -163,10 +163,15 @@ int frk_hip_launch_dense_ffn_swiglu(const frk_matvec_launch *gate, const frk_mat
  * Scratch memory (quantized activations, intermediates) is one library-owned buffer PER STREAM, held by
  * the calling thread while it enqueues a call's launches: calls on different streams never share
  * scratch, calls on one stream from several threads go out one after the other (as the reference's
- * rayon workers call the seam, gpu_backend.rs:722-725).  A buffer that is too small is replaced, not
- * freed in place, and nothing in these calls waits for the device.  While a stream is being captured
- * into a graph its buffer cannot grow: run each shape once before capturing it (a call that would need
- * to grow returns FRK_ERR_HIP and launches nothing). */
+ * rayon workers call the seam, gpu_backend.rs:722-725).  A buffer that is too small is replaced by a
+ * larger one (a hipMalloc on the first call of a larger shape; the old one is retired behind an event
+ * and reused, never given back to the driver by a call: nothing in these calls waits for the device).
+ * HIP graphs: while a stream is being captured its buffer cannot grow -- run each shape once before
+ * capturing it (a call that would need to grow returns FRK_ERR_HIP and launches nothing) -- and a
+ * buffer that was current during a capture belongs to that graph from then on: a later, larger call
+ * on the stream gets a new buffer and the old one stays allocated and untouched until the process
+ * ends, so replays of the graph stay valid (at the price of that memory).  Callers that capture
+ * without a warm call, or cannot have the library allocate at all, use frk_hip_gemm_noalloc_dev. */
 
 /* y[rows] = W x for one activation vector in HBM.  K-quants: x is quantized to Q8_K
  * on the device first (bit-exact with quantize_activations_q8_k,

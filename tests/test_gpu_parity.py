@@ -283,7 +283,8 @@ def test_gemv_quantizes_a_nan_to_zero_inside_the_launch(fa, kind, rows, cols):
 
 
 @pytest.mark.parametrize("rows,cols", [(5, 2048), (8, 2048), (100, 2048), (1, 4096), (4, 4096), (131, 4096), (3, 8192), (50, 8192),
-                                       (1, 16384), (33, 16384), (4100, 4096), (10301, 4096), (14336, 4096)])
+                                       (1, 16384), (33, 16384), (4100, 4096), (10301, 4096), (14336, 4096), (8200, 2048),
+                                       (4096, 8192)])
 @pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q5_K])
 def test_q4_k_gemv_over_whole_cache_lines(fa, kind, rows, cols):
     """Rows of 2048 .. 16384 columns take the kernel that gives a wavefront 64 consecutive blocks (8, 4, 2 or
@@ -604,10 +605,20 @@ def test_gemm_large_tiles_with_ragged_edges(fa, rows, cols, batch):
     w.release()
 
 
+def _oracle_gemm_all_rows(data, rows, cols, x):
+    """The oracle's integer-dot GEMM over EVERY weight row.  Its AVX2 form is held bit-equal to the scalar
+    functions by tests/test_oracle_goldens.py and does 14336 x 4096 x 512 in a fraction of a second; a host
+    without AVX2 falls back to the scalar functions, threaded."""
+    if fo.have_avx2():
+        import os
+        return fo.avx2_gemm_q4_k_q8k(data, rows, cols, x, threads=min(16, os.cpu_count() or 1))
+    return fo.gemm(fo.Q4_K, data, rows, cols, x)
+
+
 @pytest.mark.parametrize("rows,cols", [(4096, 4096), (14336, 4096)])
 def test_full_size_prefill_gemm(fa, rows, cols):
-    """M=512 with 1% outliers at +-20: every output row of the batch against the oracle on a
-    slice of weight rows (the oracle takes seconds per 512 rows), plus exact homogeneity."""
+    """M=512 with 1% outliers at +-20: every output of the batch, all weight rows, against the oracle,
+    plus exact homogeneity."""
     from frink_amd import synth
     print("full gemm", rows, cols, flush=True)
     batch = 512
@@ -615,11 +626,13 @@ def test_full_size_prefill_gemm(fa, rows, cols):
     x = synth.activations(77, batch, cols, outlier_frac=0.01)
     w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
     y = w.gemm(to_dev(x)).cpu().numpy()
-    for row0 in (0, rows // 2 - 64, rows - 256):
-        want = fo.gemm(fo.Q4_K, data, rows, cols, x, row0=row0, nrows=256)
-        ninf = np.abs(want).max(axis=1)
-        err = np.abs(y[:, row0:row0 + 256] - want).max(axis=1)
-        assert (err <= TOL * ninf).all(), (row0, float((err / ninf).max()))
+    want = _oracle_gemm_all_rows(data, rows, cols, x)
+    # (the scalar functions themselves on one slice, whatever the host)
+    assert np.array_equal(bits(want[:, 512:544]), bits(fo.gemm(fo.Q4_K, data, rows, cols, x, row0=512, nrows=32)))
+    ninf = np.abs(want).max(axis=1)
+    err = np.abs(y - want).max(axis=1)
+    record("Q4_K gemm M=512 %dx%d, all rows" % (rows, cols), float((err / ninf).max()))
+    assert (err <= TOL * ninf).all(), float((err / ninf).max())
     y2 = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
     assert np.array_equal(bits(y2), bits(y * np.float32(0.5)))
     w.release()
@@ -662,13 +675,7 @@ def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False, sigma=0.
     shapes = ((n_experts * ffn, hidden), (n_experts * ffn, hidden), (n_experts * hidden, ffn))
     out = []
     for i, (rows, cols) in enumerate(shapes):
-        if random_blocks == "encoded":
-            # N(0, sigma) from numpy's generator (the documented splitmix generator takes minutes for
-            # 600 M values), encoded by the oracle's threaded Q4_K encoder
-            w = np.random.default_rng(seed + i).standard_normal((rows, cols), dtype=np.float32) * np.float32(sigma)
-            out.append(fo.encode_matrix(fo.Q4_K, w))
-            del w
-        elif random_blocks:
+        if random_blocks:
             # any bytes are a valid block; keep the two f16 super-scales small and finite
             rng = np.random.default_rng(seed + i)
             nblk = rows * cols // 256
@@ -722,14 +729,16 @@ def _end_to_end_gate(got, want, what, strict):
     intermediate to the next int8 level, which shifts that output row by d_act*|w|, and the fewer
     columns the down projection has the larger that is against ||y||inf.  So the stage-by-stage gates
     are the strict ones, and end to end a full-size layer (strict) must hold the tolerance on at least
-    99 % of its rows and twice the tolerance on every row (measured on the 128-expert layer of 2048/768:
-    1 row of 512 at 1.3e-3, the rest below 5e-7 apart from such flips), the small test shapes on 90 % of
-    the rows and ten times the tolerance on every row."""
+    99 % of its rows and one and a half times the tolerance on every row (measured on the 128-expert layer of
+    2048/768: at most one row of 512 above 1e-3, the rest below 5e-7 apart from such flips;
+    _report_flipped_levels prints the intermediate behind the worst row), the small test shapes on 90 % of the
+    rows and ten times the tolerance on every row."""
     rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
     print("%s end-to-end: rows over 1e-3: %d of %d, worst %.3g" % (what, (rel > TOL).sum(), rel.size, rel.max()), flush=True)
     record(what, rel.max())
+    record(what + ": rows over 1e-3", float((rel > TOL).sum()))
     if strict:
-        assert (rel <= TOL).mean() >= 0.99 and rel.max() <= 2 * TOL, "%s: worst row %.3g of ||y||inf" % (what, rel.max())
+        assert (rel <= TOL).mean() >= 0.99 and rel.max() <= 1.5 * TOL, "%s: worst row %.3g of ||y||inf" % (what, rel.max())
     else:
         assert (rel <= TOL).mean() >= 0.9 and rel.max() <= 10 * TOL, "%s: worst row %.3g" % (what, rel.max())
 
@@ -801,8 +810,37 @@ def _moe_case(fa, n_experts, k, hidden, ffn, batch, seed, random_blocks=False, i
     assert_rows_close(got, chained, "down+combine E=%d k=%d batch=%d" % (n_experts, k, batch))
 
     want = _moe_oracle(down_kind, gate, up, down, n_experts, hidden, ffn, x, ids, w)
+    if strict:
+        _report_flipped_levels(what, got, want, gb, ub, hidden, ffn, x, ids, pos, act_q)
     _end_to_end_gate(got, want, what, strict)
     return got, want
+
+
+def _report_flipped_levels(what, got, want, gb, ub, hidden, ffn, x, ids, pos, act_q):
+    """What stands behind the worst row of an end-to-end comparison: the oracle's own chain for that token (its gate
+    and up, its SwiGLU, its Q8_K levels) beside the levels the device quantized from ITS gate and up.  A last-bit
+    difference in a gate or up output that sits on a rounding boundary of the quantizer moves one int8 level; the
+    line printed (and recorded) says how many of the token's k * ffn levels differ and by how much."""
+    rel = np.abs(got - want).max(axis=1) / np.abs(want).max(axis=1)
+    t = int(rel.argmax())
+    flips = []
+    for sl in range(ids.shape[1]):
+        e = int(ids[t, sl])
+        g = fo.gemm(fo.Q4_K, gb[e], ffn, hidden, x[t:t + 1])
+        u = fo.gemm(fo.Q4_K, ub[e], ffn, hidden, x[t:t + 1])
+        q, _, _ = fo.quantize_q8_k(fo.swiglu(g.ravel(), u.ravel()))
+        dev = act_q.reshape(-1, ffn)[int(pos[t, sl])]
+        for i in np.nonzero(q != dev)[0]:
+            flips.append((sl, e, int(i), int(dev[i]), int(q[i])))
+    line = "%s: worst row is token %d at %.3g of ||y||inf; of its %d intermediate levels %d differ from the oracle's own chain: %s" % (
+        what, t, rel[t], ids.shape[1] * ffn, len(flips),
+        "; ".join("slot %d expert %d column %d device %d oracle %d" % f for f in flips[:6]) or "none")
+    print(line, flush=True)
+    import os
+    d = os.environ.get("FRK_TEST_OUT", "")
+    if d and os.path.isdir(d):
+        with open(os.path.join(d, "parity_worst_rows.txt"), "a") as f:
+            f.write(line + "\n")
 
 
 def _moe_per_token_checks(fa, got, gate, up, down, n_experts, k, hidden, ffn, batch, x, ids, w):
@@ -884,9 +922,9 @@ def test_moe_ffn_with_idle_experts_and_one_hot_routing(fa):
 
 def test_moe_ffn_full_size_layer(fa):
     """The MoE configuration itself: 128 experts, top-8, hidden 2048, ffn 768, all Q4_K encoded from
-    N(0, 0.02), 512 tokens N(0, 1): every stage and every token row against the oracle, and the whole
-    layer end to end (_end_to_end_gate, strict)."""
-    got, want = _moe_case(fa, 128, 8, 2048, 768, 512, seed=5, random_blocks="encoded", sigma=0.02, strict=True)
+    N(0, 0.02) of the documented generator (frink_amd/synth.py), 512 tokens N(0, 1): every stage and every token
+    row against the oracle, and the whole layer end to end (_end_to_end_gate, strict)."""
+    got, want = _moe_case(fa, 128, 8, 2048, 768, 512, seed=5, sigma=0.02, strict=True)
     assert np.isfinite(got).all()
 
 
@@ -992,6 +1030,55 @@ def test_other_kinds_gemv_matches_the_oracle(fa, kind, rows, cols, batch):
         w.gemv(to_dev(x[0]), act_mode=fa.ACT_INT8)
     assert e.value.code == fa.ERR_UNSUPPORTED
     w.release()
+
+
+@pytest.mark.parametrize("kind", [fo.Q5_0, fo.IQ4_XS, fo.MXFP4])
+def test_other_kinds_through_the_shared_activation_entry_points(fa, kind):
+    """Q5_0 / IQ4_XS / MXFP4 matrices as q/k/v-style groups (frk_hip_gemv_multi_dev, alone and mixed with a K-quant)
+    and as an FFN's projections (frk_hip_ffn_swiglu_dev and the host-buffer forms): the backend lists these kinds, so
+    every entry point a model's projections go through must take them.  Each output against the oracle: the f32 dot
+    for these kinds, the integer dot for the K-quant beside them."""
+    from frink_amd import synth
+    hidden, ffn = 512, 768
+    bb, be = fo.BLOCK[kind]
+    gate = _other_kind_blocks(kind, ffn, hidden, seed=kind + 1)
+    up = _other_kind_blocks(kind, ffn, hidden, seed=kind + 2)
+    down = _other_kind_blocks(kind, hidden, ffn, seed=kind + 3)
+    kq = make_weights(fo.Q4_K, 96, hidden, seed=kind + 4)
+    x = synth.activations(kind + 5, 1, hidden)[0]
+    wg, wu, wd = (fa.Weights.from_host(kind, d, r, c) for d, r, c in ((gate, ffn, hidden), (up, ffn, hidden), (down, hidden, ffn)))
+    wk = fa.Weights.from_host(fo.Q4_K, kq, 96, hidden)
+    xd = to_dev(x)
+    g_want = fo.gemv(kind, gate, ffn, hidden, x, fo.F32_DOT)
+    u_want = fo.gemv(kind, up, ffn, hidden, x, fo.F32_DOT)
+    k_want = fo.gemv(fo.Q4_K, kq, 96, hidden, x)
+    for group, wants in (([wg, wu], [g_want, u_want]), ([wg, wk, wu], [g_want, k_want, u_want]), ([wk, wg], [k_want, g_want])):
+        outs = fa.gemv_multi(group, xd)
+        for i, (o, want) in enumerate(zip(outs, wants)):
+            assert_rows_close(o.cpu().numpy()[None], want[None], "gemv_multi kind %d, matrix %d of %d" % (kind, i, len(group)))
+    # the FFN: gate, up, SwiGLU, down -- each stage from the device's previous one
+    y = fa.ffn_swiglu(wg, wu, wd, xd).cpu().numpy()
+    g_dev, u_dev = (t.cpu().numpy() for t in fa.gemv_multi([wg, wu], xd))
+    act = fo.swiglu(g_dev, u_dev)
+    assert_rows_close(y[None], fo.gemv(kind, down, hidden, ffn, act, fo.F32_DOT)[None], "ffn_swiglu kind %d" % kind)
+    # mixed: K-quant gate and up, a down projection of this kind
+    g4, u4 = make_weights(fo.Q4_K, ffn, hidden, seed=kind + 6), make_weights(fo.Q4_K, ffn, hidden, seed=kind + 7)
+    w4g, w4u = fa.Weights.from_host(fo.Q4_K, g4, ffn, hidden), fa.Weights.from_host(fo.Q4_K, u4, ffn, hidden)
+    y = fa.ffn_swiglu(w4g, w4u, wd, xd).cpu().numpy()
+    g_dev, u_dev = (t.cpu().numpy() for t in fa.gemv_multi([w4g, w4u], xd))
+    assert_rows_close(y[None], fo.gemv(kind, down, hidden, ffn, fo.swiglu(g_dev, u_dev), fo.F32_DOT)[None], "ffn, down kind %d" % kind)
+    # the host-buffer forms
+    rb = hidden // be * bb
+    outs = fa.launch_matvec_multi(x, [fa.MatvecLaunch.of(kind, gate, ffn, rb), fa.MatvecLaunch.of(fo.Q4_K, kq, 96, hidden // 256 * 144)])
+    assert_rows_close(outs[0][None], g_want[None], "launch_matvec_multi kind %d" % kind)
+    assert_rows_close(outs[1][None], k_want[None], "launch_matvec_multi beside kind %d" % kind)
+    out = fa.launch_dense_ffn_swiglu(fa.MatvecLaunch.of(kind, gate, ffn, rb), fa.MatvecLaunch.of(kind, up, ffn, rb),
+                                     fa.MatvecLaunch.of(kind, down, hidden, ffn // be * bb), x)
+    want = fo.gemv(kind, down, hidden, ffn, fo.swiglu(g_want, u_want), fo.F32_DOT)
+    rel = np.abs(out - want).max() / np.abs(want).max()
+    assert rel <= 10 * TOL, rel  # (end to end over f32 stages: no quantizer between them, reassociation only)
+    for h in (wg, wu, wd, wk, w4g, w4u):
+        h.release()
 
 
 # ------------------------------------------------------------------ the K-quants' f32 dot (the reference's x86 decode default)
@@ -1173,8 +1260,9 @@ def test_gemm_q8_0_keeps_scales_below_the_f16_normal_range(fa):
 
 @pytest.mark.parametrize("kind,rows,cols,seed", [(fo.Q4_K, 14336, 4096, 21), (fo.Q6_K, 4096, 14336, 22)])
 def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
-    """Batched decode, M=8, at the FFN shapes: slices of weight rows against the oracle for every
-    activation row, and each batch row against the decode GEMV of that row."""
+    """Batched decode, M=8, at the FFN shapes: every weight row against the oracle for every
+    activation row (0.5 G multiply-adds: seconds on the threaded scalar oracle), and each batch row
+    against the decode GEMV of that row."""
     from frink_amd import synth
     print("full thin gemm", kind, rows, cols, flush=True)
     data = make_weights(kind, rows, cols, seed=seed)
@@ -1182,11 +1270,11 @@ def test_full_size_thin_gemm_m8(fa, kind, rows, cols, seed):
     w = fa.Weights.from_host(kind, data, rows, cols)
     xd = to_dev(x)
     y = w.gemm(xd).cpu().numpy()
-    for row0 in (0, rows // 2 - 100, rows - 200):
-        want = fo.gemm(kind, data, rows, cols, x, row0=row0, nrows=200)
-        ninf = np.abs(want).max(axis=1)
-        err = np.abs(y[:, row0:row0 + 200] - want).max(axis=1)
-        assert (err <= TOL * ninf).all(), (row0, float((err / ninf).max()))
+    want = fo.gemm(kind, data, rows, cols, x)
+    ninf = np.abs(want).max(axis=1)
+    err = np.abs(y - want).max(axis=1)
+    record("thin gemm M=8 kind %d %dx%d, all rows" % (kind, rows, cols), float((err / ninf).max()))
+    assert (err <= TOL * ninf).all(), float((err / ninf).max())
     one = w.gemv(xd[5].contiguous()).cpu().numpy()
     assert np.abs(one - y[5]).max() <= 1e-5 * np.abs(one).max()
     w.release()
@@ -1370,3 +1458,77 @@ def test_gemm_pair_is_two_gemms_over_one_quantization(fa, kinds, rows, cols, bat
         assert np.array_equal(bits(y.cpu().numpy()), bits(w.gemm(xd).cpu().numpy()))
         assert_rows_close(y.cpu().numpy(), fo.gemm(k, d, r, cols, x), "gemm pair kind %d" % k)
         w.release()
+
+
+def test_host_entry_points_from_four_threads(fa):
+    """frk_hip_launch_matvec / frk_hip_launch_mul_mm called from four threads at once, the way the reference's rayon
+    workers call the seam (crates/frink-core/src/weight_matrix/gpu_backend.rs:722-725): different kinds and shapes
+    per thread, every result the oracle's."""
+    import threading
+    from frink_amd import synth
+    jobs = []
+    for t, (kind, rows, cols, batch) in enumerate(((fo.Q4_K, 200, 1024, 5), (fo.Q6_K, 120, 2048, 3), (fo.Q8_0, 150, 512, 4),
+                                                   (fo.Q4_K, 64, 4096, 40))):
+        bb, be = fo.BLOCK[kind]
+        data = make_weights(kind, rows, cols, seed=1200 + t)
+        x = synth.activations(1210 + t, batch, cols)
+        mode = fo.F32_DOT if kind == fo.Q8_0 else fo.INT_DOT
+        want_v = fo.gemv(kind, data, rows, cols, x[0], mode)
+        want_m = fo.gemm(kind, data, rows, cols, x)  # (a Q8_0 batch is the integer path, as in the reference)
+        jobs.append((kind, data, x, rows, cols, batch, cols // be * bb, want_v, want_m))
+    errors = []
+
+    def work(job):
+        kind, data, x, rows, cols, batch, rb, want_v, want_m = job
+        try:
+            for rep in range(8):
+                got = fa.launch_matvec(kind, data, x[0], rows, rb)
+                assert_rows_close(got[None], want_v[None], "launch_matvec from a thread, kind %d" % kind)
+                got = fa.launch_mul_mm(kind, data, x, rows, cols, batch, rb)
+                assert_rows_close(got, want_m, "launch_mul_mm from a thread, kind %d" % kind)
+        except Exception as e:  # noqa: BLE001 - reported in the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(180)
+    assert not any(t.is_alive() for t in threads), "a thread is still running"
+    assert not errors, errors
+
+
+def test_a_captured_graph_survives_a_larger_call_on_its_stream(fa):
+    """A graph captured from a stream replays the address of the stream's scratch buffer.  A larger call on the same
+    stream afterwards gets a new buffer; the graph's one must stay allocated and untouched: every replay, with larger
+    eager calls on that stream and on another between them, equals the eager result bit for bit."""
+    import torch
+    from frink_amd import synth
+    rows, cols = 384, 1024
+    data = make_weights(fo.Q4_K, rows, cols, seed=1301)
+    w = fa.Weights.from_host(fo.Q4_K, data, rows, cols)
+    big = fa.Weights.from_host(fo.Q4_K, make_weights(fo.Q4_K, 512, 2048, seed=1302), 512, 2048)
+    x = to_dev(synth.activations(1303, 40, cols))
+    xb = to_dev(synth.activations(1304, 300, 2048))
+    stream, other = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        eager = w.gemm(x).clone()          # (sizes the stream's buffer for this shape)
+        y = torch.empty_like(eager)
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            w.gemm(x, out=y)
+        for rep in range(4):
+            y.zero_()
+            g.replay()
+            stream.synchronize()
+            assert np.array_equal(bits(y.cpu().numpy()), bits(eager.cpu().numpy())), rep
+            big.gemm(xb)                   # a larger shape on the graph's stream: the buffer is replaced
+            with torch.cuda.stream(other):
+                big.gemm(xb)               # and one on another stream, which must not be handed the graph's buffer
+            other.synchronize()
+            stream.synchronize()
+    want = fo.gemm(fo.Q4_K, data, rows, cols, x.cpu().numpy())
+    assert_rows_close(eager.cpu().numpy(), want, "gemm under a graph")
+    w.release()
+    big.release()
