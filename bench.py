@@ -30,15 +30,35 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 INT8_PEAK_TOPS = 5000.0  # dense int8 MFMA
 COPIES = 16
+HEADLINE_KERNEL = "gemv_q4_k_lines_kernel<16, 0, 8, false, 4, false>"
 # steps captured per HIP graph in the two timed loops of the headline (a multiple of COPIES): a graph
 # replay starts with a few microseconds of nothing, which 400 steps dilute and 16 would not
 GRAPH_STEPS = 400
-# HBM bytes per launch of the roofline kernel at 14336x4096, from two rocprofv3 --pmc runs of this
-# script (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter reads for
-# copy_kernel over 32,256 KiB: see profiles/bench_kernels_hbm_traffic_pmc.txt
-GEMV_FETCH_KIB, GEMV_WRITE_KIB = 16230.5, 56.0
-COPY_FETCH_KIB, COPY_WRITE_KIB, COPY_KIB = 16138.0, 32256.0, 32256.0
-GEMV_TRAFFIC_BYTES = int((GEMV_FETCH_KIB * COPY_KIB / COPY_FETCH_KIB + GEMV_WRITE_KIB * COPY_KIB / COPY_WRITE_KIB) * 1024)
+# HBM bytes per launch of the roofline kernel: not measurable from inside this script (hardware counters
+# need rocprofv3 around it), so the record carries what the last two rocprofv3 --pmc runs of this script
+# found -- FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same counter reads for
+# copy_kernel over a known size -- read from the summary those runs are kept in, and names that file.
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_kernels_hbm_traffic_pmc.txt")
+
+
+def traffic_from_profile(kernel_prefix):
+    """(bytes per launch, source) from the lines `traffic <kernel> fetch_kib=F write_kib=W` and
+    `calibration copy_kernel kib=K fetch_kib=F write_kib=W` of TRAFFIC_PROFILE; (None, reason) without them."""
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None, "%s is missing" % TRAFFIC_PROFILE
+
+    def fields(line):
+        return {k: float(v) for k, v in (w.split("=") for w in line.split() if "=" in w)}
+    cal = [fields(l) for l in lines if l.startswith("calibration copy_kernel")]
+    mine = [fields(l) for l in lines if l.startswith("traffic " + kernel_prefix)]
+    if not cal or not mine:
+        return None, "%s has no line for %s" % (TRAFFIC_PROFILE, kernel_prefix)
+    c, m = cal[0], mine[0]
+    kib = m["fetch_kib"] * c["kib"] / c["fetch_kib"] + m["write_kib"] * c["kib"] / c["write_kib"]
+    return int(kib * 1024), "%s (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script, scaled by copy_kernel)" % TRAFFIC_PROFILE
 
 
 def random_blocks(kind, rows, cols, seed):
@@ -163,12 +183,33 @@ def cpu_baseline(kind, data, rows, cols, x, y_gpu, xb):
         t, n = best_of(lambda: fo.avx2_gemm_q4_k_q8k(data, rows, cols, xb, threads), 8.0, 5)
         legs["gemm_m512_int_dot_avx2_TOPS"] = round(2.0 * xb.shape[0] * rows * cols / t / 1e12, 4)
         legs["gemm_m512_ms"] = round(t * 1e3, 1)
+        # batched decode, M=8: the same row-outer integer dots, eight activations per weight row (the shape the
+        # reference's 8-row repack tier serves, crates/frink-core/src/weight_matrix.rs:2954-3057)
+        t, n = best_of(lambda: fo.avx2_gemm_q4_k_q8k(data, rows, cols, xb[:8], threads), 3.0)
+        legs["gemm_m8_int_dot_avx2_GBs"] = round(data.size / t / 1e9, 2)
+        legs["gemm_m8_ms"] = round(t * 1e3, 2)
     else:
         headline, what = legs["decode_int_dot_scalar_GBs"], "scalar integer dot (this host has no AVX2+FMA)"
+    # the MoE layer (128 experts, top-8, 2048/768, 512 tokens) as the reference's bucket path runs it
+    # (Decoder::moe_ffn_batch, crates/frink-models/src/decoder/ffn_batch.rs:343-434): the oracle's scalar integer
+    # dots, experts over the threads; one pass (seconds)
+    E, K, H, F, T = 128, 8, 2048, 768, 512
+    from frink_amd import Q4_K, synth
+    gate, up, down = (random_blocks(Q4_K, r, c, seed=80 + j) for j, (r, c) in enumerate(((E * F, H), (E * F, H), (E * H, F))))
+    xm = synth.activations(7, T, H)
+    logits = synth.normal(8, T * E).reshape(T, E)
+    routed = [fo.route_top_k_softmax(l, K, True) for l in logits]
+    ids = np.stack([r[0] for r in routed]).astype(np.int32)
+    wts = np.stack([r[1] for r in routed])
+    t, n = best_of(lambda: fo.moe_ffn(Q4_K, gate, up, down, E, H, F, xm, ids, wts, threads), 6.0, 3)
+    legs["moe_layer_512_tokens_scalar_int_dot_ms"] = round(t * 1e3, 1)
+    legs["moe_layer_512_tokens_tokens_per_s"] = round(T / t, 1)
+    del gate, up, down
     out = {"value": round(headline, 2), "unit": "GB/s", "cores": threads, "kind": "port",
            "sample": "the whole workload (%dx%d Q4_K decode GEMV) as %s; legs: the same GEMV on the integer path "
-                     "(Q8_K quantization + AVX2 integer dot, and the scalar oracle), and the whole M=512 GEMM as "
-                     "AVX2 integer dots with the weight row outermost; %d OpenMP threads = physical cores"
+                     "(Q8_K quantization + AVX2 integer dot, and the scalar oracle), the whole M=512 GEMM and the M=8 batch as "
+                     "AVX2 integer dots with the weight row outermost, and one pass of the 128-expert MoE layer at 512 "
+                     "tokens on the scalar oracle; %d OpenMP threads = physical cores"
                      % (rows, cols, what, threads),
            "legs": legs, "gpu_vs_cpu_max_err_over_ninf": err}
     out.update(host)
@@ -204,7 +245,18 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--read-sweep", action="store_true", help="only: time of a read-only stream against its size")
+    ap.add_argument("--only", default="", help="comma-separated groups of secondary workloads to run (ceilings, gemv, gemm, "
+                    "moe, thin, qkv): a profiler run replays only the kernels it is about")
+    ap.add_argument("--graph-steps", type=int, default=GRAPH_STEPS, help="most steps captured in one HIP graph")
     args = ap.parse_args()
+    only = set(w for w in args.only.split(",") if w)
+
+    def want(group):
+        return not only or group in only
+    graph_cap = max(1, args.graph_steps)
+
+    def timed(fn, n, per_graph):
+        return time_graph(torch, fn, n, max(1, min(per_graph, graph_cap)))
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus,
               file=sys.stderr)
@@ -235,7 +287,7 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    wall, ev = time_graph(torch, step, args.steps, GRAPH_STEPS)
+    wall, ev = timed(step, args.steps, GRAPH_STEPS)
     sec_per_step = ev / args.steps
     wbytes = data.size
     value = wbytes / sec_per_step / 1e9
@@ -252,9 +304,10 @@ def main():
         ws[i % COPIES].gemv_q8k(acts, out=y)
 
     n_k = max(COPIES * 8, min(args.steps, 4000))
-    _, ev_k = time_graph(torch, gemv_only, n_k, GRAPH_STEPS)
+    _, ev_k = timed(gemv_only, n_k, GRAPH_STEPS)
     k_sec = ev_k / n_k
 
+    traffic_bytes, traffic_src = traffic_from_profile("gemv_q4_k_lines_kernel")
     out = {
         "metric": "Q4_K GEMV HBM GB/s", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 6),
@@ -264,12 +317,12 @@ def main():
                                "activation quantization + GEMV per step (one kernel), %d weight copies rotated "
                                "(cache-cold)" % COPIES,
                    "graph": "%d steps timed with HIP events as replays of a HIP graph of %d steps, behind one untimed "
-                            "replay with no synchronization between" % (args.steps, min(args.steps, GRAPH_STEPS)),
+                            "replay with no synchronization between" % (args.steps, min(args.steps, GRAPH_STEPS, graph_cap)),
                    "weight_bytes": int(wbytes), "device": info["name"], "arch": info["gcn_arch"],
                    "compute_units": info["compute_units"], "wall_ms_per_step": round(wall / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "gemv_q4_k_lines_kernel<16, 0, 8, false, 4, false>", "algorithmic_bytes": int(alg_bytes),
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_bytes, "traffic_source": traffic_src,
+                     "kernel": HEADLINE_KERNEL, "algorithmic_bytes": int(alg_bytes),
                      "avg_launch_us": round(sec_per_step * 1e6, 3), "launches": args.steps,
                      "prequantized_form": {"kernel": "gemv_q4_k_lines_kernel<16, 1, 8, false, 0, false>",
                                            "avg_launch_us": round(k_sec * 1e6, 3), "launches": n_k,
@@ -279,244 +332,251 @@ def main():
 
     if not args.no_extra:
         extra = {}
-        # practical ceilings at the same size: a read-only stream and a copy
-        src = [torch.empty(wbytes, dtype=torch.uint8, device=dev).random_() for _ in range(COPIES)]
-        dst = torch.empty(wbytes, dtype=torch.uint8, device=dev)
-        sink = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
-        L, C = fa.lib(), __import__("ctypes")
+        if want('ceilings'):
+            # practical ceilings at the same size: a read-only stream and a copy
+            src = [torch.empty(wbytes, dtype=torch.uint8, device=dev).random_() for _ in range(COPIES)]
+            dst = torch.empty(wbytes, dtype=torch.uint8, device=dev)
+            sink = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+            L, C = fa.lib(), __import__("ctypes")
 
-        def read_only(i):
-            fa.check(L.frk_hip_read_dev(C.c_void_p(src[i % COPIES].data_ptr()), wbytes, C.c_void_p(sink.data_ptr()),
-                                        fa._stream()))
+            def read_only(i):
+                fa.check(L.frk_hip_read_dev(C.c_void_p(src[i % COPIES].data_ptr()), wbytes, C.c_void_p(sink.data_ptr()),
+                                            fa._stream()))
 
-        def copy(i):
-            fa.check(L.frk_hip_copy_dev(C.c_void_p(src[i % COPIES].data_ptr()), C.c_void_p(dst.data_ptr()), wbytes,
-                                        fa._stream()))
-        _, t = time_graph(torch, read_only, 800, GRAPH_STEPS)
-        extra["read_only_stream_33MB_GBs"] = round(wbytes / (t / 800) / 1e9, 1)
-        _, t = time_graph(torch, copy, 800, GRAPH_STEPS)
-        extra["copy_33MB_read_plus_write_GBs"] = round(2 * wbytes / (t / 800) / 1e9, 1)
-        del src, dst
-        for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
-                                 ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
-                                 ("Q5_K GEMV 14336x4096 (one launch)", fa.Q5_K, 14336, 4096),
-                                 ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096),
-                                 ("Q4_K GEMV 4096x14336 (a Q4_K down projection)", fa.Q4_K, 4096, 14336),
-                                 ("Q4_K GEMV 4096x4096 (attention projection)", fa.Q4_K, 4096, 4096),
-                                 ("Q8_0 GEMV 4096x14336", fa.Q8_0, 4096, 14336)):
-            d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
-            n_copies = max(COPIES, -(-560_000_000 // d2.numel()))  # (past the 256 MB Infinity Cache, like the headline's copies)
-            w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]
-            x2 = torch.from_numpy(synth.activations(5, 1, c2)[0]).to(dev)
-            y2 = torch.empty(r2, dtype=torch.float32, device=dev)
+            def copy(i):
+                fa.check(L.frk_hip_copy_dev(C.c_void_p(src[i % COPIES].data_ptr()), C.c_void_p(dst.data_ptr()), wbytes,
+                                            fa._stream()))
+            _, t = timed(read_only, 800, GRAPH_STEPS)
+            extra["read_only_stream_33MB_GBs"] = round(wbytes / (t / 800) / 1e9, 1)
+            _, t = timed(copy, 800, GRAPH_STEPS)
+            extra["copy_33MB_read_plus_write_GBs"] = round(2 * wbytes / (t / 800) / 1e9, 1)
+            del src, dst
+        if want('gemv'):
+            for name, k2, r2, c2 in (("Q6_K GEMV 4096x14336 (FFN down)", fa.Q6_K, 4096, 14336),
+                                     ("Q8_0 GEMV 4096x4096", fa.Q8_0, 4096, 4096),
+                                     ("Q5_K GEMV 14336x4096 (one launch)", fa.Q5_K, 14336, 4096),
+                                     ("Q4_0 GEMV 14336x4096 (f32 dot)", fa.Q4_0, 14336, 4096),
+                                     ("Q4_K GEMV 4096x14336 (a Q4_K down projection)", fa.Q4_K, 4096, 14336),
+                                     ("Q4_K GEMV 4096x4096 (attention projection)", fa.Q4_K, 4096, 4096),
+                                     ("Q8_0 GEMV 4096x14336", fa.Q8_0, 4096, 14336)):
+                d2 = torch.from_numpy(random_blocks(k2, r2, c2, seed=77)).to(dev)
+                n_copies = max(COPIES, -(-560_000_000 // d2.numel()))  # (past the 256 MB Infinity Cache, like the headline's copies)
+                w2 = [fa.Weights.from_device(k2, d2, r2, c2) for _ in range(n_copies)]
+                x2 = torch.from_numpy(synth.activations(5, 1, c2)[0]).to(dev)
+                y2 = torch.empty(r2, dtype=torch.float32, device=dev)
 
-            def step2(i):
-                w2[i % n_copies].gemv(x2, out=y2)
-            _, t = time_graph(torch, step2, 1600, 25 * n_copies)
-            extra[name] = {"GBs": round(d2.numel() / (t / 1600) / 1e9, 1), "us_per_step": round(t / 1600 * 1e6, 3),
-                           "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
-            for w in w2:
+                def step2(i):
+                    w2[i % n_copies].gemv(x2, out=y2)
+                _, t = timed(step2, 1600, 25 * n_copies)
+                extra[name] = {"GBs": round(d2.numel() / (t / 1600) / 1e9, 1), "us_per_step": round(t / 1600 * 1e6, 3),
+                               "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
+                for w in w2:
+                    w.release()
+        if want('gemm'):
+            # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step.  The step is
+            # the activations' quantization + the GEMM kernel; the kernel alone is timed over activations
+            # quantized beforehand (frk_hip_gemm_acts_dev: a graph of nothing but that kernel, HIP events).
+            xb = torch.from_numpy(synth.activations(6, 512, cols, outlier_frac=0.01)).to(dev)
+            acts512 = fa.BatchActs(512, cols).quantize(xb)
+            gemm_records = []
+            for name, r2, kname in (("Q4_K GEMM M=512 4096x4096", 4096, "gemm_q4_k_pipe_kernel<4, 2, 2>"),
+                                    ("Q4_K GEMM M=512 14336x4096", 14336, "gemm_q4_k_pipe_kernel<8, 1, 4>")):
+                d2 = torch.from_numpy(random_blocks(kind, r2, cols, seed=78)).to(dev)
+                w2 = [fa.Weights.from_device(kind, d2, r2, cols) for _ in range(8)]
+                yb = torch.empty((512, r2), dtype=torch.float32, device=dev)
+
+                def step3(i):
+                    w2[i % 8].gemm(xb, out=yb)
+
+                def step3p(i):
+                    w2[i % 8].gemm_acts(acts512, out=yb)
+                _, t = timed(step3, 200, 100)
+                _, tp = timed(step3p, 200, 100)
+                ops = 2.0 * 512 * r2 * cols
+                tops = ops / (t / 200) / 1e12
+                k_us = tp / 200 * 1e6
+                extra[name] = {"TOPS": round(tops, 1), "us_per_step": round(t / 200 * 1e6, 2),
+                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+                gemm_records.append({"bound": "mfma", "workload": name, "kernel": kname, "achieved": round(ops / k_us / 1e6, 1),
+                                     "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops / k_us / 1e6 / INT8_PEAK_TOPS, 4),
+                                     "ops": ops, "avg_launch_us": round(k_us, 2), "launches": 200,
+                                     "how": "HIP events around graphs of this kernel alone, over activations quantized beforehand",
+                                     "step_us_with_quantization": round(t / 200 * 1e6, 2)})
+                for w in w2:
+                    w.release()
+            out["roofline_gemm"] = gemm_records
+            acts512.release()
+            # Q5_K at M=512: the tiled matrix-core kernel with the fifth bits as a third int8 plane
+            d5g = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=84)).to(dev)
+            w5 = [fa.Weights.from_device(fa.Q5_K, d5g, rows, cols) for _ in range(4)]
+            yb5 = torch.empty((512, rows), dtype=torch.float32, device=dev)
+
+            def step3e(i):
+                w5[i % 4].gemm(xb, out=yb5)
+            _, t = timed(step3e, 40, 20)
+            tops = 2.0 * 512 * rows * cols / (t / 40) / 1e12
+            extra["Q5_K GEMM M=512 14336x4096 (three int8 planes)"] = {
+                "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            for w in w5:
                 w.release()
-        # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step.  The step is
-        # the activations' quantization + the GEMM kernel; the kernel alone is what a second matrix over
-        # the same quantized activations adds (frk_hip_gemm_pair_dev: one quantization, two GEMM launches).
-        xb = torch.from_numpy(synth.activations(6, 512, cols, outlier_frac=0.01)).to(dev)
-        gemm_records = []
-        for name, r2, kname in (("Q4_K GEMM M=512 4096x4096", 4096, "gemm_q4_k_pipe_kernel<4, 2, 2>"),
-                                ("Q4_K GEMM M=512 14336x4096", 14336, "gemm_q4_k_pipe_kernel<8, 1, 4>")):
-            d2 = torch.from_numpy(random_blocks(kind, r2, cols, seed=78)).to(dev)
-            w2 = [fa.Weights.from_device(kind, d2, r2, cols) for _ in range(8)]
-            yb = torch.empty((512, r2), dtype=torch.float32, device=dev)
-            yb2 = torch.empty((512, r2), dtype=torch.float32, device=dev)
+            del d5g, yb5
+            # the FFN down projection of a Q4_K_M model at M=512: Q6_K on the matrix cores
+            d6g = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=78)).to(dev)
+            w6 = [fa.Weights.from_device(fa.Q6_K, d6g, cols, rows) for _ in range(4)]
+            xb6 = torch.from_numpy(synth.activations(6, 512, rows)).to(dev)
+            yb6 = torch.empty((512, cols), dtype=torch.float32, device=dev)
 
-            def step3(i):
-                w2[i % 8].gemm(xb, out=yb)
-
-            def step3p(i):
-                fa.gemm_pair(w2[(2 * i) % 8], w2[(2 * i + 1) % 8], xb, outs=(yb, yb2))
-            _, t = time_graph(torch, step3, 200, 100)
-            _, tp = time_graph(torch, step3p, 200, 100)
-            ops = 2.0 * 512 * r2 * cols
-            tops = ops / (t / 200) / 1e12
-            k_us = (tp - t) / 200 * 1e6
-            extra[name] = {"TOPS": round(tops, 1), "us_per_step": round(t / 200 * 1e6, 2),
-                           "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-            gemm_records.append({"bound": "mfma", "workload": name, "kernel": kname, "achieved": round(ops / k_us / 1e6, 1),
-                                 "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(ops / k_us / 1e6 / INT8_PEAK_TOPS, 4),
-                                 "ops": ops, "avg_launch_us": round(k_us, 2), "launches": 200,
-                                 "how": "pair step (one quantization + two GEMM launches) minus single step, HIP events",
-                                 "step_us_with_quantization": round(t / 200 * 1e6, 2)})
-            for w in w2:
+            def step3b(i):
+                w6[i % 4].gemm(xb6, out=yb6)
+            _, t = timed(step3b, 100, 50)
+            tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+            extra["Q6_K GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                                   "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            for w in w6:
                 w.release()
-        out["roofline_gemm"] = gemm_records
-        # Q5_K at M=512: the tiled matrix-core kernel with the fifth bits as a third int8 plane
-        d5g = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=84)).to(dev)
-        w5 = [fa.Weights.from_device(fa.Q5_K, d5g, rows, cols) for _ in range(4)]
-        yb5 = torch.empty((512, rows), dtype=torch.float32, device=dev)
+            # the shape the reference quotes its int8 Q8_0 GEMM on (crates/frink-cuda/src/mmq/kernel.rs:30-36)
+            d8g = torch.from_numpy(random_blocks(fa.Q8_0, cols, rows, seed=79)).to(dev)
+            w8 = [fa.Weights.from_device(fa.Q8_0, d8g, cols, rows) for _ in range(4)]
 
-        def step3e(i):
-            w5[i % 4].gemm(xb, out=yb5)
-        _, t = time_graph(torch, step3e, 40, 20)
-        tops = 2.0 * 512 * rows * cols / (t / 40) / 1e12
-        extra["Q5_K GEMM M=512 14336x4096 (three int8 planes)"] = {
-            "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-        for w in w5:
-            w.release()
-        del d5g, yb5
-        # the FFN down projection of a Q4_K_M model at M=512: Q6_K on the matrix cores
-        d6g = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=78)).to(dev)
-        w6 = [fa.Weights.from_device(fa.Q6_K, d6g, cols, rows) for _ in range(4)]
-        xb6 = torch.from_numpy(synth.activations(6, 512, rows)).to(dev)
-        yb6 = torch.empty((512, cols), dtype=torch.float32, device=dev)
-
-        def step3b(i):
-            w6[i % 4].gemm(xb6, out=yb6)
-        _, t = time_graph(torch, step3b, 100, 50)
-        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
-        extra["Q6_K GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
-                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-        for w in w6:
-            w.release()
-        # the shape the reference quotes its int8 Q8_0 GEMM on (crates/frink-cuda/src/mmq/kernel.rs:30-36)
-        d8g = torch.from_numpy(random_blocks(fa.Q8_0, cols, rows, seed=79)).to(dev)
-        w8 = [fa.Weights.from_device(fa.Q8_0, d8g, cols, rows) for _ in range(4)]
-
-        def step3c(i):
-            w8[i % 4].gemm(xb6, out=yb6)
-        _, t = time_graph(torch, step3c, 100, 50)
-        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
-        extra["Q8_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
-                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-        for w in w8:
-            w.release()
-        # the same kernel on Q4_0 weights (nibbles turned into signed bytes while they are staged)
-        d40 = torch.from_numpy(random_blocks(fa.Q4_0, cols, rows, seed=81)).to(dev)
-        w40 = [fa.Weights.from_device(fa.Q4_0, d40, cols, rows) for _ in range(4)]
-
-        def step3d(i):
-            w40[i % 4].gemm(xb6, out=yb6)
-        _, t = time_graph(torch, step3d, 100, 50)
-        tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
-        extra["Q4_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
-                                               "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
-        for w in w40:
-            w.release()
-        # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
-        E, K, H, F, T = 128, 8, 2048, 768, 512
-        experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)
-                   for j, (r, c) in enumerate(((E * F, H), (E * F, H), (E * H, F)))]
-        xm = torch.from_numpy(synth.activations(7, T, H)).to(dev)
-        logits = torch.from_numpy(synth.normal(8, T * E).reshape(T, E)).to(dev)
-        ids, wts = fa.route_top_k_softmax(logits, K, True)
-        ym = torch.empty((T, H), dtype=torch.float32, device=dev)
-
-        def step4(i):
-            fa.moe_ffn(experts[0], experts[1], experts[2], E, xm, ids, wts, out=ym)
-        _, t = time_graph(torch, step4, 100, 50)
-        moe_bytes = 3 * E * F * H // 256 * 144 + 2 * T * H * 4 + 2 * T * K * 4
-        extra["MoE layer 128x top-8, 2048/768, 512 tokens"] = {
-            "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
-            "algorithmic_GBs": round(moe_bytes / (t / 100) / 1e9, 1),
-            "frac_of_hbm_peak": round(moe_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4),
-            "TOPS": round(2.0 * T * K * 3 * F * H / (t / 100) / 1e12, 1)}
-        # the same layer for ONE token (decode): 16 routings in turn that between them visit all 128
-        # experts once, so that no expert's weights are still cached when its turn comes again
-        perm = np.random.default_rng(11).permutation(E).astype(np.int32).reshape(16, 1, K)
-        ids1 = [torch.from_numpy(np.ascontiguousarray(p)).to(dev) for p in perm]
-        w1 = torch.full((1, K), 1.0 / K, dtype=torch.float32, device=dev)
-        x1 = xm[:1].contiguous()
-        y1 = torch.empty((1, H), dtype=torch.float32, device=dev)
-
-        def step4b(i):
-            fa.moe_ffn(experts[0], experts[1], experts[2], E, x1, ids1[i % 16], w1, out=y1)
-        _, t = time_graph(torch, step4b, 800, 400)
-        tok_bytes = K * 3 * F * H // 256 * 144
-        extra["MoE layer 128x top-8, 2048/768, 1 token (decode)"] = {
-            "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok_bytes / (t / 800) / 1e9, 1),
-            "frac_of_hbm_peak": round(tok_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
-        # the same layer with its down experts in Q6_K (a Q4_K_M file keeps some layers' that way), 512 tokens and 1
-        down6 = fa.Weights.from_device(fa.Q6_K, torch.from_numpy(random_blocks(fa.Q6_K, E * H, F, seed=83)).to(dev), E * H, F)
-
-        def step4c(i):
-            fa.moe_ffn(experts[0], experts[1], down6, E, xm, ids, wts, out=ym)
-        _, t = time_graph(torch, step4c, 100, 50)
-        moe6_bytes = E * F * H // 256 * (2 * 144 + 210) + 2 * T * H * 4 + 2 * T * K * 4
-        extra["MoE layer 128x top-8, 2048/768, 512 tokens, down experts Q6_K"] = {
-            "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
-            "algorithmic_GBs": round(moe6_bytes / (t / 100) / 1e9, 1),
-            "frac_of_hbm_peak": round(moe6_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4)}
-
-        def step4d(i):
-            fa.moe_ffn(experts[0], experts[1], down6, E, x1, ids1[i % 16], w1, out=y1)
-        _, t = time_graph(torch, step4d, 800, 400)
-        tok6_bytes = K * F * H // 256 * (2 * 144 + 210)
-        extra["MoE layer 128x top-8, 2048/768, 1 token (decode), down experts Q6_K"] = {
-            "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok6_bytes / (t / 800) / 1e9, 1),
-            "frac_of_hbm_peak": round(tok6_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
-        down6.release()
-        for w in experts:
-            w.release()
-        # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call
-        # (gate and up share one quantized activation, SwiGLU, down)
-        g8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
-        u8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
-        d6 = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=79)).to(dev)
-        dn = [fa.Weights.from_device(fa.Q6_K, d6, cols, rows) for _ in range(8)]
-        x8 = torch.from_numpy(synth.activations(9, 8, cols)).to(dev)
-        h8 = torch.from_numpy(synth.activations(10, 8, rows)).to(dev)
-        y8 = torch.empty((8, rows), dtype=torch.float32, device=dev)
-        z8 = torch.empty((8, cols), dtype=torch.float32, device=dev)
-        d5 = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=80)).to(dev)
-        q5 = [fa.Weights.from_device(fa.Q5_K, d5, rows, cols) for _ in range(8)]
-        for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096", g8, x8, y8),
-                                      ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8),
-                                      ("Q5_K thin GEMM M=8 14336x4096", q5, x8, y8)):
-            def step5(i, mats=mats, xin=xin, yout=yout):
-                mats[i % 8].gemm(xin, out=yout)
-            _, t = time_graph(torch, step5, 400, 200)
-            wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
-            extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
-                           "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
-        # the same M=8 batches from activations quantized beforehand (by the kernel that produced them, or
-        # shared with another projection): the multiplying launch alone
-        for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096, activations quantized beforehand", g8, x8, y8),
-                                      ("Q6_K thin GEMM M=8 4096x14336, activations quantized beforehand", dn, h8, z8)):
-            acts8 = fa.quantize_q8_k(xin)
-
-            def step5q(i, mats=mats, acts8=acts8, yout=yout):
-                mats[i % 8].gemm_q8k(acts8, 8, out=yout)
-            _, t = time_graph(torch, step5q, 400, 200)
-            wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
-            extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
-                           "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
-        yf = torch.empty(cols, dtype=torch.float32, device=dev)
-
-        def step6(i):
-            fa.ffn_swiglu(g8[i % 8], u8[i % 8], dn[i % 8], xd, out=yf)
-        _, t = time_graph(torch, step6, 400, 200)
-        fb = 2 * wbytes + d6.numel()
-        extra["decode FFN 4096->14336->4096 (gate, up Q4_K; down Q6_K)"] = {
-            "us_per_step": round(t / 400 * 1e6, 2), "GBs": round(fb / (t / 400) / 1e9, 1),
-            "frac_of_hbm_peak": round(fb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
-        for w in g8 + u8 + dn + q5:
-            w.release()
-        # q/k/v of a Llama-3-8B layer (4096, 1024 and 1024 rows of 4096): one launch for the three;
-        # 40 sets of weights in turn (566 MB > the 256 MB Infinity Cache)
-        qkv_rows = (4096, 1024, 1024)
-        qkv_dev = [torch.from_numpy(random_blocks(kind, r, cols, seed=90 + j)).to(dev) for j, r in enumerate(qkv_rows)]
-        qkv_sets = [[fa.Weights.from_device(kind, d.clone(), r, cols) for d, r in zip(qkv_dev, qkv_rows)] for _ in range(40)]
-        qkv_out = [torch.empty(r, dtype=torch.float32, device=dev) for r in qkv_rows]
-
-        def step7(i):
-            fa.gemv_multi(qkv_sets[i % 40], xd, outs=qkv_out)
-        _, t = time_graph(torch, step7, 800, 400)
-        qb = sum(qkv_rows) * (cols // 256) * 144
-        extra["Q4_K q/k/v multi-GEMV (4096+1024+1024)x4096, one launch"] = {
-            "us_per_step": round(t / 800 * 1e6, 2), "GBs": round(qb / (t / 800) / 1e9, 1),
-            "frac_of_hbm_peak": round(qb / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
-        for ws_ in qkv_sets:
-            for w in ws_:
+            def step3c(i):
+                w8[i % 4].gemm(xb6, out=yb6)
+            _, t = timed(step3c, 100, 50)
+            tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+            extra["Q8_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                                   "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            for w in w8:
                 w.release()
+            # the same kernel on Q4_0 weights (nibbles turned into signed bytes while they are staged)
+            d40 = torch.from_numpy(random_blocks(fa.Q4_0, cols, rows, seed=81)).to(dev)
+            w40 = [fa.Weights.from_device(fa.Q4_0, d40, cols, rows) for _ in range(4)]
+
+            def step3d(i):
+                w40[i % 4].gemm(xb6, out=yb6)
+            _, t = timed(step3d, 100, 50)
+            tops = 2.0 * 512 * rows * cols / (t / 100) / 1e12
+            extra["Q4_0 GEMM M=512 4096x14336"] = {"TOPS": round(tops, 1), "us_per_step": round(t / 100 * 1e6, 2),
+                                                   "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+            for w in w40:
+                w.release()
+        if want('moe'):
+            # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
+            E, K, H, F, T = 128, 8, 2048, 768, 512
+            experts = [fa.Weights.from_device(kind, torch.from_numpy(random_blocks(kind, r, c, seed=80 + j)).to(dev), r, c)
+                       for j, (r, c) in enumerate(((E * F, H), (E * F, H), (E * H, F)))]
+            xm = torch.from_numpy(synth.activations(7, T, H)).to(dev)
+            logits = torch.from_numpy(synth.normal(8, T * E).reshape(T, E)).to(dev)
+            ids, wts = fa.route_top_k_softmax(logits, K, True)
+            ym = torch.empty((T, H), dtype=torch.float32, device=dev)
+
+            def step4(i):
+                fa.moe_ffn(experts[0], experts[1], experts[2], E, xm, ids, wts, out=ym)
+            _, t = timed(step4, 100, 50)
+            moe_bytes = 3 * E * F * H // 256 * 144 + 2 * T * H * 4 + 2 * T * K * 4
+            extra["MoE layer 128x top-8, 2048/768, 512 tokens"] = {
+                "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
+                "algorithmic_GBs": round(moe_bytes / (t / 100) / 1e9, 1),
+                "frac_of_hbm_peak": round(moe_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4),
+                "TOPS": round(2.0 * T * K * 3 * F * H / (t / 100) / 1e12, 1)}
+            # the same layer for ONE token (decode): 16 routings in turn that between them visit all 128
+            # experts once, so that no expert's weights are still cached when its turn comes again
+            perm = np.random.default_rng(11).permutation(E).astype(np.int32).reshape(16, 1, K)
+            ids1 = [torch.from_numpy(np.ascontiguousarray(p)).to(dev) for p in perm]
+            w1 = torch.full((1, K), 1.0 / K, dtype=torch.float32, device=dev)
+            x1 = xm[:1].contiguous()
+            y1 = torch.empty((1, H), dtype=torch.float32, device=dev)
+
+            def step4b(i):
+                fa.moe_ffn(experts[0], experts[1], experts[2], E, x1, ids1[i % 16], w1, out=y1)
+            _, t = timed(step4b, 800, 400)
+            tok_bytes = K * 3 * F * H // 256 * 144
+            extra["MoE layer 128x top-8, 2048/768, 1 token (decode)"] = {
+                "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok_bytes / (t / 800) / 1e9, 1),
+                "frac_of_hbm_peak": round(tok_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+            # the same layer with its down experts in Q6_K (a Q4_K_M file keeps some layers' that way), 512 tokens and 1
+            down6 = fa.Weights.from_device(fa.Q6_K, torch.from_numpy(random_blocks(fa.Q6_K, E * H, F, seed=83)).to(dev), E * H, F)
+
+            def step4c(i):
+                fa.moe_ffn(experts[0], experts[1], down6, E, xm, ids, wts, out=ym)
+            _, t = timed(step4c, 100, 50)
+            moe6_bytes = E * F * H // 256 * (2 * 144 + 210) + 2 * T * H * 4 + 2 * T * K * 4
+            extra["MoE layer 128x top-8, 2048/768, 512 tokens, down experts Q6_K"] = {
+                "us_per_step": round(t / 100 * 1e6, 2), "tokens_per_s": round(T / (t / 100), 0),
+                "algorithmic_GBs": round(moe6_bytes / (t / 100) / 1e9, 1),
+                "frac_of_hbm_peak": round(moe6_bytes / (t / 100) / 1e9 / HBM_PEAK_GBS, 4)}
+
+            def step4d(i):
+                fa.moe_ffn(experts[0], experts[1], down6, E, x1, ids1[i % 16], w1, out=y1)
+            _, t = timed(step4d, 800, 400)
+            tok6_bytes = K * F * H // 256 * (2 * 144 + 210)
+            extra["MoE layer 128x top-8, 2048/768, 1 token (decode), down experts Q6_K"] = {
+                "us_per_step": round(t / 800 * 1e6, 2), "algorithmic_GBs": round(tok6_bytes / (t / 800) / 1e9, 1),
+                "frac_of_hbm_peak": round(tok6_bytes / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+            down6.release()
+            for w in experts:
+                w.release()
+        if want('thin'):
+            # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call
+            # (gate and up share one quantized activation, SwiGLU, down)
+            g8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
+            u8 = [fa.Weights.from_device(kind, data_dev, rows, cols) for _ in range(8)]
+            d6 = torch.from_numpy(random_blocks(fa.Q6_K, cols, rows, seed=79)).to(dev)
+            dn = [fa.Weights.from_device(fa.Q6_K, d6, cols, rows) for _ in range(8)]
+            x8 = torch.from_numpy(synth.activations(9, 8, cols)).to(dev)
+            h8 = torch.from_numpy(synth.activations(10, 8, rows)).to(dev)
+            y8 = torch.empty((8, rows), dtype=torch.float32, device=dev)
+            z8 = torch.empty((8, cols), dtype=torch.float32, device=dev)
+            d5 = torch.from_numpy(random_blocks(fa.Q5_K, rows, cols, seed=80)).to(dev)
+            q5 = [fa.Weights.from_device(fa.Q5_K, d5, rows, cols) for _ in range(8)]
+            for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096", g8, x8, y8),
+                                          ("Q6_K thin GEMM M=8 4096x14336", dn, h8, z8),
+                                          ("Q5_K thin GEMM M=8 14336x4096", q5, x8, y8)):
+                def step5(i, mats=mats, xin=xin, yout=yout):
+                    mats[i % 8].gemm(xin, out=yout)
+                _, t = timed(step5, 400, 200)
+                wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
+                extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
+                               "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+            # the same M=8 batches from activations quantized beforehand (by the kernel that produced them, or
+            # shared with another projection): the multiplying launch alone
+            for name, mats, xin, yout in (("Q4_K thin GEMM M=8 14336x4096, activations quantized beforehand", g8, x8, y8),
+                                          ("Q6_K thin GEMM M=8 4096x14336, activations quantized beforehand", dn, h8, z8)):
+                acts8 = fa.quantize_q8_k(xin)
+
+                def step5q(i, mats=mats, acts8=acts8, yout=yout):
+                    mats[i % 8].gemm_q8k(acts8, 8, out=yout)
+                _, t = timed(step5q, 400, 200)
+                wb = mats[0].rows * (mats[0].cols // 256) * fa.BLOCK[mats[0].kind][0]
+                extra[name] = {"us_per_step": round(t / 400 * 1e6, 2), "GBs": round(wb / (t / 400) / 1e9, 1),
+                               "frac_of_hbm_peak": round(wb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+            yf = torch.empty(cols, dtype=torch.float32, device=dev)
+
+            def step6(i):
+                fa.ffn_swiglu(g8[i % 8], u8[i % 8], dn[i % 8], xd, out=yf)
+            _, t = timed(step6, 400, 200)
+            fb = 2 * wbytes + d6.numel()
+            extra["decode FFN 4096->14336->4096 (gate, up Q4_K; down Q6_K)"] = {
+                "us_per_step": round(t / 400 * 1e6, 2), "GBs": round(fb / (t / 400) / 1e9, 1),
+                "frac_of_hbm_peak": round(fb / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
+            for w in g8 + u8 + dn + q5:
+                w.release()
+        if want('qkv'):
+            # q/k/v of a Llama-3-8B layer (4096, 1024 and 1024 rows of 4096): one launch for the three;
+            # 40 sets of weights in turn (566 MB > the 256 MB Infinity Cache)
+            qkv_rows = (4096, 1024, 1024)
+            qkv_dev = [torch.from_numpy(random_blocks(kind, r, cols, seed=90 + j)).to(dev) for j, r in enumerate(qkv_rows)]
+            qkv_sets = [[fa.Weights.from_device(kind, d.clone(), r, cols) for d, r in zip(qkv_dev, qkv_rows)] for _ in range(40)]
+            qkv_out = [torch.empty(r, dtype=torch.float32, device=dev) for r in qkv_rows]
+
+            def step7(i):
+                fa.gemv_multi(qkv_sets[i % 40], xd, outs=qkv_out)
+            _, t = timed(step7, 800, 400)
+            qb = sum(qkv_rows) * (cols // 256) * 144
+            extra["Q4_K q/k/v multi-GEMV (4096+1024+1024)x4096, one launch"] = {
+                "us_per_step": round(t / 800 * 1e6, 2), "GBs": round(qb / (t / 800) / 1e9, 1),
+                "frac_of_hbm_peak": round(qb / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+            for ws_ in qkv_sets:
+                for w in ws_:
+                    w.release()
         out["extra"] = extra
 
     if not args.no_cpu:

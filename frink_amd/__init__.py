@@ -30,7 +30,8 @@ EXPORTS = [
     "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
     "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
-    "frk_hip_gemm_dev", "frk_hip_gemm_q8k_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
+    "frk_hip_gemm_dev", "frk_hip_gemm_q8k_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev",
+    "frk_hip_batch_acts_create", "frk_hip_batch_acts_release", "frk_hip_quantize_batch_acts_dev", "frk_hip_gemm_acts_dev", "frk_hip_route_top_k_softmax_dev", "frk_hip_moe_ffn_dev",
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
@@ -92,6 +93,10 @@ def lib():
             "frk_hip_gemm_q8k_dev": (i, [vp, vp, vp, vp, sz, vp, vp]),
             "frk_hip_gemm_noalloc_dev": (i, [vp, vp, sz, vp, vp]),
             "frk_hip_gemm_pair_dev": (i, [vp, vp, vp, sz, vp, vp, vp]),
+            "frk_hip_batch_acts_create": (i, [sz, sz, C.POINTER(vp)]),
+            "frk_hip_batch_acts_release": (i, [vp]),
+            "frk_hip_quantize_batch_acts_dev": (i, [vp, vp, sz, vp]),
+            "frk_hip_gemm_acts_dev": (i, [vp, vp, vp, vp]),
             "frk_hip_route_top_k_softmax_dev": (i, [vp, sz, sz, sz, i, vp, vp, vp]),
             "frk_hip_moe_ffn_dev": (i, [vp, vp, vp, sz, vp, sz, vp, vp, sz, vp, vp]),
             "frk_hip_moe_intermediates_dev": (i, [sz, sz, sz, sz, sz, vp, vp, vp, vp, vp, vp]),
@@ -216,6 +221,13 @@ class Weights:
                                      _stream()))
         return y
 
+    def gemm_acts(self, acts, out=None):
+        """apply_batch_with_acts: this matrix over a batch that a BatchActs holds quantized."""
+        import torch
+        y = out if out is not None else torch.empty((acts.batch, self.rows), dtype=torch.float32, device="cuda")
+        check(lib().frk_hip_gemm_acts_dev(self.handle, acts.handle, C.c_void_p(y.data_ptr()), _stream()))
+        return y
+
     def gemm_noalloc(self, x, out):
         """frk_hip_gemm_noalloc_dev: the caller brings the output; the call allocates nothing."""
         import torch
@@ -231,6 +243,29 @@ class Weights:
         out = torch.empty((self.rows, self.cols), dtype=torch.float32, device="cuda")
         check(lib().frk_hip_dequant_dev(self.handle, C.c_void_p(out.data_ptr()), _stream()))
         return out
+
+
+class BatchActs:
+    """A batch's activations quantized once for any number of matrices (the reference's BatchActs::Q8K):
+    frk_hip_batch_acts_create / frk_hip_quantize_batch_acts_dev / frk_hip_batch_acts_release."""
+
+    def __init__(self, max_batch, cols):
+        h = C.c_void_p()
+        check(lib().frk_hip_batch_acts_create(max_batch, cols, C.byref(h)))
+        self.handle, self.max_batch, self.cols, self.batch = h, max_batch, cols, 0
+
+    def quantize(self, x):
+        import torch
+        assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.shape[-1] == self.cols
+        batch = x.numel() // self.cols
+        check(lib().frk_hip_quantize_batch_acts_dev(self.handle, C.c_void_p(x.data_ptr()), batch, _stream()))
+        self.batch = batch
+        return self
+
+    def release(self):
+        if self.handle:
+            check(lib().frk_hip_batch_acts_release(self.handle))
+            self.handle = None
 
 
 def _get_rows_dev(self, ids):

@@ -219,6 +219,25 @@ int frk_hip_gemm_q8k_dev(const frk_weights *w, const int8_t *q_dev, const float 
 int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const float *x_dev, size_t batch,
                           float *y0_dev, float *y1_dev, void *stream);
 
+/* A batch's activations quantized ONCE and multiplied by any number of matrices at ANY batch size:
+ * WeightMatrix::quantize_batch_acts -> BatchActs::Q8K -> apply_batch_with_acts / apply_batch_pair_with_acts
+ * (crates/frink-core/src/weight_matrix.rs:2348-2426, 757-768, 2481-2487, 2447-2479): the q/k/v triple or
+ * gate and up of a prefill, or activations a caller keeps.  The object owns its device memory
+ * (frk_hip_batch_acts_create allocates for up to max_batch rows of cols columns, _release frees; neither
+ * belongs in a hot loop) and holds the batch in whichever form the kernels of that batch size read: plain
+ * Q8_K rows (the decode and thin kernels), the tiled form of the matrix-core GEMMs, or both.
+ * frk_hip_quantize_batch_acts_dev and frk_hip_gemm_acts_dev allocate nothing themselves (a GEMM whose
+ * blocks are split between workgroups takes room for the parts from the stream's scratch buffer, like
+ * frk_hip_gemm_dev); y is bit for bit frk_hip_gemm_dev's.  K-quant matrices (Q4_K, Q5_K, Q6_K) of `cols`
+ * columns; other kinds return FRK_ERR_UNSUPPORTED.  A quantization and the GEMMs that read it are ordered
+ * by the stream they are enqueued on; the object is not to be re-quantized while a GEMM that reads it is
+ * still in flight on another stream. */
+typedef struct frk_batch_acts frk_batch_acts;
+int frk_hip_batch_acts_create(size_t max_batch, size_t cols, frk_batch_acts **out);
+int frk_hip_batch_acts_release(frk_batch_acts *acts);
+int frk_hip_quantize_batch_acts_dev(frk_batch_acts *acts, const float *x_dev, size_t batch, void *stream);
+int frk_hip_gemm_acts_dev(const frk_weights *w, const frk_batch_acts *acts, float *y_dev, void *stream);
+
 /* frk_hip_gemm_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments, same
  * kernels and bit for bit the same y, but the scratch memory (quantized activations, the parts of a

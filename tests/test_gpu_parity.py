@@ -1532,3 +1532,54 @@ def test_a_captured_graph_survives_a_larger_call_on_its_stream(fa):
     assert_rows_close(eager.cpu().numpy(), want, "gemm under a graph")
     w.release()
     big.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols", [(fo.Q4_K, 384, 1024), (fo.Q6_K, 264, 2048), (fo.Q5_K, 200, 1024)])
+def test_batch_acts_quantized_once_feed_any_batch(fa, kind, rows, cols):
+    """quantize_batch_acts -> BatchActs::Q8K -> apply_batch_with_acts (weight_matrix.rs:2348-2426, 757-768,
+    2481-2487): one quantization of a batch multiplied by several matrices, at every batch size -- one row, the
+    thin kernels' batches, the batches where both forms are held, and the wide matrix-core batches.  Each result
+    bit for bit frk_hip_gemm_dev's and within the tolerance of the oracle."""
+    from frink_amd import synth
+    data = make_weights(kind, rows, cols, seed=1400 + kind)
+    data2 = make_weights(fo.Q4_K, 136, cols, seed=1410 + kind)
+    w, w2 = fa.Weights.from_host(kind, data, rows, cols), fa.Weights.from_host(fo.Q4_K, data2, 136, cols)
+    acts = fa.BatchActs(300, cols)
+    for batch in (1, 2, 8, 16, 17, 25, 33, 64, 65, 130, 300):
+        x = synth.activations(1420 + batch, batch, cols, outlier_frac=0.01)
+        xd = to_dev(x)
+        acts.quantize(xd)
+        for ww, dd, rr, kk in ((w, data, rows, kind), (w2, data2, 136, fo.Q4_K)):
+            got = ww.gemm_acts(acts).cpu().numpy()
+            ref = ww.gemm(xd).cpu().numpy()
+            assert np.array_equal(bits(got), bits(ref)), (batch, kk)
+            assert_rows_close(got, fo.gemm(kk, dd, rr, cols, x), "gemm_acts kind %d batch %d" % (kk, batch))
+    with pytest.raises(fa.BackendError) as e:
+        acts.quantize(to_dev(np.zeros((301, cols), np.float32)))
+    assert e.value.code == fa.ERR_SHAPE
+    w8 = fa.Weights.from_host(fo.Q8_0, make_weights(fo.Q8_0, 40, cols, seed=3), 40, cols)
+    acts.quantize(to_dev(np.zeros((4, cols), np.float32)))
+    with pytest.raises(fa.BackendError) as e:
+        w8.gemm_acts(acts)
+    assert e.value.code == fa.ERR_UNSUPPORTED
+    other = fa.Weights.from_host(fo.Q4_K, make_weights(fo.Q4_K, 40, 2 * cols, seed=4), 40, 2 * cols)
+    with pytest.raises(fa.BackendError) as e:
+        other.gemm_acts(acts)
+    assert e.value.code == fa.ERR_SHAPE
+    acts.release()
+    for h in (w, w2, w8, other):
+        h.release()
+
+
+def test_batch_acts_at_the_prefill_shape(fa):
+    """M=512 over 4096 x 4096 Q4_K: the GEMM over held activations equals frk_hip_gemm_dev bit for bit (the kernel
+    bench.py times on its own through this entry point)."""
+    from bench import random_blocks
+    from frink_amd import synth
+    rows = cols = 4096
+    w = fa.Weights.from_host(fo.Q4_K, random_blocks(fo.Q4_K, rows, cols, 9), rows, cols)
+    xd = to_dev(synth.activations(1500, 512, cols, outlier_frac=0.01))
+    acts = fa.BatchActs(512, cols).quantize(xd)
+    assert np.array_equal(bits(w.gemm_acts(acts).cpu().numpy()), bits(w.gemm(xd).cpu().numpy()))
+    acts.release()
+    w.release()
