@@ -532,17 +532,144 @@ __device__ __forceinline__ void tail_piece(int i, TileTail &E, const BPlanes &B,
     }
 }
 
+// Up to four pieces of 1 KB that lie 1 KB apart in LDS and whose lane offsets already carry the matching
+// distance in global memory: a request's instruction offset moves BOTH of its addresses (checked on the
+// device), so one write of M0 serves the four.  `lds_uniform` and `base_uniform` must be scalar values.
+template <int N>
+__device__ __forceinline__ void dma16_run(uint32_t lds_uniform, const void *base_uniform, uint32_t o0, uint32_t o1, uint32_t o2,
+                                          uint32_t o3) {
+    static_assert(N >= 1 && N <= 4, "the instruction offset reaches 3072");
+    if (N == 4)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                     "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
+                     :
+                     : "s"(lds_uniform), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(base_uniform)
+                     : "memory");
+    else if (N == 2)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024"
+                     :
+                     : "s"(lds_uniform), "v"(o0), "v"(o1), "s"(base_uniform)
+                     : "memory");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_uniform), "v"(o0), "s"(base_uniform) : "memory");
+}
+
+// The block's scales as the packed multiply wants them: for sub-block j one register with sh_j = sc_j >> 3 in
+// its low half and sl_j = sc_j & 7 in its high half.  The multiply picks a half for both of its 16-bit lanes
+// through op_sel, so nothing has to be replicated.
+struct ScalePairs {
+    uint32_t p0, p1, p2, p3, p4, p5, p6, p7;
+};
+__device__ __forceinline__ ScalePairs scale_pairs(const BlockScales &s) {
+    const uint32_t sh_lo = (s.sc_lo >> 3) & 0x07070707u, sl_lo = s.sc_lo & 0x07070707u;
+    const uint32_t sh_hi = (s.sc_hi >> 3) & 0x07070707u, sl_hi = s.sc_hi & 0x07070707u;
+    // v_perm_b32: selector bytes 0..3 take the second operand's bytes, 4..7 the first's, 0x0c gives zero
+    ScalePairs r;
+    r.p0 = __builtin_amdgcn_perm(sl_lo, sh_lo, 0x0c040c00u);
+    r.p1 = __builtin_amdgcn_perm(sl_lo, sh_lo, 0x0c050c01u);
+    r.p2 = __builtin_amdgcn_perm(sl_lo, sh_lo, 0x0c060c02u);
+    r.p3 = __builtin_amdgcn_perm(sl_lo, sh_lo, 0x0c070c03u);
+    r.p4 = __builtin_amdgcn_perm(sl_hi, sh_hi, 0x0c040c00u);
+    r.p5 = __builtin_amdgcn_perm(sl_hi, sh_hi, 0x0c050c01u);
+    r.p6 = __builtin_amdgcn_perm(sl_hi, sh_hi, 0x0c060c02u);
+    r.p7 = __builtin_amdgcn_perm(sl_hi, sh_hi, 0x0c070c03u);
+    return r;
+}
+// bytes of `nib` (each below 16) times the low (H) and the high (L) half of `pair`: bytes stay below 106
+__device__ __forceinline__ void scaled_planes(uint32_t nib, uint32_t pair, int &h, int &l) {
+    asm("v_pk_mul_lo_u16 %0, %1, %2 op_sel_hi:[1,0]" : "=v"(h) : "v"(nib), "v"(pair));
+    asm("v_pk_mul_lo_u16 %0, %1, %2 op_sel:[0,1] op_sel_hi:[1,1]" : "=v"(l) : "v"(nib), "v"(pair));
+}
+__device__ __forceinline__ void unpack_pair_sel(const v4i q, uint32_t pair0, uint32_t pair1, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint32_t w = (uint32_t)q[c];
+        int h0, l0, h1, l1;
+        scaled_planes(w & 0x0f0f0f0fu, pair0, h0, l0);
+        scaled_planes((w >> 4) & 0x0f0f0f0fu, pair1, h1, l1);
+        H0[c] = h0, L0[c] = l0, H1[c] = h1, L1[c] = l1;
+    }
+}
+__device__ __forceinline__ void unpack_block_sel(const RawBlock &R, int lg, BPlanes &B) {
+    const BlockScales s = block_scales(R);
+    const ScalePairs p = scale_pairs(s);
+    unpack_pair_sel(R.q0, p.p0, p.p1, B.H0, B.L0, B.H1, B.L1);
+    unpack_pair_sel(R.q1, p.p2, p.p3, B.H2, B.L2, B.H3, B.L3);
+    unpack_pair_sel(R.q2, p.p4, p.p5, B.H4, B.L4, B.H5, B.L5);
+    unpack_pair_sel(R.q3, p.p6, p.p7, B.H6, B.L6, B.H7, B.L7);
+    unpack_rest(R, s, lg, B);
+}
+
+// The chain of a tile with its operands released two at a time (half as many waits as tile_chain, which the
+// Q5_K form keeps): the reads were requested in the order a0..a7, sums, and EXTRA more behind them.
+template <int N, class V>
+__device__ __forceinline__ void wait_lgkm2(V &r0, V &r1, v16i &acc) {
+    asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(r0), "+v"(r1), "+v"(acc) : "n"(N));
+}
+template <int EXTRA, class Between, class Next>
+__device__ __forceinline__ v16i tile_chain_pairs(TileOperands &T, const BPlanes &B, Between between, Next next) {
+    const v16i zi = {0};
+    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(T.a0), "+v"(T.a1) : "n"(7 + EXTRA));
+    v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.H0, zi, 0, 0, 0);
+    between(0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.H1, acc, 0, 0, 0);
+    between(1);
+    wait_lgkm2<5 + EXTRA>(T.a2, T.a3, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.H2, acc, 0, 0, 0);
+    between(2);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.H3, acc, 0, 0, 0);
+    between(3);
+    wait_lgkm2<3 + EXTRA>(T.a4, T.a5, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.H4, acc, 0, 0, 0);
+    between(4);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.H5, acc, 0, 0, 0);
+    between(5);
+    wait_lgkm2<1 + EXTRA>(T.a6, T.a7, acc);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.H6, acc, 0, 0, 0);
+    between(6);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.H7, acc, 0, 0, 0);
+    between(7);
+    wait_lgkm<0>(T.bs, acc);  // (and the EXTRA reads behind the sums)
+    acc = acc << 3;
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a0, B.L0, acc, 0, 0, 0);
+    between(8);
+    next(0);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a1, B.L1, acc, 0, 0, 0);
+    next(1);
+    between(9);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a2, B.L2, acc, 0, 0, 0);
+    next(2);
+    between(10);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a3, B.L3, acc, 0, 0, 0);
+    next(3);
+    between(11);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a4, B.L4, acc, 0, 0, 0);
+    next(4);
+    between(12);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a5, B.L5, acc, 0, 0, 0);
+    next(5);
+    between(13);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a6, B.L6, acc, 0, 0, 0);
+    next(6);
+    between(14);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(T.a7, B.L7, acc, 0, 0, 0);
+    next(7);
+    between(15);
+    return acc;
+}
+
 template <int RG, int KS, int MT, bool Q5 = false>
 __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
     using L = PipeLds<RG, KS, MT, Q5>;
     constexpr int BB = L::BB, PR = BB / 16;          // bytes of a block, its 16-byte pieces
     constexpr int NC = (32 * PR + 63) / 64;          // requests that move a wavefront's 32 rows of a block (the last: half)
     static_assert(32 * PR == 64 * (NC - 1) + 32, "the last request of a block is 32 lanes wide");
+    static_assert(NC == 5 || NC == 6, "four requests share one write of M0, the rest follow");
     constexpr int NW = L::NW, NT = L::NT, ROWS = 32 * RG, TM = 32 * MT;
-    static_assert(NW == 8 && NT == 4, "eight wavefronts share the four tile slots of a stage");
+    static_assert(NW == 8 && NT == 4 && (MT == 2 || MT == 4), "eight wavefronts share the four tile slots of a stage");
     extern __shared__ uint4 smem_gemm[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_gemm);
-    const uint32_t lds0 = lds_address(lds);
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_address(lds));
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 31, lg = lane >> 5;
@@ -561,22 +688,34 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
     const int kb0 = nb * (int)blockIdx.y / g.k_split, kb1 = nb * ((int)blockIdx.y + 1) / g.k_split;
     const int steps = (kb1 - kb0 + KS - 1) / KS;
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
-    auto block_of = [&](int share, int i) { return min(kb0 + share * steps + i, kb1 - 1); };  // uniform
-    auto tile_of = [&](int slot) { return min(tile0 + slot % MT, last_tile); };               // uniform
+    auto tile_of = [&](int slot) { return min(tile0 + slot % MT, last_tile); };  // uniform
 
-    // ---- what this wavefront fetches per step (all bases scalar, all lane offsets fixed) ----
-    // quants: the four consecutive k-slices (4 KB) (wave & 1) * 4 .. of tile slot wave / 2
-    const uint8_t *Qb = reinterpret_cast<const uint8_t *>(g.a.q);
-    const uint8_t *Sb = reinterpret_cast<const uint8_t *>(g.a.bs);
-    const uint8_t *Db = reinterpret_cast<const uint8_t *>(g.a.d);
-    const int slot_q = wave >> 1, slice_q = (wave & 1) * 4;
-    const int slot_s = wave & 3;                // sums of one tile slot (the second four wavefronts repeat the first)
-    const int slot_d = (wave & 1) * 2;          // scales of two tile slots, one per lane half
+    // ---- the fetch side.  Every address is a scalar pointer that moves on by one block a step plus a lane
+    // offset that never changes, and a stage of the rings is a scalar offset that rotates: a step's requests
+    // cost a handful of scalar instructions.  The first four wavefronts -- the ones the SIMDs' arbiters
+    // favour (they are the older of each SIMD's two), which otherwise wait at the step's barrier for the
+    // other four -- fetch the activations: wavefront f the record of tile slot f (8 KB of quants, 1 KB of
+    // sums), wavefronts 0 and 1 the scales of two slots each.  Every wavefront fetches its own weight rows.
+    const bool fetches_acts = wave < NT;
+    const bool fetches_scales = wave < 2;
     const uint32_t lane16 = (uint32_t)lane * 16;
+    const int slot_f = wave & 3, slot_d = (wave & 1) * 2;
+    // (a share past its last block keeps requesting that block: nobody multiplies it)
+    int next_kb_a = kb0 + (slot_f / MT) * steps;  // the block of this wavefront's activation slot at the next request
+    int next_kb_d = kb0 + (slot_d / MT) * steps;
+    int next_kb_w = kb0 + ks * steps;
+    const uint8_t *src_q = (const uint8_t *)scalar_pointer(reinterpret_cast<const uint8_t *>(g.a.q) +
+                                                           ((size_t)tile_of(slot_f) * nb + min(next_kb_a, kb1 - 1)) * 8192);
+    const uint8_t *src_s = (const uint8_t *)scalar_pointer(reinterpret_cast<const uint8_t *>(g.a.bs) +
+                                                           ((size_t)tile_of(slot_f) * nb + min(next_kb_a, kb1 - 1)) * 1024);
+    const uint8_t *src_d = (const uint8_t *)scalar_pointer(reinterpret_cast<const uint8_t *>(g.a.d) +
+                                                           ((size_t)tile_of(slot_d) * nb + min(next_kb_d, kb1 - 1)) * 128);
     const uint32_t lane_d = (uint32_t)(lane & 31) * 4 +
                             (lane >= 32 ? (uint32_t)(tile_of(slot_d + 1) - tile_of(slot_d)) * (uint32_t)nb * 128u : 0u);
-    // weights: this wavefront's 32 rows x 9 sixteen-byte pieces, piece p = 64 * c + lane of chunk c, so
-    // that LDS holds the rows back to back (144 bytes each).  Rows past the matrix read its last row.
+    // weights: this wavefront's 32 rows x PR sixteen-byte pieces, piece p = 64 * c + lane of chunk c, so that LDS
+    // holds the rows back to back.  Rows past the matrix read its last row.  Chunks 1..3 ride on chunk 0's M0
+    // with instruction offsets, which move the global address too: their lane offsets are short of it by as
+    // much (the pointer is kept 4096 bytes low and every offset 4096 high, so that none goes negative).
     const uint32_t stride = (uint32_t)g.row_stride;
     const int row_base = min(row_tile * ROWS + rg * 32, g.rows - 1);
     uint32_t w_off[NC];
@@ -584,29 +723,35 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
     for (int c = 0; c < NC; c++) {
         const int p = 64 * c + lane;
         const int r = min(p / PR, g.rows - 1 - row_base);
-        w_off[c] = (uint32_t)r * stride + (uint32_t)(p % PR) * 16;
+        w_off[c] = (uint32_t)r * stride + (uint32_t)(p % PR) * 16 + 4096u - (c < 4 ? 1024u * c : 0u);
     }
-    const uint8_t *Wrow = g.W + (size_t)row_base * stride;
+    const uint8_t *src_w = (const uint8_t *)scalar_pointer(g.W + (size_t)row_base * stride + (size_t)min(next_kb_w, kb1 - 1) * BB - 4096);
     const uint32_t lds_w = lds0 + L::OFF_W + wave * L::W_SLOT;
-
-    auto fetch_acts_part = [&](int j, int i) {  // j = 0..5: request part j of step i's activations
-        const uint32_t st = lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE;
-        if (j < 4) {
-            const size_t rec = (size_t)tile_of(slot_q) * nb + block_of(slot_q / MT, i);
-            dma16(st + slot_q * 8192 + (slice_q + j) * 1024, Qb + rec * 8192 + (size_t)(slice_q + j) * 1024, lane16);
-        } else if (j == 4) {
-            const size_t rec = (size_t)tile_of(slot_s) * nb + block_of(slot_s / MT, i);
-            dma16(st + L::OFF_BS + slot_s * 1024, Sb + rec * 1024, lane16);
-        } else {
-            const size_t rec = (size_t)tile_of(slot_d) * nb + block_of(slot_d / MT, i);
-            dma4(lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + slot_d * 128, Db + rec * 128, lane_d);
-        }
+    // the rings: activations three stages (a step's stage, the next one's, the one being filled), scales four
+    uint32_t st_cur = lds0, st_next = lds0 + L::A_STAGE, st_fill = lds0;  // st_fill: where the next request lands
+    uint32_t da_fill = lds0 + L::OFF_DA;
+    auto fetch_quants = [&](int half) {  // half of the slot's record: 4 KB
+        dma16_run<4>(st_fill + slot_f * 8192 + half * 4096, src_q + half * 4096, lane16, lane16, lane16, lane16);
     };
-    auto fetch_weights = [&](int i) {  // NC requests
-        const uint8_t *src = Wrow + (size_t)block_of(ks, i) * BB;
-#pragma unroll
-        for (int c = 0; c < NC - 1; c++) dma16(lds_w + c * 1024, src, w_off[c]);
-        if (lane < 32) dma16(lds_w + (NC - 1) * 1024, src, w_off[NC - 1]);
+    auto fetch_sums_scales = [&]() {
+        dma16_run<1>(st_fill + L::OFF_BS + slot_f * 1024, src_s, lane16, 0, 0, 0);
+        if (fetches_scales) dma4(da_fill + slot_d * 128, src_d, lane_d);
+    };
+    auto acts_fetched = [&]() {  // the request for a step is out: everything moves on to the step after
+        const bool adv_a = next_kb_a + 1 < kb1, adv_d = next_kb_d + 1 < kb1;
+        next_kb_a++, next_kb_d++;
+        src_q += adv_a ? 8192 : 0;
+        src_s += adv_a ? 1024 : 0;
+        src_d += adv_d ? 128 : 0;
+        st_fill = st_fill == lds0 + 2 * L::A_STAGE ? lds0 : st_fill + L::A_STAGE;
+        da_fill = da_fill == lds0 + L::OFF_DA + 3 * L::DA_STAGE ? lds0 + L::OFF_DA : da_fill + L::DA_STAGE;
+    };
+    auto fetch_weights = [&]() {  // NC requests
+        dma16_run<4>(lds_w, src_w, w_off[0], w_off[1], w_off[2], w_off[3]);
+        if (NC == 6) dma16_run<1>(lds_w + 4096, src_w, w_off[4], 0, 0, 0);
+        if (lane < 32) dma16_run<1>(lds_w + (NC - 1) * 1024, src_w, w_off[NC - 1], 0, 0, 0);
+        src_w += next_kb_w + 1 < kb1 ? BB : 0;
+        next_kb_w++;
     };
 
     v16f sum[MT];
@@ -628,41 +773,42 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
         }
     };
     auto unpack = [&]() {
-        unpack_block(R, lg, B);
+        unpack_block_sel(R, lg, B);
         if (Q5) unpack_fifth(R, F, P);
         fold_mins(B);
     };
 
     // prologue: activations of steps 0 and 1, weights of step 0; then the weights of step 1
-#pragma unroll
-    for (int j = 0; j < 6; j++) fetch_acts_part(j, 0);
-    fetch_weights(0);
-    if (steps > 1) {
-#pragma unroll
-        for (int j = 0; j < 6; j++) fetch_acts_part(j, 1);
+    if (fetches_acts) {
+        fetch_quants(0), fetch_quants(1), fetch_sums_scales(), acts_fetched();
     }
-    // where step i's first tile slot of this wavefront's share sits in LDS: quants and sums (lane offsets in)
-    auto quants_of = [&](int i) { return lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + (uint32_t)(ks * MT) * 8192 + lane16; };
-    auto sums_of = [&](int i) {
-        return lds0 + (uint32_t)(i % L::A_STAGES) * L::A_STAGE + L::OFF_BS + (uint32_t)(ks * MT) * 1024 + lane16;
-    };
-    auto is_active = [&](int i) { return kb0 + ks * steps + i < kb1; };  // uniform per wavefront
+    fetch_weights();
+    if (steps > 1 && fetches_acts) {
+        fetch_quants(0), fetch_quants(1), fetch_sums_scales(), acts_fetched();
+    }
+    // how many requests of a step's activations this wavefront makes (they stay in flight over the step's end)
+    const int acts_requests = fetches_scales ? 10 : fetches_acts ? 9 : 0;
+    // where a step's first tile slot of this wavefront's share sits in its stage (lane offsets in)
+    const uint32_t rd_q = (uint32_t)(ks * MT) * 8192 + lane16, rd_b = L::OFF_BS + (uint32_t)(ks * MT) * 1024 + lane16;
+    const uint32_t rd_d = lds0 + L::OFF_DA + (uint32_t)(ks * MT) * 128 + lg * 16;
+    const int my_steps = max(0, min(steps, kb1 - (kb0 + ks * steps)));  // the steps in which this wavefront's share has a block
     TileOperands T;  // the first tile's operands of the step about to run: requested behind the barrier, so that
                      // they travel while the block is unpacked
     wait_vm<0>();
     lds_barrier();
     {
         read_block();
-        if (steps > 1) fetch_weights(1);
-        if (is_active(0)) read_tile<0>(T, quants_of(0), sums_of(0));
+        if (steps > 1) fetch_weights();
+        if (my_steps > 0) read_tile<0>(T, st_cur + rd_q, st_cur + rd_b);
         unpack();
     }
 
     for (int i = 0; i < steps; i++) {
-        const bool active = is_active(i);
-        const uint32_t qa = quants_of(i), ba = sums_of(i);
-        const uint32_t sa = lds0 + L::OFF_DA + (uint32_t)(i % L::DA_STAGES) * L::DA_STAGE + (uint32_t)(ks * MT) * 128 + lg * 16;
+        const bool active = i < my_steps;
+        const uint32_t qa = st_cur + rd_q, ba = st_cur + rd_b;
+        const uint32_t sa = rd_d + (uint32_t)(i & 3) * L::DA_STAGE;
         const bool more_acts = i + 2 < steps;
+        const bool fetch_now = more_acts && fetches_acts;
         if (active) {
             TileOperands Tn;
             TileTail E;
@@ -672,7 +818,11 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
                 constexpr int mt = decltype(mt_c)::value;
                 auto between = [&](int j) {
                     if (mt == 0) {
-                        if (j < 6 && more_acts) fetch_acts_part(j, i + 2);
+                        if (fetch_now) {
+                            if (j == 1) fetch_quants(0);
+                            if (j == 3) fetch_quants(1);
+                            if (j == 5) fetch_sums_scales(), acts_fetched();
+                        }
                     } else {
                         // the scales of the tile before were the last reads requested ahead of this chain:
                         // they have landed once the chain has waited for everything, in front of MFMA 8, and
@@ -698,7 +848,7 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
                 constexpr int EXTRA = mt > 0 ? 4 : 0;
                 v16i s1;
                 if constexpr (Q5) s1 = tile_chain<EXTRA, true>(T, B, between, next, fifth_chain<EXTRA>(T, P));
-                else s1 = tile_chain<EXTRA>(T, B, between, next);
+                else s1 = tile_chain_pairs<EXTRA>(T, B, between, next);
                 E.s1 = s1;
                 E.bs = T.bs;
                 if (mt + 1 < MT) {
@@ -716,19 +866,21 @@ __global__ __launch_bounds__(512) void gemm_q4_k_pipe_kernel(GemmArgs g) {
             wait_scales<0>(E.S);
 #pragma unroll
             for (int j = 0; j < 16; j++) tail_piece(j, E, B, sum[MT - 1]);
-        } else if (more_acts) {
-#pragma unroll
-            for (int j = 0; j < 6; j++) fetch_acts_part(j, i + 2);
+        } else if (fetch_now) {
+            fetch_quants(0), fetch_quants(1), fetch_sums_scales(), acts_fetched();
         }
         if (i + 1 < steps) {
             // step i+1's raw weights (requested a step ago) leave their slot, which is refilled at once;
             // the activations of step i+2, younger than they, may stay in flight
-            if (more_acts) wait_vm<6>();
-            else wait_vm<0>();
+            if (!fetch_now) wait_vm<0>();
+            else if (acts_requests == 10) wait_vm<10>();
+            else wait_vm<9>();
             read_block();
-            if (more_acts) fetch_weights(i + 2);
+            if (more_acts) fetch_weights();
             lds_barrier();
-            if (is_active(i + 1)) read_tile<0>(T, quants_of(i + 1), sums_of(i + 1));
+            st_cur = st_next;
+            st_next = st_next == lds0 + 2 * L::A_STAGE ? lds0 : st_next + L::A_STAGE;
+            if (i + 1 < my_steps) read_tile<0>(T, st_cur + rd_q, st_cur + rd_b);
             unpack();
         } else {
             lds_barrier();
