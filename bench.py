@@ -237,6 +237,18 @@ def read_sweep(torch, fa):
         print("%10d  %7.2f  %7.1f" % (nbytes, t / n * 1e6, nbytes / (t / n) / 1e9), flush=True)
 
 
+def issue_probe(fa):
+    """frk_hip_issue_probe: a chain of dependent v_mfma_i32_32x32x32_i8 with N cheap vector instructions behind each,
+    two wavefronts per SIMD on every compute unit."""
+    import ctypes as C
+    out = (C.c_float * 16)()
+    fa.check(fa.lib().frk_hip_issue_probe(out))
+    print("# v_mfma_i32_32x32x32_i8 (32 clocks of the matrix core) + N x v_and_b32 per MFMA, 2 wavefronts per SIMD")
+    print("# N  cycles per MFMA and SIMD  shader MHz  launch us  first wavefront's share of the launch")
+    for k, n in enumerate((0, 4, 8, 12)):
+        print("%3d  %8.1f  %8.0f  %9.1f  %6.2f" % (n, out[4 * k], out[4 * k + 1], out[4 * k + 2], out[4 * k + 3]), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -245,6 +257,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--read-sweep", action="store_true", help="only: time of a read-only stream against its size")
+    ap.add_argument("--issue-probe", action="store_true", help="only: what a matrix-core instruction costs the vector ALU, "
+                    "and the shader clock under matrix-core load")
     ap.add_argument("--only", default="", help="comma-separated groups of secondary workloads to run (ceilings, gemv, gemm, "
                     "moe, thin, qkv): a profiler run replays only the kernels it is about")
     ap.add_argument("--graph-steps", type=int, default=GRAPH_STEPS, help="most steps captured in one HIP graph")
@@ -267,6 +281,9 @@ def main():
 
     if args.read_sweep:
         read_sweep(torch, fa)
+        return
+    if args.issue_probe:
+        issue_probe(fa)
         return
     info = fa.probe()
     dev = torch.device("cuda:0")

@@ -8,7 +8,7 @@ fn main() {
     let hipcc = std::env::var("HIPCC").unwrap_or_else(|_| "/opt/rocm/bin/hipcc".into());
     let srcs = [
         "frk_runtime.cpp", "frk_quant.hip", "frk_gemv.hip", "frk_gemv_fused.hip", "frk_gemm.hip", "frk_gemm_q6.hip",
-        "frk_gemm_q8.hip", "frk_moe.hip", "frk_thin.hip", "frk_gemv_direct.hip", "frk_gemv_f32dot.hip", "frk_kinds.hip",
+        "frk_gemm_q8.hip", "frk_moe.hip", "frk_thin.hip", "frk_gemv_direct.hip", "frk_gemv_f32dot.hip", "frk_kinds.hip", "frk_probe.hip",
     ];
     let mut objs = vec![];
     for s in srcs {

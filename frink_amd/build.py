@@ -10,7 +10,7 @@ LIBDIR = os.path.join(HERE, "lib")
 SO = os.path.join(LIBDIR, "libfrink_hip.so")
 STATIC = os.path.join(LIBDIR, "libfrink_hip.a")
 
-SOURCES = ["frk_runtime.cpp", "frk_quant.hip", "frk_gemv.hip", "frk_gemv_fused.hip", "frk_gemm.hip", "frk_gemm_q6.hip", "frk_gemm_q8.hip", "frk_moe.hip", "frk_thin.hip", "frk_gemv_direct.hip", "frk_gemv_f32dot.hip", "frk_kinds.hip"]
+SOURCES = ["frk_runtime.cpp", "frk_quant.hip", "frk_gemv.hip", "frk_gemv_fused.hip", "frk_gemm.hip", "frk_gemm_q6.hip", "frk_gemm_q8.hip", "frk_moe.hip", "frk_thin.hip", "frk_gemv_direct.hip", "frk_gemv_f32dot.hip", "frk_kinds.hip", "frk_probe.hip"]
 
 # -ffp-contract=off: the bit-exact kernels must round every f32 operation separately, and the
 # others spell fmaf() where they want a fused multiply-add.  Packed-FP32 instructions are

@@ -410,6 +410,17 @@ int frk_hip_copy_dev(const void *src, void *dst, size_t bytes, void *stream) {
     return launch_copy(src, dst, bytes, (hipStream_t)stream);
 }
 
+int frk_hip_issue_probe(float *out16_host) {
+    clear_error();
+    if (!out16_host) return set_error(FRK_ERR_ARG, "frk_hip_issue_probe: null argument");
+    {
+        std::lock_guard<std::mutex> lk(g_dev.mu);
+        int rc = ensure_device_locked();
+        if (rc) return rc;
+    }
+    return launch_issue_probe(out16_host, nullptr);
+}
+
 int frk_hip_read_dev(const void *src, size_t bytes, void *sink, void *stream) {
     clear_error();
     if (!src || !sink) return set_error(FRK_ERR_ARG, "frk_hip_read_dev: null argument");

@@ -928,6 +928,180 @@ __global__ __launch_bounds__(512) void thin_span_q4_k_kernel(const uint8_t *__re
         if (4 * g + r < batch && row < rows) y[(size_t)(4 * g + r) * rows + row] = acc[r];
 }
 
+// ------------------------------------------------------------------ thin GEMM streamed in chunks (Q6_K)
+//
+// The Q6_K kernel above loads a block's planes into registers with five gather-like loads per lane (sixteen
+// rows an instruction) and walks a row group's blocks as a chain of round trips.  Here a workgroup is ONE row
+// group of 16 rows and its wavefronts split the row's blocks; a wavefront moves a chunk -- S6_CB blocks of its 16
+// rows, and the same blocks of the (at most 8) quantized activation rows -- into an LDS buffer of its own with
+// global_load_lds (a lane names its own 16-byte piece: the LDS image is the rows back to back,
+// [ql CB x 128 | qh CB x 64 | sc CB x 16 | the 16 bytes around the chunk's d] a row; the activations CB x 16 pieces a
+// row and one of padding, so that the rows of a read fall in different banks), and multiplies the chunk when it
+// has landed; with two buffers the next chunk travels meanwhile.  Nothing is shared before the sums: no barrier in
+// the loop.  The arithmetic is the kernel's above.  (The longer a chunk, the longer the contiguous runs the
+// planar rows give the memory system: a block's run is 128 bytes.)
+// Measured at 4096 x 14336, 8 rows, from quantized activations (us): chunks of 2 blocks, one buffer, 14 wavefronts 16.3;
+// 2 blocks, two buffers, 7 wavefronts 16.7 - 17.1; one block, two to four buffers, 6 to 13 wavefronts 17.8 - 20.0; chunks of 4
+// blocks 23 and more; the kernel above 19.7.  More wavefronts beat deeper buffers: a wavefront issues one instruction
+// in five clocks or so, and a chunk is some 600 of them.
+constexpr int S6_CB = 2;                                // blocks of a chunk (2 or 4: the chunk's d sit in one aligned 16 bytes)
+constexpr int S6_BUFS = 1;                              // 1 or 2
+constexpr int S6_MAX_WAVES = 14;
+constexpr int S6_WPIECES = 13 * S6_CB + 1;              // 27 / 53: odd, rows 8 banks apart
+constexpr int S6_WROW = S6_WPIECES * 16;
+constexpr int S6_WBUF = 16 * S6_WROW;
+constexpr int S6_APIECES = 16 * S6_CB + 1;
+constexpr int S6_AROW = S6_APIECES * 16;
+constexpr int S6_ABUF = 8 * S6_AROW + S6_CB * 32;       // quants of 8 rows, then the scales [CB blocks][8 rows]
+constexpr int S6_BUF = S6_WBUF + S6_ABUF;
+constexpr int S6_WREQ = (16 * S6_WPIECES + 63) / 64, S6_AREQ = (8 * S6_APIECES + 63) / 64;
+constexpr int S6_REQUESTS = S6_WREQ + S6_AREQ + 1;      // requests of a chunk
+static_assert(S6_BUF % 16 == 0 && (size_t)S6_MAX_WAVES * S6_BUFS * S6_BUF <= 160 * 1024 && S6_REQUESTS < 64, "LDS of a CU; vmcnt");
+
+__global__ __launch_bounds__(64 * S6_MAX_WAVES) void thin_stream_q6_k_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
+                                                                           int batch, const int8_t *__restrict__ aq,
+                                                                           const float *__restrict__ ad, float *__restrict__ y) {
+    extern __shared__ uint4 smem[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem);
+    const int cols = nb * QK_K;
+    // a batch wider than 8 is a grid of groups of 8 activation rows: blockIdx.y picks the group
+    aq += (size_t)blockIdx.y * 8 * cols;
+    ad += (size_t)blockIdx.y * 8 * nb;
+    y += (size_t)blockIdx.y * 8 * rows;
+    batch = min(8, batch - (int)blockIdx.y * 8);
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = (int)blockDim.x >> 6;
+    const int j = lane & 15, g = lane >> 4;
+    const int row0 = (int)blockIdx.x * 16;
+    const int chunks = nb / S6_CB;  // (nb is a multiple of S6_CB)
+    const int c_begin = chunks * wave / waves, c_end = chunks * (wave + 1) / waves;
+    uint8_t *const my_lds = lds + (size_t)wave * S6_BUFS * S6_BUF;
+    const uint32_t my_lds_a = lds_address(my_lds);
+
+    // ---- what a lane fetches of a chunk: fixed pieces, the chunk number moves the addresses ----
+    // weights: slot piece s = 64 i + lane is row s / S6_WPIECES, piece s % S6_WPIECES of that row's image
+    const int rbase = min(row0, rows - 1);  // (rows past the matrix read its last row and store nothing)
+    const uint8_t *w_base = (const uint8_t *)scalar_pointer(W + (size_t)rbase * lay.row_stride);
+    uint32_t w_off[S6_WREQ], w_step[S6_WREQ];
+    bool w_is_d[S6_WREQ];
+#pragma unroll
+    for (int i = 0; i < S6_WREQ; i++) {
+        const int sidx = min(64 * i + lane, 16 * S6_WPIECES - 1);
+        const int r = sidx / S6_WPIECES, p = sidx % S6_WPIECES;
+        const uint32_t ro = (uint32_t)(min(row0 + r, rows - 1) - rbase) * (uint32_t)lay.row_stride;
+        w_is_d[i] = p == 13 * S6_CB;
+        if (p < 8 * S6_CB) w_off[i] = ro + (uint32_t)p * 16, w_step[i] = 128 * S6_CB;
+        else if (p < 12 * S6_CB) w_off[i] = ro + (uint32_t)lay.off_a + (uint32_t)(p - 8 * S6_CB) * 16, w_step[i] = 64 * S6_CB;
+        else if (p < 13 * S6_CB) w_off[i] = ro + (uint32_t)lay.off_b + (uint32_t)(p - 12 * S6_CB) * 16, w_step[i] = 16 * S6_CB;
+        else w_off[i] = ro + (uint32_t)lay.off_c, w_step[i] = 16;  // the aligned 16 bytes that hold the chunk's scales d
+    }
+    // quants: piece s = 64 i + lane is activation row s / S6_APIECES, piece s % S6_APIECES (the last: the one before again)
+    uint32_t a_off[S6_AREQ];
+#pragma unroll
+    for (int i = 0; i < S6_AREQ; i++) {
+        const int sidx = min(64 * i + lane, 8 * S6_APIECES - 1);
+        const int a = min(sidx / S6_APIECES, batch - 1), p = min(sidx % S6_APIECES, 16 * S6_CB - 1);
+        a_off[i] = (uint32_t)a * (uint32_t)cols + (uint32_t)p * 16;
+    }
+    const uint32_t d_off = ((uint32_t)min(lane & 7, batch - 1) * (uint32_t)nb + (uint32_t)((lane >> 3) % S6_CB)) * 4u;  // [block][row]
+    auto fetch_chunk = [&](int c, int buf) {  // S6_REQUESTS requests
+        const uint32_t base = my_lds_a + (uint32_t)buf * S6_BUF;
+#pragma unroll
+        for (int i = 0; i < S6_WREQ; i++) {
+            const uint32_t off = w_off[i] + (w_is_d[i] ? (uint32_t)(c * S6_CB >> 3) : (uint32_t)c) * w_step[i];
+            if (i < S6_WREQ - 1 || lane < 16 * S6_WPIECES - (S6_WREQ - 1) * 64) dma16(base + i * 1024, w_base, off);
+        }
+        const int8_t *q_base = aq + (size_t)c * (S6_CB * QK_K);
+#pragma unroll
+        for (int i = 0; i < S6_AREQ; i++)
+            if (i < S6_AREQ - 1 || lane < 8 * S6_APIECES - (S6_AREQ - 1) * 64) dma16(base + S6_WBUF + i * 1024, q_base, a_off[i]);
+        if (lane < 8 * S6_CB) dma4(base + S6_WBUF + 8 * S6_AROW, ad + (size_t)c * S6_CB, d_off);
+    };
+
+    // activation operand row j of the MFMA: activation j % 8, and only the k-groups of its half are real
+    const bool real = (j < 8) == (g < 2);
+    auto as_long = [](uint2 v) { return (long)(((unsigned long)v.y << 32) | v.x); };
+    v4f_t acc = {0.f, 0.f, 0.f, 0.f};
+    auto multiply_chunk = [&](int c, int buf) {
+        const uint8_t *wb = my_lds + (size_t)buf * S6_BUF + j * S6_WROW;
+        const uint8_t *ab = my_lds + (size_t)buf * S6_BUF + S6_WBUF;
+        const uint8_t *a_q = ab + (size_t)(j & 7) * S6_AROW + 8 * g;
+        const float *a_d = reinterpret_cast<const float *>(ab + 8 * S6_AROW) + 4 * (g & 1);
+#pragma unroll
+        for (int b = 0; b < S6_CB; b++) {
+            const uint4 scv = *reinterpret_cast<const uint4 *>(wb + 192 * S6_CB + 16 * b);
+            const uint32_t scw[4] = {scv.x, scv.y, scv.z, scv.w};
+            const float d = h2f(*reinterpret_cast<const uint16_t *>(wb + 208 * S6_CB + (((S6_CB * c + b) * 2) & 15)));
+            const v4i_t zero = {0, 0, 0, 0};
+            v4i_t isum = {0, 0, 0, 0};
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint2 qla = *reinterpret_cast<const uint2 *>(wb + 128 * b + h * 64 + 8 * g);
+                const uint2 qlb = *reinterpret_cast<const uint2 *>(wb + 128 * b + h * 64 + 32 + 8 * g);
+                const uint2 qh = *reinterpret_cast<const uint2 *>(wb + 128 * S6_CB + 64 * b + h * 32 + 8 * g);
+#pragma unroll
+                for (int v = 0; v < 4; v++) {  // weights h*128 + 32*v + l, l = 8g .. 8g+7
+                    const uint2 ql = (v & 1) ? qlb : qla;
+                    auto code = [&](uint32_t lo, uint32_t hi) {  // four 6-bit codes, as signed bytes q - 32
+                        const uint32_t nib = (v >= 2 ? lo >> 4 : lo) & 0x0f0f0f0fu;
+                        const uint32_t top = ((hi >> (2 * v)) & 0x03030303u) << 4;
+                        return ((nib | top) + 0x60606060u) ^ 0x80808080u;
+                    };
+                    const uint2 wq = make_uint2(code(ql.x, qh.x), code(ql.y, qh.y));
+                    uint2 a = *reinterpret_cast<const uint2 *>(a_q + b * QK_K + h * 128 + 32 * v);
+                    if (!real) a = make_uint2(0u, 0u);
+                    const v4i_t t = __builtin_amdgcn_mfma_i32_16x16x32_i8(as_long(a), as_long(wq), zero, 0, 0, 0);
+                    const int si = h * 8 + 2 * v + (g >> 1);  // the scale of this lane's 16-wide group
+                    const int sc = (int)(int8_t)((scw[si >> 2] >> (8 * (si & 3))) & 0xff);
+#pragma unroll
+                    for (int r = 0; r < 4; r++) isum[r] += __mul24(sc, t[r]);
+                }
+            }
+            const v4f_t da = *reinterpret_cast<const v4f_t *>(a_d + b * 8);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += (d * da[r]) * (float)isum[r];
+        }
+    };
+
+    // requests complete in order, so "all but the youngest chunk's requests" means the older chunk has landed
+    if (c_begin < c_end) fetch_chunk(c_begin, 0);
+    for (int c = c_begin; c < c_end; c++) {
+        const int buf = S6_BUFS > 1 ? (c - c_begin) & 1 : 0;
+        if (S6_BUFS > 1 && c + 1 < c_end) {
+            fetch_chunk(c + 1, buf ^ 1);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S6_REQUESTS) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        multiply_chunk(c, buf);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the buffer has been read: a later chunk may land in it
+        if (S6_BUFS == 1 && c + 1 < c_end) fetch_chunk(c + 1, 0);
+    }
+    // the two 16-wide halves of every result sit 32 lanes apart
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[r] += __shfl_xor(acc[r], 32);
+    if (waves > 1) {  // the wavefronts' shares of the row meet in LDS and are added in their order
+        __syncthreads();
+        float *red = reinterpret_cast<float *>(lds);
+        if (wave > 0) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) red[((wave - 1) * 4 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int k = 0; k < waves - 1; k++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[r] += red[(k * 4 + r) * 64 + lane];
+    }
+    if (g < 2) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int b = 4 * g + r;
+            if (b < batch && row0 + j < rows) y[(size_t)b * rows + row0 + j] = acc[r];
+        }
+    }
+}
+
 // ------------------------------------------------------------------ launchers
 
 #define FRK_LAUNCH_CHECK(what)                                                                          \
@@ -1066,6 +1240,29 @@ static int launch_thin_mfma6_rg(const frk_weights *w, int batch, Q8KActs a, floa
     }
 }
 
+// ---- the streamed Q6_K kernel: rows of whole chunks of blocks, groups of 8 activation rows ----
+static bool thin_stream6_fits(const frk_weights *w) {
+    const size_t nb = w->cols / QK_K;
+    return w->kind == FRK_KIND_Q6_K && nb >= S6_CB && nb % S6_CB == 0 && (uint64_t)w->layout.row_stride * 16 < (1ull << 32) &&
+           (uint64_t)w->cols * 8 < (1ull << 32);
+}
+static int launch_thin_stream6(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
+    const size_t groups = (w->rows + 15) / 16, chunks = w->cols / QK_K / S6_CB;
+    // a wavefront per four chunks or so, as many as LDS holds buffers for
+    const int waves = (int)std::max<size_t>(1, std::min<size_t>(S6_MAX_WAVES, (chunks + 3) / 4));
+    const size_t shmem = (size_t)waves * S6_BUFS * S6_BUF;
+    static bool sized = false;
+    if (!sized) {
+        FRK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(&thin_stream_q6_k_kernel),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)TM_LDS_LIMIT));
+        sized = true;
+    }
+    hipLaunchKernelGGL(thin_stream_q6_k_kernel, dim3((unsigned)groups, (unsigned)((batch + 7) / 8)), dim3(64 * waves), shmem, s, w->dev,
+                       w->layout, (int)w->rows, (int)(w->cols / QK_K), batch, a.q, a.d, y);
+    FRK_LAUNCH_CHECK("thin stream gemm (Q6_K)");
+    return FRK_OK;
+}
+
 // ---- the span kernel: Q4_K rows of 4, 8, .. 32 blocks (a wavefront per four), up to 16 activation rows ----
 static bool thin_span_fits(const frk_weights *w, int batch) {
     const size_t nb = w->cols / QK_K, n_kg = nb / 4;
@@ -1111,6 +1308,7 @@ int thin_gemm_wide_rows(const frk_weights *w) {
 int launch_thin_gemm_wide(const frk_weights *w, int batch, Q8KActs a, float *y, hipStream_t s) {
     // Q5_K: many groups of activation rows fill the chip whatever the matrix, so a workgroup takes eight row groups
     if (w->kind == FRK_KIND_Q5_K) return launch_thin_mfma<8, 16>(w, batch, a, y, s);
+    if (thin_stream6_fits(w)) return launch_thin_stream6(w, batch, a, y, s);
     return launch_thin_mfma6_rg<8>(w, batch, a, y, s);
 }
 
@@ -1125,6 +1323,7 @@ int launch_thin_gemm(const frk_weights *w, int batch, Q8KActs a, float *y, hipSt
         if (batch <= 8) return launch_thin_mfma_rg<8>(w, batch, a, y, s);
         return launch_thin_mfma_rg<16>(w, batch, a, y, s);
     }
+    if (w->kind == FRK_KIND_Q6_K && batch > 2 && thin_stream6_fits(w)) return launch_thin_stream6(w, batch, a, y, s);
     if (w->kind == FRK_KIND_Q6_K && batch > 2 && thin_mfma6_acts(w) >= (batch > 4 ? 8 : 4))
         return batch > 4 ? launch_thin_mfma6_rg<8>(w, batch, a, y, s) : launch_thin_mfma6_rg<4>(w, batch, a, y, s);
     if (batch > 4) return launch_thin_nb<8>(w, batch, a, y, s);

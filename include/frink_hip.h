@@ -309,6 +309,13 @@ int frk_hip_copy_dev(const void *src_dev, void *dst_dev, size_t bytes, void *str
  * written -- a thread stores into sink_dev (>= 64 KiB) only if its words fold to one particular
  * value, which is there to keep the loads alive. */
 int frk_hip_read_dev(const void *src_dev, size_t bytes, void *sink_dev, void *stream);
+/* Calibration of the matrix-core kernels' issue budget (no counterpart in the reference; synchronous, allocates,
+ * not for a hot loop).  Four launches of a loop of dependent v_mfma_i32_32x32x32_i8 with 0, 4, 8 and 12 independent
+ * vector instructions behind each MFMA, two wavefronts per SIMD; per launch four floats: shader cycles per MFMA and
+ * SIMD (the launch's duration at the clock measured in it), the shader clock in MHz during the loop (cycle counter
+ * against the constant 100 MHz counter), microseconds of the launch, and the share of the launch that the first
+ * wavefront's own loop took. */
+int frk_hip_issue_probe(float *out16_host);
 
 #ifdef __cplusplus
 }

@@ -1127,6 +1127,8 @@ def test_k_quant_f32_dot_refuses_long_rows(fa):
     (fo.Q4_K, 1000, 4096, 9), (fo.Q4_K, 31, 8192, 13), (fo.Q4_K, 20, 16384, 6), (fo.Q4_K, 18, 32768, 5),
     (fo.Q6_K, 70, 1024, 2), (fo.Q6_K, 33, 512, 3), (fo.Q6_K, 48, 14336, 8), (fo.Q6_K, 64, 256, 7),
     (fo.Q6_K, 40, 2048, 11), (fo.Q6_K, 24, 768, 40), (fo.Q6_K, 19, 28672, 4), (fo.Q6_K, 50, 4096, 5),
+    # (the streamed Q6_K kernel: rows of 2, 6, 14 and 28 blocks -- one wavefront, uneven shares, a last row group partly empty)
+    (fo.Q6_K, 37, 1536, 8), (fo.Q6_K, 20, 3584, 6), (fo.Q6_K, 16, 7168, 8), (fo.Q6_K, 33, 512, 17),
 ])
 def test_thin_gemm_matches_the_oracle_and_the_gemv(fa, kind, rows, cols, batch):
     from frink_amd import synth
