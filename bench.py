@@ -237,6 +237,42 @@ def read_sweep(torch, fa):
         print("%10d  %7.2f  %7.1f" % (nbytes, t / n * 1e6, nbytes / (t / n) / 1e9), flush=True)
 
 
+def read_shapes(torch, fa):
+    """frk_hip_read_shape_dev over the headline matrix's 33,030,144 bytes, cache-cold: which span per wavefront,
+    wavefronts per workgroup, landing place and cache bits fetch it fastest, with frk_hip_read_dev beside them"""
+    import ctypes as C
+    dev = torch.device("cuda:0")
+    nbytes = 14336 * 4096 // 256 * 144
+    slots = COPIES
+    pool = torch.empty(slots * nbytes, dtype=torch.uint8, device=dev).random_()
+    sink = torch.empty(1 << 16, dtype=torch.uint8, device=dev)
+    L = fa.lib()
+
+    def run(fn):
+        _, t = time_graph(torch, fn, 400, 400)
+        return t / 400 * 1e6
+
+    def plain(i):
+        fa.check(L.frk_hip_read_dev(C.c_void_p(pool.data_ptr() + (i % slots) * nbytes), nbytes, C.c_void_p(sink.data_ptr()),
+                                    fa._stream()))
+    print("# fetch of %d bytes, cache-cold (%d copies in turn), 400 launches in one graph; us per launch" % (nbytes, slots))
+    print("frk_hip_read_dev  %6.2f" % run(plain), flush=True)
+    print("# span KB  wavefronts/workgroup  landing  policy  us  GB/s")
+    names = ("-", "nt", "sc1", "sc0 sc1")
+    for to_lds in (0, 1):
+        for span in (2, 4, 9, 18):
+            for waves in (4, 8, 16):
+                if to_lds and waves * min(span, 8) > 160:
+                    continue
+                for policy in (0, 1, 2, 3):
+                    def rd(i):
+                        fa.check(L.frk_hip_read_shape_dev(C.c_void_p(pool.data_ptr() + (i % slots) * nbytes), nbytes,
+                                                          C.c_void_p(sink.data_ptr()), span, waves, to_lds, policy, fa._stream()))
+                    us = run(rd)
+                    print("%3d  %3d  %-9s  %-8s  %6.2f  %7.1f" % (span, waves, "LDS" if to_lds else "registers", names[policy], us,
+                                                                 nbytes / us / 1e3), flush=True)
+
+
 def issue_probe(fa):
     """frk_hip_issue_probe: a chain of dependent v_mfma_i32_32x32x32_i8 with N cheap vector instructions behind each,
     two wavefronts per SIMD on every compute unit."""
@@ -257,6 +293,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--read-sweep", action="store_true", help="only: time of a read-only stream against its size")
+    ap.add_argument("--read-shapes", action="store_true", help="only: the headline matrix's bytes fetched in the decode "
+                    "kernels' shape -- span per wavefront, wavefronts per workgroup, registers or LDS, cache bits")
     ap.add_argument("--issue-probe", action="store_true", help="only: what a matrix-core instruction costs the vector ALU, "
                     "and the shader clock under matrix-core load")
     ap.add_argument("--only", default="", help="comma-separated groups of secondary workloads to run (ceilings, gemv, gemm, "
@@ -281,6 +319,9 @@ def main():
 
     if args.read_sweep:
         read_sweep(torch, fa)
+        return
+    if args.read_shapes:
+        read_shapes(torch, fa)
         return
     if args.issue_probe:
         issue_probe(fa)

@@ -35,7 +35,7 @@ EXPORTS = [
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
-    "frk_hip_copy_dev", "frk_hip_read_dev", "frk_hip_issue_probe",
+    "frk_hip_copy_dev", "frk_hip_read_dev", "frk_hip_issue_probe", "frk_hip_read_shape_dev",
 ]
 
 
@@ -108,6 +108,7 @@ def lib():
             "frk_hip_copy_dev": (i, [vp, vp, sz, vp]),
             "frk_hip_read_dev": (i, [vp, sz, vp, vp]),
             "frk_hip_issue_probe": (i, [vp]),
+            "frk_hip_read_shape_dev": (i, [vp, sz, vp, i, i, i, i, vp]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)

@@ -71,6 +71,28 @@ __device__ __forceinline__ void dma16(uint32_t lds_uniform, const void *base_uni
                  : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
                  : "memory");
 }
+// Loads with the non-temporal bit, for weights a decode step fetches once (see dma16_nt for what the bit buys).
+typedef uint32_t nt_u4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t nt_u2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 stream_load16(const void *p) {
+    const nt_u4_t v = __builtin_nontemporal_load(reinterpret_cast<const nt_u4_t *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ uint2 stream_load8(const void *p) {
+    const nt_u2_t v = __builtin_nontemporal_load(reinterpret_cast<const nt_u2_t *>(p));
+    return make_uint2(v.x, v.y);
+}
+__device__ __forceinline__ uint16_t stream_load2(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(p));
+}
+// The same with the non-temporal bit: for data fetched once per launch (a decode step's weights).  Measured on
+// the bare fetch of 33 MB in 9 KB spans, cache-cold: 5.97 us per launch with the bit, 6.45 without.
+__device__ __forceinline__ void dma16_nt(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_uniform)), "v"(lane_off), "s"(scalar_pointer(base_uniform))
+                 : "memory");
+}
 __device__ __forceinline__ void dma4(uint32_t lds_uniform, const void *base_uniform, uint32_t lane_off) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                  :

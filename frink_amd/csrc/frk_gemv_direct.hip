@@ -393,8 +393,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_0_f32_shared_kernel(const 
 #pragma unroll
     for (int j = 0; j < U; j++) {
         const int u = min(lane + 64 * j, units - 1);
-        qv[j] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
-        dbits[j] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2);
+        qv[j] = stream_load16(row + (size_t)u * 16);
+        dbits[j] = stream_load2(row + lay.off_a + (size_t)(u >> 1) * 2);
     }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * U) : "memory");  // the activation piece has landed
     lds_barrier();
@@ -454,8 +454,8 @@ __global__ __launch_bounds__(1024) void gemv_q8_0_f32_cols_kernel(const uint8_t 
 #pragma unroll
     for (int k = 0; k < R; k++) {
         const uint8_t *row = W + (size_t)min(r0 + k, rows - 1) * lay.row_stride;  // (a row past the end: the last again)
-        qv[k] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
-        dbits[k] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)(u >> 1) * 2);
+        qv[k] = stream_load16(row + (size_t)u * 16);
+        dbits[k] = stream_load2(row + lay.off_a + (size_t)(u >> 1) * 2);
     }
 #pragma unroll
     for (int k = 0; k < R; k++) {
@@ -504,8 +504,8 @@ __global__ __launch_bounds__(1024) void gemv_q4_0_f32_cols_kernel(const uint8_t 
 #pragma unroll
     for (int k = 0; k < R; k++) {
         const uint8_t *row = W + (size_t)min(r0 + k, rows - 1) * lay.row_stride;  // (a row past the end: the last again)
-        qv[k] = *reinterpret_cast<const uint4 *>(row + (size_t)u * 16);
-        dbits[k] = *reinterpret_cast<const uint16_t *>(row + lay.off_a + (size_t)u * 2);
+        qv[k] = stream_load16(row + (size_t)u * 16);
+        dbits[k] = stream_load2(row + lay.off_a + (size_t)u * 2);
     }
     float xsum = 0.0f;
 #pragma unroll

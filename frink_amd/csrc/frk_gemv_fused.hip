@@ -508,7 +508,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
     const uint32_t left = (uint32_t)min((size_t)SPAN, bytes - span_c * SPAN);  // (the last span may be short)
     const uint32_t slot = lds_address(sw) + (uint32_t)wave * SPAN;
 #pragma unroll
-    for (int c = 0; c < FIRST; c++) dma16(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+    for (int c = 0; c < FIRST; c++) dma16_nt(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
 
     // ---- the activation into LDS ----
     if (MODE == MODE_FUSED) {
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_lines_kernel(const uint8
     // starts multiplying when ITS blocks have landed, whatever the others' have done.
     lds_barrier();
 #pragma unroll
-    for (int c = FIRST; c < PIECES; c++) dma16(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+    for (int c = FIRST; c < PIECES; c++) dma16_nt(slot + c * 1024, span_src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the span has landed (in this wavefront's own slot)
     if (!has_rows) return;
 
@@ -655,7 +655,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q4_k_rows_kernel(const uint8_
         const uint32_t left = (uint32_t)min((size_t)span_bytes, bytes - span_c * span_bytes);
         const uint32_t slot = lds_address(sw) + (uint32_t)wave * SLOT;
 #pragma unroll
-        for (int c = 0; c < PIECES; c++) dma16(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
+        for (int c = 0; c < PIECES; c++) dma16_nt(slot + c * 1024, src, min((uint32_t)(c * 1024 + lane * 16), left - 16));
     }
     if (MODE == MODE_FUSED) {
         asm volatile("s_waitcnt vmcnt(%8)"

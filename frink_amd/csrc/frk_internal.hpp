@@ -144,6 +144,7 @@ int launch_copy(const void *src, void *dst, size_t bytes, hipStream_t s);
 int launch_read(const void *src, size_t bytes, void *sink, hipStream_t s);
 // calibration of the matrix-core kernels' issue budget (frk_probe.hip): 16 floats, four per count of vector instructions
 int launch_issue_probe(float *out, hipStream_t s);
+int launch_read_shape(const void *src, size_t bytes, void *sink, int span_kb, int waves, int to_lds, int policy, hipStream_t s);
 
 struct Q8KActs {  // Q8_K activations in HBM, struct-of-arrays per activation row
     const int8_t *q;      // [batch][cols]

@@ -98,4 +98,99 @@ int launch_issue_probe(float *out, hipStream_t s) {
     return rc;
 }
 
+// read_shape_kernel: the bare fetch of a buffer in the shape the decode kernels use -- every wavefront owns one
+// contiguous span of SPAN KB and issues all of its 16-byte loads before it waits for the first -- so that the
+// shape's parameters can be priced one at a time: the span, the wavefronts per workgroup, whether the data lands
+// in registers or is copied straight into LDS, and the cache policy bits of the load (POLICY 0 none, 1 nt,
+// 2 sc1, 3 sc0 sc1).  Nothing is done with the data beyond what keeps the loads alive.
+template <int POLICY>
+__device__ __forceinline__ v4i_p load16_policy(const uint4 *p) {
+    v4i_p v;
+    if (POLICY == 0) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    if (POLICY == 1) asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(v) : "v"(p) : "memory");
+    if (POLICY == 2) asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    if (POLICY == 3) asm volatile("global_load_dwordx4 %0, %1, off sc0 sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int POLICY>
+__device__ __forceinline__ void dma16_policy(uint32_t lds_uniform, const uint4 *p) {
+    const uint32_t m = __builtin_amdgcn_readfirstlane(lds_uniform);
+    if (POLICY == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m), "v"(p) : "memory");
+    if (POLICY == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" : : "s"(m), "v"(p) : "memory");
+    if (POLICY == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off sc1" : : "s"(m), "v"(p) : "memory");
+    if (POLICY == 3) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off sc0 sc1" : : "s"(m), "v"(p) : "memory");
+}
+
+template <int SPAN, int POLICY, bool TO_LDS>
+__global__ __launch_bounds__(1024) void read_shape_kernel(const uint4 *__restrict__ src, size_t spans, uint32_t *__restrict__ sink) {
+    extern __shared__ uint4 landing[];  // TO_LDS: min(SPAN, 8) KB per wavefront
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const size_t span = (size_t)blockIdx.x * (blockDim.x >> 6) + wave;
+    if (span >= spans) return;
+    const uint4 *p = src + span * (SPAN * 64) + lane;
+    uint32_t acc = 0;
+    if (TO_LDS) {
+        constexpr int ROOM = SPAN < 8 ? SPAN : 8;
+        const uint32_t base = lds_address(landing) + wave * (ROOM * 1024);
+#pragma unroll
+        for (int i = 0; i < SPAN; i++) dma16_policy<POLICY>(base + (i % ROOM) * 1024, p + i * 64);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
+        v4i_p v[SPAN];
+#pragma unroll
+        for (int i = 0; i < SPAN; i++) v[i] = load16_policy<POLICY>(p + i * 64);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < SPAN; i++) {
+            asm volatile("" : "+v"(v[i]));  // (the values exist only after the wait above)
+            acc ^= (uint32_t)(v[i][0] ^ v[i][1] ^ v[i][2] ^ v[i][3]);
+        }
+        if (acc == 0x9e3779b9u) sink[(blockIdx.x * 64 + lane) & 16383] = acc;
+    }
+}
+
+template <int SPAN, int POLICY>
+static int launch_read_shape_sp(const void *src, size_t spans, void *sink, int waves, bool to_lds, hipStream_t s) {
+    const unsigned grid = (unsigned)((spans + waves - 1) / waves);
+    if (to_lds) {
+        const size_t room = (size_t)waves * (SPAN < 8 ? SPAN : 8) * 1024;
+        auto k = read_shape_kernel<SPAN, POLICY, true>;
+        FRK_HIP_TRY(hipFuncSetAttribute((const void *)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)room));
+        hipLaunchKernelGGL(k, dim3(grid), dim3(waves * 64), room, s, (const uint4 *)src, spans, (uint32_t *)sink);
+    } else {
+        hipLaunchKernelGGL((read_shape_kernel<SPAN, POLICY, false>), dim3(grid), dim3(waves * 64), 0, s, (const uint4 *)src, spans,
+                           (uint32_t *)sink);
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return set_error(FRK_ERR_HIP, "read shape launch: %s", hipGetErrorString(e));
+    return FRK_OK;
+}
+template <int SPAN>
+static int launch_read_shape_s(const void *src, size_t spans, void *sink, int waves, bool to_lds, int policy, hipStream_t s) {
+    switch (policy) {
+        case 0: return launch_read_shape_sp<SPAN, 0>(src, spans, sink, waves, to_lds, s);
+        case 1: return launch_read_shape_sp<SPAN, 1>(src, spans, sink, waves, to_lds, s);
+        case 2: return launch_read_shape_sp<SPAN, 2>(src, spans, sink, waves, to_lds, s);
+        case 3: return launch_read_shape_sp<SPAN, 3>(src, spans, sink, waves, to_lds, s);
+    }
+    return set_error(FRK_ERR_ARG, "read shape: policy %d is not one of 0..3", policy);
+}
+
+// Reads floor(bytes / (span_kb KB)) spans of the buffer; span_kb in {2, 4, 9, 18}, waves (per workgroup) in 1..16.
+int launch_read_shape(const void *src, size_t bytes, void *sink, int span_kb, int waves, int to_lds, int policy, hipStream_t s) {
+    if (waves < 1 || waves > 16) return set_error(FRK_ERR_ARG, "read shape: %d wavefronts per workgroup", waves);
+    const size_t spans = bytes / ((size_t)span_kb * 1024);
+    if (spans == 0 || spans / waves >= 0x7fffffffu) return set_error(FRK_ERR_ARG, "read shape: %zu bytes", bytes);
+    if (to_lds && (size_t)waves * (span_kb < 8 ? span_kb : 8) * 1024 > 160 * 1024)
+        return set_error(FRK_ERR_ARG, "read shape: %d wavefronts of %d KB do not fit the LDS", waves, span_kb);
+    switch (span_kb) {
+        case 2: return launch_read_shape_s<2>(src, spans, sink, waves, to_lds != 0, policy, s);
+        case 4: return launch_read_shape_s<4>(src, spans, sink, waves, to_lds != 0, policy, s);
+        case 9: return launch_read_shape_s<9>(src, spans, sink, waves, to_lds != 0, policy, s);
+        case 18: return launch_read_shape_s<18>(src, spans, sink, waves, to_lds != 0, policy, s);
+    }
+    return set_error(FRK_ERR_ARG, "read shape: span of %d KB is not one of 2, 4, 9, 18", span_kb);
+}
+
+
 }  // namespace frk

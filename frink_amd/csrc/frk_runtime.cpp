@@ -428,6 +428,13 @@ int frk_hip_read_dev(const void *src, size_t bytes, void *sink, void *stream) {
     return launch_read(src, bytes, sink, (hipStream_t)stream);
 }
 
+int frk_hip_read_shape_dev(const void *src, size_t bytes, void *sink, int span_kb, int waves, int to_lds, int policy,
+                           void *stream) {
+    clear_error();
+    if (!src || !sink) return set_error(FRK_ERR_ARG, "frk_hip_read_shape_dev: null argument");
+    return launch_read_shape(src, bytes, sink, span_kb, waves, to_lds, policy, (hipStream_t)stream);
+}
+
 // Where one call's scratch memory comes from: the stream's leased buffer (grown on demand), or a fixed
 // region that has to suffice (the entry point that allocates nothing).  It must outlive the launches that
 // use the memory; nested requests of one call get the same start address, as with the lease.

@@ -316,6 +316,13 @@ int frk_hip_read_dev(const void *src_dev, size_t bytes, void *sink_dev, void *st
  * against the constant 100 MHz counter), microseconds of the launch, and the share of the launch that the first
  * wavefront's own loop took. */
 int frk_hip_issue_probe(float *out16_host);
+/* Calibration of the decode kernels' fetch shape (no counterpart in the reference).  Reads the first
+ * floor(bytes / span) spans of the buffer and writes nothing: every wavefront owns one contiguous span of span_kb KB
+ * (2, 4, 9 or 18) and issues all its 16-byte loads before it waits; waves_per_group 1..16; to_lds 0 = into registers,
+ * 1 = copied straight into LDS (global_load_lds); policy = cache bits on the loads (0 none, 1 nt, 2 sc1, 3 sc0 sc1).
+ * sink_dev as for frk_hip_read_dev. */
+int frk_hip_read_shape_dev(const void *src_dev, size_t bytes, void *sink_dev, int span_kb, int waves_per_group,
+                           int to_lds, int policy, void *stream);
 
 #ifdef __cplusplus
 }
