@@ -35,7 +35,7 @@ EXPORTS = [
     "frk_hip_moe_intermediates_dev",
     "frk_hip_quantize_q8_k_dev", "frk_hip_quantize_q8_0_dev", "frk_hip_dequant_dev",
     "frk_hip_get_rows_dev", "frk_hip_get_rows",
-    "frk_hip_copy_dev", "frk_hip_read_dev", "frk_hip_issue_probe", "frk_hip_read_shape_dev",
+    "frk_hip_copy_dev", "frk_hip_read_dev", "frk_hip_issue_probe", "frk_hip_read_shape_dev", "frk_hip_gemm_grouped_dev",
 ]
 
 
@@ -108,6 +108,7 @@ def lib():
             "frk_hip_copy_dev": (i, [vp, vp, sz, vp]),
             "frk_hip_read_dev": (i, [vp, sz, vp, vp]),
             "frk_hip_issue_probe": (i, [vp]),
+            "frk_hip_gemm_grouped_dev": (i, [vp, sz, vp, vp, vp, sz, sz, vp, vp]),
             "frk_hip_read_shape_dev": (i, [vp, sz, vp, i, i, i, i, vp]),
         }
         for name, (res, args) in sig.items():
@@ -352,6 +353,25 @@ def moe_ffn(gate, up, down, n_experts, x, ids, weights, out=None):
     check(lib().frk_hip_moe_ffn_dev(gate.handle, up.handle, down.handle, n_experts, C.c_void_p(x.data_ptr()), batch,
                                     C.c_void_p(ids.data_ptr()), C.c_void_p(weights.data_ptr()), k,
                                     C.c_void_p(y.data_ptr()), _stream()))
+    return y
+
+
+def gemm_grouped(stacked, n_groups, group_off, x, gather=None, out=None):
+    """The grouped (indexed) GEMM: pair p of group g (group_off[g] <= p < group_off[g+1]) is row gather[p] of x
+    (row p without a gather list) times group g's matrix, rows [g*R, (g+1)*R) of `stacked`; out[pairs][R]."""
+    import torch
+    assert x.dtype == torch.float32 and x.is_cuda and x.is_contiguous() and x.shape[-1] == stacked.cols
+    assert group_off.dtype == torch.int32 and group_off.is_cuda and group_off.numel() == n_groups + 1
+    x_rows = x.numel() // stacked.cols
+    if gather is not None:
+        assert gather.dtype == torch.int32 and gather.is_cuda and gather.is_contiguous()
+        pairs = gather.numel()
+    else:
+        pairs = x_rows
+    y = out if out is not None else torch.empty((pairs, stacked.rows // n_groups), dtype=torch.float32, device=x.device)
+    check(lib().frk_hip_gemm_grouped_dev(stacked.handle, n_groups, C.c_void_p(group_off.data_ptr()),
+                                         C.c_void_p(gather.data_ptr()) if gather is not None else None,
+                                         C.c_void_p(x.data_ptr()), x_rows, pairs, C.c_void_p(y.data_ptr()), _stream()))
     return y
 
 

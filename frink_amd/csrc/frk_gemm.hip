@@ -72,12 +72,12 @@ struct GemmArgs {
 // The grouped form: work items (tile, matrix, row group of 256 rows) streamed by persistent workgroups.
 struct StreamArgs {
     const uint8_t *W[2];
-    float *y[2];  // [32 * tiles][rows]
+    float *y[2];  // row (tile's first row of y + r) x [rows]: tile row r
     int n_mat;
     size_t row_stride;
     int rows, nb;  // of one expert
     Q8KTiled a;
-    const int4 *tiles;  // {expert, 32 * t, rows in use, 0}
+    const int4 *tiles;  // {expert, first row of the grouped order, rows in use, first row of y}
     const int *n_tiles;
     int row_tiles;  // ceil(rows / 256)
     // the gathering form: the activations are the source rows' Q8_K, quantized once each, and row r of the
@@ -944,14 +944,14 @@ struct StreamLds {
     static constexpr int A_STAGE = 2 * A_HALF;       // a tile is two records
     static constexpr int A_STAGES = 4;
     static constexpr int OFF_A = W_STAGES * W_STAGE;
-    // {expert, rows in use} of each of the workgroup's items, filled once: looked up from LDS, an
+    // {expert, rows in use, first row of y} of each of the workgroup's items, filled once: looked up from LDS, an
     // item change costs no global load (whose completion would count in vmcnt, in the middle of the
     // prefetch bookkeeping)
     static constexpr int OFF_ITEMS = OFF_A + A_STAGES * A_STAGE;
     static constexpr int MAX_ITEMS = GATHER ? 64 : 128;
     // GATHER: the source rows of each item's tile, row r of the first half in the low 16 bits of word r and
     // row 32 + r in the high ones
-    static constexpr int OFF_SRC = OFF_ITEMS + MAX_ITEMS * 8;
+    static constexpr int OFF_SRC = OFF_ITEMS + MAX_ITEMS * 16;
     static constexpr size_t BYTES = (size_t)OFF_SRC + (GATHER ? MAX_ITEMS * 128 : 0);
     static_assert(BYTES <= 160 * 1024, "LDS of a CU");
 };
@@ -986,10 +986,10 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         rg = w - m * g.row_tiles;
     };
     {
-        int2 *table = reinterpret_cast<int2 *>(lds + L::OFF_ITEMS);
+        int4 *table = reinterpret_cast<int4 *>(lds + L::OFF_ITEMS);
         for (int i = tid; i < my_items; i += 64 * L::RG) {
             const int4 ti = g.tiles[xcd + 8 * ((slot + i * per_xcd) / per_tile)];
-            table[i] = make_int2(ti.x, ti.z);
+            table[i] = make_int4(ti.x, ti.z, ti.w, 0);
         }
         if (GATHER) {
             uint32_t *src_rows = reinterpret_cast<uint32_t *>(lds + L::OFF_SRC);
@@ -1002,11 +1002,12 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         __syncthreads();
     }
     const uint32_t lds_items = lds_address(lds + L::OFF_ITEMS);
-    auto item_info = [&](int ord, int &expert, int &count) {
-        v2i v;
-        asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_items + ord * 8));
+    auto item_info = [&](int ord, int &expert, int &count, int &y_row) {
+        v4i v;
+        asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(lds_items + ord * 16));
         expert = __builtin_amdgcn_readfirstlane(v.x);
         count = __builtin_amdgcn_readfirstlane(v.y);
+        y_row = __builtin_amdgcn_readfirstlane(v.z);
     };
 
     // ---- the fetch side: a cursor (item, block) three steps ahead of the arithmetic ----
@@ -1033,9 +1034,9 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
     bool f_two = false;  // the cursor's tile has rows in its second half
     int issued = 0;      // loads of the fetch most recently issued by this wavefront
     auto point_at = [&](int ord) {  // uniform
-        int t, m, rg, expert, count;
+        int t, m, rg, expert, count, y_row;
         item_of(ord, t, m, rg);
-        item_info(ord, expert, count);
+        item_info(ord, expert, count, y_row);
         f_w = (m ? g.W[1] : g.W[0]) + (size_t)expert * g.rows * g.row_stride;
         const int l = opaque_lane();
         w_off0 = (uint32_t)(rg * (32 * L::RG) + wave * 32 + l / 9) * (uint32_t)g.row_stride + (uint32_t)(l % 9) * 16;
@@ -1130,8 +1131,8 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
     BPlanes B0, B1;
     v16f accF0 = v16f{0.0f}, accF1 = v16f{0.0f};  // the tile's two halves
     const bool fetch_late = wave >= L::RG / 2;
-    int c_ord = 0, c_kb = 0, c_count = 0;
-    int pending = -1, pending_count = 0;  // item whose results wait to be stored
+    int c_ord = 0, c_kb = 0, c_count = 0, c_y_row = 0;
+    int pending = -1, pending_count = 0, pending_y_row = 0;  // item whose results wait to be stored
     auto raw_of_step = [&](int s) {  // this lane's part of its row's block, read and arrived
         const int l = opaque_lane(), li = l & 31, lg = l >> 5;
         const uint32_t wa = lds0 + (s & 1) * L::W_STAGE + (wave * 32 + li) * Q4_K_BYTES;
@@ -1160,7 +1161,7 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         const uint32_t st = lds0 + L::OFF_A + (s & 3) * L::A_STAGE;
         if (c_kb == 0) {
             int expert;
-            item_info(c_ord, expert, c_count);
+            item_info(c_ord, expert, c_count, c_y_row);
         }
         const BlockScales sc = block_scales(R);
         const int lg_next = opaque_lane() >> 5;
@@ -1175,6 +1176,7 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         if (++c_kb == nb) {
             pending = c_ord++;
             pending_count = c_count;
+            pending_y_row = c_y_row;
             c_kb = 0;
         }
     };
@@ -1188,7 +1190,7 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         const int row = rg * (32 * L::RG) + wave * 32 + li;
         int rows = g.rows;
         asm volatile("" : "+s"(rows));  // opaque: keeps the 16 row offsets from being hoisted out of the loop and held
-        float *y = (m ? g.y[1] : g.y[0]) + (size_t)t * MOE_TILE * rows;
+        float *y = (m ? g.y[1] : g.y[0]) + (size_t)pending_y_row * rows;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = (r >> 2) * 8 + lg * 4 + (r & 3);

@@ -242,12 +242,14 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
     const int tile0 = tok0 / 32, last_tile = (g.M - 1) / 32;
     uint32_t expert_base = 0;  // byte offset of the expert's first weight row
     int tok_end = g.M;         // first activation row that is not stored
+    int y_shift = 0;           // activation row r is stored as row r + y_shift of y
     if (g.tiles) {             // (uniform per workgroup)
         const int t = in_grp >> 3;
         if (t >= *g.n_tiles) return;
         const int4 ti = g.tiles[t];
         expert_base = (uint32_t)ti.x * (uint32_t)g.rows * g.row_stride;
         tok_end = ti.y + ti.z;
+        y_shift = ti.w - ti.y;
     }
     auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
         int l = lane;
@@ -407,7 +409,7 @@ __global__ __launch_bounds__(512) void gemm_q6_k_mfma_kernel(Q6GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + (tile_first + mt) * 32 + (r >> 2) * 8 + lg * 4 + (r & 3);
-            if (row < g.rows && tok < tok_end) dst[(size_t)tok * g.rows + row] = accF[mt][r];
+            if (row < g.rows && tok < tok_end) dst[(size_t)(tok + y_shift) * g.rows + row] = accF[mt][r];
         }
 }
 

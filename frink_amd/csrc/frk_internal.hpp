@@ -246,6 +246,11 @@ bool gemm_q4_k_stream_gathers(size_t src_rows, size_t cols);
 int launch_gemm_q4_k_stream(const frk_weights *w0, const frk_weights *w1, size_t rows_e, Q8KTiled a,
                             const Q8KRows *src, const int *gather, const int4 *tiles, const int *n_tiles,
                             int max_tiles, float *y0, float *y1, hipStream_t s);
+// The grouped GEMM over groups the caller lists (Q4_K or Q6_K weights stacked group by group): y[p] = W[group of
+// p] . x[gather ? gather[p] : p]; ws must hold grouped_gemm_workspace_bytes(...)
+size_t grouped_gemm_workspace_bytes(size_t n_groups, size_t x_rows, size_t pairs, size_t cols);
+int launch_gemm_grouped(const frk_weights *w, size_t n_groups, const int32_t *group_off, const int32_t *gather,
+                        const float *x, size_t x_rows, size_t pairs, float *y, void *ws, hipStream_t s);
 // MoE expert FFN over stacked Q4_K experts; ws must hold moe_workspace_bytes(...)
 size_t moe_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);
 int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,

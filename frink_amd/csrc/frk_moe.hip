@@ -100,7 +100,7 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *wave_tot, int &t
 //   gather[max_rows] token of each row of the grouped order, -1 in a gap and past the last tile
 //   pos_of[pairs]    row of pair (tok*k + slot); -1 for an id outside [0, E)
 //   cpos_of[pairs]   the pair's place in the order without the gaps
-//   tiles / n_tiles  {expert, first row, rows in use, 0} per tile
+//   tiles / n_tiles  {expert, first row, rows in use, first row of the GEMMs' output (the same row)} per tile
 // One workgroup of 1024 threads; E <= 1024.  No atomic decides an order: a round takes `round`
 // pairs, marks pair j of expert e as bit j of row e of a bit matrix in LDS (an OR, so the result
 // does not depend on who comes first; the matrix is stored word-major so that the per-expert
@@ -169,7 +169,7 @@ __device__ __forceinline__ void moe_group(const GroupArgs &a) {
             for (int i = 0; i < nt; i++) {
                 const int t = i < big ? tb + i : ts;
                 const int used = min(MOE_TILE, c - MOE_TILE * i);
-                tiles[t] = make_int4(tid, MOE_TILE * t, used, 0);
+                tiles[t] = make_int4(tid, MOE_TILE * t, used, MOE_TILE * t);
             }
         }
         if (tid == 0) {
@@ -238,6 +238,84 @@ __global__ __launch_bounds__(1024) void moe_group_quantize_kernel(GroupArgs a, c
                                                                   Q8KRows out) {
     if (blockIdx.x == 0) {
         moe_group(a);
+        return;
+    }
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int b = ((int)blockIdx.x - 1) * 16 + wave; b < n_blocks; b += ((int)gridDim.x - 1) * 16) {
+        const float4 v = reinterpret_cast<const float4 *>(x + (size_t)b * QK_K)[lane];
+        float dd;
+        int bs;
+        const uint32_t packed = quantize_q8_k_lane(v, dd, bs);
+        reinterpret_cast<uint32_t *>(out.q + (size_t)b * QK_K)[lane] = packed;
+        if ((lane & 3) == 0) out.bs[(size_t)b * 16 + (lane >> 2)] = (_Float16)bs;
+        if (lane == 0) out.d[b] = dd;
+    }
+}
+
+// The grouped GEMM with the groups given (enqueue_mul_mm_grouped_dev, crates/frink-cuda/src/mul_mm_launch.rs:391-470):
+// pairs group_off[g] .. group_off[g+1]-1 belong to group g and pair p reads activation row gather[p] (row p without
+// a gather list).  This cuts the groups into the tiles the grouped kernels walk -- {group, first row of the grouped
+// order, rows in use, first pair}: the kernels store tile row r as row (first pair + r) of y, so y comes out as
+// [pairs][rows] without gaps -- and lists every tile row's source row (-1: not in use).  Tiles with more than 32
+// rows in use first, as in moe_group.  One workgroup of 1024 threads, at most 1024 groups.
+struct GroupedTilesArgs {
+    const int32_t *group_off, *gather;  // gather may be null
+    int n_groups, pairs, x_rows, max_rows;
+    int *src_rows;  // [max_rows]
+    int4 *tiles;
+    int *n_tiles;
+};
+struct GroupedTilesLds {
+    int off[1025], tile_big[1024], n_big[1024], tile_small[1024];
+    int wave_tot[16];
+};
+__device__ __forceinline__ void grouped_tiles(const GroupedTilesArgs &a) {
+    __shared__ GroupedTilesLds L;
+    const int tid = threadIdx.x;
+    for (int r = tid; r < a.max_rows; r += 1024) a.src_rows[r] = -1;
+    // (offsets outside 0 .. pairs or out of order: clamped, so that no tile row points outside the lists)
+    for (int g = tid; g <= a.n_groups; g += 1024) L.off[g] = min(max(a.group_off[g], 0), a.pairs);
+    __syncthreads();
+    {
+        const int c = tid < a.n_groups ? max(L.off[tid + 1] - L.off[tid], 0) : 0;
+        const int nt = (c + MOE_TILE - 1) / MOE_TILE;
+        const int last = c - MOE_TILE * (nt - 1);
+        const int big = nt == 0 ? 0 : nt - 1 + (last > 32);
+        const int small = nt - big;  // 0 or 1
+        int total_big, total_small;
+        const int tb = block_exclusive_scan(big, L.wave_tot, total_big);
+        const int ts = total_big + block_exclusive_scan(small, L.wave_tot, total_small);
+        L.tile_big[tid] = tb;
+        L.n_big[tid] = big;
+        L.tile_small[tid] = ts;
+        for (int i = 0; i < nt; i++) {
+            const int t = i < big ? tb + i : ts;
+            a.tiles[t] = make_int4(tid, MOE_TILE * t, min(MOE_TILE, c - MOE_TILE * i), L.off[tid] + MOE_TILE * i);
+        }
+        if (tid == 0) *a.n_tiles = total_big + total_small;
+    }
+    __syncthreads();
+    for (int p = tid; p < a.pairs; p += 1024) {
+        int lo = 0, hi = a.n_groups;  // the group g with off[g] <= p < off[g+1]: the last g with off[g] <= p
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (L.off[mid] <= p) lo = mid;
+            else hi = mid;
+        }
+        const int rank = p - L.off[lo];
+        if (rank < 0 || p >= L.off[lo + 1]) continue;  // (a pair before the first group or in a clamped hole)
+        const int i = rank / MOE_TILE;
+        const int t = i < L.n_big[lo] ? L.tile_big[lo] + i : L.tile_small[lo];
+        const int src = a.gather ? a.gather[p] : p;
+        a.src_rows[MOE_TILE * t + rank % MOE_TILE] = min(max(src, 0), a.x_rows - 1);
+    }
+}
+__global__ __launch_bounds__(1024) void grouped_tiles_kernel(GroupedTilesArgs a) { grouped_tiles(a); }
+// the same beside the quantization of the activation rows, as in moe_group_quantize_kernel
+__global__ __launch_bounds__(1024) void grouped_tiles_quantize_kernel(GroupedTilesArgs a, const float *__restrict__ x, int n_blocks,
+                                                                      Q8KRows out) {
+    if (blockIdx.x == 0) {
+        grouped_tiles(a);
         return;
     }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -542,6 +620,63 @@ int launch_moe_ffn(const frk_weights *gate, const frk_weights *up, const frk_wei
                        hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);
     FRK_LAUNCH_CHECK("moe_combine");
     return FRK_OK;
+}
+
+// The grouped GEMM as an entry of its own.  Scratch: the activations' Q8_K (plain rows, or gathered into the
+// grouped order when the kernel cannot address the plain rows or the weights are Q6_K), the tile list and the
+// tile rows' source rows.
+struct GroupedScratch {
+    Q8KTiled xa;
+    Q8KRows xr;
+    int *src_rows, *n_tiles;
+    int4 *tiles;
+};
+static GroupedScratch grouped_carve(void *base, size_t n_groups, size_t x_rows, size_t pairs, size_t cols, size_t *end) {
+    const size_t rows = moe_max_rows(pairs, (int)n_groups), nb = cols / QK_K;
+    char *p = (char *)base;
+    auto take = [&](size_t bytes) {
+        char *r = p;
+        p += round_up(bytes, 256);
+        return r;
+    };
+    GroupedScratch m;
+    const size_t plain = round_up(x_rows * cols, 256) + round_up(x_rows * nb * 32, 256) + x_rows * nb * 4;
+    char *room = take(std::max(q8k_tiled_bytes(rows, cols), plain));
+    m.xa = q8k_tiled_carve(room, rows, cols);
+    m.xr.q = (int8_t *)room;
+    m.xr.bs = (_Float16 *)(room + round_up(x_rows * cols, 256));
+    m.xr.d = (float *)(room + round_up(x_rows * cols, 256) + round_up(x_rows * nb * 32, 256));
+    m.src_rows = (int *)take(rows * 4);
+    m.n_tiles = (int *)take(256);
+    m.tiles = (int4 *)take((rows / MOE_TILE + 1) * 16);
+    if (end) *end = (size_t)(p - (char *)base);
+    return m;
+}
+size_t grouped_gemm_workspace_bytes(size_t n_groups, size_t x_rows, size_t pairs, size_t cols) {
+    size_t end = 0;
+    (void)grouped_carve(nullptr, n_groups, x_rows, pairs, cols, &end);
+    return end;
+}
+int launch_gemm_grouped(const frk_weights *w, size_t n_groups, const int32_t *group_off, const int32_t *gather,
+                        const float *x, size_t x_rows, size_t pairs, float *y, void *ws, hipStream_t s) {
+    const size_t rows_g = w->rows / n_groups, cols = w->cols, rows = moe_max_rows(pairs, (int)n_groups);
+    const GroupedScratch m = grouped_carve(ws, n_groups, x_rows, pairs, cols, nullptr);
+    const int max_tiles = (int)(rows / MOE_TILE);
+    const GroupedTilesArgs ta{group_off, gather, (int)n_groups, (int)pairs, (int)x_rows, (int)rows, m.src_rows, m.tiles, m.n_tiles};
+    if (w->kind == FRK_KIND_Q4_K && gemm_q4_k_stream_gathers(x_rows, cols)) {
+        const size_t n_blocks = x_rows * (cols / QK_K);
+        const unsigned quantizers = (unsigned)std::min<size_t>((n_blocks + 15) / 16, 512);
+        hipLaunchKernelGGL(grouped_tiles_quantize_kernel, dim3(1 + quantizers), dim3(1024), 0, s, ta, x, (int)n_blocks, m.xr);
+        FRK_LAUNCH_CHECK("grouped_tiles_quantize");
+        return launch_gemm_q4_k_stream(w, nullptr, rows_g, m.xa, &m.xr, m.src_rows, m.tiles, m.n_tiles, max_tiles, y, nullptr, s);
+    }
+    hipLaunchKernelGGL(grouped_tiles_kernel, dim3(1), dim3(1024), 0, s, ta);
+    FRK_LAUNCH_CHECK("grouped_tiles");
+    int rc = launch_quantize_q8_k_gather(x, cols, m.src_rows, rows, m.xa, s);
+    if (rc) return rc;
+    return w->kind == FRK_KIND_Q6_K
+               ? launch_gemm_q6_k_grouped(w, rows_g, m.xa, m.tiles, m.n_tiles, max_tiles, y, s)
+               : launch_gemm_q4_k_stream(w, nullptr, rows_g, m.xa, nullptr, nullptr, m.tiles, m.n_tiles, max_tiles, y, nullptr, s);
 }
 
 }  // namespace frk

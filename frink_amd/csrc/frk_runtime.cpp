@@ -1002,6 +1002,25 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
     return launch_moe_ffn(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, lease.ptr, (hipStream_t)stream);
 }
 
+int frk_hip_gemm_grouped_dev(const frk_weights *stacked, size_t n_groups, const int32_t *group_off, const int32_t *gather,
+                             const float *x, size_t x_rows, size_t pairs, float *y, void *stream) {
+    clear_error();
+    if (!stacked || !group_off || (pairs && (!x || !y))) return set_error(FRK_ERR_ARG, "frk_hip_gemm_grouped_dev: null argument");
+    if (n_groups == 0 || n_groups > 1024) return set_error(FRK_ERR_SHAPE, "groups=%zu (1 .. 1024)", n_groups);
+    if (stacked->kind != FRK_KIND_Q4_K && stacked->kind != FRK_KIND_Q6_K)
+        return set_error(FRK_ERR_UNSUPPORTED, "the grouped GEMM takes Q4_K or Q6_K weights (got kind %d)", stacked->kind);
+    if (stacked->rows % n_groups)
+        return set_error(FRK_ERR_SHAPE, "stacked rows %zu do not divide into %zu groups", stacked->rows, n_groups);
+    if (pairs > (size_t)1 << 30 || x_rows > (size_t)1 << 30)
+        return set_error(FRK_ERR_SHAPE, "pairs=%zu, activation rows=%zu: too many", pairs, x_rows);
+    if (pairs == 0) return FRK_OK;
+    if (x_rows == 0) return set_error(FRK_ERR_SHAPE, "%zu pairs over no activation rows", pairs);
+    WorkspaceLease lease;
+    int rc = workspace(grouped_gemm_workspace_bytes(n_groups, x_rows, pairs, stacked->cols), (hipStream_t)stream, lease);
+    if (rc) return rc;
+    return launch_gemm_grouped(stacked, n_groups, group_off, gather, x, x_rows, pairs, y, lease.ptr, (hipStream_t)stream);
+}
+
 int frk_hip_moe_intermediates_dev(size_t batch, size_t k, size_t n_experts, size_t hidden, size_t ffn,
                                   float *gate_out, float *up_out, int8_t *act_q, float *act_d, int32_t *pos_of,
                                   void *stream) {

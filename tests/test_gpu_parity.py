@@ -688,6 +688,113 @@ def _stacked_experts(n_experts, hidden, ffn, seed, random_blocks=False, sigma=0.
     return out
 
 
+def _grouped_case(kind, n_groups, rows_g, cols, counts, x_rows, seed, with_gather):
+    """Weights of n_groups stacked matrices, x, the offsets of groups of the given sizes and a gather list (or none:
+    pair p reads row p, so x has exactly one row per pair)."""
+    from frink_amd import synth
+    off = np.zeros(n_groups + 1, np.int32)
+    off[1:] = np.cumsum(counts)
+    pairs = int(off[-1])
+    if not with_gather:
+        x_rows = pairs
+    data = make_weights(kind, n_groups * rows_g, cols, seed=seed)
+    x = synth.activations(seed + 1, max(x_rows, 1), cols, outlier_frac=0.01)[:x_rows]
+    gather = np.random.default_rng(seed + 2).integers(0, max(x_rows, 1), pairs).astype(np.int32) if with_gather else None
+    return data, x, off, gather, pairs
+
+
+def _grouped_oracle(kind, data, n_groups, rows_g, cols, x, off, gather):
+    """enqueue_mul_mm_grouped_dev's contract (crates/frink-cuda/src/mul_mm_launch.rs:391-470) from the oracle's
+    GEMM, one group at a time."""
+    per = data.reshape(n_groups, -1)
+    want = np.zeros((int(off[-1]), rows_g), np.float32)
+    for g in range(n_groups):
+        p0, p1 = int(off[g]), int(off[g + 1])
+        if p1 > p0:
+            src = gather[p0:p1] if gather is not None else np.arange(p0, p1)
+            want[p0:p1] = fo.gemm(kind, per[g], rows_g, cols, x[src])
+    return want
+
+
+@pytest.mark.parametrize("kind", [fo.Q4_K, fo.Q6_K])
+@pytest.mark.parametrize("with_gather", [True, False])
+def test_grouped_gemm_on_its_own(fa, kind, with_gather):
+    """Groups of 0, 1, 31..33, 64, 65 and 150 pairs (tiles of every fill, a group of several tiles, empty groups at
+    both ends), rows that are not a multiple of the kernels' 256-row groups, a gather list that repeats rows."""
+    counts = [0, 1, 31, 0, 32, 33, 64, 65, 150, 7, 0]
+    n_groups, rows_g, cols = len(counts), 200, 768
+    print("grouped gemm", kind, with_gather, flush=True)
+    data, x, off, gather, pairs = _grouped_case(kind, n_groups, rows_g, cols, counts, 90, 77 + kind, with_gather)
+    w = fa.Weights.from_host(kind, data, n_groups * rows_g, cols)
+    import torch
+    y = torch.full((pairs, rows_g), float("nan"), dtype=torch.float32, device="cuda")
+    got = fa.gemm_grouped(w, n_groups, to_dev(off), to_dev(x), to_dev(gather) if with_gather else None, out=y).cpu().numpy()
+    want = _grouped_oracle(kind, data, n_groups, rows_g, cols, x, off, gather)
+    assert not np.isnan(got).any()  # every pair's row written
+    assert_rows_close(got, want, "grouped gemm kind %d gather %s" % (kind, with_gather))
+    # a second, smaller call on the same stream's scratch
+    counts2 = [5, 0, 40]
+    data2, x2, off2, gather2, pairs2 = _grouped_case(kind, 3, rows_g, cols, counts2, 20, 99, with_gather)
+    w2 = fa.Weights.from_host(kind, data2, 3 * rows_g, cols)
+    got2 = fa.gemm_grouped(w2, 3, to_dev(off2), to_dev(x2), to_dev(gather2) if with_gather else None).cpu().numpy()
+    assert_rows_close(got2, _grouped_oracle(kind, data2, 3, rows_g, cols, x2, off2, gather2), "grouped gemm, second call")
+    w.release()
+    w2.release()
+
+
+def test_grouped_gemm_at_the_expert_shape(fa):
+    """128 groups of 768 x 2048 (the routed layer's gate experts), 4096 pairs of 512 rows: every output against the
+    oracle."""
+    from frink_amd import synth
+    n_groups, rows_g, cols, x_rows, k = 128, 768, 2048, 512, 8
+    print("grouped gemm 128 x 768 x 2048", flush=True)
+    data = make_weights(fo.Q4_K, n_groups * rows_g, cols, seed=5)
+    x = synth.activations(6, x_rows, cols, outlier_frac=0.01)
+    rng = np.random.default_rng(7)
+    ids = np.stack([rng.permutation(n_groups)[:k] for _ in range(x_rows)]).astype(np.int32)
+    order = np.argsort(ids.ravel(), kind="stable")  # pairs by group, tokens ascending inside a group
+    gather = (order // k).astype(np.int32)
+    off = np.zeros(n_groups + 1, np.int32)
+    off[1:] = np.cumsum(np.bincount(ids.ravel(), minlength=n_groups))
+    w = fa.Weights.from_host(fo.Q4_K, data, n_groups * rows_g, cols)
+    got = fa.gemm_grouped(w, n_groups, to_dev(off), to_dev(x), to_dev(gather)).cpu().numpy()
+    want = _grouped_oracle(fo.Q4_K, data, n_groups, rows_g, cols, x, off, gather)
+    assert_rows_close(got, want, "grouped gemm at the expert shape")
+    w.release()
+
+
+def test_grouped_gemm_over_more_rows_than_the_gathering_kernel_addresses(fa):
+    """70000 activation rows (the gathering kernel's table holds 16-bit rows): the rows in use are gathered into the
+    grouped order and quantized there."""
+    counts = [3, 70, 0, 33]
+    n_groups, rows_g, cols = len(counts), 64, 256
+    print("grouped gemm, 70000 activation rows", flush=True)
+    data, x, off, gather, pairs = _grouped_case(fo.Q4_K, n_groups, rows_g, cols, counts, 70000, 123, True)
+    gather[:4] = [69999, 0, 65536, 65535]
+    w = fa.Weights.from_host(fo.Q4_K, data, n_groups * rows_g, cols)
+    got = fa.gemm_grouped(w, n_groups, to_dev(off), to_dev(x), to_dev(gather)).cpu().numpy()
+    assert_rows_close(got, _grouped_oracle(fo.Q4_K, data, n_groups, rows_g, cols, x, off, gather), "grouped gemm, 70000 rows")
+    w.release()
+
+
+def test_grouped_gemm_refuses_what_it_cannot_run(fa):
+    data = make_weights(fo.Q8_0, 64, 256, seed=1)
+    w = fa.Weights.from_host(fo.Q8_0, data, 64, 256)
+    off = to_dev(np.array([0, 1, 2], np.int32))
+    x = to_dev(np.zeros((2, 256), np.float32))
+    with pytest.raises(fa.BackendError):
+        fa.gemm_grouped(w, 2, off, x)
+    w.release()
+    data = make_weights(fo.Q4_K, 96, 256, seed=1)
+    w = fa.Weights.from_host(fo.Q4_K, data, 96, 256)
+    with pytest.raises(fa.BackendError):  # 96 rows do not divide into 5 groups
+        fa.gemm_grouped(w, 5, to_dev(np.zeros(6, np.int32)), x)
+    # no pairs: nothing to do, no error
+    y = fa.gemm_grouped(w, 2, to_dev(np.zeros(3, np.int32)), x, gather=to_dev(np.zeros(0, np.int32)))
+    assert y.shape == (0, 48)
+    w.release()
+
+
 def _slot_order(ids_row, batch):
     """The order in which the reference adds a token's routed slots: ascending expert id on its bucket
     path (32 tokens and more, ffn_batch.rs:355, 388-423), routing order below that
