@@ -237,7 +237,10 @@ __global__ __launch_bounds__(256) void read_kernel(const uint4 *__restrict__ src
     size_t base = (size_t)blockIdx.x * 512;
     for (; base + 512 <= n; base += stride) {
         const uint4 *p = src + base + threadIdx.x;
-        const uint4 a = p[0], b = p[256];
+        // (non-temporal loads: 0.4 us of 6.4 at 33 MB)
+        typedef uint32_t nt4_t __attribute__((ext_vector_type(4)));
+        const nt4_t a = __builtin_nontemporal_load(reinterpret_cast<const nt4_t *>(p));
+        const nt4_t b = __builtin_nontemporal_load(reinterpret_cast<const nt4_t *>(p + 256));
         acc ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
     }
     if (base < n) {  // at most one workgroup holds the ragged tail
