@@ -270,6 +270,9 @@ int launch_gemv_q6_k_direct(const frk_weights *w, Q8KActs a, float *y, hipStream
 int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // Q5_0, IQ4_XS, MXFP4: dequantizer / row gather and the f32-dot decode GEMV
 bool is_unit_kind(int kind);
+// the integer tier of Q5_0 / MXFP4 (Q8_0 activation blocks) and IQ4_XS (Q8_K quants and block scales)
+bool gemv_units_int_fits(const frk_weights *w);
+int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s);
 int launch_dequant_units(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s);
 int launch_gemv_units_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // K-quant GEMV on dequantized weights and the f32 activation (the reference's default x86 decode numerics)

@@ -6,7 +6,7 @@
 // The resident copy keeps the GGUF bytes of a row in place (rows start 16-byte aligned); a weight is the
 // dequantizer's value bit for bit.  The GEMV is the f32 dot of the reference's decode path: a wavefront
 // per row, a lane per unit of 32 weights, the activation staged in LDS; the integer tier of these kinds
-// (Q8_0 / Q8_K activations, crates/frink-quant/src/legacy_q8.rs, iq4_xs_q8.rs) is not built.
+// (Q8_0 / Q8_K activations, crates/frink-quant/src/legacy_q8.rs, iq4_xs_q8.rs) is the second half of this file.
 #include "frk_device.hpp"
 
 namespace frk {
@@ -157,6 +157,150 @@ __global__ __launch_bounds__(512) void gemv_units_f32_kernel(const uint8_t *__re
     }
 }
 
+// ---- the integer tier: Q5_0 and MXFP4 rows against Q8_0 activation blocks (dot_q5_0_q8 / dot_mxfp4_q8,
+// crates/frink-quant/src/legacy_q8.rs:169-213), IQ4_XS rows against Q8_K activations (dot_iq4_xs_q8_k,
+// crates/frink-quant/src/iq4_xs_q8.rs:67-98).  A unit decodes to 32 signed bytes (Q5_0: nibble | fifth bit << 4,
+// minus 16; MXFP4: the doubled E2M1 table, with the halved E8M0 scale; IQ4_XS: kvalues_iq4nl), four to a register,
+// and meets the activation's bytes in v_dot4: the integers are the reference's, the float step per block its
+// expression -- act.d[b] * (scale * isum) for the 32-element kinds, d * act.d[b] * sum(ls * s) per 256 for IQ4_XS.
+
+// bit k of the low four bits of b to bit 8k (k = 0..3): the four shifted copies do not overlap, so no carry
+__device__ __forceinline__ uint32_t spread4(uint32_t b) { return ((b & 0xfu) * 0x00204081u) & 0x01010101u; }
+// four 5-bit codes (one a byte) minus 16, as signed bytes: with 128 added first no byte borrows
+__device__ __forceinline__ uint32_t minus16_bytes(uint32_t c) { return ((c | 0x80808080u) - 0x10101010u) ^ 0x80808080u; }
+// kvalues_mxfp4 (E2M1 times two) of four 4-bit codes: 0 1 2 3 4 6 8 12, the code's bit 3 the sign
+__device__ __forceinline__ uint32_t mxfp4_x2_lookup4(uint32_t n) {
+    const uint32_t sel = n & 0x07070707u;
+    const uint32_t pos = perm8(0x0C080604u, 0x03020100u, sel);
+    const uint32_t neg = perm8(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+    const uint32_t m = ((n >> 3) & 0x01010101u) * 0xffu;
+    return (neg & m) | (pos & ~m);
+}
+// ggml_e8m0_to_fp32_half (legacy_q8.rs:154-161): 2^(e - 128), the two subnormal patterns for e < 2
+__device__ __forceinline__ float e8m0_half_scale(uint32_t e) { return __uint_as_float(e < 2 ? 0x00200000u << e : (e - 1) << 23); }
+
+// The 32 codes of unit u of a row held in LDS, as eight registers of four signed bytes: c[0..3] = elements 0..15,
+// c[4..7] = elements 16..31; `scale` = the unit's multiplier (Q5_0: d; MXFP4: the halved E8M0 scale; IQ4_XS: ls - 32
+// as an integer in scale_i, the block's d in scale).
+template <int KIND>
+__device__ __forceinline__ void unit_codes(const uint8_t *row, int u, uint32_t (&c)[8], float &scale, int &scale_i) {
+    scale_i = 1;
+    if (KIND == FRK_KIND_Q5_0) {
+        const uint8_t *blk = row + u * Q5_0_BYTES;  // 2-byte aligned
+        scale = h2f(load_u16(blk));
+        const uint32_t qh = load_u16(blk + 2) | (load_u16(blk + 4) << 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t q = load_u16(blk + 6 + 4 * i) | (load_u16(blk + 8 + 4 * i) << 16);
+            c[i] = minus16_bytes((q & 0x0f0f0f0fu) | (spread4(qh >> (4 * i)) << 4));
+            c[4 + i] = minus16_bytes(((q >> 4) & 0x0f0f0f0fu) | (spread4(qh >> (16 + 4 * i)) << 4));
+        }
+    } else if (KIND == FRK_KIND_IQ4_XS) {
+        const int b = u >> 3, ib = u & 7;
+        const uint8_t *blk = row + b * IQ4_XS_BYTES;  // 8-byte aligned
+        const uint32_t head = *reinterpret_cast<const uint32_t *>(blk), sl = *reinterpret_cast<const uint32_t *>(blk + 4);
+        scale = h2f(head & 0xffffu);
+        const uint32_t scales_h = head >> 16;
+        scale_i = (int)(((sl >> (8 * (ib >> 1) + 4 * (ib & 1))) & 0xf) | (((scales_h >> (2 * ib)) & 3) << 4)) - 32;
+        const uint2 qa = *reinterpret_cast<const uint2 *>(blk + 8 + ib * 16), qb = *reinterpret_cast<const uint2 *>(blk + 16 + ib * 16);
+        const uint32_t q[4] = {qa.x, qa.y, qb.x, qb.y};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            c[i] = iq4nl_lookup4(q[i] & 0x0f0f0f0fu);
+            c[4 + i] = iq4nl_lookup4((q[i] >> 4) & 0x0f0f0f0fu);
+        }
+    } else {  // MXFP4: 17-byte blocks, no alignment -- the sixteen code bytes out of five aligned words
+        const uint32_t at = (uint32_t)u * MXFP4_BYTES;
+        scale = e8m0_half_scale(row[at]);
+        const uint32_t *words = reinterpret_cast<const uint32_t *>(row) + ((at + 1) >> 2);
+        const uint32_t shift = (at + 1) & 3;  // (0: the fifth word is read and not used; the slot ends in slack for it)
+        const uint32_t g0 = words[0], g1 = words[1], g2 = words[2], g3 = words[3], g4 = words[4];
+        const uint32_t q[4] = {__builtin_amdgcn_alignbyte(g1, g0, shift), __builtin_amdgcn_alignbyte(g2, g1, shift),
+                               __builtin_amdgcn_alignbyte(g3, g2, shift), __builtin_amdgcn_alignbyte(g4, g3, shift)};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            c[i] = mxfp4_x2_lookup4(q[i] & 0x0f0f0f0fu);
+            c[4 + i] = mxfp4_x2_lookup4((q[i] >> 4) & 0x0f0f0f0fu);
+        }
+    }
+}
+
+// A wavefront per row, a lane per unit.  The quantized activation sits in LDS for the whole launch; a row's bytes go
+// global -> registers (whole 16-byte pieces, the next row's while this one is multiplied) -> the wavefront's own
+// LDS slot, from where the lanes pick their blocks apart (22- and 17-byte blocks have no alignment to load by).
+template <int KIND, int MAXP>
+__global__ __launch_bounds__(512) void gemv_units_int_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int cols,
+                                                            const int8_t *__restrict__ aq, const float *__restrict__ ad,
+                                                            float *__restrict__ y) {
+    extern __shared__ uint4 smem_kinds[];
+    uint8_t *lds = reinterpret_cast<uint8_t *>(smem_kinds);
+    const int units = cols / 32, nd = KIND == FRK_KIND_IQ4_XS ? cols / QK_K : units;
+    int8_t *sq = reinterpret_cast<int8_t *>(lds);
+    float *sd = reinterpret_cast<float *>(lds + cols);
+    const int pieces = (int)(row_stride / 16);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    typedef uint32_t piece_t __attribute__((ext_vector_type(4)));
+    piece_t *mine = reinterpret_cast<piece_t *>(lds + ((cols + nd * 4 + 15) & ~15)) + (size_t)wave * pieces;
+    for (int i = threadIdx.x; i < cols / 16; i += 512) reinterpret_cast<uint4 *>(sq)[i] = reinterpret_cast<const uint4 *>(aq)[i];
+    for (int i = threadIdx.x; i < nd; i += 512) sd[i] = ad[i];
+    // (a piece past the row's end: the row's last piece again, stored to the same place by the lanes that hold it;
+    // the array is only ever indexed by unrolled constants, and no lambda takes it: it stays in registers)
+    piece_t pre[MAXP];
+    const int step = (int)gridDim.x * 8;
+    int r = (int)blockIdx.x * 8 + wave;
+    {
+        const piece_t *src = reinterpret_cast<const piece_t *>(W + (size_t)min(r, rows - 1) * row_stride);
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) pre[p] = src[min(lane + 64 * p, pieces - 1)];
+    }
+    __syncthreads();
+    for (; r < rows; r += step) {
+#pragma unroll
+        for (int p = 0; p < MAXP; p++) mine[min(lane + 64 * p, pieces - 1)] = pre[p];
+        {
+            const piece_t *src = reinterpret_cast<const piece_t *>(W + (size_t)min(r + step, rows - 1) * row_stride);
+#pragma unroll
+            for (int p = 0; p < MAXP; p++) pre[p] = src[min(lane + 64 * p, pieces - 1)];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint8_t *row = reinterpret_cast<const uint8_t *>(mine);
+        float acc = 0.0f;
+        for (int u0 = 0; u0 < units; u0 += 64) {  // (uniform: the lanes of an IQ4_XS block exchange their sums)
+            const bool live = u0 + lane < units;
+            const int u = live ? u0 + lane : units - 1;
+            uint32_t c[8];
+            float scale;
+            int scale_i;
+            unit_codes<KIND>(row, u, c, scale, scale_i);
+            const uint4 a0 = *reinterpret_cast<const uint4 *>(sq + u * 32), a1 = *reinterpret_cast<const uint4 *>(sq + u * 32 + 16);
+            int isum = 0;
+            isum = dot4(c[0], a0.x, isum);
+            isum = dot4(c[1], a0.y, isum);
+            isum = dot4(c[2], a0.z, isum);
+            isum = dot4(c[3], a0.w, isum);
+            isum = dot4(c[4], a1.x, isum);
+            isum = dot4(c[5], a1.y, isum);
+            isum = dot4(c[6], a1.z, isum);
+            isum = dot4(c[7], a1.w, isum);
+            if (KIND == FRK_KIND_IQ4_XS) {
+                int t = live ? scale_i * isum : 0;  // |ls| <= 32, |s| <= 32 * 127 * 127: fits
+                t += __shfl_xor(t, 1);
+                t += __shfl_xor(t, 2);
+                t += __shfl_xor(t, 4);
+                if (live && (u & 7) == 0) acc += scale * sd[u >> 3] * (float)t;
+            } else if (live) {
+                acc += sd[u] * (scale * (float)isum);
+            }
+        }
+        acc = part_sum<64>(acc);
+        if (lane == 0) y[r] = acc;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();  // (the slot is rewritten at the top of the loop)
+    }
+}
+
 #define FRK_LAUNCH_CHECK(what)                                                                          \
     do {                                                                                                \
         hipError_t e_ = hipGetLastError();                                                              \
@@ -192,6 +336,45 @@ int launch_gemv_units_f32(const frk_weights *w, const float *x, float *y, hipStr
 #undef FRK_GO
     FRK_LAUNCH_CHECK("gemv_units_f32");
     return FRK_OK;
+}
+
+// y = W x on the integer tier: aq / ad are the activation's Q8_0 blocks (Q5_0, MXFP4) or its Q8_K quants and
+// block scales (IQ4_XS)
+size_t gemv_units_int_lds(const frk_weights *w) {
+    const size_t nd = w->kind == FRK_KIND_IQ4_XS ? w->cols / QK_K : w->cols / 32;
+    return ((w->cols + nd * 4 + 15) & ~(size_t)15) + 8 * w->layout.row_stride + 16;  // (16 bytes of slack behind the last slot)
+}
+bool gemv_units_int_fits(const frk_weights *w) { return gemv_units_int_lds(w) <= 160 * 1024 && w->layout.row_stride <= 12 * 1024; }
+template <int KIND, int MAXP>
+static int launch_gemv_units_int_as(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    const size_t shmem = gemv_units_int_lds(w);
+    static size_t sized = 0;  // a benign race: every thread raises the same attribute
+    if (shmem > sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_units_int_kernel<KIND, MAXP>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv units int): %s", hipGetErrorString(e));
+        sized = 160 * 1024;
+    }
+    const unsigned grid = (unsigned)std::min<size_t>((w->rows + 7) / 8, 2048);
+    hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP>), dim3(grid), dim3(512), shmem, s, w->dev, w->layout.row_stride, (int)w->rows,
+                       (int)w->cols, aq, ad, y);
+    FRK_LAUNCH_CHECK("gemv_units_int");
+    return FRK_OK;
+}
+template <int KIND>
+static int launch_gemv_units_int_kind(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    const size_t per_lane = (w->layout.row_stride / 16 + 63) / 64;
+    if (per_lane <= 3) return launch_gemv_units_int_as<KIND, 3>(w, aq, ad, y, s);
+    if (per_lane <= 6) return launch_gemv_units_int_as<KIND, 6>(w, aq, ad, y, s);
+    return launch_gemv_units_int_as<KIND, 12>(w, aq, ad, y, s);
+}
+int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    if (!gemv_units_int_fits(w))
+        return set_error(FRK_ERR_UNSUPPORTED, "the integer GEMV of quant kind %d takes rows of at most %d bytes (%zu columns)", w->kind,
+                         12 * 1024, w->cols);
+    if (w->kind == FRK_KIND_Q5_0) return launch_gemv_units_int_kind<FRK_KIND_Q5_0>(w, aq, ad, y, s);
+    if (w->kind == FRK_KIND_IQ4_XS) return launch_gemv_units_int_kind<FRK_KIND_IQ4_XS>(w, aq, ad, y, s);
+    return launch_gemv_units_int_kind<FRK_KIND_MXFP4>(w, aq, ad, y, s);
 }
 
 }  // namespace frk

@@ -477,6 +477,29 @@ static int quantize_acts_q8_k(const frk_weights *w, const float *x, size_t batch
     return FRK_OK;
 }
 
+// The integer tier of Q5_0 / MXFP4 (the activation as Q8_0 blocks: q8_row_dot, crates/frink-core/src/weight_matrix.rs:
+// 392-407) and of IQ4_XS (as Q8_K: q8k_row_dot, :415-420): one activation row quantized into the call's scratch
+// memory, then the integer GEMV.
+static int gemv_units_int(const frk_weights *w, const float *x, float *y, hipStream_t s, Scratch &scratch) {
+    if (!gemv_units_int_fits(w))
+        return set_error(FRK_ERR_UNSUPPORTED, "the integer GEMV of quant kind %d does not take rows of %zu columns", w->kind, w->cols);
+    if (w->kind == FRK_KIND_IQ4_XS) {
+        Q8KActs a;
+        int rc = quantize_acts_q8_k(w, x, 1, s, scratch, &a);
+        if (rc) return rc;
+        return launch_gemv_units_int(w, a.q, a.d, y, s);
+    }
+    const size_t n = w->cols;
+    void *ws = nullptr;
+    int rc = scratch.get(round_up(n, 256) + n / 32 * 4, s, &ws);
+    if (rc) return rc;
+    int8_t *q = (int8_t *)ws;
+    float *d = (float *)((char *)ws + round_up(n, 256));
+    rc = launch_quantize_q8_0(x, n, q, d, s);
+    if (rc) return rc;
+    return launch_gemv_units_int(w, q, d, y, s);
+}
+
 static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mode, hipStream_t s, Scratch &scratch) {
     if (act_mode == FRK_ACT_F32_DOT && (w->kind == FRK_KIND_Q4_K || w->kind == FRK_KIND_Q5_K || w->kind == FRK_KIND_Q6_K)) {
         if (!kquant_f32_gemv_fits(w))
@@ -485,9 +508,8 @@ static int gemv_impl(const frk_weights *w, const float *x, float *y, int act_mod
     }
     if (act_mode == FRK_ACT_F32_DOT) act_mode = FRK_ACT_F32;  // (Q8_0 and Q4_0: their FRK_ACT_F32 is the f32 dot)
     if (is_unit_kind(w->kind)) {
-        if (act_mode != FRK_ACT_F32)
-            return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has the f32-dot GEMV only", w->kind);
-        return launch_gemv_units_f32(w, x, y, s);
+        if (act_mode == FRK_ACT_F32) return launch_gemv_units_f32(w, x, y, s);
+        return gemv_units_int(w, x, y, s, scratch);
     }
     switch (w->kind) {
     case FRK_KIND_Q4_K:

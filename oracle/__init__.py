@@ -54,10 +54,19 @@ def lib():
             "fo_dot_q4_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q5_k_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_dot_q6_k_f32": (C.c_float, [u8p, sz, f32p]),
+            "fo_dot_q5_0_f32": (C.c_float, [u8p, sz, f32p]),
+            "fo_dot_iq4_xs_f32": (C.c_float, [u8p, sz, f32p]),
+            "fo_dot_mxfp4_f32": (C.c_float, [u8p, sz, f32p]),
             "fo_quantize_q8_k": (None, [f32p, sz, i8p, f32p, i16p]),
             "fo_quantize_q8_0": (None, [f32p, sz, C.c_int, i8p, f32p]),
             "fo_dot_q8_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
             "fo_dot_q4_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
+            "fo_dot_q5_0_q8": (C.c_float, [u8p, sz, i8p, f32p]),
+            "fo_dot_mxfp4_q8": (C.c_float, [u8p, sz, i8p, f32p]),
+            "fo_dot_iq4_xs_q8k": (C.c_float, [u8p, sz, i8p, f32p]),
+            "fo_decode_q5_0_block": (None, [u8p, i8p]),
+            "fo_decode_mxfp4_block": (None, [u8p, i8p]),
+            "fo_e8m0_half_scale": (C.c_float, [C.c_uint8]),
             "fo_dot_q4_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
             "fo_dot_q5_k_q8k": (C.c_float, [u8p, sz, i8p, f32p, i16p]),
             "fo_dot_q6_k_q8k": (C.c_float, [u8p, sz, i8p, f32p]),
@@ -131,7 +140,8 @@ def element(kind, block, i):
 def dot_f32(kind, row, x):
     row, x = _u8(row), _f32(x)
     fn = {Q4_0: lib().fo_dot_q4_0_f32, Q8_0: lib().fo_dot_q8_0_f32, Q4_K: lib().fo_dot_q4_k_f32, Q5_K: lib().fo_dot_q5_k_f32,
-          Q6_K: lib().fo_dot_q6_k_f32}[kind]
+          Q6_K: lib().fo_dot_q6_k_f32, Q5_0: lib().fo_dot_q5_0_f32, IQ4_XS: lib().fo_dot_iq4_xs_f32,
+          MXFP4: lib().fo_dot_mxfp4_f32}[kind]
     return fn(_p(row, C.c_uint8), row.size, _p(x, C.c_float))
 
 
@@ -156,11 +166,14 @@ def quantize_q8_0(x, form=FORM_AVX):
 
 def dot_int(kind, row, acts):
     row = _u8(row)
-    if kind in (Q8_0, Q4_0):
+    if kind in (Q8_0, Q4_0, Q5_0, MXFP4):
         q, d = acts
-        fn = lib().fo_dot_q8_0_q8 if kind == Q8_0 else lib().fo_dot_q4_0_q8
+        fn = {Q8_0: lib().fo_dot_q8_0_q8, Q4_0: lib().fo_dot_q4_0_q8, Q5_0: lib().fo_dot_q5_0_q8,
+              MXFP4: lib().fo_dot_mxfp4_q8}[kind]
         return fn(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
     q, d, bs = acts
+    if kind == IQ4_XS:
+        return lib().fo_dot_iq4_xs_q8k(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float))
     if kind in (Q4_K, Q5_K):
         fn = lib().fo_dot_q4_k_q8k if kind == Q4_K else lib().fo_dot_q5_k_q8k
         return fn(_p(row, C.c_uint8), row.size, _p(q, C.c_int8), _p(d, C.c_float), _p(bs, C.c_int16))

@@ -634,6 +634,97 @@ float fo_dot_q4_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, cons
     return acc;
 }
 
+/* ---- the 32-element block kinds against Q8_0 activation blocks (crates/frink-quant/src/legacy_q8.rs) ----
+ * One body (dot_scalar<B>, :169-184) over a per-kind decoder (Block::decode, :63-86) and scale (Block::scale,
+ * :58-60): a block contributes act.d[b] * (scale * isum as f32).
+ * parity unpinned: the reference holds no numeric vector for these dots; the tests pin them through the
+ * dequantizers (decoded integer x scale == the dequantized value, bit for bit, for every code and every
+ * E8M0 scale byte) and through exact integer arithmetic on random blocks. */
+/* legacy_q8.rs:108-116 with q5_fifth_bits (src/lib.rs:4346-4350): w = (nibble | fifth << 4) - 16 */
+void fo_decode_q5_0_block(const uint8_t *blk, int8_t *w) {
+    uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+    const uint8_t *qs = blk + 6;
+    for (int j = 0; j < 16; j++) {
+        uint8_t xh0, xh1;
+        q5_fifth_bits(qh, j, &xh0, &xh1);
+        w[j] = (int8_t)((int)((qs[j] & 0x0F) | xh0) - 16);
+        w[j + 16] = (int8_t)((int)((qs[j] >> 4) | xh1) - 16);
+    }
+}
+/* legacy_q8.rs:150 (ggml's kvalues_mxfp4: E2M1 times two) */
+static const int8_t KVALUES_MXFP4_X2[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+/* legacy_q8.rs:154-161 (ggml_e8m0_to_fp32_half): 2^(e - 128), the two subnormal patterns for e < 2 */
+float fo_e8m0_half_scale(uint8_t e) {
+    uint32_t bits = e < 2 ? (0x00200000u << e) : ((uint32_t)(e - 1) << 23);
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+/* legacy_q8.rs:133-147: codes through the doubled E2M1 table, low nibble -> element j, high -> j + 16 */
+void fo_decode_mxfp4_block(const uint8_t *blk, int8_t *w) {
+    for (int j = 0; j < 16; j++) {
+        w[j] = KVALUES_MXFP4_X2[blk[1 + j] & 0xf];
+        w[j + 16] = KVALUES_MXFP4_X2[blk[1 + j] >> 4];
+    }
+}
+static float dot_legacy_q8(int kind, const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d) {
+    size_t bb = kind == FO_KIND_Q5_0 ? Q5_0_BYTES : MXFP4_BYTES, nb = row_bytes / bb;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * bb;
+        int8_t w[32];
+        float scale;
+        if (kind == FO_KIND_Q5_0) {
+            fo_decode_q5_0_block(blk, w);
+            scale = rd_f16(blk);
+        } else {
+            fo_decode_mxfp4_block(blk, w);
+            scale = fo_e8m0_half_scale(blk[0]);
+        }
+        int32_t isum = 0;
+        for (int i = 0; i < 32; i++) isum += (int32_t)w[i] * (int32_t)q[b * 32 + i];
+        float block_acc = scale * (float)isum;
+        acc += d[b] * block_acc;
+    }
+    return acc;
+}
+/* legacy_q8.rs:210 (dot_q5_0_q8_scalar) */
+float fo_dot_q5_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d) {
+    return dot_legacy_q8(FO_KIND_Q5_0, row, row_bytes, q, d);
+}
+/* legacy_q8.rs:213 (dot_mxfp4_q8_scalar) */
+float fo_dot_mxfp4_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d) {
+    return dot_legacy_q8(FO_KIND_MXFP4, row, row_bytes, q, d);
+}
+/* crates/frink-quant/src/iq4_xs_q8.rs:40-45 (sub_scale) and :67-98 (dot_iq4_xs_q8_k_scalar): per block the
+ * integer sum of (ls - 32) * (codebook . q8) over the eight sub-blocks, then d * act.d[b] * sumi.
+ * parity unpinned, as above: pinned through the dequantizer and exact integers. */
+float fo_dot_iq4_xs_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *dact) {
+    size_t nb = row_bytes / IQ4_XS_BYTES;
+    float acc = 0.0f;
+    for (size_t b = 0; b < nb; b++) {
+        const uint8_t *blk = row + b * IQ4_XS_BYTES;
+        float d = rd_f16(blk);
+        unsigned scales_h = (unsigned)blk[2] | ((unsigned)blk[3] << 8);
+        const uint8_t *scales_l = blk + 4, *qs = blk + 8;
+        const int8_t *q8 = q + b * QK_K;
+        int32_t sumi = 0;
+        for (int ib = 0; ib < 8; ib++) {
+            int32_t lo = (scales_l[ib / 2] >> (4 * (ib % 2))) & 0xf, hi = (scales_h >> (2 * ib)) & 3;
+            int32_t ls = (lo | (hi << 4)) - 32;
+            int32_t s = 0;
+            for (int j = 0; j < 16; j++) {
+                uint8_t byte = qs[ib * 16 + j];
+                s += (int32_t)KVALUES_IQ4NL[byte & 0xf] * (int32_t)q8[ib * 32 + j];
+                s += (int32_t)KVALUES_IQ4NL[byte >> 4] * (int32_t)q8[ib * 32 + 16 + j];
+            }
+            sumi += ls * s;
+        }
+        acc += d * dact[b] * (float)sumi;
+    }
+    return acc;
+}
+
 /* src/lib.rs:822-869 */
 float fo_dot_q4_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *dact,
                       const int16_t *bsums_all) {
@@ -1136,8 +1227,9 @@ int fo_encode_matrix(int kind, const float *src, size_t rows, size_t cols, uint8
 /* ---- dispatch-level restatement ----
  * WeightMatrix::apply_cpu / apply_batch_with_acts (frink-core/src/weight_matrix.rs:1716-2073,
  * 2481-3365): out[b*rows + r] = dot(row r, activation b); int-dot tier quantizes each
- * activation row once (Q8_K for the K-quants, Q8_0 host form for Q8_0; an x86 host with AVX
- * takes the Avx form, src/act_quant.rs:129-148). */
+ * activation row once (Q8_K for the K-quants and IQ4_XS, Q8_0 host form for Q8_0, Q4_0, Q5_0 and MXFP4 --
+ * q8k_row_dot / q8_row_dot, weight_matrix.rs:392-420; an x86 host with AVX takes the Avx form,
+ * src/act_quant.rs:129-148). */
 typedef struct {
     int8_t *q;
     float *d;
@@ -1148,7 +1240,7 @@ static int acts_alloc(acts_t *a, int kind, size_t cols, size_t batch) {
     size_t be = (size_t)fo_block_elems(kind);
     a->q = (int8_t *)malloc(batch * cols);
     a->d = (float *)malloc(batch * (cols / be) * sizeof(float));
-    int q8_0_acts = kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0;
+    int q8_0_acts = kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0 || kind == FO_KIND_Q5_0 || kind == FO_KIND_MXFP4;
     a->bsums = q8_0_acts ? NULL : (int16_t *)malloc(batch * (cols / 16) * sizeof(int16_t));
     return a->q && a->d && (q8_0_acts || a->bsums) ? 0 : -1;
 }
@@ -1157,7 +1249,7 @@ static void acts_free(acts_t *a) { free(a->q); free(a->d); free(a->bsums); }
 static void acts_quantize(acts_t *a, int kind, const float *x, size_t cols, size_t batch) {
     size_t be = (size_t)fo_block_elems(kind);
     for (size_t b = 0; b < batch; b++) {
-        if (kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0)
+        if (kind == FO_KIND_Q8_0 || kind == FO_KIND_Q4_0 || kind == FO_KIND_Q5_0 || kind == FO_KIND_MXFP4)
             fo_quantize_q8_0(x + b * cols, cols, FO_Q8_0_FORM_AVX, a->q + b * cols, a->d + b * (cols / be));
         else
             fo_quantize_q8_k(x + b * cols, cols, a->q + b * cols, a->d + b * (cols / be),
@@ -1173,6 +1265,9 @@ static inline float row_dot_int(int kind, const uint8_t *row, size_t row_bytes, 
     switch (kind) {
     case FO_KIND_Q8_0: return fo_dot_q8_0_q8(row, row_bytes, q, d);
     case FO_KIND_Q4_0: return fo_dot_q4_0_q8(row, row_bytes, q, d);
+    case FO_KIND_Q5_0: return fo_dot_q5_0_q8(row, row_bytes, q, d);
+    case FO_KIND_MXFP4: return fo_dot_mxfp4_q8(row, row_bytes, q, d);
+    case FO_KIND_IQ4_XS: return fo_dot_iq4_xs_q8k(row, row_bytes, q, d);
     case FO_KIND_Q4_K: return fo_dot_q4_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
     case FO_KIND_Q5_K: return fo_dot_q5_k_q8k(row, row_bytes, q, d, a->bsums + b * (cols / 16));
     default: return fo_dot_q6_k_q8k(row, row_bytes, q, d);
@@ -1197,8 +1292,6 @@ int fo_gemm_rows(int kind, const uint8_t *w, size_t rows, size_t cols, size_t ro
     if (!be || cols == 0 || cols % (size_t)be || row0 + nrows > rows) return -1;
     size_t row_bytes = cols / (size_t)be * (size_t)bb;
     threads = pick_threads(threads);
-    /* (the integer tier of these kinds, crates/frink-quant/src/legacy_q8.rs and iq4_xs_q8.rs, is not restated) */
-    if (mode == FO_MODE_INT_DOT && (kind == FO_KIND_Q5_0 || kind == FO_KIND_IQ4_XS || kind == FO_KIND_MXFP4)) return -4;
     acts_t a = {0, 0, 0};
     if (mode == FO_MODE_INT_DOT) {
         if (acts_alloc(&a, kind, cols, batch)) { acts_free(&a); return -3; }

@@ -71,6 +71,14 @@ void fo_quantize_q8_0(const float *x, size_t n, int form, int8_t *q, float *d);
 /* integer dots against quantized activations */
 float fo_dot_q8_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
 float fo_dot_q4_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
+/* legacy_q8.rs: Q5_0 and GGUF MXFP4 rows against Q8_0 activation blocks; the decoders and the halved E8M0 scale */
+void fo_decode_q5_0_block(const uint8_t *blk, int8_t *w32);
+void fo_decode_mxfp4_block(const uint8_t *blk, int8_t *w32);
+float fo_e8m0_half_scale(uint8_t e);
+float fo_dot_q5_0_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
+float fo_dot_mxfp4_q8(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d);
+/* iq4_xs_q8.rs: IQ4_XS rows against Q8_K activations (q, d per 256; the 16-wide sums are not used) */
+float fo_dot_iq4_xs_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *dact);
 float fo_dot_q4_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d,
                       const int16_t *bsums);
 float fo_dot_q5_k_q8k(const uint8_t *row, size_t row_bytes, const int8_t *q, const float *d,

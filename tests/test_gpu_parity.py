@@ -1133,8 +1133,39 @@ def test_other_kinds_gemv_matches_the_oracle(fa, kind, rows, cols, batch):
     deq = fo.dequant(kind, data).reshape(rows, cols).astype(np.float64)
     bound = 4e-6 * (np.abs(deq) @ np.abs(x.T).astype(np.float64)).T
     assert (np.abs(got - (deq @ x.T.astype(np.float64)).T) <= bound).all()
+    w.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols", [
+    (fo.Q5_0, 70, 1024), (fo.Q5_0, 300, 4096), (fo.Q5_0, 17, 96), (fo.Q5_0, 9, 16384), (fo.Q5_0, 2100, 512),
+    (fo.IQ4_XS, 70, 1024), (fo.IQ4_XS, 130, 4096), (fo.IQ4_XS, 9, 16384), (fo.IQ4_XS, 5, 256), (fo.IQ4_XS, 33, 4352),
+    (fo.MXFP4, 70, 1024), (fo.MXFP4, 64, 2880), (fo.MXFP4, 9, 16384), (fo.MXFP4, 5, 32),
+])
+def test_other_kinds_integer_gemv_matches_the_oracle(fa, kind, rows, cols):
+    """FRK_ACT_INT8 on Q5_0 / MXFP4 (the activation as Q8_0 blocks: dot_q5_0_q8 / dot_mxfp4_q8) and IQ4_XS (as Q8_K:
+    dot_iq4_xs_q8_k): rows of one block and of 512, more rows than one round of workgroups, unit counts that are
+    not a multiple of 64 (the lanes of a wavefront's last round idle), the subnormal MXFP4 scales."""
+    from frink_amd import synth
+    print("other kinds, integer tier", kind, rows, cols, flush=True)
+    data = _other_kind_blocks(kind, rows, cols, seed=kind * 5 + rows)
+    x = synth.activations(rows + cols + 1, 1, cols, outlier_frac=0.01)[0]
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    got = w.gemv(to_dev(x), act_mode=fa.ACT_INT8).cpu().numpy()
+    want = fo.gemv(kind, data, rows, cols, x, fo.INT_DOT)
+    assert_rows_close(got[None], want[None], "integer gemv kind %d %dx%d" % (kind, rows, cols))
+    # the integers are exact and the float step is a handful of operations a block: far inside the tolerance
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+    # homogeneity: a power of two on the activation scales its Q8 scales exactly and leaves the quants alone
+    y4 = w.gemv(to_dev(x * np.float32(4.0)), act_mode=fa.ACT_INT8).cpu().numpy()
+    assert np.array_equal(bits(y4), bits(got * np.float32(4.0)))
+    w.release()
+
+
+def test_other_kinds_integer_gemv_refuses_rows_it_cannot_hold(fa):
+    data = _other_kind_blocks(fo.Q5_0, 2, 32768, seed=1)
+    w = fa.Weights.from_host(fo.Q5_0, data, 2, 32768)
     with pytest.raises(fa.BackendError) as e:
-        w.gemv(to_dev(x[0]), act_mode=fa.ACT_INT8)
+        w.gemv(to_dev(np.zeros(32768, np.float32)), act_mode=fa.ACT_INT8)
     assert e.value.code == fa.ERR_UNSUPPORTED
     w.release()
 

@@ -472,11 +472,11 @@ def test_exact_rebuilds_agree_with_the_dequantizers():
 # ---------------------------------------------------------------- dispatch level
 # crates/frink-core/src/weight_matrix.rs:4747-5350: apply_batch == N x apply; out is [batch][rows]
 
-@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K])
+@pytest.mark.parametrize("kind", [fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K, fo.Q5_0, fo.IQ4_XS, fo.MXFP4])
 @pytest.mark.parametrize("mode", [fo.F32_DOT, fo.INT_DOT])
 def test_gemm_is_batch_times_gemv_and_output_is_batch_major(kind, mode):
     rows, cols, batch = 24, 512, 5
-    data = _weights(kind, rows, cols)
+    data = _weights(kind, rows, cols) if kind in (fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K) else _random_blocks(kind, rows * cols // fo.BLOCK[kind][1], 77).ravel()
     x = RNG.standard_normal((batch, cols)).astype(np.float32)
     y = fo.gemm(kind, data, rows, cols, x, mode, threads=3)
     assert y.shape == (batch, rows)
@@ -752,5 +752,77 @@ def test_f32_dots_of_the_other_kinds_are_the_dequantized_dot(kind):
                     acc = np.float32(acc + deq[r, 32 * g + j] * x[32 * g + j])
                     acc = np.float32(acc + deq[r, 32 * g + 16 + j] * x[32 * g + 16 + j])
         assert got[r] == acc
-    with pytest.raises(ValueError):
-        fo.gemv(kind, blocks.ravel(), 6, cols, x, fo.INT_DOT, 1)
+
+
+def test_the_integer_tiers_decoders_are_the_dequantizers_values():
+    """legacy_q8.rs:108-161: a Q5_0 / MXFP4 block decodes to 32 small integers and one scale whose product is the
+    dequantized value -- bit for bit, for every code, every fifth bit and every E8M0 scale byte (the doubled E2M1 table
+    goes with the HALVED scale 2^(e - 128), subnormal patterns for e < 2 included)."""
+    import ctypes as C
+    L = fo.lib()
+    w = np.zeros(32, np.int8)
+    # MXFP4: every scale byte x every code (255 is not a finite scale)
+    for e in range(255):
+        blk = np.concatenate([[e], (np.arange(16) * 17) % 256]).astype(np.uint8)  # byte j = code j in both nibbles
+        L.fo_decode_mxfp4_block(blk.ctypes.data_as(C.POINTER(C.c_uint8)), w.ctypes.data_as(C.POINTER(C.c_int8)))
+        half = np.float32(L.fo_e8m0_half_scale(e))
+        assert half == np.float32(2.0) ** np.float32(e - 128) or e < 2
+        got, want = w.astype(np.float32) * half, fo.dequant(fo.MXFP4, blk)
+        # (code 8 is -0.0 in the E2M1 table and the integer 0 here: equal as values, which is all a dot can see)
+        nz = want != 0
+        assert np.array_equal(got, want) and np.array_equal(got[nz].view(np.uint32), want[nz].view(np.uint32)), e
+    assert np.float32(L.fo_e8m0_half_scale(0)).view(np.uint32) == 0x00200000 and np.float32(L.fo_e8m0_half_scale(1)).view(np.uint32) == 0x00400000
+    assert w.tolist()[:16] == [0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12]
+    # Q5_0: random blocks, scale 1.0 so that the dequantized values are the integers themselves
+    blocks = _random_blocks(fo.Q5_0, 200, 21)
+    blocks[:, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    deq = fo.dequant(fo.Q5_0, blocks.ravel()).reshape(200, 32)
+    for b in range(200):
+        L.fo_decode_q5_0_block(blocks[b].ctypes.data_as(C.POINTER(C.c_uint8)), w.ctypes.data_as(C.POINTER(C.c_int8)))
+        assert np.array_equal(w.astype(np.float32), deq[b]) and w.min() >= -16 and w.max() <= 15
+
+
+@pytest.mark.parametrize("kind", [fo.Q5_0, fo.MXFP4, fo.IQ4_XS])
+def test_the_other_kinds_integer_dots_in_exact_arithmetic(kind):
+    """dot_q5_0_q8 / dot_mxfp4_q8 (legacy_q8.rs:169-213, Q8_0 activation blocks) and dot_iq4_xs_q8_k
+    (iq4_xs_q8.rs:67-98, Q8_K activations): the dot of the dequantized row with the dequantized activation, to f32
+    rounding of a handful of operations per block -- exact integers inside a block, so a wrong element order, sign,
+    sub-scale or scale shows at once.  And the reference's own invariant: within 5 % of the f32 dot."""
+    bb, be = fo.BLOCK[kind]
+    cols, rows = 1024, 8
+    blocks = _random_blocks(kind, rows * cols // be, 31 + kind).reshape(rows, -1)
+    x = np.random.default_rng(100 + kind).standard_normal(cols).astype(np.float32)
+    if kind == fo.IQ4_XS:
+        q, d, bs = fo.quantize_q8_k(x)
+        acts = (q, d, bs)
+        xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), 256)
+    else:
+        q, d = fo.quantize_q8_0(x)
+        acts = (q, d)
+        xa = q.astype(np.float64) * np.repeat(d.astype(np.float64), 32)
+    for r in range(rows):
+        w = fo.dequant(kind, blocks[r]).astype(np.float64)
+        want = float(np.dot(w, xa))
+        got = fo.dot_int(kind, blocks[r], acts)
+        assert abs(got - want) <= 2e-6 * float(np.abs(w * xa).sum())
+        f32 = fo.dot_f32(kind, blocks[r], x)
+        assert abs(got - f32) <= 0.05 * max(abs(f32), float(np.abs(w * xa).sum()) / np.sqrt(cols))
+    # the dispatch level takes the same functions: gemv in integer mode, every row
+    y = fo.gemv(kind, blocks.ravel(), rows, cols, x, fo.INT_DOT, 1)
+    for r in range(rows):
+        assert np.float32(fo.dot_int(kind, blocks[r], acts)).view(np.uint32) == y[r].view(np.uint32)
+    # float order of one row, one operation at a time (scale * isum first, then the activation's scale)
+    blk = blocks[0].reshape(-1, bb)
+    acc = np.float32(0)
+    if kind != fo.IQ4_XS:
+        for b in range(cols // 32):
+            wq = np.rint(fo.dequant(kind, blk[b]).astype(np.float64) / _unit_scale(kind, blk[b])).astype(np.int64)
+            isum = int(np.dot(wq, q[32 * b:32 * b + 32].astype(np.int64)))
+            acc = np.float32(acc + np.float32(d[b] * np.float32(np.float32(_unit_scale(kind, blk[b])) * np.float32(isum))))
+        assert np.float32(fo.dot_int(kind, blocks[0], acts)).view(np.uint32) == acc.view(np.uint32)
+
+
+def _unit_scale(kind, blk):
+    if kind == fo.Q5_0:
+        return float(blk[0:2].copy().view(np.float16)[0])
+    return float(np.float32(fo.lib().fo_e8m0_half_scale(int(blk[0]))))
