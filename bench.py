@@ -77,7 +77,9 @@ def random_blocks(kind, rows, cols, seed):
         data[:, 2:4] = f16(1e-3, 3e-3)
     elif kind == 14:    # Q6_K: d
         data[:, 208:210] = f16(2e-5, 6e-5)
-    else:               # Q8_0, Q4_0: d
+    elif kind == 39:    # MXFP4: an E8M0 scale byte, 2^-10 .. 2^-6
+        data[:, 0] = rng.integers(118, 123, nb)
+    else:               # Q8_0, Q4_0, Q5_0, IQ4_XS: d
         data[:, 0:2] = f16(3e-4, 6e-4)
     return data.reshape(-1)
 
@@ -430,6 +432,22 @@ def main():
                                "frac_of_hbm_peak": round(d2.numel() / (t / 1600) / 1e9 / HBM_PEAK_GBS, 4)}
                 for w in w2:
                     w.release()
+            # the other kinds behind the seam, 14336x4096: the f32 dot of the reference's decode path and the integer tier
+            for name_o, k2 in (("Q5_0", fa.Q5_0), ("IQ4_XS", fa.IQ4_XS), ("MXFP4", fa.MXFP4)):
+                d2 = torch.from_numpy(random_blocks(k2, 14336, 4096, seed=91)).to(dev)
+                n_copies = max(COPIES, -(-560_000_000 // d2.numel()))
+                w2 = [fa.Weights.from_device(k2, d2, 14336, 4096) for _ in range(n_copies)]
+                x2 = torch.from_numpy(synth.activations(5, 1, 4096)[0]).to(dev)
+                y2 = torch.empty(14336, dtype=torch.float32, device=dev)
+                for mode, label in ((fa.ACT_F32, "f32 dot"), (fa.ACT_INT8, "integer tier, with its quantization launch")):
+                    def step2o(i):
+                        w2[i % n_copies].gemv(x2, out=y2, act_mode=mode)
+                    _, t = timed(step2o, 800, 25 * n_copies)
+                    extra["%s GEMV 14336x4096 (%s)" % (name_o, label)] = {
+                        "GBs": round(d2.numel() / (t / 800) / 1e9, 1), "us_per_step": round(t / 800 * 1e6, 3),
+                        "frac_of_hbm_peak": round(d2.numel() / (t / 800) / 1e9 / HBM_PEAK_GBS, 4)}
+                for w in w2:
+                    w.release()
         if want('gemm'):
             # prefill GEMM M=512 on the int8 matrix cores: 2*M*rows*cols integer ops per step.  The step is
             # the activations' quantization + the GEMM kernel; the kernel alone is timed over activations
@@ -516,6 +534,21 @@ def main():
                                                    "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
             for w in w40:
                 w.release()
+            del d40
+            # Q5_0 and MXFP4 batches: decoded into the Q8_0 planar form in scratch memory, then the Q8_0 kernel
+            for kind_o, name_o in ((fa.Q5_0, "Q5_0"), (fa.MXFP4, "MXFP4")):
+                do = torch.from_numpy(random_blocks(kind_o, cols, rows, seed=85)).to(dev)
+                wo = [fa.Weights.from_device(kind_o, do, cols, rows) for _ in range(4)]
+
+                def step3f(i):
+                    wo[i % 4].gemm(xb6, out=yb6)
+                _, t = timed(step3f, 40, 20)
+                tops = 2.0 * 512 * rows * cols / (t / 40) / 1e12
+                extra["%s GEMM M=512 4096x14336 (decoded to int8 planes per call)" % name_o] = {
+                    "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+                for w in wo:
+                    w.release()
+                del do
         if want('moe'):
             # MoE layer: 128 experts, top-8, hidden 2048, ffn 768, 512 tokens (routing done beforehand)
             E, K, H, F, T = 128, 8, 2048, 768, 512

@@ -338,8 +338,20 @@ size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows) {
 }
 
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
-    if (M > (size_t)1 << 30 || w->rows > (size_t)1 << 30)
-        return set_error(FRK_ERR_SHAPE, "gemm_q8_0: %zu activation rows x %zu weight rows is too many", M, w->rows);
+    return launch_gemm_q8_0_planar(w->dev, w->layout.row_stride, w->layout.off_a, w->rows, w->cols, w->kind == FRK_KIND_Q4_0, x, M, y,
+                                   ws, s);
+}
+
+// The same over any rows in the planar form -- quants [nb][32] (q4: nibbles [nb][16]), then the f16 scales [nb] at
+// off_d of every row: the resident Q8_0 / Q4_0 matrices, and other 32-element kinds decoded into that form.
+int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, bool q4, const float *x,
+                            size_t M, float *y, void *ws, hipStream_t s) {
+    if (M > (size_t)1 << 30 || rows > (size_t)1 << 30)
+        return set_error(FRK_ERR_SHAPE, "gemm_q8_0: %zu activation rows x %zu weight rows is too many", M, rows);
+    struct {
+        size_t rows, cols;
+    } dims = {rows, cols};
+    const auto *w = &dims;
     int8_t *aq = (int8_t *)ws;
     uint16_t *ad = (uint16_t *)((char *)ws + round_up(M * w->cols, 256));
     const size_t n_blocks = M * (w->cols / 32);
@@ -347,9 +359,9 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
                        (int)(w->cols / 32), aq, ad);
     FRK_LAUNCH_CHECK("quantize_q8_0_gemm");
     Q8GemmArgs g;
-    g.W = w->dev;
-    g.row_stride = w->layout.row_stride;
-    g.off_d = w->layout.off_a;
+    g.W = W;
+    g.row_stride = row_stride;
+    g.off_d = off_d;
     g.aq = aq;
     g.ad = ad;
     g.y = y;
@@ -372,7 +384,6 @@ int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, v
         }
         sized = true;
     }
-    const bool q4 = w->kind == FRK_KIND_Q4_0;
     const int ks = q8_0_split(w->rows, M, (size_t)g.nb);
     g.k_split = ks;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));

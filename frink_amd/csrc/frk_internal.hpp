@@ -103,6 +103,8 @@ struct frk_weights {
     uint8_t fingerprint[192] = {0};
     int refcount = 1;
     bool cached = false;
+    // MXFP4: the range of the E8M0 scale bytes (the batched integer path needs them to be f16 values)
+    int e8m0_min = 0, e8m0_max = 255;
 };
 
 namespace frk {
@@ -225,6 +227,8 @@ size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows);
 // y[n] = partial[0][n] + partial[1][n] + ... in that order (the split GEMMs' second step; frk_gemm_q6.hip)
 int launch_sum_parts(const float *partial, int parts, size_t n, float *y, hipStream_t s);
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
+int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, bool q4, const float *x,
+                            size_t M, float *y, void *ws, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
 // tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the
 // stacked matrices; *n_tiles <= max_tiles.  w1/y1 (nullable) is a second stacked matrix over the
@@ -273,6 +277,11 @@ bool is_unit_kind(int kind);
 // the integer tier of Q5_0 / MXFP4 (Q8_0 activation blocks) and IQ4_XS (Q8_K quants and block scales)
 bool gemv_units_int_fits(const frk_weights *w);
 int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s);
+// Q5_0 / MXFP4 rows decoded into the Q8_0 planar form (signed bytes and f16 scales; `dst` rows dst_stride apart, the
+// scales at off_d): what the batched integer path multiplies.  MXFP4 scales must be f16 values (mxfp4_scale_range).
+int launch_units_to_q8_0_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s);
+// the smallest and largest E8M0 scale byte of an MXFP4 matrix (synchronous; at registration)
+int mxfp4_scale_range(const frk_weights *w, int *e_min, int *e_max, hipStream_t s);
 int launch_dequant_units(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s);
 int launch_gemv_units_f32(const frk_weights *w, const float *x, float *y, hipStream_t s);
 // K-quant GEMV on dequantized weights and the f32 activation (the reference's default x86 decode numerics)

@@ -377,4 +377,75 @@ int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *a
     return launch_gemv_units_int_kind<FRK_KIND_MXFP4>(w, aq, ad, y, s);
 }
 
+// ---- the batched integer path of Q5_0 / MXFP4: the codes as signed bytes and the scales as f16, in the planar
+// form the Q8_0 matrix-core GEMM reads (one v_mfma_i32_32x32x32_i8 per block, the scales' outer product by an f16
+// MFMA).  Q5_0's scale is an f16 already; MXFP4's halved E8M0 scale 2^(e - 128) is one for e in 104..143. ----
+template <int KIND>
+__global__ __launch_bounds__(256) void units_to_q8_0_planar_kernel(const uint8_t *__restrict__ W, size_t row_stride, size_t rows,
+                                                                  size_t units, uint8_t *__restrict__ dst, size_t dst_stride,
+                                                                  size_t off_d) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * units) return;
+    const size_t r = i / units, u = i % units;
+    uint32_t c[8];
+    float scale;
+    int scale_i;
+    unit_codes<KIND>(W + r * row_stride, (int)u, c, scale, scale_i);
+    uint4 *q = reinterpret_cast<uint4 *>(dst + r * dst_stride + u * 32);
+    q[0] = make_uint4(c[0], c[1], c[2], c[3]);
+    q[1] = make_uint4(c[4], c[5], c[6], c[7]);
+    reinterpret_cast<uint16_t *>(dst + r * dst_stride + off_d)[u] = f2h_bits(scale);
+}
+int launch_units_to_q8_0_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s) {
+    const size_t units = w->cols / 32;
+    const unsigned g = (unsigned)((w->rows * units + 255) / 256);
+    if (w->kind == FRK_KIND_Q5_0)
+        hipLaunchKernelGGL((units_to_q8_0_planar_kernel<FRK_KIND_Q5_0>), dim3(g), dim3(256), 0, s, w->dev, w->layout.row_stride, w->rows,
+                           units, dst, dst_stride, off_d);
+    else if (w->kind == FRK_KIND_MXFP4)
+        hipLaunchKernelGGL((units_to_q8_0_planar_kernel<FRK_KIND_MXFP4>), dim3(g), dim3(256), 0, s, w->dev, w->layout.row_stride, w->rows,
+                           units, dst, dst_stride, off_d);
+    else
+        return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has no Q8_0 planar form", w->kind);
+    FRK_LAUNCH_CHECK("units_to_q8_0_planar");
+    return FRK_OK;
+}
+
+__global__ __launch_bounds__(256) void mxfp4_scale_range_kernel(const uint8_t *__restrict__ W, size_t row_stride, size_t rows, size_t units,
+                                                               int *__restrict__ range) {
+    int lo = 255, hi = 0;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < rows * units; i += (size_t)gridDim.x * 256) {
+        const int e = W[(i / units) * row_stride + (i % units) * MXFP4_BYTES];
+        lo = min(lo, e);
+        hi = max(hi, e);
+    }
+    for (int m = 32; m > 0; m >>= 1) {
+        lo = min(lo, __shfl_xor(lo, m));
+        hi = max(hi, __shfl_xor(hi, m));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicMin(&range[0], lo);
+        atomicMax(&range[1], hi);
+    }
+}
+int mxfp4_scale_range(const frk_weights *w, int *e_min, int *e_max, hipStream_t s) {
+    int *range = nullptr;
+    FRK_HIP_TRY(hipMalloc((void **)&range, 8));
+    int h[2] = {255, 0};
+    hipError_t e = hipMemcpyAsync(range, h, 8, hipMemcpyHostToDevice, s);
+    if (e == hipSuccess) {
+        const size_t units = w->cols / 32;
+        const unsigned g = (unsigned)std::min<size_t>((w->rows * units + 255) / 256, 4096);
+        hipLaunchKernelGGL(mxfp4_scale_range_kernel, dim3(g), dim3(256), 0, s, w->dev, w->layout.row_stride, w->rows, units, range);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipMemcpyAsync(h, range, 8, hipMemcpyDeviceToHost, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    (void)hipFree(range);
+    if (e != hipSuccess) return set_error(FRK_ERR_HIP, "mxfp4 scale range: %s", hipGetErrorString(e));
+    *e_min = h[0];
+    *e_max = h[1];
+    return FRK_OK;
+}
+
 }  // namespace frk

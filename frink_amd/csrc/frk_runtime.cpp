@@ -208,6 +208,8 @@ static int make_resident(int kind, const uint8_t *src_dev, size_t rows, size_t c
         e = hipMemsetAsync(w->dev + w->layout.row_stride * rows, 0, 256, s);
         if (e != hipSuccess) rc = set_error(FRK_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
     }
+    // (MXFP4: whether the scales are f16 values decides the batched path; one pass over the scale bytes, once)
+    if (rc == FRK_OK && kind == FRK_KIND_MXFP4) rc = mxfp4_scale_range(w, &w->e8m0_min, &w->e8m0_max, s);
     if (rc != FRK_OK) {
         (void)hipFree(w->dev);
         delete w;
@@ -281,8 +283,9 @@ const char *frk_hip_matvec_kernel(int kind) {
 }
 int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
 int frk_hip_gemm_supported(int kind) {
+    // (Q5_0 and MXFP4 through the Q8_0 matrix-core kernel; IQ4_XS batches run the integer decode kernel per row)
     return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0 ||
-           kind == FRK_KIND_Q4_0;
+           kind == FRK_KIND_Q4_0 || kind == FRK_KIND_Q5_0 || kind == FRK_KIND_MXFP4;
 }
 int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
 int frk_hip_block_elems(int kind) { return block_elems(kind); }
@@ -627,6 +630,56 @@ static int thin_gemm_acts(const frk_weights *w, const Q8KActs &a, size_t batch, 
     return FRK_OK;
 }
 
+// Whether a Q5_0 / MXFP4 batch goes through the matrix cores: the weights decoded into the Q8_0 planar form (signed
+// bytes, f16 scales) in scratch memory, then the Q8_0 GEMM.  From four rows on (below that the decode kernel per row
+// reads less than the decoded copy costs); MXFP4 only when every scale 2^(e - 128) is an f16 value.
+static bool units_batch_takes_the_matrix_cores(const frk_weights *w, size_t batch) {
+    if (batch < 4) return false;
+    if (w->kind == FRK_KIND_Q5_0) return true;
+    return w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143;
+}
+static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, float *y, hipStream_t s, Scratch &scratch) {
+    if (units_batch_takes_the_matrix_cores(w, batch)) {
+        const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
+        const size_t planar_bytes = round_up(planar.row_stride * w->rows + 256, 256);
+        void *ws = nullptr;
+        int rc = scratch.get(planar_bytes + gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), s, &ws);
+        if (rc) return rc;
+        uint8_t *decoded = (uint8_t *)ws;
+        rc = launch_units_to_q8_0_planar(w, decoded, planar.row_stride, planar.off_a, s);
+        if (rc) return rc;
+        return launch_gemm_q8_0_planar(decoded, planar.row_stride, planar.off_a, w->rows, w->cols, false, x, batch, y,
+                                       (char *)ws + planar_bytes, s);
+    }
+    if (!gemv_units_int_fits(w))
+        return set_error(FRK_ERR_UNSUPPORTED, "the integer tier of quant kind %d does not take rows of %zu columns", w->kind, w->cols);
+    if (w->kind == FRK_KIND_IQ4_XS) {  // one Q8_K quantization of the batch, the decode kernel per row
+        Q8KActs a;
+        int rc = quantize_acts_q8_k(w, x, batch, s, scratch, &a);
+        if (rc) return rc;
+        const size_t nb = w->cols / QK_K;
+        for (size_t b = 0; b < batch; b++) {
+            rc = launch_gemv_units_int(w, a.q + b * w->cols, a.d + b * nb, y + b * w->rows, s);
+            if (rc) return rc;
+        }
+        return FRK_OK;
+    }
+    // one Q8_0 quantization of the batch (the decode path's kernel, block by block), the decode kernel per row
+    const size_t n = batch * w->cols;
+    void *ws = nullptr;
+    int rc = scratch.get(round_up(n, 256) + n / 32 * 4, s, &ws);
+    if (rc) return rc;
+    int8_t *q = (int8_t *)ws;
+    float *d = (float *)((char *)ws + round_up(n, 256));
+    rc = launch_quantize_q8_0(x, n, q, d, s);
+    if (rc) return rc;
+    for (size_t b = 0; b < batch; b++) {
+        rc = launch_gemv_units_int(w, q + b * w->cols, d + b * (w->cols / 32), y + b * w->rows, s);
+        if (rc) return rc;
+    }
+    return FRK_OK;
+}
+
 static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
     if (q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch)) {  // (frk_hip_gemm_pair_dev: the same test)
         void *ws = nullptr;
@@ -649,6 +702,9 @@ static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *
         if (rc) return rc;
         return launch_gemm_q8_0(w, x, batch, y, ws, (hipStream_t)stream);
     }
+    // Q5_0 / IQ4_XS / MXFP4: a batch is the integer tier too, as in the reference (q8_row_dot / q8k_row_dot per
+    // (row, activation) over activations quantized once, crates/frink-core/src/weight_matrix.rs:392-420)
+    if (is_unit_kind(w->kind) && batch >= 2) return gemm_units_int(w, x, batch, y, (hipStream_t)stream, scratch);
     // thin batches of the K-quants: the weights are read once per 8 (Q6_K) or 16 (Q4_K) activation rows
     if (batch_takes_the_thin_kernels(w, batch)) {
         const int thin = thin_gemm_max_batch(w);

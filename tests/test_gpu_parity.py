@@ -1121,13 +1121,14 @@ def test_other_kinds_dequant_and_get_rows_are_bit_exact(fa, kind, rows, cols):
     (fo.MXFP4, 70, 1024, 1), (fo.MXFP4, 64, 2880, 4),
 ])
 def test_other_kinds_gemv_matches_the_oracle(fa, kind, rows, cols, batch):
-    """The decode GEMV of Q5_0 / IQ4_XS / MXFP4 is the f32 dot of the reference's decode path; a batch is a GEMV per row."""
+    """The decode GEMV of Q5_0 / IQ4_XS / MXFP4 is the f32 dot of the reference's decode path."""
     from frink_amd import synth
     print("other kinds", kind, rows, cols, batch, flush=True)
     data = _other_kind_blocks(kind, rows, cols, seed=kind * 3 + rows)
     x = synth.activations(rows + cols, batch, cols, outlier_frac=0.01)
     w = fa.Weights.from_host(kind, data, rows, cols)
-    got = w.gemm(to_dev(x)).cpu().numpy() if batch > 1 else w.gemv(to_dev(x[0])).cpu().numpy()[None]
+    # (a batch would take the integer tier: here every row through the decode entry point)
+    got = np.stack([w.gemv(to_dev(x[b])).cpu().numpy() for b in range(batch)])
     want = fo.gemm(kind, data, rows, cols, x, fo.F32_DOT)
     assert_rows_close(got, want, "kind %d" % kind)
     deq = fo.dequant(kind, data).reshape(rows, cols).astype(np.float64)
@@ -1158,6 +1159,48 @@ def test_other_kinds_integer_gemv_matches_the_oracle(fa, kind, rows, cols):
     # homogeneity: a power of two on the activation scales its Q8 scales exactly and leaves the quants alone
     y4 = w.gemv(to_dev(x * np.float32(4.0)), act_mode=fa.ACT_INT8).cpu().numpy()
     assert np.array_equal(bits(y4), bits(got * np.float32(4.0)))
+    w.release()
+
+
+@pytest.mark.parametrize("kind,rows,cols,batch", [
+    (fo.Q5_0, 70, 1024, 2), (fo.Q5_0, 300, 4096, 3), (fo.Q5_0, 96, 512, 4), (fo.Q5_0, 200, 1056, 40), (fo.Q5_0, 130, 2048, 130),
+    (fo.Q5_0, 64, 96, 33), (fo.MXFP4, 70, 1024, 2), (fo.MXFP4, 64, 2880, 4), (fo.MXFP4, 200, 1056, 40), (fo.MXFP4, 130, 2048, 130),
+    (fo.MXFP4, 96, 32, 7), (fo.IQ4_XS, 70, 1024, 2), (fo.IQ4_XS, 130, 4096, 5), (fo.IQ4_XS, 40, 768, 17),
+])
+def test_other_kinds_batches_take_the_integer_tier(fa, kind, rows, cols, batch):
+    """A batch of Q5_0 / MXFP4 / IQ4_XS is the reference's integer tier (q8_row_dot / q8k_row_dot per (row, activation),
+    crates/frink-core/src/weight_matrix.rs:392-420): up to three rows the decode kernel per row, from four on Q5_0 and
+    MXFP4 decoded into the Q8_0 planar form and multiplied on the matrix cores -- every workgroup shape of that kernel,
+    ragged tiles, rows that are not a multiple of its 256-column step; IQ4_XS the decode kernel per row at any size."""
+    from frink_amd import synth
+    print("other kinds, batch", kind, rows, cols, batch, flush=True)
+    data = _other_kind_blocks(kind, rows, cols, seed=kind * 7 + rows + batch)
+    if kind == fo.MXFP4:
+        blk = data.reshape(-1, 17)
+        blk[:2, 0] = (104, 143)  # the ends of the range whose halved scales are f16 values: 2^-24 and 2^15
+    x = synth.activations(rows + cols + batch, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    want = fo.gemm(kind, data, rows, cols, x, fo.INT_DOT)
+    assert got.shape == (batch, rows)
+    assert_rows_close(got, want, "batch of kind %d %dx%d x %d" % (kind, rows, cols, batch))
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+    half = w.gemm(to_dev(x * np.float32(0.5))).cpu().numpy()
+    assert np.array_equal(bits(half), bits(got * np.float32(0.5)))
+    w.release()
+
+
+def test_mxfp4_batch_with_scales_outside_f16_keeps_the_decode_kernel(fa):
+    """Halved E8M0 scales below 2^-24 or above 2^15 are not f16 values: such a matrix's batches run the integer decode
+    kernel per row (f32 scales), with the same results to the tolerance."""
+    from frink_amd import synth
+    rows, cols, batch = 64, 1024, 9
+    data = _other_kind_blocks(fo.MXFP4, rows, cols, seed=5)
+    data.reshape(-1, 17)[::7, 0] = 160  # 2^32
+    x = synth.activations(6, batch, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(fo.MXFP4, data, rows, cols)
+    got = w.gemm(to_dev(x)).cpu().numpy()
+    assert_rows_close(got, fo.gemm(fo.MXFP4, data, rows, cols, x, fo.INT_DOT), "mxfp4 with wide scales")
     w.release()
 
 
