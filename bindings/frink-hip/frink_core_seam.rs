@@ -23,7 +23,10 @@ impl BackendCaps for Hip {
         .then(|| kind.name())
     }
     fn gemm_supported(kind: QuantKind) -> bool {
-        matches!(kind, QuantKind::Q4_0 | QuantKind::Q8_0 | QuantKind::Q4K | QuantKind::Q5K | QuantKind::Q6K)
+        matches!(
+            kind,
+            QuantKind::Q4_0 | QuantKind::Q5_0 | QuantKind::Q8_0 | QuantKind::Q4K | QuantKind::Q5K | QuantKind::Q6K | QuantKind::Mxfp4Gguf
+        )
     }
 }
 

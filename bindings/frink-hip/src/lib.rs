@@ -16,6 +16,10 @@ use std::ffi::{c_char, c_int, c_void, CStr};
 pub struct FrkWeights {
     _p: [u8; 0],
 }
+#[repr(C)]
+pub struct FrkBatchActs {
+    _p: [u8; 0],
+}
 
 #[repr(C)]
 pub struct FrkDeviceInfo {
@@ -92,6 +96,12 @@ extern "C" {
                              y1: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_gemm_noalloc_dev(w: *const FrkWeights, x: *const f32, batch: usize, y: *mut f32,
                                 stream: *mut c_void) -> c_int;
+    fn frk_hip_batch_acts_create(max_batch: usize, cols: usize, out: *mut *mut FrkBatchActs) -> c_int;
+    fn frk_hip_batch_acts_release(acts: *mut FrkBatchActs) -> c_int;
+    fn frk_hip_quantize_batch_acts_dev(acts: *mut FrkBatchActs, x: *const f32, batch: usize, stream: *mut c_void) -> c_int;
+    fn frk_hip_gemm_acts_dev(w: *const FrkWeights, acts: *const FrkBatchActs, y: *mut f32, stream: *mut c_void) -> c_int;
+    fn frk_hip_gemm_grouped_dev(stacked: *const FrkWeights, n_groups: usize, group_off: *const i32, gather: *const i32,
+                                x: *const f32, x_rows: usize, pairs: usize, y: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_route_top_k_softmax_dev(logits: *const f32, batch: usize, n_experts: usize, k: usize, norm: c_int,
                                        ids: *mut i32, weights: *mut f32, stream: *mut c_void) -> c_int;
     fn frk_hip_moe_ffn_dev(gate: *const FrkWeights, up: *const FrkWeights, down: *const FrkWeights, n_experts: usize,
@@ -334,6 +344,42 @@ pub mod dev {
     pub unsafe fn gemm_noalloc(w: &Weights, x: *const f32, batch: usize, y: *mut f32, stream: *mut c_void)
         -> Result<(), HipError> {
         check(frk_hip_gemm_noalloc_dev(w.0, x, batch, y, stream))
+    }
+    /// `BatchActs::Q8K` (weight_matrix.rs:757-768) on the device: a batch quantized once for any number of
+    /// matrices of `cols` columns, at any batch size up to `max_batch`.
+    pub struct BatchActs(pub(crate) *mut FrkBatchActs);
+    impl BatchActs {
+        pub fn new(max_batch: usize, cols: usize) -> Result<Self, HipError> {
+            let mut p = std::ptr::null_mut();
+            check(unsafe { frk_hip_batch_acts_create(max_batch, cols, &mut p) })?;
+            Ok(BatchActs(p))
+        }
+        /// `quantize_batch_acts` (weight_matrix.rs:2348-2426).
+        /// # Safety
+        /// `x` holds `batch * cols` floats on the device.
+        pub unsafe fn quantize(&mut self, x: *const f32, batch: usize, stream: *mut c_void) -> Result<(), HipError> {
+            check(frk_hip_quantize_batch_acts_dev(self.0, x, batch, stream))
+        }
+    }
+    impl Drop for BatchActs {
+        fn drop(&mut self) {
+            unsafe { frk_hip_batch_acts_release(self.0) };
+        }
+    }
+    /// `apply_batch_with_acts` (weight_matrix.rs:2481-2487) over a `BatchActs`: `y[batch][rows]`, bit for bit `gemm`.
+    /// # Safety
+    /// `y` has room for the quantized batch times `w.rows()` floats.
+    pub unsafe fn gemm_acts(w: &Weights, acts: &BatchActs, y: *mut f32, stream: *mut c_void) -> Result<(), HipError> {
+        check(frk_hip_gemm_acts_dev(w.0, acts.0, y, stream))
+    }
+    /// The grouped GEMM (`enqueue_mul_mm_grouped_dev`, crates/frink-cuda/src/mul_mm_launch.rs:391-470): group `g` is
+    /// rows `[g*R, (g+1)*R)` of `stacked`; pair `p` of group `g` reads row `gather[p]` of `x` (row `p` when `gather`
+    /// is null) and writes `y[p][R]`.
+    /// # Safety
+    /// `group_off[n_groups + 1]`, `gather[pairs]` (or null), `x[x_rows][cols]`, `y[pairs][R]` on the device.
+    pub unsafe fn gemm_grouped(stacked: &Weights, n_groups: usize, group_off: *const i32, gather: *const i32, x: *const f32,
+                               x_rows: usize, pairs: usize, y: *mut f32, stream: *mut c_void) -> Result<(), HipError> {
+        check(frk_hip_gemm_grouped_dev(stacked.0, n_groups, group_off, gather, x, x_rows, pairs, y, stream))
     }
     /// `frink_moe::route_top_k_softmax` (crates/frink-moe/src/lib.rs:567-589) for a batch of tokens.
     /// # Safety

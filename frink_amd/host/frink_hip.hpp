@@ -191,6 +191,16 @@ class WeightMatrix {
         return true;
     }
 
+    // y[pairs][rows / n_groups]: this matrix as n_groups stacked groups, pair p of group g (group_off[g] <= p <
+    // group_off[g + 1]) times row gather[p] of x (row p without a gather list); everything on the device
+    // (enqueue_mul_mm_grouped_dev, crates/frink-cuda/src/mul_mm_launch.rs:391-470)
+    Result<bool> apply_grouped_dev(size_t n_groups, const int32_t *group_off_dev, const int32_t *gather_dev, const float *x_dev,
+                                   size_t x_rows, size_t pairs, float *y_dev, void *stream) const {
+        int rc = frk_hip_gemm_grouped_dev(h_, n_groups, group_off_dev, gather_dev, x_dev, x_rows, pairs, y_dev, stream);
+        if (rc != FRK_OK) return last_error(rc);
+        return true;
+    }
+
   private:
     WeightMatrix(frk_weights *h, QuantKind k, size_t r, size_t c) : h_(h), kind_(k), rows_(r), cols_(c) {}
     void reset() {
@@ -200,6 +210,48 @@ class WeightMatrix {
     frk_weights *h_ = nullptr;
     QuantKind kind_ = QuantKind::Q8_0;
     size_t rows_ = 0, cols_ = 0;
+};
+
+// BatchActs::Q8K (crates/frink-core/src/weight_matrix.rs:757-768): a batch's activations quantized once for any number
+// of matrices of `cols` columns (quantize_batch_acts, :2348-2426), at any batch size up to max_batch.  Move-only.
+class BatchActs {
+  public:
+    static Result<BatchActs> with_room_for(size_t max_batch, size_t cols) {
+        frk_batch_acts *h = nullptr;
+        int rc = frk_hip_batch_acts_create(max_batch, cols, &h);
+        if (rc != FRK_OK) return last_error(rc);
+        return BatchActs(h);
+    }
+    BatchActs() = default;
+    BatchActs(BatchActs &&o) noexcept : h_(o.h_) { o.h_ = nullptr; }
+    BatchActs &operator=(BatchActs &&o) noexcept {
+        if (this != &o) {
+            if (h_) frk_hip_batch_acts_release(h_);
+            h_ = o.h_;
+            o.h_ = nullptr;
+        }
+        return *this;
+    }
+    BatchActs(const BatchActs &) = delete;
+    BatchActs &operator=(const BatchActs &) = delete;
+    ~BatchActs() {
+        if (h_) frk_hip_batch_acts_release(h_);
+    }
+    Result<bool> quantize_dev(const float *x_dev, size_t batch, void *stream) {
+        int rc = frk_hip_quantize_batch_acts_dev(h_, x_dev, batch, stream);
+        if (rc != FRK_OK) return last_error(rc);
+        return true;
+    }
+    // WeightMatrix::apply_batch_with_acts (:2481-2487): y[batch][rows], bit for bit apply_batch_dev's result
+    Result<bool> apply_dev(const WeightMatrix &w, float *y_dev, void *stream) const {
+        int rc = frk_hip_gemm_acts_dev(w.handle(), h_, y_dev, stream);
+        if (rc != FRK_OK) return last_error(rc);
+        return true;
+    }
+
+  private:
+    explicit BatchActs(frk_batch_acts *h) : h_(h) {}
+    frk_batch_acts *h_ = nullptr;
 };
 
 // One MoE layer's experts, stacked per projection (ExpertWeights{gate, up, down} x n_experts).
