@@ -149,7 +149,7 @@ __global__ __launch_bounds__(FUSED ? 1024 : 256) void gemv_q6_k_direct_kernel(
 // Round j of a wavefront covers rows 4j .. 4j+3 of the workgroup: lane = 16 * (row of the round) + unit,
 // unit = (block of the slice, half, 16-byte column) as above.
 constexpr int COLS_WAVE_LDS = 4 * (QK_K + 32 + 4);  // four blocks: quants, 16-wide sums, scale
-template <int U>
+template <int U, bool NT = false>
 __global__ __launch_bounds__(1024) void gemv_q6_k_cols_kernel(const uint8_t *__restrict__ W, Layout lay, int rows, int nb,
                                                              const float *__restrict__ x, float *__restrict__ y) {
     typedef float xv_t __attribute__((ext_vector_type(4)));
@@ -182,9 +182,15 @@ __global__ __launch_bounds__(1024) void gemv_q6_k_cols_kernel(const uint8_t *__r
         const uint8_t *p_h = row + lay.off_a + (size_t)b * 64 + h * 32 + t * 16;
         const uint8_t *p_s = row + lay.off_b + (size_t)b * 16 + h * 8;
         const uint8_t *p_d = row + lay.off_c + (size_t)b * 2;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qla[j]) : "v"(p_l) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(qlb[j]) : "v"(p_l) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qh[j]) : "v"(p_h) : "memory");
+        if (NT) {  // (rows that start on a cache line: a wavefront's share of the two big planes is whole lines)
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(qla[j]) : "v"(p_l) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:32 nt" : "=v"(qlb[j]) : "v"(p_l) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(qh[j]) : "v"(p_h) : "memory");
+        } else {
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qla[j]) : "v"(p_l) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off offset:32" : "=v"(qlb[j]) : "v"(p_l) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qh[j]) : "v"(p_h) : "memory");
+        }
         asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(scv[j]) : "v"(p_s) : "memory");
         asm volatile("global_load_ushort %0, %1, off" : "=v"(dbits[j]) : "v"(p_d) : "memory");
     };
@@ -607,8 +613,12 @@ int launch_gemv_q6_k_fused(const frk_weights *w, const float *x, float *y, hipSt
         }
         const size_t lds = (size_t)waves * (COLS_WAVE_LDS + 4 * best_u * 4);
         const dim3 grid((unsigned)((w->rows + 4 * best_u - 1) / (4 * best_u))), block(64 * waves);
-#define FRK_GO_COLS(UU) \
-    hipLaunchKernelGGL((gemv_q6_k_cols_kernel<UU>), grid, block, lds, s, w->dev, w->layout, (int)w->rows, nb, x, y)
+        const bool whole_lines = w->layout.row_stride % 128 == 0 && nb % 4 == 0;  // (every wavefront's four blocks of ql: 512 bytes)
+#define FRK_GO_COLS(UU)                                                                                                              \
+    if (whole_lines)                                                                                                                 \
+        hipLaunchKernelGGL((gemv_q6_k_cols_kernel<UU, true>), grid, block, lds, s, w->dev, w->layout, (int)w->rows, nb, x, y);      \
+    else                                                                                                                             \
+        hipLaunchKernelGGL((gemv_q6_k_cols_kernel<UU, false>), grid, block, lds, s, w->dev, w->layout, (int)w->rows, nb, x, y)
         if (best_u == 1) FRK_GO_COLS(1);
         else if (best_u == 2) FRK_GO_COLS(2);
         else if (best_u == 3) FRK_GO_COLS(3);

@@ -73,7 +73,10 @@ inline Layout layout_for(int kind, size_t cols) {
         l.off_a = nb * 128;
         l.off_b = l.off_a + nb * 64;
         l.off_c = l.off_b + nb * 16;
-        l.row_stride = round_up(l.off_c + nb * 2, 16);
+        // rows start on a cache line where that costs under 2 % (the ql and qh planes then do too: a wavefront's
+        // share of them is whole lines), else 16-byte aligned
+        const size_t raw = l.off_c + nb * 2, lines = round_up(raw, 128);
+        l.row_stride = (lines - raw) * 50 < raw ? lines : round_up(raw, 16);
     } else if (kind == FRK_KIND_Q8_0) {
         l.off_a = nb * 32;
         l.row_stride = round_up(l.off_a + nb * 2, 16);
