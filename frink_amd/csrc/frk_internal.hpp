@@ -280,6 +280,12 @@ bool is_unit_kind(int kind);
 // the integer tier of Q5_0 / MXFP4 (Q8_0 activation blocks) and IQ4_XS (Q8_K quants and block scales)
 bool gemv_units_int_fits(const frk_weights *w);
 int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s);
+int launch_gemv_units_int_jobs(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
+                               const int8_t *aq, const float *ad, float *y, hipStream_t s);
+// the routed layer over experts of these kinds: every (token, slot) pair a job of the integer decode kernel
+size_t moe_units_workspace_bytes(size_t batch, int k, int hidden, int ffn);
+int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts, const float *x,
+                         size_t batch, const int32_t *ids, const float *weights, int k, float *out, void *ws, hipStream_t s);
 // Q5_0 / MXFP4 rows decoded into the Q8_0 planar form (signed bytes and f16 scales; `dst` rows dst_stride apart, the
 // scales at off_d): what the batched integer path multiplies.  MXFP4 scales must be f16 values (mxfp4_scale_range).
 int launch_units_to_q8_0_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s);

@@ -228,13 +228,29 @@ __device__ __forceinline__ void unit_codes(const uint8_t *row, int u, uint32_t (
 // A wavefront per row, a lane per unit.  The quantized activation sits in LDS for the whole launch; a row's bytes go
 // global -> registers (whole 16-byte pieces, the next row's while this one is multiplied) -> the wavefront's own
 // LDS slot, from where the lanes pick their blocks apart (22- and 17-byte blocks have no alignment to load by).
-template <int KIND, int MAXP>
+// JOBS: a grid of expert-indexed jobs (run_expert's projections, crates/frink-moe/src/lib.rs:1068-1165): job
+// blockIdx.y multiplies the rows of expert ids[job] (a slice of `rows` rows of the stacked matrix) with activation
+// row job / act_div and writes output row job; a job whose id is outside the experts does nothing.
+struct UnitsJobs {
+    const int32_t *ids;
+    int n_experts, job0, act_div;
+};
+template <int KIND, int MAXP, bool JOBS = false>
 __global__ __launch_bounds__(512) void gemv_units_int_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int cols,
                                                             const int8_t *__restrict__ aq, const float *__restrict__ ad,
-                                                            float *__restrict__ y) {
+                                                            float *__restrict__ y, UnitsJobs jobs) {
     extern __shared__ uint4 smem_kinds[];
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_kinds);
     const int units = cols / 32, nd = KIND == FRK_KIND_IQ4_XS ? cols / QK_K : units;
+    if (JOBS) {
+        const int job = jobs.job0 + (int)blockIdx.y;
+        const int e = jobs.ids[job];
+        if (e < 0 || e >= jobs.n_experts) return;  // (uniform per workgroup)
+        W += (size_t)e * rows * row_stride;
+        aq += (size_t)(job / jobs.act_div) * cols;
+        ad += (size_t)(job / jobs.act_div) * nd;
+        y += (size_t)job * rows;
+    }
     int8_t *sq = reinterpret_cast<int8_t *>(lds);
     float *sd = reinterpret_cast<float *>(lds + cols);
     const int pieces = (int)(row_stride / 16);
@@ -357,9 +373,47 @@ static int launch_gemv_units_int_as(const frk_weights *w, const int8_t *aq, cons
     }
     const unsigned grid = (unsigned)std::min<size_t>((w->rows + 7) / 8, 2048);
     hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP>), dim3(grid), dim3(512), shmem, s, w->dev, w->layout.row_stride, (int)w->rows,
-                       (int)w->cols, aq, ad, y);
+                       (int)w->cols, aq, ad, y, UnitsJobs{nullptr, 0, 0, 1});
     FRK_LAUNCH_CHECK("gemv_units_int");
     return FRK_OK;
+}
+template <int KIND, int MAXP>
+static int launch_gemv_units_jobs_as(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
+                                     const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    const size_t shmem = gemv_units_int_lds(w);
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_units_int_kernel<KIND, MAXP, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(gemv units jobs): %s", hipGetErrorString(e));
+        sized = true;
+    }
+    const unsigned gx = (unsigned)std::min<size_t>((rows_e + 7) / 8, 2048);
+    for (size_t j0 = 0; j0 < n_jobs; j0 += 32768) {  // (the grid's second dimension holds 65535)
+        const unsigned gy = (unsigned)std::min<size_t>(n_jobs - j0, 32768);
+        hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP, true>), dim3(gx, gy), dim3(512), shmem, s, w->dev, w->layout.row_stride,
+                           (int)rows_e, (int)w->cols, aq, ad, y, UnitsJobs{ids, n_experts, (int)j0, act_div});
+        FRK_LAUNCH_CHECK("gemv_units_int (jobs)");
+    }
+    return FRK_OK;
+}
+template <int KIND>
+static int launch_gemv_units_jobs_kind(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs,
+                                       int act_div, const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    const size_t per_lane = (w->layout.row_stride / 16 + 63) / 64;
+    if (per_lane <= 3) return launch_gemv_units_jobs_as<KIND, 3>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    if (per_lane <= 6) return launch_gemv_units_jobs_as<KIND, 6>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    return launch_gemv_units_jobs_as<KIND, 12>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+}
+// y[job][rows_e] = W[expert ids[job]] . activation row job / act_div, on the integer tier; w stacks the experts
+int launch_gemv_units_int_jobs(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
+                               const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+    if (!gemv_units_int_fits(w))
+        return set_error(FRK_ERR_UNSUPPORTED, "the integer GEMV of quant kind %d does not take rows of %zu columns", w->kind, w->cols);
+    if (w->kind == FRK_KIND_Q5_0) return launch_gemv_units_jobs_kind<FRK_KIND_Q5_0>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    if (w->kind == FRK_KIND_IQ4_XS)
+        return launch_gemv_units_jobs_kind<FRK_KIND_IQ4_XS>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    return launch_gemv_units_jobs_kind<FRK_KIND_MXFP4>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
 }
 template <int KIND>
 static int launch_gemv_units_int_kind(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s) {

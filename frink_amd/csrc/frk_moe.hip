@@ -679,4 +679,64 @@ int launch_gemm_grouped(const frk_weights *w, size_t n_groups, const int32_t *gr
                : launch_gemm_q4_k_stream(w, nullptr, rows_g, m.xa, nullptr, nullptr, m.tiles, m.n_tiles, max_tiles, y, nullptr, s);
 }
 
+// Experts in Q5_0 / IQ4_XS / MXFP4 (run_expert takes any WeightMatrix, crates/frink-moe/src/lib.rs:1068-1165; gpt-oss
+// keeps its experts in MXFP4): every (token, slot) pair is a job of the integer decode kernel -- gate and up over the
+// token's quantized activation, silu(g) * u, that row quantized, down -- and the weighted sum in the reference's order
+// for the batch size.  Q8_0 activation blocks for Q5_0 and MXFP4 projections, Q8_K for IQ4_XS ones.  (A batch of
+// hundreds of tokens reads an expert's matrices once per pair here, out of the caches: correct, not fast.)
+struct UnitsActs {
+    int8_t *q;
+    float *d;
+    int16_t *bsums;  // Q8_K only
+};
+static size_t units_acts_bytes(size_t rows, size_t cols) {
+    return round_up(rows * cols, 256) + round_up(rows * cols / 32 * 4, 256) + round_up(rows * cols / 16 * 2, 256);
+}
+static UnitsActs units_acts_carve(char *base, size_t rows, size_t cols) {
+    UnitsActs a;
+    a.q = (int8_t *)base;
+    a.d = (float *)(base + round_up(rows * cols, 256));
+    a.bsums = (int16_t *)(base + round_up(rows * cols, 256) + round_up(rows * cols / 32 * 4, 256));
+    return a;
+}
+static int quantize_for_units(int kind, const float *x, size_t n, const UnitsActs &a, hipStream_t s) {
+    return kind == FRK_KIND_IQ4_XS ? launch_quantize_q8_k(x, n, a.q, a.d, a.bsums, s) : launch_quantize_q8_0(x, n, a.q, a.d, s);
+}
+size_t moe_units_workspace_bytes(size_t batch, int k, int hidden, int ffn) {
+    const size_t pairs = batch * (size_t)k;
+    return units_acts_bytes(batch, hidden) + 2 * round_up(pairs * ffn * 4, 256) + units_acts_bytes(pairs, ffn) +
+           round_up(pairs * hidden * 4, 256);
+}
+int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts, const float *x,
+                         size_t batch, const int32_t *ids, const float *weights, int k, float *out, void *ws, hipStream_t s) {
+    const int hidden = (int)gate->cols, ffn = (int)down->cols;
+    const size_t pairs = batch * (size_t)k;
+    char *p = (char *)ws;
+    const UnitsActs xa = units_acts_carve(p, batch, hidden);
+    p += units_acts_bytes(batch, hidden);
+    float *g_out = (float *)p;
+    p += round_up(pairs * ffn * 4, 256);
+    float *u_out = (float *)p;
+    p += round_up(pairs * ffn * 4, 256);
+    const UnitsActs aa = units_acts_carve(p, pairs, ffn);
+    p += units_acts_bytes(pairs, ffn);
+    float *d_out = (float *)p;
+    int rc = quantize_for_units(gate->kind, x, batch * (size_t)hidden, xa, s);
+    if (rc) return rc;
+    rc = launch_gemv_units_int_jobs(gate, (size_t)ffn, n_experts, ids, pairs, k, xa.q, xa.d, g_out, s);
+    if (rc) return rc;
+    rc = launch_gemv_units_int_jobs(up, (size_t)ffn, n_experts, ids, pairs, k, xa.q, xa.d, u_out, s);
+    if (rc) return rc;
+    rc = launch_swiglu(g_out, u_out, pairs * (size_t)ffn, g_out, s);  // (in place: element by element)
+    if (rc) return rc;
+    rc = quantize_for_units(down->kind, g_out, pairs * (size_t)ffn, aa, s);
+    if (rc) return rc;
+    rc = launch_gemv_units_int_jobs(down, (size_t)hidden, n_experts, ids, pairs, 1, aa.q, aa.d, d_out, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch, (unsigned)((hidden + 1023) / 1024)), dim3(256), 0, s, d_out, ids, weights,
+                       (const int *)nullptr, k, hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);
+    FRK_LAUNCH_CHECK("moe_combine");
+    return FRK_OK;
+}
+
 }  // namespace frk

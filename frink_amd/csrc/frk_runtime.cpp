@@ -1061,10 +1061,13 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
         return set_error(FRK_ERR_SHAPE, "empty shape: batch=%zu experts=%zu k=%zu", batch, n_experts, k);
     if (n_experts > 1024 || k > 64 || k > n_experts)
         return set_error(FRK_ERR_SHAPE, "experts=%zu (max 1024), k=%zu (max 64, at most the expert count)", n_experts, k);
-    if (gate->kind != FRK_KIND_Q4_K || up->kind != FRK_KIND_Q4_K || (down->kind != FRK_KIND_Q4_K && down->kind != FRK_KIND_Q6_K))
+    const bool unit_experts = is_unit_kind(gate->kind) && up->kind == gate->kind && is_unit_kind(down->kind);
+    if (!unit_experts &&
+        (gate->kind != FRK_KIND_Q4_K || up->kind != FRK_KIND_Q4_K || (down->kind != FRK_KIND_Q4_K && down->kind != FRK_KIND_Q6_K)))
         return set_error(FRK_ERR_UNSUPPORTED,
-                         "the expert GEMMs take Q4_K gate and up and Q4_K or Q6_K down experts (got kinds %d/%d/%d)", gate->kind,
-                         up->kind, down->kind);
+                         "the expert GEMMs take Q4_K gate and up and Q4_K or Q6_K down experts, or Q5_0 / IQ4_XS / MXFP4 experts "
+                         "with gate and up of one kind (got kinds %d/%d/%d)",
+                         gate->kind, up->kind, down->kind);
     if (gate->rows % n_experts || down->rows % n_experts)
         return set_error(FRK_ERR_SHAPE, "stacked rows %zu/%zu do not divide into %zu experts", gate->rows, down->rows,
                          n_experts);
@@ -1075,6 +1078,14 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
                          gate->rows, gate->cols, up->rows, up->cols, down->rows, down->cols, n_experts, hidden, ffn);
     if (batch * k > (size_t)1 << 30) return set_error(FRK_ERR_SHAPE, "batch*k = %zu pairs is too many", batch * k);
     WorkspaceLease lease;
+    if (unit_experts) {
+        if (!gemv_units_int_fits(gate) || !gemv_units_int_fits(down))
+            return set_error(FRK_ERR_UNSUPPORTED, "experts of kinds %d/%d with rows of %zu / %zu columns", gate->kind, down->kind,
+                             gate->cols, down->cols);
+        int rc = workspace(moe_units_workspace_bytes(batch, (int)k, (int)hidden, (int)ffn), (hipStream_t)stream, lease);
+        if (rc) return rc;
+        return launch_moe_ffn_units(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, lease.ptr, (hipStream_t)stream);
+    }
     int rc = workspace(moe_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, lease);
     if (rc) return rc;
     return launch_moe_ffn(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, lease.ptr, (hipStream_t)stream);

@@ -1012,6 +1012,50 @@ def test_moe_ffn_with_q6_k_down_experts(fa, n_experts, k, hidden, ffn, batch):
     _moe_case(fa, n_experts, k, hidden, ffn, batch, seed=n_experts * 7 + batch, down_kind=fo.Q6_K)
 
 
+@pytest.mark.parametrize("gate_kind,down_kind,n_experts,k,hidden,ffn,batch", [
+    (fo.MXFP4, fo.MXFP4, 8, 2, 512, 256, 1), (fo.MXFP4, fo.MXFP4, 16, 4, 512, 768, 40), (fo.Q5_0, fo.Q5_0, 8, 2, 256, 512, 9),
+    (fo.IQ4_XS, fo.IQ4_XS, 8, 3, 512, 256, 33), (fo.MXFP4, fo.Q5_0, 6, 2, 256, 256, 5),
+])
+def test_moe_ffn_with_experts_of_the_other_kinds(fa, gate_kind, down_kind, n_experts, k, hidden, ffn, batch):
+    """Experts in MXFP4 / Q5_0 / IQ4_XS (run_expert takes any WeightMatrix, crates/frink-moe/src/lib.rs:1068-1165):
+    every (token, slot) pair on the integer tier of its kind, the slots added in the reference's order for the batch
+    size (routing order below 32 tokens, ascending expert id from 32 on), an id outside the experts left out."""
+    from frink_amd import synth
+    print("moe, other kinds", gate_kind, down_kind, n_experts, k, hidden, ffn, batch, flush=True)
+    gate = _other_kind_blocks(gate_kind, n_experts * ffn, hidden, seed=41)
+    up = _other_kind_blocks(gate_kind, n_experts * ffn, hidden, seed=42)
+    down = _other_kind_blocks(down_kind, n_experts * hidden, ffn, seed=43)
+    for kind, data in ((gate_kind, gate), (gate_kind, up), (down_kind, down)):
+        if kind == fo.MXFP4:  # weight-sized scales, 2^-17 .. 2^-6: the intermediate's Q8_0 scales are f16 values
+            blk = data.reshape(-1, 17)
+            blk[:, 0] = 110 + blk[:, 0] % 12
+    x = synth.activations(44, batch, hidden)
+    ids, w = _route(synth.normal(45, batch * n_experts).reshape(batch, n_experts), k)
+    ids = ids.astype(np.int32)
+    ids[0, 0] = n_experts + 3  # an id outside the experts contributes nothing
+    wg = fa.Weights.from_host(gate_kind, gate, n_experts * ffn, hidden)
+    wu = fa.Weights.from_host(gate_kind, up, n_experts * ffn, hidden)
+    wd = fa.Weights.from_host(down_kind, down, n_experts * hidden, ffn)
+    got = fa.moe_ffn(wg, wu, wd, n_experts, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    gb, ub, db = (m.reshape(n_experts, -1) for m in (gate, up, down))
+    pair_out = np.zeros((batch, k, hidden), np.float32)
+    for e in range(n_experts):
+        toks, slots = np.nonzero(ids == e)
+        if toks.size:
+            g = fo.gemm(gate_kind, gb[e], ffn, hidden, x[toks], fo.INT_DOT)
+            u = fo.gemm(gate_kind, ub[e], ffn, hidden, x[toks], fo.INT_DOT)
+            act = fo.swiglu(g.ravel(), u.ravel()).reshape(toks.size, ffn)
+            pair_out[toks, slots] = fo.gemm(down_kind, db[e], hidden, ffn, act, fo.INT_DOT)
+    want = np.zeros((batch, hidden), np.float32)
+    for t in range(batch):
+        for sl in _slot_order(ids[t], batch):
+            if 0 <= ids[t, sl] < n_experts:
+                want[t] += w[t, sl] * pair_out[t, sl]
+    _end_to_end_gate(got, want, "moe kinds %d/%d E=%d k=%d %d/%d batch=%d" % (gate_kind, down_kind, n_experts, k, hidden, ffn, batch), False)
+    for h in (wg, wu, wd):
+        h.release()
+
+
 def test_moe_ffn_refuses_other_expert_kinds(fa):
     w4 = fa.Weights.from_host(fo.Q4_K, make_weights(fo.Q4_K, 2 * 256, 256, seed=1), 2 * 256, 256)
     w8 = fa.Weights.from_host(fo.Q8_0, make_weights(fo.Q8_0, 2 * 256, 256, seed=2), 2 * 256, 256)
