@@ -681,6 +681,8 @@ static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, fl
 }
 
 static int gemm_impl(const frk_weights *w, const float *x, size_t batch, float *y, void *stream, Scratch &scratch) {
+    // one row is the decode path, whatever the kind
+    if (batch == 1) return gemv_impl(w, x, y, FRK_ACT_F32, (hipStream_t)stream, scratch);
     if (q4_k_takes_the_matrix_cores(w, batch) || q5_k_takes_the_matrix_cores(w, batch)) {  // (frk_hip_gemm_pair_dev: the same test)
         void *ws = nullptr;
         int rc = scratch.get(gemm_q4_k_workspace_bytes(batch, w->cols, w->rows, w->kind == FRK_KIND_Q5_K),

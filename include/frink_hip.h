@@ -228,7 +228,9 @@ int frk_hip_gemm_pair_dev(const frk_weights *w0, const frk_weights *w1, const fl
  * Q8_K rows (the decode and thin kernels), the tiled form of the matrix-core GEMMs, or both.
  * frk_hip_quantize_batch_acts_dev and frk_hip_gemm_acts_dev allocate nothing themselves (a GEMM whose
  * blocks are split between workgroups takes room for the parts from the stream's scratch buffer, like
- * frk_hip_gemm_dev); y is bit for bit frk_hip_gemm_dev's.  K-quant matrices (Q4_K, Q5_K, Q6_K) of `cols`
+ * frk_hip_gemm_dev); y is bit for bit frk_hip_gemm_dev's for two rows and more, and frk_hip_gemv_q8k_dev's for
+ * one (which is frk_hip_gemv_dev's wherever both forms of the decode step are one kernel, and the same integers
+ * added in another order for rows of more than 20 blocks).  K-quant matrices (Q4_K, Q5_K, Q6_K) of `cols`
  * columns; other kinds return FRK_ERR_UNSUPPORTED.  A quantization and the GEMMs that read it are ordered
  * by the stream they are enqueued on; the object is not to be re-quantized while a GEMM that reads it is
  * still in flight on another stream. */

@@ -209,6 +209,8 @@ def encode_matrix(kind, w, threads=0):
     bb, be = BLOCK[kind]
     out = np.empty(rows * (cols // be) * bb, np.uint8)
     rc = lib().fo_encode_matrix(kind, _p(w, C.c_float), rows, cols, _p(out, C.c_uint8), threads)
+    if rc == -2:
+        raise ValueError("quant kind %d has no encoder here" % kind)
     if rc:
         raise ValueError("cols %d is not a whole number of %d-element blocks" % (cols, be))
     return out

@@ -1208,6 +1208,8 @@ static int pick_threads(int threads) {
 int fo_encode_matrix(int kind, const float *src, size_t rows, size_t cols, uint8_t *out, int threads) {
     int be = fo_block_elems(kind), bb = fo_block_bytes(kind);
     if (!be || cols % (size_t)be) return -1;
+    /* (only these four have an encoder: any other kind would be written with another kind's block size) */
+    if (kind != FO_KIND_Q8_0 && kind != FO_KIND_Q4_K && kind != FO_KIND_Q5_K && kind != FO_KIND_Q6_K) return -2;
     size_t row_bytes = cols / (size_t)be * (size_t)bb;
     threads = pick_threads(threads);
     int rc = 0;

@@ -605,6 +605,28 @@ def test_gemm_large_tiles_with_ragged_edges(fa, rows, cols, batch):
     w.release()
 
 
+@pytest.mark.parametrize("kind,rows,cols", [(fo.Q4_K, 70, 4096), (fo.Q5_K, 660, 4096), (fo.Q5_K, 40, 14336), (fo.Q6_K, 50, 2048),
+                                            (fo.Q8_0, 64, 1024), (fo.Q4_0, 64, 1024)])
+def test_a_batch_of_one_row_is_the_decode_path(fa, kind, rows, cols):
+    """frk_hip_gemm_dev with one activation row returns the bits of frk_hip_gemv_dev (a Q5_K row of 16 blocks once took
+    the generic kernel behind a quantization launch there); the batch-activations form returns frk_hip_gemv_q8k_dev's."""
+    from frink_amd import synth
+    data = _random_q4_0(rows, cols, rows) if kind == fo.Q4_0 else make_weights(kind, rows, cols, seed=rows)
+    x = synth.activations(rows + 1, 1, cols, outlier_frac=0.01)
+    w = fa.Weights.from_host(kind, data, rows, cols)
+    one = w.gemv(to_dev(x[0])).cpu().numpy()
+    assert np.array_equal(bits(w.gemm(to_dev(x)).cpu().numpy()[0]), bits(one))
+    if kind in (fo.Q4_K, fo.Q5_K, fo.Q6_K):
+        # (from quantized activations a long row takes another kernel than the one-launch form: the same integers,
+        # added in another order)
+        acts = fa.BatchActs(4, cols).quantize(to_dev(x))
+        got = w.gemm_acts(acts).cpu().numpy()[0]
+        assert np.abs(got - one).max() <= 1e-5 * np.abs(one).max()
+        assert np.array_equal(bits(got), bits(w.gemv_q8k(fa.quantize_q8_k(to_dev(x[0]))).cpu().numpy()))
+        acts.release()
+    w.release()
+
+
 def _oracle_gemm_all_rows(data, rows, cols, x):
     """The oracle's integer-dot GEMM over EVERY weight row.  Its AVX2 form is held bit-equal to the scalar
     functions by tests/test_oracle_goldens.py and does 14336 x 4096 x 512 in a fraction of a second; a host

@@ -255,6 +255,12 @@ def test_q4_0_dots_follow_the_dequantized_row():
     assert abs(fo.dot_int(fo.Q4_0, row, (q, d)) - want) <= 2e-6 * float(np.abs(w * xa).sum())
 
 
+def test_a_kind_without_an_encoder_is_refused_not_written_with_another_kinds_blocks():
+    for kind in (fo.Q4_0, fo.Q5_0, fo.IQ4_XS, fo.MXFP4):
+        with pytest.raises(ValueError):
+            fo.encode_matrix(kind, np.zeros((2, 1024), np.float32))
+
+
 def test_misaligned_buffers_are_refused():
     for kind in (fo.Q4_0, fo.Q8_0, fo.Q4_K, fo.Q5_K, fo.Q6_K):
         with pytest.raises(ValueError):
