@@ -277,7 +277,10 @@ __device__ __forceinline__ void tile_epilogue(const TileAcc &X, const TileScales
 // operand is there.)
 #define FRK_WAIT_LGKM(n, reg, acc) asm volatile("s_waitcnt lgkmcnt(" #n ")" : "+v"(reg), "+v"(acc))
 // between(i, acc) is called after MFMA i of the integer chain has been issued, i = 0..14: what it does
-// shares the gaps of the chain, every MFMA of which waits for the one before it.
+// shares the gaps of the chain, every MFMA of which waits for the one before it.  It must not branch:
+// hipcc counts the wait states between an MFMA and a vector instruction that reads its result within
+// one basic block only, and a branch between MFMA 7 and the shift of its sums left the shift three
+// instructions behind the MFMA (the last two registers of the sums were read before they were written).
 struct NothingBetween {
     __device__ __forceinline__ void operator()(int, v16i &) const {}
 };
