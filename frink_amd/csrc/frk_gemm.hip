@@ -593,6 +593,29 @@ __device__ __forceinline__ void unpack_pair_sel(const v4i q, uint32_t pair0, uin
         H0[c] = h0, L0[c] = l0, H1[c] = h1, L1[c] = l1;
     }
 }
+// The same in plain vector arithmetic (the compiler finds the op_sel forms itself), for a kernel that leaves
+// the place of the unpacking to the compiler: statements of inline assembly stay where they are written.
+__device__ __forceinline__ void unpack_pair_free(const v4i q, uint32_t pair0, uint32_t pair1, v4i &H0, v4i &L0, v4i &H1, v4i &L1) {
+    us2 p0, p1;
+    __builtin_memcpy(&p0, &pair0, 4);
+    __builtin_memcpy(&p1, &pair1, 4);
+    const us2 h0 = {p0.x, p0.x}, l0 = {p0.y, p0.y}, h1 = {p1.x, p1.x}, l1 = {p1.y, p1.y};
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint32_t w = (uint32_t)q[c];
+        const uint32_t nl = w & 0x0f0f0f0fu, nh = (w >> 4) & 0x0f0f0f0fu;
+        us2 a, b;
+        __builtin_memcpy(&a, &nl, 4);
+        __builtin_memcpy(&b, &nh, 4);
+        const us2 r0 = a * h0, r1 = a * l0, r2 = b * h1, r3 = b * l1;  // bytes stay below 106
+        int o0, o1, o2, o3;
+        __builtin_memcpy(&o0, &r0, 4);
+        __builtin_memcpy(&o1, &r1, 4);
+        __builtin_memcpy(&o2, &r2, 4);
+        __builtin_memcpy(&o3, &r3, 4);
+        H0[c] = o0, L0[c] = o1, H1[c] = o2, L1[c] = o3;
+    }
+}
 __device__ __forceinline__ void unpack_block_sel(const RawBlock &R, int lg, BPlanes &B) {
     const BlockScales s = block_scales(R);
     const ScalePairs p = scale_pairs(s);
@@ -1017,21 +1040,28 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
     // weights of a step: this wavefront's 32 rows x 9 sixteen-byte pieces, piece p = 64*c + lane of
     // chunk c (4.5 chunks, 5 loads); activations: quant slice `wave`, plus the sums (wavefront 0) or
     // the scales (wavefront 1).  Addresses are a uniform base that moves with the cursor plus a lane
-    // offset that is fixed per item.  Registers are short here, so of the five weight offsets only
-    // the first is kept: piece p + 64 = 7 rows + 1 piece further on, one more row where the piece
-    // index wraps past 8.  (Everything else the fetch needs is recomputed from the lane number.)
-    uint32_t w_off0 = 0;
-    // activations: quant slice `wave` of each half in use, plus one of the four small pieces: sums
-    // (wavefronts 0, 2) and scales (1, 3) of the first (0, 1) and second half (2, 3)
-    const bool x_sums = (wave & 1) == 0;
+    // offset that is fixed per item.
+    // Per item, kept in registers (recomputing them from the lane number for every request cost ~60 vector
+    // instructions a step): the five weight offsets w_off (rows past the matrix, in a last partial row group,
+    // fetch the matrix's last piece instead) and the offsets of the activation pieces.
+    uint32_t w_off[5] = {0, 0, 0, 0, 0};
     auto opaque_lane = [&]() {  // the lane number as a value the compiler cannot hoist expressions of
         int l = lane;
         asm volatile("" : "+v"(l));
         return l;
     };
+    // activations: quant slice `wave` of each half in use, plus one of the four small pieces: sums
+    // (wavefronts 0, 2) and scales (1, 3) of the first (0, 1) and second half (2, 3)
+    const bool x_sums = (wave & 1) == 0;
+    const bool x_small = wave < 4, x_second = wave >= 2;  // fetches a small piece at all; the second half's
+    uint32_t qa_off, qb_off, x_off;
+    if (!GATHER) {
+        qa_off = (uint32_t)(wave * 1024 + lane * 16);
+        qb_off = qa_off + (uint32_t)nb * 8192;
+        x_off = x_sums ? (uint32_t)lane * 16 : (uint32_t)(lane & 31) * 4;  // both lane halves fetch the same 32 scales
+    }
     const uint8_t *f_w, *f_x;
     const int8_t *f_q;
-    uint32_t f_src = 0;  // GATHER: this lane's source rows of the cursor's tile (row lane % 32 of either half)
     const uint32_t lds_src = lds_address(lds + L::OFF_SRC);
     int f_ord = 0, f_kb = 0, f_step = 0;
     bool f_two = false;  // the cursor's tile has rows in its second half
@@ -1041,15 +1071,31 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         item_of(ord, t, m, rg);
         item_info(ord, expert, count, y_row);
         f_w = (m ? g.W[1] : g.W[0]) + (size_t)expert * g.rows * g.row_stride;
-        const int l = opaque_lane();
-        w_off0 = (uint32_t)(rg * (32 * L::RG) + wave * 32 + l / 9) * (uint32_t)g.row_stride + (uint32_t)(l % 9) * 16;
+        const uint32_t stride = (uint32_t)g.row_stride, r0 = (uint32_t)lane % 9;
+        const uint32_t off0 = (uint32_t)(rg * (32 * L::RG) + wave * 32 + lane / 9) * stride + r0 * 16;
+        const uint32_t last = (uint32_t)(g.rows - 1) * stride + 128;
+#pragma unroll
+        for (int c = 0; c < 5; c++) {
+            // piece p + 64 = 7 rows + 1 piece further on, one more row where the piece index wraps past 8
+            w_off[c] = min(off0 + c * (7 * stride + 16) + (r0 + c >= 9 ? stride - Q4_K_BYTES : 0u), last);
+            asm volatile("" : "+v"(w_off[c]));
+        }
         f_two = count > 32;
         if (GATHER) {
-            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(f_src) : "v"(lds_src + ord * 128 + (l & 31) * 4));
+            // piece (row, 16-byte half hk) of quant slice `wave`: bytes 32 * wave + 16 * hk of the row's block;
+            // of the sums: 16 * hk of the block's 32 bytes; the scale: the block's 4 bytes
+            uint32_t src;  // this lane's source rows of the tile (row lane % 32 of either half)
+            asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(src) : "v"(lds_src + ord * 128 + (lane & 31) * 4));
+            const uint32_t row_a = src & 0xffffu, row_b = src >> 16, hk = (uint32_t)(lane >> 5) * 16;
+            const uint32_t cols = (uint32_t)nb * QK_K, row = x_second ? row_b : row_a;
+            qa_off = row_a * cols + (uint32_t)wave * 32 + hk;
+            qb_off = row_b * cols + (uint32_t)wave * 32 + hk;
+            x_off = x_sums ? row * (uint32_t)nb * 32 + hk : row * (uint32_t)nb * 4;
+            asm volatile("" : "+v"(qa_off), "+v"(qb_off), "+v"(x_off));
             f_q = g.src.q;
             f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.src.bs) : reinterpret_cast<const uint8_t *>(g.src.d);
         } else {
-            const size_t rec = (size_t)(2 * t + (wave >> 1 & 1)) * nb;  // the small piece's half
+            const size_t rec = (size_t)(2 * t + (x_second ? 1 : 0)) * nb;  // the small piece's half
             f_q = g.a.q + (size_t)2 * t * nb * 8192;
             f_x = x_sums ? reinterpret_cast<const uint8_t *>(g.a.bs + rec * 512)
                          : reinterpret_cast<const uint8_t *>(g.a.d + rec * 32);
@@ -1057,53 +1103,24 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
     };
     auto fetch_acts = [&]() {  // of the cursor's step
         uint8_t *st = lds + L::OFF_A + (f_step & 3) * L::A_STAGE;
-        const int l = opaque_lane();
-        if (GATHER) {
-            // piece (row, 16-byte half hk) of quant slice `wave`: bytes 32 * wave + 16 * hk of the row's block;
-            // of the sums: 16 * hk of the block's 32 bytes; the scale: the block's 4 bytes
-            const uint32_t row_a = f_src & 0xffffu, row_b = f_src >> 16, hk = (uint32_t)(l >> 5) * 16;
-            const uint32_t cols = (uint32_t)nb * QK_K;
-            load_to_lds16(f_q + (row_a * cols + (uint32_t)wave * 32 + hk), st + wave * 1024);
-            issued = 1;
-            if (f_two) {
-                load_to_lds16(f_q + (row_b * cols + (uint32_t)wave * 32 + hk), st + L::A_HALF + wave * 1024);
-                issued = 2;
-            }
-            if (wave < 2 || (wave < 4 && f_two)) {
-                uint8_t *half = st + (wave >> 1) * L::A_HALF;
-                const uint32_t row = (wave >> 1) ? row_b : row_a;
-                if (x_sums) load_to_lds16(f_x + (row * (uint32_t)nb * 32 + hk), half + L::A_BS);
-                else load_to_lds4(f_x + row * (uint32_t)nb * 4, half + L::A_DA);
-                issued++;
-            }
-            return;
-        }
-        const uint32_t q_off = (uint32_t)(wave * 1024 + l * 16);
-        const uint32_t x_off = x_sums ? (uint32_t)l * 16 : (uint32_t)(l & 31) * 4;
-        load_to_lds16(f_q + q_off, st + wave * 1024);
+        load_to_lds16(f_q + qa_off, st + wave * 1024);
         issued = 1;
         if (f_two) {
-            load_to_lds16(f_q + (size_t)nb * 8192 + q_off, st + L::A_HALF + wave * 1024);
+            load_to_lds16(f_q + qb_off, st + L::A_HALF + wave * 1024);
             issued = 2;
         }
-        if (wave < 2 || (wave < 4 && f_two)) {
-            uint8_t *half = st + (wave >> 1) * L::A_HALF;
+        if (x_small && (!x_second || f_two)) {
+            uint8_t *half = st + (x_second ? L::A_HALF : 0);
             if (x_sums) load_to_lds16(f_x + x_off, half + L::A_BS);
-            else load_to_lds4(f_x + x_off, half + L::A_DA);  // both lane halves fetch the same 32 scales
+            else load_to_lds4(f_x + x_off, half + L::A_DA);
             issued++;
         }
     };
     auto fetch_weights = [&]() {  // of the cursor's step; moves the cursor on
         uint8_t *st = lds + (f_step & 1) * L::W_STAGE + wave * L::W_WAVE;
-        const int l = opaque_lane();
-        const uint32_t r0 = (uint32_t)l % 9, stride = (uint32_t)g.row_stride;
-        // rows past the matrix (a last, partial row group) fetch its last piece instead
-        const uint32_t last = (uint32_t)(g.rows - 1) * stride + 128;
 #pragma unroll
-        for (int c = 0; c < 5; c++) {
-            const uint32_t off = w_off0 + c * (7 * stride + 16) + (r0 + c >= 9 ? stride - Q4_K_BYTES : 0u);
-            if (c < 4 || l < 32) load_to_lds16(f_w + min(off, last), st + c * 1024);
-        }
+        for (int c = 0; c < 5; c++)
+            if (c < 4 || lane < 32) load_to_lds16(f_w + w_off[c], st + c * 1024);
         issued += 5;
         f_step++;
         f_w += Q4_K_BYTES;
@@ -1168,11 +1185,12 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
         }
         const BlockScales sc = block_scales(R);
         const int lg_next = opaque_lane() >> 5;
+        const ScalePairs sp = scale_pairs(sc);
         multiply_half(st, accF0, B, [&](int i, v16i &) {
-            if (i == 0) unpack_pair(R.q0, sc.sc_lo, Bnext.H0, Bnext.L0, Bnext.H1, Bnext.L1);
-            if (i == 2) unpack_pair(R.q1, sc.sc_lo >> 16, Bnext.H2, Bnext.L2, Bnext.H3, Bnext.L3);
-            if (i == 4) unpack_pair(R.q2, sc.sc_hi, Bnext.H4, Bnext.L4, Bnext.H5, Bnext.L5);
-            if (i == 6) unpack_pair(R.q3, sc.sc_hi >> 16, Bnext.H6, Bnext.L6, Bnext.H7, Bnext.L7);
+            if (i == 0) unpack_pair_free(R.q0, sp.p0, sp.p1, Bnext.H0, Bnext.L0, Bnext.H1, Bnext.L1);
+            if (i == 2) unpack_pair_free(R.q1, sp.p2, sp.p3, Bnext.H2, Bnext.L2, Bnext.H3, Bnext.L3);
+            if (i == 4) unpack_pair_free(R.q2, sp.p4, sp.p5, Bnext.H4, Bnext.L4, Bnext.H5, Bnext.L5);
+            if (i == 6) unpack_pair_free(R.q3, sp.p6, sp.p7, Bnext.H6, Bnext.L6, Bnext.H7, Bnext.L7);
             if (i == 8) unpack_rest(R, sc, lg_next, Bnext);
         });
         if (c_count > 32) multiply_half(st + L::A_HALF, accF1, B, NothingBetween());
@@ -1212,7 +1230,7 @@ __global__ __launch_bounds__(512) void gemm_q4_k_stream_kernel(StreamArgs g) {
 
     {  // step 0's weights into the first set; its stage is refilled at once
         const RawBlock R = raw_of_step(0);
-        unpack_block(R, lg, B0);
+        unpack_block_sel(R, lg, B0);
         if (total_steps > 2) {
             fetch_acts();
             fetch_weights();
