@@ -535,8 +535,9 @@ def main():
             for w in w40:
                 w.release()
             del d40
-            # Q5_0 and MXFP4 batches: decoded into the Q8_0 planar form in scratch memory, then the Q8_0 kernel
-            for kind_o, name_o in ((fa.Q5_0, "Q5_0"), (fa.MXFP4, "MXFP4")):
+            # Q5_0 and MXFP4 batches: decoded into the Q8_0 planar form in scratch memory, then the Q8_0 kernel;
+            # IQ4_XS: decoded to signed bytes with integer block scales, the same kernel's form for Q8_K activations
+            for kind_o, name_o in ((fa.Q5_0, "Q5_0"), (fa.MXFP4, "MXFP4"), (fa.IQ4_XS, "IQ4_XS")):
                 do = torch.from_numpy(random_blocks(kind_o, cols, rows, seed=85)).to(dev)
                 wo = [fa.Weights.from_device(kind_o, do, cols, rows) for _ in range(4)]
 

@@ -25,7 +25,8 @@ impl BackendCaps for Hip {
     fn gemm_supported(kind: QuantKind) -> bool {
         matches!(
             kind,
-            QuantKind::Q4_0 | QuantKind::Q5_0 | QuantKind::Q8_0 | QuantKind::Q4K | QuantKind::Q5K | QuantKind::Q6K | QuantKind::Mxfp4Gguf
+            QuantKind::Q4_0 | QuantKind::Q5_0 | QuantKind::Q8_0 | QuantKind::Q4K | QuantKind::Q5K | QuantKind::Q6K
+                | QuantKind::IQ4XS | QuantKind::Mxfp4Gguf
         )
     }
 }

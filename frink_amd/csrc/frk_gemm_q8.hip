@@ -117,7 +117,14 @@ __device__ __forceinline__ int q4_0_bytes(uint32_t t) {
 // Q4: the weights are Q4_0 (dot_q4_0_q8, crates/frink-quant/src/lib.rs:772-796) -- 16 bytes of nibbles a
 // block, byte i holding element i low and element i + 16 high -- and become the same signed bytes
 // nibble - 8 on their way from the staging registers to LDS; everything behind that is the Q8_0 kernel.
-template <int TT, int RT, bool Q4>
+//
+// SUB: blocks with an integer scale of their own under a float scale per 256 (IQ4_XS decoded to signed bytes:
+// dot_iq4_xs_q8k, crates/frink-quant/src/iq4_xs_q8.rs:50-67), against Q8_K activations -- the 16 bytes behind a
+// weight row's chunk hold the eight block scales ls - 32 as signed bytes and the f16 d, a token's hold its f32 d.
+// A block's sums are multiplied by its integer scale and added up as integers; once a chunk (one block of 256)
+// the integers meet the float scales d_w * d_a, whose outer product a v_mfma_f32_32x32x2f32 returns in the
+// registers' layout.
+template <int TT, int RT, bool Q4, bool SUB = false>
 __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs g) {
     constexpr int NT = 64 * TT * RT;
     // 16-byte pieces a thread stages per chunk (a piece of Q4_0 nibbles is a whole block)
@@ -147,9 +154,11 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     // (RT + TT) / 2 wavefronts stages those of weight row i, or of token i - 32 * RT, of the tile.
     const bool stages_scales = wave < (RT + TT) / 2;
     const bool stages_weight_scales = tid < 32 * RT;
+    // (SUB: a token's scales are one f32 per chunk, [M][nb / 8])
     const uint8_t *s_src = stages_weight_scales
                                ? g.W + (size_t)min(row0 + tid, g.rows - 1) * g.row_stride + g.off_d
-                               : (const uint8_t *)(g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * ((g.nb + 7) & ~7));
+                               : SUB ? (const uint8_t *)g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * (g.nb / 8) * 4
+                                     : (const uint8_t *)(g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * ((g.nb + 7) & ~7));
     uint8_t *s_dst = stages_weight_scales ? lds_w + tid * Q8_LDS_ROW + 256 : lds_a + (tid - 32 * RT) * Q8_LDS_ROW + 256;
     const bool low_half = lane < 32;
     const int n_full = g.nb / Q8_CHUNK_BLOCKS;  // chunks of eight whole blocks
@@ -185,7 +194,9 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
                 in.w[i - AP] = *reinterpret_cast<const q8_v4i *>(w_src + (size_t)row * g.row_stride + piece);
             }
         } else if (stages_scales) {
-            if (whole || !stages_weight_scales || blk0 + 8 <= g.nb) {
+            if (SUB && !stages_weight_scales) {
+                in.s = q8_v4i{*reinterpret_cast<const int *>(s_src + (size_t)chunk * 4), 0, 0, 0};
+            } else if (whole || !stages_weight_scales || blk0 + 8 <= g.nb) {
                 // (a token's scales are padded with zeros to whole chunks)
                 in.s = *reinterpret_cast<const q8_v4i *>(s_src + (size_t)blk0 * 2);
             } else {  // a weight row's last chunk when it is not a multiple of 256 columns
@@ -220,16 +231,25 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
             };
             auto products = [&](int b, const q8_v4i &qa, const q8_v4i &qw, q8_v16i &isum, q8_v16f &scale) {
                 isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(qa, qw, zero_i, 0, 0, 0);
-                scale = __builtin_amdgcn_mfma_f32_32x32x8f16(q8_as_k0(q8_pick(sa, b)), q8_as_k0(q8_pick(sw, b)), zero_f, 0, 0, 0);
+                if (!SUB)
+                    scale = __builtin_amdgcn_mfma_f32_32x32x8f16(q8_as_k0(q8_pick(sa, b)), q8_as_k0(q8_pick(sw, b)), zero_f, 0, 0, 0);
             };
+            uint32_t ls_lo = 0, ls_hi = 0;  // SUB: this lane's weight row's eight block scales, a signed byte each
+            float sub_da = 0.0f, sub_dw = 0.0f;
             {
                 const q8_v4i va = *reinterpret_cast<const q8_v4i *>(frag_a + (c & 1) * LDS_COPY - (lane >> 5) * 16 + 256);
                 const q8_v4i vw = *reinterpret_cast<const q8_v4i *>(frag_w + (c & 1) * LDS_COPY - (lane >> 5) * 16 + 256);
+                if (SUB) {
+                    ls_lo = (uint32_t)vw[0], ls_hi = (uint32_t)vw[1];
+                    sub_da = low_half ? __uint_as_float((uint32_t)va[0]) : 0.0f;
+                    sub_dw = low_half ? h2f((uint32_t)vw[2] & 0xffffu) : 0.0f;
+                }
                 sa = Q8Scales{low_half ? (uint32_t)va[0] : 0u, low_half ? (uint32_t)va[1] : 0u, low_half ? (uint32_t)va[2] : 0u,
                               low_half ? (uint32_t)va[3] : 0u};
                 sw = Q8Scales{low_half ? (uint32_t)vw[0] : 0u, low_half ? (uint32_t)vw[1] : 0u, low_half ? (uint32_t)vw[2] : 0u,
                               low_half ? (uint32_t)vw[3] : 0u};
             }
+            q8_v16i iacc = zero_i;
             q8_v4i qa1, qw1, qa2, qw2;
             q8_v16i isum_next;
             q8_v16f scale_next;
@@ -248,13 +268,26 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
 #pragma unroll
                     for (int i = b * LOADS_A_BLOCK; i < (b + 1) * LOADS_A_BLOCK && i < LOADS; i++) fetch(i, c + 2, true, in);
                 }
+                if (SUB) {
+                    // |ls| <= 32 and |isum| <= 32 * 127 * 127: 24-bit factors, and eight blocks' products fit 32 bits
+                    const int ls = (int)(int8_t)(((b < 4 ? ls_lo : ls_hi) >> (8 * (b & 3))) & 0xff);
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[r] = __builtin_fmaf(scale[r], (float)isum[r], acc[r]);
+                    for (int r = 0; r < 16; r++) iacc[r] = __mul24(isum[r], ls) + iacc[r];
+                    if (b == Q8_CHUNK_BLOCKS - 1) {
+                        const q8_v16f dd = __builtin_amdgcn_mfma_f32_32x32x2f32(sub_da, sub_dw, zero_f, 0, 0, 0);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[r] = __builtin_fmaf(dd[r], (float)iacc[r], acc[r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[r] = __builtin_fmaf(scale[r], (float)isum[r], acc[r]);
+                }
                 if (b + 2 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS reads
                 if (b + 1 < Q8_CHUNK_BLOCKS) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMAs
                 // keeps the float step here: sunk towards the loop's end it would leave every
                 // block's matrix results alive at once
                 asm volatile("" : "+v"(acc));
+                if (SUB) asm volatile("" : "+v"(iacc));
                 __builtin_amdgcn_sched_barrier(0);
                 qa1 = qa2, qw1 = qw2;
             }
@@ -337,6 +370,8 @@ size_t gemm_q8_0_workspace_bytes(size_t M, size_t cols, size_t rows) {
     return round_up(M * cols, 256) + round_up(M * round_up(cols / 32, 8) * 2, 256) + (ks > 1 ? (size_t)ks * M * rows * sizeof(float) : 0);
 }
 
+static int launch_q8_mfma(Q8GemmArgs g, bool q4, bool sub, hipStream_t s);
+
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s) {
     return launch_gemm_q8_0_planar(w->dev, w->layout.row_stride, w->layout.off_a, w->rows, w->cols, w->kind == FRK_KIND_Q4_0, x, M, y,
                                    ws, s);
@@ -368,42 +403,79 @@ int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, s
     g.rows = (int)w->rows;
     g.nb = (int)(w->cols / 32);
     g.M = (int)M;
-    // the widest token tile the batch fills; two row tiles per workgroup with it, one wavefront a
-    // workgroup for the thinnest batches, whose grids are small
+    g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));
+    return launch_q8_mfma(g, q4, false, s);
+}
+
+// The kernel over operands that are ready: the widest token tile the batch fills; two row tiles per workgroup
+// with it, one wavefront a workgroup for the thinnest batches, whose grids are small.  g.partial: room for the
+// parts' sums where the chunks are split (q8_0_split).
+static int launch_q8_mfma(Q8GemmArgs g, bool q4, bool sub, hipStream_t s) {
     auto lds_bytes = [](int tt, int rt) { return (size_t)2 * (tt + rt) * 32 * Q8_LDS_ROW; };
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
-        const void *big[4] = {reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, false>),
+        const void *big[6] = {reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, false>),
                               reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, true>),
                               reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, false>),
-                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, true>)};
-        for (int i = 0; i < 4; i++) {
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, true>),
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<4, 2, false, true>),
+                              reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, false, true>)};
+        for (int i = 0; i < 6; i++) {
             hipError_t e = hipFuncSetAttribute(big[i], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(4, 2));
             if (e != hipSuccess)
                 return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", lds_bytes(4, 2), hipGetErrorString(e));
         }
         sized = true;
     }
-    const int ks = q8_0_split(w->rows, M, (size_t)g.nb);
+    const size_t rows = (size_t)g.rows, M = (size_t)g.M;
+    const int ks = q8_0_split(rows, M, (size_t)g.nb);
     g.k_split = ks;
-    g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));
     const unsigned kz = (unsigned)ks;
+#define FRK_GO(TT, RT, grid, threads)                                                                                        \
+    do {                                                                                                                     \
+        if (sub) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<TT, RT, false, true>), grid, dim3(threads), lds_bytes(TT, RT), s, g); \
+        else if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<TT, RT, true>), grid, dim3(threads), lds_bytes(TT, RT), s, g);  \
+        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<TT, RT, false>), grid, dim3(threads), lds_bytes(TT, RT), s, g);         \
+    } while (0)
     if (M > 64) {
-        const dim3 grid((unsigned)((w->rows + 63) / 64), (unsigned)((M + 127) / 128), kz);
-        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, true>), grid, dim3(512), lds_bytes(4, 2), s, g);
-        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<4, 2, false>), grid, dim3(512), lds_bytes(4, 2), s, g);
+        const dim3 grid((unsigned)((rows + 63) / 64), (unsigned)((M + 127) / 128), kz);
+        FRK_GO(4, 2, grid, 512);
     } else if (M > 32) {
-        const dim3 grid((unsigned)((w->rows + 63) / 64), 1u, kz);
-        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, true>), grid, dim3(256), lds_bytes(2, 2), s, g);
-        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, false>), grid, dim3(256), lds_bytes(2, 2), s, g);
+        const dim3 grid((unsigned)((rows + 63) / 64), 1u, kz);
+        FRK_GO(2, 2, grid, 256);
     } else {
-        const dim3 grid((unsigned)((w->rows + 31) / 32), 1u, kz);
-        if (q4) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, true>), grid, dim3(64), lds_bytes(1, 1), s, g);
-        else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<1, 1, false>), grid, dim3(64), lds_bytes(1, 1), s, g);
+        const dim3 grid((unsigned)((rows + 31) / 32), 1u, kz);
+        FRK_GO(1, 1, grid, 64);
     }
+#undef FRK_GO
     FRK_LAUNCH_CHECK("gemm_q8_0_mfma");
-    if (ks > 1) return launch_sum_parts(g.partial, ks, M * w->rows, y, s);
+    if (ks > 1) return launch_sum_parts(g.partial, ks, M * rows, g.y, s);
     return FRK_OK;
+}
+
+// Rows of signed bytes with an integer scale per 32 and an f16 scale per 256 in the slots behind the quants (SUB
+// above) against Q8_K activations: quants aq [M][cols], scales ad [M][cols / 256].  `partial`: room for
+// gemm_sub_partial_bytes.
+size_t gemm_sub_partial_bytes(size_t M, size_t cols, size_t rows) {
+    const int ks = q8_0_split(rows, M, cols / 32);
+    return ks > 1 ? (size_t)ks * M * rows * sizeof(float) : 0;
+}
+int launch_gemm_sub_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, const int8_t *aq,
+                           const float *ad, size_t M, float *y, void *partial, hipStream_t s) {
+    if (M > (size_t)1 << 30 || rows > (size_t)1 << 30 || cols % QK_K)
+        return set_error(FRK_ERR_SHAPE, "gemm_sub: %zu activation rows x %zu weight rows x %zu columns", M, rows, cols);
+    Q8GemmArgs g;
+    g.W = W;
+    g.row_stride = row_stride;
+    g.off_d = off_d;
+    g.aq = aq;
+    g.ad = reinterpret_cast<const uint16_t *>(ad);
+    g.y = y;
+    g.rows = (int)rows;
+    g.nb = (int)(cols / 32);
+    g.M = (int)M;
+    g.partial = (float *)partial;
+    return launch_q8_mfma(g, false, true, s);
 }
 
 }  // namespace frk

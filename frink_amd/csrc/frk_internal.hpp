@@ -232,6 +232,12 @@ int launch_sum_parts(const float *partial, int parts, size_t n, float *y, hipStr
 int launch_gemm_q8_0(const frk_weights *w, const float *x, size_t M, float *y, void *ws, hipStream_t s);
 int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, bool q4, const float *x,
                             size_t M, float *y, void *ws, hipStream_t s);
+// IQ4_XS on the matrix cores: the rows decoded to signed bytes with their block scales (launch_iq4_xs_to_sub_planar,
+// rows of layout_for(FRK_KIND_Q8_0, cols)'s stride) against Q8_K activations
+int launch_iq4_xs_to_sub_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s);
+size_t gemm_sub_partial_bytes(size_t M, size_t cols, size_t rows);
+int launch_gemm_sub_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, const int8_t *aq,
+                           const float *ad, size_t M, float *y, void *partial, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by
 // tiles[t] = {expert, 64*t, rows in use, 0}; expert e owns rows [e*rows_e, (e+1)*rows_e) of the
 // stacked matrices; *n_tiles <= max_tiles.  w1/y1 (nullable) is a second stacked matrix over the

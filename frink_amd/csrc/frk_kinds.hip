@@ -465,6 +465,39 @@ int launch_units_to_q8_0_planar(const frk_weights *w, uint8_t *dst, size_t dst_s
     return FRK_OK;
 }
 
+// IQ4_XS into the form the sub-scaled matrix-core GEMM reads: the codebook's signed bytes [cols], then per block of
+// 256 a 16-byte slot -- the eight block scales ls - 32 as signed bytes, the f16 d, zeros.
+__global__ __launch_bounds__(256) void iq4_xs_to_sub_planar_kernel(const uint8_t *__restrict__ W, size_t row_stride, size_t rows,
+                                                                  size_t units, uint8_t *__restrict__ dst, size_t dst_stride,
+                                                                  size_t off_d) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * units) return;
+    const size_t r = i / units, u = i % units;
+    uint32_t c[8];
+    float scale;
+    int scale_i;
+    unit_codes<FRK_KIND_IQ4_XS>(W + r * row_stride, (int)u, c, scale, scale_i);
+    uint4 *q = reinterpret_cast<uint4 *>(dst + r * dst_stride + u * 32);
+    q[0] = make_uint4(c[0], c[1], c[2], c[3]);
+    q[1] = make_uint4(c[4], c[5], c[6], c[7]);
+    uint8_t *slot = dst + r * dst_stride + off_d + (u >> 3) * 16;
+    slot[u & 7] = (uint8_t)(int8_t)scale_i;
+    if ((u & 7) == 0) {
+        reinterpret_cast<uint16_t *>(slot)[4] = f2h_bits(scale);  // (d is an f16 value: the bits it came from)
+        reinterpret_cast<uint16_t *>(slot)[5] = 0;
+        reinterpret_cast<uint32_t *>(slot)[3] = 0;
+    }
+}
+int launch_iq4_xs_to_sub_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s) {
+    if (w->kind != FRK_KIND_IQ4_XS) return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has no sub-scaled planar form", w->kind);
+    const size_t units = w->cols / 32;
+    const unsigned g = (unsigned)((w->rows * units + 255) / 256);
+    hipLaunchKernelGGL(iq4_xs_to_sub_planar_kernel, dim3(g), dim3(256), 0, s, w->dev, w->layout.row_stride, w->rows, units, dst,
+                       dst_stride, off_d);
+    FRK_LAUNCH_CHECK("iq4_xs_to_sub_planar");
+    return FRK_OK;
+}
+
 __global__ __launch_bounds__(256) void mxfp4_scale_range_kernel(const uint8_t *__restrict__ W, size_t row_stride, size_t rows, size_t units,
                                                                int *__restrict__ range) {
     int lo = 255, hi = 0;

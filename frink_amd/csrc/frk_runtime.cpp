@@ -283,9 +283,9 @@ const char *frk_hip_matvec_kernel(int kind) {
 }
 int frk_hip_has_launch(int kind) { return frk_hip_matvec_kernel(kind) != nullptr; }
 int frk_hip_gemm_supported(int kind) {
-    // (Q5_0 and MXFP4 through the Q8_0 matrix-core kernel; IQ4_XS batches run the integer decode kernel per row)
+    // (Q5_0 and MXFP4 through the Q8_0 matrix-core kernel, IQ4_XS through its form with integer block scales)
     return kind == FRK_KIND_Q4_K || kind == FRK_KIND_Q5_K || kind == FRK_KIND_Q6_K || kind == FRK_KIND_Q8_0 ||
-           kind == FRK_KIND_Q4_0 || kind == FRK_KIND_Q5_0 || kind == FRK_KIND_MXFP4;
+           kind == FRK_KIND_Q4_0 || kind == FRK_KIND_Q5_0 || kind == FRK_KIND_MXFP4 || kind == FRK_KIND_IQ4_XS;
 }
 int frk_hip_block_bytes(int kind) { return block_bytes(kind); }
 int frk_hip_block_elems(int kind) { return block_elems(kind); }
@@ -653,6 +653,25 @@ static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, fl
     }
     if (!gemv_units_int_fits(w))
         return set_error(FRK_ERR_UNSUPPORTED, "the integer tier of quant kind %d does not take rows of %zu columns", w->kind, w->cols);
+    if (w->kind == FRK_KIND_IQ4_XS && batch >= 4) {
+        // the matrix cores: the rows decoded to signed bytes with their block scales, the batch quantized to Q8_K
+        const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
+        const size_t planar_bytes = round_up(planar.row_stride * w->rows + 256, 256);
+        const size_t n = batch * w->cols;
+        const size_t q_bytes = round_up(n, 256), d_bytes = round_up(n / QK_K * 4, 256), b_bytes = round_up(n / 16 * 2, 256);
+        void *ws = nullptr;
+        int rc = scratch.get(planar_bytes + q_bytes + d_bytes + b_bytes + gemm_sub_partial_bytes(batch, w->cols, w->rows), s, &ws);
+        if (rc) return rc;
+        uint8_t *decoded = (uint8_t *)ws;
+        int8_t *q = (int8_t *)((char *)ws + planar_bytes);
+        float *d = (float *)((char *)q + q_bytes);
+        int16_t *bs = (int16_t *)((char *)d + d_bytes);
+        rc = launch_iq4_xs_to_sub_planar(w, decoded, planar.row_stride, planar.off_a, s);
+        if (rc) return rc;
+        rc = launch_quantize_q8_k(x, n, q, d, bs, s);
+        if (rc) return rc;
+        return launch_gemm_sub_planar(decoded, planar.row_stride, planar.off_a, w->rows, w->cols, q, d, batch, y, (char *)bs + b_bytes, s);
+    }
     if (w->kind == FRK_KIND_IQ4_XS) {  // one Q8_K quantization of the batch, the decode kernel per row
         Q8KActs a;
         int rc = quantize_acts_q8_k(w, x, batch, s, scratch, &a);

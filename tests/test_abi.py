@@ -43,7 +43,7 @@ def test_every_kind_the_backend_claims_can_be_launched():
         else:
             assert name is None and fa.lib().frk_hip_block_bytes(kind) == 0
     assert all(fa.lib().frk_hip_gemm_supported(k) for k in (fa.Q4_0, fa.Q4_K, fa.Q5_K, fa.Q6_K, fa.Q8_0, fa.Q5_0, fa.MXFP4))
-    assert not fa.lib().frk_hip_gemm_supported(fa.IQ4_XS)  # (its batches run the integer decode kernel per row)
+    assert fa.lib().frk_hip_gemm_supported(fa.IQ4_XS)
     assert not fa.lib().frk_hip_worth_a_gemm(1) and fa.lib().frk_hip_worth_a_gemm(2)
 
 

@@ -1232,12 +1232,16 @@ def test_other_kinds_integer_gemv_matches_the_oracle(fa, kind, rows, cols):
     (fo.Q5_0, 70, 1024, 2), (fo.Q5_0, 300, 4096, 3), (fo.Q5_0, 96, 512, 4), (fo.Q5_0, 200, 1056, 40), (fo.Q5_0, 130, 2048, 130),
     (fo.Q5_0, 64, 96, 33), (fo.MXFP4, 70, 1024, 2), (fo.MXFP4, 64, 2880, 4), (fo.MXFP4, 200, 1056, 40), (fo.MXFP4, 130, 2048, 130),
     (fo.MXFP4, 96, 32, 7), (fo.IQ4_XS, 70, 1024, 2), (fo.IQ4_XS, 130, 4096, 5), (fo.IQ4_XS, 40, 768, 17),
+    (fo.IQ4_XS, 64, 256, 4), (fo.IQ4_XS, 100, 2304, 33), (fo.IQ4_XS, 200, 1280, 64), (fo.IQ4_XS, 130, 2048, 130),
+    (fo.IQ4_XS, 33, 14336, 40), (fo.IQ4_XS, 1000, 512, 300),
 ])
 def test_other_kinds_batches_take_the_integer_tier(fa, kind, rows, cols, batch):
     """A batch of Q5_0 / MXFP4 / IQ4_XS is the reference's integer tier (q8_row_dot / q8k_row_dot per (row, activation),
     crates/frink-core/src/weight_matrix.rs:392-420): up to three rows the decode kernel per row, from four on Q5_0 and
     MXFP4 decoded into the Q8_0 planar form and multiplied on the matrix cores -- every workgroup shape of that kernel,
-    ragged tiles, rows that are not a multiple of its 256-column step; IQ4_XS the decode kernel per row at any size."""
+    ragged tiles, rows that are not a multiple of its 256-column step -- and IQ4_XS decoded to signed bytes with their
+    integer block scales, against Q8_K activations (the same kernel's form with a float scale per 256; long rows
+    split between workgroups, grids of several token tiles)."""
     from frink_amd import synth
     print("other kinds, batch", kind, rows, cols, batch, flush=True)
     data = _other_kind_blocks(kind, rows, cols, seed=kind * 7 + rows + batch)
