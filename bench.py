@@ -606,6 +606,23 @@ def main():
             down6.release()
             for w in experts:
                 w.release()
+            # a layer of MXFP4 experts in gpt-oss-20b's shape (32 experts, top-4, 2880/2880), 512 tokens: the experts
+            # decoded to signed bytes per call, the grouped form of the Q8_0 matrix-core kernel
+            E4, K4, H4, F4 = 32, 4, 2880, 2880
+            ex4 = [fa.Weights.from_device(fa.MXFP4, torch.from_numpy(random_blocks(fa.MXFP4, r, c, seed=90 + j)).to(dev), r, c)
+                   for j, (r, c) in enumerate(((E4 * F4, H4), (E4 * F4, H4), (E4 * H4, F4)))]
+            xm4 = torch.from_numpy(synth.activations(9, T, H4)).to(dev)
+            ids4, wts4 = fa.route_top_k_softmax(torch.from_numpy(synth.normal(10, T * E4).reshape(T, E4)).to(dev), K4, True)
+            ym4 = torch.empty((T, H4), dtype=torch.float32, device=dev)
+
+            def step4e(i):
+                fa.moe_ffn(ex4[0], ex4[1], ex4[2], E4, xm4, ids4, wts4, out=ym4)
+            _, t = timed(step4e, 20, 10)
+            extra["MoE layer 32x top-4, 2880/2880, 512 tokens, MXFP4 experts"] = {
+                "us_per_step": round(t / 20 * 1e6, 2), "tokens_per_s": round(T / (t / 20), 0),
+                "TOPS": round(2.0 * T * K4 * 3 * F4 * H4 / (t / 20) / 1e12, 1)}
+            for w in ex4:
+                w.release()
         if want('thin'):
             # batched decode, M=8 (weights read once per batch), and the whole decode FFN in one call
             # (gate and up share one quantized activation, SwiGLU, down)

@@ -45,6 +45,11 @@ struct Q8GemmArgs {
     int rows, nb, M;
     int k_split;     // 1, or 2/4/8: blockIdx.z takes that share of the 256-column chunks (whole pairs of them)
     float *partial;  // [k_split][M][rows], added up in order afterwards
+    // GROUPED: W stacks the groups' matrices of `rows` rows each; tile blockIdx.y = {group, first row of the grouped
+    // order, rows in use, first row of y} multiplies the activation rows src_rows[first + r] (first + r without a list)
+    const int4 *tiles;
+    const int *n_tiles;
+    const int *src_rows;
 };
 
 constexpr int Q8_CHUNK_BLOCKS = 8;   // 256 columns a step
@@ -124,7 +129,11 @@ __device__ __forceinline__ int q4_0_bytes(uint32_t t) {
 // A block's sums are multiplied by its integer scale and added up as integers; once a chunk (one block of 256)
 // the integers meet the float scales d_w * d_a, whose outer product a v_mfma_f32_32x32x2f32 returns in the
 // registers' layout.
-template <int TT, int RT, bool Q4, bool SUB = false>
+//
+// GROUPED: the indexed form (enqueue_mul_mm_grouped_dev, crates/frink-cuda/src/mul_mm_launch.rs:391-470; the MoE
+// prefill over experts of these kinds): a workgroup's tokens are one tile of at most 32 * TT rows of one group, the
+// activation rows come through a list, and the results go to the tile's rows of y.
+template <int TT, int RT, bool Q4, bool SUB = false, bool GROUPED = false>
 __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs g) {
     constexpr int NT = 64 * TT * RT;
     // 16-byte pieces a thread stages per chunk (a piece of Q4_0 nibbles is a whole block)
@@ -136,7 +145,21 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tt = wave % TT, rt = wave / TT;
-    const int tok0 = blockIdx.y * (32 * TT), row0 = blockIdx.x * (32 * RT);
+    const int row0 = blockIdx.x * (32 * RT);
+    int tok0 = blockIdx.y * (32 * TT), tok_end = g.M, y_shift = 0;  // tokens tok0 .. tok_end - 1; token t is row t + y_shift of y
+    if (GROUPED) {
+        if ((int)blockIdx.y >= *g.n_tiles) return;
+        const int4 tile = g.tiles[blockIdx.y];
+        g.W += (size_t)tile.x * g.rows * g.row_stride;
+        tok0 = tile.y;
+        tok_end = tile.y + tile.z;
+        y_shift = tile.w - tile.y;
+    }
+    // the activation row of token t (past the end: the last one again)
+    auto act_row = [&](int t) {
+        t = max(min(t, tok_end - 1), tok0);
+        return GROUPED && g.src_rows ? max(g.src_rows[t], 0) : t;
+    };
     const size_t cols = (size_t)g.nb * 32;
     const int n_chunks = (g.nb + Q8_CHUNK_BLOCKS - 1) / Q8_CHUNK_BLOCKS;
     // this workgroup's chunks c0 .. c1 - 1; c0 is even, so that the chunks of even number are the same
@@ -157,8 +180,8 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     // (SUB: a token's scales are one f32 per chunk, [M][nb / 8])
     const uint8_t *s_src = stages_weight_scales
                                ? g.W + (size_t)min(row0 + tid, g.rows - 1) * g.row_stride + g.off_d
-                               : SUB ? (const uint8_t *)g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * (g.nb / 8) * 4
-                                     : (const uint8_t *)(g.ad + (size_t)min(tok0 + tid - 32 * RT, g.M - 1) * ((g.nb + 7) & ~7));
+                               : SUB ? (const uint8_t *)g.ad + (size_t)act_row(tok0 + tid - 32 * RT) * (g.nb / 8) * 4
+                                     : (const uint8_t *)(g.ad + (size_t)act_row(tok0 + tid - 32 * RT) * ((g.nb + 7) & ~7));
     uint8_t *s_dst = stages_weight_scales ? lds_w + tid * Q8_LDS_ROW + 256 : lds_a + (tid - 32 * RT) * Q8_LDS_ROW + 256;
     const bool low_half = lane < 32;
     const int n_full = g.nb / Q8_CHUNK_BLOCKS;  // chunks of eight whole blocks
@@ -172,6 +195,9 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
     const uint8_t *frag_a = lds_a + (tt * 32 + (lane & 31)) * Q8_LDS_ROW + (lane >> 5) * 16;
     const uint8_t *frag_w = lds_w + (rt * 32 + (lane & 31)) * Q8_LDS_ROW + (lane >> 5) * 16;
 
+    int a_rows[AP];  // the activation rows of this thread's pieces
+#pragma unroll
+    for (int i = 0; i < AP; i++) a_rows[i] = act_row(tok0 + r0 + i * (NT / 16));
     Q8Scales sa, sw;
     // The loads of a chunk: quant piece i < AP + WP, or (i == AP + WP) the scales.  `whole` says that the
     // chunk is known to be eight whole blocks.
@@ -182,8 +208,7 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
         // that is not stored.
         const size_t piece = whole || blk0 + (p >> 1) < g.nb ? (size_t)blk0 * 32 + p * 16 : 0;
         if (i < AP) {
-            const int tok = min(tok0 + r0 + i * (NT / 16), g.M - 1);
-            in.a[i] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)tok * cols + piece);
+            in.a[i] = *reinterpret_cast<const q8_v4i *>(a_src + (size_t)a_rows[i] * cols + piece);
         } else if (i < AP + WP) {
             if (Q4) {
                 const int row = min(row0 + rq + (i - AP) * (NT / 8), g.rows - 1);
@@ -342,7 +367,7 @@ __global__ __launch_bounds__(64 * TT * RT) void gemm_q8_0_mfma_kernel(Q8GemmArgs
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int tok = tok0 + tt * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (tok < g.M) dst[(size_t)tok * g.rows + row] = acc[r];
+            if (tok < tok_end) dst[(size_t)(tok + y_shift) * g.rows + row] = acc[r];
         }
     }
 }
@@ -404,6 +429,9 @@ int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, s
     g.nb = (int)(w->cols / 32);
     g.M = (int)M;
     g.partial = reinterpret_cast<float *>((char *)ws + round_up(M * w->cols, 256) + round_up(M * round_up(w->cols / 32, 8) * 2, 256));
+    g.tiles = nullptr;
+    g.n_tiles = nullptr;
+    g.src_rows = nullptr;
     return launch_q8_mfma(g, q4, false, s);
 }
 
@@ -475,7 +503,64 @@ int launch_gemm_sub_planar(const uint8_t *W, size_t row_stride, size_t off_d, si
     g.nb = (int)(cols / 32);
     g.M = (int)M;
     g.partial = (float *)partial;
+    g.tiles = nullptr;
+    g.n_tiles = nullptr;
+    g.src_rows = nullptr;
     return launch_q8_mfma(g, false, true, s);
+}
+
+// The grouped form over decoded rows (Q8_0 planar form, or with sub = true the form with integer block scales): W
+// stacks the groups' matrices of rows_g rows; tiles / n_tiles as grouped_tiles and moe_group write them (tiles of at
+// most 64 rows); activation row of grouped row r: src_rows[r], or r itself without a list.  aq / ad: the activations'
+// quants and scales as the plain forms above take them ([..][cols]; f16 per 32 padded to eights, or f32 per 256).
+int launch_gemm_planar_grouped(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows_g, size_t cols, bool sub,
+                               const int8_t *aq, const void *ad, const int *src_rows, const int4 *tiles, const int *n_tiles,
+                               size_t max_tiles, float *y, hipStream_t s) {
+    if (rows_g > (size_t)1 << 30 || max_tiles > 65535 || (sub && cols % QK_K))
+        return set_error(FRK_ERR_SHAPE, "grouped gemm: %zu rows a group, %zu tiles, %zu columns", rows_g, max_tiles, cols);
+    if (max_tiles == 0) return FRK_OK;
+    Q8GemmArgs g;
+    g.W = W;
+    g.row_stride = row_stride;
+    g.off_d = off_d;
+    g.aq = aq;
+    g.ad = reinterpret_cast<const uint16_t *>(ad);
+    g.y = y;
+    g.rows = (int)rows_g;
+    g.nb = (int)(cols / 32);
+    g.M = 0;
+    g.k_split = 1;
+    g.partial = nullptr;
+    g.tiles = tiles;
+    g.n_tiles = n_tiles;
+    g.src_rows = src_rows;
+    const size_t lds = (size_t)2 * (2 + 2) * 32 * Q8_LDS_ROW;
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        const void *k[2] = {reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, false, false, true>),
+                            reinterpret_cast<const void *>(&gemm_q8_0_mfma_kernel<2, 2, false, true, true>)};
+        for (int i = 0; i < 2; i++) {
+            hipError_t e = hipFuncSetAttribute(k[i], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(LDS %zu): %s", lds, hipGetErrorString(e));
+        }
+        sized = true;
+    }
+    const dim3 grid((unsigned)((rows_g + 63) / 64), (unsigned)max_tiles, 1u);
+    if (sub) hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, false, true, true>), grid, dim3(256), lds, s, g);
+    else hipLaunchKernelGGL((gemm_q8_0_mfma_kernel<2, 2, false, false, true>), grid, dim3(256), lds, s, g);
+    FRK_LAUNCH_CHECK("gemm_planar_grouped");
+    return FRK_OK;
+}
+
+// quantize_activations_q8 for the kernels above: quants [rows][cols], f16 scales [rows][cols / 32 rounded up to 8]
+size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols) { return round_up(rows * cols, 256) + round_up(rows * round_up(cols / 32, 8) * 2, 256); }
+int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s) {
+    const size_t n_blocks = rows * (cols / 32);
+    if (n_blocks == 0) return FRK_OK;
+    hipLaunchKernelGGL(quantize_q8_0_gemm_kernel, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, s, x, n_blocks,
+                       (int)(cols / 32), q, d);
+    FRK_LAUNCH_CHECK("quantize_q8_0_gemm");
+    return FRK_OK;
 }
 
 }  // namespace frk

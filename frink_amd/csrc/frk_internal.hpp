@@ -236,6 +236,18 @@ int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, s
 // rows of layout_for(FRK_KIND_Q8_0, cols)'s stride) against Q8_K activations
 int launch_iq4_xs_to_sub_planar(const frk_weights *w, uint8_t *dst, size_t dst_stride, size_t off_d, hipStream_t s);
 size_t gemm_sub_partial_bytes(size_t M, size_t cols, size_t rows);
+// the grouped form over decoded rows of either form, and the Q8_0 activation blocks it reads
+int launch_gemm_planar_grouped(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows_g, size_t cols, bool sub,
+                               const int8_t *aq, const void *ad, const int *src_rows, const int4 *tiles, const int *n_tiles,
+                               size_t max_tiles, float *y, hipStream_t s);
+size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols);
+int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s);
+// MoE layer over Q5_0 / IQ4_XS / MXFP4 experts by bucket, on the matrix cores (32 tokens and more)
+bool moe_units_takes_grouped_path(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t batch);
+size_t moe_units_grouped_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);
+int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
+                                 const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
+                                 void *ws, hipStream_t s);
 int launch_gemm_sub_planar(const uint8_t *W, size_t row_stride, size_t off_d, size_t rows, size_t cols, const int8_t *aq,
                            const float *ad, size_t M, float *y, void *partial, hipStream_t s);
 // grouped (per-expert) GEMM: tile t = rows [64*t, 64*t+64) of the activations and of y, described by

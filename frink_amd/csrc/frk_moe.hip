@@ -739,4 +739,132 @@ int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const f
     return FRK_OK;
 }
 
+// The same layer from 32 tokens on, when every projection's kind has a decoded form the matrix cores read (Q5_0;
+// MXFP4 with scales that are f16 values; IQ4_XS): the reference's bucket path (crates/frink-models/src/decoder/
+// ffn_batch.rs:343-434) -- the pairs bucketed by expert, every expert's rows read once -- with the experts decoded
+// into signed bytes in the call's scratch memory and the grouped form of the Q8_0 matrix-core kernel.  The
+// activations are quantized per token (gate and up) and per grouped row (down) exactly as the per-pair jobs
+// quantize them, and the integers are the same: the two paths differ in the order of the float additions only.
+bool moe_units_takes_grouped_path(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t batch) {
+    auto planar = [](const frk_weights *w) {
+        return w->kind == FRK_KIND_Q5_0 || w->kind == FRK_KIND_IQ4_XS ||
+               (w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143);
+    };
+    return batch >= MOE_BUCKET_ORDER_FROM && planar(gate) && planar(up) && planar(down);
+}
+struct UnitsGroupedScratch {
+    uint8_t *gate_w, *up_w, *down_w;  // decoded experts
+    char *x_acts, *a_acts;            // quantized token rows; quantized intermediate rows (grouped order)
+    float *gate_out, *up_out, *down_out;
+    int *group_off, *gather, *pos_of, *cpos_of, *n_tiles;
+    int4 *tiles;
+};
+static size_t units_planar_bytes(size_t rows, size_t cols) {
+    return round_up(layout_for(FRK_KIND_Q8_0, cols).row_stride * rows + 256, 256);
+}
+// room for a batch of rows quantized either way: Q8_0 blocks in the GEMM's form, or Q8_K (quants, scales, sums)
+static size_t units_grouped_acts_bytes(size_t rows, size_t cols) {
+    const size_t q8k = round_up(rows * cols, 256) + round_up(rows * cols / QK_K * 4 + 4, 256) + round_up(rows * cols / 16 * 2 + 2, 256);
+    return std::max(q8_0_gemm_acts_bytes(rows, cols), q8k);
+}
+static UnitsGroupedScratch units_grouped_carve(void *base, size_t batch, int k, int n_experts, int hidden, int ffn, size_t *end) {
+    const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts);
+    char *p = (char *)base;
+    auto take = [&](size_t bytes) {
+        char *r = p;
+        p += round_up(bytes, 256);
+        return r;
+    };
+    UnitsGroupedScratch m;
+    m.gate_w = (uint8_t *)take(units_planar_bytes((size_t)n_experts * ffn, hidden));
+    m.up_w = (uint8_t *)take(units_planar_bytes((size_t)n_experts * ffn, hidden));
+    m.down_w = (uint8_t *)take(units_planar_bytes((size_t)n_experts * hidden, ffn));
+    m.x_acts = take(units_grouped_acts_bytes(batch, hidden));
+    m.a_acts = take(units_grouped_acts_bytes(rows, ffn));
+    m.gate_out = (float *)take(rows * ffn * 4);
+    m.up_out = (float *)take(rows * ffn * 4);
+    m.down_out = (float *)take(rows * hidden * 4);
+    m.group_off = (int *)take((n_experts + 1) * 4);
+    m.gather = (int *)take(rows * 4);
+    m.pos_of = (int *)take(pairs * 4);
+    m.cpos_of = (int *)take(pairs * 4);
+    m.n_tiles = (int *)take(256);
+    m.tiles = (int4 *)take((rows / MOE_TILE + 1) * 16);
+    if (end) *end = (size_t)(p - (char *)base);
+    return m;
+}
+size_t moe_units_grouped_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn) {
+    size_t end = 0;
+    (void)units_grouped_carve(nullptr, batch, k, n_experts, hidden, ffn, &end);
+    return end;
+}
+// rows x cols floats quantized into `room` for a projection of `kind`; the pointers the grouped GEMM takes
+struct UnitsGroupedActs {
+    const int8_t *q;
+    const void *d;
+};
+static int quantize_for_units_grouped(int kind, const float *x, size_t rows, size_t cols, char *room, UnitsGroupedActs *a, hipStream_t s) {
+    int8_t *q = (int8_t *)room;
+    a->q = q;
+    if (kind == FRK_KIND_IQ4_XS) {
+        float *d = (float *)(room + round_up(rows * cols, 256));
+        int16_t *bs = (int16_t *)(room + round_up(rows * cols, 256) + round_up(rows * cols / QK_K * 4 + 4, 256));
+        a->d = d;
+        return launch_quantize_q8_k(x, rows * cols, q, d, bs, s);
+    }
+    uint16_t *d = (uint16_t *)(room + round_up(rows * cols, 256));
+    a->d = d;
+    return launch_quantize_q8_0_gemm(x, rows, cols, q, d, s);
+}
+static int decode_units_planar(const frk_weights *w, uint8_t *dst, hipStream_t s) {
+    const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
+    return w->kind == FRK_KIND_IQ4_XS ? launch_iq4_xs_to_sub_planar(w, dst, planar.row_stride, planar.off_a, s)
+                                      : launch_units_to_q8_0_planar(w, dst, planar.row_stride, planar.off_a, s);
+}
+int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
+                                 const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
+                                 void *ws, hipStream_t s) {
+    const int hidden = (int)gate->cols, ffn = (int)down->cols;
+    const size_t pairs = batch * (size_t)k, rows = moe_max_rows(pairs, n_experts), max_tiles = rows / MOE_TILE;
+    const UnitsGroupedScratch m = units_grouped_carve(ws, batch, k, n_experts, hidden, ffn, nullptr);
+    static bool sized = false;  // a benign race: every thread sets the same attribute
+    if (!sized) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&moe_group_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GroupLds));
+        if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFuncSetAttribute(moe_group): %s", hipGetErrorString(e));
+        sized = true;
+    }
+    const GroupArgs ga{ids, (int)pairs, k, n_experts, m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles, (int)rows};
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ga);
+    FRK_LAUNCH_CHECK("moe_group");
+    int rc = decode_units_planar(gate, m.gate_w, s);
+    if (rc) return rc;
+    rc = decode_units_planar(up, m.up_w, s);
+    if (rc) return rc;
+    rc = decode_units_planar(down, m.down_w, s);
+    if (rc) return rc;
+    UnitsGroupedActs xa, aa;
+    rc = quantize_for_units_grouped(gate->kind, x, batch, (size_t)hidden, m.x_acts, &xa, s);
+    if (rc) return rc;
+    const Layout lg = layout_for(FRK_KIND_Q8_0, (size_t)hidden), ld = layout_for(FRK_KIND_Q8_0, (size_t)ffn);
+    rc = launch_gemm_planar_grouped(m.gate_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, gate->kind == FRK_KIND_IQ4_XS, xa.q,
+                                    xa.d, m.gather, m.tiles, m.n_tiles, max_tiles, m.gate_out, s);
+    if (rc) return rc;
+    rc = launch_gemm_planar_grouped(m.up_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, up->kind == FRK_KIND_IQ4_XS, xa.q,
+                                    xa.d, m.gather, m.tiles, m.n_tiles, max_tiles, m.up_out, s);
+    if (rc) return rc;
+    // (rows of the grouped order that no pair uses hold whatever the memory held: nothing reads their results)
+    rc = launch_swiglu(m.gate_out, m.up_out, rows * (size_t)ffn, m.gate_out, s);
+    if (rc) return rc;
+    rc = quantize_for_units_grouped(down->kind, m.gate_out, rows, (size_t)ffn, m.a_acts, &aa, s);
+    if (rc) return rc;
+    rc = launch_gemm_planar_grouped(m.down_w, ld.row_stride, ld.off_a, (size_t)hidden, (size_t)ffn, down->kind == FRK_KIND_IQ4_XS, aa.q,
+                                    aa.d, nullptr, m.tiles, m.n_tiles, max_tiles, m.down_out, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch, (unsigned)((hidden + 1023) / 1024)), dim3(256), 0, s, m.down_out, ids,
+                       weights, m.pos_of, k, hidden, n_experts, 1, out);
+    FRK_LAUNCH_CHECK("moe_combine");
+    return FRK_OK;
+}
+
 }  // namespace frk

@@ -1099,6 +1099,12 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
                          gate->rows, gate->cols, up->rows, up->cols, down->rows, down->cols, n_experts, hidden, ffn);
     if (batch * k > (size_t)1 << 30) return set_error(FRK_ERR_SHAPE, "batch*k = %zu pairs is too many", batch * k);
     WorkspaceLease lease;
+    if (unit_experts && moe_units_takes_grouped_path(gate, up, down, batch)) {
+        int rc = workspace(moe_units_grouped_workspace_bytes(batch, (int)k, (int)n_experts, (int)hidden, (int)ffn), (hipStream_t)stream, lease);
+        if (rc) return rc;
+        return launch_moe_ffn_units_grouped(gate, up, down, (int)n_experts, x, batch, ids, weights, (int)k, out, lease.ptr,
+                                            (hipStream_t)stream);
+    }
     if (unit_experts) {
         if (!gemv_units_int_fits(gate) || !gemv_units_int_fits(down))
             return set_error(FRK_ERR_UNSUPPORTED, "experts of kinds %d/%d with rows of %zu / %zu columns", gate->kind, down->kind,

@@ -267,9 +267,10 @@ int frk_hip_route_top_k_softmax_dev(const float *logits_dev, size_t batch, size_
  * ffn_batch.rs:355), routing order below (the per-position path's combine_expert_outputs,
  * crates/frink-moe/src/lib.rs:1246-1263).  gate/up/down hold the experts stacked row-wise
  * (expert e = rows [e*ffn, (e+1)*ffn) of gate and up, [e*hidden, (e+1)*hidden) of down); gate and up
- * are Q4_K, down is Q4_K or Q6_K; or all three of Q5_0 / IQ4_XS / MXFP4 (gate and up of one kind), where every
- * (token, slot) pair runs on the integer decode kernel of its kind -- any batch, correct, not tuned for hundreds of
- * tokens.  Other combinations: FRK_ERR_UNSUPPORTED.
+ * are Q4_K, down is Q4_K or Q6_K; or all three of Q5_0 / IQ4_XS / MXFP4 (gate and up of one kind): below 32 tokens
+ * every (token, slot) pair runs on the integer decode kernel of its kind, from 32 on the pairs are bucketed by
+ * expert and the experts, decoded to signed bytes in scratch memory, run on the grouped matrix-core kernel (an MXFP4
+ * stack with scale bytes outside 104..143 keeps the per-pair jobs).  Other combinations: FRK_ERR_UNSUPPORTED.
  * ids[batch][k] / weights[batch][k] are a RoutingDecision per token (lib.rs:112-115); an id outside
  * [0, n_experts) contributes nothing. */
 int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const frk_weights *down,

@@ -1037,11 +1037,16 @@ def test_moe_ffn_with_q6_k_down_experts(fa, n_experts, k, hidden, ffn, batch):
 @pytest.mark.parametrize("gate_kind,down_kind,n_experts,k,hidden,ffn,batch", [
     (fo.MXFP4, fo.MXFP4, 8, 2, 512, 256, 1), (fo.MXFP4, fo.MXFP4, 16, 4, 512, 768, 40), (fo.Q5_0, fo.Q5_0, 8, 2, 256, 512, 9),
     (fo.IQ4_XS, fo.IQ4_XS, 8, 3, 512, 256, 33), (fo.MXFP4, fo.Q5_0, 6, 2, 256, 256, 5),
+    (fo.Q5_0, fo.Q5_0, 8, 2, 256, 512, 70), (fo.MXFP4, fo.Q5_0, 6, 2, 320, 96, 45), (fo.IQ4_XS, fo.Q5_0, 4, 2, 512, 160, 64),
+    (fo.MXFP4, fo.IQ4_XS, 32, 4, 576, 512, 300), (fo.MXFP4, fo.MXFP4, 5, 2, 64, 64, 200),
 ])
 def test_moe_ffn_with_experts_of_the_other_kinds(fa, gate_kind, down_kind, n_experts, k, hidden, ffn, batch):
     """Experts in MXFP4 / Q5_0 / IQ4_XS (run_expert takes any WeightMatrix, crates/frink-moe/src/lib.rs:1068-1165):
     every (token, slot) pair on the integer tier of its kind, the slots added in the reference's order for the batch
-    size (routing order below 32 tokens, ascending expert id from 32 on), an id outside the experts left out."""
+    size (routing order below 32 tokens, ascending expert id from 32 on), an id outside the experts left out.  Below 32
+    tokens a decode job per pair; from 32 on the pairs bucketed by expert and the experts, decoded to signed bytes, on
+    the grouped matrix-core kernel (tiles of every fill, several tiles an expert, experts nobody chose, rows that are
+    not a multiple of the kernel's 256-column step)."""
     from frink_amd import synth
     print("moe, other kinds", gate_kind, down_kind, n_experts, k, hidden, ffn, batch, flush=True)
     gate = _other_kind_blocks(gate_kind, n_experts * ffn, hidden, seed=41)
@@ -1051,6 +1056,9 @@ def test_moe_ffn_with_experts_of_the_other_kinds(fa, gate_kind, down_kind, n_exp
         if kind == fo.MXFP4:  # weight-sized scales, 2^-17 .. 2^-6: the intermediate's Q8_0 scales are f16 values
             blk = data.reshape(-1, 17)
             blk[:, 0] = 110 + blk[:, 0] % 12
+        if kind == fo.IQ4_XS and down_kind != fo.IQ4_XS:  # (the same: d * (ls - 32) * code reaches 200 at d = 0.05)
+            blk = data.reshape(-1, 136)
+            blk[:, 0:2] = np.random.default_rng(46).uniform(-5e-4, 5e-4, blk.shape[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
     x = synth.activations(44, batch, hidden)
     ids, w = _route(synth.normal(45, batch * n_experts).reshape(batch, n_experts), k)
     ids = ids.astype(np.int32)
