@@ -242,6 +242,11 @@ int launch_gemm_planar_grouped(const uint8_t *W, size_t row_stride, size_t off_d
                                size_t max_tiles, float *y, hipStream_t s);
 size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols);
 int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s);
+// the grouped GEMM over groups of Q5_0 / IQ4_XS / MXFP4 matrices that have a decoded form for the matrix cores
+bool units_have_planar_form(const frk_weights *w);
+size_t grouped_units_workspace_bytes(size_t n_groups, size_t w_rows, size_t x_rows, size_t pairs, size_t cols);
+int launch_gemm_grouped_units(const frk_weights *w, size_t n_groups, const int32_t *group_off, const int32_t *gather, const float *x,
+                              size_t x_rows, size_t pairs, float *y, void *ws, hipStream_t s);
 // MoE layer over Q5_0 / IQ4_XS / MXFP4 experts by bucket, on the matrix cores (32 tokens and more)
 bool moe_units_takes_grouped_path(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t batch);
 size_t moe_units_grouped_workspace_bytes(size_t batch, int k, int n_experts, int hidden, int ffn);

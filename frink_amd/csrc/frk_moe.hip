@@ -745,12 +745,9 @@ int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const f
 // into signed bytes in the call's scratch memory and the grouped form of the Q8_0 matrix-core kernel.  The
 // activations are quantized per token (gate and up) and per grouped row (down) exactly as the per-pair jobs
 // quantize them, and the integers are the same: the two paths differ in the order of the float additions only.
+bool units_have_planar_form(const frk_weights *w);
 bool moe_units_takes_grouped_path(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t batch) {
-    auto planar = [](const frk_weights *w) {
-        return w->kind == FRK_KIND_Q5_0 || w->kind == FRK_KIND_IQ4_XS ||
-               (w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143);
-    };
-    return batch >= MOE_BUCKET_ORDER_FROM && planar(gate) && planar(up) && planar(down);
+    return batch >= MOE_BUCKET_ORDER_FROM && units_have_planar_form(gate) && units_have_planar_form(up) && units_have_planar_form(down);
 }
 struct UnitsGroupedScratch {
     uint8_t *gate_w, *up_w, *down_w;  // decoded experts
@@ -821,6 +818,58 @@ static int decode_units_planar(const frk_weights *w, uint8_t *dst, hipStream_t s
     return w->kind == FRK_KIND_IQ4_XS ? launch_iq4_xs_to_sub_planar(w, dst, planar.row_stride, planar.off_a, s)
                                       : launch_units_to_q8_0_planar(w, dst, planar.row_stride, planar.off_a, s);
 }
+// The grouped GEMM as an entry of its own over groups of these kinds: the tile list, the stack decoded, the
+// activation rows quantized once (Q8_0 blocks, or Q8_K for IQ4_XS), the grouped kernel gathering through the list.
+bool units_have_planar_form(const frk_weights *w) {
+    return w->kind == FRK_KIND_Q5_0 || w->kind == FRK_KIND_IQ4_XS ||
+           (w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143);
+}
+struct GroupedUnitsScratch {
+    uint8_t *decoded;
+    char *acts;
+    int *src_rows, *n_tiles;
+    int4 *tiles;
+};
+static GroupedUnitsScratch grouped_units_carve(void *base, size_t n_groups, size_t w_rows, size_t x_rows, size_t pairs, size_t cols,
+                                               size_t *end) {
+    const size_t rows = moe_max_rows(pairs, (int)n_groups);
+    char *p = (char *)base;
+    auto take = [&](size_t bytes) {
+        char *r = p;
+        p += round_up(bytes, 256);
+        return r;
+    };
+    GroupedUnitsScratch m;
+    m.decoded = (uint8_t *)take(units_planar_bytes(w_rows, cols));
+    m.acts = take(units_grouped_acts_bytes(x_rows, cols));
+    m.src_rows = (int *)take(rows * 4);
+    m.n_tiles = (int *)take(256);
+    m.tiles = (int4 *)take((rows / MOE_TILE + 1) * 16);
+    if (end) *end = (size_t)(p - (char *)base);
+    return m;
+}
+size_t grouped_units_workspace_bytes(size_t n_groups, size_t w_rows, size_t x_rows, size_t pairs, size_t cols) {
+    size_t end = 0;
+    (void)grouped_units_carve(nullptr, n_groups, w_rows, x_rows, pairs, cols, &end);
+    return end;
+}
+int launch_gemm_grouped_units(const frk_weights *w, size_t n_groups, const int32_t *group_off, const int32_t *gather, const float *x,
+                              size_t x_rows, size_t pairs, float *y, void *ws, hipStream_t s) {
+    const size_t rows_g = w->rows / n_groups, cols = w->cols, rows = moe_max_rows(pairs, (int)n_groups);
+    const GroupedUnitsScratch m = grouped_units_carve(ws, n_groups, w->rows, x_rows, pairs, cols, nullptr);
+    const GroupedTilesArgs ta{group_off, gather, (int)n_groups, (int)pairs, (int)x_rows, (int)rows, m.src_rows, m.tiles, m.n_tiles};
+    hipLaunchKernelGGL(grouped_tiles_kernel, dim3(1), dim3(1024), 0, s, ta);
+    FRK_LAUNCH_CHECK("grouped_tiles");
+    int rc = decode_units_planar(w, m.decoded, s);
+    if (rc) return rc;
+    UnitsGroupedActs xa;
+    rc = quantize_for_units_grouped(w->kind, x, x_rows, cols, m.acts, &xa, s);
+    if (rc) return rc;
+    const Layout l = layout_for(FRK_KIND_Q8_0, cols);
+    return launch_gemm_planar_grouped(m.decoded, l.row_stride, l.off_a, rows_g, cols, w->kind == FRK_KIND_IQ4_XS, xa.q, xa.d, m.src_rows,
+                                      m.tiles, m.n_tiles, rows / MOE_TILE, y, s);
+}
+
 int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts,
                                  const float *x, size_t batch, const int32_t *ids, const float *weights, int k, float *out,
                                  void *ws, hipStream_t s) {

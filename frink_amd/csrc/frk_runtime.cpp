@@ -1123,8 +1123,11 @@ int frk_hip_gemm_grouped_dev(const frk_weights *stacked, size_t n_groups, const 
     clear_error();
     if (!stacked || !group_off || (pairs && (!x || !y))) return set_error(FRK_ERR_ARG, "frk_hip_gemm_grouped_dev: null argument");
     if (n_groups == 0 || n_groups > 1024) return set_error(FRK_ERR_SHAPE, "groups=%zu (1 .. 1024)", n_groups);
-    if (stacked->kind != FRK_KIND_Q4_K && stacked->kind != FRK_KIND_Q6_K)
-        return set_error(FRK_ERR_UNSUPPORTED, "the grouped GEMM takes Q4_K or Q6_K weights (got kind %d)", stacked->kind);
+    const bool units = is_unit_kind(stacked->kind) && units_have_planar_form(stacked);
+    if (stacked->kind != FRK_KIND_Q4_K && stacked->kind != FRK_KIND_Q6_K && !units)
+        return set_error(FRK_ERR_UNSUPPORTED,
+                         "the grouped GEMM takes Q4_K, Q6_K, Q5_0, IQ4_XS or MXFP4 (scale bytes within 104..143) weights (got kind %d)",
+                         stacked->kind);
     if (stacked->rows % n_groups)
         return set_error(FRK_ERR_SHAPE, "stacked rows %zu do not divide into %zu groups", stacked->rows, n_groups);
     if (pairs > (size_t)1 << 30 || x_rows > (size_t)1 << 30)
@@ -1132,6 +1135,11 @@ int frk_hip_gemm_grouped_dev(const frk_weights *stacked, size_t n_groups, const 
     if (pairs == 0) return FRK_OK;
     if (x_rows == 0) return set_error(FRK_ERR_SHAPE, "%zu pairs over no activation rows", pairs);
     WorkspaceLease lease;
+    if (units) {
+        int rc = workspace(grouped_units_workspace_bytes(n_groups, stacked->rows, x_rows, pairs, stacked->cols), (hipStream_t)stream, lease);
+        if (rc) return rc;
+        return launch_gemm_grouped_units(stacked, n_groups, group_off, gather, x, x_rows, pairs, y, lease.ptr, (hipStream_t)stream);
+    }
     int rc = workspace(grouped_gemm_workspace_bytes(n_groups, x_rows, pairs, stacked->cols), (hipStream_t)stream, lease);
     if (rc) return rc;
     return launch_gemm_grouped(stacked, n_groups, group_off, gather, x, x_rows, pairs, y, lease.ptr, (hipStream_t)stream);

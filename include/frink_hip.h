@@ -280,12 +280,13 @@ int frk_hip_moe_ffn_dev(const frk_weights *gate, const frk_weights *up, const fr
 /* The grouped (indexed) GEMM on its own, for a caller with its own routing and activation:
  * enqueue_mul_mm_grouped_dev (crates/frink-cuda/src/mul_mm_launch.rs:391-470) and enqueue_mmq_grouped
  * (crates/frink-cuda/src/mmq/mod.rs:144-217).  Group g's matrix is rows [g*R, (g+1)*R) of `stacked` (R = rows /
- * n_groups; the reference's table[g], here one resident stack), Q4_K or Q6_K (others: FRK_ERR_UNSUPPORTED);
+ * n_groups; the reference's table[g], here one resident stack), Q4_K or Q6_K, or Q5_0 / IQ4_XS / MXFP4 with scale
+ * bytes within 104..143 (decoded to signed bytes per call); others: FRK_ERR_UNSUPPORTED;
  * group_off_dev[n_groups + 1] are non-decreasing pair indices from 0 to pairs; pair p of group g reads activation
  * row gather_dev[p] of x_dev[x_rows][cols] (row p when gather_dev is null) and writes y_dev[p][R] -- every pair of
  * every group, no gaps.  Everything is read on the device, so the call can follow the kernel that built the
- * lists without a host round trip; the activation rows are quantized to Q8_K once each, as the reference's
- * integer tier does.  n_groups <= 1024.  Offsets out of order or gather entries outside x are clamped, not
+ * lists without a host round trip; the activation rows are quantized once each, to Q8_K or (Q5_0, MXFP4) to
+ * Q8_0 blocks, as the reference's integer tier does.  n_groups <= 1024.  Offsets out of order or gather entries outside x are clamped, not
  * trusted. */
 int frk_hip_gemm_grouped_dev(const frk_weights *stacked, size_t n_groups, const int32_t *group_off_dev,
                              const int32_t *gather_dev, const float *x_dev, size_t x_rows, size_t pairs, float *y_dev,

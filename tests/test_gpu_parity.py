@@ -799,6 +799,43 @@ def test_grouped_gemm_over_more_rows_than_the_gathering_kernel_addresses(fa):
     w.release()
 
 
+@pytest.mark.parametrize("kind,cols", [(fo.Q5_0, 96), (fo.MXFP4, 2880), (fo.IQ4_XS, 768), (fo.MXFP4, 256)])
+@pytest.mark.parametrize("with_gather", [True, False])
+def test_grouped_gemm_over_the_other_kinds(fa, kind, cols, with_gather):
+    """The grouped entry over stacks of Q5_0 / MXFP4 / IQ4_XS matrices: the stack decoded to signed bytes per call, the
+    activation rows quantized once (Q8_0 blocks; Q8_K for IQ4_XS), the grouped matrix-core kernel gathering through the
+    list -- every pair against the integer tier of its kind (q8_row_dot / q8k_row_dot,
+    crates/frink-core/src/weight_matrix.rs:392-420)."""
+    from frink_amd import synth
+    counts = [0, 1, 31, 0, 32, 33, 64, 65, 150, 7, 0]
+    n_groups, rows_g = len(counts), 72
+    print("grouped gemm, other kinds", kind, cols, with_gather, flush=True)
+    off = np.zeros(n_groups + 1, np.int32)
+    off[1:] = np.cumsum(counts)
+    pairs = int(off[-1])
+    x_rows = 90 if with_gather else pairs
+    data = _other_kind_blocks(kind, n_groups * rows_g, cols, seed=kind + cols)
+    if kind == fo.MXFP4:
+        data.reshape(-1, 17)[:, 0] = 104 + data.reshape(-1, 17)[:, 0] % 40  # scales that are f16 values
+    x = synth.activations(5, x_rows, cols, outlier_frac=0.01)
+    gather = np.random.default_rng(6).integers(0, x_rows, pairs).astype(np.int32) if with_gather else None
+    w = fa.Weights.from_host(kind, data, n_groups * rows_g, cols)
+    import torch
+    y = torch.full((pairs, rows_g), float("nan"), dtype=torch.float32, device="cuda")
+    got = fa.gemm_grouped(w, n_groups, to_dev(off), to_dev(x), to_dev(gather) if with_gather else None, out=y).cpu().numpy()
+    per = data.reshape(n_groups, -1)
+    want = np.zeros((pairs, rows_g), np.float32)
+    for g in range(n_groups):
+        p0, p1 = int(off[g]), int(off[g + 1])
+        if p1 > p0:
+            src = gather[p0:p1] if with_gather else np.arange(p0, p1)
+            want[p0:p1] = fo.gemm(kind, per[g], rows_g, cols, x[src], fo.INT_DOT)
+    assert not np.isnan(got).any()  # every pair's row written
+    assert_rows_close(got, want, "grouped gemm kind %d gather %s" % (kind, with_gather))
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max()
+    w.release()
+
+
 def test_grouped_gemm_refuses_what_it_cannot_run(fa):
     data = make_weights(fo.Q8_0, 64, 256, seed=1)
     w = fa.Weights.from_host(fo.Q8_0, data, 64, 256)
