@@ -548,6 +548,12 @@ def main():
                 extra["%s GEMM M=512 4096x14336 (decoded to int8 planes per call)" % name_o] = {
                     "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
                 for w in wo:
+                    w.keep_decoded()
+                _, t = timed(step3f, 40, 20)
+                tops = 2.0 * 512 * rows * cols / (t / 40) / 1e12
+                extra["%s GEMM M=512 4096x14336 (decoded copy kept)" % name_o] = {
+                    "TOPS": round(tops, 1), "us_per_step": round(t / 40 * 1e6, 2), "frac_of_int8_mfma_peak": round(tops / INT8_PEAK_TOPS, 4)}
+                for w in wo:
                     w.release()
                 del do
         if want('moe'):
@@ -619,6 +625,12 @@ def main():
                 fa.moe_ffn(ex4[0], ex4[1], ex4[2], E4, xm4, ids4, wts4, out=ym4)
             _, t = timed(step4e, 20, 10)
             extra["MoE layer 32x top-4, 2880/2880, 512 tokens, MXFP4 experts"] = {
+                "us_per_step": round(t / 20 * 1e6, 2), "tokens_per_s": round(T / (t / 20), 0),
+                "TOPS": round(2.0 * T * K4 * 3 * F4 * H4 / (t / 20) / 1e12, 1)}
+            for w in ex4:
+                w.keep_decoded()
+            _, t = timed(step4e, 20, 10)
+            extra["MoE layer 32x top-4, 2880/2880, 512 tokens, MXFP4 experts (decoded copies kept)"] = {
                 "us_per_step": round(t / 20 * 1e6, 2), "tokens_per_s": round(T / (t / 20), 0),
                 "TOPS": round(2.0 * T * K4 * 3 * F4 * H4 / (t / 20) / 1e12, 1)}
             for w in ex4:

@@ -77,6 +77,7 @@ extern "C" {
     fn frk_hip_weights_from_device(kind: c_int, dev_bytes: *const c_void, len: usize, rows: usize, cols: usize,
                                    stream: *mut c_void, out: *mut *mut FrkWeights) -> c_int;
     fn frk_hip_weights_release(w: *mut FrkWeights) -> c_int;
+    fn frk_hip_weights_keep_decoded(w: *mut FrkWeights, stream: *mut c_void) -> c_int;
     fn frk_hip_weights_rows(w: *const FrkWeights) -> usize;
     fn frk_hip_weights_cols(w: *const FrkWeights) -> usize;
     fn frk_hip_weights_kind(w: *const FrkWeights) -> c_int;
@@ -267,6 +268,11 @@ impl Weights {
     pub fn cols(&self) -> usize { unsafe { frk_hip_weights_cols(self.0) } }
     pub fn kind(&self) -> c_int { unsafe { frk_hip_weights_kind(self.0) } }
     pub fn raw(&self) -> *const FrkWeights { self.0 }
+    /// Q5_0 / IQ4_XS / MXFP4: keep the rows decoded for the matrix cores beside the resident copy (decodes on
+    /// `stream` and synchronizes it); batched calls then skip their per-call decoding.
+    pub fn keep_decoded(&mut self, stream: *mut c_void) -> Result<(), HipError> {
+        check(unsafe { frk_hip_weights_keep_decoded(self.0, stream) })
+    }
 
     /// `WeightMatrix::dequant_row` / get_rows (crates/frink-cuda/src/get_rows.rs): host ids, host rows.
     pub fn get_rows(&self, ids: &[i32]) -> Result<Vec<f32>, HipError> {

@@ -27,7 +27,7 @@ EXPORTS = [
     "frk_hip_probe", "frk_hip_dense_enabled", "frk_hip_last_error", "frk_hip_matvec_kernel",
     "frk_hip_gemm_supported", "frk_hip_has_launch", "frk_hip_block_bytes", "frk_hip_block_elems",
     "frk_hip_worth_a_gemm", "frk_hip_weights_register", "frk_hip_weights_from_device",
-    "frk_hip_weights_release", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
+    "frk_hip_weights_release", "frk_hip_weights_keep_decoded", "frk_hip_weights_rows", "frk_hip_weights_cols", "frk_hip_weights_kind",
     "frk_hip_launch_matvec", "frk_hip_launch_mul_mm", "frk_hip_launch_matvec_multi",
     "frk_hip_launch_dense_ffn_swiglu", "frk_hip_gemv_multi_dev", "frk_hip_ffn_swiglu_dev", "frk_hip_gemv_dev", "frk_hip_gemv_q8k_dev",
     "frk_hip_gemm_dev", "frk_hip_gemm_q8k_dev", "frk_hip_gemm_pair_dev", "frk_hip_gemm_noalloc_dev",
@@ -78,6 +78,7 @@ def lib():
             "frk_hip_weights_register": (i, [i, vp, sz, sz, sz, C.POINTER(vp)]),
             "frk_hip_weights_from_device": (i, [i, vp, sz, sz, sz, vp, C.POINTER(vp)]),
             "frk_hip_weights_release": (i, [vp]),
+            "frk_hip_weights_keep_decoded": (i, [vp, vp]),
             "frk_hip_weights_rows": (sz, [vp]),
             "frk_hip_weights_cols": (sz, [vp]),
             "frk_hip_weights_kind": (i, [vp]),
@@ -174,6 +175,11 @@ class Weights:
         check(lib().frk_hip_weights_from_device(kind, C.c_void_p(data_dev.data_ptr()), data_dev.numel(), rows, cols,
                                                 _stream(), C.byref(h)))
         return cls(h, kind, rows, cols)
+
+    def keep_decoded(self):
+        """Q5_0 / IQ4_XS / MXFP4: keep the rows decoded for the matrix cores beside the resident copy."""
+        check(lib().frk_hip_weights_keep_decoded(self.handle, _stream()))
+        return self
 
     def release(self):
         if self.handle:

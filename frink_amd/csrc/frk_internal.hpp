@@ -108,6 +108,9 @@ struct frk_weights {
     bool cached = false;
     // MXFP4: the range of the E8M0 scale bytes (the batched integer path needs them to be f16 values)
     int e8m0_min = 0, e8m0_max = 255;
+    // Q5_0 / IQ4_XS / MXFP4: the rows decoded to signed bytes for the matrix cores, kept beside the resident copy
+    // on request (frk_hip_weights_keep_decoded); without it every batched call decodes into its scratch memory
+    uint8_t *decoded = nullptr;
 };
 
 namespace frk {
@@ -244,6 +247,11 @@ size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols);
 int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s);
 // the grouped GEMM over groups of Q5_0 / IQ4_XS / MXFP4 matrices that have a decoded form for the matrix cores
 bool units_have_planar_form(const frk_weights *w);
+// that form: rows of layout_for(FRK_KIND_Q8_0, cols) -- signed bytes, then f16 scales per 32 (IQ4_XS: per block of
+// 256 the eight integer block scales and the f16 d).  units_decoded: the kept copy, or the rows decoded into `room`.
+size_t units_planar_bytes(size_t rows, size_t cols);
+int launch_units_decode(const frk_weights *w, uint8_t *dst, hipStream_t s);
+int units_decoded(const frk_weights *w, uint8_t *room, hipStream_t s, const uint8_t **out);
 size_t grouped_units_workspace_bytes(size_t n_groups, size_t w_rows, size_t x_rows, size_t pairs, size_t cols);
 int launch_gemm_grouped_units(const frk_weights *w, size_t n_groups, const int32_t *group_off, const int32_t *gather, const float *x,
                               size_t x_rows, size_t pairs, float *y, void *ws, hipStream_t s);

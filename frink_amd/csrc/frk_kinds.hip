@@ -535,4 +535,23 @@ int mxfp4_scale_range(const frk_weights *w, int *e_min, int *e_max, hipStream_t 
     return FRK_OK;
 }
 
+bool units_have_planar_form(const frk_weights *w) {
+    return w->kind == FRK_KIND_Q5_0 || w->kind == FRK_KIND_IQ4_XS ||
+           (w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143);
+}
+size_t units_planar_bytes(size_t rows, size_t cols) { return round_up(layout_for(FRK_KIND_Q8_0, cols).row_stride * rows + 256, 256); }
+int launch_units_decode(const frk_weights *w, uint8_t *dst, hipStream_t s) {
+    const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
+    return w->kind == FRK_KIND_IQ4_XS ? launch_iq4_xs_to_sub_planar(w, dst, planar.row_stride, planar.off_a, s)
+                                      : launch_units_to_q8_0_planar(w, dst, planar.row_stride, planar.off_a, s);
+}
+int units_decoded(const frk_weights *w, uint8_t *room, hipStream_t s, const uint8_t **out) {
+    if (w->decoded) {
+        *out = w->decoded;
+        return FRK_OK;
+    }
+    *out = room;
+    return launch_units_decode(w, room, s);
+}
+
 }  // namespace frk

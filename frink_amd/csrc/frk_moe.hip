@@ -745,7 +745,6 @@ int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const f
 // into signed bytes in the call's scratch memory and the grouped form of the Q8_0 matrix-core kernel.  The
 // activations are quantized per token (gate and up) and per grouped row (down) exactly as the per-pair jobs
 // quantize them, and the integers are the same: the two paths differ in the order of the float additions only.
-bool units_have_planar_form(const frk_weights *w);
 bool moe_units_takes_grouped_path(const frk_weights *gate, const frk_weights *up, const frk_weights *down, size_t batch) {
     return batch >= MOE_BUCKET_ORDER_FROM && units_have_planar_form(gate) && units_have_planar_form(up) && units_have_planar_form(down);
 }
@@ -756,9 +755,6 @@ struct UnitsGroupedScratch {
     int *group_off, *gather, *pos_of, *cpos_of, *n_tiles;
     int4 *tiles;
 };
-static size_t units_planar_bytes(size_t rows, size_t cols) {
-    return round_up(layout_for(FRK_KIND_Q8_0, cols).row_stride * rows + 256, 256);
-}
 // room for a batch of rows quantized either way: Q8_0 blocks in the GEMM's form, or Q8_K (quants, scales, sums)
 static size_t units_grouped_acts_bytes(size_t rows, size_t cols) {
     const size_t q8k = round_up(rows * cols, 256) + round_up(rows * cols / QK_K * 4 + 4, 256) + round_up(rows * cols / 16 * 2 + 2, 256);
@@ -813,17 +809,8 @@ static int quantize_for_units_grouped(int kind, const float *x, size_t rows, siz
     a->d = d;
     return launch_quantize_q8_0_gemm(x, rows, cols, q, d, s);
 }
-static int decode_units_planar(const frk_weights *w, uint8_t *dst, hipStream_t s) {
-    const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
-    return w->kind == FRK_KIND_IQ4_XS ? launch_iq4_xs_to_sub_planar(w, dst, planar.row_stride, planar.off_a, s)
-                                      : launch_units_to_q8_0_planar(w, dst, planar.row_stride, planar.off_a, s);
-}
 // The grouped GEMM as an entry of its own over groups of these kinds: the tile list, the stack decoded, the
 // activation rows quantized once (Q8_0 blocks, or Q8_K for IQ4_XS), the grouped kernel gathering through the list.
-bool units_have_planar_form(const frk_weights *w) {
-    return w->kind == FRK_KIND_Q5_0 || w->kind == FRK_KIND_IQ4_XS ||
-           (w->kind == FRK_KIND_MXFP4 && w->e8m0_min >= 104 && w->e8m0_max <= 143);
-}
 struct GroupedUnitsScratch {
     uint8_t *decoded;
     char *acts;
@@ -860,13 +847,14 @@ int launch_gemm_grouped_units(const frk_weights *w, size_t n_groups, const int32
     const GroupedTilesArgs ta{group_off, gather, (int)n_groups, (int)pairs, (int)x_rows, (int)rows, m.src_rows, m.tiles, m.n_tiles};
     hipLaunchKernelGGL(grouped_tiles_kernel, dim3(1), dim3(1024), 0, s, ta);
     FRK_LAUNCH_CHECK("grouped_tiles");
-    int rc = decode_units_planar(w, m.decoded, s);
+    const uint8_t *decoded = nullptr;
+    int rc = units_decoded(w, m.decoded, s, &decoded);
     if (rc) return rc;
     UnitsGroupedActs xa;
     rc = quantize_for_units_grouped(w->kind, x, x_rows, cols, m.acts, &xa, s);
     if (rc) return rc;
     const Layout l = layout_for(FRK_KIND_Q8_0, cols);
-    return launch_gemm_planar_grouped(m.decoded, l.row_stride, l.off_a, rows_g, cols, w->kind == FRK_KIND_IQ4_XS, xa.q, xa.d, m.src_rows,
+    return launch_gemm_planar_grouped(decoded, l.row_stride, l.off_a, rows_g, cols, w->kind == FRK_KIND_IQ4_XS, xa.q, xa.d, m.src_rows,
                                       m.tiles, m.n_tiles, rows / MOE_TILE, y, s);
 }
 
@@ -886,20 +874,21 @@ int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up,
     const GroupArgs ga{ids, (int)pairs, k, n_experts, m.group_off, m.gather, m.pos_of, m.cpos_of, m.tiles, m.n_tiles, (int)rows};
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), sizeof(GroupLds), s, ga);
     FRK_LAUNCH_CHECK("moe_group");
-    int rc = decode_units_planar(gate, m.gate_w, s);
+    const uint8_t *gate_w = nullptr, *up_w = nullptr, *down_w = nullptr;
+    int rc = units_decoded(gate, m.gate_w, s, &gate_w);
     if (rc) return rc;
-    rc = decode_units_planar(up, m.up_w, s);
+    rc = units_decoded(up, m.up_w, s, &up_w);
     if (rc) return rc;
-    rc = decode_units_planar(down, m.down_w, s);
+    rc = units_decoded(down, m.down_w, s, &down_w);
     if (rc) return rc;
     UnitsGroupedActs xa, aa;
     rc = quantize_for_units_grouped(gate->kind, x, batch, (size_t)hidden, m.x_acts, &xa, s);
     if (rc) return rc;
     const Layout lg = layout_for(FRK_KIND_Q8_0, (size_t)hidden), ld = layout_for(FRK_KIND_Q8_0, (size_t)ffn);
-    rc = launch_gemm_planar_grouped(m.gate_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, gate->kind == FRK_KIND_IQ4_XS, xa.q,
+    rc = launch_gemm_planar_grouped(gate_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, gate->kind == FRK_KIND_IQ4_XS, xa.q,
                                     xa.d, m.gather, m.tiles, m.n_tiles, max_tiles, m.gate_out, s);
     if (rc) return rc;
-    rc = launch_gemm_planar_grouped(m.up_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, up->kind == FRK_KIND_IQ4_XS, xa.q,
+    rc = launch_gemm_planar_grouped(up_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, up->kind == FRK_KIND_IQ4_XS, xa.q,
                                     xa.d, m.gather, m.tiles, m.n_tiles, max_tiles, m.up_out, s);
     if (rc) return rc;
     // (rows of the grouped order that no pair uses hold whatever the memory held: nothing reads their results)
@@ -907,7 +896,7 @@ int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up,
     if (rc) return rc;
     rc = quantize_for_units_grouped(down->kind, m.gate_out, rows, (size_t)ffn, m.a_acts, &aa, s);
     if (rc) return rc;
-    rc = launch_gemm_planar_grouped(m.down_w, ld.row_stride, ld.off_a, (size_t)hidden, (size_t)ffn, down->kind == FRK_KIND_IQ4_XS, aa.q,
+    rc = launch_gemm_planar_grouped(down_w, ld.row_stride, ld.off_a, (size_t)hidden, (size_t)ffn, down->kind == FRK_KIND_IQ4_XS, aa.q,
                                     aa.d, nullptr, m.tiles, m.n_tiles, max_tiles, m.down_out, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch, (unsigned)((hidden + 1023) / 1024)), dim3(256), 0, s, m.down_out, ids,

@@ -367,8 +367,32 @@ int frk_hip_weights_release(frk_weights *w) {
     }
     if (w->cached) g_dev.cache.erase(std::make_pair(w->host_key, w->host_len));
     hipError_t e = hipFree(w->dev);
+    if (w->decoded) {
+        const hipError_t e2 = hipFree(w->decoded);
+        if (e == hipSuccess) e = e2;
+    }
     delete w;
     if (e != hipSuccess) return set_error(FRK_ERR_HIP, "hipFree: %s", hipGetErrorString(e));
+    return FRK_OK;
+}
+
+int frk_hip_weights_keep_decoded(frk_weights *w, void *stream) {
+    clear_error();
+    if (!w) return set_error(FRK_ERR_ARG, "frk_hip_weights_keep_decoded: null argument");
+    if (!is_unit_kind(w->kind) || !units_have_planar_form(w))
+        return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has no decoded form to keep (Q5_0, IQ4_XS, MXFP4 with scale bytes within 104..143)",
+                         w->kind);
+    std::lock_guard<std::mutex> lk(g_dev.mu);
+    if (w->decoded) return FRK_OK;
+    uint8_t *room = nullptr;
+    FRK_HIP_TRY(hipMalloc((void **)&room, units_planar_bytes(w->rows, w->cols)));
+    int rc = launch_units_decode(w, room, (hipStream_t)stream);
+    hipError_t e = rc ? hipSuccess : hipStreamSynchronize((hipStream_t)stream);
+    if (rc || e != hipSuccess) {
+        (void)hipFree(room);
+        return rc ? rc : set_error(FRK_ERR_HIP, "frk_hip_weights_keep_decoded: %s", hipGetErrorString(e));
+    }
+    w->decoded = room;  // (published behind the synchronization: any stream may read it from here on)
     return FRK_OK;
 }
 
@@ -645,8 +669,8 @@ static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, fl
         void *ws = nullptr;
         int rc = scratch.get(planar_bytes + gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), s, &ws);
         if (rc) return rc;
-        uint8_t *decoded = (uint8_t *)ws;
-        rc = launch_units_to_q8_0_planar(w, decoded, planar.row_stride, planar.off_a, s);
+        const uint8_t *decoded = nullptr;
+        rc = units_decoded(w, (uint8_t *)ws, s, &decoded);
         if (rc) return rc;
         return launch_gemm_q8_0_planar(decoded, planar.row_stride, planar.off_a, w->rows, w->cols, false, x, batch, y,
                                        (char *)ws + planar_bytes, s);
@@ -662,11 +686,11 @@ static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, fl
         void *ws = nullptr;
         int rc = scratch.get(planar_bytes + q_bytes + d_bytes + b_bytes + gemm_sub_partial_bytes(batch, w->cols, w->rows), s, &ws);
         if (rc) return rc;
-        uint8_t *decoded = (uint8_t *)ws;
+        const uint8_t *decoded = nullptr;
         int8_t *q = (int8_t *)((char *)ws + planar_bytes);
         float *d = (float *)((char *)q + q_bytes);
         int16_t *bs = (int16_t *)((char *)d + d_bytes);
-        rc = launch_iq4_xs_to_sub_planar(w, decoded, planar.row_stride, planar.off_a, s);
+        rc = units_decoded(w, (uint8_t *)ws, s, &decoded);
         if (rc) return rc;
         rc = launch_quantize_q8_k(x, n, q, d, bs, s);
         if (rc) return rc;

@@ -201,6 +201,14 @@ class WeightMatrix {
         return true;
     }
 
+    // Q5_0 / IQ4_XS / MXFP4: the rows decoded for the matrix cores kept beside the resident copy (no counterpart in
+    // the reference, whose GEMM dequantizes inside the kernel: crates/frink-cuda/src/mul_mm.rs:146-205)
+    Result<bool> keep_decoded(void *stream) {
+        int rc = frk_hip_weights_keep_decoded(h_, stream);
+        if (rc != FRK_OK) return last_error(rc);
+        return true;
+    }
+
   private:
     WeightMatrix(frk_weights *h, QuantKind k, size_t r, size_t c) : h_(h), kind_(k), rows_(r), cols_(c) {}
     void reset() {

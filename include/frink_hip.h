@@ -116,6 +116,14 @@ int frk_hip_weights_register(int kind, const void *host_bytes, size_t len, size_
 int frk_hip_weights_from_device(int kind, const void *dev_bytes, size_t len, size_t rows,
                                 size_t cols, void *stream, frk_weights **out);
 int frk_hip_weights_release(frk_weights *w);
+/* Q5_0 / IQ4_XS / MXFP4 (scale bytes within 104..143) reach the matrix cores decoded to signed bytes; a batched call
+ * (frk_hip_gemm_dev from four rows on, frk_hip_gemm_grouped_dev, frk_hip_moe_ffn_dev from 32 tokens on) decodes
+ * into its scratch memory each time.  This keeps the decoded rows beside the resident ones until the handle is
+ * released -- twice the bytes of a Q8_0 matrix of that shape, for a part with HBM to spare -- and those calls skip
+ * the decoding (same results, bit for bit).  Decodes on `stream` and synchronizes it.  The reference has no
+ * counterpart: its GPU GEMM dequantizes inside the kernel (crates/frink-cuda/src/mul_mm.rs:146-205).  Other kinds:
+ * FRK_ERR_UNSUPPORTED. */
+int frk_hip_weights_keep_decoded(frk_weights *w, void *stream);
 size_t frk_hip_weights_rows(const frk_weights *w);
 size_t frk_hip_weights_cols(const frk_weights *w);
 int frk_hip_weights_kind(const frk_weights *w);

@@ -82,6 +82,7 @@ def test_null_arguments_are_errors():
     assert L.frk_hip_probe(None) == fa.ERR_ARG
     assert L.frk_hip_gemv_dev(None, None, None, 0, None) == fa.ERR_ARG
     assert L.frk_hip_weights_release(None) == fa.OK
+    assert L.frk_hip_weights_keep_decoded(None, None) == fa.ERR_ARG
     h = C.c_void_p()
     assert L.frk_hip_weights_register(fa.Q4_K, None, 144, 1, 256, C.byref(h)) == fa.ERR_ARG
     buf = np.zeros(144, np.uint8)

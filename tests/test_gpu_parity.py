@@ -836,6 +836,47 @@ def test_grouped_gemm_over_the_other_kinds(fa, kind, cols, with_gather):
     w.release()
 
 
+@pytest.mark.parametrize("kind", [fo.Q5_0, fo.IQ4_XS, fo.MXFP4])
+def test_a_kept_decoded_copy_changes_no_bit(fa, kind):
+    """frk_hip_weights_keep_decoded: the batched GEMM, the grouped GEMM and the MoE layer read the kept rows instead of
+    decoding per call -- the same kernels over the same bytes, so every output bit is the same; kinds without a decoded
+    form are refused."""
+    from frink_amd import synth
+    import torch
+    E, k, hidden, ffn, batch = 4, 2, 512, 256, 70
+    stacks = [_other_kind_blocks(kind, r, c, seed=60 + j) for j, (r, c) in enumerate(((E * ffn, hidden), (E * ffn, hidden), (E * hidden, ffn)))]
+    for data in stacks:
+        if kind == fo.MXFP4:
+            data.reshape(-1, 17)[:, 0] = 110 + data.reshape(-1, 17)[:, 0] % 12
+    x = synth.activations(63, batch, hidden)
+    ids, wts = _route(synth.normal(64, batch * E).reshape(batch, E), k)
+    off = to_dev(np.array([0, 10, 10, 50, 70], np.int32))
+
+    def run(keep):
+        ws = [fa.Weights.from_host(kind, d, r, c) for d, (r, c) in zip(stacks, ((E * ffn, hidden), (E * ffn, hidden), (E * hidden, ffn)))]
+        if keep:
+            for w in ws:
+                w.keep_decoded()
+                w.keep_decoded()  # (a second request: nothing to do)
+        out = [ws[0].gemm(to_dev(x)).cpu().numpy(), fa.gemm_grouped(ws[0], E, off, to_dev(x)).cpu().numpy(),
+               fa.moe_ffn(ws[0], ws[1], ws[2], E, to_dev(x), to_dev(ids.astype(np.int32)), to_dev(wts)).cpu().numpy()]
+        for w in ws:
+            w.release()
+        return out
+    for a, b in zip(run(False), run(True)):
+        assert not np.isnan(a).any() and np.array_equal(bits(a), bits(b))
+    w4 = fa.Weights.from_host(fo.Q4_K, make_weights(fo.Q4_K, 32, 256, seed=1), 32, 256)
+    with pytest.raises(fa.BackendError):
+        w4.keep_decoded()
+    w4.release()
+    if kind == fo.MXFP4:  # scales that are not f16 values: no decoded form
+        stacks[0].reshape(-1, 17)[::5, 0] = 160
+        wx = fa.Weights.from_host(kind, stacks[0], E * ffn, hidden)
+        with pytest.raises(fa.BackendError):
+            wx.keep_decoded()
+        wx.release()
+
+
 def test_grouped_gemm_refuses_what_it_cannot_run(fa):
     data = make_weights(fo.Q8_0, 64, 256, seed=1)
     w = fa.Weights.from_host(fo.Q8_0, data, 64, 256)
