@@ -1,6 +1,7 @@
 // Shared internals of libfrink_hip: error plumbing, the weights handle, kernel launchers.
 #pragma once
 
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -110,7 +111,8 @@ struct frk_weights {
     int e8m0_min = 0, e8m0_max = 255;
     // Q5_0 / IQ4_XS / MXFP4: the rows decoded to signed bytes for the matrix cores, kept beside the resident copy
     // on request (frk_hip_weights_keep_decoded); without it every batched call decodes into its scratch memory
-    uint8_t *decoded = nullptr;
+    // (written once, under the registry's lock and behind a stream synchronization; read by calls on any thread)
+    std::atomic<uint8_t *> decoded{nullptr};
 };
 
 namespace frk {

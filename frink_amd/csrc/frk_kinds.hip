@@ -546,8 +546,8 @@ int launch_units_decode(const frk_weights *w, uint8_t *dst, hipStream_t s) {
                                       : launch_units_to_q8_0_planar(w, dst, planar.row_stride, planar.off_a, s);
 }
 int units_decoded(const frk_weights *w, uint8_t *room, hipStream_t s, const uint8_t **out) {
-    if (w->decoded) {
-        *out = w->decoded;
+    if (const uint8_t *kept = w->decoded.load(std::memory_order_acquire)) {
+        *out = kept;
         return FRK_OK;
     }
     *out = room;

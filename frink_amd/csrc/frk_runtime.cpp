@@ -367,8 +367,8 @@ int frk_hip_weights_release(frk_weights *w) {
     }
     if (w->cached) g_dev.cache.erase(std::make_pair(w->host_key, w->host_len));
     hipError_t e = hipFree(w->dev);
-    if (w->decoded) {
-        const hipError_t e2 = hipFree(w->decoded);
+    if (uint8_t *kept = w->decoded.load(std::memory_order_acquire)) {
+        const hipError_t e2 = hipFree(kept);
         if (e == hipSuccess) e = e2;
     }
     delete w;
@@ -383,7 +383,7 @@ int frk_hip_weights_keep_decoded(frk_weights *w, void *stream) {
         return set_error(FRK_ERR_UNSUPPORTED, "quant kind %d has no decoded form to keep (Q5_0, IQ4_XS, MXFP4 with scale bytes within 104..143)",
                          w->kind);
     std::lock_guard<std::mutex> lk(g_dev.mu);
-    if (w->decoded) return FRK_OK;
+    if (w->decoded.load(std::memory_order_acquire)) return FRK_OK;
     uint8_t *room = nullptr;
     FRK_HIP_TRY(hipMalloc((void **)&room, units_planar_bytes(w->rows, w->cols)));
     int rc = launch_units_decode(w, room, (hipStream_t)stream);
@@ -392,7 +392,7 @@ int frk_hip_weights_keep_decoded(frk_weights *w, void *stream) {
         (void)hipFree(room);
         return rc ? rc : set_error(FRK_ERR_HIP, "frk_hip_weights_keep_decoded: %s", hipGetErrorString(e));
     }
-    w->decoded = room;  // (published behind the synchronization: any stream may read it from here on)
+    w->decoded.store(room, std::memory_order_release);  // (behind the synchronization: any stream may read it from here on)
     return FRK_OK;
 }
 
