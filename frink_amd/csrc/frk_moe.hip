@@ -363,12 +363,19 @@ __global__ __launch_bounds__(64 * SWIGLU_WAVES) void swiglu_quantize_kernel(cons
 
 // silu(gate) * up, elementwise (frink_core::matmul::swiglu, crates/frink-core/src/matmul.rs:634-650;
 // glu_mul_device in crates/frink-cuda/src/matvec_launch.rs:551-570)
-__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ gate, const float *__restrict__ up,
-                                                     size_t n, float *__restrict__ act) {
+// (act may be gate: every element is read before it is written, by the thread that writes it)
+__global__ __launch_bounds__(256) void swiglu_kernel(const float *gate, const float *__restrict__ up, size_t n, float *act) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= n) return;
     const float g = gate[i];
     act[i] = silu_as_host(g) * up[i];
+}
+// four elements a thread, for lengths and addresses that are multiples of four floats
+__global__ __launch_bounds__(256) void swiglu4_kernel(const float4 *gate, const float4 *__restrict__ up, size_t n4, float4 *act) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4 g = gate[i], u = up[i];
+    act[i] = make_float4(silu_as_host(g.x) * u.x, silu_as_host(g.y) * u.y, silu_as_host(g.z) * u.z, silu_as_host(g.w) * u.w);
 }
 
 int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s);
@@ -439,7 +446,13 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     } while (0)
 
 int launch_swiglu(const float *gate, const float *up, size_t n, float *act, hipStream_t s) {
-    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gate, up, n, act);
+    if (n == 0) return FRK_OK;
+    const bool by_four = n % 4 == 0 && ((reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) | reinterpret_cast<uintptr_t>(act)) & 15) == 0;
+    if (by_four)
+        hipLaunchKernelGGL(swiglu4_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s, reinterpret_cast<const float4 *>(gate),
+                           reinterpret_cast<const float4 *>(up), n / 4, reinterpret_cast<float4 *>(act));
+    else
+        hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gate, up, n, act);
     FRK_LAUNCH_CHECK("swiglu");
     return FRK_OK;
 }
@@ -683,7 +696,8 @@ int launch_gemm_grouped(const frk_weights *w, size_t n_groups, const int32_t *gr
 // keeps its experts in MXFP4): every (token, slot) pair is a job of the integer decode kernel -- gate and up over the
 // token's quantized activation, silu(g) * u, that row quantized, down -- and the weighted sum in the reference's order
 // for the batch size.  Q8_0 activation blocks for Q5_0 and MXFP4 projections, Q8_K for IQ4_XS ones.  (A batch of
-// hundreds of tokens reads an expert's matrices once per pair here, out of the caches: correct, not fast.)
+// hundreds of tokens would read an expert's matrices once per pair here: from 32 tokens on the layer takes the
+// bucketed path below instead, where the kinds have a decoded form.)
 struct UnitsActs {
     int8_t *q;
     float *d;
