@@ -627,6 +627,20 @@ def main():
             extra["MoE layer 32x top-4, 2880/2880, 512 tokens, MXFP4 experts"] = {
                 "us_per_step": round(t / 20 * 1e6, 2), "tokens_per_s": round(T / (t / 20), 0),
                 "TOPS": round(2.0 * T * K4 * 3 * F4 * H4 / (t / 20) / 1e12, 1)}
+            # ONE token of that layer (decode): eight routings in turn that between them visit all 32 experts once
+            perm4 = np.random.default_rng(12).permutation(E4).astype(np.int32).reshape(8, 1, K4)
+            ids41 = [torch.from_numpy(np.ascontiguousarray(p)).to(dev) for p in perm4]
+            w41 = torch.full((1, K4), 1.0 / K4, dtype=torch.float32, device=dev)
+            x41 = xm4[:1].contiguous()
+            y41 = torch.empty((1, H4), dtype=torch.float32, device=dev)
+
+            def step4f(i):
+                fa.moe_ffn(ex4[0], ex4[1], ex4[2], E4, x41, ids41[i % 8], w41, out=y41)
+            _, t = timed(step4f, 400, 200)
+            tok4_bytes = K4 * 3 * F4 * H4 // 32 * 17
+            extra["MoE layer 32x top-4, 2880/2880, 1 token (decode), MXFP4 experts"] = {
+                "us_per_step": round(t / 400 * 1e6, 2), "algorithmic_GBs": round(tok4_bytes / (t / 400) / 1e9, 1),
+                "frac_of_hbm_peak": round(tok4_bytes / (t / 400) / 1e9 / HBM_PEAK_GBS, 4)}
             for w in ex4:
                 w.keep_decoded()
             _, t = timed(step4e, 20, 10)

@@ -145,6 +145,8 @@ hipStream_t own_stream();  // the stream host-buffer entry points run on
 
 // ---- launchers (each validates nothing: callers have checked shapes) ----
 int launch_quantize_q8_k(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s);
+int launch_swiglu_quantize_q8_k(const float *gate, const float *up, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s);
+int launch_swiglu_quantize_q8_0(const float *gate, const float *up, size_t n, int8_t *q, float *d, hipStream_t s);
 int launch_quantize_q8_0(const float *x, size_t n, int8_t *q, float *d, hipStream_t s);
 int launch_dequant(const frk_weights *w, float *out, hipStream_t s);
 int launch_dequant_rows(const frk_weights *w, const int32_t *ids, size_t n_out, float *out, hipStream_t s);
@@ -313,8 +315,8 @@ bool is_unit_kind(int kind);
 // the integer tier of Q5_0 / MXFP4 (Q8_0 activation blocks) and IQ4_XS (Q8_K quants and block scales)
 bool gemv_units_int_fits(const frk_weights *w);
 int launch_gemv_units_int(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s);
-int launch_gemv_units_int_jobs(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
-                               const int8_t *aq, const float *ad, float *y, hipStream_t s);
+int launch_gemv_units_int_jobs(const frk_weights *w, const frk_weights *w2, size_t rows_e, int n_experts, const int32_t *ids,
+                               size_t n_jobs, int act_div, const int8_t *aq, const float *ad, float *y, float *y2, hipStream_t s);
 // the routed layer over experts of these kinds: every (token, slot) pair a job of the integer decode kernel
 size_t moe_units_workspace_bytes(size_t batch, int k, int hidden, int ffn);
 int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const frk_weights *down, int n_experts, const float *x,

@@ -234,6 +234,11 @@ __device__ __forceinline__ void unit_codes(const uint8_t *row, int u, uint32_t (
 struct UnitsJobs {
     const int32_t *ids;
     int n_experts, job0, act_div;
+    // a second stack of the same shape over the same jobs and activations (gate and up in one launch): grid rows
+    // n_jobs .. 2 * n_jobs - 1 multiply W2 and write y2
+    const uint8_t *W2;
+    float *y2;
+    int n_jobs;
 };
 template <int KIND, int MAXP, bool JOBS = false>
 __global__ __launch_bounds__(512) void gemv_units_int_kernel(const uint8_t *__restrict__ W, size_t row_stride, int rows, int cols,
@@ -243,7 +248,12 @@ __global__ __launch_bounds__(512) void gemv_units_int_kernel(const uint8_t *__re
     uint8_t *lds = reinterpret_cast<uint8_t *>(smem_kinds);
     const int units = cols / 32, nd = KIND == FRK_KIND_IQ4_XS ? cols / QK_K : units;
     if (JOBS) {
-        const int job = jobs.job0 + (int)blockIdx.y;
+        int job = jobs.job0 + (int)blockIdx.y;
+        if (jobs.W2 && job >= jobs.n_jobs) {  // (uniform per workgroup)
+            job -= jobs.n_jobs;
+            W = jobs.W2;
+            y = jobs.y2;
+        }
         const int e = jobs.ids[job];
         if (e < 0 || e >= jobs.n_experts) return;  // (uniform per workgroup)
         W += (size_t)e * rows * row_stride;
@@ -373,13 +383,13 @@ static int launch_gemv_units_int_as(const frk_weights *w, const int8_t *aq, cons
     }
     const unsigned grid = (unsigned)std::min<size_t>((w->rows + 7) / 8, 2048);
     hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP>), dim3(grid), dim3(512), shmem, s, w->dev, w->layout.row_stride, (int)w->rows,
-                       (int)w->cols, aq, ad, y, UnitsJobs{nullptr, 0, 0, 1});
+                       (int)w->cols, aq, ad, y, UnitsJobs{nullptr, 0, 0, 1, nullptr, nullptr, 0});
     FRK_LAUNCH_CHECK("gemv_units_int");
     return FRK_OK;
 }
 template <int KIND, int MAXP>
-static int launch_gemv_units_jobs_as(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
-                                     const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+static int launch_gemv_units_jobs_as(const frk_weights *w, const frk_weights *w2, size_t rows_e, int n_experts, const int32_t *ids,
+                                     size_t n_jobs, int act_div, const int8_t *aq, const float *ad, float *y, float *y2, hipStream_t s) {
     const size_t shmem = gemv_units_int_lds(w);
     static bool sized = false;  // a benign race: every thread sets the same attribute
     if (!sized) {
@@ -389,31 +399,46 @@ static int launch_gemv_units_jobs_as(const frk_weights *w, size_t rows_e, int n_
         sized = true;
     }
     const unsigned gx = (unsigned)std::min<size_t>((rows_e + 7) / 8, 2048);
-    for (size_t j0 = 0; j0 < n_jobs; j0 += 32768) {  // (the grid's second dimension holds 65535)
-        const unsigned gy = (unsigned)std::min<size_t>(n_jobs - j0, 32768);
-        hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP, true>), dim3(gx, gy), dim3(512), shmem, s, w->dev, w->layout.row_stride,
-                           (int)rows_e, (int)w->cols, aq, ad, y, UnitsJobs{ids, n_experts, (int)j0, act_div});
-        FRK_LAUNCH_CHECK("gemv_units_int (jobs)");
+    if (w2 && 2 * n_jobs <= 65535) {  // both stacks in one launch
+        hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP, true>), dim3(gx, (unsigned)(2 * n_jobs)), dim3(512), shmem, s, w->dev,
+                           w->layout.row_stride, (int)rows_e, (int)w->cols, aq, ad, y,
+                           UnitsJobs{ids, n_experts, 0, act_div, w2->dev, y2, (int)n_jobs});
+        FRK_LAUNCH_CHECK("gemv_units_int (jobs, two stacks)");
+        return FRK_OK;
+    }
+    for (int m = 0; m < (w2 ? 2 : 1); m++) {
+        const frk_weights *wm = m ? w2 : w;
+        for (size_t j0 = 0; j0 < n_jobs; j0 += 32768) {  // (the grid's second dimension holds 65535)
+            const unsigned gy = (unsigned)std::min<size_t>(n_jobs - j0, 32768);
+            hipLaunchKernelGGL((gemv_units_int_kernel<KIND, MAXP, true>), dim3(gx, gy), dim3(512), shmem, s, wm->dev, wm->layout.row_stride,
+                               (int)rows_e, (int)wm->cols, aq, ad, m ? y2 : y, UnitsJobs{ids, n_experts, (int)j0, act_div, nullptr, nullptr, 0});
+            FRK_LAUNCH_CHECK("gemv_units_int (jobs)");
+        }
     }
     return FRK_OK;
 }
 template <int KIND>
-static int launch_gemv_units_jobs_kind(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs,
-                                       int act_div, const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+static int launch_gemv_units_jobs_kind(const frk_weights *w, const frk_weights *w2, size_t rows_e, int n_experts, const int32_t *ids,
+                                       size_t n_jobs, int act_div, const int8_t *aq, const float *ad, float *y, float *y2, hipStream_t s) {
     const size_t per_lane = (w->layout.row_stride / 16 + 63) / 64;
-    if (per_lane <= 3) return launch_gemv_units_jobs_as<KIND, 3>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
-    if (per_lane <= 6) return launch_gemv_units_jobs_as<KIND, 6>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
-    return launch_gemv_units_jobs_as<KIND, 12>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    if (per_lane <= 3) return launch_gemv_units_jobs_as<KIND, 3>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
+    if (per_lane <= 6) return launch_gemv_units_jobs_as<KIND, 6>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
+    return launch_gemv_units_jobs_as<KIND, 12>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
 }
-// y[job][rows_e] = W[expert ids[job]] . activation row job / act_div, on the integer tier; w stacks the experts
-int launch_gemv_units_int_jobs(const frk_weights *w, size_t rows_e, int n_experts, const int32_t *ids, size_t n_jobs, int act_div,
-                               const int8_t *aq, const float *ad, float *y, hipStream_t s) {
+// y[job][rows_e] = W[expert ids[job]] . activation row job / act_div, on the integer tier; w stacks the experts.
+// With w2 (a stack of the same kind and shape: gate and up), y2 the same over w2, in the same launch where the grid
+// holds both.
+int launch_gemv_units_int_jobs(const frk_weights *w, const frk_weights *w2, size_t rows_e, int n_experts, const int32_t *ids,
+                               size_t n_jobs, int act_div, const int8_t *aq, const float *ad, float *y, float *y2, hipStream_t s) {
     if (!gemv_units_int_fits(w))
         return set_error(FRK_ERR_UNSUPPORTED, "the integer GEMV of quant kind %d does not take rows of %zu columns", w->kind, w->cols);
-    if (w->kind == FRK_KIND_Q5_0) return launch_gemv_units_jobs_kind<FRK_KIND_Q5_0>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+    if (w2 && (w2->kind != w->kind || w2->rows != w->rows || w2->cols != w->cols || w2->layout.row_stride != w->layout.row_stride))
+        return set_error(FRK_ERR_SHAPE, "two stacks in one launch must agree in kind and shape");
+    if (w->kind == FRK_KIND_Q5_0)
+        return launch_gemv_units_jobs_kind<FRK_KIND_Q5_0>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
     if (w->kind == FRK_KIND_IQ4_XS)
-        return launch_gemv_units_jobs_kind<FRK_KIND_IQ4_XS>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
-    return launch_gemv_units_jobs_kind<FRK_KIND_MXFP4>(w, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, s);
+        return launch_gemv_units_jobs_kind<FRK_KIND_IQ4_XS>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
+    return launch_gemv_units_jobs_kind<FRK_KIND_MXFP4>(w, w2, rows_e, n_experts, ids, n_jobs, act_div, aq, ad, y, y2, s);
 }
 template <int KIND>
 static int launch_gemv_units_int_kind(const frk_weights *w, const int8_t *aq, const float *ad, float *y, hipStream_t s) {

@@ -737,15 +737,13 @@ int launch_moe_ffn_units(const frk_weights *gate, const frk_weights *up, const f
     float *d_out = (float *)p;
     int rc = quantize_for_units(gate->kind, x, batch * (size_t)hidden, xa, s);
     if (rc) return rc;
-    rc = launch_gemv_units_int_jobs(gate, (size_t)ffn, n_experts, ids, pairs, k, xa.q, xa.d, g_out, s);
+    // five launches: the tokens quantized; gate and up of every pair; silu(g) * u quantized; down; the weighted sum
+    rc = launch_gemv_units_int_jobs(gate, up, (size_t)ffn, n_experts, ids, pairs, k, xa.q, xa.d, g_out, u_out, s);
     if (rc) return rc;
-    rc = launch_gemv_units_int_jobs(up, (size_t)ffn, n_experts, ids, pairs, k, xa.q, xa.d, u_out, s);
+    rc = down->kind == FRK_KIND_IQ4_XS ? launch_swiglu_quantize_q8_k(g_out, u_out, pairs * (size_t)ffn, aa.q, aa.d, aa.bsums, s)
+                                      : launch_swiglu_quantize_q8_0(g_out, u_out, pairs * (size_t)ffn, aa.q, aa.d, s);
     if (rc) return rc;
-    rc = launch_swiglu(g_out, u_out, pairs * (size_t)ffn, g_out, s);  // (in place: element by element)
-    if (rc) return rc;
-    rc = quantize_for_units(down->kind, g_out, pairs * (size_t)ffn, aa, s);
-    if (rc) return rc;
-    rc = launch_gemv_units_int_jobs(down, (size_t)hidden, n_experts, ids, pairs, 1, aa.q, aa.d, d_out, s);
+    rc = launch_gemv_units_int_jobs(down, nullptr, (size_t)hidden, n_experts, ids, pairs, 1, aa.q, aa.d, d_out, nullptr, s);
     if (rc) return rc;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)batch, (unsigned)((hidden + 1023) / 1024)), dim3(256), 0, s, d_out, ids, weights,
                        (const int *)nullptr, k, hidden, n_experts, (int)(batch >= MOE_BUCKET_ORDER_FROM), out);

@@ -5,7 +5,7 @@
 // separately (d*sc, dmin*m, d1*nib, the subtraction), and a fused multiply-add changes low bits.
 #include <algorithm>
 
-#include "frk_internal.hpp"
+#include "frk_device.hpp"
 
 namespace frk {
 
@@ -24,13 +24,20 @@ __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
 
 // ---- quantize_activations_q8_k (crates/frink-quant/src/act_quant.rs:69-104) ----
 // One wavefront per 256-value block, four consecutive values per lane.
-__global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restrict__ x, size_t n_blocks,
+// GLU: what is quantized is silu(x) * up, element by element (GluAct::Swiglu, crates/frink-core/src/matmul.rs:634-650,
+// in front of the down projection's own quantization, ffn_batch.rs:405-415): one launch for the two.
+template <bool GLU>
+__global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restrict__ x, const float *__restrict__ up, size_t n_blocks,
                                                             int8_t *__restrict__ q, float *__restrict__ d,
                                                             int16_t *__restrict__ bsums) {
     const int lane = threadIdx.x & 63;
     const size_t b = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= n_blocks) return;
-    const float4 v = reinterpret_cast<const float4 *>(x + b * QK_K)[lane];
+    float4 v = reinterpret_cast<const float4 *>(x + b * QK_K)[lane];
+    if (GLU) {
+        const float4 u = reinterpret_cast<const float4 *>(up + b * QK_K)[lane];
+        v = make_float4(silu_as_host(v.x) * u.x, silu_as_host(v.y) * u.y, silu_as_host(v.z) * u.z, silu_as_host(v.w) * u.w);
+    }
     // f32::max ignores a NaN operand, as fmaxf does; max is exact, so the fold order is free
     float amax = fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f);
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
@@ -61,13 +68,18 @@ __global__ __launch_bounds__(256) void quantize_q8_k_kernel(const float *__restr
 
 // ---- quantize_activations_q8, Avx form (crates/frink-quant/src/act_quant.rs:157-189) ----
 // Eight lanes per 32-value block.
-__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, size_t n_blocks,
+template <bool GLU>
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restrict__ x, const float *__restrict__ up, size_t n_blocks,
                                                             int8_t *__restrict__ q, float *__restrict__ d) {
     const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t b = t >> 3;
     const bool live = b < n_blocks;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = reinterpret_cast<const float4 *>(x)[t];
+    if (GLU && live) {
+        const float4 u = reinterpret_cast<const float4 *>(up)[t];
+        v = make_float4(silu_as_host(v.x) * u.x, silu_as_host(v.y) * u.y, silu_as_host(v.z) * u.z, silu_as_host(v.w) * u.w);
+    }
     float amax = fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f);
     for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     if (!live) return;
@@ -265,15 +277,29 @@ static inline unsigned blocks_for(size_t n, size_t per) { return (unsigned)((n +
 
 int launch_quantize_q8_k(const float *x, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s) {
     const size_t nb = n / QK_K;
-    hipLaunchKernelGGL(quantize_q8_k_kernel, dim3(blocks_for(nb, 4)), dim3(256), 0, s, x, nb, q, d, bsums);
+    hipLaunchKernelGGL(quantize_q8_k_kernel<false>, dim3(blocks_for(nb, 4)), dim3(256), 0, s, x, (const float *)nullptr, nb, q, d, bsums);
     FRK_LAUNCH_CHECK("quantize_q8_k");
     return FRK_OK;
 }
 
 int launch_quantize_q8_0(const float *x, size_t n, int8_t *q, float *d, hipStream_t s) {
     const size_t nb = n / Q8_0_ELEMS;
-    hipLaunchKernelGGL(quantize_q8_0_kernel, dim3(blocks_for(nb * 8, 256)), dim3(256), 0, s, x, nb, q, d);
+    hipLaunchKernelGGL(quantize_q8_0_kernel<false>, dim3(blocks_for(nb * 8, 256)), dim3(256), 0, s, x, (const float *)nullptr, nb, q, d);
     FRK_LAUNCH_CHECK("quantize_q8_0");
+    return FRK_OK;
+}
+
+// silu(gate) * up quantized in the same launch (n a multiple of the block)
+int launch_swiglu_quantize_q8_k(const float *gate, const float *up, size_t n, int8_t *q, float *d, int16_t *bsums, hipStream_t s) {
+    const size_t nb = n / QK_K;
+    hipLaunchKernelGGL(quantize_q8_k_kernel<true>, dim3(blocks_for(nb, 4)), dim3(256), 0, s, gate, up, nb, q, d, bsums);
+    FRK_LAUNCH_CHECK("swiglu_quantize_q8_k");
+    return FRK_OK;
+}
+int launch_swiglu_quantize_q8_0(const float *gate, const float *up, size_t n, int8_t *q, float *d, hipStream_t s) {
+    const size_t nb = n / Q8_0_ELEMS;
+    hipLaunchKernelGGL(quantize_q8_0_kernel<true>, dim3(blocks_for(nb * 8, 256)), dim3(256), 0, s, gate, up, nb, q, d);
+    FRK_LAUNCH_CHECK("swiglu_quantize_q8_0");
     return FRK_OK;
 }
 
