@@ -75,13 +75,19 @@ __device__ __forceinline__ q8_v4h q8_as_k0(uint32_t h) {  // {h, 0, 0, 0}
 // same quants as frk_quant.hip's kernel; the block scales leave as the f16 values they are, a token's
 // scales padded with zeros to a multiple of eight so that the GEMM reads any chunk's eight in one load.
 // Eight lanes per 32-value block.
-__global__ __launch_bounds__(256) void quantize_q8_0_gemm_kernel(const float *__restrict__ x, size_t n_blocks, int nb,
-                                                                 int8_t *__restrict__ q, uint16_t *__restrict__ d) {
+// GLU: what is quantized is silu(x) * up, element by element (the intermediate in front of a down projection).
+template <bool GLU>
+__global__ __launch_bounds__(256) void quantize_q8_0_gemm_kernel(const float *__restrict__ x, const float *__restrict__ up, size_t n_blocks,
+                                                                 int nb, int8_t *__restrict__ q, uint16_t *__restrict__ d) {
     const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t b = t >> 3;
     const bool live = b < n_blocks;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = reinterpret_cast<const float4 *>(x)[t];
+    if (GLU && live) {
+        const float4 u = reinterpret_cast<const float4 *>(up)[t];
+        v = make_float4(silu_as_host(v.x) * u.x, silu_as_host(v.y) * u.y, silu_as_host(v.z) * u.z, silu_as_host(v.w) * u.w);
+    }
     float amax = fmaxf(fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))), 0.0f);
     for (int off = 4; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     if (!live) return;
@@ -415,8 +421,8 @@ int launch_gemm_q8_0_planar(const uint8_t *W, size_t row_stride, size_t off_d, s
     int8_t *aq = (int8_t *)ws;
     uint16_t *ad = (uint16_t *)((char *)ws + round_up(M * w->cols, 256));
     const size_t n_blocks = M * (w->cols / 32);
-    hipLaunchKernelGGL(quantize_q8_0_gemm_kernel, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, s, x, n_blocks,
-                       (int)(w->cols / 32), aq, ad);
+    hipLaunchKernelGGL(quantize_q8_0_gemm_kernel<false>, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, s, x,
+                       (const float *)nullptr, n_blocks, (int)(w->cols / 32), aq, ad);
     FRK_LAUNCH_CHECK("quantize_q8_0_gemm");
     Q8GemmArgs g;
     g.W = W;
@@ -564,11 +570,13 @@ int launch_gemm_planar_grouped(const uint8_t *W, size_t row_stride, size_t off_d
 
 // quantize_activations_q8 for the kernels above: quants [rows][cols], f16 scales [rows][cols / 32 rounded up to 8]
 size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols) { return round_up(rows * cols, 256) + round_up(rows * round_up(cols / 32, 8) * 2, 256); }
-int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s) {
+// (with `up`: silu(x) * up is what is quantized)
+int launch_quantize_q8_0_gemm(const float *x, const float *up, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s) {
     const size_t n_blocks = rows * (cols / 32);
     if (n_blocks == 0) return FRK_OK;
-    hipLaunchKernelGGL(quantize_q8_0_gemm_kernel, dim3((unsigned)((n_blocks * 8 + 255) / 256)), dim3(256), 0, s, x, n_blocks,
-                       (int)(cols / 32), q, d);
+    const dim3 grid((unsigned)((n_blocks * 8 + 255) / 256));
+    if (up) hipLaunchKernelGGL(quantize_q8_0_gemm_kernel<true>, grid, dim3(256), 0, s, x, up, n_blocks, (int)(cols / 32), q, d);
+    else hipLaunchKernelGGL(quantize_q8_0_gemm_kernel<false>, grid, dim3(256), 0, s, x, up, n_blocks, (int)(cols / 32), q, d);
     FRK_LAUNCH_CHECK("quantize_q8_0_gemm");
     return FRK_OK;
 }

@@ -248,7 +248,7 @@ int launch_gemm_planar_grouped(const uint8_t *W, size_t row_stride, size_t off_d
                                const int8_t *aq, const void *ad, const int *src_rows, const int4 *tiles, const int *n_tiles,
                                size_t max_tiles, float *y, hipStream_t s);
 size_t q8_0_gemm_acts_bytes(size_t rows, size_t cols);
-int launch_quantize_q8_0_gemm(const float *x, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s);
+int launch_quantize_q8_0_gemm(const float *x, const float *up, size_t rows, size_t cols, int8_t *q, uint16_t *d, hipStream_t s);
 // the grouped GEMM over groups of Q5_0 / IQ4_XS / MXFP4 matrices that have a decoded form for the matrix cores
 bool units_have_planar_form(const frk_weights *w);
 // that form: rows of layout_for(FRK_KIND_Q8_0, cols) -- signed bytes, then f16 scales per 32 (IQ4_XS: per block of

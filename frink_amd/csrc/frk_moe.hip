@@ -808,18 +808,20 @@ struct UnitsGroupedActs {
     const int8_t *q;
     const void *d;
 };
-static int quantize_for_units_grouped(int kind, const float *x, size_t rows, size_t cols, char *room, UnitsGroupedActs *a, hipStream_t s) {
+// (with `up`: silu(x) * up is what is quantized)
+static int quantize_for_units_grouped(int kind, const float *x, const float *up, size_t rows, size_t cols, char *room,
+                                      UnitsGroupedActs *a, hipStream_t s) {
     int8_t *q = (int8_t *)room;
     a->q = q;
     if (kind == FRK_KIND_IQ4_XS) {
         float *d = (float *)(room + round_up(rows * cols, 256));
         int16_t *bs = (int16_t *)(room + round_up(rows * cols, 256) + round_up(rows * cols / QK_K * 4 + 4, 256));
         a->d = d;
-        return launch_quantize_q8_k(x, rows * cols, q, d, bs, s);
+        return up ? launch_swiglu_quantize_q8_k(x, up, rows * cols, q, d, bs, s) : launch_quantize_q8_k(x, rows * cols, q, d, bs, s);
     }
     uint16_t *d = (uint16_t *)(room + round_up(rows * cols, 256));
     a->d = d;
-    return launch_quantize_q8_0_gemm(x, rows, cols, q, d, s);
+    return launch_quantize_q8_0_gemm(x, up, rows, cols, q, d, s);
 }
 // The grouped GEMM as an entry of its own over groups of these kinds: the tile list, the stack decoded, the
 // activation rows quantized once (Q8_0 blocks, or Q8_K for IQ4_XS), the grouped kernel gathering through the list.
@@ -863,7 +865,7 @@ int launch_gemm_grouped_units(const frk_weights *w, size_t n_groups, const int32
     int rc = units_decoded(w, m.decoded, s, &decoded);
     if (rc) return rc;
     UnitsGroupedActs xa;
-    rc = quantize_for_units_grouped(w->kind, x, x_rows, cols, m.acts, &xa, s);
+    rc = quantize_for_units_grouped(w->kind, x, nullptr, x_rows, cols, m.acts, &xa, s);
     if (rc) return rc;
     const Layout l = layout_for(FRK_KIND_Q8_0, cols);
     return launch_gemm_planar_grouped(decoded, l.row_stride, l.off_a, rows_g, cols, w->kind == FRK_KIND_IQ4_XS, xa.q, xa.d, m.src_rows,
@@ -894,7 +896,7 @@ int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up,
     rc = units_decoded(down, m.down_w, s, &down_w);
     if (rc) return rc;
     UnitsGroupedActs xa, aa;
-    rc = quantize_for_units_grouped(gate->kind, x, batch, (size_t)hidden, m.x_acts, &xa, s);
+    rc = quantize_for_units_grouped(gate->kind, x, nullptr, batch, (size_t)hidden, m.x_acts, &xa, s);
     if (rc) return rc;
     const Layout lg = layout_for(FRK_KIND_Q8_0, (size_t)hidden), ld = layout_for(FRK_KIND_Q8_0, (size_t)ffn);
     rc = launch_gemm_planar_grouped(gate_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, gate->kind == FRK_KIND_IQ4_XS, xa.q,
@@ -903,10 +905,9 @@ int launch_moe_ffn_units_grouped(const frk_weights *gate, const frk_weights *up,
     rc = launch_gemm_planar_grouped(up_w, lg.row_stride, lg.off_a, (size_t)ffn, (size_t)hidden, up->kind == FRK_KIND_IQ4_XS, xa.q,
                                     xa.d, m.gather, m.tiles, m.n_tiles, max_tiles, m.up_out, s);
     if (rc) return rc;
-    // (rows of the grouped order that no pair uses hold whatever the memory held: nothing reads their results)
-    rc = launch_swiglu(m.gate_out, m.up_out, rows * (size_t)ffn, m.gate_out, s);
-    if (rc) return rc;
-    rc = quantize_for_units_grouped(down->kind, m.gate_out, rows, (size_t)ffn, m.a_acts, &aa, s);
+    // silu(gate) * up, quantized in the same launch (rows of the grouped order that no pair uses hold whatever the
+    // memory held: nothing reads their results)
+    rc = quantize_for_units_grouped(down->kind, m.gate_out, m.up_out, rows, (size_t)ffn, m.a_acts, &aa, s);
     if (rc) return rc;
     rc = launch_gemm_planar_grouped(down_w, ld.row_stride, ld.off_a, (size_t)hidden, (size_t)ffn, down->kind == FRK_KIND_IQ4_XS, aa.q,
                                     aa.d, nullptr, m.tiles, m.n_tiles, max_tiles, m.down_out, s);
