@@ -665,7 +665,8 @@ static bool units_batch_takes_the_matrix_cores(const frk_weights *w, size_t batc
 static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, float *y, hipStream_t s, Scratch &scratch) {
     if (units_batch_takes_the_matrix_cores(w, batch)) {
         const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
-        const size_t planar_bytes = round_up(planar.row_stride * w->rows + 256, 256);
+        // (no room for the decoded rows where a copy of them is kept)
+        const size_t planar_bytes = w->decoded.load(std::memory_order_acquire) ? 0 : round_up(planar.row_stride * w->rows + 256, 256);
         void *ws = nullptr;
         int rc = scratch.get(planar_bytes + gemm_q8_0_workspace_bytes(batch, w->cols, w->rows), s, &ws);
         if (rc) return rc;
@@ -680,7 +681,8 @@ static int gemm_units_int(const frk_weights *w, const float *x, size_t batch, fl
     if (w->kind == FRK_KIND_IQ4_XS && batch >= 4) {
         // the matrix cores: the rows decoded to signed bytes with their block scales, the batch quantized to Q8_K
         const Layout planar = layout_for(FRK_KIND_Q8_0, w->cols);
-        const size_t planar_bytes = round_up(planar.row_stride * w->rows + 256, 256);
+        // (no room for the decoded rows where a copy of them is kept)
+        const size_t planar_bytes = w->decoded.load(std::memory_order_acquire) ? 0 : round_up(planar.row_stride * w->rows + 256, 256);
         const size_t n = batch * w->cols;
         const size_t q_bytes = round_up(n, 256), d_bytes = round_up(n / QK_K * 4, 256), b_bytes = round_up(n / 16 * 2, 256);
         void *ws = nullptr;
